@@ -1,0 +1,48 @@
+"""Compiles the two native libraries in-tree:
+
+  bpt_amd/csrc/libbptgraph.so  host C++ (g++)            <- bptgraph.cpp
+  bpt_amd/csrc/libbptattn.so   gfx950 HIP (hipcc)        <- bptattn.hip
+
+hipcc cross-compiles for gfx950 without a GPU.  Run `python -m bpt_amd._build`.
+"""
+import os
+import subprocess
+import sys
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+GRAPH_SO = os.path.join(CSRC, "libbptgraph.so")
+ATTN_SO = os.path.join(CSRC, "libbptattn.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed FP32 forms (v_pk_*_f32) are kept out of the generated code on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-variable", "-Wno-unused-but-set-variable",
+]
+
+
+def build_graph(verbose=True):
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+           os.path.join(CSRC, "bptgraph.cpp"), "-o", GRAPH_SO]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return GRAPH_SO
+
+
+def build_attn(verbose=True, extra=()):
+    cmd = [HIPCC] + HIP_FLAGS + list(extra) + [os.path.join(CSRC, "bptattn.hip"), "-o", ATTN_SO]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return ATTN_SO
+
+
+def build_all(verbose=True):
+    return build_graph(verbose), build_attn(verbose)
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

@@ -1,0 +1,94 @@
+"""ctypes bindings of the two native libraries (C ABIs in include/bptgraph.h and include/bptattn.h).
+
+There is no Python or CPU fallback for the device ops: if libbptattn.so is missing, importing
+`bpt_amd.graphop` raises.  Build with `python -m bpt_amd._build`.
+"""
+import ctypes
+import os
+
+from ._build import ATTN_SO, GRAPH_SO
+
+c_i64 = ctypes.c_int64
+c_vp = ctypes.c_void_p
+
+
+class PlanStruct(ctypes.Structure):
+    """Mirror of `bpt_plan` (include/bptattn.h)."""
+    _fields_ = [("rowptr", c_vp), ("idx", c_vp), ("eid", c_vp), ("items", c_vp), ("heavy", c_vp),
+                ("n_rows", c_i64), ("n_edges", c_i64), ("n_items", c_i64), ("n_heavy", c_i64), ("n_slots", c_i64)]
+
+
+class PlanInfo(ctypes.Structure):
+    """Mirror of `bptg_plan_info` (include/bptgraph.h)."""
+    _fields_ = [("n_items", c_i64), ("n_heavy", c_i64), ("n_slots", c_i64), ("max_degree", c_i64), ("flags", c_i64)]
+
+
+# every exported symbol with (restype, argtypes); tests check the libraries export exactly these
+GRAPH_API = {
+    "bptg_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "bptg_graph_sizes": (ctypes.c_int, [ctypes.c_int, c_i64, ctypes.c_int, c_i64, c_i64, c_vp, c_vp, c_vp]),
+    "bptg_graph_fill": (ctypes.c_int, [ctypes.c_int, c_i64, ctypes.c_int, c_i64, c_i64, c_i64, c_vp, c_vp, c_vp, c_vp, c_vp]),
+    "bptg_partition_csr_count": (ctypes.c_int, [c_vp, c_i64, c_i64, c_vp]),
+    "bptg_partition_csr_fill": (ctypes.c_int, [c_vp, c_i64, c_i64, c_vp, c_vp]),
+    "bptg_build_csr": (ctypes.c_int, [c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp]),
+    "bptg_plan_sizes": (ctypes.c_int, [c_vp, c_vp, c_i64, c_i64, c_i64, ctypes.POINTER(PlanInfo)]),
+    "bptg_plan_fill": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64,
+                                      c_vp, c_vp, c_vp, c_vp, c_vp, ctypes.POINTER(PlanInfo)]),
+}
+
+_PP = ctypes.POINTER(PlanStruct)
+_tail = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_vp]          # h, d, dtype, stream
+ATTN_API = {
+    "bpt_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "bpt_set_force_generic": (ctypes.c_int, [ctypes.c_int]),
+    "bpt_workspace_bytes": (c_i64, [ctypes.c_int, _PP, _PP, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "bpt_maskedmm_csr_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp] + _tail),
+    "bpt_maskedmm_csr_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
+    "bpt_node_mul_edge_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp] + _tail),
+    "bpt_node_mul_edge_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
+    "bpt_sparse_softmax_forward": (ctypes.c_int, [_PP, c_vp, c_vp, ctypes.c_int, ctypes.c_int, c_vp]),
+    "bpt_sparse_softmax_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, ctypes.c_int, ctypes.c_int, c_vp]),
+    "bpt_vector_spmm_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
+    "bpt_vector_spmm_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
+    "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float] + _tail),
+    "bpt_attention_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
+                                             ctypes.c_float] + _tail),
+}
+
+_graph = None
+_attn = None
+
+
+def _load(path, api, what):
+    if not os.path.exists(path):
+        raise ImportError(f"{what} is not built ({path} missing): run `python -m bpt_amd._build`")
+    lib = ctypes.CDLL(path)
+    for name, (res, args) in api.items():
+        fn = getattr(lib, name)          # AttributeError if the library does not export it
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+def graph_lib():
+    global _graph
+    if _graph is None:
+        _graph = _load(GRAPH_SO, GRAPH_API, "libbptgraph")
+    return _graph
+
+
+def attn_lib():
+    global _attn
+    if _attn is None:
+        _attn = _load(ATTN_SO, ATTN_API, "libbptattn (HIP kernels)")
+    return _attn
+
+
+def check_graph(status):
+    if status != 0:
+        raise ValueError("bptgraph: " + graph_lib().bptg_strerror(status).decode())
+
+
+def check_attn(status, what):
+    if status != 0:
+        raise RuntimeError(f"{what}: " + attn_lib().bpt_strerror(status).decode() + f" (status {status})")

@@ -1,0 +1,943 @@
+// libbptattn: gfx950 HIP kernels of the BPT graph-attention path (C ABI in include/bptattn.h).
+//
+// Execution model.  One 64-lane wavefront owns one work item of the plan: a whole row of the
+// CSR side it walks, or one segment of a row that is longer than the plan's segment length.
+// Whole rows write their result directly; segments write a partial result into the workspace
+// and a second kernel combines the partials of each split row in slot order.  No atomics
+// anywhere, so every output is bit-reproducible run to run.
+//
+// Two kernel families:
+//   * "generic": any h, d and f32 / f64 / bf16, lanes stride over the columns of a node row;
+//   * "fast":    compile-time (h, d) for f32 / bf16.  A node row of C = h*d elements is spread
+//                over the wavefront so that lane l holds C/64 elements of head l / (64/h) and
+//                every 16-byte load instruction of the wavefront covers whole 128-byte lines.
+//                A per-head dot product is then C/64 FMAs plus log2(64/h) DPP additions.
+// Work items are dealt to workgroups so that each XCD (blocks are distributed round-robin over
+// the 8 XCDs) walks a contiguous range of rows: neighbouring tokens share most of their
+// neighbours, which keeps the gathered K/V rows in that XCD's L2.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cmath>
+#include <cstdint>
+
+#include "../../include/bptattn.h"
+
+namespace {
+
+constexpr int WAVE = 64;
+constexpr int WAVES_PER_BLOCK = 4;
+constexpr int BLOCK = WAVE * WAVES_PER_BLOCK;
+constexpr float M_INIT_LOG2 = -1.4426950408889634e9f;   // -1e9 (graphop_kernel.cu:428) in base-2 units
+constexpr float LOG2E = 1.4426950408889634f;
+
+std::atomic<int> g_force_generic{0};
+
+// ------------------------------------------------------------------------------------------
+// element types
+// ------------------------------------------------------------------------------------------
+struct bf16_t { uint16_t bits; };
+
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);   // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                              // round to nearest even
+    return (uint16_t)(u >> 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    using acc_t = float;
+    static __device__ __forceinline__ float ld(const float *p) { return *p; }
+    static __device__ __forceinline__ void st(float *p, float v) { *p = v; }
+};
+template <> struct Elem<double> {
+    using acc_t = double;
+    static __device__ __forceinline__ double ld(const double *p) { return *p; }
+    static __device__ __forceinline__ void st(double *p, double v) { *p = v; }
+};
+template <> struct Elem<bf16_t> {
+    using acc_t = float;
+    static __device__ __forceinline__ float ld(const bf16_t *p) { return bf16_to_f32(p->bits); }
+    static __device__ __forceinline__ void st(bf16_t *p, float v) { p->bits = f32_to_bf16(v); }
+};
+
+__device__ __forceinline__ float exp_acc(float x) { return expf(x); }
+__device__ __forceinline__ double exp_acc(double x) { return exp(x); }
+
+// ------------------------------------------------------------------------------------------
+// work distribution
+// ------------------------------------------------------------------------------------------
+struct Item { int row, begin, end, slot; };
+
+// Blocks go round-robin to the 8 XCDs; remap so XCD x gets a contiguous run of block indices.
+__device__ __forceinline__ int xcd_contiguous_block() {
+    const int nb = gridDim.x, b = blockIdx.x;
+    const int q = nb >> 3, rem = nb & 7, x = b & 7, k = b >> 3;
+    return x * q + (x < rem ? x : rem) + k;
+}
+
+__device__ __forceinline__ bool fetch_item(const bpt_plan &P, Item &it) {
+    const int w = xcd_contiguous_block() * WAVES_PER_BLOCK + (int)(threadIdx.x >> 6);
+    if (w >= (int)P.n_items) return false;
+    const int4 v = reinterpret_cast<const int4 *>(P.items)[w];
+    // the item is the same for all lanes of the wavefront: keep it in scalar registers
+    it.row = __builtin_amdgcn_readfirstlane(v.x);
+    it.begin = __builtin_amdgcn_readfirstlane(v.y);
+    it.end = __builtin_amdgcn_readfirstlane(v.z);
+    it.slot = __builtin_amdgcn_readfirstlane(v.w);
+    return true;
+}
+
+template <typename A> __device__ __forceinline__ A wave_sum(A x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+template <typename A> __device__ __forceinline__ A wave_max(A x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        A y = __shfl_xor(x, o);
+        x = x > y ? x : y;
+    }
+    return x;
+}
+
+// Reduction over NW wavefronts of a block (NW == 1: a single wavefront, no LDS, no barrier).
+template <typename A, int NW, bool IS_MAX> __device__ __forceinline__ A group_reduce(A x, A *smem) {
+    x = IS_MAX ? wave_max(x) : wave_sum(x);
+    if (NW == 1) return x;
+    const int w = threadIdx.x >> 6;
+    __syncthreads();                       // smem may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) smem[w] = x;
+    __syncthreads();
+    A r = smem[0];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) r = IS_MAX ? (r > smem[i] ? r : smem[i]) : r + smem[i];
+    return r;
+}
+
+// ------------------------------------------------------------------------------------------
+// generic kernels
+// ------------------------------------------------------------------------------------------
+// y[eid[p], h] = sum_d A[row, h, d] * B[..]   MODE 0: B (n, H, D) row idx[p];  MODE 1: B (E, D) row eid[p]
+template <typename T, int MODE>
+__global__ __launch_bounds__(BLOCK) void k_sddmm_generic(bpt_plan P, const T *__restrict__ A, const T *__restrict__ B,
+                                                         T *__restrict__ y, int H, int D) {
+    using acc_t = typename Elem<T>::acc_t;
+    Item it;
+    if (!fetch_item(P, it)) return;
+    const int lane = threadIdx.x & 63;
+    const T *a = A + (size_t)it.row * H * D;
+    for (int p = it.begin; p < it.end; ++p) {
+        const int e = P.eid[p];
+        const T *b = (MODE == 0) ? B + (size_t)P.idx[p] * H * D : B + (size_t)e * D;
+        for (int h = 0; h < H; ++h) {
+            acc_t s = 0;
+            for (int dd = lane; dd < D; dd += WAVE)
+                s += (acc_t)Elem<T>::ld(a + h * D + dd) * (acc_t)Elem<T>::ld(b + (MODE == 0 ? h * D : 0) + dd);
+            s = wave_sum(s);
+            if (lane == 0) Elem<T>::st(y + (size_t)e * H + h, s);
+        }
+    }
+}
+
+// Y[row, j] = sum_p W[eid[p], j / D] * X[..]   MODE 0: X (n, H, D) row idx[p];  MODE 1: X (E, D) row eid[p], column j % D
+template <typename T, int MODE>
+__global__ __launch_bounds__(BLOCK) void k_spmm_generic(bpt_plan P, const T *__restrict__ W, const T *__restrict__ X,
+                                                        T *__restrict__ Y, typename Elem<T>::acc_t *__restrict__ ws,
+                                                        int H, int D) {
+    using acc_t = typename Elem<T>::acc_t;
+    Item it;
+    if (!fetch_item(P, it)) return;
+    const int lane = threadIdx.x & 63;
+    const int C = H * D;
+    for (int j = lane; j < C; j += WAVE) {
+        const int h = j / D;
+        acc_t s = 0;
+        for (int p = it.begin; p < it.end; ++p) {
+            const int e = P.eid[p];
+            const acc_t w = Elem<T>::ld(W + (size_t)e * H + h);
+            const acc_t xv = (MODE == 0) ? Elem<T>::ld(X + (size_t)P.idx[p] * C + j) : Elem<T>::ld(X + (size_t)e * D + (j - h * D));
+            s += w * xv;
+        }
+        if (it.slot < 0) Elem<T>::st(Y + (size_t)it.row * C + j, s);
+        else ws[(size_t)it.slot * C + j] = s;
+    }
+}
+
+// Y[row, :] = sum of the row's partial slots, in slot order.  One block per split row.
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_combine_sum(const int32_t *__restrict__ heavy,
+                                                       const typename Elem<T>::acc_t *__restrict__ ws, T *__restrict__ Y, int C) {
+    using acc_t = typename Elem<T>::acc_t;
+    const int row = heavy[3 * blockIdx.x], s0 = heavy[3 * blockIdx.x + 1], ns = heavy[3 * blockIdx.x + 2];
+    for (int j = threadIdx.x; j < C; j += BLOCK) {
+        acc_t s = 0;
+        for (int k = 0; k < ns; ++k) s += ws[(size_t)(s0 + k) * C + j];
+        Elem<T>::st(Y + (size_t)row * C + j, s);
+    }
+}
+
+// dB[eid[p], d] = sum_h dy[eid[p], h] * A[row, h, d]      (graphop_kernel.cu:79-94)
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_nme_dB_generic(bpt_plan P, const T *__restrict__ A, const T *__restrict__ dy,
+                                                          T *__restrict__ dB, int H, int D) {
+    using acc_t = typename Elem<T>::acc_t;
+    Item it;
+    if (!fetch_item(P, it)) return;
+    const int lane = threadIdx.x & 63;
+    const T *a = A + (size_t)it.row * H * D;
+    for (int p = it.begin; p < it.end; ++p) {
+        const int e = P.eid[p];
+        for (int dd = lane; dd < D; dd += WAVE) {
+            acc_t s = 0;
+            for (int h = 0; h < H; ++h) s += (acc_t)Elem<T>::ld(dy + (size_t)e * H + h) * (acc_t)Elem<T>::ld(a + h * D + dd);
+            Elem<T>::st(dB + (size_t)e * D + dd, s);
+        }
+    }
+}
+
+// Row softmax.  NW == 1: one wavefront per whole-row item (segments of split rows exit);
+// NW == WAVES_PER_BLOCK: one block per split row (grid = n_heavy).
+template <typename T, int NW>
+__global__ __launch_bounds__(BLOCK) void k_softmax_fwd(bpt_plan P, const T *__restrict__ x, T *__restrict__ y, int H) {
+    using acc_t = typename Elem<T>::acc_t;
+    __shared__ acc_t smem[WAVES_PER_BLOCK];
+    int begin, end, tid;
+    if (NW == 1) {
+        Item it;
+        if (!fetch_item(P, it) || it.slot >= 0) return;
+        begin = it.begin; end = it.end; tid = threadIdx.x & 63;
+    } else {
+        const int row = P.heavy[3 * blockIdx.x];
+        begin = P.rowptr[row]; end = P.rowptr[row + 1]; tid = threadIdx.x;
+    }
+    constexpr int NT = NW * WAVE;
+    for (int h = 0; h < H; ++h) {
+        acc_t m = (acc_t)-1e9;
+        for (int p = begin + tid; p < end; p += NT) {
+            const acc_t v = Elem<T>::ld(x + (size_t)P.eid[p] * H + h);
+            m = v > m ? v : m;
+        }
+        m = group_reduce<acc_t, NW, true>(m, smem);
+        acc_t s = 0;
+        for (int p = begin + tid; p < end; p += NT) s += exp_acc((acc_t)Elem<T>::ld(x + (size_t)P.eid[p] * H + h) - m);
+        s = group_reduce<acc_t, NW, false>(s, smem);
+        for (int p = begin + tid; p < end; p += NT) {
+            const size_t o = (size_t)P.eid[p] * H + h;
+            Elem<T>::st(y + o, exp_acc((acc_t)Elem<T>::ld(x + o) - m) / s);
+        }
+    }
+}
+
+// dx = dy*y - (sum_row dy*y) * y      (graphop_kernel.cu:208-230)
+template <typename T, int NW>
+__global__ __launch_bounds__(BLOCK) void k_softmax_bwd(bpt_plan P, const T *__restrict__ y, const T *__restrict__ dy,
+                                                       T *__restrict__ dx, int H) {
+    using acc_t = typename Elem<T>::acc_t;
+    __shared__ acc_t smem[WAVES_PER_BLOCK];
+    int begin, end, tid;
+    if (NW == 1) {
+        Item it;
+        if (!fetch_item(P, it) || it.slot >= 0) return;
+        begin = it.begin; end = it.end; tid = threadIdx.x & 63;
+    } else {
+        const int row = P.heavy[3 * blockIdx.x];
+        begin = P.rowptr[row]; end = P.rowptr[row + 1]; tid = threadIdx.x;
+    }
+    constexpr int NT = NW * WAVE;
+    for (int h = 0; h < H; ++h) {
+        acc_t s = 0;
+        for (int p = begin + tid; p < end; p += NT) {
+            const size_t o = (size_t)P.eid[p] * H + h;
+            s += (acc_t)Elem<T>::ld(dy + o) * (acc_t)Elem<T>::ld(y + o);
+        }
+        s = group_reduce<acc_t, NW, false>(s, smem);
+        for (int p = begin + tid; p < end; p += NT) {
+            const size_t o = (size_t)P.eid[p] * H + h;
+            const acc_t yv = Elem<T>::ld(y + o);
+            Elem<T>::st(dx + o, (acc_t)Elem<T>::ld(dy + o) * yv - s * yv);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// fast family: compile-time (H, D), f32 / bf16
+// ------------------------------------------------------------------------------------------
+template <typename T, int H_, int D_> struct Lay {
+    static constexpr int H = H_, D = D_, C = H_ * D_;
+    static constexpr int LPH = 64 / H_;                 // lanes per head
+    static constexpr int EPL = C / 64;                  // elements per lane (all of one head)
+    static constexpr int VE = 16 / (int)sizeof(T);      // elements per 16-byte vector
+    static constexpr int NV = EPL / VE;                 // 16-byte vectors per lane
+    static_assert(64 % H_ == 0 && C % 64 == 0 && EPL % VE == 0 && NV >= 1, "unsupported fast shape");
+    static_assert(D_ == NV * LPH * VE, "layout does not tile the head");
+    // element offset inside a node row of vector i of `lane`: LPH consecutive lanes cover
+    // LPH*16 contiguous bytes of their head
+    static __device__ __forceinline__ int off(int lane, int i) { return (lane / LPH) * D + (i * LPH + lane % LPH) * VE; }
+};
+
+template <typename T, int H, int D>
+__device__ __forceinline__ void load_row(const T *__restrict__ row, int lane, float (&out)[Lay<T, H, D>::EPL]) {
+    using L = Lay<T, H, D>;
+#pragma unroll
+    for (int i = 0; i < L::NV; ++i) {
+        if constexpr (sizeof(T) == 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(row) + L::off(lane, i));
+            out[4 * i] = v.x; out[4 * i + 1] = v.y; out[4 * i + 2] = v.z; out[4 * i + 3] = v.w;
+        } else {
+            const uint4 v = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(row) + L::off(lane, i));
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                out[8 * i + 2 * c] = __uint_as_float(w[c] << 16);
+                out[8 * i + 2 * c + 1] = __uint_as_float(w[c] & 0xffff0000u);
+            }
+        }
+    }
+}
+
+template <typename T, int H, int D>
+__device__ __forceinline__ void store_row(T *__restrict__ row, int lane, const float (&in)[Lay<T, H, D>::EPL]) {
+    using L = Lay<T, H, D>;
+#pragma unroll
+    for (int i = 0; i < L::NV; ++i) {
+        if constexpr (sizeof(T) == 4) {
+            *reinterpret_cast<float4 *>(reinterpret_cast<float *>(row) + L::off(lane, i)) =
+                make_float4(in[4 * i], in[4 * i + 1], in[4 * i + 2], in[4 * i + 3]);
+        } else {
+            uint32_t w[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                w[c] = (uint32_t)f32_to_bf16(in[8 * i + 2 * c]) | ((uint32_t)f32_to_bf16(in[8 * i + 2 * c + 1]) << 16);
+            *reinterpret_cast<uint4 *>(reinterpret_cast<uint16_t *>(row) + L::off(lane, i)) = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+    }
+}
+
+// f32 partial rows in the workspace use the same lane layout with 4-element vectors
+template <int H, int D>
+__device__ __forceinline__ void store_row_ws(float *__restrict__ row, int lane, const float (&in)[H * D / 64]) {
+    constexpr int LPH = 64 / H, EPL = H * D / 64;
+#pragma unroll
+    for (int i = 0; i < EPL / 4; ++i)
+        *reinterpret_cast<float4 *>(row + (lane / LPH) * D + (i * LPH + lane % LPH) * 4) =
+            make_float4(in[4 * i], in[4 * i + 1], in[4 * i + 2], in[4 * i + 3]);
+}
+
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the LPH lanes that hold one head; the result is in all of them.
+template <int LPH> __device__ __forceinline__ float head_sum(float x) {
+    if constexpr (LPH >= 2) x += dpp_mov<0xB1>(x);    // quad_perm [1,0,3,2]
+    if constexpr (LPH >= 4) x += dpp_mov<0x4E>(x);    // quad_perm [2,3,0,1]
+    if constexpr (LPH >= 8) x += dpp_mov<0x141>(x);   // row_half_mirror
+    if constexpr (LPH >= 16) x += dpp_mov<0x140>(x);  // row_mirror
+    if constexpr (LPH >= 32) x += __shfl_xor(x, 16);
+    if constexpr (LPH >= 64) x += __shfl_xor(x, 32);
+    return x;
+}
+
+template <int N> __device__ __forceinline__ float dot_n(const float (&a)[N], const float (&b)[N]) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < N; ++i) s = fmaf(a[i], b[i], s);
+    return s;
+}
+
+// The gathers are latency bound: all row loads of a batch must be in flight before the first
+// one is consumed.  Without this fence the instruction scheduler interleaves loads and FMAs to
+// save registers and waits for every load separately.
+__device__ __forceinline__ void issue_loads_first() { __builtin_amdgcn_sched_barrier(0); }
+
+// weight loads for the fast SpMM: the unfused API passes T-typed edge data, the fused backward f32
+template <typename WT> __device__ __forceinline__ float ld_w(const WT *p) { return Elem<WT>::ld(p); }
+
+// y[eid[p], head] = A[row, head, :] . B[idx[p], head, :]
+template <typename T, int H, int D, int BATCH>
+__global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ y) {
+    using L = Lay<T, H, D>;
+    Item it;
+    if (!fetch_item(P, it)) return;
+    const int lane = threadIdx.x & 63, head = lane / L::LPH;
+    float a[L::EPL];
+    load_row<T, H, D>(A + (size_t)it.row * L::C, lane, a);
+    for (int p0 = it.begin; p0 < it.end; p0 += WAVE) {
+        const int cnt = min(WAVE, it.end - p0);
+        const int my_idx = lane < cnt ? P.idx[p0 + lane] : 0;
+        const int my_eid = lane < cnt ? P.eid[p0 + lane] : 0;
+        for (int b = 0; b < cnt; b += BATCH) {
+            float bv[BATCH][L::EPL];
+            int ee[BATCH];
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const int j = (b + e < cnt) ? b + e : b;
+                ee[e] = __builtin_amdgcn_readlane(my_eid, j);
+                load_row<T, H, D>(B + (size_t)__builtin_amdgcn_readlane(my_idx, j) * L::C, lane, bv[e]);
+            }
+            issue_loads_first();
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const float s = head_sum<L::LPH>(dot_n<L::EPL>(a, bv[e]));
+                if (b + e < cnt && lane % L::LPH == 0) Elem<T>::st(y + (size_t)ee[e] * H + head, s);
+            }
+        }
+    }
+}
+
+// Y0[row] = sum_p W0[eid[p], head] * X0[idx[p]]  (and the same with W1, X1 -> Y1 when NOUT == 2)
+template <typename T, typename WT, int H, int D, int BATCH, int NOUT>
+__global__ __launch_bounds__(BLOCK) void k_spmm_fast(bpt_plan P, const WT *__restrict__ W0, const T *__restrict__ X0, T *__restrict__ Y0,
+                                                     const WT *__restrict__ W1, const T *__restrict__ X1, T *__restrict__ Y1,
+                                                     float *__restrict__ ws0, float *__restrict__ ws1) {
+    using L = Lay<T, H, D>;
+    Item it;
+    if (!fetch_item(P, it)) return;
+    const int lane = threadIdx.x & 63, head = lane / L::LPH;
+    float acc0[L::EPL], acc1[L::EPL];
+#pragma unroll
+    for (int i = 0; i < L::EPL; ++i) { acc0[i] = 0.f; acc1[i] = 0.f; }
+    for (int p0 = it.begin; p0 < it.end; p0 += WAVE) {
+        const int cnt = min(WAVE, it.end - p0);
+        const int my_idx = lane < cnt ? P.idx[p0 + lane] : 0;
+        const int my_eid = lane < cnt ? P.eid[p0 + lane] : 0;
+        for (int b = 0; b < cnt; b += BATCH) {
+            float x0[BATCH][L::EPL], x1[NOUT == 2 ? BATCH : 1][L::EPL];
+            float w0[BATCH], w1[BATCH];
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const bool ok = b + e < cnt;
+                const int j = ok ? b + e : b;
+                const int src = __builtin_amdgcn_readlane(my_idx, j);
+                const int ed = __builtin_amdgcn_readlane(my_eid, j);
+                load_row<T, H, D>(X0 + (size_t)src * L::C, lane, x0[e]);
+                w0[e] = ok ? ld_w(W0 + (size_t)ed * H + head) : 0.f;
+                if constexpr (NOUT == 2) {
+                    load_row<T, H, D>(X1 + (size_t)src * L::C, lane, x1[e]);
+                    w1[e] = ok ? ld_w(W1 + (size_t)ed * H + head) : 0.f;
+                }
+            }
+            issue_loads_first();
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+#pragma unroll
+                for (int i = 0; i < L::EPL; ++i) {
+                    acc0[i] = fmaf(w0[e], x0[e][i], acc0[i]);
+                    if constexpr (NOUT == 2) acc1[i] = fmaf(w1[e], x1[e][i], acc1[i]);
+                }
+            }
+        }
+    }
+    if (it.slot < 0) {
+        store_row<T, H, D>(Y0 + (size_t)it.row * L::C, lane, acc0);
+        if constexpr (NOUT == 2) store_row<T, H, D>(Y1 + (size_t)it.row * L::C, lane, acc1);
+    } else {
+        store_row_ws<H, D>(ws0 + (size_t)it.slot * L::C, lane, acc0);
+        if constexpr (NOUT == 2) store_row_ws<H, D>(ws1 + (size_t)it.slot * L::C, lane, acc1);
+    }
+}
+
+// Fused forward: per destination row, online softmax over the in-edges in batches of BATCH.
+// Scores are kept in base-2 units (q is pre-multiplied by scale*log2(e)).
+template <typename T, int H, int D, int BATCH>
+__global__ __launch_bounds__(BLOCK) void k_attn_fwd(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
+                                                    T *__restrict__ o, float *__restrict__ lse, float *__restrict__ ws_acc,
+                                                    float *__restrict__ ws_ml, float scale_log2e) {
+    using L = Lay<T, H, D>;
+    Item it;
+    if (!fetch_item(P, it)) return;
+    const int lane = threadIdx.x & 63, head = lane / L::LPH;
+    float qv[L::EPL], acc[L::EPL];
+    load_row<T, H, D>(q + (size_t)it.row * L::C, lane, qv);
+#pragma unroll
+    for (int i = 0; i < L::EPL; ++i) { qv[i] *= scale_log2e; acc[i] = 0.f; }
+    float m = M_INIT_LOG2, l = 0.f;
+    for (int p0 = it.begin; p0 < it.end; p0 += WAVE) {
+        const int cnt = min(WAVE, it.end - p0);
+        const int my_idx = lane < cnt ? P.idx[p0 + lane] : 0;
+        for (int b = 0; b < cnt; b += BATCH) {
+            float kv[BATCH][L::EPL], vv[BATCH][L::EPL], s[BATCH];
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const int src = __builtin_amdgcn_readlane(my_idx, (b + e < cnt) ? b + e : b);
+                load_row<T, H, D>(k + (size_t)src * L::C, lane, kv[e]);
+                load_row<T, H, D>(v + (size_t)src * L::C, lane, vv[e]);
+            }
+            issue_loads_first();
+            float mx = m;
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const float t = head_sum<L::LPH>(dot_n<L::EPL>(qv, kv[e]));
+                s[e] = (b + e < cnt) ? t : -INFINITY;
+                mx = fmaxf(mx, s[e]);
+            }
+            const float alpha = __builtin_amdgcn_exp2f(m - mx);
+            l *= alpha;
+#pragma unroll
+            for (int i = 0; i < L::EPL; ++i) acc[i] *= alpha;
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const float pe = __builtin_amdgcn_exp2f(s[e] - mx);
+                l += pe;
+#pragma unroll
+                for (int i = 0; i < L::EPL; ++i) acc[i] = fmaf(pe, vv[e][i], acc[i]);
+            }
+            m = mx;
+        }
+    }
+    if (it.slot < 0) {
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+        for (int i = 0; i < L::EPL; ++i) acc[i] *= inv;
+        store_row<T, H, D>(o + (size_t)it.row * L::C, lane, acc);
+        if (lane % L::LPH == 0) lse[(size_t)it.row * H + head] = l > 0.f ? m + log2f(l) : 0.f;
+    } else {
+        store_row_ws<H, D>(ws_acc + (size_t)it.slot * L::C, lane, acc);
+        if (lane % L::LPH == 0) {
+            ws_ml[((size_t)it.slot * H + head) * 2] = m;
+            ws_ml[((size_t)it.slot * H + head) * 2 + 1] = l;
+        }
+    }
+}
+
+// Combine the (m, l, acc) partials of each split row in slot order.  One block per split row.
+template <typename T, int H, int D>
+__global__ __launch_bounds__(BLOCK) void k_attn_fwd_combine(const int32_t *__restrict__ heavy, const float *__restrict__ ws_acc,
+                                                            const float *__restrict__ ws_ml, T *__restrict__ o, float *__restrict__ lse) {
+    constexpr int C = H * D;
+    const int row = heavy[3 * blockIdx.x], s0 = heavy[3 * blockIdx.x + 1], ns = heavy[3 * blockIdx.x + 2];
+    for (int j = threadIdx.x; j < C; j += BLOCK) {
+        const int head = j / D;
+        float M = M_INIT_LOG2;
+        for (int kk = 0; kk < ns; ++kk) M = fmaxf(M, ws_ml[((size_t)(s0 + kk) * H + head) * 2]);
+        float lsum = 0.f, a = 0.f;
+        for (int kk = 0; kk < ns; ++kk) {
+            const float w = __builtin_amdgcn_exp2f(ws_ml[((size_t)(s0 + kk) * H + head) * 2] - M);
+            lsum = fmaf(ws_ml[((size_t)(s0 + kk) * H + head) * 2 + 1], w, lsum);
+            a = fmaf(ws_acc[(size_t)(s0 + kk) * C + j], w, a);
+        }
+        Elem<T>::st(o + (size_t)row * C + j, lsum > 0.f ? a / lsum : 0.f);
+        if (j % D == 0) lse[(size_t)row * H + head] = lsum > 0.f ? M + log2f(lsum) : 0.f;
+    }
+}
+
+// Fused backward, destination side: recompute p from lse, delta = dO.O, ds = p*(dO.v - delta)*scale,
+// dQ[row] = sum ds*k; p and ds go to (E, H) f32 buffers addressed by edge id for the source-side pass.
+template <typename T, int H, int D, int BATCH>
+__global__ __launch_bounds__(BLOCK) void k_attn_bwd_dst(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
+                                                        const T *__restrict__ o, const T *__restrict__ d_o, const float *__restrict__ lse,
+                                                        T *__restrict__ dq, float *__restrict__ pbuf, float *__restrict__ dsbuf,
+                                                        float *__restrict__ ws_dq, float scale, float scale_log2e) {
+    using L = Lay<T, H, D>;
+    Item it;
+    if (!fetch_item(P, it)) return;
+    const int lane = threadIdx.x & 63, head = lane / L::LPH;
+    float qv[L::EPL], dov[L::EPL], dqa[L::EPL];
+    float delta;
+    {
+        float ov[L::EPL];
+        load_row<T, H, D>(o + (size_t)it.row * L::C, lane, ov);
+        load_row<T, H, D>(d_o + (size_t)it.row * L::C, lane, dov);
+        delta = head_sum<L::LPH>(dot_n<L::EPL>(dov, ov));
+    }
+    load_row<T, H, D>(q + (size_t)it.row * L::C, lane, qv);
+#pragma unroll
+    for (int i = 0; i < L::EPL; ++i) dqa[i] = 0.f;
+    const float lse2 = lse[(size_t)it.row * H + head];
+    for (int p0 = it.begin; p0 < it.end; p0 += WAVE) {
+        const int cnt = min(WAVE, it.end - p0);
+        const int my_idx = lane < cnt ? P.idx[p0 + lane] : 0;
+        const int my_eid = lane < cnt ? P.eid[p0 + lane] : 0;
+        for (int b = 0; b < cnt; b += BATCH) {
+            float kv[BATCH][L::EPL], vv[BATCH][L::EPL];
+            int ee[BATCH];
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const int j = (b + e < cnt) ? b + e : b;
+                const int src = __builtin_amdgcn_readlane(my_idx, j);
+                ee[e] = __builtin_amdgcn_readlane(my_eid, j);
+                load_row<T, H, D>(k + (size_t)src * L::C, lane, kv[e]);
+                load_row<T, H, D>(v + (size_t)src * L::C, lane, vv[e]);
+            }
+            issue_loads_first();
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const float s = head_sum<L::LPH>(dot_n<L::EPL>(qv, kv[e]));
+                const float dp = head_sum<L::LPH>(dot_n<L::EPL>(dov, vv[e]));
+                const bool ok = b + e < cnt;
+                const float pe = ok ? __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2)) : 0.f;
+                const float ds = pe * (dp - delta) * scale;
+#pragma unroll
+                for (int i = 0; i < L::EPL; ++i) dqa[i] = fmaf(ds, kv[e][i], dqa[i]);
+                if (ok && lane % L::LPH == 0) {
+                    pbuf[(size_t)ee[e] * H + head] = pe;
+                    dsbuf[(size_t)ee[e] * H + head] = ds;
+                }
+            }
+        }
+    }
+    if (it.slot < 0) store_row<T, H, D>(dq + (size_t)it.row * L::C, lane, dqa);
+    else store_row_ws<H, D>(ws_dq + (size_t)it.slot * L::C, lane, dqa);
+}
+
+// ------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------
+inline int grid_for(const bpt_plan *p) { return (int)((p->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK); }
+
+inline int check_plan(const bpt_plan *p, bool need_idx) {
+    if (!p) return BPT_ERR_NULL;
+    if (p->n_rows < 0 || p->n_edges < 0 || p->n_items < 0 || p->n_heavy < 0 || p->n_slots < 0) return BPT_ERR_SIZE;
+    if (p->n_items > 0 && (!p->items || !p->rowptr)) return BPT_ERR_NULL;
+    if (p->n_edges > 0 && (!p->eid || (need_idx && !p->idx))) return BPT_ERR_NULL;
+    if (p->n_heavy > 0 && !p->heavy) return BPT_ERR_NULL;
+    if (p->n_items < p->n_rows) return BPT_ERR_SIZE;     // every row owns at least one item
+    return BPT_OK;
+}
+
+inline int check_shape(int h, int d, int dtype) {
+    if (dtype != BPT_F32 && dtype != BPT_F64 && dtype != BPT_BF16) return BPT_ERR_DTYPE;
+    if (h < 1 || d < 1 || (int64_t)h * d > (1 << 20)) return BPT_ERR_SHAPE;
+    return BPT_OK;
+}
+
+inline size_t acc_size(int dtype) { return dtype == BPT_F64 ? 8 : 4; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int launch_status() {
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? BPT_OK : (int)e;
+}
+
+// (H, D) pairs with a fast instantiation.  bf16 needs C >= 512 (eight elements per 16-byte vector).
+#define BPT_FAST_SHAPES_F32(X) X(4, 64) X(8, 64) X(16, 64) X(8, 32)
+#define BPT_FAST_SHAPES_BF16(X) X(8, 64) X(16, 64)
+
+inline bool fast_shape(int h, int d, int dtype) {
+    if (g_force_generic.load(std::memory_order_relaxed)) return false;
+#define X(HH, DD) if (h == HH && d == DD) return true;
+    if (dtype == BPT_F32) { BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return false;
+}
+
+constexpr int FAST_BATCH = 4;
+
+// ---- generic launchers (dtype dispatch) ----
+template <typename T, int MODE>
+int run_sddmm_generic(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_sddmm_generic<T, MODE>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)B, (T *)y, h, d);
+    return launch_status();
+}
+
+template <typename T, int MODE>
+int run_spmm_generic(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, hipStream_t s) {
+    using acc_t = typename Elem<T>::acc_t;
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_spmm_generic<T, MODE>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)W, (const T *)X, (T *)Y, (acc_t *)ws, h, d);
+    int st = launch_status();
+    if (st != BPT_OK || P->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const acc_t *)ws, (T *)Y, h * d);
+    return launch_status();
+}
+
+template <typename T>
+int run_softmax_fwd(const bpt_plan *P, const void *x, void *y, int h, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_softmax_fwd<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)x, (T *)y, h);
+    int st = launch_status();
+    if (st != BPT_OK || P->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_softmax_fwd<T, WAVES_PER_BLOCK>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, *P, (const T *)x, (T *)y, h);
+    return launch_status();
+}
+
+template <typename T>
+int run_softmax_bwd(const bpt_plan *P, const void *y, const void *dy, void *dx, int h, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_softmax_bwd<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)y, (const T *)dy, (T *)dx, h);
+    int st = launch_status();
+    if (st != BPT_OK || P->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_softmax_bwd<T, WAVES_PER_BLOCK>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, *P, (const T *)y, (const T *)dy, (T *)dx, h);
+    return launch_status();
+}
+
+template <typename T>
+int run_nme_dB(const bpt_plan *P, const void *A, const void *dy, void *dB, int h, int d, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_nme_dB_generic<T>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)dy, (T *)dB, h, d);
+    return launch_status();
+}
+
+#define DISPATCH_DTYPE(dtype, CALL)                     \
+    switch (dtype) {                                    \
+        case BPT_F32: { using T = float; return CALL; } \
+        case BPT_F64: { using T = double; return CALL; }\
+        case BPT_BF16: { using T = bf16_t; return CALL; }\
+        default: return BPT_ERR_DTYPE;                  \
+    }
+
+int sddmm_generic(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s) {
+    DISPATCH_DTYPE(dtype, (run_sddmm_generic<T, 0>(P, A, B, y, h, d, s)))
+}
+int sddmm_edge_generic(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s) {
+    DISPATCH_DTYPE(dtype, (run_sddmm_generic<T, 1>(P, A, B, y, h, d, s)))
+}
+int spmm_generic(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, int dtype, hipStream_t s) {
+    DISPATCH_DTYPE(dtype, (run_spmm_generic<T, 0>(P, W, X, Y, ws, h, d, s)))
+}
+int spmm_edge_generic(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, int dtype, hipStream_t s) {
+    DISPATCH_DTYPE(dtype, (run_spmm_generic<T, 1>(P, W, X, Y, ws, h, d, s)))
+}
+
+// ---- fast launchers ----
+template <typename T, int H, int D>
+int run_sddmm_fast(const bpt_plan *P, const void *A, const void *B, void *y, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_sddmm_fast<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)B, (T *)y);
+    return launch_status();
+}
+
+template <typename T, typename WT, int H, int D, int NOUT>
+int run_spmm_fast(const bpt_plan *P, const void *W0, const void *X0, void *Y0, const void *W1, const void *X1, void *Y1,
+                  float *ws, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    float *ws1 = ws ? ws + (size_t)P->n_slots * H * D : nullptr;
+    hipLaunchKernelGGL((k_spmm_fast<T, WT, H, D, FAST_BATCH, NOUT>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const WT *)W0,
+                       (const T *)X0, (T *)Y0, (const WT *)W1, (const T *)X1, (T *)Y1, ws, ws1);
+    int st = launch_status();
+    if (st != BPT_OK || P->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const float *)ws, (T *)Y0, H * D);
+    st = launch_status();
+    if (st != BPT_OK || NOUT == 1) return st;
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const float *)ws1, (T *)Y1, H * D);
+    return launch_status();
+}
+
+int sddmm_fast(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s) {
+#define X(HH, DD) if (h == HH && d == DD) return run_sddmm_fast<T, HH, DD>(P, A, B, y, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
+int spmm_fast(const bpt_plan *P, const void *W, const void *Xp, void *Y, void *ws, int h, int d, int dtype, hipStream_t s) {
+#define X(HH, DD) if (h == HH && d == DD) return run_spmm_fast<T, T, HH, DD, 1>(P, W, Xp, Y, nullptr, nullptr, nullptr, (float *)ws, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
+// SDDMM / SpMM with automatic family choice
+int sddmm(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s) {
+    if (fast_shape(h, d, dtype) && aligned16(A) && aligned16(B)) return sddmm_fast(P, A, B, y, h, d, dtype, s);
+    return sddmm_generic(P, A, B, y, h, d, dtype, s);
+}
+int spmm(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, int dtype, hipStream_t s) {
+    if (fast_shape(h, d, dtype) && aligned16(X) && aligned16(Y) && aligned16(ws)) return spmm_fast(P, W, X, Y, ws, h, d, dtype, s);
+    return spmm_generic(P, W, X, Y, ws, h, d, dtype, s);
+}
+
+inline int64_t round16(int64_t b) { return (b + 15) & ~(int64_t)15; }
+
+template <typename T, int H, int D>
+int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v, void *o, float *lse, void *ws, float scale, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    float *ws_acc = (float *)ws;
+    float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
+    hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
+                       (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+    int st = launch_status();
+    if (st != BPT_OK || P->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_attn_fwd_combine<T, H, D>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const float *)ws_acc,
+                       (const float *)ws_ml, (T *)o, lse);
+    return launch_status();
+}
+
+template <typename T, int H, int D>
+int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
+                 const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
+    if (Pin->n_items == 0) return BPT_OK;
+    const size_t EH = (size_t)Pin->n_edges * H;
+    float *pbuf = (float *)ws;
+    float *dsbuf = pbuf + round16((int64_t)EH * 4) / 4;
+    float *ws_rows = dsbuf + round16((int64_t)EH * 4) / 4;
+    hipLaunchKernelGGL((k_attn_bwd_dst<T, H, D, FAST_BATCH>), dim3(grid_for(Pin)), dim3(BLOCK), 0, s, *Pin, (const T *)q, (const T *)k,
+                       (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pbuf, dsbuf, ws_rows, scale, scale * LOG2E);
+    int st = launch_status();
+    if (st != BPT_OK) return st;
+    if (Pin->n_heavy > 0) {
+        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy), dim3(BLOCK), 0, s, Pin->heavy, (const float *)ws_rows, (T *)dq, H * D);
+        st = launch_status();
+        if (st != BPT_OK) return st;
+    }
+    // source side: dK[src] = sum ds * q[dst], dV[src] = sum p * dO[dst]
+    return run_spmm_fast<T, float, H, D, 2>(Pout, dsbuf, q, dk, pbuf, d_o, dv, ws_rows, s);
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------------
+extern "C" {
+
+const char *bpt_strerror(int status) {
+    if (status > 0) return hipGetErrorString((hipError_t)status);
+    switch (status) {
+        case BPT_OK: return "ok";
+        case BPT_ERR_NULL: return "required pointer is NULL";
+        case BPT_ERR_SIZE: return "negative or inconsistent size";
+        case BPT_ERR_DTYPE: return "unknown dtype";
+        case BPT_ERR_SHAPE: return "h and d must be positive (h*d <= 2^20)";
+        case BPT_ERR_WORKSPACE: return "workspace missing or too small";
+        case BPT_ERR_PLAN: return "plans do not describe the same graph";
+        case BPT_ERR_UNSUPPORTED: return "combination not implemented";
+        default: return "unknown bptattn status";
+    }
+}
+
+int bpt_set_force_generic(int on) { return g_force_generic.exchange(on ? 1 : 0); }
+
+int64_t bpt_workspace_bytes(int op, const bpt_plan *plan, const bpt_plan *plan_t, int h, int d, int dtype) {
+    if (!plan || h < 1 || d < 1) return -1;
+    const int64_t C = (int64_t)h * d, a = (int64_t)acc_size(dtype);
+    const int64_t s0 = plan->n_slots, s1 = plan_t ? plan_t->n_slots : 0;
+    switch (op) {
+        case BPT_OP_MASKEDMM_BWD: return round16((s0 > s1 ? s0 : s1) * C * a);
+        case BPT_OP_NODE_MUL_EDGE_BWD:
+        case BPT_OP_SPMM_FWD: return round16(s0 * C * a);
+        case BPT_OP_SPMM_BWD: return round16(s1 * C * a);
+        case BPT_OP_ATTN_FWD: return round16(s0 * (C + 2 * h) * 4);
+        case BPT_OP_ATTN_BWD: {
+            const int64_t rows = s0 > 2 * s1 ? s0 : 2 * s1;
+            return 2 * round16(plan->n_edges * h * 4) + round16(rows * C * 4);
+        }
+        default: return -1;
+    }
+}
+
+#define CHECK(expr) do { const int st_ = (expr); if (st_ != BPT_OK) return st_; } while (0)
+
+int bpt_maskedmm_csr_forward(const bpt_plan *plan, const void *A, const void *B, void *y, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan, true));
+    CHECK(check_shape(h, d, dtype));
+    if (plan->n_edges > 0 && (!A || !B || !y)) return BPT_ERR_NULL;
+    return sddmm(plan, A, B, y, h, d, dtype, (hipStream_t)stream);
+}
+
+int bpt_maskedmm_csr_backward(const bpt_plan *plan_r, const bpt_plan *plan_c, const void *A, const void *B, const void *dy,
+                              void *dA, void *dB, void *workspace, int64_t workspace_bytes, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan_r, true));
+    CHECK(check_plan(plan_c, true));
+    CHECK(check_shape(h, d, dtype));
+    if (plan_r->n_edges != plan_c->n_edges) return BPT_ERR_PLAN;
+    if (!dA || !dB || (plan_r->n_edges > 0 && (!A || !B || !dy))) return BPT_ERR_NULL;
+    const int64_t need = bpt_workspace_bytes(BPT_OP_MASKEDMM_BWD, plan_r, plan_c, h, d, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    CHECK(spmm(plan_r, dy, B, dA, workspace, h, d, dtype, (hipStream_t)stream));
+    return spmm(plan_c, dy, A, dB, workspace, h, d, dtype, (hipStream_t)stream);
+}
+
+int bpt_node_mul_edge_forward(const bpt_plan *plan, const void *A, const void *B, void *y, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan, false));
+    CHECK(check_shape(h, d, dtype));
+    if (plan->n_edges > 0 && (!A || !B || !y)) return BPT_ERR_NULL;
+    return sddmm_edge_generic(plan, A, B, y, h, d, dtype, (hipStream_t)stream);
+}
+
+int bpt_node_mul_edge_backward(const bpt_plan *plan, const void *A, const void *B, const void *dy, void *dA, void *dB,
+                               void *workspace, int64_t workspace_bytes, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan, false));
+    CHECK(check_shape(h, d, dtype));
+    if (!dA || (plan->n_edges > 0 && (!A || !B || !dy || !dB))) return BPT_ERR_NULL;
+    const int64_t need = bpt_workspace_bytes(BPT_OP_NODE_MUL_EDGE_BWD, plan, nullptr, h, d, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    CHECK(spmm_edge_generic(plan, dy, B, dA, workspace, h, d, dtype, (hipStream_t)stream));
+    DISPATCH_DTYPE(dtype, (run_nme_dB<T>(plan, A, dy, dB, h, d, (hipStream_t)stream)))
+}
+
+int bpt_sparse_softmax_forward(const bpt_plan *plan, const void *x, void *y, int h, int dtype, void *stream) {
+    CHECK(check_plan(plan, false));
+    CHECK(check_shape(h, 1, dtype));
+    if (plan->n_edges > 0 && (!x || !y)) return BPT_ERR_NULL;
+    DISPATCH_DTYPE(dtype, (run_softmax_fwd<T>(plan, x, y, h, (hipStream_t)stream)))
+}
+
+int bpt_sparse_softmax_backward(const bpt_plan *plan, const void *y, const void *dy, void *dx, int h, int dtype, void *stream) {
+    CHECK(check_plan(plan, false));
+    CHECK(check_shape(h, 1, dtype));
+    if (plan->n_edges > 0 && (!y || !dy || !dx)) return BPT_ERR_NULL;
+    DISPATCH_DTYPE(dtype, (run_softmax_bwd<T>(plan, y, dy, dx, h, (hipStream_t)stream)))
+}
+
+int bpt_vector_spmm_forward(const bpt_plan *plan, const void *edata, const void *x, void *y, void *workspace,
+                            int64_t workspace_bytes, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan, true));
+    CHECK(check_shape(h, d, dtype));
+    if (!y || (plan->n_edges > 0 && (!edata || !x))) return BPT_ERR_NULL;
+    const int64_t need = bpt_workspace_bytes(BPT_OP_SPMM_FWD, plan, nullptr, h, d, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    return spmm(plan, edata, x, y, workspace, h, d, dtype, (hipStream_t)stream);
+}
+
+int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const void *edata, const void *dy, const void *x,
+                             void *dedata, void *dx, void *workspace, int64_t workspace_bytes, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan, true));
+    CHECK(check_plan(plan_t, true));
+    CHECK(check_shape(h, d, dtype));
+    if (plan->n_edges != plan_t->n_edges) return BPT_ERR_PLAN;
+    if (!dx || (plan->n_edges > 0 && (!edata || !dy || !x || !dedata))) return BPT_ERR_NULL;
+    const int64_t need = bpt_workspace_bytes(BPT_OP_SPMM_BWD, plan, plan_t, h, d, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    CHECK(sddmm(plan, dy, x, dedata, h, d, dtype, (hipStream_t)stream));
+    return spmm(plan_t, edata, dy, dx, workspace, h, d, dtype, (hipStream_t)stream);
+}
+
+int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v, void *o, float *lse,
+                          void *workspace, int64_t workspace_bytes, float scale, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan_in, true));
+    CHECK(check_shape(h, d, dtype));
+    if (!q || !k || !v || !o || !lse) return BPT_ERR_NULL;
+    if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(workspace))
+        return BPT_ERR_UNSUPPORTED;
+    const int64_t need = bpt_workspace_bytes(BPT_OP_ATTN_FWD, plan_in, nullptr, h, d, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+#define X(HH, DD) if (h == HH && d == DD) return run_attn_fwd<T, HH, DD>(plan_in, q, k, v, o, lse, workspace, scale, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
+int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, const void *q, const void *k, const void *v,
+                           const void *o, const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *workspace,
+                           int64_t workspace_bytes, float scale, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan_in, true));
+    CHECK(check_plan(plan_out, true));
+    CHECK(check_shape(h, d, dtype));
+    if (plan_in->n_edges != plan_out->n_edges || plan_in->n_rows != plan_out->n_rows) return BPT_ERR_PLAN;
+    if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return BPT_ERR_NULL;
+    if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) ||
+        !aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !aligned16(workspace))
+        return BPT_ERR_UNSUPPORTED;
+    const int64_t need = bpt_workspace_bytes(BPT_OP_ATTN_BWD, plan_in, plan_out, h, d, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+#define X(HH, DD) \
+    if (h == HH && d == DD) return run_attn_bwd<T, HH, DD>(plan_in, plan_out, q, k, v, o, d_o, lse, dq, dk, dv, workspace, scale, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
+}  // extern "C"

@@ -1,0 +1,343 @@
+// libbptgraph: host-side integer half of the BPT graph-attention path (see include/bptgraph.h).
+//
+// Graph generators reproduce the edge ORDER of the reference bit for bit because edge ids are
+// positions in that order (graph/lm.py:96-98) and every (E, .) tensor on the device is addressed
+// by edge id.  Generators are written against a sink so the same walk first counts and then
+// writes straight into caller-owned int64 arrays (no intermediate vectors, no allocation).
+#include "../../include/bptgraph.h"
+
+#include <algorithm>
+#include <climits>
+#include <cstring>
+#include <vector>
+
+namespace {
+
+struct CountSink {
+    int64_t n = 0;
+    inline void operator()(int64_t, int64_t, int64_t) { ++n; }
+};
+
+struct WriteSink {
+    int64_t *src, *dst, *etype;
+    int64_t shift;
+    int64_t n = 0;
+    inline void operator()(int64_t s, int64_t d, int64_t t) {
+        if (src) src[n] = s + shift;
+        if (dst) dst[n] = d + shift;
+        if (etype) etype[n] = t;
+        ++n;
+    }
+};
+
+// Level table of the binary partition tree: level 0 = tokens, each next level halves (rounding
+// up) until a single root remains (builder.pyx:43-57).
+struct Levels {
+    std::vector<int64_t> size, offset;
+    int64_t n_nodes = 0;
+    explicit Levels(int64_t length) {
+        int64_t n = length;
+        while (n >= 2) {
+            size.push_back(n);
+            offset.push_back(n_nodes);
+            n_nodes += n;
+            n = (n + 1) >> 1;
+        }
+        size.push_back(1);
+        offset.push_back(n_nodes);
+        n_nodes += 1;
+    }
+    int64_t count() const { return (int64_t)size.size(); }
+};
+
+// builder.pyx:64-116.  For token `tok` two cursors walk outwards, `step` nodes per side per
+// level, then move one level up.  When a cursor stops on a node whose sibling was already
+// taken, the parent would overlap it, so the first neighbour on the next level is that child
+// itself (taken from the level below).  The right-hand bound is checked against the CURRENT
+// level even in that case — for odd level sizes this yields the first node of the current level
+// instead of a child; kept, since edge lists must match the reference exactly.
+template <class Sink>
+void walk_binary_partition(const Levels &lv, int64_t length, bool causal, int64_t step, int64_t clip, Sink &out) {
+    const int64_t n_lvl = lv.count();
+    for (int64_t tok = 0; tok < length; ++tok) {
+        int64_t left = tok - 1, right = tok + 1, ancestor = tok;
+        bool left_child = false, right_child = false;
+        for (int64_t j = 0; j < n_lvl; ++j) {
+            const int64_t type0 = (2 * step + 1) * std::min(j, clip);
+            for (int64_t s = 0; s < step; ++s) {
+                if (!causal && right < lv.size[j]) {
+                    out(right_child ? lv.offset[j - 1] + 2 * right + 1 : lv.offset[j] + right, tok, type0 + 2 * (s + 1));
+                    right_child = false;
+                }
+                ++right;
+                if (left >= 0) {
+                    out(left_child ? lv.offset[j - 1] + 2 * left : lv.offset[j] + left, tok, type0 + 2 * s + 1);
+                    left_child = false;
+                }
+                --left;
+            }
+            if ((left & 1) == 0) left_child = true;
+            if ((right & 1) == 1) right_child = true;
+            right >>= 1;
+            left >>= 1;                       // arithmetic shift: stays negative once it is
+            out(tok, lv.offset[j] + ancestor, type0);   // self loop (j = 0) / token -> ancestor
+            ancestor >>= 1;
+        }
+    }
+}
+
+// builder.pyx:243-274
+template <class Sink>
+void walk_fully_connected(int64_t length, bool causal, int64_t window, Sink &out) {
+    const int64_t reach = std::min(length, window + 1);
+    for (int64_t i = 0; i < length; ++i) {
+        out(i, i, 0);
+        for (int64_t j = 1; j < reach; ++j) {
+            if (i >= j) out(i - j, i, 2 * j - 1);
+            if (!causal && i + j < length) out(i + j, i, 2 * j);
+        }
+        out(i, length, 0);
+    }
+}
+
+// builder.pyx:171-199
+template <class Sink>
+void walk_openai_sparse(int64_t length, int64_t stride, int64_t c, Sink &out) {
+    for (int64_t i = 0; i < length; ++i) {
+        for (int64_t j = (i / stride) * stride; j <= i; ++j) out(j, i, 0);
+        for (int64_t blk = 1; blk <= i / stride; ++blk)
+            for (int64_t k = stride * blk - c; k < stride * blk; ++k) out(k, i, 0);
+        out(i, length, 0);
+    }
+}
+
+bool graph_args_ok(int kind, int64_t length, int64_t a, int64_t b) {
+    if (length < 1) return false;
+    if (kind == 0) return a >= 1 && b >= 0;
+    if (kind == 1) return a >= 0;
+    if (kind == 2) return a >= 1 && b >= 0 && b <= a;
+    return false;
+}
+
+template <class Sink>
+void walk(int kind, int64_t length, int triu, int64_t a, int64_t b, Sink &sink) {
+    if (kind == 0) {
+        Levels lv(length);
+        walk_binary_partition(lv, length, triu != 0, a, b, sink);
+    } else if (kind == 1) {
+        walk_fully_connected(length, triu != 0, a, sink);
+    } else {
+        walk_openai_sparse(length, a, b, sink);
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *bptg_strerror(int status) {
+    switch (status) {
+        case BPTG_OK: return "ok";
+        case BPTG_ERR_NULL: return "required pointer is NULL";
+        case BPTG_ERR_SIZE: return "negative, inconsistent or too large size";
+        case BPTG_ERR_ORDER: return "units must be grouped by row: `row` and `indptr` non-decreasing";
+        case BPTG_ERR_RANGE: return "row id, index or edge id out of range";
+        case BPTG_ERR_ARG: return "invalid scalar argument";
+        default: return "unknown bptgraph status";
+    }
+}
+
+int bptg_graph_sizes(int kind, int64_t length, int triu, int64_t a, int64_t b,
+                     int64_t *n_nodes, int64_t *n_edges, int64_t *n_levels) {
+    if (!n_nodes || !n_edges || !n_levels) return BPTG_ERR_NULL;
+    if (!graph_args_ok(kind, length, a, b)) return BPTG_ERR_ARG;
+    if (kind == 0) {
+        Levels lv(length);
+        *n_nodes = lv.n_nodes;
+        *n_levels = lv.count();
+    } else {
+        *n_nodes = length + 1;
+        *n_levels = 2;
+    }
+    CountSink cnt;
+    walk(kind, length, triu, a, b, cnt);
+    *n_edges = cnt.n;
+    return BPTG_OK;
+}
+
+int bptg_graph_fill(int kind, int64_t length, int triu, int64_t a, int64_t b, int64_t v_shift,
+                    int64_t *src, int64_t *dst, int64_t *etype, int64_t *pos, int64_t *lvl_sizes) {
+    if (!graph_args_ok(kind, length, a, b)) return BPTG_ERR_ARG;
+    if (src || dst || etype) {
+        WriteSink w{src, dst, etype, v_shift};
+        walk(kind, length, triu, a, b, w);
+    }
+    if (kind == 0) {
+        Levels lv(length);
+        if (lvl_sizes)
+            for (int64_t j = 0; j < lv.count(); ++j) lvl_sizes[j] = lv.size[j];
+        if (pos) {
+            // builder.pyx:46,57-62: last token covered by the node, clipped to the sequence
+            int64_t p = 0;
+            for (int64_t j = 0; j + 1 < lv.count(); ++j)
+                for (int64_t i = 0; i < lv.size[j]; ++i) pos[p++] = std::min(((i + 1) << j) - 1, length - 1);
+            pos[p] = length - 1;
+        }
+    } else {
+        if (lvl_sizes) { lvl_sizes[0] = length; lvl_sizes[1] = 1; }
+        if (pos) {
+            for (int64_t i = 0; i < length; ++i) pos[i] = i;
+            pos[length] = (kind == 1) ? length : length - 1;   // builder.pyx:274 / :199
+        }
+    }
+    return BPTG_OK;
+}
+
+int bptg_partition_csr_count(const int64_t *indptr, int64_t n_indptr, int64_t chunk_size, int64_t *n_units) {
+    if (!indptr || !n_units) return BPTG_ERR_NULL;
+    if (n_indptr < 1) return BPTG_ERR_SIZE;
+    if (chunk_size < 1) return BPTG_ERR_ARG;
+    int64_t n = 0;
+    for (int64_t r = 0; r + 1 < n_indptr; ++r) {
+        const int64_t deg = indptr[r + 1] - indptr[r];
+        if (deg < 0) return BPTG_ERR_ORDER;
+        n += (deg + chunk_size - 1) / chunk_size;
+    }
+    *n_units = n;
+    return BPTG_OK;
+}
+
+int bptg_partition_csr_fill(const int64_t *indptr, int64_t n_indptr, int64_t chunk_size,
+                            int64_t *row, int64_t *indptr_units) {
+    if (!indptr || !indptr_units) return BPTG_ERR_NULL;
+    if (n_indptr < 1) return BPTG_ERR_SIZE;
+    if (chunk_size < 1) return BPTG_ERR_ARG;
+    int64_t u = 0;
+    for (int64_t r = 0; r + 1 < n_indptr; ++r)
+        for (int64_t p = indptr[r]; p < indptr[r + 1]; p += chunk_size) {
+            if (!row) return BPTG_ERR_NULL;
+            row[u] = r;
+            indptr_units[u] = p;
+            ++u;
+        }
+    indptr_units[u] = indptr[n_indptr - 1];
+    return BPTG_OK;
+}
+
+int bptg_build_csr(const int64_t *rows, const int64_t *cols, int64_t n_edges, int64_t n_nodes,
+                   int64_t *indptr, int64_t *indices, int64_t *eid) {
+    if (!indptr || (n_edges > 0 && (!rows || !cols || !indices || !eid))) return BPTG_ERR_NULL;
+    if (n_edges < 0 || n_nodes < 0) return BPTG_ERR_SIZE;
+    std::memset(indptr, 0, sizeof(int64_t) * (size_t)(n_nodes + 1));
+    for (int64_t e = 0; e < n_edges; ++e) {
+        if (rows[e] < 0 || rows[e] >= n_nodes || cols[e] < 0 || cols[e] >= n_nodes) return BPTG_ERR_RANGE;
+        ++indptr[rows[e] + 1];
+    }
+    for (int64_t r = 0; r < n_nodes; ++r) indptr[r + 1] += indptr[r];
+    std::vector<int64_t> cursor(indptr, indptr + n_nodes);
+    for (int64_t e = 0; e < n_edges; ++e) {          // ascending e => ascending eid inside a row
+        const int64_t p = cursor[rows[e]]++;
+        indices[p] = cols[e];
+        eid[p] = e;
+    }
+    return BPTG_OK;
+}
+
+// ---- plan --------------------------------------------------------------------------------------
+
+static int plan_scan(const int64_t *row, const int64_t *ip, int64_t n_units, int64_t n_nodes, int64_t seg_len,
+                     int32_t *rowptr, int32_t *items, int32_t *heavy, bptg_plan_info *info) {
+    if (!info || (n_units > 0 && (!row || !ip))) return BPTG_ERR_NULL;
+    if (n_units < 0 || n_nodes < 0 || n_nodes >= INT32_MAX) return BPTG_ERR_SIZE;
+    if (seg_len < 1) return BPTG_ERR_ARG;
+    const int64_t first = n_units ? ip[0] : 0, last = n_units ? ip[n_units] : 0;
+    if (first < 0 || last >= INT32_MAX) return BPTG_ERR_SIZE;
+    for (int64_t u = 0; u < n_units; ++u) {
+        if (row[u] < 0 || row[u] >= n_nodes) return BPTG_ERR_RANGE;
+        if (u && row[u] < row[u - 1]) return BPTG_ERR_ORDER;
+        if (ip[u + 1] < ip[u]) return BPTG_ERR_ORDER;
+    }
+    int64_t n_items = 0, n_heavy = 0, n_slots = 0, max_deg = 0;
+    int64_t u = 0;
+    for (int64_t r = 0; r < n_nodes; ++r) {
+        const int64_t u0 = u;
+        while (u < n_units && row[u] == r) ++u;
+        const int64_t begin = (u0 < n_units) ? ip[u0] : last;
+        const int64_t end = (u > u0) ? ip[u] : begin;
+        const int64_t deg = end - begin;
+        max_deg = std::max(max_deg, deg);
+        if (rowptr) rowptr[r] = (int32_t)begin;
+        if (deg <= seg_len) {
+            if (items) {
+                int32_t *it = items + 4 * n_items;
+                it[0] = (int32_t)r; it[1] = (int32_t)begin; it[2] = (int32_t)end; it[3] = -1;
+            }
+            ++n_items;
+        } else {
+            const int64_t n_seg = (deg + seg_len - 1) / seg_len;
+            if (heavy) {
+                int32_t *hv = heavy + 3 * n_heavy;
+                hv[0] = (int32_t)r; hv[1] = (int32_t)n_slots; hv[2] = (int32_t)n_seg;
+            }
+            for (int64_t s = 0; s < n_seg; ++s) {
+                if (items) {
+                    int32_t *it = items + 4 * n_items;
+                    it[0] = (int32_t)r;
+                    it[1] = (int32_t)(begin + s * seg_len);
+                    it[2] = (int32_t)std::min(end, begin + (s + 1) * seg_len);
+                    it[3] = (int32_t)(n_slots + s);
+                }
+                ++n_items;
+            }
+            ++n_heavy;
+            n_slots += n_seg;
+        }
+    }
+    if (rowptr) rowptr[n_nodes] = (int32_t)last;
+    if (n_items >= INT32_MAX) return BPTG_ERR_SIZE;
+    info->n_items = n_items;
+    info->n_heavy = n_heavy;
+    info->n_slots = n_slots;
+    info->max_degree = max_deg;
+    info->flags = 0;
+    return BPTG_OK;
+}
+
+int bptg_plan_sizes(const int64_t *row, const int64_t *indptr_units, int64_t n_units,
+                    int64_t n_nodes, int64_t seg_len, bptg_plan_info *info) {
+    return plan_scan(row, indptr_units, n_units, n_nodes, seg_len, nullptr, nullptr, nullptr, info);
+}
+
+int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_units,
+                   const int64_t *eid, const int64_t *indices, int64_t n_edges,
+                   int64_t n_nodes, int64_t n_index_nodes, int64_t seg_len,
+                   int32_t *rowptr, int32_t *idx32, int32_t *eid32, int32_t *items, int32_t *heavy,
+                   bptg_plan_info *info) {
+    if (!rowptr || !items || (n_edges > 0 && (!eid || !idx32 || !eid32))) return BPTG_ERR_NULL;
+    if (n_edges < 0 || n_edges >= INT32_MAX || n_index_nodes < 0 || n_index_nodes >= INT32_MAX) return BPTG_ERR_SIZE;
+    int st = plan_scan(row, indptr_units, n_units, n_nodes, seg_len, rowptr, items, heavy, info);
+    if (st != BPTG_OK) return st;
+    if (info->n_heavy > 0 && !heavy) return BPTG_ERR_NULL;
+    // the units must address slots inside the eid / indices arrays
+    if (n_units > 0 && indptr_units[n_units] > n_edges) return BPTG_ERR_RANGE;
+    std::vector<uint8_t> seen((size_t)n_edges, 0);
+    bool perm = (n_units > 0) ? (indptr_units[0] == 0 && indptr_units[n_units] == n_edges) : (n_edges == 0);
+    for (int64_t p = 0; p < n_edges; ++p) {
+        const int64_t e = eid[p];
+        if (e < 0 || e >= n_edges) return BPTG_ERR_RANGE;
+        if (seen[(size_t)e]) perm = false;
+        seen[(size_t)e] = 1;
+        eid32[p] = (int32_t)e;
+        if (indices) {
+            const int64_t c = indices[p];
+            if (c < 0 || c >= n_index_nodes) return BPTG_ERR_RANGE;
+            idx32[p] = (int32_t)c;
+        } else {
+            idx32[p] = 0;
+        }
+    }
+    info->flags = perm ? 1 : 0;
+    return BPTG_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,166 @@
+"""Host graph builder with the API of the reference's Cython module `graphbuilder`
+(graph_builder/builder.pyx): `BinaryPartition`, `FullyConnected`, `OpenAISparse`, `partition_csr`,
+backed by libbptgraph (C++).  Arrays are numpy int64 exactly as `np.asarray(vector) + v_shift`
+yields there.  Also provides what graph/base.py:71-86 and graph/lm.py:53-98 obtain through DGL and
+scipy: `build_csr`, `get_csrs`, `merge_graphs`.
+"""
+import ctypes
+
+import numpy as np
+
+from ._lib import check_graph, graph_lib
+
+__all__ = ["BinaryPartition", "FullyConnected", "OpenAISparse", "partition_csr",
+           "build_csr", "get_csrs", "merge_graphs"]
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+class _Graph:
+    _kind = -1
+
+    def _init(self, length, triu, a, b):
+        lib = graph_lib()
+        self._length, self._triu, self._a, self._b = int(length), bool(triu), int(a), int(b)
+        n, e, lv = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+        check_graph(lib.bptg_graph_sizes(self._kind, self._length, int(self._triu), self._a, self._b,
+                                         ctypes.byref(n), ctypes.byref(e), ctypes.byref(lv)))
+        self._n_nodes, self._n_edges, self._n_lvl = n.value, e.value, lv.value
+        self._lvl_sizes = np.empty(self._n_lvl, dtype=np.int64)
+        check_graph(lib.bptg_graph_fill(self._kind, self._length, int(self._triu), self._a, self._b, 0,
+                                        None, None, None, None, _ptr(self._lvl_sizes)))
+
+    # builder.pyx:118-132
+    @property
+    def number_of_nodes(self):
+        return self._n_nodes
+
+    @property
+    def number_of_edges(self):
+        return self._n_edges
+
+    @property
+    def is_triu(self):
+        return self._triu
+
+    # builder.pyx:134
+    def get_pos(self):
+        pos = np.empty(self._n_nodes, dtype=np.int64)
+        check_graph(graph_lib().bptg_graph_fill(self._kind, self._length, int(self._triu), self._a, self._b, 0,
+                                                None, None, None, _ptr(pos), None))
+        return pos
+
+    # builder.pyx:137-140
+    def get_edges(self, v_shift=0):
+        src, dst, et = (np.empty(self._n_edges, dtype=np.int64) for _ in range(3))
+        check_graph(graph_lib().bptg_graph_fill(self._kind, self._length, int(self._triu), self._a, self._b, int(v_shift),
+                                                _ptr(src), _ptr(dst), _ptr(et), None, None))
+        return src, dst, et
+
+    # builder.pyx:142-149
+    def leaf_ids(self, v_shift=0, start=0):
+        return np.arange(v_shift + start, v_shift + self._length)
+
+    def internal_ids(self, v_shift=0):
+        return np.arange(v_shift + self._length, v_shift + self._n_nodes)
+
+    def root_id(self, v_shift=0):
+        return v_shift + self._n_nodes - 1
+
+
+class BinaryPartition(_Graph):
+    """builder.pyx:23-152."""
+    _kind = 0
+
+    def __init__(self, length, triu=False, step=1, clip_dist=10):
+        self._init(length, triu, step, clip_dist)
+
+    def __reduce__(self):
+        return BinaryPartition, (self._length, self._triu, self._a, self._b)
+
+    @property
+    def number_of_levels(self):
+        return self._n_lvl
+
+    def number_of_nodes_at_lvl(self, i):
+        return int(self._lvl_sizes[i])
+
+
+class FullyConnected(_Graph):
+    """builder.pyx:228-303."""
+    _kind = 1
+
+    def __init__(self, length, triu=False, window=8192):
+        self._init(length, triu, window, 0)
+
+    def __reduce__(self):
+        return FullyConnected, (self._length, self._triu, self._a)
+
+
+class OpenAISparse(_Graph):
+    """builder.pyx:154-225."""
+    _kind = 2
+
+    def __init__(self, length, stride, c, triu=True):
+        assert triu, "bidirectional model is not supported"
+        self._init(length, triu, stride, c)
+
+    def __reduce__(self):
+        return OpenAISparse, (self._length, self._a, self._b, self._triu)
+
+
+def partition_csr(indptr, chunk_size=32):
+    """builder.pyx:305-321: (row, indptr_) of the chunked units, int64 numpy."""
+    indptr = np.ascontiguousarray(indptr, dtype=np.int64)
+    lib = graph_lib()
+    n = ctypes.c_int64()
+    check_graph(lib.bptg_partition_csr_count(_ptr(indptr), len(indptr), int(chunk_size), ctypes.byref(n)))
+    row = np.empty(n.value, dtype=np.int64)
+    units = np.empty(n.value + 1, dtype=np.int64)
+    check_graph(lib.bptg_partition_csr_fill(_ptr(indptr), len(indptr), int(chunk_size), _ptr(row), _ptr(units)))
+    return row, units
+
+
+def build_csr(rows, cols, n_nodes):
+    """(indptr, indices, eid) of the edge list grouped by `rows`; ascending edge id inside a row."""
+    rows = np.ascontiguousarray(rows, dtype=np.int64)
+    cols = np.ascontiguousarray(cols, dtype=np.int64)
+    if rows.shape != cols.shape:
+        raise ValueError("rows and cols must have the same length")
+    indptr = np.empty(n_nodes + 1, dtype=np.int64)
+    indices = np.empty(len(rows), dtype=np.int64)
+    eid = np.empty(len(rows), dtype=np.int64)
+    check_graph(graph_lib().bptg_build_csr(_ptr(rows), _ptr(cols), len(rows), int(n_nodes),
+                                           _ptr(indptr), _ptr(indices), _ptr(eid)))
+    return indptr, indices, eid
+
+
+def get_csrs(src, dst, n_nodes, chunk_size=32, as_torch=True):
+    """Replacement of graph/base.py:71-86 without DGL: returns
+    (out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C) with csr = (indptr, indices, eid), all int64
+    (torch CPU tensors by default, numpy with as_torch=False)."""
+    out_csr = build_csr(src, dst, n_nodes)
+    in_csr = build_csr(dst, src, n_nodes)
+    ROW, INDPTR_R = partition_csr(out_csr[0], chunk_size)
+    COL, INDPTR_C = partition_csr(in_csr[0], chunk_size)
+    res = (out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C)
+    if as_torch:
+        import torch
+        t = torch.from_numpy
+        res = (tuple(map(t, out_csr)), tuple(map(t, in_csr)), t(ROW), t(INDPTR_R), t(COL), t(INDPTR_C))
+    return res
+
+
+def merge_graphs(graphs):
+    """Block-diagonal batch merge of graph/lm.py:53-98 / graph/text_classification.py:30-67:
+    returns (src, dst, etype, pos, n_nodes); the edge id of an edge is its position."""
+    v_shift = 0
+    src, dst, et, pos = [], [], [], []
+    for g in graphs:
+        s, d, e = g.get_edges(v_shift=v_shift)
+        src.append(s); dst.append(d); et.append(e); pos.append(g.get_pos())
+        v_shift += g.number_of_nodes
+    cat = np.concatenate
+    return cat(src), cat(dst), cat(et), cat(pos), v_shift

@@ -1,0 +1,261 @@
+"""The `graphop` operator surface of the reference (graph_kernel/graphop.cpp:216-225) on MI355X.
+
+Same eight names, positional argument orders and return arities as the pybind module that
+modules/op.py imports with `from graphop import *`; each call validates its tensors like the
+reference shim (graphop.cpp:4-6: CUDA + contiguous), looks up the launch plan of its index
+tensors and enqueues HIP kernels from libbptattn on the current stream.  Nothing here computes on
+the CPU; without the built HIP library the import fails.
+
+Beyond the reference: bf16 tensors are accepted, `attention_forward/backward` expose the fused
+SDDMM -> edge-softmax -> SpMM pass, and vector_spmm_backward returns the complete dx (the
+reference's launch drops trailing units of the transposed side, graphop_kernel.cu:566,588).
+"""
+import ctypes
+import math
+
+import torch
+
+from ._lib import attn_lib, check_attn
+from .plan import plan_cache
+
+__all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forward", "node_mul_edge_backward",
+           "sparse_softmax_forward", "sparse_softmax_backward", "vector_spmm_forward", "vector_spmm_backward"]
+
+_LIB = attn_lib()          # fail at import time if the HIP library is missing
+
+_DTYPE = {torch.float32: 0, torch.float64: 1, torch.bfloat16: 2}
+OP_MASKEDMM_BWD, OP_NME_BWD, OP_SPMM_FWD, OP_SPMM_BWD, OP_ATTN_FWD, OP_ATTN_BWD = 1, 2, 3, 4, 5, 6
+
+
+def _check_input(t, name):
+    # graphop.cpp:4-6
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _check_all(**tensors):
+    for name, t in tensors.items():
+        _check_input(t, name)
+
+
+def _dtype(t):
+    try:
+        return _DTYPE[t.dtype]
+    except KeyError:
+        raise RuntimeError(f"unsupported dtype {t.dtype}: float32, float64 and bfloat16 are implemented") from None
+
+
+def _hd(A):
+    # graphop_kernel.cu:245-247: (n, d) means a single head
+    if A.dim() == 2:
+        return 1, A.size(1)
+    if A.dim() == 3:
+        return A.size(1), A.size(2)
+    raise RuntimeError("node tensors must be (n, d) or (n, h, d)")
+
+
+def _edge_h(x):
+    return 1 if x.dim() == 1 else x.size(1)
+
+
+def _same_dtype(*ts):
+    for t in ts[1:]:
+        if t.dtype != ts[0].dtype:
+            raise RuntimeError("all floating point arguments must share one dtype")
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() else None
+
+
+def _workspace(op, plan, plan_t, h, d, dt, device):
+    n = _LIB.bpt_workspace_bytes(op, plan.ref, plan_t.ref if plan_t is not None else None, h, d, dt)
+    if n < 0:
+        raise RuntimeError("bpt_workspace_bytes failed")
+    if n == 0:
+        return None, 0
+    return torch.empty(n, dtype=torch.uint8, device=device), n
+
+
+def _edge_out(plan, shape, like):
+    # kernels write every edge id the plan covers; zero-fill only when some edge is not covered
+    return (torch.empty if plan.covers_all_edges else torch.zeros)(shape, dtype=like.dtype, device=like.device)
+
+
+def maskedmm_csr_forward(row, indptr, eid, indices, A, B):
+    """y[eid[p]] = <A[row], B[indices[p]]> per head (graphop.cpp:16-31, graphop_kernel.cu:269-304)."""
+    _check_all(row=row, indptr=indptr, eid=eid, indices=indices, A=A, B=B)
+    _same_dtype(A, B)
+    h, d = _hd(A)
+    plan = plan_cache.get(row, indptr, eid, indices, A.size(0), B.size(0))
+    e = eid.size(0)
+    y = _edge_out(plan, (e,) if A.dim() == 2 else (e, h), A)
+    with torch.cuda.device_of(A):
+        check_attn(_LIB.bpt_maskedmm_csr_forward(plan.ref, _ptr(A), _ptr(B), _ptr(y), h, d, _dtype(A), _stream()),
+                   "maskedmm_csr_forward")
+    return y
+
+
+def maskedmm_csr_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, A, B, dy):
+    """[dA, dB] (graphop.cpp:108-139, graphop_kernel.cu:355-409)."""
+    _check_all(row=row, indptr_r=indptr_r, eid_r=eid_r, indices_r=indices_r, col=col, indptr_c=indptr_c,
+               eid_c=eid_c, indices_c=indices_c, A=A, B=B)
+    dy = dy.contiguous()
+    _same_dtype(A, B, dy)
+    h, d = _hd(A)
+    plan_r = plan_cache.get(row, indptr_r, eid_r, indices_r, A.size(0), B.size(0))
+    plan_c = plan_cache.get(col, indptr_c, eid_c, indices_c, B.size(0), A.size(0))
+    dA, dB = torch.empty_like(A), torch.empty_like(B)
+    dt = _dtype(A)
+    ws, nws = _workspace(OP_MASKEDMM_BWD, plan_r, plan_c, h, d, dt, A.device)
+    with torch.cuda.device_of(A):
+        check_attn(_LIB.bpt_maskedmm_csr_backward(plan_r.ref, plan_c.ref, _ptr(A), _ptr(B), _ptr(dy), _ptr(dA), _ptr(dB),
+                                                  _ptr(ws), nws, h, d, dt, _stream()), "maskedmm_csr_backward")
+    return [dA, dB]
+
+
+def node_mul_edge_forward(row, indptr, eid, A, B):
+    """y[eid[p], h] = <A[row, h], B[eid[p]]> with B (e, d) (graphop.cpp:39-51, graphop_kernel.cu:235-266)."""
+    _check_all(row=row, indptr=indptr, eid=eid, A=A, B=B)
+    _same_dtype(A, B)
+    h, d = _hd(A)
+    plan = plan_cache.get(row, indptr, eid, None, A.size(0), None)
+    e = eid.size(0)
+    y = _edge_out(plan, (e,) if A.dim() == 2 else (e, h), A)
+    with torch.cuda.device_of(A):
+        check_attn(_LIB.bpt_node_mul_edge_forward(plan.ref, _ptr(A), _ptr(B), _ptr(y), h, d, _dtype(A), _stream()),
+                   "node_mul_edge_forward")
+    return y
+
+
+def node_mul_edge_backward(row, indptr, eid, A, B, dy):
+    """[dA, dB] (graphop.cpp:141-155, graphop_kernel.cu:306-351)."""
+    _check_all(row=row, indptr=indptr, eid=eid, A=A, B=B)
+    dy = dy.contiguous()
+    _same_dtype(A, B, dy)
+    h, d = _hd(A)
+    plan = plan_cache.get(row, indptr, eid, None, A.size(0), None)
+    dA = torch.empty_like(A)
+    dB = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(B)
+    dt = _dtype(A)
+    ws, nws = _workspace(OP_NME_BWD, plan, None, h, d, dt, A.device)
+    with torch.cuda.device_of(A):
+        check_attn(_LIB.bpt_node_mul_edge_backward(plan.ref, _ptr(A), _ptr(B), _ptr(dy), _ptr(dA), _ptr(dB),
+                                                   _ptr(ws), nws, h, d, dt, _stream()), "node_mul_edge_backward")
+    return [dA, dB]
+
+
+def sparse_softmax_forward(row, indptr, eid, x):
+    """softmax of x over the slots of each row (graphop.cpp:59-71, graphop_kernel.cu:411-463)."""
+    _check_all(row=row, indptr=indptr, eid=eid, x=x)
+    plan = plan_cache.get(row, indptr, eid, None, None, None)
+    y = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(x)
+    with torch.cuda.device_of(x):
+        check_attn(_LIB.bpt_sparse_softmax_forward(plan.ref, _ptr(x), _ptr(y), _edge_h(x), _dtype(x), _stream()),
+                   "sparse_softmax_forward")
+    return y
+
+
+def sparse_softmax_backward(row, indptr, eid, y, dy):
+    """dx = y * (dy - sum_row dy*y) (graphop.cpp:163-177, graphop_kernel.cu:465-507)."""
+    _check_all(row=row, indptr=indptr, eid=eid, y=y, dy=dy)
+    _same_dtype(y, dy)
+    plan = plan_cache.get(row, indptr, eid, None, None, None)
+    dx = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(dy)
+    with torch.cuda.device_of(y):
+        check_attn(_LIB.bpt_sparse_softmax_backward(plan.ref, _ptr(y), _ptr(dy), _ptr(dx), _edge_h(dy), _dtype(y), _stream()),
+                   "sparse_softmax_backward")
+    return dx
+
+
+def vector_spmm_forward(row, indptr, eid, indices, edata, x):
+    """y[row] = sum_p edata[eid[p]] * x[indices[p]] (graphop.cpp:79-95, graphop_kernel.cu:509-542)."""
+    _check_all(row=row, indptr=indptr, eid=eid, indices=indices, edata=edata, x=x)
+    _same_dtype(edata, x)
+    h, d = _hd(x)
+    if _edge_h(edata) != h:
+        raise RuntimeError("edata and x disagree on the number of heads")
+    plan = plan_cache.get(row, indptr, eid, indices, x.size(0), x.size(0))
+    y = torch.empty_like(x)
+    dt = _dtype(x)
+    ws, nws = _workspace(OP_SPMM_FWD, plan, None, h, d, dt, x.device)
+    with torch.cuda.device_of(x):
+        check_attn(_LIB.bpt_vector_spmm_forward(plan.ref, _ptr(edata), _ptr(x), _ptr(y), _ptr(ws), nws, h, d, dt, _stream()),
+                   "vector_spmm_forward")
+    return y
+
+
+def vector_spmm_backward(row, indptr, eid, indices, col, indptr_t, eid_t, indices_t, edata, dy, x):
+    """[dedata, dx] (graphop.cpp:190-214, graphop_kernel.cu:544-600; dx over all units of the transposed side)."""
+    _check_all(row=row, indptr=indptr, eid=eid, indices=indices, col=col, indptr_t=indptr_t, eid_t=eid_t,
+               indices_t=indices_t, edata=edata, x=x)
+    dy = dy.contiguous()
+    _same_dtype(edata, dy, x)
+    h, d = _hd(x)
+    plan = plan_cache.get(row, indptr, eid, indices, x.size(0), x.size(0))
+    plan_t = plan_cache.get(col, indptr_t, eid_t, indices_t, x.size(0), x.size(0))
+    dedata = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(edata)
+    dx = torch.empty_like(x)
+    dt = _dtype(x)
+    ws, nws = _workspace(OP_SPMM_BWD, plan, plan_t, h, d, dt, x.device)
+    with torch.cuda.device_of(x):
+        check_attn(_LIB.bpt_vector_spmm_backward(plan.ref, plan_t.ref, _ptr(edata), _ptr(dy), _ptr(x), _ptr(dedata), _ptr(dx),
+                                                 _ptr(ws), nws, h, d, dt, _stream()), "vector_spmm_backward")
+    return [dedata, dx]
+
+
+# ---- fused attention (no counterpart in the reference's extension) ---------------------------
+def attention_supported(q):
+    """True if the fused kernels have an instantiation for q's (h, d, dtype)."""
+    h, d = _hd(q)
+    fast = {torch.float32: {(4, 64), (8, 64), (16, 64), (8, 32)}, torch.bfloat16: {(8, 64), (16, 64)}}
+    return q.dim() == 3 and (h, d) in fast.get(q.dtype, ())
+
+
+def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None):
+    """o[dst] = sum over in-edges softmax(q[dst].k[src]*scale) v[src]; returns (o, lse) with lse (n, h) float32
+    in base-2 units.  Arithmetic of modules/attention.py:66-77 (no dropout, no rel-pos) in one pass."""
+    _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v)
+    _same_dtype(q, k, v)
+    h, d = _hd(q)
+    scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
+    plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
+    o = torch.empty_like(q)
+    lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
+    dt = _dtype(q)
+    ws, nws = _workspace(OP_ATTN_FWD, plan, None, h, d, dt, q.device)
+    with torch.cuda.device_of(q):
+        check_attn(_LIB.bpt_attention_forward(plan.ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws), nws,
+                                              scale, h, d, dt, _stream()), "attention_forward")
+    return o, lse
+
+
+def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, do, scale=None):
+    """(dq, dk, dv) of attention_forward."""
+    _check_all(row=row, indptr_r=indptr_r, eid_r=eid_r, indices_r=indices_r, col=col, indptr_c=indptr_c,
+               eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v, o=o, lse=lse)
+    do = do.contiguous()
+    _same_dtype(q, k, v, o, do)
+    h, d = _hd(q)
+    scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
+    plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
+    plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0))
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dt = _dtype(q)
+    ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device)
+    with torch.cuda.device_of(q):
+        check_attn(_LIB.bpt_attention_backward(plan_in.ref, plan_out.ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do),
+                                               _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
+                                               scale, h, d, dt, _stream()), "attention_backward")
+    return dq, dk, dv
+
+
+def set_force_generic(on):
+    """Testing hook: route every op through the shape-generic kernels."""
+    return bool(_LIB.bpt_set_force_generic(1 if on else 0))

@@ -1,0 +1,125 @@
+"""Autograd operators with the surface of the reference's modules/op.py:10-70 (same Function
+names, argument orders, saved tensors and `None` gradient slots), running on the HIP kernels,
+plus `bpt_attention`, the fused layer core.
+"""
+import math
+
+import torch
+from torch.autograd import Function
+
+from . import graphop as _g
+from .graphop import (maskedmm_csr_backward, maskedmm_csr_forward, node_mul_edge_backward, node_mul_edge_forward,
+                      sparse_softmax_backward, sparse_softmax_forward, vector_spmm_backward, vector_spmm_forward)
+
+__all__ = ["SparseSoftmax", "MaskedMMCSR", "NodeMulEdge", "VectorSPMM", "BPTAttention",
+           "sparse_softmax", "masked_mm", "node_mul_edge", "vec_spmm", "bpt_attention"]
+
+
+class SparseSoftmax(Function):
+    # modules/op.py:10-20
+    @staticmethod
+    def forward(ctx, row, indptr, eid, x):
+        y = sparse_softmax_forward(row, indptr, eid, x)
+        ctx.save_for_backward(row, indptr, eid, y)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        row, indptr, eid, y = ctx.saved_tensors
+        return None, None, None, sparse_softmax_backward(row, indptr, eid, y, dy.contiguous())
+
+
+class MaskedMMCSR(Function):
+    # modules/op.py:23-33
+    @staticmethod
+    def forward(ctx, row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, A, B):
+        ctx.save_for_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, A, B)
+        return maskedmm_csr_forward(row, indptr_r, eid_r, indices_r, A, B)
+
+    @staticmethod
+    def backward(ctx, grad):
+        row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, A, B = ctx.saved_tensors
+        dA, dB = maskedmm_csr_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, A, B, grad)
+        return None, None, None, None, None, None, None, None, dA, dB
+
+
+class NodeMulEdge(Function):
+    # modules/op.py:35-45
+    @staticmethod
+    def forward(ctx, row, indptr, eid, A, B):
+        ctx.save_for_backward(row, indptr, eid, A, B)
+        return node_mul_edge_forward(row, indptr, eid, A, B)
+
+    @staticmethod
+    def backward(ctx, grad):
+        row, indptr, eid, A, B = ctx.saved_tensors
+        dA, dB = node_mul_edge_backward(row, indptr, eid, A, B, grad)
+        return None, None, None, dA, dB
+
+
+class VectorSPMM(Function):
+    # modules/op.py:47-58
+    @staticmethod
+    def forward(ctx, row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x):
+        y = vector_spmm_forward(row, indptr, eid, indices, edata, x)
+        ctx.save_for_backward(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x = ctx.saved_tensors
+        dedata, dx = vector_spmm_backward(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, dy, x)
+        return None, None, None, None, None, None, None, None, dedata, dx
+
+
+class BPTAttention(Function):
+    """Fused masked_mm -> scale -> sparse_softmax -> vec_spmm (modules/attention.py:66-77 with
+    rel_pos off and dropout 0).  Saves q, k, v, o and the per-(node, head) log-sum-exp instead of
+    the (E, h) score and probability tensors."""
+
+    @staticmethod
+    def forward(ctx, row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale):
+        o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale)
+        ctx.save_for_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse)
+        ctx.scale = scale
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse = ctx.saved_tensors
+        dq, dk, dv = _g.attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c,
+                                           q, k, v, o, lse, do, ctx.scale)
+        return None, None, None, None, None, None, None, None, dq, dk, dv, None
+
+
+def sparse_softmax(row, indptr, eid, x):
+    return SparseSoftmax.apply(row, indptr, eid, x)
+
+
+def masked_mm(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, A, B):
+    return MaskedMMCSR.apply(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, A, B)
+
+
+def node_mul_edge(row, indptr, eid, A, B):
+    return NodeMulEdge.apply(row, indptr, eid, A, B)
+
+
+def vec_spmm(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x):
+    return VectorSPMM.apply(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x)
+
+
+def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale=None, fused=None):
+    """Attention over the graph: (ROW, INDPTR_R, out_eid, out_idx) is the out-CSR side (rows =
+    sources), (COL, INDPTR_C, in_eid, in_idx) the in-CSR side (rows = destinations), exactly the
+    eight graph arguments modules/attention.py:66-67 passes to masked_mm.
+
+    fused=None picks the fused kernels when they cover (h, d, dtype) and otherwise composes the
+    unfused HIP ops in the reference's order; both run on the GPU."""
+    scale = 1.0 / math.sqrt(q.size(-1)) if scale is None else float(scale)
+    if fused is None:
+        fused = _g.attention_supported(q) and q.size(0) == k.size(0)
+    if fused:
+        return BPTAttention.apply(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale)
+    e = masked_mm(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, k, q)
+    a = sparse_softmax(col, indptr_c, eid_c, e * scale)
+    return vec_spmm(col, indptr_c, eid_c, indices_c, row, indptr_r, eid_r, indices_r, a, v)

@@ -1,0 +1,124 @@
+"""Launch plans: the int32 row-level form of one CSR side plus the wavefront work list.
+
+The reference's ops receive (row, indptr, eid, indices) as int64 device tensors on every call
+(modules/op.py:10-70).  The HIP kernels want row ownership, so the first call that sees a given
+set of index tensors copies them to the host once, lets libbptgraph validate them and derive the
+plan (bptg_plan_fill), uploads the plan and caches it; later calls with the same tensors (all 12
+layers, forward and backward) hit the cache.  The cache keeps the key tensors alive, so a
+`data_ptr` can not be recycled for another graph while its entry exists.
+"""
+import collections
+import ctypes
+import threading
+
+import numpy as np
+import torch
+
+from ._lib import PlanInfo, PlanStruct, check_graph, graph_lib
+
+DEFAULT_SEG_LEN = 64
+_CACHE_SIZE = 64
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _host_i64(t):
+    if t is None:
+        return None
+    if isinstance(t, torch.Tensor):
+        t = t.detach().cpu().numpy()
+    return np.ascontiguousarray(t, dtype=np.int64)
+
+
+def build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len=DEFAULT_SEG_LEN):
+    """Pure host step (no GPU): returns (arrays, info) with arrays = dict of int32 numpy arrays
+    rowptr, idx, eid, items (n_items, 4), heavy (n_heavy, 3).  Raises ValueError on malformed input."""
+    row, indptr, eid, indices = map(_host_i64, (row, indptr, eid, indices))
+    if len(indptr) != len(row) + 1:
+        raise ValueError("indptr must have len(row) + 1 entries")
+    if indices is not None and len(indices) != len(eid):
+        raise ValueError("indices and eid must have the same length")
+    lib = graph_lib()
+    info = PlanInfo()
+    check_graph(lib.bptg_plan_sizes(_ptr(row), _ptr(indptr), len(row), int(n_rows), int(seg_len), ctypes.byref(info)))
+    E = len(eid)
+    arrays = {
+        "rowptr": np.empty(n_rows + 1, dtype=np.int32),
+        "idx": np.empty(E, dtype=np.int32),
+        "eid": np.empty(E, dtype=np.int32),
+        "items": np.empty((info.n_items, 4), dtype=np.int32),
+        "heavy": np.empty((info.n_heavy, 3), dtype=np.int32),
+    }
+    check_graph(lib.bptg_plan_fill(_ptr(row), _ptr(indptr), len(row), _ptr(eid), _ptr(indices), E,
+                                   int(n_rows), int(n_index_nodes), int(seg_len),
+                                   _ptr(arrays["rowptr"]), _ptr(arrays["idx"]), _ptr(arrays["eid"]),
+                                   _ptr(arrays["items"]), _ptr(arrays["heavy"]), ctypes.byref(info)))
+    return arrays, info
+
+
+class Plan:
+    """Device-resident plan of one CSR side; `.struct` is the `bpt_plan` passed to the C ABI."""
+
+    def __init__(self, row, indptr, eid, indices, n_rows, n_index_nodes, device, seg_len=DEFAULT_SEG_LEN):
+        arrays, info = build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len)
+        self.n_rows, self.n_edges = int(n_rows), len(arrays["eid"])
+        self.n_items, self.n_heavy, self.n_slots = info.n_items, info.n_heavy, info.n_slots
+        self.max_degree = info.max_degree
+        self.covers_all_edges = bool(info.flags & 1)
+        self.has_indices = indices is not None
+        self.device = torch.device(device)
+        # one allocation, 256-byte aligned sections (the items array is read as 16-byte vectors)
+        self._dev = {k: torch.from_numpy(v).to(self.device) for k, v in arrays.items()}
+        d = self._dev
+        self.struct = PlanStruct(
+            d["rowptr"].data_ptr(), d["idx"].data_ptr() if self.n_edges else None,
+            d["eid"].data_ptr() if self.n_edges else None, d["items"].data_ptr() if self.n_items else None,
+            d["heavy"].data_ptr() if self.n_heavy else None,
+            self.n_rows, self.n_edges, self.n_items, self.n_heavy, self.n_slots)
+
+    @property
+    def ref(self):
+        return ctypes.byref(self.struct)
+
+
+class PlanCache:
+    def __init__(self, capacity=_CACHE_SIZE):
+        self._d = collections.OrderedDict()
+        self._cap = capacity
+        self._lock = threading.Lock()     # forward runs on the Python thread, backward on autograd's
+        self.hits = self.misses = 0
+
+    @staticmethod
+    def _key(tensors, n_rows, n_index, seg_len):
+        return tuple((t.data_ptr(), t.numel(), t._version, str(t.device)) if t is not None else None
+                     for t in tensors) + (n_rows, n_index, seg_len)
+
+    def get(self, row, indptr, eid, indices, n_rows=None, n_index_nodes=None, seg_len=DEFAULT_SEG_LEN):
+        """n_rows None: as many rows as `row` mentions (ops that only produce edge outputs)."""
+        tensors = (row, indptr, eid, indices)
+        key = self._key(tensors, n_rows, n_index_nodes, seg_len)
+        with self._lock:
+            hit = self._d.get(key)
+            if hit is not None:
+                self._d.move_to_end(key)
+                self.hits += 1
+                return hit[0]
+        self.misses += 1
+        row_h = _host_i64(row)
+        nr = n_rows if n_rows is not None else (int(row_h[-1]) + 1 if len(row_h) else 0)
+        ni = n_index_nodes if n_index_nodes is not None else nr
+        plan = Plan(row_h, indptr, eid, indices, nr, ni, eid.device, seg_len)
+        with self._lock:
+            self._d[key] = (plan, tensors)          # tensors kept alive with the entry
+            while len(self._d) > self._cap:
+                self._d.popitem(last=False)
+        return plan
+
+    def clear(self):
+        with self._lock:
+            self._d.clear()
+
+
+plan_cache = PlanCache()

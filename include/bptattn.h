@@ -1,0 +1,127 @@
+/*
+ * libbptattn — gfx950 (MI355X) HIP kernels of the BPT graph-attention path, C ABI.
+ *
+ * Drop-in boundary for the reference's `graphop` extension (graph_kernel/graphop.cpp:216-225):
+ * one entry point per pybind function, plus the fused attention pair.  Plain pointers and sizes
+ * only; no torch types.  All data pointers are DEVICE pointers; outputs and the workspace are
+ * allocated by the caller (the library never allocates or frees device memory and never
+ * synchronises); kernels are enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ * default stream).  Every function returns 0 on success, a negative bpt_status for an argument
+ * error (nothing was launched) or a positive hipError_t if a launch failed.  Nothing throws.
+ *
+ * Graph arguments.  The reference passes chunked units (row, indptr), eid and indices as int64
+ * tensors.  Here they are passed as a `bpt_plan`: the int32 row-level form of exactly those four
+ * arrays plus the wavefront work list, produced once per graph by bptg_plan_fill()
+ * (include/bptgraph.h) and uploaded by the caller.  Row ownership replaces the reference's float
+ * atomics: every output row is written by one wavefront (rows longer than the plan's segment
+ * length by a fixed-order combine), so results are deterministic.
+ *
+ * Tensor layouts (row-major, contiguous): node tensors (n, h, d); edge tensors (n_edges, h)
+ * addressed by edge id; the per-edge feature of node_mul_edge (n_edges, d).  A reference call
+ * with 2-D node tensors (n, d) is h = 1.
+ */
+#ifndef BPTATTN_H
+#define BPTATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { BPT_F32 = 0, BPT_F64 = 1, BPT_BF16 = 2 } bpt_dtype;
+
+typedef enum {
+    BPT_OK = 0,
+    BPT_ERR_NULL = -1,        /* required pointer is NULL */
+    BPT_ERR_SIZE = -2,        /* negative or inconsistent size */
+    BPT_ERR_DTYPE = -3,       /* unknown dtype */
+    BPT_ERR_SHAPE = -4,       /* h or d not positive / too large */
+    BPT_ERR_WORKSPACE = -5,   /* workspace missing or smaller than bpt_workspace_bytes() */
+    BPT_ERR_PLAN = -6,        /* plans do not describe the same graph (edge / node counts differ) */
+    BPT_ERR_UNSUPPORTED = -7  /* combination not implemented (e.g. fused attention in f64) */
+} bpt_status;
+
+/* Device-resident plan of one CSR side (see bptg_plan_fill for the array contents). */
+typedef struct {
+    const int32_t *rowptr;   /* n_rows + 1 */
+    const int32_t *idx;      /* n_edges : other endpoint of the edge in slot p */
+    const int32_t *eid;      /* n_edges : edge id of slot p */
+    const int32_t *items;    /* n_items * 4 : row, begin, end, slot */
+    const int32_t *heavy;    /* n_heavy * 3 : row, first_slot, n_slots (may be NULL if n_heavy == 0) */
+    int64_t n_rows, n_edges, n_items, n_heavy, n_slots;
+} bpt_plan;
+
+const char *bpt_strerror(int status);
+
+/* 1: force the shape-generic kernels even where a specialised one exists (testing). Returns the old value. */
+int bpt_set_force_generic(int on);
+
+/* Bytes of workspace the call needs (0 possible).  op: one of the BPT_OP_* below. */
+enum {
+    BPT_OP_MASKEDMM_BWD = 1, BPT_OP_NODE_MUL_EDGE_BWD = 2, BPT_OP_SPMM_FWD = 3, BPT_OP_SPMM_BWD = 4,
+    BPT_OP_ATTN_FWD = 5, BPT_OP_ATTN_BWD = 6
+};
+int64_t bpt_workspace_bytes(int op, const bpt_plan *plan, const bpt_plan *plan_t, int h, int d, int dtype);
+
+/* graphop.cpp:16  maskedmm_csr_forward(row, indptr, eid, indices, A, B) -> y
+ * y[eid[p], :] = sum_d A[row, :, d] * B[indices[p], :, d]; y is (n_edges, h), fully written when
+ * the plan's eid covers every edge, so the caller zero-fills it otherwise. */
+int bpt_maskedmm_csr_forward(const bpt_plan *plan, const void *A, const void *B, void *y,
+                             int h, int d, int dtype, void *stream);
+
+/* graphop.cpp:108 maskedmm_csr_backward(row.., col.., A, B, dy) -> [dA, dB]
+ * dA[r] = sum_{p in row r of plan_r} dy[eid[p]] * B[idx[p]];  dB likewise over plan_c with A. */
+int bpt_maskedmm_csr_backward(const bpt_plan *plan_r, const bpt_plan *plan_c, const void *A, const void *B,
+                              const void *dy, void *dA, void *dB, void *workspace, int64_t workspace_bytes,
+                              int h, int d, int dtype, void *stream);
+
+/* graphop.cpp:39  node_mul_edge_forward(row, indptr, eid, A, B) -> y;  B is (n_edges, d) */
+int bpt_node_mul_edge_forward(const bpt_plan *plan, const void *A, const void *B, void *y,
+                              int h, int d, int dtype, void *stream);
+
+/* graphop.cpp:141 node_mul_edge_backward(row, indptr, eid, A, B, dy) -> [dA, dB] */
+int bpt_node_mul_edge_backward(const bpt_plan *plan, const void *A, const void *B, const void *dy,
+                               void *dA, void *dB, void *workspace, int64_t workspace_bytes,
+                               int h, int d, int dtype, void *stream);
+
+/* graphop.cpp:59  sparse_softmax_forward(row, indptr, eid, x) -> y   (softmax over each row's slots;
+ * the running maximum starts at -1e9 as in graphop_kernel.cu:428) */
+int bpt_sparse_softmax_forward(const bpt_plan *plan, const void *x, void *y, int h, int dtype, void *stream);
+
+/* graphop.cpp:163 sparse_softmax_backward(row, indptr, eid, y, dy) -> dx */
+int bpt_sparse_softmax_backward(const bpt_plan *plan, const void *y, const void *dy, void *dx,
+                                int h, int dtype, void *stream);
+
+/* graphop.cpp:79  vector_spmm_forward(row, indptr, eid, indices, edata, x) -> y
+ * y[r] = sum_p edata[eid[p]] * x[idx[p]];  every row of y is written (zero for empty rows). */
+int bpt_vector_spmm_forward(const bpt_plan *plan, const void *edata, const void *x, void *y,
+                            void *workspace, int64_t workspace_bytes, int h, int d, int dtype, void *stream);
+
+/* graphop.cpp:190 vector_spmm_backward(row.., col.., edata, dy, x) -> [dedata, dx]
+ * dedata[eid[p]] = <dy[row], x[idx[p]]> over `plan`; dx[c] = sum over ALL rows c of `plan_t` of
+ * edata[eid_t[p]] * dy[idx_t[p]].  (The reference launches the dx kernel with the grid of the
+ * other side, graphop_kernel.cu:566,588, and drops trailing units when plan_t has more units;
+ * this entry computes the complete gradient.) */
+int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const void *edata, const void *dy,
+                             const void *x, void *dedata, void *dx, void *workspace, int64_t workspace_bytes,
+                             int h, int d, int dtype, void *stream);
+
+/* Fused attention layer core = modules/attention.py:66-77 without dropout / rel-pos:
+ *   o[dst] = sum_{e: src->dst} softmax_dst( q[dst].k[src] * scale ) * v[src]
+ * plan_in: rows = destinations (the reference's COL/INDPTR_C/in_csr), plan_out: rows = sources.
+ * lse (n, h) float32 receives the base-2 log-sum-exp of the scaled scores, needed by backward.
+ * f32 and bf16 only (accumulation in f32). */
+int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v,
+                          void *o, float *lse, void *workspace, int64_t workspace_bytes,
+                          float scale, int h, int d, int dtype, void *stream);
+
+int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, const void *q, const void *k,
+                           const void *v, const void *o, const void *d_o, const float *lse,
+                           void *dq, void *dk, void *dv, void *workspace, int64_t workspace_bytes,
+                           float scale, int h, int d, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BPTATTN_H */

@@ -1,0 +1,84 @@
+/*
+ * libbptgraph — host-side (CPU) integer half of the BPT graph-attention path, C ABI.
+ *
+ * Replaces the reference's Cython module `graphbuilder` (graph_builder/builder.pyx) and the
+ * DGL adjacency export used by graph/base.py:71-86.  Everything here is host code working on
+ * caller-owned buffers: the library never allocates memory it hands out and never throws.
+ * Every function returns 0 on success or a negative bptg_status.
+ *
+ * Calling pattern: `*_sizes` tells how large the output arrays must be, the caller allocates
+ * them (numpy / torch / malloc), `*_fill` writes them.
+ */
+#ifndef BPTGRAPH_H
+#define BPTGRAPH_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    BPTG_OK = 0,
+    BPTG_ERR_NULL = -1,          /* a required pointer is NULL */
+    BPTG_ERR_SIZE = -2,          /* negative / inconsistent size, or a count exceeding int32 */
+    BPTG_ERR_ORDER = -3,         /* `row` not non-decreasing or `indptr` not non-decreasing */
+    BPTG_ERR_RANGE = -4,         /* a row id, index or edge id outside its valid range */
+    BPTG_ERR_ARG = -5            /* invalid scalar argument (e.g. chunk_size <= 0) */
+} bptg_status;
+
+const char *bptg_strerror(int status);
+
+/* ---- graph construction --------------------------------------------------------------------
+ * kind 0: BinaryPartition(length, triu, step=a, clip_dist=b)   builder.pyx:23-152
+ * kind 1: FullyConnected(length, triu, window=a)               builder.pyx:228-303
+ * kind 2: OpenAISparse(length, stride=a, c=b) (causal only)    builder.pyx:154-225
+ * Edge e goes src[e] -> dst[e]; the order of edges is part of the contract (edge id = position,
+ * graph/lm.py:96-98).  lvl_sizes receives n_levels entries (nodes per tree level). */
+int bptg_graph_sizes(int kind, int64_t length, int triu, int64_t a, int64_t b,
+                     int64_t *n_nodes, int64_t *n_edges, int64_t *n_levels);
+int bptg_graph_fill(int kind, int64_t length, int triu, int64_t a, int64_t b, int64_t v_shift,
+                    int64_t *src, int64_t *dst, int64_t *etype, int64_t *pos, int64_t *lvl_sizes);
+
+/* ---- partition_csr (builder.pyx:305-321 == graph_kernel/part_csr.py:13-27) -----------------
+ * Splits every row's slot range into chunks of at most chunk_size slots.  n_indptr = rows + 1. */
+int bptg_partition_csr_count(const int64_t *indptr, int64_t n_indptr, int64_t chunk_size, int64_t *n_units);
+int bptg_partition_csr_fill(const int64_t *indptr, int64_t n_indptr, int64_t chunk_size,
+                            int64_t *row, int64_t *indptr_units);
+
+/* ---- CSR with edge ids (what graph/base.py:72,79 obtains from DGL) -------------------------
+ * Stable counting sort of the edge list by `rows`: indptr (n+1), indices[p] = cols[eid[p]],
+ * eid[p] ascending inside each row.  For the out-CSR pass rows=src, cols=dst; in-CSR swapped. */
+int bptg_build_csr(const int64_t *rows, const int64_t *cols, int64_t n_edges, int64_t n_nodes,
+                   int64_t *indptr, int64_t *indices, int64_t *eid);
+
+/* ---- launch plan ----------------------------------------------------------------------------
+ * The reference kernels receive only chunked units (row[u], indptr[u..u+1]); a row spread over
+ * several units is combined there with float atomics.  The HIP library instead gives every row
+ * to one wavefront, and rows longer than seg_len edges to several wavefronts whose partial
+ * results are combined in a fixed order.  The plan derives that work list from the reference's
+ * arguments once per graph:
+ *   rowptr  int32[n_nodes+1]   row-level slot ranges recovered from the units
+ *   idx     int32[n_edges]     `indices` narrowed to 32 bit (zeros when indices == NULL)
+ *   eid     int32[n_edges]
+ *   items   int32[n_items*4]   (row, begin, end, slot); slot < 0: the item owns its whole row
+ *                              and writes results directly; slot >= 0: partial result number
+ *   heavy   int32[n_heavy*3]   (row, first_slot, n_slots) for every split row
+ * Every node gets at least one item (empty rows too) so kernels can write all outputs.
+ * flags bit0: eid is a permutation of 0..n_edges-1 (every edge output gets written). */
+typedef struct {
+    int64_t n_items, n_heavy, n_slots, max_degree, flags;
+} bptg_plan_info;
+
+int bptg_plan_sizes(const int64_t *row, const int64_t *indptr_units, int64_t n_units,
+                    int64_t n_nodes, int64_t seg_len, bptg_plan_info *info);
+int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_units,
+                   const int64_t *eid, const int64_t *indices, int64_t n_edges,
+                   int64_t n_nodes, int64_t n_index_nodes, int64_t seg_len,
+                   int32_t *rowptr, int32_t *idx32, int32_t *eid32, int32_t *items, int32_t *heavy,
+                   bptg_plan_info *info);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BPTGRAPH_H */

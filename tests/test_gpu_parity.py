@@ -1,0 +1,315 @@
+"""GPU parity: every op of the HIP library against the CPU oracle on the same seeded inputs.
+
+Tolerances (stated by the task): fp32 outputs rtol 1e-5 / atol 1e-5, fp32 gradients rtol 1e-4,
+bf16 rtol 2e-2; fp64 (generic kernels only) 1e-12.  The oracle runs in float64 on the float32 /
+bf16 input values, so the comparison measures the kernel's own rounding.  Index tensors are
+bit-exact by construction (tests/test_graphbuilder.py).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from bpt_amd import graphop, op
+    return graphop, op
+
+
+# --------------------------------------------------------------------------------------------
+# graphs
+# --------------------------------------------------------------------------------------------
+def block_graph(batch, l):
+    x = np.repeat(np.arange(batch * l), l)
+    y = (np.arange(batch * l * l) % l) + (np.arange(batch * l * l) // (l * l)) * l
+    return x.astype(np.int64), y.astype(np.int64), batch * l
+
+
+def bpt_graph(L, triu, step):
+    from bpt_amd import graphbuilder as gb
+    g = gb.BinaryPartition(L, triu, step, 10)
+    src, dst, _ = g.get_edges()
+    return src, dst, g.number_of_nodes
+
+
+def random_multigraph(n, E, seed=1):
+    rng = np.random.default_rng(seed)
+    src = rng.integers(0, n, E); dst = rng.integers(0, n, E)
+    dst[: E // 3] = 1; src[E // 3: E // 2] = 2
+    src[src == 0] = 3; dst[dst == 0] = 3
+    src[-1], dst[-1] = src[-2], dst[-2]
+    return src.astype(np.int64), dst.astype(np.int64), n
+
+
+GRAPHS = {
+    "blocks8x30": lambda: block_graph(8, 30),
+    "bpt512_k4": lambda: bpt_graph(512, False, 4),          # BASELINE config 1 (non-causal: duplicate edges, deg 512 row)
+    "bpt300_causal_k2": lambda: bpt_graph(300, True, 2),
+    "multigraph": lambda: random_multigraph(97, 3000),      # zero-degree node, heavy rows both sides, duplicates
+}
+
+
+class Case:
+    def __init__(self, name, chunk=32):
+        from bpt_amd import graphbuilder as gb
+        self.src, self.dst, self.n = GRAPHS[name]()
+        self.E = len(self.src)
+        self.csr = gb.get_csrs(self.src, self.dst, self.n, chunk_size=chunk, as_torch=False)
+        out_csr, in_csr, ROW, IR, COL, IC = self.csr
+        t = lambda a: torch.from_numpy(a).to(DEV)
+        # argument tuples in the reference's order
+        self.out = (t(ROW), t(IR), t(out_csr[2]), t(out_csr[1]))
+        self.inn = (t(COL), t(IC), t(in_csr[2]), t(in_csr[1]))
+        self.np_out = (ROW, IR, out_csr[2], out_csr[1])
+        self.np_in = (COL, IC, in_csr[2], in_csr[1])
+
+
+_cases = {}
+
+
+def case(name, chunk=32):
+    key = (name, chunk)
+    if key not in _cases:
+        _cases[key] = Case(name, chunk)
+    return _cases[key]
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * scale).to(dtype)
+
+
+def f64(t):
+    return t.detach().cpu().to(torch.float64).numpy()
+
+
+TOL = {torch.float32: dict(rtol=1e-5, atol=1e-5), torch.float64: dict(rtol=1e-12, atol=1e-12),
+       torch.bfloat16: dict(rtol=2e-2, atol=2e-2)}
+GTOL = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.float64: dict(rtol=1e-11, atol=1e-12),
+        torch.bfloat16: dict(rtol=2e-2, atol=2e-2)}
+
+
+def close(got, want, tol, what):
+    got = f64(got)
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    err = np.abs(got - want)
+    bound = tol["atol"] + tol["rtol"] * np.abs(want)
+    assert np.all(err <= bound), f"{what}: max err {err.max():.3e}, worst excess {(err - bound).max():.3e}"
+
+
+# --------------------------------------------------------------------------------------------
+# the eight ops
+# --------------------------------------------------------------------------------------------
+SHAPES = [(8, 64), (1, 40), (3, 20), (4, 64)]   # (8,64)/(4,64) have specialised kernels, the others are generic
+
+
+@pytest.mark.parametrize("force_generic", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("hd", SHAPES)
+@pytest.mark.parametrize("gname,chunk", [("blocks8x30", 32), ("blocks8x30", 7), ("bpt512_k4", 32), ("multigraph", 8)])
+def test_ops_match_oracle(ops, gname, chunk, hd, dtype, force_generic):
+    graphop, _ = ops
+    h, d = hd
+    if force_generic and (hd not in ((8, 64), (4, 64)) or dtype == torch.float64):
+        pytest.skip("already generic")
+    c = case(gname, chunk)
+    n, E = c.n, c.E
+    A = rand((n, h, d), dtype, 1, 0.5).to(DEV)
+    B = rand((n, h, d), dtype, 2, 0.5).to(DEV)
+    w = rand((E, h), dtype, 3).to(DEV)
+    gy = rand((n, h, d), dtype, 4).to(DEV)
+    Be = rand((E, d), dtype, 5, 0.5).to(DEV)
+    tol, gtol = TOL[dtype], GTOL[dtype]
+    graphop.set_force_generic(force_generic)
+    try:
+        # SDDMM as attention.py:66-67 calls it: out-CSR, A = k, B = q
+        y = graphop.maskedmm_csr_forward(*c.out, A, B)
+        close(y, oracle.maskedmm_csr_forward(*c.np_out, f64(A), f64(B)), tol, "maskedmm fwd")
+        dA, dB = graphop.maskedmm_csr_backward(*c.out, *c.inn, A, B, w)
+        rA, rB = oracle.maskedmm_csr_backward(*c.np_out, *c.np_in, f64(A), f64(B), f64(w))
+        close(dA, rA, gtol, "maskedmm dA"); close(dB, rB, gtol, "maskedmm dB")
+        # edge softmax over in-edges
+        a = graphop.sparse_softmax_forward(*c.inn[:3], w)
+        ra = oracle.sparse_softmax_forward(*c.np_in[:3], f64(w), n_nodes=n)
+        close(a, ra, tol, "softmax fwd")
+        dx = graphop.sparse_softmax_backward(*c.inn[:3], a, w)
+        close(dx, oracle.sparse_softmax_backward(*c.np_in[:3], f64(a), f64(w), n_nodes=n), gtol, "softmax bwd")
+        # SpMM over the in-CSR
+        o = graphop.vector_spmm_forward(*c.inn, w, A)
+        close(o, oracle.vector_spmm_forward(*c.np_in, f64(w), f64(A)), tol if dtype != torch.float32 else gtol, "spmm fwd")
+        dw, dxx = graphop.vector_spmm_backward(*c.inn, *c.out, w, gy, A)
+        rdw, rdx = oracle.vector_spmm_backward(*c.np_in, *c.np_out, f64(w), f64(gy), f64(A))
+        close(dw, rdw, gtol, "spmm dedata"); close(dxx, rdx, gtol, "spmm dx")
+        # node . edge (rel-pos term), in-CSR, A = q
+        yn = graphop.node_mul_edge_forward(*c.inn[:3], A, Be)
+        close(yn, oracle.node_mul_edge_forward(*c.np_in[:3], f64(A), f64(Be)), tol, "node_mul_edge fwd")
+        dAn, dBe = graphop.node_mul_edge_backward(*c.inn[:3], A, Be, w)
+        rAn, rBe = oracle.node_mul_edge_backward(*c.np_in[:3], f64(A), f64(Be), f64(w))
+        close(dAn, rAn, gtol, "node_mul_edge dA"); close(dBe, rBe, gtol, "node_mul_edge dB")
+    finally:
+        graphop.set_force_generic(False)
+
+
+def test_single_head_2d_inputs(ops):
+    """(n, d) node tensors and (e,) edge tensors, graph_kernel/test.py:148-301 (dim 1024)."""
+    graphop, _ = ops
+    c = case("blocks8x30")
+    A = rand((c.n, 1024), torch.float32, 1, 0.1).to(DEV)
+    B = rand((c.n, 1024), torch.float32, 2, 0.1).to(DEV)
+    w = rand((c.E,), torch.float32, 3).to(DEV)
+    y = graphop.maskedmm_csr_forward(*c.out, A, B)
+    assert y.shape == (c.E,)
+    close(y, oracle.maskedmm_csr_forward(*c.np_out, f64(A), f64(B)), TOL[torch.float32], "2-D maskedmm")
+    a = graphop.sparse_softmax_forward(*c.out[:3], w)
+    assert a.shape == (c.E,)
+    close(a, oracle.sparse_softmax_forward(*c.np_out[:3], f64(w), n_nodes=c.n), TOL[torch.float32], "2-D softmax")
+    o = graphop.vector_spmm_forward(*c.out, a, A)
+    close(o, oracle.vector_spmm_forward(*c.np_out, f64(a), f64(A)), TOL[torch.float32], "2-D spmm")
+
+
+# --------------------------------------------------------------------------------------------
+# the attention layer: fused kernels and the unfused op chain, forward + backward
+# --------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("dtype,hd", [(torch.float32, (8, 64)), (torch.float32, (16, 64)), (torch.float32, (8, 32)),
+                                      (torch.bfloat16, (8, 64)), (torch.bfloat16, (16, 64)), (torch.float32, (2, 24))])
+@pytest.mark.parametrize("gname", ["bpt512_k4", "bpt300_causal_k2", "multigraph"])
+def test_attention_layer(ops, gname, dtype, hd, fused):
+    graphop, op = ops
+    h, d = hd
+    if fused and hd == (2, 24):
+        pytest.skip("no fused instantiation; covered by the unfused chain")
+    c = case(gname)
+    q, k, v, do = (rand((c.n, h, d), dtype, s, 1.0 / 8).to(DEV) for s in (11, 12, 13, 14))   # N(0,1)/sqrt(64)
+    q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+    o = op.bpt_attention(*c.out, *c.inn, q, k, v, fused=fused)
+    o.backward(do)
+    ro, ra = oracle.attention_forward(c.csr, f64(q), f64(k), f64(v))
+    rdq, rdk, rdv = oracle.attention_backward(c.csr, f64(q), f64(k), f64(v), ra, f64(do))
+    close(o, ro, TOL[dtype], "o")
+    close(q.grad, rdq, GTOL[dtype], "dq"); close(k.grad, rdk, GTOL[dtype], "dk"); close(v.grad, rdv, GTOL[dtype], "dv")
+
+
+def test_attention_with_rel_pos_chain(ops):
+    """modules/attention.py:66-77 with rel_pos: masked_mm + node_mul_edge -> softmax -> spmm, through autograd."""
+    _, op = ops
+    c = case("bpt300_causal_k2")
+    h, d = 8, 64
+    q, k, v, do = (rand((c.n, h, d), torch.float32, s, 1.0 / 8).to(DEV).requires_grad_(s < 14) for s in (11, 12, 13, 14))
+    ak = rand((c.E, d), torch.float32, 15, 1.0 / 8).to(DEV).requires_grad_(True)
+    e = op.masked_mm(*c.out, *c.inn, k, q)
+    e_rel = op.node_mul_edge(*c.inn[:3], q, ak)
+    a = op.sparse_softmax(*c.inn[:3], (e_rel + e) / np.sqrt(d))
+    o = op.vec_spmm(*c.inn, *c.out, a, v)
+    o.backward(do)
+    ro, ra = oracle.attention_forward(c.csr, f64(q), f64(k), f64(v), f64(ak))
+    rdq, rdk, rdv, rdak = oracle.attention_backward(c.csr, f64(q), f64(k), f64(v), ra, f64(do), f64(ak))
+    close(o, ro, TOL[torch.float32], "o")
+    for got, want, nm in ((q.grad, rdq, "dq"), (k.grad, rdk, "dk"), (v.grad, rdv, "dv"), (ak.grad, rdak, "dak")):
+        close(got, want, GTOL[torch.float32], nm)
+
+
+def test_headline_graph_full_parity(ops):
+    """BASELINE config 3 at full size (L=8192, k=4, causal, 8x64 fp32) directly against the oracle."""
+    _, op = ops
+    from bpt_amd import graphbuilder as gb
+    g = gb.BinaryPartition(8192, True, 4, 10)
+    src, dst, _ = g.get_edges()
+    n = g.number_of_nodes
+    csr = gb.get_csrs(src, dst, n, as_torch=False)
+    out_csr, in_csr, ROW, IR, COL, IC = csr
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    args = (t(ROW), t(IR), t(out_csr[2]), t(out_csr[1]), t(COL), t(IC), t(in_csr[2]), t(in_csr[1]))
+    gen = torch.Generator().manual_seed(2345)
+    q, k, v, do = (torch.randn(n, 8, 64, generator=gen) / 8 for _ in range(4))
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    o = op.bpt_attention(*args, qd, kd, vd)
+    o.backward(do.to(DEV))
+    ro, ra = oracle.attention_forward(csr, f64(q), f64(k), f64(v))
+    rdq, rdk, rdv = oracle.attention_backward(csr, f64(q), f64(k), f64(v), ra, f64(do))
+    close(o, ro, TOL[torch.float32], "o")
+    close(qd.grad, rdq, GTOL[torch.float32], "dq"); close(kd.grad, rdk, GTOL[torch.float32], "dk")
+    close(vd.grad, rdv, GTOL[torch.float32], "dv")
+    # unfused chain agrees with the fused kernels
+    o2 = op.bpt_attention(*args, qd.detach(), kd.detach(), vd.detach(), fused=False)
+    assert torch.allclose(o2, o.detach(), rtol=1e-5, atol=1e-5)
+
+
+def test_stress_graph_properties(ops):
+    """BASELINE config 5 (L=32768, k=8, causal, 16x64, bf16): size-independent properties."""
+    _, op = ops
+    from bpt_amd import graphbuilder as gb
+    g = gb.BinaryPartition(32768, True, 8, 10)
+    src, dst, _ = g.get_edges()
+    n = g.number_of_nodes
+    assert (n, len(src)) == (65535, 3293955)
+    csr = gb.get_csrs(src, dst, n)
+    out_csr, in_csr, ROW, IR, COL, IC = csr
+    args = tuple(x.to(DEV) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
+    gen = torch.Generator().manual_seed(2345)
+    q, k, do = (((torch.randn(n, 16, 64, generator=gen) / 8).to(torch.bfloat16)).to(DEV) for _ in range(3))
+    # 1. v == 1  =>  o == 1 wherever a node has in-edges (softmax rows sum to one); every node has one here
+    ones = torch.ones(n, 16, 64, dtype=torch.bfloat16, device=DEV)
+    o = op.bpt_attention(*args, q, k, ones)
+    assert torch.allclose(o.float(), torch.ones_like(o, dtype=torch.float32), rtol=1e-2, atol=1e-2)
+    # 2. column sums of dV equal column sums of dO (sum_e p_e = 1 per destination)
+    v = ones.clone().requires_grad_(True)
+    qg = q.clone().requires_grad_(True)
+    op.bpt_attention(*args, qg, k, v).backward(do)
+    assert torch.allclose(v.grad.float().sum(0), do.float().sum(0), rtol=2e-2, atol=0.5)
+    # 3. with constant v the output does not depend on q: dq == 0 (dp == delta for every edge)
+    assert qg.grad.float().abs().max().item() < 2e-2
+    # 4. run-to-run bit reproducibility (no atomics)
+    o2 = op.bpt_attention(*args, q, k, ones)
+    assert torch.equal(o, o2)
+
+
+def test_determinism_and_cache(ops):
+    graphop, op = ops
+    from bpt_amd.plan import plan_cache
+    c = case("bpt512_k4")
+    q, k, v, do = (rand((c.n, 8, 64), torch.float32, s, 1.0 / 8).to(DEV) for s in (1, 2, 3, 4))
+    outs = []
+    for _ in range(2):
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (q, k, v))
+        o = op.bpt_attention(*c.out, *c.inn, qq, kk, vv)
+        o.backward(do)
+        outs.append((o.detach(), qq.grad, kk.grad, vv.grad))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    h0 = plan_cache.hits
+    graphop.sparse_softmax_forward(*c.inn[:3], rand((c.E, 8), torch.float32, 5).to(DEV))
+    graphop.sparse_softmax_forward(*c.inn[:3], rand((c.E, 8), torch.float32, 6).to(DEV))
+    assert plan_cache.hits >= h0 + 1
+
+
+def test_input_checks(ops):
+    graphop, _ = ops
+    c = case("blocks8x30")
+    A = rand((c.n, 8, 64), torch.float32, 1).to(DEV)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):          # graphop.cpp:4
+        graphop.maskedmm_csr_forward(*c.out, A.cpu(), A)
+    with pytest.raises(RuntimeError, match="must be contiguous"):             # graphop.cpp:5
+        graphop.maskedmm_csr_forward(*c.out, A.transpose(0, 1).contiguous().transpose(0, 1), A)
+    with pytest.raises(RuntimeError, match="dtype"):
+        graphop.maskedmm_csr_forward(*c.out, A.half(), A.half())
+    bad_idx = c.out[3].clone(); bad_idx[0] = c.n + 5
+    with pytest.raises(ValueError, match="out of range"):
+        graphop.maskedmm_csr_forward(c.out[0], c.out[1], c.out[2], bad_idx, A, A)
+
+
+def test_zero_degree_rows_are_zero(ops):
+    graphop, _ = ops
+    c = case("multigraph")
+    x = rand((c.n, 8, 64), torch.float32, 1).to(DEV)
+    w = rand((c.E, 8), torch.float32, 2).to(DEV)
+    y = graphop.vector_spmm_forward(*c.inn, w, x)
+    assert torch.all(y[0] == 0)
+    o, lse = graphop.attention_forward(*c.inn, x, x, x)
+    assert torch.all(o[0] == 0)

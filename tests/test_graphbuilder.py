@@ -1,0 +1,133 @@
+"""Host graph builder of the product (libbptgraph) against the golden vectors written by the
+reference's own builder, and against the independent oracle restatement."""
+import hashlib
+import json
+import os
+import pickle
+
+import numpy as np
+import pytest
+
+import oracle
+from bpt_amd import graphbuilder as gb
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+SMALL = np.load(os.path.join(GOLD, "builder_small.npz"))
+DIGESTS = json.load(open(os.path.join(GOLD, "builder_digests.json")))
+
+
+def digest(*arrays):
+    h = hashlib.sha256()
+    for a in arrays:
+        h.update(np.ascontiguousarray(np.asarray(a).astype("<i8")).tobytes())
+    return h.hexdigest()
+
+
+def _keys(prefix):
+    return sorted({k[:-4] for k in SMALL.files if k.startswith(prefix) and k.endswith("_src") and "shift" not in k})
+
+
+def _args(key):
+    return [int(p[1:]) for p in key.split("_")[1:]]
+
+
+@pytest.mark.parametrize("key", _keys("bp_L"))
+def test_binary_partition_golden(key):
+    L, triu, step, clip = _args(key)
+    g = gb.BinaryPartition(L, bool(triu), step, clip)
+    src, dst, et = g.get_edges()
+    assert src.dtype == np.int64
+    assert [g.number_of_nodes, g.number_of_edges, g.number_of_levels] == SMALL[key + "_meta"].tolist()
+    assert np.array_equal(src, SMALL[key + "_src"]) and np.array_equal(dst, SMALL[key + "_dst"])
+    assert np.array_equal(et, SMALL[key + "_etype"]) and np.array_equal(g.get_pos(), SMALL[key + "_pos"])
+
+
+@pytest.mark.parametrize("key", sorted(DIGESTS))
+def test_large_digests(key):
+    a = _args(key)
+    g = gb.BinaryPartition(a[0], bool(a[1]), a[2], a[3]) if key.startswith("bp_") else gb.FullyConnected(a[0], bool(a[1]), a[2])
+    src, dst, et = g.get_edges()
+    assert (g.number_of_nodes, g.number_of_edges) == (DIGESTS[key]["n_nodes"], DIGESTS[key]["n_edges"])
+    assert digest(src, dst, et, g.get_pos()) == DIGESTS[key]["sha256_src_dst_etype_pos"]
+
+
+@pytest.mark.parametrize("key", _keys("fc_"))
+def test_fully_connected_golden(key):
+    L, triu, window = _args(key)
+    g = gb.FullyConnected(L, bool(triu), window)
+    src, dst, et = g.get_edges()
+    assert np.array_equal(src, SMALL[key + "_src"]) and np.array_equal(dst, SMALL[key + "_dst"])
+    assert np.array_equal(et, SMALL[key + "_etype"]) and np.array_equal(g.get_pos(), SMALL[key + "_pos"])
+
+
+@pytest.mark.parametrize("key", _keys("oa_"))
+def test_openai_sparse_golden(key):
+    L, stride, c = _args(key)
+    g = gb.OpenAISparse(L, stride, c)
+    src, dst, et = g.get_edges()
+    assert np.array_equal(src, SMALL[key + "_src"]) and np.array_equal(dst, SMALL[key + "_dst"])
+    assert np.array_equal(et, SMALL[key + "_etype"]) and np.array_equal(g.get_pos(), SMALL[key + "_pos"])
+
+
+def test_api_surface_and_pickle():
+    g = gb.BinaryPartition(13, True, 2, 10)
+    s, d, _ = g.get_edges(v_shift=100)
+    assert np.array_equal(s, SMALL["bp_shift_src"]) and np.array_equal(d, SMALL["bp_shift_dst"])
+    assert np.array_equal(g.leaf_ids(v_shift=100, start=3), SMALL["bp_shift_leaf"])
+    assert np.array_equal(g.internal_ids(v_shift=100), SMALL["bp_shift_internal"])
+    assert g.root_id(v_shift=100) == SMALL["bp_shift_root"][0] and g.is_triu
+    assert [g.number_of_nodes_at_lvl(i) for i in range(g.number_of_levels)] == SMALL["bp_shift_lvls"].tolist()
+    g2 = pickle.loads(pickle.dumps(g))                    # builder.pyx:38-39
+    assert all(np.array_equal(a, b) for a, b in zip(g.get_edges(), g2.get_edges()))
+    f2 = pickle.loads(pickle.dumps(gb.FullyConnected(5, True, 3)))
+    assert f2.number_of_edges == gb.FullyConnected(5, True, 3).number_of_edges
+    with pytest.raises(ValueError):
+        gb.BinaryPartition(0)
+    with pytest.raises(AssertionError):
+        gb.OpenAISparse(8, 4, 1, triu=False)
+
+
+@pytest.mark.parametrize("i", range(5))
+def test_partition_csr_golden(i):
+    row, ip = gb.partition_csr(SMALL[f"pc{i}_indptr"], int(SMALL[f"pc{i}_chunk"][0]))
+    assert row.dtype == np.int64 and ip.dtype == np.int64
+    assert np.array_equal(row, SMALL[f"pc{i}_row"]) and np.array_equal(ip, SMALL[f"pc{i}_out"])
+
+
+def test_partition_csr_errors():
+    with pytest.raises(ValueError):
+        gb.partition_csr(np.array([0, 4]), 0)
+    with pytest.raises(ValueError):
+        gb.partition_csr(np.array([0, 4, 2]), 4)
+
+
+@pytest.mark.parametrize("L,triu,step", [(37, False, 2), (100, True, 4), (5, False, 1)])
+def test_get_csrs_matches_oracle(L, triu, step):
+    g = gb.BinaryPartition(L, triu, step, 10)
+    src, dst, _ = g.get_edges()
+    got = gb.get_csrs(src, dst, g.number_of_nodes, as_torch=False)
+    want = oracle.get_csrs(src, dst, g.number_of_nodes)
+    for a, b in zip(got[0] + got[1] + got[2:], want[0] + want[1] + want[2:]):
+        assert a.dtype == np.int64 and np.array_equal(a, b)
+    t = gb.get_csrs(src, dst, g.number_of_nodes)
+    import torch
+    assert t[2].dtype == torch.long and t[0][1].dtype == torch.long
+
+
+def test_build_csr_rejects_out_of_range():
+    with pytest.raises(ValueError):
+        gb.build_csr(np.array([0, 5]), np.array([0, 1]), 3)
+
+
+def test_batch_merge_cfg2_shape():
+    """BASELINE config 2: 32 causal graphs with seeded lengths merged block-diagonally."""
+    lengths = np.random.default_rng(2345).integers(64, 1025, 32)
+    assert lengths[:4].tolist() == [171, 550, 518, 514] and lengths.sum() == 16736
+    cache = {}
+    gs = [cache.setdefault(int(L), gb.BinaryPartition(int(L), True, 4, 10)) for L in lengths]
+    src, dst, et, pos, n = gb.merge_graphs(gs)
+    assert (n, len(src)) == (33598, 573520)
+    ogs = [oracle.BinaryPartition(int(L), True, 4, 10) for L in lengths[:3]]
+    osrc, odst, oet, opos, on = oracle.merge_graphs(ogs)
+    assert np.array_equal(src[:len(osrc)], osrc) and np.array_equal(dst[:len(osrc)], odst)
+    assert np.array_equal(et[:len(osrc)], oet) and np.array_equal(pos[:on], opos)

@@ -1,0 +1,119 @@
+"""Host logic of the launch plan, and that both shared libraries load and export every symbol
+their headers declare (no GPU needed, no compute calls)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import oracle
+from bpt_amd import _lib
+from bpt_amd import graphbuilder as gb
+from bpt_amd.plan import build_plan_host
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header, prefix):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(" + prefix + r"\w+)\s*\(", text)))
+
+
+def test_libraries_export_every_declared_symbol():
+    g = _declared("bptgraph.h", "bptg_")
+    a = _declared("bptattn.h", "bpt_")
+    assert len(g) >= 8 and len(a) >= 13
+    glib, alib = _lib.graph_lib(), _lib.attn_lib()
+    for name in g:
+        assert hasattr(glib, name), name
+    for name in a:
+        assert hasattr(alib, name), name
+    # the Python bindings cover exactly the declared API
+    assert sorted(_lib.GRAPH_API) == g and sorted(_lib.ATTN_API) == a
+
+
+def test_error_strings_and_argument_errors_without_gpu():
+    alib = _lib.attn_lib()
+    assert alib.bpt_strerror(0) == b"ok" and b"workspace" in alib.bpt_strerror(-5)
+    # argument errors are detected before anything touches the device
+    assert alib.bpt_maskedmm_csr_forward(None, None, None, None, 8, 64, 0, None) == -1
+    plan = _lib.PlanStruct(None, None, None, None, None, 0, 0, 0, 0, 0)
+    assert alib.bpt_sparse_softmax_forward(ctypes.byref(plan), None, None, 8, 7, None) == -3          # dtype
+    assert alib.bpt_vector_spmm_forward(ctypes.byref(plan), None, None, None, None, 0, 0, 64, 0, None) == -4   # h = 0
+    plan_bad = _lib.PlanStruct(None, None, None, None, None, 0, -1, 0, 0, 0)
+    assert alib.bpt_sparse_softmax_forward(ctypes.byref(plan_bad), None, None, 8, 0, None) == -2
+    assert alib.bpt_workspace_bytes(5, ctypes.byref(plan), None, 8, 64, 0) == 0
+    assert _lib.graph_lib().bptg_strerror(-4).startswith(b"row id")
+
+
+def _bpt_csr(L, triu, step):
+    g = gb.BinaryPartition(L, triu, step, 10)
+    src, dst, _ = g.get_edges()
+    return g, src, dst, gb.get_csrs(src, dst, g.number_of_nodes, as_torch=False)
+
+
+@pytest.mark.parametrize("seg", [4, 64])
+@pytest.mark.parametrize("L,triu,step", [(64, True, 4), (37, False, 2), (1, False, 1)])
+def test_plan_properties(L, triu, step, seg):
+    g, src, dst, (out_csr, in_csr, ROW, IR, COL, IC) = _bpt_csr(L, triu, step)
+    n, E = g.number_of_nodes, g.number_of_edges
+    for (indptr, indices, eid), units, ip in ((out_csr, ROW, IR), (in_csr, COL, IC)):
+        arr, info = build_plan_host(units, ip, eid, indices, n, n, seg)
+        assert np.array_equal(arr["rowptr"], indptr)                      # row-level indptr recovered from the units
+        assert np.array_equal(arr["idx"], indices) and np.array_equal(arr["eid"], eid)
+        items, heavy = arr["items"], arr["heavy"]
+        assert info.flags & 1 and info.max_degree == np.diff(indptr).max()
+        # items tile every row exactly once, in order, each at most seg long
+        assert np.all(items[:, 2] - items[:, 1] <= seg) and np.all(np.diff(items[:, 0]) >= 0)
+        assert set(items[:, 0].tolist()) == set(range(n))
+        pos = 0
+        for r, b, e, slot in items.tolist():
+            if e > b:
+                assert b == pos
+                pos = e
+            assert indptr[r] <= b and e <= indptr[r + 1]
+            assert (slot >= 0) == (indptr[r + 1] - indptr[r] > seg)
+        assert pos == E
+        # heavy rows: consecutive slots, ceil(deg / seg) each
+        slots = items[items[:, 3] >= 0]
+        assert np.array_equal(slots[:, 3], np.arange(info.n_slots))
+        for r, s0, ns in heavy.tolist():
+            assert ns == -(-(indptr[r + 1] - indptr[r]) // seg)
+            assert np.all(slots[s0:s0 + ns, 0] == r)
+        assert heavy[:, 2].sum() == info.n_slots
+
+
+def test_plan_handles_empty_rows_and_partial_edge_cover():
+    # 5 nodes, rows 1 and 3 have slots; eid covers 0..4 but the units stop before the last slot
+    row = np.array([1, 3]); ip = np.array([0, 2, 4]); eid = np.array([4, 0, 2, 1, 3]); idx = np.array([0, 1, 2, 3, 4])
+    arr, info = build_plan_host(row, ip, eid, idx, 5, 5, 64)
+    assert arr["rowptr"].tolist() == [0, 0, 2, 2, 4, 4] and info.n_items == 5 and not (info.flags & 1)
+    assert arr["items"].tolist() == [[0, 0, 0, -1], [1, 0, 2, -1], [2, 2, 2, -1], [3, 2, 4, -1], [4, 4, 4, -1]]
+
+
+def test_plan_rejects_malformed_graphs():
+    ok = dict(row=np.array([0, 1]), indptr=np.array([0, 1, 2]), eid=np.array([0, 1]), indices=np.array([1, 0]))
+    build_plan_host(**ok, n_rows=2, n_index_nodes=2)
+    bad = [dict(ok, row=np.array([1, 0])),                 # rows not grouped
+           dict(ok, indptr=np.array([0, 2, 1])),           # indptr decreasing
+           dict(ok, indices=np.array([1, 2])),             # index out of range
+           dict(ok, eid=np.array([0, 2])),                 # edge id out of range
+           dict(ok, row=np.array([0, 2])),                 # row id out of range
+           dict(ok, indptr=np.array([0, 1, 3]))]           # units beyond the edge arrays
+    for kw in bad:
+        with pytest.raises(ValueError):
+            build_plan_host(**kw, n_rows=2, n_index_nodes=2)
+    with pytest.raises(ValueError):
+        build_plan_host(ok["row"], np.array([0, 1]), ok["eid"], ok["indices"], 2, 2)
+
+
+def test_cfg3_plan_numbers():
+    """Headline graph: L=8192, k=4, causal."""
+    g, src, dst, (out_csr, in_csr, ROW, IR, COL, IC) = _bpt_csr(8192, True, 4)
+    assert (g.number_of_nodes, g.number_of_edges, len(COL), len(ROW)) == (16383, 430237, 25475, 21902)
+    deg_in = np.diff(in_csr[0])
+    assert deg_in[:8192].max() == 46 and deg_in.max() == 8192 and np.diff(out_csr[0]).max() == 3587
+    arr, info = build_plan_host(COL, IC, in_csr[2], in_csr[1], 16383, 16383, 64)
+    assert info.n_heavy == 127 and info.n_slots == 896
