@@ -1,0 +1,234 @@
+#!/usr/bin/env python3
+"""Benchmark of the BPT graph-attention hot path on one MI355X.
+
+A step = one fused attention layer forward + backward (SDDMM -> edge softmax -> SpMM and their
+gradients) over one synthetic graph batch, inputs resident in HBM.  Default workload: BASELINE
+config 3, L=8192 tokens, k=4, causal binary-partition graph, 8 heads x 64, fp32.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg1|cfg2|cfg5|cfg4-kN|cfg4-w128]
+                  [--dtype f32|bf16] [--no-cpu-baseline] [--no-graph]
+
+Prints ONE JSON line on stdout (details go to stderr).  `value` = graph edges per second of the
+whole fwd+bwd step; `roofline` describes the dominant kernel, timed live with HIP events on the
+launch stream; `cpu_baseline` is the PyTorch-CPU restatement of the same arithmetic (oracle/), timed
+on this host's cores on the same workload.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published peak
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_workload(name):
+    """Returns (description, list of graphs, h, d, default dtype)."""
+    import numpy as np
+    from bpt_amd import graphbuilder as gb
+    if name == "cfg1":
+        return "cfg1: L=512 k=4 non-causal BPT graph, 8x64", [gb.BinaryPartition(512, False, 4, 10)], 8, 64, "f32"
+    if name == "cfg2":
+        lengths = np.random.default_rng(2345).integers(64, 1025, 32)
+        cache = {}
+        gs = [cache.setdefault(int(L), gb.BinaryPartition(int(L), True, 4, 10)) for L in lengths]
+        return "cfg2: 32 causal BPT graphs, L~U[64,1024] (seed 2345), k=4, 8x64", gs, 8, 64, "f32"
+    if name == "cfg3":
+        return "cfg3: L=8192 k=4 causal BPT graph, 8x64", [gb.BinaryPartition(8192, True, 4, 10)], 8, 64, "f32"
+    if name == "cfg5":
+        return "cfg5: L=32768 k=8 causal BPT graph, 16x64", [gb.BinaryPartition(32768, True, 8, 10)], 16, 64, "bf16"
+    if name.startswith("cfg4-k"):
+        k = int(name[6:])
+        return f"cfg4: L=4096 k={k} causal BPT graph, 8x64", [gb.BinaryPartition(4096, True, k, 10)], 8, 64, "f32"
+    if name == "cfg4-w128":
+        return "cfg4: L=4096 window-128 causal dense graph, 8x64", [gb.FullyConnected(4096, True, 128)], 8, 64, "f32"
+    raise SystemExit(f"unknown workload {name}")
+
+
+def algorithmic_bytes(N, E, H, D, s):
+    """Compulsory HBM traffic of the fused fwd+bwd step (every distinct input read once, every output
+    written once): 12*N*C*s + 2*N*H*4 + 3*E*4 + 2*(N+1)*4, split over the three main kernels so the parts
+    add up to the total."""
+    C = H * D
+    fwd = 4 * N * C * s + N * H * 4 + E * 4 + (N + 1) * 4          # read q,k,v; write o, lse; in-CSR
+    bwd_dst = 6 * N * C * s + N * H * 4 + E * 4                    # read q,k,v,o,dO, lse; write dq; in-CSR
+    bwd_src = 2 * N * C * s + E * 4 + (N + 1) * 4                  # write dk,dv; out-CSR (q, dO counted above)
+    return {"attn_fwd": fwd, "attn_bwd_dst": bwd_dst, "attn_bwd_src": bwd_src, "total": fwd + bwd_dst + bwd_src}
+
+
+def cpu_baseline(src, dst, N, H, D, seed, budget_s=25.0):
+    """PyTorch-CPU gather / index_add restatement (oracle/torch_ops.py), all host threads, fp32."""
+    import torch
+    from oracle import torch_ops
+    gen = torch.Generator().manual_seed(seed)
+    q, k, v, do = (torch.randn(N, H, D, generator=gen) / 8 for _ in range(4))
+    s, d_ = torch.from_numpy(src), torch.from_numpy(dst)
+    cores = torch.get_num_threads()
+    t0 = time.perf_counter()
+    torch_ops.attention_fwd_bwd(s, d_, q, k, v, do)                 # warm-up (allocator, threads)
+    warm = time.perf_counter() - t0
+    times = []
+    while len(times) < 5 and (sum(times) + warm) < budget_s:
+        t0 = time.perf_counter()
+        torch_ops.attention_fwd_bwd(s, d_, q, k, v, do)
+        times.append(time.perf_counter() - t0)
+    if not times:
+        times = [warm]
+    med = sorted(times)[len(times) // 2]
+    return {"value": len(src) / med, "unit": "edges/s", "cores": cores, "kind": "port",
+            "sample": f"{len(times)} timed fwd+bwd passes of the full workload after 1 warm-up (median {med * 1e3:.1f} ms), fp32"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg3")
+    ap.add_argument("--dtype", default=None, choices=[None, "f32", "bf16"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
+    ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import numpy as np
+    import torch
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd import graphop
+    from bpt_amd._lib import attn_lib
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    desc, graphs, H, D, default_dtype = make_workload(args.workload)
+    dtype_name = args.dtype or default_dtype
+    tdtype = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
+    esize = {"f32": 4, "bf16": 2}[dtype_name]
+
+    t0 = time.perf_counter()
+    src, dst, _, _, N = gb.merge_graphs(graphs)
+    E = len(src)
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, N)
+    t_graph = time.perf_counter() - t0
+    gargs = tuple(x.to(dev) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
+    gen = torch.Generator().manual_seed(2345)
+    q, k, v, do = ((torch.randn(N, H, D, generator=gen) / 8).to(tdtype).to(dev) for _ in range(4))
+    log(f"{desc}: N={N} E={E} dtype={dtype_name}; host graph+CSR build {t_graph * 1e3:.1f} ms")
+
+    if args.unfused:
+        from bpt_amd import op
+
+        def step():
+            qq, kk, vv = (x.detach().requires_grad_(True) for x in (q, k, v))
+            o = op.bpt_attention(*gargs, qq, kk, vv, fused=False)
+            o.backward(do)
+            return o, qq.grad, kk.grad, vv.grad
+    else:
+        def step():
+            o, lse = graphop.attention_forward(*gargs[4:], q, k, v)
+            dq, dk, dv = graphop.attention_backward(*gargs, q, k, v, o, lse, do)
+            return o, dq, dk, dv
+
+    ref = step()                                   # builds + caches the plans
+    torch.cuda.synchronize()
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / steps
+
+    t_eager = timed(step, args.steps, args.warmup)
+    t_step, mode = t_eager, "eager"
+    t_graph_replay = None
+    if not args.no_graph and not args.unfused:
+        try:
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    step()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                gout = step()
+            g.replay(); torch.cuda.synchronize()
+            g.replay(); torch.cuda.synchronize()
+            same = all(torch.equal(a, b) for a, b in zip(gout, ref))
+            if same:
+                t_graph_replay = timed(g.replay, args.steps, args.warmup)
+                same = all(torch.equal(a, b) for a, b in zip(gout, ref))
+            if same and t_graph_replay < t_step:
+                t_step, mode = t_graph_replay, "hipgraph-replay"
+            elif not same:
+                log("HIP graph replay did not reproduce the eager result; using eager timing")
+        except Exception as exc:          # graph capture is an optimisation of the launch path only
+            log("HIP graph capture unavailable:", exc)
+
+    # ---- per-kernel durations, HIP events recorded by the library around the kernel on its launch stream
+    lib = attn_lib()
+    kernels = {}
+    if not args.unfused:
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(); ev1.record(); torch.cuda.synchronize()
+        for which, name in ((1, "attn_fwd"), (2, "attn_bwd_dst"), (3, "attn_bwd_src")):
+            lib.bpt_profile_kernel(which, ev0.cuda_event, ev1.cuda_event)
+            ts = []
+            for i in range(min(args.steps, 100) + 5):
+                step()
+                torch.cuda.synchronize()
+                if i >= 5:
+                    ts.append(ev0.elapsed_time(ev1))
+            lib.bpt_profile_kernel(0, None, None)
+            kernels[name] = sum(ts) / len(ts)          # ms, average launch duration
+    alg = algorithmic_bytes(N, E, H, D, esize)
+    roofline = None
+    if kernels:
+        dom = max(kernels, key=kernels.get)
+        achieved = alg[dom] / (kernels[dom] * 1e-3) / 1e9
+        traffic = None
+        tpath = os.path.join(ROOT, "profiles", "traffic.json")
+        if os.path.exists(tpath):
+            traffic = json.load(open(tpath)).get(f"{args.workload}-{dtype_name}", {}).get(dom)
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                    "algorithmic_bytes": alg[dom], "avg_launch_ms": round(kernels[dom], 5)}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(src, dst, N, H, D, 2345)
+
+    step_gbs = alg["total"] / t_step / 1e9
+    out = {
+        "metric": "attention edges/s fwd+bwd at n=8192 k=4 8h x64; % of HBM roofline",
+        "value": E / t_step, "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype_name, "data": "synthetic",
+        "config": {"workload": desc + (" (unfused op chain)" if args.unfused else " (fused fwd+bwd)"), "n_nodes": N,
+                   "n_edges": E, "heads": H, "d_head": D, "launch": mode},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "step_roofline": {"algorithmic_bytes": alg["total"], "achieved_GBps": round(step_gbs, 1),
+                          "frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4)},
+        "ms_per_step_eager": t_eager * 1e3,
+        "ms_per_step_graph": None if t_graph_replay is None else t_graph_replay * 1e3,
+        "kernel_ms": {k_: round(v_, 5) for k_, v_ in kernels.items()},
+    }
+    log(json.dumps(out, indent=1))
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

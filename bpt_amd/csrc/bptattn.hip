@@ -33,6 +33,21 @@ constexpr float LOG2E = 1.4426950408889634f;
 
 std::atomic<int> g_force_generic{0};
 
+// optional measurement hook (bpt_profile_kernel): which main kernel to bracket with events
+std::atomic<int> g_prof_which{0};
+std::atomic<void *> g_prof_start{nullptr}, g_prof_stop{nullptr};
+
+struct ProfScope {
+    hipStream_t s;
+    bool on;
+    ProfScope(int which, hipStream_t stream) : s(stream), on(g_prof_which.load(std::memory_order_relaxed) == which) {
+        if (on) (void)hipEventRecord((hipEvent_t)g_prof_start.load(), s);
+    }
+    ~ProfScope() {
+        if (on) (void)hipEventRecord((hipEvent_t)g_prof_stop.load(), s);
+    }
+};
+
 // ------------------------------------------------------------------------------------------
 // element types
 // ------------------------------------------------------------------------------------------
@@ -317,14 +332,17 @@ __device__ __forceinline__ void store_row(T *__restrict__ row, int lane, const f
     }
 }
 
-// f32 partial rows in the workspace use the same lane layout with 4-element vectors
-template <int H, int D>
-__device__ __forceinline__ void store_row_ws(float *__restrict__ row, int lane, const float (&in)[H * D / 64]) {
-    constexpr int LPH = 64 / H, EPL = H * D / 64;
+// f32 partial rows in the workspace are stored in natural column order (the combine kernels
+// index them by column), whatever the element type of the node tensors
+template <typename T, int H, int D>
+__device__ __forceinline__ void store_row_ws(float *__restrict__ row, int lane, const float (&in)[Lay<T, H, D>::EPL]) {
+    using L = Lay<T, H, D>;
 #pragma unroll
-    for (int i = 0; i < EPL / 4; ++i)
-        *reinterpret_cast<float4 *>(row + (lane / LPH) * D + (i * LPH + lane % LPH) * 4) =
-            make_float4(in[4 * i], in[4 * i + 1], in[4 * i + 2], in[4 * i + 3]);
+    for (int i = 0; i < L::NV; ++i)
+#pragma unroll
+        for (int c = 0; c < L::VE / 4; ++c)
+            *reinterpret_cast<float4 *>(row + L::off(lane, i) + 4 * c) =
+                make_float4(in[L::VE * i + 4 * c], in[L::VE * i + 4 * c + 1], in[L::VE * i + 4 * c + 2], in[L::VE * i + 4 * c + 3]);
 }
 
 template <int CTRL> __device__ __forceinline__ float dpp_mov(float x) {
@@ -436,8 +454,8 @@ __global__ __launch_bounds__(BLOCK) void k_spmm_fast(bpt_plan P, const WT *__res
         store_row<T, H, D>(Y0 + (size_t)it.row * L::C, lane, acc0);
         if constexpr (NOUT == 2) store_row<T, H, D>(Y1 + (size_t)it.row * L::C, lane, acc1);
     } else {
-        store_row_ws<H, D>(ws0 + (size_t)it.slot * L::C, lane, acc0);
-        if constexpr (NOUT == 2) store_row_ws<H, D>(ws1 + (size_t)it.slot * L::C, lane, acc1);
+        store_row_ws<T, H, D>(ws0 + (size_t)it.slot * L::C, lane, acc0);
+        if constexpr (NOUT == 2) store_row_ws<T, H, D>(ws1 + (size_t)it.slot * L::C, lane, acc1);
     }
 }
 
@@ -496,7 +514,7 @@ __global__ __launch_bounds__(BLOCK) void k_attn_fwd(bpt_plan P, const T *__restr
         store_row<T, H, D>(o + (size_t)it.row * L::C, lane, acc);
         if (lane % L::LPH == 0) lse[(size_t)it.row * H + head] = l > 0.f ? m + log2f(l) : 0.f;
     } else {
-        store_row_ws<H, D>(ws_acc + (size_t)it.slot * L::C, lane, acc);
+        store_row_ws<T, H, D>(ws_acc + (size_t)it.slot * L::C, lane, acc);
         if (lane % L::LPH == 0) {
             ws_ml[((size_t)it.slot * H + head) * 2] = m;
             ws_ml[((size_t)it.slot * H + head) * 2 + 1] = l;
@@ -581,7 +599,7 @@ __global__ __launch_bounds__(BLOCK) void k_attn_bwd_dst(bpt_plan P, const T *__r
         }
     }
     if (it.slot < 0) store_row<T, H, D>(dq + (size_t)it.row * L::C, lane, dqa);
-    else store_row_ws<H, D>(ws_dq + (size_t)it.slot * L::C, lane, dqa);
+    else store_row_ws<T, H, D>(ws_dq + (size_t)it.slot * L::C, lane, dqa);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -708,8 +726,11 @@ int run_spmm_fast(const bpt_plan *P, const void *W0, const void *X0, void *Y0, c
                   float *ws, hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
     float *ws1 = ws ? ws + (size_t)P->n_slots * H * D : nullptr;
-    hipLaunchKernelGGL((k_spmm_fast<T, WT, H, D, FAST_BATCH, NOUT>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const WT *)W0,
-                       (const T *)X0, (T *)Y0, (const WT *)W1, (const T *)X1, (T *)Y1, ws, ws1);
+    {
+        ProfScope prof(NOUT == 2 ? BPT_KERNEL_ATTN_BWD_SRC : -1, s);
+        hipLaunchKernelGGL((k_spmm_fast<T, WT, H, D, FAST_BATCH, NOUT>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const WT *)W0,
+                           (const T *)X0, (T *)Y0, (const WT *)W1, (const T *)X1, (T *)Y1, ws, ws1);
+    }
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
     hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const float *)ws, (T *)Y0, H * D);
@@ -752,8 +773,11 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     if (P->n_items == 0) return BPT_OK;
     float *ws_acc = (float *)ws;
     float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
-    hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
-                       (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+    {
+        ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
+        hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
+                           (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+    }
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
     hipLaunchKernelGGL((k_attn_fwd_combine<T, H, D>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const float *)ws_acc,
@@ -769,8 +793,12 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     float *pbuf = (float *)ws;
     float *dsbuf = pbuf + round16((int64_t)EH * 4) / 4;
     float *ws_rows = dsbuf + round16((int64_t)EH * 4) / 4;
-    hipLaunchKernelGGL((k_attn_bwd_dst<T, H, D, FAST_BATCH>), dim3(grid_for(Pin)), dim3(BLOCK), 0, s, *Pin, (const T *)q, (const T *)k,
-                       (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pbuf, dsbuf, ws_rows, scale, scale * LOG2E);
+    {
+        ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
+        hipLaunchKernelGGL((k_attn_bwd_dst<T, H, D, FAST_BATCH>), dim3(grid_for(Pin)), dim3(BLOCK), 0, s, *Pin, (const T *)q,
+                           (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pbuf, dsbuf, ws_rows, scale,
+                           scale * LOG2E);
+    }
     int st = launch_status();
     if (st != BPT_OK) return st;
     if (Pin->n_heavy > 0) {
@@ -805,6 +833,14 @@ const char *bpt_strerror(int status) {
 }
 
 int bpt_set_force_generic(int on) { return g_force_generic.exchange(on ? 1 : 0); }
+
+int bpt_profile_kernel(int which, void *start_event, void *stop_event) {
+    if (which != 0 && (!start_event || !stop_event)) return BPT_ERR_NULL;
+    g_prof_start.store(start_event);
+    g_prof_stop.store(stop_event);
+    g_prof_which.store(which);
+    return BPT_OK;
+}
 
 int64_t bpt_workspace_bytes(int op, const bpt_plan *plan, const bpt_plan *plan_t, int h, int d, int dtype) {
     if (!plan || h < 1 || d < 1) return -1;

@@ -57,6 +57,12 @@ const char *bpt_strerror(int status);
 /* 1: force the shape-generic kernels even where a specialised one exists (testing). Returns the old value. */
 int bpt_set_force_generic(int on);
 
+/* Measurement aid (no counterpart in the reference): while `which` is one of BPT_KERNEL_*, every launch
+ * of that main kernel of the fused path is bracketed by hipEventRecord(start_event) / (stop_event) on
+ * the launch stream, so a benchmark can time one kernel with HIP events; 0 switches it off. */
+enum { BPT_KERNEL_NONE = 0, BPT_KERNEL_ATTN_FWD = 1, BPT_KERNEL_ATTN_BWD_DST = 2, BPT_KERNEL_ATTN_BWD_SRC = 3 };
+int bpt_profile_kernel(int which, void *start_event, void *stop_event);
+
 /* Bytes of workspace the call needs (0 possible).  op: one of the BPT_OP_* below. */
 enum {
     BPT_OP_MASKEDMM_BWD = 1, BPT_OP_NODE_MUL_EDGE_BWD = 2, BPT_OP_SPMM_FWD = 3, BPT_OP_SPMM_BWD = 4,
