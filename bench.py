@@ -96,6 +96,8 @@ def main():
     ap.add_argument("--dtype", default=None, choices=[None, "f32", "bf16"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three 256 MiB device-to-device copies (known HBM bytes) so counter runs can be scaled")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -205,6 +207,13 @@ def main():
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                     "algorithmic_bytes": alg[dom], "avg_launch_ms": round(kernels[dom], 5)}
+
+    if args.calibrate_copy:
+        a = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)                    # reads 256 MiB and writes 256 MiB per launch
+        torch.cuda.synchronize()
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -182,15 +182,26 @@ __global__ __launch_bounds__(BLOCK) void k_spmm_generic(bpt_plan P, const T *__r
     }
 }
 
-// Y[row, :] = sum of the row's partial slots, in slot order.  One block per split row.
+// Y[row, :] = sum of the row's partial slots, in slot order.  One block per split row.  Slots are
+// loaded eight at a time (independent loads) and added in slot order, so the result does not depend
+// on the batching.
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void k_combine_sum(const int32_t *__restrict__ heavy,
                                                        const typename Elem<T>::acc_t *__restrict__ ws, T *__restrict__ Y, int C) {
     using acc_t = typename Elem<T>::acc_t;
     const int row = heavy[3 * blockIdx.x], s0 = heavy[3 * blockIdx.x + 1], ns = heavy[3 * blockIdx.x + 2];
     for (int j = threadIdx.x; j < C; j += BLOCK) {
+        const acc_t *col = ws + (size_t)s0 * C + j;
         acc_t s = 0;
-        for (int k = 0; k < ns; ++k) s += ws[(size_t)(s0 + k) * C + j];
+        int k = 0;
+        for (; k + 8 <= ns; k += 8) {
+            acc_t t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = col[(size_t)(k + u) * C];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += t[u];
+        }
+        for (; k < ns; ++k) s += col[(size_t)k * C];
         Elem<T>::st(Y + (size_t)row * C + j, s);
     }
 }
@@ -522,7 +533,8 @@ __global__ __launch_bounds__(BLOCK) void k_attn_fwd(bpt_plan P, const T *__restr
     }
 }
 
-// Combine the (m, l, acc) partials of each split row in slot order.  One block per split row.
+// Combine the (m, l, acc) partials of each split row in slot order.  One block per split row; slots
+// are read eight at a time so the loads of a batch are independent.
 template <typename T, int H, int D>
 __global__ __launch_bounds__(BLOCK) void k_attn_fwd_combine(const int32_t *__restrict__ heavy, const float *__restrict__ ws_acc,
                                                             const float *__restrict__ ws_ml, T *__restrict__ o, float *__restrict__ lse) {
@@ -530,13 +542,38 @@ __global__ __launch_bounds__(BLOCK) void k_attn_fwd_combine(const int32_t *__res
     const int row = heavy[3 * blockIdx.x], s0 = heavy[3 * blockIdx.x + 1], ns = heavy[3 * blockIdx.x + 2];
     for (int j = threadIdx.x; j < C; j += BLOCK) {
         const int head = j / D;
+        const float *ml = ws_ml + ((size_t)s0 * H + head) * 2;      // slot stride 2*H
+        const float *col = ws_acc + (size_t)s0 * C + j;              // slot stride C
         float M = M_INIT_LOG2;
-        for (int kk = 0; kk < ns; ++kk) M = fmaxf(M, ws_ml[((size_t)(s0 + kk) * H + head) * 2]);
+        int kk = 0;
+        for (; kk + 8 <= ns; kk += 8) {
+            float t[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) t[u] = ml[(size_t)(kk + u) * 2 * H];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) M = fmaxf(M, t[u]);
+        }
+        for (; kk < ns; ++kk) M = fmaxf(M, ml[(size_t)kk * 2 * H]);
         float lsum = 0.f, a = 0.f;
-        for (int kk = 0; kk < ns; ++kk) {
-            const float w = __builtin_amdgcn_exp2f(ws_ml[((size_t)(s0 + kk) * H + head) * 2] - M);
-            lsum = fmaf(ws_ml[((size_t)(s0 + kk) * H + head) * 2 + 1], w, lsum);
-            a = fmaf(ws_acc[(size_t)(s0 + kk) * C + j], w, a);
+        for (kk = 0; kk + 8 <= ns; kk += 8) {
+            float tm[8], tl[8], ta[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                tm[u] = ml[(size_t)(kk + u) * 2 * H];
+                tl[u] = ml[(size_t)(kk + u) * 2 * H + 1];
+                ta[u] = col[(size_t)(kk + u) * C];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float w = __builtin_amdgcn_exp2f(tm[u] - M);
+                lsum = fmaf(tl[u], w, lsum);
+                a = fmaf(ta[u], w, a);
+            }
+        }
+        for (; kk < ns; ++kk) {
+            const float w = __builtin_amdgcn_exp2f(ml[(size_t)kk * 2 * H] - M);
+            lsum = fmaf(ml[(size_t)kk * 2 * H + 1], w, lsum);
+            a = fmaf(col[(size_t)kk * C], w, a);
         }
         Elem<T>::st(o + (size_t)row * C + j, lsum > 0.f ? a / lsum : 0.f);
         if (j % D == 0) lse[(size_t)row * H + head] = lsum > 0.f ? M + log2f(lsum) : 0.f;

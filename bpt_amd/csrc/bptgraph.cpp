@@ -337,6 +337,29 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
         }
     }
     info->flags = perm ? 1 : 0;
+    // Locality order: consecutive work items should touch the same neighbour rows, because the
+    // kernels hand consecutive items to the same XCD (shared L2) at about the same time.  Key =
+    // smallest neighbour id of the item.  For the binary-partition graphs this interleaves every
+    // span node with the tokens it covers and spreads the long token rows evenly over the item
+    // list (in plain row order all token rows come first and half of the XCDs get all of them).
+    if (indices && info->n_items > 1) {
+        const int64_t n_items = info->n_items;
+        std::vector<int32_t> key((size_t)n_items), order((size_t)n_items);
+        for (int64_t i = 0; i < n_items; ++i) {
+            const int32_t *it = items + 4 * i;
+            int32_t k = it[0] < n_index_nodes ? it[0] : (int32_t)n_index_nodes;   // empty row: its own id
+            if (it[2] > it[1]) {
+                k = idx32[it[1]];
+                for (int32_t p = it[1] + 1; p < it[2]; ++p) k = std::min(k, idx32[p]);
+            }
+            key[(size_t)i] = k;
+            order[(size_t)i] = (int32_t)i;
+        }
+        std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return key[(size_t)a] < key[(size_t)b]; });
+        std::vector<int32_t> sorted((size_t)n_items * 4);
+        for (int64_t i = 0; i < n_items; ++i) std::memcpy(&sorted[(size_t)i * 4], items + 4 * (int64_t)order[(size_t)i], 4 * sizeof(int32_t));
+        std::memcpy(items, sorted.data(), sorted.size() * sizeof(int32_t));
+    }
     return BPTG_OK;
 }
 

@@ -65,6 +65,8 @@ int bptg_build_csr(const int64_t *rows, const int64_t *cols, int64_t n_edges, in
  *                              and writes results directly; slot >= 0: partial result number
  *   heavy   int32[n_heavy*3]   (row, first_slot, n_slots) for every split row
  * Every node gets at least one item (empty rows too) so kernels can write all outputs.
+ * When `indices` is given the items are ordered by the smallest neighbour id they touch (ties in row
+ * order) so that consecutive items share neighbours; otherwise they are in row order.
  * flags bit0: eid is a permutation of 0..n_edges-1 (every edge output gets written). */
 typedef struct {
     int64_t n_items, n_heavy, n_slots, max_degree, flags;

@@ -66,10 +66,13 @@ def test_plan_properties(L, triu, step, seg):
         items, heavy = arr["items"], arr["heavy"]
         assert info.flags & 1 and info.max_degree == np.diff(indptr).max()
         # items tile every row exactly once, in order, each at most seg long
-        assert np.all(items[:, 2] - items[:, 1] <= seg) and np.all(np.diff(items[:, 0]) >= 0)
+        assert np.all(items[:, 2] - items[:, 1] <= seg)
         assert set(items[:, 0].tolist()) == set(range(n))
+        # locality order: non-decreasing smallest neighbour id (empty rows: their own id)
+        keys = [indices[b:e].min() if e > b else r for r, b, e, _ in items.tolist()]
+        assert np.all(np.diff(keys) >= 0)
         pos = 0
-        for r, b, e, slot in items.tolist():
+        for r, b, e, slot in sorted(items.tolist(), key=lambda it: (it[1], it[2])):
             if e > b:
                 assert b == pos
                 pos = e
@@ -78,6 +81,7 @@ def test_plan_properties(L, triu, step, seg):
         assert pos == E
         # heavy rows: consecutive slots, ceil(deg / seg) each
         slots = items[items[:, 3] >= 0]
+        slots = slots[np.argsort(slots[:, 3])]
         assert np.array_equal(slots[:, 3], np.arange(info.n_slots))
         for r, s0, ns in heavy.tolist():
             assert ns == -(-(indptr[r + 1] - indptr[r]) // seg)
