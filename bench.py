@@ -43,6 +43,9 @@ def make_workload(name):
         return "cfg2: 32 causal BPT graphs, L~U[64,1024] (seed 2345), k=4, 8x64", gs, 8, 64, "f32"
     if name == "cfg3":
         return "cfg3: L=8192 k=4 causal BPT graph, 8x64", [gb.BinaryPartition(8192, True, 4, 10)], 8, 64, "f32"
+    if name.startswith("long-"):            # e.g. long-32768: cfg3's graph family at another length
+        L = int(name[5:])
+        return f"L={L} k=4 causal BPT graph, 8x64", [gb.BinaryPartition(L, True, 4, 10)], 8, 64, "f32"
     if name == "cfg5":
         return "cfg5: L=32768 k=8 causal BPT graph, 16x64", [gb.BinaryPartition(32768, True, 8, 10)], 16, 64, "bf16"
     if name.startswith("cfg4-k"):
@@ -98,6 +101,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies (known HBM bytes) so counter runs can be scaled")
+    ap.add_argument("--rows", action="store_true", help="fused kernels with one wavefront per row (no row groups)")
+    ap.add_argument("--variants", default=None, help="row-group kernel variants fwd,bwd_dst,bwd_src (each 2, 3 or 4)")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -111,6 +116,9 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
+    graphop.set_row_groups(not args.rows)
+    if args.variants:
+        graphop.set_group_variant(*[int(x) for x in args.variants.split(",")])
     desc, graphs, H, D, default_dtype = make_workload(args.workload)
     dtype_name = args.dtype or default_dtype
     tdtype = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
@@ -226,7 +234,8 @@ def main():
         "ms_per_step": t_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype_name, "data": "synthetic",
         "config": {"workload": desc + (" (unfused op chain)" if args.unfused else " (fused fwd+bwd)"), "n_nodes": N,
-                   "n_edges": E, "heads": H, "d_head": D, "launch": mode},
+                   "n_edges": E, "heads": H, "d_head": D, "launch": mode,
+                   "kernels": "per-row" if args.rows else "row-groups" + (f"({args.variants})" if args.variants else "")},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "step_roofline": {"algorithmic_bytes": alg["total"], "achieved_GBps": round(step_gbs, 1),

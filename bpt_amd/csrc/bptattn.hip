@@ -32,6 +32,9 @@ constexpr float M_INIT_LOG2 = -1.4426950408889634e9f;   // -1e9 (graphop_kernel.
 constexpr float LOG2E = 1.4426950408889634f;
 
 std::atomic<int> g_force_generic{0};
+// tuning of the row-group kernels, one value per kernel (fwd, bwd_dst, bwd_src): 4 = batches of four
+// neighbour rows; 2 = batches of two; 3 = batches of two compiled for three waves per SIMD
+std::atomic<int> g_group_variant[3] = {{2}, {2}, {2}};
 
 // optional measurement hook (bpt_profile_kernel): which main kernel to bracket with events
 std::atomic<int> g_prof_which{0};
@@ -182,27 +185,40 @@ __global__ __launch_bounds__(BLOCK) void k_spmm_generic(bpt_plan P, const T *__r
     }
 }
 
-// Y[row, :] = sum of the row's partial slots, in slot order.  One block per split row.  Slots are
-// loaded eight at a time (independent loads) and added in slot order, so the result does not depend
-// on the batching.
+// Y[row, :] = sum of the row's partial slots.  Grid (n_heavy, ceil(C / 64), n_out): one block per split
+// row, 64-column strip and output tensor (output z reads its partials n_slots*C further into the
+// workspace).  Wave w adds slots w, w+4, ... (eight independent loads per step); the four wave sums
+// are then added in wave order, so the result is a fixed function of the plan.
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void k_combine_sum(const int32_t *__restrict__ heavy,
-                                                       const typename Elem<T>::acc_t *__restrict__ ws, T *__restrict__ Y, int C) {
+                                                       const typename Elem<T>::acc_t *__restrict__ ws, T *__restrict__ Y0,
+                                                       T *__restrict__ Y1, int C, size_t ws_stride) {
     using acc_t = typename Elem<T>::acc_t;
+    __shared__ acc_t part[WAVES_PER_BLOCK][WAVE];
     const int row = heavy[3 * blockIdx.x], s0 = heavy[3 * blockIdx.x + 1], ns = heavy[3 * blockIdx.x + 2];
-    for (int j = threadIdx.x; j < C; j += BLOCK) {
-        const acc_t *col = ws + (size_t)s0 * C + j;
-        acc_t s = 0;
-        int k = 0;
-        for (; k + 8 <= ns; k += 8) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int j = blockIdx.y * WAVE + lane;
+    T *Y = blockIdx.z == 0 ? Y0 : Y1;
+    acc_t s = 0;
+    if (j < C) {
+        const acc_t *col = ws + (size_t)blockIdx.z * ws_stride + (size_t)s0 * C + j;
+        int k = w;
+        for (; k + 7 * WAVES_PER_BLOCK < ns; k += 8 * WAVES_PER_BLOCK) {
             acc_t t[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) t[u] = col[(size_t)(k + u) * C];
+            for (int u = 0; u < 8; ++u) t[u] = col[(size_t)(k + u * WAVES_PER_BLOCK) * C];
 #pragma unroll
             for (int u = 0; u < 8; ++u) s += t[u];
         }
-        for (; k < ns; ++k) s += col[(size_t)k * C];
-        Elem<T>::st(Y + (size_t)row * C + j, s);
+        for (; k < ns; k += WAVES_PER_BLOCK) s += col[(size_t)k * C];
+    }
+    part[w][lane] = s;
+    __syncthreads();
+    if (w == 0 && j < C) {
+        acc_t r = part[0][lane];
+#pragma unroll
+        for (int i = 1; i < WAVES_PER_BLOCK; ++i) r += part[i][lane];
+        Elem<T>::st(Y + (size_t)row * C + j, r);
     }
 }
 
@@ -533,50 +549,67 @@ __global__ __launch_bounds__(BLOCK) void k_attn_fwd(bpt_plan P, const T *__restr
     }
 }
 
-// Combine the (m, l, acc) partials of each split row in slot order.  One block per split row; slots
-// are read eight at a time so the loads of a batch are independent.
+// Combine the (m, l, acc) partials of each split row.  Grid (n_heavy, C / 64): one block per split row
+// and 64-column strip; wave w folds slots w, w+4, ... with a running maximum (one pass, eight
+// independent loads per step), then the four wave results are merged in wave order.
 template <typename T, int H, int D>
 __global__ __launch_bounds__(BLOCK) void k_attn_fwd_combine(const int32_t *__restrict__ heavy, const float *__restrict__ ws_acc,
                                                             const float *__restrict__ ws_ml, T *__restrict__ o, float *__restrict__ lse) {
     constexpr int C = H * D;
+    static_assert(C % WAVE == 0, "strip width");
+    __shared__ float pm[WAVES_PER_BLOCK][WAVE], pl[WAVES_PER_BLOCK][WAVE], pa[WAVES_PER_BLOCK][WAVE];
     const int row = heavy[3 * blockIdx.x], s0 = heavy[3 * blockIdx.x + 1], ns = heavy[3 * blockIdx.x + 2];
-    for (int j = threadIdx.x; j < C; j += BLOCK) {
-        const int head = j / D;
-        const float *ml = ws_ml + ((size_t)s0 * H + head) * 2;      // slot stride 2*H
-        const float *col = ws_acc + (size_t)s0 * C + j;              // slot stride C
-        float M = M_INIT_LOG2;
-        int kk = 0;
-        for (; kk + 8 <= ns; kk += 8) {
-            float t[8];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int j = blockIdx.y * WAVE + lane, head = j / D;
+    const float *ml = ws_ml + ((size_t)s0 * H + head) * 2;      // slot stride 2*H
+    const float *col = ws_acc + (size_t)s0 * C + j;              // slot stride C
+    float M = M_INIT_LOG2, lsum = 0.f, a = 0.f;
+    int kk = w;
+    for (; kk + 7 * WAVES_PER_BLOCK < ns; kk += 8 * WAVES_PER_BLOCK) {
+        float tm[8], tl[8], ta[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) t[u] = ml[(size_t)(kk + u) * 2 * H];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) M = fmaxf(M, t[u]);
+        for (int u = 0; u < 8; ++u) {
+            const size_t sl = (size_t)(kk + u * WAVES_PER_BLOCK);
+            tm[u] = ml[sl * 2 * H];
+            tl[u] = ml[sl * 2 * H + 1];
+            ta[u] = col[sl * C];
         }
-        for (; kk < ns; ++kk) M = fmaxf(M, ml[(size_t)kk * 2 * H]);
-        float lsum = 0.f, a = 0.f;
-        for (kk = 0; kk + 8 <= ns; kk += 8) {
-            float tm[8], tl[8], ta[8];
+        float mx = M;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                tm[u] = ml[(size_t)(kk + u) * 2 * H];
-                tl[u] = ml[(size_t)(kk + u) * 2 * H + 1];
-                ta[u] = col[(size_t)(kk + u) * C];
-            }
+        for (int u = 0; u < 8; ++u) mx = fmaxf(mx, tm[u]);
+        const float resc = __builtin_amdgcn_exp2f(M - mx);
+        lsum *= resc;
+        a *= resc;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const float w = __builtin_amdgcn_exp2f(tm[u] - M);
-                lsum = fmaf(tl[u], w, lsum);
-                a = fmaf(ta[u], w, a);
-            }
+        for (int u = 0; u < 8; ++u) {
+            const float wgt = __builtin_amdgcn_exp2f(tm[u] - mx);
+            lsum = fmaf(tl[u], wgt, lsum);
+            a = fmaf(ta[u], wgt, a);
         }
-        for (; kk < ns; ++kk) {
-            const float w = __builtin_amdgcn_exp2f(ml[(size_t)kk * 2 * H] - M);
-            lsum = fmaf(ml[(size_t)kk * 2 * H + 1], w, lsum);
-            a = fmaf(col[(size_t)kk * C], w, a);
+        M = mx;
+    }
+    for (; kk < ns; kk += WAVES_PER_BLOCK) {
+        const float tm = ml[(size_t)kk * 2 * H], mx = fmaxf(M, tm);
+        const float resc = __builtin_amdgcn_exp2f(M - mx), wgt = __builtin_amdgcn_exp2f(tm - mx);
+        lsum = fmaf(ml[(size_t)kk * 2 * H + 1], wgt, lsum * resc);
+        a = fmaf(col[(size_t)kk * C], wgt, a * resc);
+        M = mx;
+    }
+    pm[w][lane] = M; pl[w][lane] = lsum; pa[w][lane] = a;
+    __syncthreads();
+    if (w == 0) {
+        float Mx = pm[0][lane];
+#pragma unroll
+        for (int i = 1; i < WAVES_PER_BLOCK; ++i) Mx = fmaxf(Mx, pm[i][lane]);
+        float L = 0.f, A = 0.f;
+#pragma unroll
+        for (int i = 0; i < WAVES_PER_BLOCK; ++i) {
+            const float wgt = __builtin_amdgcn_exp2f(pm[i][lane] - Mx);
+            L = fmaf(pl[i][lane], wgt, L);
+            A = fmaf(pa[i][lane], wgt, A);
         }
-        Elem<T>::st(o + (size_t)row * C + j, lsum > 0.f ? a / lsum : 0.f);
-        if (j % D == 0) lse[(size_t)row * H + head] = lsum > 0.f ? M + log2f(lsum) : 0.f;
+        Elem<T>::st(o + (size_t)row * C + j, L > 0.f ? A / L : 0.f);
+        if (j % D == 0) lse[(size_t)row * H + head] = L > 0.f ? Mx + log2f(L) : 0.f;
     }
 }
 
@@ -640,6 +673,301 @@ __global__ __launch_bounds__(BLOCK) void k_attn_bwd_dst(bpt_plan P, const T *__r
 }
 
 // ------------------------------------------------------------------------------------------
+// row-group kernels of the fused path: one wavefront owns up to R rows (or row segments) that
+// share neighbours; every neighbour row of the group's union is loaded once and used for all
+// members that have an edge to it (entry mask).  One wavefront per workgroup.
+// ------------------------------------------------------------------------------------------
+template <int R> struct GroupHead {
+    int rows[R], slots[R], begin, end;
+};
+
+template <int R> __device__ __forceinline__ GroupHead<R> fetch_group(const bpt_plan &P, int g) {
+    GroupHead<R> gh;
+#pragma unroll
+    for (int m = 0; m < R; ++m) {
+        gh.rows[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)g * R + m) * 2]);
+        gh.slots[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)g * R + m) * 2 + 1]);
+    }
+    gh.begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[g]);
+    gh.end = __builtin_amdgcn_readfirstlane(P.grp_ptr[g + 1]);
+    return gh;
+}
+
+// All three kernels run the same two-stage software pipeline over the group's entries: while the
+// rows of batch i are being used, the loads of batch i+1 are already in flight (two register
+// buffers, unconditional loads: a batch past the end re-reads the chunk's first row with an empty mask).
+template <typename T, int H, int D, int R, int BATCH, int WPE>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_fwd_grp(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k,
+                                                       const T *__restrict__ v, T *__restrict__ o, float *__restrict__ lse,
+                                                       float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+    using L = Lay<T, H, D>;
+    const int g = xcd_contiguous_block();
+    const int lane = threadIdx.x, head = lane / L::LPH;
+    const GroupHead<R> gh = fetch_group<R>(P, g);
+    float qv[R][L::EPL], acc[R][L::EPL], mrun[R], lrun[R];
+#pragma unroll
+    for (int m = 0; m < R; ++m) {
+        load_row<T, H, D>(q + (size_t)max(gh.rows[m], 0) * L::C, lane, qv[m]);
+        mrun[m] = M_INIT_LOG2;
+        lrun[m] = 0.f;
+#pragma unroll
+        for (int i = 0; i < L::EPL; ++i) { qv[m][i] *= scale_log2e; acc[m][i] = 0.f; }
+    }
+    struct Batch {
+        float kv[BATCH][L::EPL], vv[BATCH][L::EPL];
+        int mk[BATCH], any;
+    };
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
+        const int cnt = min(WAVE, gh.end - p0);
+        const int4 ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
+        auto load_batch = [&](Batch &B, int b) {
+            B.any = 0;
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const bool ok = b + e < cnt;
+                const int j = ok ? b + e : 0;
+                const int src = __builtin_amdgcn_readlane(ent.x, j);
+                B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
+                B.any |= B.mk[e];
+                load_row<T, H, D>(k + (size_t)src * L::C, lane, B.kv[e]);
+                load_row<T, H, D>(v + (size_t)src * L::C, lane, B.vv[e]);
+            }
+        };
+        auto compute = [&](const Batch &B) {
+#pragma unroll
+            for (int m = 0; m < R; ++m) {
+                const int bit = 1 << m;
+                if ((B.any & bit) == 0) continue;
+                float s[BATCH], mx = mrun[m];
+#pragma unroll
+                for (int e = 0; e < BATCH; ++e) {
+                    s[e] = -INFINITY;
+                    if (B.mk[e] & bit) {
+                        s[e] = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], B.kv[e]));
+                        mx = fmaxf(mx, s[e]);
+                    }
+                }
+                const float alpha = __builtin_amdgcn_exp2f(mrun[m] - mx);
+                lrun[m] *= alpha;
+#pragma unroll
+                for (int i = 0; i < L::EPL; ++i) acc[m][i] *= alpha;
+#pragma unroll
+                for (int e = 0; e < BATCH; ++e) {
+                    if (B.mk[e] & bit) {
+                        const float pe = __builtin_amdgcn_exp2f(s[e] - mx);
+                        lrun[m] += pe;
+#pragma unroll
+                        for (int i = 0; i < L::EPL; ++i) acc[m][i] = fmaf(pe, B.vv[e][i], acc[m][i]);
+                    }
+                }
+                mrun[m] = mx;
+            }
+        };
+        Batch A, B;
+        load_batch(A, 0);
+        for (int b = 0; b < cnt; b += 2 * BATCH) {
+            load_batch(B, b + BATCH);
+            issue_loads_first();
+            compute(A);
+            issue_loads_first();
+            load_batch(A, b + 2 * BATCH);
+            issue_loads_first();
+            compute(B);
+            issue_loads_first();
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < R; ++m) {
+        if (gh.rows[m] < 0) continue;
+        if (gh.slots[m] < 0) {
+            const float inv = lrun[m] > 0.f ? 1.f / lrun[m] : 0.f;
+#pragma unroll
+            for (int i = 0; i < L::EPL; ++i) acc[m][i] *= inv;
+            store_row<T, H, D>(o + (size_t)gh.rows[m] * L::C, lane, acc[m]);
+            if (lane % L::LPH == 0) lse[(size_t)gh.rows[m] * H + head] = lrun[m] > 0.f ? mrun[m] + log2f(lrun[m]) : 0.f;
+        } else {
+            store_row_ws<T, H, D>(ws_acc + (size_t)gh.slots[m] * L::C, lane, acc[m]);
+            if (lane % L::LPH == 0) {
+                ws_ml[((size_t)gh.slots[m] * H + head) * 2] = mrun[m];
+                ws_ml[((size_t)gh.slots[m] * H + head) * 2 + 1] = lrun[m];
+            }
+        }
+    }
+}
+
+// Backward, destination side, row groups.  pds[(pair, head)] = (p, ds) in the pair order of the
+// source-side plan (P.grp_pairs maps this plan's pairs to it).
+template <typename T, int H, int D, int R, int BATCH, int WPE>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_dst_grp(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k,
+                                                           const T *__restrict__ v, const T *__restrict__ o, const T *__restrict__ d_o,
+                                                           const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
+                                                           float *__restrict__ ws_dq, float scale, float scale_log2e) {
+    using L = Lay<T, H, D>;
+    const int g = xcd_contiguous_block();
+    const int lane = threadIdx.x, head = lane / L::LPH;
+    const GroupHead<R> gh = fetch_group<R>(P, g);
+    float qv[R][L::EPL], dov[R][L::EPL], dqa[R][L::EPL], delta[R], lse2[R];
+#pragma unroll
+    for (int m = 0; m < R; ++m) {
+        const size_t row = (size_t)max(gh.rows[m], 0);
+        float ov[L::EPL];
+        load_row<T, H, D>(o + row * L::C, lane, ov);
+        load_row<T, H, D>(d_o + row * L::C, lane, dov[m]);
+        load_row<T, H, D>(q + row * L::C, lane, qv[m]);
+        delta[m] = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], ov));
+        lse2[m] = lse[row * H + head];
+#pragma unroll
+        for (int i = 0; i < L::EPL; ++i) dqa[m][i] = 0.f;
+    }
+    struct Batch {
+        float kv[BATCH][L::EPL], vv[BATCH][L::EPL];
+        int mk[BATCH], xp[BATCH], any;
+    };
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    const int last_pair = (int)P.n_edges - 1;
+    for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
+        const int cnt = min(WAVE, gh.end - p0);
+        const int4 ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
+        auto load_batch = [&](Batch &B, int b) {
+            B.any = 0;
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const bool ok = b + e < cnt;
+                const int j = ok ? b + e : 0;
+                const int src = __builtin_amdgcn_readlane(ent.x, j);
+                B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
+                B.any |= B.mk[e];
+                // lane r (< R) fetches the scratch position of this entry's r-th pair
+                B.xp[e] = P.grp_pairs[min(__builtin_amdgcn_readlane(ent.z, j) + (lane & (R - 1)), last_pair)];
+                load_row<T, H, D>(k + (size_t)src * L::C, lane, B.kv[e]);
+                load_row<T, H, D>(v + (size_t)src * L::C, lane, B.vv[e]);
+            }
+        };
+        auto compute = [&](const Batch &B) {
+#pragma unroll
+            for (int m = 0; m < R; ++m) {
+                const int bit = 1 << m;
+                if ((B.any & bit) == 0) continue;
+#pragma unroll
+                for (int e = 0; e < BATCH; ++e) {
+                    if (B.mk[e] & bit) {
+                        const int pos = __builtin_amdgcn_readlane(B.xp[e], __builtin_popcount(B.mk[e] & (bit - 1)));
+                        const float s = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], B.kv[e]));
+                        const float dp = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], B.vv[e]));
+                        const float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
+                        const float ds = pe * (dp - delta[m]) * scale;
+#pragma unroll
+                        for (int i = 0; i < L::EPL; ++i) dqa[m][i] = fmaf(ds, B.kv[e][i], dqa[m][i]);
+                        if (lane % L::LPH == 0) pds[(size_t)pos * H + head] = make_float2(pe, ds);
+                    }
+                }
+            }
+        };
+        Batch A, B;
+        load_batch(A, 0);
+        for (int b = 0; b < cnt; b += 2 * BATCH) {
+            load_batch(B, b + BATCH);
+            issue_loads_first();
+            compute(A);
+            issue_loads_first();
+            load_batch(A, b + 2 * BATCH);
+            issue_loads_first();
+            compute(B);
+            issue_loads_first();
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < R; ++m) {
+        if (gh.rows[m] < 0) continue;
+        if (gh.slots[m] < 0) store_row<T, H, D>(dq + (size_t)gh.rows[m] * L::C, lane, dqa[m]);
+        else store_row_ws<T, H, D>(ws_dq + (size_t)gh.slots[m] * L::C, lane, dqa[m]);
+    }
+}
+
+// Backward, source side, row groups: dK[src] = sum ds * q[dst], dV[src] = sum p * dO[dst]; the (p, ds)
+// of this plan's pair number n sits at pds[n].
+template <typename T, int H, int D, int R, int BATCH, int WPE>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_src_grp(bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o,
+                                                           const float2 *__restrict__ pds, T *__restrict__ dk, T *__restrict__ dv,
+                                                           float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
+    using L = Lay<T, H, D>;
+    const int g = xcd_contiguous_block();
+    const int lane = threadIdx.x, head = lane / L::LPH;
+    const GroupHead<R> gh = fetch_group<R>(P, g);
+    float ak[R][L::EPL], av[R][L::EPL];
+#pragma unroll
+    for (int m = 0; m < R; ++m)
+#pragma unroll
+        for (int i = 0; i < L::EPL; ++i) { ak[m][i] = 0.f; av[m][i] = 0.f; }
+    struct Batch {
+        float qr[BATCH][L::EPL], dr[BATCH][L::EPL];
+        float2 w[BATCH][R];
+        int mk[BATCH];
+    };
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
+        const int cnt = min(WAVE, gh.end - p0);
+        const int4 ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
+        auto load_batch = [&](Batch &B, int b) {
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                const bool ok = b + e < cnt;
+                const int j = ok ? b + e : 0;
+                const int dst = __builtin_amdgcn_readlane(ent.x, j);
+                B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
+                const int pb = __builtin_amdgcn_readlane(ent.z, j);
+                load_row<T, H, D>(q + (size_t)dst * L::C, lane, B.qr[e]);
+                load_row<T, H, D>(d_o + (size_t)dst * L::C, lane, B.dr[e]);
+#pragma unroll
+                for (int m = 0; m < R; ++m) {
+                    B.w[e][m] = make_float2(0.f, 0.f);
+                    if (B.mk[e] & (1 << m)) B.w[e][m] = pds[(size_t)(pb + __builtin_popcount(B.mk[e] & ((1 << m) - 1))) * H + head];
+                }
+            }
+        };
+        auto compute = [&](const Batch &B) {
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+#pragma unroll
+                for (int m = 0; m < R; ++m) {
+                    if (B.mk[e] & (1 << m)) {
+#pragma unroll
+                        for (int i = 0; i < L::EPL; ++i) {
+                            ak[m][i] = fmaf(B.w[e][m].y, B.qr[e][i], ak[m][i]);
+                            av[m][i] = fmaf(B.w[e][m].x, B.dr[e][i], av[m][i]);
+                        }
+                    }
+                }
+            }
+        };
+        Batch A, B;
+        load_batch(A, 0);
+        for (int b = 0; b < cnt; b += 2 * BATCH) {
+            load_batch(B, b + BATCH);
+            issue_loads_first();
+            compute(A);
+            issue_loads_first();
+            load_batch(A, b + 2 * BATCH);
+            issue_loads_first();
+            compute(B);
+            issue_loads_first();
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < R; ++m) {
+        if (gh.rows[m] < 0) continue;
+        if (gh.slots[m] < 0) {
+            store_row<T, H, D>(dk + (size_t)gh.rows[m] * L::C, lane, ak[m]);
+            store_row<T, H, D>(dv + (size_t)gh.rows[m] * L::C, lane, av[m]);
+        } else {
+            store_row_ws<T, H, D>(ws_dk + (size_t)gh.slots[m] * L::C, lane, ak[m]);
+            store_row_ws<T, H, D>(ws_dv + (size_t)gh.slots[m] * L::C, lane, av[m]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
 inline int grid_for(const bpt_plan *p) { return (int)((p->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK); }
@@ -651,6 +979,8 @@ inline int check_plan(const bpt_plan *p, bool need_idx) {
     if (p->n_edges > 0 && (!p->eid || (need_idx && !p->idx))) return BPT_ERR_NULL;
     if (p->n_heavy > 0 && !p->heavy) return BPT_ERR_NULL;
     if (p->n_items < p->n_rows) return BPT_ERR_SIZE;     // every row owns at least one item
+    if (p->n_groups < 0 || p->grp_R < 0 || p->grp_R > 8) return BPT_ERR_SIZE;
+    if (p->n_groups > 0 && (!p->grp_members || !p->grp_ptr || (p->n_edges > 0 && !p->grp_entries))) return BPT_ERR_NULL;
     return BPT_OK;
 }
 
@@ -698,7 +1028,8 @@ int run_spmm_generic(const bpt_plan *P, const void *W, const void *X, void *Y, v
     hipLaunchKernelGGL((k_spmm_generic<T, MODE>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)W, (const T *)X, (T *)Y, (acc_t *)ws, h, d);
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
-    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const acc_t *)ws, (T *)Y, h * d);
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy, (h * d + WAVE - 1) / WAVE, 1), dim3(BLOCK), 0, s, P->heavy,
+                       (const acc_t *)ws, (T *)Y, (T *)nullptr, h * d, (size_t)0);
     return launch_status();
 }
 
@@ -770,10 +1101,8 @@ int run_spmm_fast(const bpt_plan *P, const void *W0, const void *X0, void *Y0, c
     }
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
-    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const float *)ws, (T *)Y0, H * D);
-    st = launch_status();
-    if (st != BPT_OK || NOUT == 1) return st;
-    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const float *)ws1, (T *)Y1, H * D);
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy, H * D / WAVE, NOUT), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
+                       (T *)Y0, (T *)Y1, H * D, (size_t)P->n_slots * H * D);
     return launch_status();
 }
 
@@ -805,6 +1134,12 @@ int spmm(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int
 
 inline int64_t round16(int64_t b) { return (b + 15) & ~(int64_t)15; }
 
+constexpr int GROUP_R = 4;
+
+inline bool has_groups(const bpt_plan *P) {
+    return P->n_groups > 0 && P->grp_R == GROUP_R && P->grp_members && P->grp_ptr && P->grp_entries;
+}
+
 template <typename T, int H, int D>
 int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v, void *o, float *lse, void *ws, float scale, hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
@@ -812,13 +1147,68 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
-        hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
-                           (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+        if (has_groups(P)) {
+#define LAUNCH_FWD_GRP(B, W)                                                                                                   \
+    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, GROUP_R, B, W>), dim3((int)P->n_groups), dim3(WAVE), 0, s, *P, (const T *)q,   \
+                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E)
+            const int var = g_group_variant[0].load(std::memory_order_relaxed);
+            if (var == 4) LAUNCH_FWD_GRP(4, 1);
+            else if (var == 3) LAUNCH_FWD_GRP(2, 3);
+            else LAUNCH_FWD_GRP(2, 1);
+#undef LAUNCH_FWD_GRP
+        } else {
+            hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
+                               (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+        }
     }
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
-    hipLaunchKernelGGL((k_attn_fwd_combine<T, H, D>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, (const float *)ws_acc,
-                       (const float *)ws_ml, (T *)o, lse);
+    hipLaunchKernelGGL((k_attn_fwd_combine<T, H, D>), dim3((int)P->n_heavy, H * D / WAVE), dim3(BLOCK), 0, s, P->heavy,
+                       (const float *)ws_acc, (const float *)ws_ml, (T *)o, lse);
+    return launch_status();
+}
+
+template <typename T, int H, int D>
+int run_attn_bwd_grouped(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
+                         const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
+    const size_t EH = (size_t)Pin->n_edges * H;
+    float2 *pds = (float2 *)ws;
+    float *ws_rows = (float *)ws + 2 * (round16((int64_t)EH * 4) / 4);
+    {
+        ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
+#define LAUNCH_DST_GRP(B, W)                                                                                                       \
+    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, GROUP_R, B, W>), dim3((int)Pin->n_groups), dim3(WAVE), 0, s, *Pin, (const T *)q, \
+                       (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E)
+        const int var = g_group_variant[1].load(std::memory_order_relaxed);
+        if (var == 4) LAUNCH_DST_GRP(4, 1);
+        else if (var == 3) LAUNCH_DST_GRP(2, 3);
+        else LAUNCH_DST_GRP(2, 1);
+#undef LAUNCH_DST_GRP
+    }
+    int st = launch_status();
+    if (st != BPT_OK) return st;
+    if (Pin->n_heavy > 0) {
+        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, Pin->heavy,
+                           (const float *)ws_rows, (T *)dq, (T *)nullptr, H * D, (size_t)0);
+        st = launch_status();
+        if (st != BPT_OK) return st;
+    }
+    float *ws_dk = ws_rows, *ws_dv = ws_rows + (size_t)Pout->n_slots * H * D;
+    {
+        ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
+#define LAUNCH_SRC_GRP(B, W)                                                                                                          \
+    hipLaunchKernelGGL((k_attn_bwd_src_grp<T, H, D, GROUP_R, B, W>), dim3((int)Pout->n_groups), dim3(WAVE), 0, s, *Pout, (const T *)q, \
+                       (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv)
+        const int var = g_group_variant[2].load(std::memory_order_relaxed);
+        if (var == 4) LAUNCH_SRC_GRP(4, 1);
+        else if (var == 3) LAUNCH_SRC_GRP(2, 3);
+        else LAUNCH_SRC_GRP(2, 1);
+#undef LAUNCH_SRC_GRP
+    }
+    st = launch_status();
+    if (st != BPT_OK || Pout->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pout->n_heavy, H * D / WAVE, 2), dim3(BLOCK), 0, s, Pout->heavy,
+                       (const float *)ws_dk, (T *)dk, (T *)dv, H * D, (size_t)Pout->n_slots * H * D);
     return launch_status();
 }
 
@@ -826,6 +1216,8 @@ template <typename T, int H, int D>
 int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
                  const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
     if (Pin->n_items == 0) return BPT_OK;
+    if (has_groups(Pin) && has_groups(Pout) && Pin->grp_pairs)
+        return run_attn_bwd_grouped<T, H, D>(Pin, Pout, q, k, v, o, d_o, lse, dq, dk, dv, ws, scale, s);
     const size_t EH = (size_t)Pin->n_edges * H;
     float *pbuf = (float *)ws;
     float *dsbuf = pbuf + round16((int64_t)EH * 4) / 4;
@@ -839,7 +1231,8 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     int st = launch_status();
     if (st != BPT_OK) return st;
     if (Pin->n_heavy > 0) {
-        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy), dim3(BLOCK), 0, s, Pin->heavy, (const float *)ws_rows, (T *)dq, H * D);
+        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, Pin->heavy,
+                           (const float *)ws_rows, (T *)dq, (T *)nullptr, H * D, (size_t)0);
         st = launch_status();
         if (st != BPT_OK) return st;
     }
@@ -870,6 +1263,12 @@ const char *bpt_strerror(int status) {
 }
 
 int bpt_set_force_generic(int on) { return g_force_generic.exchange(on ? 1 : 0); }
+
+int bpt_set_group_variant(int kernel, int variant) {
+    if (kernel < 0 || kernel > 2 || (variant != 2 && variant != 3 && variant != 4)) return BPT_ERR_SIZE;
+    g_group_variant[kernel].store(variant);
+    return BPT_OK;
+}
 
 int bpt_profile_kernel(int which, void *start_event, void *stop_event) {
     if (which != 0 && (!start_event || !stop_event)) return BPT_ERR_NULL;

@@ -363,4 +363,126 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
     return BPTG_OK;
 }
 
+// ---- row groups --------------------------------------------------------------------------------
+// Greedy clustering of work items (rows / row segments) that read mostly the same neighbour rows.
+// Items are visited in locality order; an item opens a group and the next `window` unused items
+// join it while at least half of their neighbours are already in the group's union (at most R
+// members).  For every group the union of neighbour ids becomes a list of entries
+// (idx, member mask, first pair); a pair = one original edge = (entry, member).  Pairs are numbered
+// entry by entry, members ascending — the order in which the kernels visit them.
+int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32, const int32_t *eid32,
+                    int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window,
+                    int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid,
+                    int64_t *n_groups_out, int64_t *n_entries_out) {
+    if (!items || !members || !grp_ptr || !n_groups_out || !n_entries_out) return BPTG_ERR_NULL;
+    if (n_edges > 0 && (!idx32 || !eid32 || !entries || !pair_eid)) return BPTG_ERR_NULL;
+    if (n_items < 0 || n_edges < 0 || n_index_nodes < 0) return BPTG_ERR_SIZE;
+    if (R < 1 || R > 8 || window < 0) return BPTG_ERR_ARG;
+    for (int64_t i = 0; i < n_items; ++i) {
+        const int32_t *it = items + 4 * i;
+        if (it[1] < 0 || it[2] < it[1] || it[2] > n_edges) return BPTG_ERR_RANGE;
+    }
+    for (int64_t p = 0; p < n_edges; ++p)
+        if (idx32[p] < 0 || idx32[p] >= n_index_nodes) return BPTG_ERR_RANGE;
+
+    // locality order of the items (they may already be sorted; sorting again is cheap and makes the
+    // function independent of the caller's order)
+    std::vector<int32_t> key((size_t)n_items), order((size_t)n_items);
+    for (int64_t i = 0; i < n_items; ++i) {
+        const int32_t *it = items + 4 * i;
+        int32_t k = INT32_MAX;
+        for (int32_t p = it[1]; p < it[2]; ++p) k = std::min(k, idx32[p]);
+        key[(size_t)i] = k;
+        order[(size_t)i] = (int32_t)i;
+    }
+    std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return key[(size_t)a] < key[(size_t)b]; });
+
+    std::vector<uint8_t> used((size_t)n_items, 0);
+    std::vector<int64_t> stamp((size_t)n_index_nodes, -1);     // stamp[node] == group id  <=>  node in the union
+    struct Triple { int32_t idx, member, eid; };
+    std::vector<Triple> tri;
+    std::vector<int32_t> grp_items;
+    int64_t n_groups = 0, n_entries = 0, n_pairs = 0;
+    grp_ptr[0] = 0;
+    for (int64_t oi = 0; oi < n_items; ++oi) {
+        const int32_t first = order[(size_t)oi];
+        if (used[(size_t)first]) continue;
+        used[(size_t)first] = 1;
+        grp_items.clear();
+        grp_items.push_back(first);
+        {
+            const int32_t *it = items + 4 * (int64_t)first;
+            for (int32_t p = it[1]; p < it[2]; ++p) stamp[(size_t)idx32[p]] = n_groups;
+        }
+        int32_t seen = 0;
+        for (int64_t oj = oi + 1; oj < n_items && (int32_t)grp_items.size() < R && seen < window; ++oj) {
+            const int32_t cand = order[(size_t)oj];
+            if (used[(size_t)cand]) continue;
+            ++seen;
+            const int32_t *it = items + 4 * (int64_t)cand;
+            const int32_t len = it[2] - it[1];
+            if (len == 0) continue;
+            int32_t hit = 0;
+            for (int32_t p = it[1]; p < it[2]; ++p) hit += (stamp[(size_t)idx32[p]] == n_groups);
+            if (2 * hit >= len) {
+                used[(size_t)cand] = 1;
+                grp_items.push_back(cand);
+                for (int32_t p = it[1]; p < it[2]; ++p) stamp[(size_t)idx32[p]] = n_groups;
+            }
+        }
+        // members in ascending item order (deterministic, independent of the join order)
+        std::sort(grp_items.begin(), grp_items.end());
+        tri.clear();
+        for (int32_t m = 0; m < R; ++m) {
+            int32_t *mem = members + ((int64_t)n_groups * R + m) * 2;
+            if (m < (int32_t)grp_items.size()) {
+                const int32_t *it = items + 4 * (int64_t)grp_items[(size_t)m];
+                mem[0] = it[0];
+                mem[1] = it[3];
+                for (int32_t p = it[1]; p < it[2]; ++p) tri.push_back({idx32[p], m, eid32[p]});
+            } else {
+                mem[0] = -1;
+                mem[1] = -1;
+            }
+        }
+        std::stable_sort(tri.begin(), tri.end(), [](const Triple &a, const Triple &b) {
+            return a.idx != b.idx ? a.idx < b.idx : a.member < b.member;
+        });
+        // one run of equal idx -> as many entries as the largest multiplicity among the members
+        size_t a = 0;
+        while (a < tri.size()) {
+            size_t b = a;
+            int32_t cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            size_t start[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            while (b < tri.size() && tri[b].idx == tri[a].idx) {
+                if (cnt[tri[b].member] == 0) start[tri[b].member] = b;
+                ++cnt[tri[b].member];
+                ++b;
+            }
+            int32_t mult = 0;
+            for (int32_t m = 0; m < R; ++m) mult = std::max(mult, cnt[m]);
+            for (int32_t t = 0; t < mult; ++t) {
+                int32_t mask = 0;
+                int32_t *en = entries + 4 * n_entries;
+                en[0] = tri[a].idx;
+                en[2] = (int32_t)n_pairs;
+                en[3] = 0;
+                for (int32_t m = 0; m < R; ++m)
+                    if (cnt[m] > t) {
+                        mask |= 1 << m;
+                        pair_eid[n_pairs++] = tri[start[m] + (size_t)t].eid;
+                    }
+                en[1] = mask;
+                ++n_entries;
+            }
+            a = b;
+        }
+        ++n_groups;
+        grp_ptr[n_groups] = (int32_t)n_entries;
+    }
+    *n_groups_out = n_groups;
+    *n_entries_out = n_entries;
+    return BPTG_OK;
+}
+
 }  // extern "C"

@@ -226,6 +226,8 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None):
     h, d = _hd(q)
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
+    if _USE_GROUPS:
+        plan.ensure_groups()
     o = torch.empty_like(q)
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
@@ -249,11 +251,31 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dt = _dtype(q)
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device)
+    in_ref = plan_in.ref
+    if _USE_GROUPS and plan_in.covers_all_edges and plan_out.covers_all_edges:
+        in_ref = ctypes.byref(plan_in.linked_to(plan_out))
     with torch.cuda.device_of(q):
-        check_attn(_LIB.bpt_attention_backward(plan_in.ref, plan_out.ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do),
+        check_attn(_LIB.bpt_attention_backward(in_ref, plan_out.ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do),
                                                _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
                                                scale, h, d, dt, _stream()), "attention_backward")
     return dq, dk, dv
+
+
+_USE_GROUPS = True
+
+
+def set_row_groups(on):
+    """Fused attention: let one wavefront own several rows that share neighbours (default) or one row each."""
+    global _USE_GROUPS
+    old, _USE_GROUPS = _USE_GROUPS, bool(on)
+    return old
+
+
+def set_group_variant(fwd=None, bwd_dst=None, bwd_src=None):
+    """Tuning of the row-group kernels (see bpt_set_group_variant): 4, 2 or 3 per kernel; None keeps the current one."""
+    for kernel, var in enumerate((fwd, bwd_dst, bwd_src)):
+        if var is not None:
+            check_attn(_LIB.bpt_set_group_variant(kernel, int(var)), "set_group_variant")
 
 
 def set_force_generic(on):

@@ -17,6 +17,8 @@ import torch
 from ._lib import PlanInfo, PlanStruct, check_graph, graph_lib
 
 DEFAULT_SEG_LEN = 64
+GROUP_R = 4            # rows per wavefront in the fused row-group kernels (matches the HIP library)
+GROUP_WINDOW = 32      # how many following items the greedy grouping examines per group
 _CACHE_SIZE = 64
 
 
@@ -58,6 +60,25 @@ def build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len=DE
     return arrays, info
 
 
+def build_groups_host(arrays, n_index_nodes, R=GROUP_R, window=GROUP_WINDOW):
+    """Pure host step: clusters the plan's items into row groups (bptg_group_plan).  Returns a dict
+    with members (n_groups, R, 2), grp_ptr (n_groups + 1), entries (n_entries, 4), pair_eid (n_edges)."""
+    items = np.ascontiguousarray(arrays["items"], dtype=np.int32)
+    idx = np.ascontiguousarray(arrays["idx"], dtype=np.int32)
+    eid = np.ascontiguousarray(arrays["eid"], dtype=np.int32)
+    n_items, E = len(items), len(eid)
+    members = np.empty((max(n_items, 1), R, 2), dtype=np.int32)
+    grp_ptr = np.empty(n_items + 1, dtype=np.int32)
+    entries = np.empty((max(E, 1), 4), dtype=np.int32)
+    pair_eid = np.empty(max(E, 1), dtype=np.int32)
+    ng, ne = ctypes.c_int64(), ctypes.c_int64()
+    check_graph(graph_lib().bptg_group_plan(_ptr(items), n_items, _ptr(idx), _ptr(eid), E, int(n_index_nodes), R, window,
+                                            _ptr(members), _ptr(grp_ptr), _ptr(entries), _ptr(pair_eid),
+                                            ctypes.byref(ng), ctypes.byref(ne)))
+    return {"members": members[:ng.value].copy(), "grp_ptr": grp_ptr[:ng.value + 1].copy(),
+            "entries": entries[:ne.value].copy(), "pair_eid": pair_eid[:E].copy()}
+
+
 class Plan:
     """Device-resident plan of one CSR side; `.struct` is the `bpt_plan` passed to the C ABI."""
 
@@ -69,6 +90,11 @@ class Plan:
         self.covers_all_edges = bool(info.flags & 1)
         self.has_indices = indices is not None
         self.device = torch.device(device)
+        self.n_index_nodes = int(n_index_nodes)
+        self._host = arrays                  # kept for the (lazy) row-group construction
+        self._groups = None
+        self._links = {}
+        self._lock = threading.Lock()
         # one allocation, 256-byte aligned sections (the items array is read as 16-byte vectors)
         self._dev = {k: torch.from_numpy(v).to(self.device) for k, v in arrays.items()}
         d = self._dev
@@ -81,6 +107,43 @@ class Plan:
     @property
     def ref(self):
         return ctypes.byref(self.struct)
+
+    # ---- row groups for the fused attention kernels ----
+    def ensure_groups(self):
+        """Builds the row-group arrays once (host) and uploads them; returns the host dict."""
+        with self._lock:
+            if self._groups is None:
+                grp = build_groups_host(self._host, self.n_index_nodes)
+                self._grp_dev = {k: torch.from_numpy(v).to(self.device) for k, v in grp.items() if k != "pair_eid"}
+                d = self._grp_dev
+                self.n_groups = len(grp["members"])
+                self.struct.grp_members = d["members"].data_ptr() if self.n_groups else None
+                self.struct.grp_ptr = d["grp_ptr"].data_ptr()
+                self.struct.grp_entries = d["entries"].data_ptr() if len(grp["entries"]) else None
+                self.struct.grp_pairs = None
+                self.struct.n_groups = self.n_groups
+                self.struct.grp_R = GROUP_R
+                self._groups = grp
+        return self._groups
+
+    def linked_to(self, plan_src):
+        """`bpt_plan` of this (destination-side) plan whose grp_pairs maps each of its pairs to the number of
+        the same edge's pair in `plan_src` (the source-side plan of the same graph)."""
+        mine, theirs = self.ensure_groups(), plan_src.ensure_groups()
+        key = id(plan_src)
+        with self._lock:
+            hit = self._links.get(key)
+            if hit is None:
+                if self.n_edges != plan_src.n_edges or not (self.covers_all_edges and plan_src.covers_all_edges):
+                    raise ValueError("the two plans do not describe the same edge set")
+                pos_of_eid = np.empty(self.n_edges, dtype=np.int32)
+                pos_of_eid[theirs["pair_eid"]] = np.arange(self.n_edges, dtype=np.int32)
+                pairs = torch.from_numpy(pos_of_eid[mine["pair_eid"]]).to(self.device)
+                st = PlanStruct.from_buffer_copy(self.struct)
+                st.grp_pairs = pairs.data_ptr() if self.n_edges else None
+                hit = (st, pairs, plan_src)          # keeps the mapping and the partner alive
+                self._links[key] = hit
+        return hit[0]
 
 
 class PlanCache:

@@ -42,7 +42,9 @@ typedef enum {
     BPT_ERR_UNSUPPORTED = -7  /* combination not implemented (e.g. fused attention in f64) */
 } bpt_status;
 
-/* Device-resident plan of one CSR side (see bptg_plan_fill for the array contents). */
+/* Device-resident plan of one CSR side (see bptg_plan_fill / bptg_group_plan for the array contents).
+ * The grp_* fields are optional (n_groups == 0: none); the fused attention entries use them to let one
+ * wavefront own up to grp_R rows that share neighbours, loading each neighbour row once for all. */
 typedef struct {
     const int32_t *rowptr;   /* n_rows + 1 */
     const int32_t *idx;      /* n_edges : other endpoint of the edge in slot p */
@@ -50,12 +52,24 @@ typedef struct {
     const int32_t *items;    /* n_items * 4 : row, begin, end, slot */
     const int32_t *heavy;    /* n_heavy * 3 : row, first_slot, n_slots (may be NULL if n_heavy == 0) */
     int64_t n_rows, n_edges, n_items, n_heavy, n_slots;
+    const int32_t *grp_members;  /* n_groups * grp_R * 2 : (row, slot), row = -1 unused */
+    const int32_t *grp_ptr;      /* n_groups + 1 : entry range of each group */
+    const int32_t *grp_entries;  /* n_entries * 4 : neighbour id, member mask, first pair, 0 */
+    const int32_t *grp_pairs;    /* n_edges or NULL.  On the destination-side plan of the fused backward:
+                                    for every pair of this plan, the number of the same edge's pair in the
+                                    source-side plan (the per-edge scratch is laid out in that order) */
+    int64_t n_groups, grp_R;
 } bpt_plan;
 
 const char *bpt_strerror(int status);
 
 /* 1: force the shape-generic kernels even where a specialised one exists (testing). Returns the old value. */
 int bpt_set_force_generic(int on);
+
+/* Tuning knob of the row-group kernels.  kernel: 0 forward, 1 backward destination side, 2 backward source
+ * side.  variant: 4 = load batches of four neighbour rows, 2 = batches of two, 3 = batches of two compiled
+ * for three resident wavefronts per SIMD. */
+int bpt_set_group_variant(int kernel, int variant);
 
 /* Measurement aid (no counterpart in the reference): while `which` is one of BPT_KERNEL_*, every launch
  * of that main kernel of the fused path is bracketed by hipEventRecord(start_event) / (stop_event) on

@@ -80,6 +80,22 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
                    int32_t *rowptr, int32_t *idx32, int32_t *eid32, int32_t *items, int32_t *heavy,
                    bptg_plan_info *info);
 
+/* ---- row groups ------------------------------------------------------------------------------
+ * Clusters the plan's items (rows / row segments) into groups of at most R (<= 8) members that read
+ * mostly the same neighbour rows, so that one wavefront can load each neighbour row once for all of
+ * them.  Inputs are the arrays bptg_plan_fill produced.  Outputs (caller allocates the upper bounds
+ * given in brackets):
+ *   members  int32[n_items*R*2]   per group R x (row, slot); row = -1 for an unused member
+ *   grp_ptr  int32[n_items+1]     entry range of each group
+ *   entries  int32[n_edges*4]     (neighbour id, member bit mask, first pair, 0)
+ *   pair_eid int32[n_edges]       edge id of every pair; pairs are numbered entry by entry, members
+ *                                 ascending, and every edge of the plan appears exactly once
+ * A neighbour that a member reaches through several parallel edges gets one entry per multiplicity. */
+int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32, const int32_t *eid32,
+                    int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window,
+                    int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid,
+                    int64_t *n_groups, int64_t *n_entries);
+
 #ifdef __cplusplus
 }
 #endif
