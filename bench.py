@@ -102,6 +102,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies (known HBM bytes) so counter runs can be scaled")
     ap.add_argument("--rows", action="store_true", help="fused kernels with one wavefront per row (no row groups)")
+    ap.add_argument("--waves", default=None, help="persistent wavefronts per XCD fwd,bwd_dst,bwd_src (0 = one per group)")
     ap.add_argument("--variants", default=None, help="row-group kernel variants fwd,bwd_dst,bwd_src (each 2, 3 or 4)")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
     args = ap.parse_args()
@@ -117,6 +118,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
     graphop.set_row_groups(not args.rows)
+    if args.waves:
+        graphop.set_group_waves(*[int(x) for x in args.waves.split(",")])
     if args.variants:
         graphop.set_group_variant(*[int(x) for x in args.variants.split(",")])
     desc, graphs, H, D, default_dtype = make_workload(args.workload)

@@ -31,8 +31,8 @@ def build_graph(verbose=True):
     return GRAPH_SO
 
 
-def build_attn(verbose=True, extra=()):
-    cmd = [HIPCC] + HIP_FLAGS + list(extra) + [os.path.join(CSRC, "bptattn.hip"), "-o", ATTN_SO]
+def build_attn(verbose=True, extra=(), out=None):
+    cmd = [HIPCC] + HIP_FLAGS + list(extra) + [os.path.join(CSRC, "bptattn.hip"), "-o", out or ATTN_SO]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

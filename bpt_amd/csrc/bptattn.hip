@@ -35,6 +35,8 @@ std::atomic<int> g_force_generic{0};
 // tuning of the row-group kernels, one value per kernel (fwd, bwd_dst, bwd_src): 4 = batches of four
 // neighbour rows; 2 = batches of two; 3 = batches of two compiled for three waves per SIMD
 std::atomic<int> g_group_variant[3] = {{2}, {2}, {2}};
+// wavefronts per XCD that walk the groups of that XCD's chunk (0: one wavefront per group)
+std::atomic<int> g_group_waves[3] = {{0}, {0}, {0}};
 
 // optional measurement hook (bpt_profile_kernel): which main kernel to bracket with events
 std::atomic<int> g_prof_which{0};
@@ -693,278 +695,319 @@ template <int R> __device__ __forceinline__ GroupHead<R> fetch_group(const bpt_p
     return gh;
 }
 
-// All three kernels run the same two-stage software pipeline over the group's entries: while the
-// rows of batch i are being used, the loads of batch i+1 are already in flight (two register
-// buffers, unconditional loads: a batch past the end re-reads the chunk's first row with an empty mask).
-template <typename T, int H, int D, int R, int BATCH, int WPE>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_fwd_grp(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k,
-                                                       const T *__restrict__ v, T *__restrict__ o, float *__restrict__ lse,
-                                                       float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
-    using L = Lay<T, H, D>;
-    const int g = xcd_contiguous_block();
-    const int lane = threadIdx.x, head = lane / L::LPH;
-    const GroupHead<R> gh = fetch_group<R>(P, g);
-    float qv[R][L::EPL], acc[R][L::EPL], mrun[R], lrun[R];
-#pragma unroll
-    for (int m = 0; m < R; ++m) {
-        load_row<T, H, D>(q + (size_t)max(gh.rows[m], 0) * L::C, lane, qv[m]);
-        mrun[m] = M_INIT_LOG2;
-        lrun[m] = 0.f;
-#pragma unroll
-        for (int i = 0; i < L::EPL; ++i) { qv[m][i] *= scale_log2e; acc[m][i] = 0.f; }
+// Persistent walk over the groups of one XCD chunk.  Workgroup b (one wavefront) runs on XCD b % 8; it
+// takes the groups first + b/8, + stride, + 2*stride, ... of that XCD's chunk, stride = gridDim.x / 8.
+// A group costs a chain of dependent loads before its first FMA (header -> entries -> rows); the walk
+// hides it by fetching the header two groups ahead and the first 64 entries one group ahead.  With
+// gridDim.x = 8 * (largest chunk) every wavefront gets exactly one group.
+template <int R, class Body>
+__device__ __forceinline__ void walk_groups(const bpt_plan &P, Body &&body) {
+    const int x = blockIdx.x & 7, w = blockIdx.x >> 3, stride = gridDim.x >> 3;
+    const int first = __builtin_amdgcn_readfirstlane(P.grp_chunks[x]), last = __builtin_amdgcn_readfirstlane(P.grp_chunks[x + 1]);
+    int g = first + w;
+    if (g >= last) return;
+    const int lane = threadIdx.x;
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    GroupHead<R> cur = fetch_group<R>(P, g);
+    GroupHead<R> nxt = fetch_group<R>(P, min(g + stride, last - 1));
+    int4 ent_cur = lane < min(WAVE, cur.end - cur.begin) ? entries[cur.begin + lane] : make_int4(0, 0, 0, 0);
+    for (; g < last; g += stride) {
+        const GroupHead<R> nn = fetch_group<R>(P, min(g + 2 * stride, last - 1));
+        const int ncnt = g + stride < last ? min(WAVE, nxt.end - nxt.begin) : 0;
+        const int4 ent_nxt = lane < ncnt ? entries[nxt.begin + lane] : make_int4(0, 0, 0, 0);
+        body(cur, ent_cur);
+        cur = nxt;
+        nxt = nn;
+        ent_cur = ent_nxt;
     }
+}
+
+// All three kernels run the same two-stage software pipeline over a group's entries: while the rows
+// of batch i are being used, the loads of batch i+1 are already in flight (two register buffers,
+// unconditional loads: a batch past the end re-reads the chunk's first row with an empty mask).
+template <typename T, int H, int D, int R, int BATCH, int WPE>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_fwd_grp(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
+    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+    using L = Lay<T, H, D>;
+    const int lane = threadIdx.x, head = lane / L::LPH;
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     struct Batch {
         float kv[BATCH][L::EPL], vv[BATCH][L::EPL];
         int mk[BATCH], any;
     };
-    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
-    for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
-        const int cnt = min(WAVE, gh.end - p0);
-        const int4 ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
-        auto load_batch = [&](Batch &B, int b) {
-            B.any = 0;
+    walk_groups<R>(P, [&](const GroupHead<R> &gh, const int4 &ent0) {
+        float qv[R][L::EPL], acc[R][L::EPL], mrun[R], lrun[R];
 #pragma unroll
-            for (int e = 0; e < BATCH; ++e) {
-                const bool ok = b + e < cnt;
-                const int j = ok ? b + e : 0;
-                const int src = __builtin_amdgcn_readlane(ent.x, j);
-                B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
-                B.any |= B.mk[e];
-                load_row<T, H, D>(k + (size_t)src * L::C, lane, B.kv[e]);
-                load_row<T, H, D>(v + (size_t)src * L::C, lane, B.vv[e]);
-            }
-        };
-        auto compute = [&](const Batch &B) {
+        for (int m = 0; m < R; ++m) {
+            load_row<T, H, D>(q + (size_t)max(gh.rows[m], 0) * L::C, lane, qv[m]);
+            mrun[m] = M_INIT_LOG2;
+            lrun[m] = 0.f;
 #pragma unroll
-            for (int m = 0; m < R; ++m) {
-                const int bit = 1 << m;
-                if ((B.any & bit) == 0) continue;
-                float s[BATCH], mx = mrun[m];
+            for (int i = 0; i < L::EPL; ++i) { qv[m][i] *= scale_log2e; acc[m][i] = 0.f; }
+        }
+        for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
+            const int cnt = min(WAVE, gh.end - p0);
+            int4 ent = ent0;
+            if (p0 != gh.begin) ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
+            auto load_batch = [&](Batch &B, int b) {
+                B.any = 0;
 #pragma unroll
                 for (int e = 0; e < BATCH; ++e) {
-                    s[e] = -INFINITY;
-                    if (B.mk[e] & bit) {
-                        s[e] = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], B.kv[e]));
-                        mx = fmaxf(mx, s[e]);
-                    }
+                    const bool ok = b + e < cnt;
+                    const int j = ok ? b + e : 0;
+                    const int src = __builtin_amdgcn_readlane(ent.x, j);
+                    B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
+                    B.any |= B.mk[e];
+#ifdef BPT_PROBE_NO_LOADS
+#pragma unroll
+                    for (int i = 0; i < L::EPL; ++i) { B.kv[e][i] = qv[0][i] + (float)src; B.vv[e][i] = qv[1][i] - (float)src; }
+#else
+                    load_row<T, H, D>(k + (size_t)src * L::C, lane, B.kv[e]);
+                    load_row<T, H, D>(v + (size_t)src * L::C, lane, B.vv[e]);
+#endif
                 }
-                const float alpha = __builtin_amdgcn_exp2f(mrun[m] - mx);
-                lrun[m] *= alpha;
+            };
+            auto compute = [&](const Batch &B) {
+#ifdef BPT_PROBE_NO_MATH
 #pragma unroll
-                for (int i = 0; i < L::EPL; ++i) acc[m][i] *= alpha;
+                for (int e = 0; e < BATCH; ++e) acc[0][0] += B.kv[e][0] + B.vv[e][0] + B.kv[e][L::EPL - 1] + B.vv[e][L::EPL - 1];
+                return;
+#endif
 #pragma unroll
-                for (int e = 0; e < BATCH; ++e) {
-                    if (B.mk[e] & bit) {
-                        const float pe = __builtin_amdgcn_exp2f(s[e] - mx);
-                        lrun[m] += pe;
+                for (int m = 0; m < R; ++m) {
+                    const int bit = 1 << m;
+                    if ((B.any & bit) == 0) continue;
+                    float s[BATCH], mx = mrun[m];
 #pragma unroll
-                        for (int i = 0; i < L::EPL; ++i) acc[m][i] = fmaf(pe, B.vv[e][i], acc[m][i]);
+                    for (int e = 0; e < BATCH; ++e) {
+                        s[e] = -INFINITY;
+                        if (B.mk[e] & bit) {
+                            s[e] = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], B.kv[e]));
+                            mx = fmaxf(mx, s[e]);
+                        }
                     }
+                    const float alpha = __builtin_amdgcn_exp2f(mrun[m] - mx);
+                    lrun[m] *= alpha;
+#pragma unroll
+                    for (int i = 0; i < L::EPL; ++i) acc[m][i] *= alpha;
+#pragma unroll
+                    for (int e = 0; e < BATCH; ++e) {
+                        if (B.mk[e] & bit) {
+                            const float pe = __builtin_amdgcn_exp2f(s[e] - mx);
+                            lrun[m] += pe;
+#pragma unroll
+                            for (int i = 0; i < L::EPL; ++i) acc[m][i] = fmaf(pe, B.vv[e][i], acc[m][i]);
+                        }
+                    }
+                    mrun[m] = mx;
                 }
-                mrun[m] = mx;
-            }
-        };
-        Batch A, B;
-        load_batch(A, 0);
-        for (int b = 0; b < cnt; b += 2 * BATCH) {
-            load_batch(B, b + BATCH);
-            issue_loads_first();
-            compute(A);
-            issue_loads_first();
-            load_batch(A, b + 2 * BATCH);
-            issue_loads_first();
-            compute(B);
-            issue_loads_first();
-        }
-    }
-#pragma unroll
-    for (int m = 0; m < R; ++m) {
-        if (gh.rows[m] < 0) continue;
-        if (gh.slots[m] < 0) {
-            const float inv = lrun[m] > 0.f ? 1.f / lrun[m] : 0.f;
-#pragma unroll
-            for (int i = 0; i < L::EPL; ++i) acc[m][i] *= inv;
-            store_row<T, H, D>(o + (size_t)gh.rows[m] * L::C, lane, acc[m]);
-            if (lane % L::LPH == 0) lse[(size_t)gh.rows[m] * H + head] = lrun[m] > 0.f ? mrun[m] + log2f(lrun[m]) : 0.f;
-        } else {
-            store_row_ws<T, H, D>(ws_acc + (size_t)gh.slots[m] * L::C, lane, acc[m]);
-            if (lane % L::LPH == 0) {
-                ws_ml[((size_t)gh.slots[m] * H + head) * 2] = mrun[m];
-                ws_ml[((size_t)gh.slots[m] * H + head) * 2 + 1] = lrun[m];
+            };
+            Batch A, B;
+            load_batch(A, 0);
+            for (int b = 0; b < cnt; b += 2 * BATCH) {
+                load_batch(B, b + BATCH);
+                issue_loads_first();
+                compute(A);
+                issue_loads_first();
+                load_batch(A, b + 2 * BATCH);
+                issue_loads_first();
+                compute(B);
+                issue_loads_first();
             }
         }
-    }
+#pragma unroll
+        for (int m = 0; m < R; ++m) {
+            if (gh.rows[m] < 0) continue;
+            if (gh.slots[m] < 0) {
+                const float inv = lrun[m] > 0.f ? 1.f / lrun[m] : 0.f;
+#pragma unroll
+                for (int i = 0; i < L::EPL; ++i) acc[m][i] *= inv;
+                store_row<T, H, D>(o + (size_t)gh.rows[m] * L::C, lane, acc[m]);
+                if (lane % L::LPH == 0) lse[(size_t)gh.rows[m] * H + head] = lrun[m] > 0.f ? mrun[m] + log2f(lrun[m]) : 0.f;
+            } else {
+                store_row_ws<T, H, D>(ws_acc + (size_t)gh.slots[m] * L::C, lane, acc[m]);
+                if (lane % L::LPH == 0) {
+                    ws_ml[((size_t)gh.slots[m] * H + head) * 2] = mrun[m];
+                    ws_ml[((size_t)gh.slots[m] * H + head) * 2 + 1] = lrun[m];
+                }
+            }
+        }
+    });
 }
 
 // Backward, destination side, row groups.  pds[(pair, head)] = (p, ds) in the pair order of the
 // source-side plan (P.grp_pairs maps this plan's pairs to it).
 template <typename T, int H, int D, int R, int BATCH, int WPE>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_dst_grp(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k,
-                                                           const T *__restrict__ v, const T *__restrict__ o, const T *__restrict__ d_o,
-                                                           const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
-                                                           float *__restrict__ ws_dq, float scale, float scale_log2e) {
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_dst_grp(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
+    const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
+    float *__restrict__ ws_dq, float scale, float scale_log2e) {
     using L = Lay<T, H, D>;
-    const int g = xcd_contiguous_block();
     const int lane = threadIdx.x, head = lane / L::LPH;
-    const GroupHead<R> gh = fetch_group<R>(P, g);
-    float qv[R][L::EPL], dov[R][L::EPL], dqa[R][L::EPL], delta[R], lse2[R];
-#pragma unroll
-    for (int m = 0; m < R; ++m) {
-        const size_t row = (size_t)max(gh.rows[m], 0);
-        float ov[L::EPL];
-        load_row<T, H, D>(o + row * L::C, lane, ov);
-        load_row<T, H, D>(d_o + row * L::C, lane, dov[m]);
-        load_row<T, H, D>(q + row * L::C, lane, qv[m]);
-        delta[m] = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], ov));
-        lse2[m] = lse[row * H + head];
-#pragma unroll
-        for (int i = 0; i < L::EPL; ++i) dqa[m][i] = 0.f;
-    }
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    const int last_pair = (int)P.n_edges - 1;
     struct Batch {
         float kv[BATCH][L::EPL], vv[BATCH][L::EPL];
         int mk[BATCH], xp[BATCH], any;
     };
-    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
-    const int last_pair = (int)P.n_edges - 1;
-    for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
-        const int cnt = min(WAVE, gh.end - p0);
-        const int4 ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
-        auto load_batch = [&](Batch &B, int b) {
-            B.any = 0;
+    walk_groups<R>(P, [&](const GroupHead<R> &gh, const int4 &ent0) {
+        float qv[R][L::EPL], dov[R][L::EPL], dqa[R][L::EPL], delta[R], lse2[R];
 #pragma unroll
-            for (int e = 0; e < BATCH; ++e) {
-                const bool ok = b + e < cnt;
-                const int j = ok ? b + e : 0;
-                const int src = __builtin_amdgcn_readlane(ent.x, j);
-                B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
-                B.any |= B.mk[e];
-                // lane r (< R) fetches the scratch position of this entry's r-th pair
-                B.xp[e] = P.grp_pairs[min(__builtin_amdgcn_readlane(ent.z, j) + (lane & (R - 1)), last_pair)];
-                load_row<T, H, D>(k + (size_t)src * L::C, lane, B.kv[e]);
-                load_row<T, H, D>(v + (size_t)src * L::C, lane, B.vv[e]);
-            }
-        };
-        auto compute = [&](const Batch &B) {
+        for (int m = 0; m < R; ++m) {
+            const size_t row = (size_t)max(gh.rows[m], 0);
+            float ov[L::EPL];
+            load_row<T, H, D>(o + row * L::C, lane, ov);
+            load_row<T, H, D>(d_o + row * L::C, lane, dov[m]);
+            load_row<T, H, D>(q + row * L::C, lane, qv[m]);
+            delta[m] = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], ov));
+            lse2[m] = lse[row * H + head];
 #pragma unroll
-            for (int m = 0; m < R; ++m) {
-                const int bit = 1 << m;
-                if ((B.any & bit) == 0) continue;
+            for (int i = 0; i < L::EPL; ++i) dqa[m][i] = 0.f;
+        }
+        for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
+            const int cnt = min(WAVE, gh.end - p0);
+            int4 ent = ent0;
+            if (p0 != gh.begin) ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
+            auto load_batch = [&](Batch &B, int b) {
+                B.any = 0;
 #pragma unroll
                 for (int e = 0; e < BATCH; ++e) {
-                    if (B.mk[e] & bit) {
-                        const int pos = __builtin_amdgcn_readlane(B.xp[e], __builtin_popcount(B.mk[e] & (bit - 1)));
-                        const float s = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], B.kv[e]));
-                        const float dp = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], B.vv[e]));
-                        const float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
-                        const float ds = pe * (dp - delta[m]) * scale;
+                    const bool ok = b + e < cnt;
+                    const int j = ok ? b + e : 0;
+                    const int src = __builtin_amdgcn_readlane(ent.x, j);
+                    B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
+                    B.any |= B.mk[e];
+                    // lane r (< R) fetches the scratch position of this entry's r-th pair
+                    B.xp[e] = P.grp_pairs[min(__builtin_amdgcn_readlane(ent.z, j) + (lane & (R - 1)), last_pair)];
+                    load_row<T, H, D>(k + (size_t)src * L::C, lane, B.kv[e]);
+                    load_row<T, H, D>(v + (size_t)src * L::C, lane, B.vv[e]);
+                }
+            };
+            auto compute = [&](const Batch &B) {
 #pragma unroll
-                        for (int i = 0; i < L::EPL; ++i) dqa[m][i] = fmaf(ds, B.kv[e][i], dqa[m][i]);
-                        if (lane % L::LPH == 0) pds[(size_t)pos * H + head] = make_float2(pe, ds);
+                for (int m = 0; m < R; ++m) {
+                    const int bit = 1 << m;
+                    if ((B.any & bit) == 0) continue;
+#pragma unroll
+                    for (int e = 0; e < BATCH; ++e) {
+                        if (B.mk[e] & bit) {
+                            const int pos = __builtin_amdgcn_readlane(B.xp[e], __builtin_popcount(B.mk[e] & (bit - 1)));
+                            const float s = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], B.kv[e]));
+                            const float dp = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], B.vv[e]));
+                            const float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
+                            const float ds = pe * (dp - delta[m]) * scale;
+#pragma unroll
+                            for (int i = 0; i < L::EPL; ++i) dqa[m][i] = fmaf(ds, B.kv[e][i], dqa[m][i]);
+                            if (lane % L::LPH == 0) pds[(size_t)pos * H + head] = make_float2(pe, ds);
+                        }
                     }
                 }
+            };
+            Batch A, B;
+            load_batch(A, 0);
+            for (int b = 0; b < cnt; b += 2 * BATCH) {
+                load_batch(B, b + BATCH);
+                issue_loads_first();
+                compute(A);
+                issue_loads_first();
+                load_batch(A, b + 2 * BATCH);
+                issue_loads_first();
+                compute(B);
+                issue_loads_first();
             }
-        };
-        Batch A, B;
-        load_batch(A, 0);
-        for (int b = 0; b < cnt; b += 2 * BATCH) {
-            load_batch(B, b + BATCH);
-            issue_loads_first();
-            compute(A);
-            issue_loads_first();
-            load_batch(A, b + 2 * BATCH);
-            issue_loads_first();
-            compute(B);
-            issue_loads_first();
         }
-    }
 #pragma unroll
-    for (int m = 0; m < R; ++m) {
-        if (gh.rows[m] < 0) continue;
-        if (gh.slots[m] < 0) store_row<T, H, D>(dq + (size_t)gh.rows[m] * L::C, lane, dqa[m]);
-        else store_row_ws<T, H, D>(ws_dq + (size_t)gh.slots[m] * L::C, lane, dqa[m]);
-    }
+        for (int m = 0; m < R; ++m) {
+            if (gh.rows[m] < 0) continue;
+            if (gh.slots[m] < 0) store_row<T, H, D>(dq + (size_t)gh.rows[m] * L::C, lane, dqa[m]);
+            else store_row_ws<T, H, D>(ws_dq + (size_t)gh.slots[m] * L::C, lane, dqa[m]);
+        }
+    });
 }
 
 // Backward, source side, row groups: dK[src] = sum ds * q[dst], dV[src] = sum p * dO[dst]; the (p, ds)
 // of this plan's pair number n sits at pds[n].
 template <typename T, int H, int D, int R, int BATCH, int WPE>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_src_grp(bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o,
-                                                           const float2 *__restrict__ pds, T *__restrict__ dk, T *__restrict__ dv,
-                                                           float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_src_grp(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o, const float2 *__restrict__ pds, T *__restrict__ dk,
+    T *__restrict__ dv, float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
     using L = Lay<T, H, D>;
-    const int g = xcd_contiguous_block();
     const int lane = threadIdx.x, head = lane / L::LPH;
-    const GroupHead<R> gh = fetch_group<R>(P, g);
-    float ak[R][L::EPL], av[R][L::EPL];
-#pragma unroll
-    for (int m = 0; m < R; ++m)
-#pragma unroll
-        for (int i = 0; i < L::EPL; ++i) { ak[m][i] = 0.f; av[m][i] = 0.f; }
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     struct Batch {
         float qr[BATCH][L::EPL], dr[BATCH][L::EPL];
         float2 w[BATCH][R];
         int mk[BATCH];
     };
-    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
-    for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
-        const int cnt = min(WAVE, gh.end - p0);
-        const int4 ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
-        auto load_batch = [&](Batch &B, int b) {
+    walk_groups<R>(P, [&](const GroupHead<R> &gh, const int4 &ent0) {
+        float ak[R][L::EPL], av[R][L::EPL];
 #pragma unroll
-            for (int e = 0; e < BATCH; ++e) {
-                const bool ok = b + e < cnt;
-                const int j = ok ? b + e : 0;
-                const int dst = __builtin_amdgcn_readlane(ent.x, j);
-                B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
-                const int pb = __builtin_amdgcn_readlane(ent.z, j);
-                load_row<T, H, D>(q + (size_t)dst * L::C, lane, B.qr[e]);
-                load_row<T, H, D>(d_o + (size_t)dst * L::C, lane, B.dr[e]);
+        for (int m = 0; m < R; ++m)
 #pragma unroll
-                for (int m = 0; m < R; ++m) {
-                    B.w[e][m] = make_float2(0.f, 0.f);
-                    if (B.mk[e] & (1 << m)) B.w[e][m] = pds[(size_t)(pb + __builtin_popcount(B.mk[e] & ((1 << m) - 1))) * H + head];
+            for (int i = 0; i < L::EPL; ++i) { ak[m][i] = 0.f; av[m][i] = 0.f; }
+        for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
+            const int cnt = min(WAVE, gh.end - p0);
+            int4 ent = ent0;
+            if (p0 != gh.begin) ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
+            auto load_batch = [&](Batch &B, int b) {
+#pragma unroll
+                for (int e = 0; e < BATCH; ++e) {
+                    const bool ok = b + e < cnt;
+                    const int j = ok ? b + e : 0;
+                    const int dst = __builtin_amdgcn_readlane(ent.x, j);
+                    B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
+                    const int pb = __builtin_amdgcn_readlane(ent.z, j);
+                    load_row<T, H, D>(q + (size_t)dst * L::C, lane, B.qr[e]);
+                    load_row<T, H, D>(d_o + (size_t)dst * L::C, lane, B.dr[e]);
+#pragma unroll
+                    for (int m = 0; m < R; ++m) {
+                        B.w[e][m] = make_float2(0.f, 0.f);
+                        if (B.mk[e] & (1 << m))
+                            B.w[e][m] = pds[(size_t)(pb + __builtin_popcount(B.mk[e] & ((1 << m) - 1))) * H + head];
+                    }
                 }
-            }
-        };
-        auto compute = [&](const Batch &B) {
+            };
+            auto compute = [&](const Batch &B) {
 #pragma unroll
-            for (int e = 0; e < BATCH; ++e) {
+                for (int e = 0; e < BATCH; ++e) {
 #pragma unroll
-                for (int m = 0; m < R; ++m) {
-                    if (B.mk[e] & (1 << m)) {
+                    for (int m = 0; m < R; ++m) {
+                        if (B.mk[e] & (1 << m)) {
 #pragma unroll
-                        for (int i = 0; i < L::EPL; ++i) {
-                            ak[m][i] = fmaf(B.w[e][m].y, B.qr[e][i], ak[m][i]);
-                            av[m][i] = fmaf(B.w[e][m].x, B.dr[e][i], av[m][i]);
+                            for (int i = 0; i < L::EPL; ++i) {
+                                ak[m][i] = fmaf(B.w[e][m].y, B.qr[e][i], ak[m][i]);
+                                av[m][i] = fmaf(B.w[e][m].x, B.dr[e][i], av[m][i]);
+                            }
                         }
                     }
                 }
+            };
+            Batch A, B;
+            load_batch(A, 0);
+            for (int b = 0; b < cnt; b += 2 * BATCH) {
+                load_batch(B, b + BATCH);
+                issue_loads_first();
+                compute(A);
+                issue_loads_first();
+                load_batch(A, b + 2 * BATCH);
+                issue_loads_first();
+                compute(B);
+                issue_loads_first();
             }
-        };
-        Batch A, B;
-        load_batch(A, 0);
-        for (int b = 0; b < cnt; b += 2 * BATCH) {
-            load_batch(B, b + BATCH);
-            issue_loads_first();
-            compute(A);
-            issue_loads_first();
-            load_batch(A, b + 2 * BATCH);
-            issue_loads_first();
-            compute(B);
-            issue_loads_first();
         }
-    }
 #pragma unroll
-    for (int m = 0; m < R; ++m) {
-        if (gh.rows[m] < 0) continue;
-        if (gh.slots[m] < 0) {
-            store_row<T, H, D>(dk + (size_t)gh.rows[m] * L::C, lane, ak[m]);
-            store_row<T, H, D>(dv + (size_t)gh.rows[m] * L::C, lane, av[m]);
-        } else {
-            store_row_ws<T, H, D>(ws_dk + (size_t)gh.slots[m] * L::C, lane, ak[m]);
-            store_row_ws<T, H, D>(ws_dv + (size_t)gh.slots[m] * L::C, lane, av[m]);
+        for (int m = 0; m < R; ++m) {
+            if (gh.rows[m] < 0) continue;
+            if (gh.slots[m] < 0) {
+                store_row<T, H, D>(dk + (size_t)gh.rows[m] * L::C, lane, ak[m]);
+                store_row<T, H, D>(dv + (size_t)gh.rows[m] * L::C, lane, av[m]);
+            } else {
+                store_row_ws<T, H, D>(ws_dk + (size_t)gh.slots[m] * L::C, lane, ak[m]);
+                store_row_ws<T, H, D>(ws_dv + (size_t)gh.slots[m] * L::C, lane, av[m]);
+            }
         }
-    }
+    });
 }
 
 // ------------------------------------------------------------------------------------------
@@ -980,7 +1023,8 @@ inline int check_plan(const bpt_plan *p, bool need_idx) {
     if (p->n_heavy > 0 && !p->heavy) return BPT_ERR_NULL;
     if (p->n_items < p->n_rows) return BPT_ERR_SIZE;     // every row owns at least one item
     if (p->n_groups < 0 || p->grp_R < 0 || p->grp_R > 8) return BPT_ERR_SIZE;
-    if (p->n_groups > 0 && (!p->grp_members || !p->grp_ptr || (p->n_edges > 0 && !p->grp_entries))) return BPT_ERR_NULL;
+    if (p->n_groups > 0 && (!p->grp_members || !p->grp_ptr || !p->grp_chunks || (p->n_edges > 0 && !p->grp_entries))) return BPT_ERR_NULL;
+    if (p->n_groups > 0 && (p->grp_max_chunk < 1 || p->grp_max_chunk > p->n_groups)) return BPT_ERR_SIZE;
     return BPT_OK;
 }
 
@@ -1136,8 +1180,15 @@ inline int64_t round16(int64_t b) { return (b + 15) & ~(int64_t)15; }
 
 constexpr int GROUP_R = 4;
 
+inline int group_grid(const bpt_plan *P, int kernel) {
+    const int64_t per_xcd = g_group_waves[kernel].load(std::memory_order_relaxed);
+    const int64_t n = (per_xcd > 0 && per_xcd < P->grp_max_chunk) ? per_xcd : P->grp_max_chunk;
+    return (int)(8 * n);
+}
+
 inline bool has_groups(const bpt_plan *P) {
-    return P->n_groups > 0 && P->grp_R == GROUP_R && P->grp_members && P->grp_ptr && P->grp_entries;
+    return P->n_groups > 0 && P->grp_R == GROUP_R && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
+           P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups;
 }
 
 template <typename T, int H, int D>
@@ -1149,7 +1200,7 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
         if (has_groups(P)) {
 #define LAUNCH_FWD_GRP(B, W)                                                                                                   \
-    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, GROUP_R, B, W>), dim3((int)P->n_groups), dim3(WAVE), 0, s, *P, (const T *)q,   \
+    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, GROUP_R, B, W>), dim3(group_grid(P, 0)), dim3(WAVE), 0, s, *P, (const T *)q,   \
                        (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E)
             const int var = g_group_variant[0].load(std::memory_order_relaxed);
             if (var == 4) LAUNCH_FWD_GRP(4, 1);
@@ -1177,7 +1228,7 @@ int run_attn_bwd_grouped(const bpt_plan *Pin, const bpt_plan *Pout, const void *
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
 #define LAUNCH_DST_GRP(B, W)                                                                                                       \
-    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, GROUP_R, B, W>), dim3((int)Pin->n_groups), dim3(WAVE), 0, s, *Pin, (const T *)q, \
+    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, GROUP_R, B, W>), dim3(group_grid(Pin, 1)), dim3(WAVE), 0, s, *Pin, (const T *)q, \
                        (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E)
         const int var = g_group_variant[1].load(std::memory_order_relaxed);
         if (var == 4) LAUNCH_DST_GRP(4, 1);
@@ -1197,7 +1248,7 @@ int run_attn_bwd_grouped(const bpt_plan *Pin, const bpt_plan *Pout, const void *
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
 #define LAUNCH_SRC_GRP(B, W)                                                                                                          \
-    hipLaunchKernelGGL((k_attn_bwd_src_grp<T, H, D, GROUP_R, B, W>), dim3((int)Pout->n_groups), dim3(WAVE), 0, s, *Pout, (const T *)q, \
+    hipLaunchKernelGGL((k_attn_bwd_src_grp<T, H, D, GROUP_R, B, W>), dim3(group_grid(Pout, 2)), dim3(WAVE), 0, s, *Pout, (const T *)q, \
                        (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv)
         const int var = g_group_variant[2].load(std::memory_order_relaxed);
         if (var == 4) LAUNCH_SRC_GRP(4, 1);
@@ -1267,6 +1318,12 @@ int bpt_set_force_generic(int on) { return g_force_generic.exchange(on ? 1 : 0);
 int bpt_set_group_variant(int kernel, int variant) {
     if (kernel < 0 || kernel > 2 || (variant != 2 && variant != 3 && variant != 4)) return BPT_ERR_SIZE;
     g_group_variant[kernel].store(variant);
+    return BPT_OK;
+}
+
+int bpt_set_group_waves(int kernel, int waves_per_xcd) {
+    if (kernel < 0 || kernel > 2 || waves_per_xcd < 0) return BPT_ERR_SIZE;
+    g_group_waves[kernel].store(waves_per_xcd);
     return BPT_OK;
 }
 

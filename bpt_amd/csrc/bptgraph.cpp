@@ -367,17 +367,20 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
 // Greedy clustering of work items (rows / row segments) that read mostly the same neighbour rows.
 // Items are visited in locality order; an item opens a group and the next `window` unused items
 // join it while at least half of their neighbours are already in the group's union (at most R
-// members).  For every group the union of neighbour ids becomes a list of entries
-// (idx, member mask, first pair); a pair = one original edge = (entry, member).  Pairs are numbered
-// entry by entry, members ascending — the order in which the kernels visit them.
+// members).  The groups are then cut into 8 contiguous chunks of about equal work (one per XCD) and
+// ordered inside each chunk (order_mode 0: locality order; 1: groups with at least average work first,
+// the small ones last, each part in locality order; 2: by decreasing work).  For every group the union
+// of neighbour ids becomes a list of entries (idx, member mask, first pair); a pair = one original
+// edge = (entry, member).  Pairs are numbered entry by entry, members ascending — the order in which
+// the kernels visit them.
 int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32, const int32_t *eid32,
-                    int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window,
-                    int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid,
+                    int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window, int32_t order_mode,
+                    int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *chunks,
                     int64_t *n_groups_out, int64_t *n_entries_out) {
-    if (!items || !members || !grp_ptr || !n_groups_out || !n_entries_out) return BPTG_ERR_NULL;
+    if (!items || !members || !grp_ptr || !chunks || !n_groups_out || !n_entries_out) return BPTG_ERR_NULL;
     if (n_edges > 0 && (!idx32 || !eid32 || !entries || !pair_eid)) return BPTG_ERR_NULL;
     if (n_items < 0 || n_edges < 0 || n_index_nodes < 0) return BPTG_ERR_SIZE;
-    if (R < 1 || R > 8 || window < 0) return BPTG_ERR_ARG;
+    if (R < 1 || R > 8 || window < 0 || order_mode < 0 || order_mode > 2) return BPTG_ERR_ARG;
     for (int64_t i = 0; i < n_items; ++i) {
         const int32_t *it = items + 4 * i;
         if (it[1] < 0 || it[2] < it[1] || it[2] > n_edges) return BPTG_ERR_RANGE;
@@ -385,8 +388,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
     for (int64_t p = 0; p < n_edges; ++p)
         if (idx32[p] < 0 || idx32[p] >= n_index_nodes) return BPTG_ERR_RANGE;
 
-    // locality order of the items (they may already be sorted; sorting again is cheap and makes the
-    // function independent of the caller's order)
+    // locality order of the items
     std::vector<int32_t> key((size_t)n_items), order((size_t)n_items);
     for (int64_t i = 0; i < n_items; ++i) {
         const int32_t *it = items + 4 * i;
@@ -397,25 +399,27 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
     }
     std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return key[(size_t)a] < key[(size_t)b]; });
 
+    // ---- phase 1: form the groups (member item lists) in locality order
     std::vector<uint8_t> used((size_t)n_items, 0);
     std::vector<int64_t> stamp((size_t)n_index_nodes, -1);     // stamp[node] == group id  <=>  node in the union
-    struct Triple { int32_t idx, member, eid; };
-    std::vector<Triple> tri;
-    std::vector<int32_t> grp_items;
-    int64_t n_groups = 0, n_entries = 0, n_pairs = 0;
-    grp_ptr[0] = 0;
+    std::vector<int32_t> grp_items;                            // R slots per group, -1 = unused
+    std::vector<int64_t> work;                                 // pairs + fixed cost per group
+    int64_t n_groups = 0;
     for (int64_t oi = 0; oi < n_items; ++oi) {
         const int32_t first = order[(size_t)oi];
         if (used[(size_t)first]) continue;
         used[(size_t)first] = 1;
-        grp_items.clear();
-        grp_items.push_back(first);
+        int32_t mem[8] = {-1, -1, -1, -1, -1, -1, -1, -1};
+        int32_t n_mem = 1;
+        mem[0] = first;
+        int64_t w = 0;
         {
             const int32_t *it = items + 4 * (int64_t)first;
+            w += it[2] - it[1];
             for (int32_t p = it[1]; p < it[2]; ++p) stamp[(size_t)idx32[p]] = n_groups;
         }
         int32_t seen = 0;
-        for (int64_t oj = oi + 1; oj < n_items && (int32_t)grp_items.size() < R && seen < window; ++oj) {
+        for (int64_t oj = oi + 1; oj < n_items && n_mem < R && seen < window; ++oj) {
             const int32_t cand = order[(size_t)oj];
             if (used[(size_t)cand]) continue;
             ++seen;
@@ -426,17 +430,57 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
             for (int32_t p = it[1]; p < it[2]; ++p) hit += (stamp[(size_t)idx32[p]] == n_groups);
             if (2 * hit >= len) {
                 used[(size_t)cand] = 1;
-                grp_items.push_back(cand);
+                mem[n_mem++] = cand;
+                w += len;
                 for (int32_t p = it[1]; p < it[2]; ++p) stamp[(size_t)idx32[p]] = n_groups;
             }
         }
-        // members in ascending item order (deterministic, independent of the join order)
-        std::sort(grp_items.begin(), grp_items.end());
+        std::sort(mem, mem + n_mem);          // members in ascending item order (independent of the join order)
+        for (int32_t m = 0; m < R; ++m) grp_items.push_back(mem[m]);
+        work.push_back(w + 24);               // fixed cost of a wavefront, in pair equivalents
+        ++n_groups;
+    }
+
+    // ---- phase 2: 8 contiguous chunks of about equal work, then the order inside each chunk
+    std::vector<int32_t> gorder((size_t)n_groups);
+    for (int64_t g = 0; g < n_groups; ++g) gorder[(size_t)g] = (int32_t)g;
+    int64_t total = 0;
+    for (int64_t g = 0; g < n_groups; ++g) total += work[(size_t)g];
+    {
+        int64_t acc = 0, g = 0;
+        chunks[0] = 0;
+        for (int x = 1; x <= 8; ++x) {
+            const int64_t target = total * x / 8;
+            while (g < n_groups && (acc + work[(size_t)g] / 2 < target || x == 8)) acc += work[(size_t)g++];
+            chunks[x] = (int32_t)g;
+        }
+    }
+    if (order_mode != 0) {
+        for (int x = 0; x < 8; ++x) {
+            auto b = gorder.begin() + chunks[x], e = gorder.begin() + chunks[x + 1];
+            if (order_mode == 2) {
+                std::stable_sort(b, e, [&](int32_t a, int32_t c) { return work[(size_t)a] > work[(size_t)c]; });
+            } else {
+                int64_t sum = 0;
+                for (auto it = b; it != e; ++it) sum += work[(size_t)*it];
+                const int64_t avg = (e > b) ? sum / (e - b) : 0;
+                std::stable_partition(b, e, [&](int32_t a) { return work[(size_t)a] >= avg; });
+            }
+        }
+    }
+
+    // ---- phase 3: emit members, entries and pairs in the final group order
+    struct Triple { int32_t idx, member, eid; };
+    std::vector<Triple> tri;
+    int64_t n_entries = 0, n_pairs = 0;
+    grp_ptr[0] = 0;
+    for (int64_t gi = 0; gi < n_groups; ++gi) {
+        const int32_t *gmem = &grp_items[(size_t)gorder[(size_t)gi] * R];
         tri.clear();
         for (int32_t m = 0; m < R; ++m) {
-            int32_t *mem = members + ((int64_t)n_groups * R + m) * 2;
-            if (m < (int32_t)grp_items.size()) {
-                const int32_t *it = items + 4 * (int64_t)grp_items[(size_t)m];
+            int32_t *mem = members + ((int64_t)gi * R + m) * 2;
+            if (gmem[m] >= 0) {
+                const int32_t *it = items + 4 * (int64_t)gmem[m];
                 mem[0] = it[0];
                 mem[1] = it[3];
                 for (int32_t p = it[1]; p < it[2]; ++p) tri.push_back({idx32[p], m, eid32[p]});
@@ -477,8 +521,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
             }
             a = b;
         }
-        ++n_groups;
-        grp_ptr[n_groups] = (int32_t)n_entries;
+        grp_ptr[gi + 1] = (int32_t)n_entries;
     }
     *n_groups_out = n_groups;
     *n_entries_out = n_entries;

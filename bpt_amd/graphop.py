@@ -278,6 +278,13 @@ def set_group_variant(fwd=None, bwd_dst=None, bwd_src=None):
             check_attn(_LIB.bpt_set_group_variant(kernel, int(var)), "set_group_variant")
 
 
+def set_group_waves(fwd=None, bwd_dst=None, bwd_src=None):
+    """Persistent wavefronts per XCD for each row-group kernel (0: one wavefront per group); None keeps the value."""
+    for kernel, n in enumerate((fwd, bwd_dst, bwd_src)):
+        if n is not None:
+            check_attn(_LIB.bpt_set_group_waves(kernel, int(n)), "set_group_waves")
+
+
 def set_force_generic(on):
     """Testing hook: route every op through the shape-generic kernels."""
     return bool(_LIB.bpt_set_force_generic(1 if on else 0))

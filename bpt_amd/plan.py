@@ -19,6 +19,7 @@ from ._lib import PlanInfo, PlanStruct, check_graph, graph_lib
 DEFAULT_SEG_LEN = 64
 GROUP_R = 4            # rows per wavefront in the fused row-group kernels (matches the HIP library)
 GROUP_WINDOW = 32      # how many following items the greedy grouping examines per group
+GROUP_ORDER = 2        # order of the groups inside an XCD chunk: 0 locality, 1 big first / small last, 2 decreasing work
 _CACHE_SIZE = 64
 
 
@@ -60,9 +61,11 @@ def build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len=DE
     return arrays, info
 
 
-def build_groups_host(arrays, n_index_nodes, R=GROUP_R, window=GROUP_WINDOW):
+def build_groups_host(arrays, n_index_nodes, R=GROUP_R, window=GROUP_WINDOW, order_mode=None):
     """Pure host step: clusters the plan's items into row groups (bptg_group_plan).  Returns a dict
-    with members (n_groups, R, 2), grp_ptr (n_groups + 1), entries (n_entries, 4), pair_eid (n_edges)."""
+    with members (n_groups, R, 2), grp_ptr (n_groups + 1), entries (n_entries, 4), pair_eid (n_edges),
+    chunks (9,)."""
+    order_mode = GROUP_ORDER if order_mode is None else order_mode
     items = np.ascontiguousarray(arrays["items"], dtype=np.int32)
     idx = np.ascontiguousarray(arrays["idx"], dtype=np.int32)
     eid = np.ascontiguousarray(arrays["eid"], dtype=np.int32)
@@ -71,12 +74,13 @@ def build_groups_host(arrays, n_index_nodes, R=GROUP_R, window=GROUP_WINDOW):
     grp_ptr = np.empty(n_items + 1, dtype=np.int32)
     entries = np.empty((max(E, 1), 4), dtype=np.int32)
     pair_eid = np.empty(max(E, 1), dtype=np.int32)
+    chunks = np.zeros(9, dtype=np.int32)
     ng, ne = ctypes.c_int64(), ctypes.c_int64()
     check_graph(graph_lib().bptg_group_plan(_ptr(items), n_items, _ptr(idx), _ptr(eid), E, int(n_index_nodes), R, window,
-                                            _ptr(members), _ptr(grp_ptr), _ptr(entries), _ptr(pair_eid),
-                                            ctypes.byref(ng), ctypes.byref(ne)))
+                                            int(order_mode), _ptr(members), _ptr(grp_ptr), _ptr(entries), _ptr(pair_eid),
+                                            _ptr(chunks), ctypes.byref(ng), ctypes.byref(ne)))
     return {"members": members[:ng.value].copy(), "grp_ptr": grp_ptr[:ng.value + 1].copy(),
-            "entries": entries[:ne.value].copy(), "pair_eid": pair_eid[:E].copy()}
+            "entries": entries[:ne.value].copy(), "pair_eid": pair_eid[:E].copy(), "chunks": chunks}
 
 
 class Plan:
@@ -121,6 +125,8 @@ class Plan:
                 self.struct.grp_ptr = d["grp_ptr"].data_ptr()
                 self.struct.grp_entries = d["entries"].data_ptr() if len(grp["entries"]) else None
                 self.struct.grp_pairs = None
+                self.struct.grp_chunks = d["chunks"].data_ptr()
+                self.struct.grp_max_chunk = int(np.diff(grp["chunks"]).max()) if self.n_groups else 0
                 self.struct.n_groups = self.n_groups
                 self.struct.grp_R = GROUP_R
                 self._groups = grp

@@ -58,7 +58,9 @@ typedef struct {
     const int32_t *grp_pairs;    /* n_edges or NULL.  On the destination-side plan of the fused backward:
                                     for every pair of this plan, the number of the same edge's pair in the
                                     source-side plan (the per-edge scratch is laid out in that order) */
+    const int32_t *grp_chunks;   /* 9 : groups grp_chunks[x] .. grp_chunks[x+1]-1 are walked by XCD x */
     int64_t n_groups, grp_R;
+    int64_t grp_max_chunk;       /* largest chunk length; the row-group kernels launch 8 * grp_max_chunk workgroups */
 } bpt_plan;
 
 const char *bpt_strerror(int status);
@@ -70,6 +72,10 @@ int bpt_set_force_generic(int on);
  * side.  variant: 4 = load batches of four neighbour rows, 2 = batches of two, 3 = batches of two compiled
  * for three resident wavefronts per SIMD. */
 int bpt_set_group_variant(int kernel, int variant);
+
+/* How many wavefronts per XCD walk that XCD's share of the row groups (persistent wavefronts, each
+ * prefetching the next group's header and entries); 0 = one wavefront per group.  kernel as above. */
+int bpt_set_group_waves(int kernel, int waves_per_xcd);
 
 /* Measurement aid (no counterpart in the reference): while `which` is one of BPT_KERNEL_*, every launch
  * of that main kernel of the fused path is bracketed by hipEventRecord(start_event) / (stop_event) on

@@ -36,14 +36,17 @@ def plans(name, seg=64):
     return src, dst, n, csr, pin, pout
 
 
+@pytest.mark.parametrize("order_mode", [0, 1, 2])
 @pytest.mark.parametrize("seg", [8, 64])
 @pytest.mark.parametrize("name", sorted(GRAPHS))
-def test_group_plan_invariants(name, seg):
+def test_group_plan_invariants(name, seg, order_mode):
     src, dst, n, csr, pin, pout = plans(name, seg)
     E = len(src)
     for arrays, rows_of, cols_of in ((pin, dst, src), (pout, src, dst)):
-        grp = build_groups_host(arrays, n)
+        grp = build_groups_host(arrays, n, order_mode=order_mode)
         members, gptr, entries, pair_eid = grp["members"], grp["grp_ptr"], grp["entries"], grp["pair_eid"]
+        ch = grp["chunks"]
+        assert ch[0] == 0 and ch[8] == len(members) and np.all(np.diff(ch) >= 0)
         items = arrays["items"]
         ng = len(members)
         assert members.shape == (ng, GROUP_R, 2) and len(gptr) == ng + 1
@@ -170,3 +173,9 @@ def test_grouping_reduces_row_loads_on_the_headline_graph():
         grp = build_groups_host(arrays, n)
         assert len(grp["entries"]) < 0.42 * len(src)        # neighbour-row loads per kernel vs one per edge
         assert len(grp["members"]) < 0.3 * len(arrays["items"])
+        # XCD chunks carry about equal work (pairs)
+        pc = np.array([bin(m).count("1") for m in grp["entries"][:, 1]])
+        cum = np.concatenate([[0], np.cumsum(pc)])
+        ch = grp["chunks"]
+        per = [cum[grp["grp_ptr"][ch[x + 1]]] - cum[grp["grp_ptr"][ch[x]]] for x in range(8)]
+        assert max(per) < 1.10 * min(per)      # balanced on pairs + a fixed cost per group
