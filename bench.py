@@ -102,6 +102,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies (known HBM bytes) so counter runs can be scaled")
     ap.add_argument("--rows", action="store_true", help="fused kernels with one wavefront per row (no row groups)")
+    ap.add_argument("--group-rows", type=int, default=4, choices=[4, 16], help="4: one wavefront per row group (default); 16: teams of 4 wavefronts sharing rows through LDS")
     ap.add_argument("--waves", default=None, help="persistent wavefronts per XCD fwd,bwd_dst,bwd_src (0 = one per group)")
     ap.add_argument("--variants", default=None, help="row-group kernel variants fwd,bwd_dst,bwd_src (each 2, 3 or 4)")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
@@ -118,6 +119,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
     graphop.set_row_groups(not args.rows)
+    graphop.set_group_rows(args.group_rows)
     if args.waves:
         graphop.set_group_waves(*[int(x) for x in args.waves.split(",")])
     if args.variants:
@@ -238,7 +240,7 @@ def main():
         "dtype": dtype_name, "data": "synthetic",
         "config": {"workload": desc + (" (unfused op chain)" if args.unfused else " (fused fwd+bwd)"), "n_nodes": N,
                    "n_edges": E, "heads": H, "d_head": D, "launch": mode,
-                   "kernels": "per-row" if args.rows else "row-groups" + (f"({args.variants})" if args.variants else "")},
+                   "kernels": "per-row" if args.rows else ("teams(4 wavefronts x 4 rows, LDS-shared)" if args.group_rows == 16 else "row-groups(4 rows per wavefront)")},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "step_roofline": {"algorithmic_bytes": alg["total"], "achieved_GBps": round(step_gbs, 1),

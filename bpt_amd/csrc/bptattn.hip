@@ -1011,6 +1011,415 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) voi
 }
 
 // ------------------------------------------------------------------------------------------
+// team kernels of the fused path.  A team = one group of up to 16 rows (grp_R == 16) handled by a
+// workgroup of 4 wavefronts; wavefront w keeps the state of members 4w .. 4w+3 in registers.  The
+// team's neighbour rows are fetched from global memory ONCE per team: at every stage of TEAM_S = 4
+// entries wavefront w loads the two rows of entry 4*stage + w into registers (one stage ahead),
+// writes them to LDS in lane-major order (float4 slot c*64 + lane, conflict free), and after one
+// barrier every wavefront reads the rows its own members need (nibble w of the entry's 16-bit
+// mask).  LDS is double buffered, so there is one barrier per stage.  This turns the L2->L1
+// traffic of the single-wavefront row groups (each wavefront fetching its own union) into LDS reads.
+// ------------------------------------------------------------------------------------------
+constexpr int TEAM_WAVES = 4, TEAM_RW = 4, TEAM_R = TEAM_WAVES * TEAM_RW, TEAM_S = 4;
+
+// Workgroup b runs on XCD b % 8 and takes the (b / 8)-th team of that XCD's chunk (-1: none).
+__device__ __forceinline__ int team_index(const bpt_plan &P) {
+    const int x = blockIdx.x & 7, kk = blockIdx.x >> 3;
+    const int first = P.grp_chunks[x], last = P.grp_chunks[x + 1];
+    return first + kk < last ? first + kk : -1;
+}
+
+template <int EPL> __device__ __forceinline__ void lds_put_row(float4 *slot, int lane, const float (&r)[EPL]) {
+#pragma unroll
+    for (int c = 0; c < EPL / 4; ++c) slot[c * WAVE + lane] = make_float4(r[4 * c], r[4 * c + 1], r[4 * c + 2], r[4 * c + 3]);
+}
+template <int EPL> __device__ __forceinline__ void lds_get_row(const float4 *slot, int lane, float (&r)[EPL]) {
+#pragma unroll
+    for (int c = 0; c < EPL / 4; ++c) {
+        const float4 v = slot[c * WAVE + lane];
+        r[4 * c] = v.x; r[4 * c + 1] = v.y; r[4 * c + 2] = v.z; r[4 * c + 3] = v.w;
+    }
+}
+
+// Entry descriptors of up to 128 consecutive entries, two per lane (fetched with two vector loads per
+// wavefront); field f of entry j is read with v_readlane, so no memory access sits between stages.
+struct TeamDesc {
+    int4 lo, hi;
+    __device__ __forceinline__ void fetch(const int4 *ent, int count, int lane) {
+        lo = lane < count ? ent[lane] : make_int4(0, 0, 0, 0);
+        hi = lane + WAVE < count ? ent[lane + WAVE] : make_int4(0, 0, 0, 0);
+    }
+    __device__ __forceinline__ int idx(int j) const { return j < WAVE ? __builtin_amdgcn_readlane(lo.x, j) : __builtin_amdgcn_readlane(hi.x, j - WAVE); }
+    __device__ __forceinline__ int mask(int j) const { return j < WAVE ? __builtin_amdgcn_readlane(lo.y, j) : __builtin_amdgcn_readlane(hi.y, j - WAVE); }
+    __device__ __forceinline__ int pair0(int j) const { return j < WAVE ? __builtin_amdgcn_readlane(lo.z, j) : __builtin_amdgcn_readlane(hi.z, j - WAVE); }
+};
+constexpr int TEAM_SPAN = 2 * WAVE;      // entries per descriptor fetch
+
+template <typename T, int H, int D>
+__global__ __launch_bounds__(BLOCK) void k_attn_fwd_team(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k,
+                                                         const T *__restrict__ v, T *__restrict__ o, float *__restrict__ lse,
+                                                         float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+    using L = Lay<T, H, D>;
+    constexpr int S = TEAM_S, RW = TEAM_RW, F4 = L::EPL / 4;
+    __shared__ float4 lds[2][S][2][F4 * WAVE];
+    const int t = team_index(P);
+    if (t < 0) return;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), head = lane / L::LPH;
+    int rows[RW], slots[RW];
+#pragma unroll
+    for (int m = 0; m < RW; ++m) {
+        rows[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2]);
+        slots[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2 + 1]);
+    }
+    const int begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[t]);
+    const int n = __builtin_amdgcn_readfirstlane(P.grp_ptr[t + 1]) - begin;
+    const int4 *ent = reinterpret_cast<const int4 *>(P.grp_entries) + begin;
+
+    float qv[RW][L::EPL], acc[RW][L::EPL], mrun[RW], lrun[RW];
+#pragma unroll
+    for (int m = 0; m < RW; ++m) {
+        load_row<T, H, D>(q + (size_t)max(rows[m], 0) * L::C, lane, qv[m]);
+        mrun[m] = M_INIT_LOG2;
+        lrun[m] = 0.f;
+#pragma unroll
+        for (int i = 0; i < L::EPL; ++i) { qv[m][i] *= scale_log2e; acc[m][i] = 0.f; }
+    }
+    // two stages of row loads are in flight per wavefront: register set A holds even stages, B odd ones
+    struct StageRegs { float ra[L::EPL], rb[L::EPL]; };
+    for (int c0 = 0; c0 < n; c0 += TEAM_SPAN) {
+        const int cnt = min(TEAM_SPAN, n - c0);
+        const int n_stage = (cnt + S - 1) / S;
+        TeamDesc dsc;
+        dsc.fetch(ent + c0, cnt, lane);
+        auto stage_load = [&](StageRegs &R, int st) {
+            const int j = st * S + w;
+            const int idx = j < cnt ? dsc.idx(j) : 0;
+            load_row<T, H, D>(k + (size_t)idx * L::C, lane, R.ra);
+            load_row<T, H, D>(v + (size_t)idx * L::C, lane, R.rb);
+        };
+        auto stage_write = [&](const StageRegs &R, int buf) {
+            lds_put_row<L::EPL>(lds[buf][w][0], lane, R.ra);
+            lds_put_row<L::EPL>(lds[buf][w][1], lane, R.rb);
+        };
+        auto stage_compute = [&](int st, int buf) {
+            int mk[S], any = 0;
+#pragma unroll
+            for (int e = 0; e < S; ++e) {
+                const int j = st * S + e;
+                mk[e] = j < cnt ? (dsc.mask(j) >> (w * RW)) & ((1 << RW) - 1) : 0;
+                any |= mk[e];
+            }
+            if (any == 0) return;
+            float sc[RW][S];
+            // K phase: scores of this stage
+#pragma unroll
+            for (int e = 0; e < S; ++e) {
+                if (mk[e] == 0) continue;
+                float kr[L::EPL];
+                lds_get_row<L::EPL>(lds[buf][e][0], lane, kr);
+#pragma unroll
+                for (int m = 0; m < RW; ++m)
+                    if (mk[e] & (1 << m)) sc[m][e] = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], kr));
+            }
+            // one running-maximum update (and accumulator rescale) per member and stage
+#pragma unroll
+            for (int m = 0; m < RW; ++m) {
+                if ((any & (1 << m)) == 0) continue;
+                float mx = mrun[m];
+#pragma unroll
+                for (int e = 0; e < S; ++e)
+                    if (mk[e] & (1 << m)) mx = fmaxf(mx, sc[m][e]);
+                const float alpha = __builtin_amdgcn_exp2f(mrun[m] - mx);
+                lrun[m] *= alpha;
+#pragma unroll
+                for (int i = 0; i < L::EPL; ++i) acc[m][i] *= alpha;
+                mrun[m] = mx;
+            }
+            // V phase
+#pragma unroll
+            for (int e = 0; e < S; ++e) {
+                if (mk[e] == 0) continue;
+                float vr[L::EPL];
+                lds_get_row<L::EPL>(lds[buf][e][1], lane, vr);
+#pragma unroll
+                for (int m = 0; m < RW; ++m) {
+                    if (mk[e] & (1 << m)) {
+                        const float pe = __builtin_amdgcn_exp2f(sc[m][e] - mrun[m]);
+                        lrun[m] += pe;
+#pragma unroll
+                        for (int i = 0; i < L::EPL; ++i) acc[m][i] = fmaf(pe, vr[i], acc[m][i]);
+                    }
+                }
+            }
+        };
+        StageRegs A, B;
+        stage_load(A, 0);
+        stage_load(B, 1);
+        stage_write(A, 0);
+        stage_load(A, 2);
+        __syncthreads();
+        for (int st = 0; st < n_stage; st += 2) {
+            stage_compute(st, 0);
+            issue_loads_first();
+            stage_write(B, 1);         // B holds stage st + 1
+            stage_load(B, st + 3);
+            __syncthreads();
+            stage_compute(st + 1, 1);  // masks are empty past the last stage
+            issue_loads_first();
+            stage_write(A, 0);         // A holds stage st + 2
+            stage_load(A, st + 4);
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < RW; ++m) {
+        if (rows[m] < 0) continue;
+        if (slots[m] < 0) {
+            const float inv = lrun[m] > 0.f ? 1.f / lrun[m] : 0.f;
+#pragma unroll
+            for (int i = 0; i < L::EPL; ++i) acc[m][i] *= inv;
+            store_row<T, H, D>(o + (size_t)rows[m] * L::C, lane, acc[m]);
+            if (lane % L::LPH == 0) lse[(size_t)rows[m] * H + head] = lrun[m] > 0.f ? mrun[m] + log2f(lrun[m]) : 0.f;
+        } else {
+            store_row_ws<T, H, D>(ws_acc + (size_t)slots[m] * L::C, lane, acc[m]);
+            if (lane % L::LPH == 0) {
+                ws_ml[((size_t)slots[m] * H + head) * 2] = mrun[m];
+                ws_ml[((size_t)slots[m] * H + head) * 2 + 1] = lrun[m];
+            }
+        }
+    }
+}
+
+// Backward, destination side, teams.  pds[(pair, head)] = (p, ds) in the pair order of the source-side plan.
+template <typename T, int H, int D>
+__global__ __launch_bounds__(BLOCK) void k_attn_bwd_dst_team(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k,
+                                                             const T *__restrict__ v, const T *__restrict__ o, const T *__restrict__ d_o,
+                                                             const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
+                                                             float *__restrict__ ws_dq, float scale, float scale_log2e) {
+    using L = Lay<T, H, D>;
+    constexpr int S = TEAM_S, RW = TEAM_RW, F4 = L::EPL / 4;
+    static_assert(S * TEAM_R == WAVE, "one lane per (entry of the stage, pair of the entry)");
+    __shared__ float4 lds[2][S][2][F4 * WAVE];
+    const int t = team_index(P);
+    if (t < 0) return;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), head = lane / L::LPH;
+    int rows[RW], slots[RW];
+#pragma unroll
+    for (int m = 0; m < RW; ++m) {
+        rows[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2]);
+        slots[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2 + 1]);
+    }
+    const int begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[t]);
+    const int n = __builtin_amdgcn_readfirstlane(P.grp_ptr[t + 1]) - begin;
+    const int4 *ent = reinterpret_cast<const int4 *>(P.grp_entries) + begin;
+    const int last_pair = (int)P.n_edges - 1;
+
+    float qv[RW][L::EPL], dov[RW][L::EPL], dqa[RW][L::EPL], delta[RW], lse2[RW];
+#pragma unroll
+    for (int m = 0; m < RW; ++m) {
+        const size_t row = (size_t)max(rows[m], 0);
+        float ov[L::EPL];
+        load_row<T, H, D>(o + row * L::C, lane, ov);
+        load_row<T, H, D>(d_o + row * L::C, lane, dov[m]);
+        load_row<T, H, D>(q + row * L::C, lane, qv[m]);
+        delta[m] = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], ov));
+        lse2[m] = lse[row * H + head];
+#pragma unroll
+        for (int i = 0; i < L::EPL; ++i) dqa[m][i] = 0.f;
+    }
+    // xp: lane e*16 + r holds the scratch position of pair r of entry e of the stage
+    struct StageRegs { float ra[L::EPL], rb[L::EPL]; int xp; };
+    for (int c0 = 0; c0 < n; c0 += TEAM_SPAN) {
+        const int cnt = min(TEAM_SPAN, n - c0);
+        const int n_stage = (cnt + S - 1) / S;
+        TeamDesc dsc;
+        dsc.fetch(ent + c0, cnt, lane);
+        auto stage_load = [&](StageRegs &R, int st) {
+            const int j = st * S + w;
+            const int idx = j < cnt ? dsc.idx(j) : 0;
+            // first pair of entry st*S + lane/16, fetched from the lane that holds that descriptor
+            const int je = min(st * S + (lane >> 4), cnt - 1);
+            const int pb = je < WAVE ? __shfl(dsc.lo.z, je) : __shfl(dsc.hi.z, je - WAVE);
+            R.xp = P.grp_pairs[min(pb + (lane & 15), last_pair)];
+            load_row<T, H, D>(k + (size_t)idx * L::C, lane, R.ra);
+            load_row<T, H, D>(v + (size_t)idx * L::C, lane, R.rb);
+        };
+        auto stage_write = [&](const StageRegs &R, int buf) {
+            lds_put_row<L::EPL>(lds[buf][w][0], lane, R.ra);
+            lds_put_row<L::EPL>(lds[buf][w][1], lane, R.rb);
+        };
+        auto stage_compute = [&](int st, int buf, int xp) {
+#pragma unroll
+            for (int e = 0; e < S; ++e) {
+                const int j = st * S + e;
+                const int mask16 = j < cnt ? dsc.mask(j) : 0;
+                const int mk = (mask16 >> (w * RW)) & ((1 << RW) - 1);
+                if (mk == 0) continue;
+                float kr[L::EPL], vr[L::EPL];
+                lds_get_row<L::EPL>(lds[buf][e][0], lane, kr);
+                lds_get_row<L::EPL>(lds[buf][e][1], lane, vr);
+#pragma unroll
+                for (int m = 0; m < RW; ++m) {
+                    if (mk & (1 << m)) {
+                        const int rank = __builtin_popcount(mask16 & ((1 << (w * RW + m)) - 1));
+                        const unsigned pos = (unsigned)__builtin_amdgcn_readlane(xp, e * TEAM_R + rank);
+                        const float sdot = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], kr));
+                        const float dp = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], vr));
+                        const float pe = __builtin_amdgcn_exp2f(fmaf(sdot, scale_log2e, -lse2[m]));
+                        const float ds = pe * (dp - delta[m]) * scale;
+#pragma unroll
+                        for (int i = 0; i < L::EPL; ++i) dqa[m][i] = fmaf(ds, kr[i], dqa[m][i]);
+                        pds[(size_t)pos * H + head] = make_float2(pe, ds);     // all lanes of a head write the same value
+                    }
+                }
+            }
+        };
+        StageRegs A, B;
+        stage_load(A, 0);
+        stage_load(B, 1);
+        stage_write(A, 0);
+        int xp_even = A.xp, xp_odd = B.xp;
+        stage_load(A, 2);
+        __syncthreads();
+        for (int st = 0; st < n_stage; st += 2) {
+            stage_compute(st, 0, xp_even);
+            issue_loads_first();
+            stage_write(B, 1);         // B holds stage st + 1
+            xp_odd = B.xp;
+            stage_load(B, st + 3);
+            __syncthreads();
+            stage_compute(st + 1, 1, xp_odd);
+            issue_loads_first();
+            stage_write(A, 0);         // A holds stage st + 2
+            xp_even = A.xp;
+            stage_load(A, st + 4);
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < RW; ++m) {
+        if (rows[m] < 0) continue;
+        if (slots[m] < 0) store_row<T, H, D>(dq + (size_t)rows[m] * L::C, lane, dqa[m]);
+        else store_row_ws<T, H, D>(ws_dq + (size_t)slots[m] * L::C, lane, dqa[m]);
+    }
+}
+
+// Backward, source side, teams: dK[src] = sum ds * q[dst], dV[src] = sum p * dO[dst].  The (p, ds) of
+// this plan's pairs are contiguous per stage; the workgroup copies them to LDS with one 16-byte
+// load per thread.
+template <typename T, int H, int D>
+__global__ __launch_bounds__(BLOCK) void k_attn_bwd_src_team(bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o,
+                                                             const float2 *__restrict__ pds, T *__restrict__ dk, T *__restrict__ dv,
+                                                             float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
+    using L = Lay<T, H, D>;
+    constexpr int S = TEAM_S, RW = TEAM_RW, F4 = L::EPL / 4;
+    constexpr int WF4 = S * TEAM_R * H / 2;                 // float4 per stage of weights (at most S*16 pairs)
+    constexpr int WPT = (WF4 + BLOCK - 1) / BLOCK;          // float4 per thread
+    __shared__ float4 lds[2][S][2][F4 * WAVE];
+    __shared__ float4 wts[2][WPT * BLOCK];
+    const int t = team_index(P);
+    if (t < 0) return;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), head = lane / L::LPH;
+    int rows[RW], slots[RW];
+#pragma unroll
+    for (int m = 0; m < RW; ++m) {
+        rows[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2]);
+        slots[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2 + 1]);
+    }
+    const int begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[t]);
+    const int n = __builtin_amdgcn_readfirstlane(P.grp_ptr[t + 1]) - begin;
+    const int4 *ent = reinterpret_cast<const int4 *>(P.grp_entries) + begin;
+    const float4 *pds4 = reinterpret_cast<const float4 *>(pds);
+    const int n_f4 = (int)(P.n_edges * H / 2);              // float4 in the whole scratch
+
+    float ak[RW][L::EPL], av[RW][L::EPL];
+#pragma unroll
+    for (int m = 0; m < RW; ++m)
+#pragma unroll
+        for (int i = 0; i < L::EPL; ++i) { ak[m][i] = 0.f; av[m][i] = 0.f; }
+    struct StageRegs { float ra[L::EPL], rb[L::EPL]; float4 wreg[WPT]; };
+    for (int c0 = 0; c0 < n; c0 += TEAM_SPAN) {
+        const int cnt = min(TEAM_SPAN, n - c0);
+        const int n_stage = (cnt + S - 1) / S;
+        TeamDesc dsc;
+        dsc.fetch(ent + c0, cnt, lane);
+        auto stage_load = [&](StageRegs &R, int st) {
+            const int j = st * S + w;
+            const int idx = j < cnt ? dsc.idx(j) : 0;
+            const int pb0 = dsc.pair0(min(st * S, cnt - 1));                     // first pair of the stage
+#pragma unroll
+            for (int u = 0; u < WPT; ++u) R.wreg[u] = pds4[min(pb0 * (H / 2) + u * BLOCK + tid, n_f4 - 1)];
+            load_row<T, H, D>(q + (size_t)idx * L::C, lane, R.ra);
+            load_row<T, H, D>(d_o + (size_t)idx * L::C, lane, R.rb);
+        };
+        auto stage_write = [&](const StageRegs &R, int buf) {
+            lds_put_row<L::EPL>(lds[buf][w][0], lane, R.ra);
+            lds_put_row<L::EPL>(lds[buf][w][1], lane, R.rb);
+#pragma unroll
+            for (int u = 0; u < WPT; ++u) wts[buf][u * BLOCK + tid] = R.wreg[u];
+        };
+        auto stage_compute = [&](int st, int buf) {
+            if (st >= n_stage) return;
+            const float2 *wbuf = reinterpret_cast<const float2 *>(wts[buf]);
+            const int pb0 = dsc.pair0(st * S);
+#pragma unroll
+            for (int e = 0; e < S; ++e) {
+                const int j = st * S + e;
+                const int mask16 = j < cnt ? dsc.mask(j) : 0;
+                const int mk = (mask16 >> (w * RW)) & ((1 << RW) - 1);
+                if (mk == 0) continue;
+                const int pbe = dsc.pair0(j) - pb0;       // first pair of the entry, relative to the stage
+                float qr[L::EPL], dr[L::EPL];
+                lds_get_row<L::EPL>(lds[buf][e][0], lane, qr);
+                lds_get_row<L::EPL>(lds[buf][e][1], lane, dr);
+#pragma unroll
+                for (int m = 0; m < RW; ++m) {
+                    if (mk & (1 << m)) {
+                        const int lp = pbe + __builtin_popcount(mask16 & ((1 << (w * RW + m)) - 1));
+                        const float2 wgt = wbuf[lp * H + head];
+#pragma unroll
+                        for (int i = 0; i < L::EPL; ++i) {
+                            ak[m][i] = fmaf(wgt.y, qr[i], ak[m][i]);
+                            av[m][i] = fmaf(wgt.x, dr[i], av[m][i]);
+                        }
+                    }
+                }
+            }
+        };
+        StageRegs A, B;
+        stage_load(A, 0);
+        stage_load(B, 1);
+        stage_write(A, 0);
+        stage_load(A, 2);
+        __syncthreads();
+        for (int st = 0; st < n_stage; st += 2) {
+            stage_compute(st, 0);
+            issue_loads_first();
+            stage_write(B, 1);         // B holds stage st + 1
+            stage_load(B, st + 3);
+            __syncthreads();
+            stage_compute(st + 1, 1);
+            issue_loads_first();
+            stage_write(A, 0);         // A holds stage st + 2
+            stage_load(A, st + 4);
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < RW; ++m) {
+        if (rows[m] < 0) continue;
+        if (slots[m] < 0) {
+            store_row<T, H, D>(dk + (size_t)rows[m] * L::C, lane, ak[m]);
+            store_row<T, H, D>(dv + (size_t)rows[m] * L::C, lane, av[m]);
+        } else {
+            store_row_ws<T, H, D>(ws_dk + (size_t)slots[m] * L::C, lane, ak[m]);
+            store_row_ws<T, H, D>(ws_dv + (size_t)slots[m] * L::C, lane, av[m]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
 inline int grid_for(const bpt_plan *p) { return (int)((p->n_items + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK); }
@@ -1022,7 +1431,7 @@ inline int check_plan(const bpt_plan *p, bool need_idx) {
     if (p->n_edges > 0 && (!p->eid || (need_idx && !p->idx))) return BPT_ERR_NULL;
     if (p->n_heavy > 0 && !p->heavy) return BPT_ERR_NULL;
     if (p->n_items < p->n_rows) return BPT_ERR_SIZE;     // every row owns at least one item
-    if (p->n_groups < 0 || p->grp_R < 0 || p->grp_R > 8) return BPT_ERR_SIZE;
+    if (p->n_groups < 0 || p->grp_R < 0 || p->grp_R > 16) return BPT_ERR_SIZE;
     if (p->n_groups > 0 && (!p->grp_members || !p->grp_ptr || !p->grp_chunks || (p->n_edges > 0 && !p->grp_entries))) return BPT_ERR_NULL;
     if (p->n_groups > 0 && (p->grp_max_chunk < 1 || p->grp_max_chunk > p->n_groups)) return BPT_ERR_SIZE;
     return BPT_OK;
@@ -1186,6 +1595,11 @@ inline int group_grid(const bpt_plan *P, int kernel) {
     return (int)(8 * n);
 }
 
+inline bool has_teams(const bpt_plan *P) {
+    return P->n_groups > 0 && P->grp_R == TEAM_R && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
+           P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups;
+}
+
 inline bool has_groups(const bpt_plan *P) {
     return P->n_groups > 0 && P->grp_R == GROUP_R && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
            P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups;
@@ -1198,7 +1612,10 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
-        if (has_groups(P)) {
+        if (has_teams(P)) {
+            hipLaunchKernelGGL((k_attn_fwd_team<T, H, D>), dim3((int)(8 * P->grp_max_chunk)), dim3(BLOCK), 0, s, *P, (const T *)q,
+                               (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+        } else if (has_groups(P)) {
 #define LAUNCH_FWD_GRP(B, W)                                                                                                   \
     hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, GROUP_R, B, W>), dim3(group_grid(P, 0)), dim3(WAVE), 0, s, *P, (const T *)q,   \
                        (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E)
@@ -1264,9 +1681,43 @@ int run_attn_bwd_grouped(const bpt_plan *Pin, const bpt_plan *Pout, const void *
 }
 
 template <typename T, int H, int D>
+int run_attn_bwd_team(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
+                      const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
+    const size_t EH = (size_t)Pin->n_edges * H;
+    float2 *pds = (float2 *)ws;
+    float *ws_rows = (float *)ws + 2 * (round16((int64_t)EH * 4) / 4);
+    {
+        ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
+        hipLaunchKernelGGL((k_attn_bwd_dst_team<T, H, D>), dim3((int)(8 * Pin->grp_max_chunk)), dim3(BLOCK), 0, s, *Pin, (const T *)q,
+                           (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E);
+    }
+    int st = launch_status();
+    if (st != BPT_OK) return st;
+    if (Pin->n_heavy > 0) {
+        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, Pin->heavy,
+                           (const float *)ws_rows, (T *)dq, (T *)nullptr, H * D, (size_t)0);
+        st = launch_status();
+        if (st != BPT_OK) return st;
+    }
+    float *ws_dk = ws_rows, *ws_dv = ws_rows + (size_t)Pout->n_slots * H * D;
+    {
+        ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
+        hipLaunchKernelGGL((k_attn_bwd_src_team<T, H, D>), dim3((int)(8 * Pout->grp_max_chunk)), dim3(BLOCK), 0, s, *Pout, (const T *)q,
+                           (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv);
+    }
+    st = launch_status();
+    if (st != BPT_OK || Pout->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pout->n_heavy, H * D / WAVE, 2), dim3(BLOCK), 0, s, Pout->heavy,
+                       (const float *)ws_dk, (T *)dk, (T *)dv, H * D, (size_t)Pout->n_slots * H * D);
+    return launch_status();
+}
+
+template <typename T, int H, int D>
 int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
                  const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
     if (Pin->n_items == 0) return BPT_OK;
+    if (has_teams(Pin) && has_teams(Pout) && Pin->grp_pairs)
+        return run_attn_bwd_team<T, H, D>(Pin, Pout, q, k, v, o, d_o, lse, dq, dk, dv, ws, scale, s);
     if (has_groups(Pin) && has_groups(Pout) && Pin->grp_pairs)
         return run_attn_bwd_grouped<T, H, D>(Pin, Pout, q, k, v, o, d_o, lse, dq, dk, dv, ws, scale, s);
     const size_t EH = (size_t)Pin->n_edges * H;

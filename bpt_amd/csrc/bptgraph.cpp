@@ -380,7 +380,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
     if (!items || !members || !grp_ptr || !chunks || !n_groups_out || !n_entries_out) return BPTG_ERR_NULL;
     if (n_edges > 0 && (!idx32 || !eid32 || !entries || !pair_eid)) return BPTG_ERR_NULL;
     if (n_items < 0 || n_edges < 0 || n_index_nodes < 0) return BPTG_ERR_SIZE;
-    if (R < 1 || R > 8 || window < 0 || order_mode < 0 || order_mode > 2) return BPTG_ERR_ARG;
+    if (R < 1 || R > 16 || window < 0 || order_mode < 0 || order_mode > 2) return BPTG_ERR_ARG;
     for (int64_t i = 0; i < n_items; ++i) {
         const int32_t *it = items + 4 * i;
         if (it[1] < 0 || it[2] < it[1] || it[2] > n_edges) return BPTG_ERR_RANGE;
@@ -409,7 +409,8 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
         const int32_t first = order[(size_t)oi];
         if (used[(size_t)first]) continue;
         used[(size_t)first] = 1;
-        int32_t mem[8] = {-1, -1, -1, -1, -1, -1, -1, -1};
+        int32_t mem[16];
+        for (int32_t m = 0; m < 16; ++m) mem[m] = -1;
         int32_t n_mem = 1;
         mem[0] = first;
         int64_t w = 0;
@@ -496,8 +497,8 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
         size_t a = 0;
         while (a < tri.size()) {
             size_t b = a;
-            int32_t cnt[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            size_t start[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            int32_t cnt[16] = {0};
+            size_t start[16] = {0};
             while (b < tri.size() && tri[b].idx == tri[a].idx) {
                 if (cnt[tri[b].member] == 0) start[tri[b].member] = b;
                 ++cnt[tri[b].member];

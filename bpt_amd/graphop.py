@@ -271,6 +271,16 @@ def set_row_groups(on):
     return old
 
 
+def set_group_rows(R):
+    """Rows per group of the fused kernels: 16 = teams of 4 wavefronts sharing neighbour rows through LDS
+    (default), 4 = one wavefront per group.  Returns the previous value."""
+    from . import plan as _plan
+    if R not in (4, 16):
+        raise ValueError("R must be 4 or 16")
+    old, _plan.GROUP_R = _plan.GROUP_R, R
+    return old
+
+
 def set_group_variant(fwd=None, bwd_dst=None, bwd_src=None):
     """Tuning of the row-group kernels (see bpt_set_group_variant): 4, 2 or 3 per kernel; None keeps the current one."""
     for kernel, var in enumerate((fwd, bwd_dst, bwd_src)):

@@ -17,7 +17,7 @@ import torch
 from ._lib import PlanInfo, PlanStruct, check_graph, graph_lib
 
 DEFAULT_SEG_LEN = 64
-GROUP_R = 4            # rows per wavefront in the fused row-group kernels (matches the HIP library)
+GROUP_R = 4            # rows per group: 4 = one wavefront per group (default, fastest measured); 16 = a team of 4 wavefronts x 4 rows sharing rows through LDS
 GROUP_WINDOW = 32      # how many following items the greedy grouping examines per group
 GROUP_ORDER = 2        # order of the groups inside an XCD chunk: 0 locality, 1 big first / small last, 2 decreasing work
 _CACHE_SIZE = 64
@@ -61,18 +61,19 @@ def build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len=DE
     return arrays, info
 
 
-def build_groups_host(arrays, n_index_nodes, R=GROUP_R, window=GROUP_WINDOW, order_mode=None):
+def build_groups_host(arrays, n_index_nodes, R=None, window=GROUP_WINDOW, order_mode=None):
     """Pure host step: clusters the plan's items into row groups (bptg_group_plan).  Returns a dict
     with members (n_groups, R, 2), grp_ptr (n_groups + 1), entries (n_entries, 4), pair_eid (n_edges),
     chunks (9,)."""
     order_mode = GROUP_ORDER if order_mode is None else order_mode
+    R = GROUP_R if R is None else R
     items = np.ascontiguousarray(arrays["items"], dtype=np.int32)
     idx = np.ascontiguousarray(arrays["idx"], dtype=np.int32)
     eid = np.ascontiguousarray(arrays["eid"], dtype=np.int32)
     n_items, E = len(items), len(eid)
     members = np.empty((max(n_items, 1), R, 2), dtype=np.int32)
     grp_ptr = np.empty(n_items + 1, dtype=np.int32)
-    entries = np.empty((max(E, 1), 4), dtype=np.int32)
+    entries = np.zeros((E + 1, 4), dtype=np.int32)      # one zero row of padding: kernels may peek at entries[n_entries]
     pair_eid = np.empty(max(E, 1), dtype=np.int32)
     chunks = np.zeros(9, dtype=np.int32)
     ng, ne = ctypes.c_int64(), ctypes.c_int64()
@@ -80,7 +81,8 @@ def build_groups_host(arrays, n_index_nodes, R=GROUP_R, window=GROUP_WINDOW, ord
                                             int(order_mode), _ptr(members), _ptr(grp_ptr), _ptr(entries), _ptr(pair_eid),
                                             _ptr(chunks), ctypes.byref(ng), ctypes.byref(ne)))
     return {"members": members[:ng.value].copy(), "grp_ptr": grp_ptr[:ng.value + 1].copy(),
-            "entries": entries[:ne.value].copy(), "pair_eid": pair_eid[:E].copy(), "chunks": chunks}
+            "entries": entries[:ne.value].copy(), "entries_padded": entries[:ne.value + 1].copy(),
+            "pair_eid": pair_eid[:E].copy(), "chunks": chunks, "R": R}
 
 
 class Plan:
@@ -116,19 +118,21 @@ class Plan:
     def ensure_groups(self):
         """Builds the row-group arrays once (host) and uploads them; returns the host dict."""
         with self._lock:
-            if self._groups is None:
+            if self._groups is None or self._groups["R"] != GROUP_R:
+                self._links = {}
                 grp = build_groups_host(self._host, self.n_index_nodes)
-                self._grp_dev = {k: torch.from_numpy(v).to(self.device) for k, v in grp.items() if k != "pair_eid"}
+                self._grp_dev = {k: torch.from_numpy(grp[k]).to(self.device)
+                                 for k in ("members", "grp_ptr", "entries_padded", "chunks")}
                 d = self._grp_dev
                 self.n_groups = len(grp["members"])
                 self.struct.grp_members = d["members"].data_ptr() if self.n_groups else None
                 self.struct.grp_ptr = d["grp_ptr"].data_ptr()
-                self.struct.grp_entries = d["entries"].data_ptr() if len(grp["entries"]) else None
+                self.struct.grp_entries = d["entries_padded"].data_ptr()
                 self.struct.grp_pairs = None
                 self.struct.grp_chunks = d["chunks"].data_ptr()
                 self.struct.grp_max_chunk = int(np.diff(grp["chunks"]).max()) if self.n_groups else 0
                 self.struct.n_groups = self.n_groups
-                self.struct.grp_R = GROUP_R
+                self.struct.grp_R = grp["R"]
                 self._groups = grp
         return self._groups
 
@@ -136,7 +140,7 @@ class Plan:
         """`bpt_plan` of this (destination-side) plan whose grp_pairs maps each of its pairs to the number of
         the same edge's pair in `plan_src` (the source-side plan of the same graph)."""
         mine, theirs = self.ensure_groups(), plan_src.ensure_groups()
-        key = id(plan_src)
+        key = (id(plan_src), GROUP_R)
         with self._lock:
             hit = self._links.get(key)
             if hit is None:

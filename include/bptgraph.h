@@ -81,7 +81,7 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
                    bptg_plan_info *info);
 
 /* ---- row groups ------------------------------------------------------------------------------
- * Clusters the plan's items (rows / row segments) into groups of at most R (<= 8) members that read
+ * Clusters the plan's items (rows / row segments) into groups of at most R (<= 16) members that read
  * mostly the same neighbour rows, so that one wavefront can load each neighbour row once for all of
  * them.  Inputs are the arrays bptg_plan_fill produced.  Outputs (caller allocates the upper bounds
  * given in brackets):

@@ -5,7 +5,9 @@ import pytest
 
 import oracle
 from bpt_amd import graphbuilder as gb
-from bpt_amd.plan import GROUP_R, build_groups_host, build_plan_host
+from bpt_amd.plan import build_groups_host, build_plan_host
+
+from bpt_amd.plan import GROUP_R
 
 
 def bpt(L, triu, step):
@@ -36,14 +38,16 @@ def plans(name, seg=64):
     return src, dst, n, csr, pin, pout
 
 
+@pytest.mark.parametrize("GROUP_R", [4, 16])
 @pytest.mark.parametrize("order_mode", [0, 1, 2])
 @pytest.mark.parametrize("seg", [8, 64])
 @pytest.mark.parametrize("name", sorted(GRAPHS))
-def test_group_plan_invariants(name, seg, order_mode):
+def test_group_plan_invariants(name, seg, order_mode, GROUP_R):
     src, dst, n, csr, pin, pout = plans(name, seg)
     E = len(src)
     for arrays, rows_of, cols_of in ((pin, dst, src), (pout, src, dst)):
-        grp = build_groups_host(arrays, n, order_mode=order_mode)
+        grp = build_groups_host(arrays, n, R=GROUP_R, order_mode=order_mode)
+        assert grp["entries_padded"].shape[0] == grp["entries"].shape[0] + 1 and not grp["entries_padded"][-1].any()
         members, gptr, entries, pair_eid = grp["members"], grp["grp_ptr"], grp["entries"], grp["pair_eid"]
         ch = grp["chunks"]
         assert ch[0] == 0 and ch[8] == len(members) and np.all(np.diff(ch) >= 0)
@@ -170,9 +174,11 @@ def test_grouping_reduces_row_loads_on_the_headline_graph():
     pin, _ = build_plan_host(COL, IC, in_csr[2], in_csr[1], n, n)
     pout, _ = build_plan_host(ROW, IR, out_csr[2], out_csr[1], n, n)
     for arrays in (pin, pout):
-        grp = build_groups_host(arrays, n)
-        assert len(grp["entries"]) < 0.42 * len(src)        # neighbour-row loads per kernel vs one per edge
-        assert len(grp["members"]) < 0.3 * len(arrays["items"])
+        g16 = build_groups_host(arrays, n, R=16)
+        assert len(g16["entries"]) < 0.18 * len(src)        # neighbour-row fetches per kernel vs one per edge
+        assert len(g16["members"]) < 0.08 * len(arrays["items"])
+        grp = build_groups_host(arrays, n, R=4)
+        assert len(grp["entries"]) < 0.42 * len(src)
         # XCD chunks carry about equal work (pairs)
         pc = np.array([bin(m).count("1") for m in grp["entries"][:, 1]])
         cum = np.concatenate([[0], np.cumsum(pc)])
