@@ -101,10 +101,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies (known HBM bytes) so counter runs can be scaled")
+    ap.add_argument("--group-rows", type=int, default=None, choices=[4, 8], help="rows per wavefront group of the fused kernels (default: 8 where available, else 4)")
     ap.add_argument("--rows", action="store_true", help="fused kernels with one wavefront per row (no row groups)")
-    ap.add_argument("--group-rows", type=int, default=4, choices=[4, 16], help="4: one wavefront per row group (default); 16: teams of 4 wavefronts sharing rows through LDS")
-    ap.add_argument("--waves", default=None, help="persistent wavefronts per XCD fwd,bwd_dst,bwd_src (0 = one per group)")
-    ap.add_argument("--variants", default=None, help="row-group kernel variants fwd,bwd_dst,bwd_src (each 2, 3 or 4)")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -120,10 +118,6 @@ def main():
     dev = "cuda:0"
     graphop.set_row_groups(not args.rows)
     graphop.set_group_rows(args.group_rows)
-    if args.waves:
-        graphop.set_group_waves(*[int(x) for x in args.waves.split(",")])
-    if args.variants:
-        graphop.set_group_variant(*[int(x) for x in args.variants.split(",")])
     desc, graphs, H, D, default_dtype = make_workload(args.workload)
     dtype_name = args.dtype or default_dtype
     tdtype = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
@@ -240,7 +234,7 @@ def main():
         "dtype": dtype_name, "data": "synthetic",
         "config": {"workload": desc + (" (unfused op chain)" if args.unfused else " (fused fwd+bwd)"), "n_nodes": N,
                    "n_edges": E, "heads": H, "d_head": D, "launch": mode,
-                   "kernels": "per-row" if args.rows else ("teams(4 wavefronts x 4 rows, LDS-shared)" if args.group_rows == 16 else "row-groups(4 rows per wavefront)")},
+                   "kernels": "per-row" if args.rows else f"row-groups({args.group_rows or 'auto'} rows per wavefront)"},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "step_roofline": {"algorithmic_bytes": alg["total"], "achieved_GBps": round(step_gbs, 1),

@@ -17,7 +17,8 @@ class PlanStruct(ctypes.Structure):
     _fields_ = [("rowptr", c_vp), ("idx", c_vp), ("eid", c_vp), ("items", c_vp), ("heavy", c_vp),
                 ("n_rows", c_i64), ("n_edges", c_i64), ("n_items", c_i64), ("n_heavy", c_i64), ("n_slots", c_i64),
                 ("grp_members", c_vp), ("grp_ptr", c_vp), ("grp_entries", c_vp), ("grp_pairs", c_vp),
-                ("grp_chunks", c_vp), ("n_groups", c_i64), ("grp_R", c_i64), ("grp_max_chunk", c_i64)]
+                ("grp_chunks", c_vp), ("n_groups", c_i64), ("grp_R", c_i64), ("grp_max_chunk", c_i64),
+                ("n_grp_entries", c_i64)]
 
 
 class PlanInfo(ctypes.Structure):
@@ -37,7 +38,7 @@ GRAPH_API = {
     "bptg_plan_fill": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64,
                                       c_vp, c_vp, c_vp, c_vp, c_vp, ctypes.POINTER(PlanInfo)]),
     "bptg_group_plan": (ctypes.c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_i64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
-                                       c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
+                                       ctypes.c_int32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
 }
 
 _PP = ctypes.POINTER(PlanStruct)
@@ -45,8 +46,6 @@ _tail = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_vp]          # h, d, dtype,
 ATTN_API = {
     "bpt_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "bpt_set_force_generic": (ctypes.c_int, [ctypes.c_int]),
-    "bpt_set_group_variant": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
-    "bpt_set_group_waves": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
     "bpt_profile_kernel": (ctypes.c_int, [ctypes.c_int, c_vp, c_vp]),
     "bpt_workspace_bytes": (c_i64, [ctypes.c_int, _PP, _PP, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "bpt_maskedmm_csr_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp] + _tail),

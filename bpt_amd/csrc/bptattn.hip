@@ -32,11 +32,6 @@ constexpr float M_INIT_LOG2 = -1.4426950408889634e9f;   // -1e9 (graphop_kernel.
 constexpr float LOG2E = 1.4426950408889634f;
 
 std::atomic<int> g_force_generic{0};
-// tuning of the row-group kernels, one value per kernel (fwd, bwd_dst, bwd_src): 4 = batches of four
-// neighbour rows; 2 = batches of two; 3 = batches of two compiled for three waves per SIMD
-std::atomic<int> g_group_variant[3] = {{2}, {2}, {2}};
-// wavefronts per XCD that walk the groups of that XCD's chunk (0: one wavefront per group)
-std::atomic<int> g_group_waves[3] = {{0}, {0}, {0}};
 
 // optional measurement hook (bpt_profile_kernel): which main kernel to bracket with events
 std::atomic<int> g_prof_which{0};
@@ -57,6 +52,7 @@ struct ProfScope {
 // element types
 // ------------------------------------------------------------------------------------------
 struct bf16_t { uint16_t bits; };
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
@@ -317,6 +313,7 @@ template <typename T, int H_, int D_> struct Lay {
     static constexpr int VE = 16 / (int)sizeof(T);      // elements per 16-byte vector
     static constexpr int NV = EPL / VE;                 // 16-byte vectors per lane
     static_assert(64 % H_ == 0 && C % 64 == 0 && EPL % VE == 0 && NV >= 1, "unsupported fast shape");
+    static_assert(LPH >= 4, "the row-group kernels broadcast per-member values inside quads of one head");
     static_assert(D_ == NV * LPH * VE, "layout does not tile the head");
     // element offset inside a node row of vector i of `lane`: LPH consecutive lanes cover
     // LPH*16 contiguous bytes of their head
@@ -675,360 +672,102 @@ __global__ __launch_bounds__(BLOCK) void k_attn_bwd_dst(bpt_plan P, const T *__r
 }
 
 // ------------------------------------------------------------------------------------------
-// row-group kernels of the fused path: one wavefront owns up to R rows (or row segments) that
-// share neighbours; every neighbour row of the group's union is loaded once and used for all
-// members that have an edge to it (entry mask).  One wavefront per workgroup.
+// row-group kernels of the fused path: one wavefront (= one workgroup) owns a group of up to
+// R (4 or 8) rows (or row segments) that share neighbours; every neighbour row of the group's union
+// ("entry") is loaded once and used for all members that have an edge to it (entry mask).
+//
+// The kernels issue about one instruction per four cycles and SIMD, whatever its kind, so they are
+// written for a low instruction count per (member, entry) pair: 32-bit byte offsets from uniform
+// base pointers (no 64-bit vector address arithmetic), the entry list of up to GRP_CHUNK entries
+// held one per lane and read with v_readlane, per-pair scratch addressed by entry * R + member
+// (no popcounts), unmasked scratch stores.
 // ------------------------------------------------------------------------------------------
+// entries whose rows are loaded together (one where a row takes 16 registers per lane)
+template <int EPL> constexpr int grp_batch() { return EPL >= 16 ? 1 : 2; }
+constexpr int GRP_CHUNK = 56;                      // entries per lane-held list: a multiple of twice the batch, and
+                                                   // GRP_CHUNK + 3 * batch <= 64 keeps every look-ahead index a lane id
+constexpr int GRP_PAD_ENTRIES = 8;                 // the per-entry arrays are readable this far past the end
+
 template <int R> struct GroupHead {
     int rows[R], slots[R], begin, end;
 };
 
-template <int R> __device__ __forceinline__ GroupHead<R> fetch_group(const bpt_plan &P, int g) {
-    GroupHead<R> gh;
+// wavefronts per SIMD the row-group kernels are compiled for: the members' state has to stay in registers
+template <typename T, int EPL, int R> constexpr int grp_wpe() { return R * EPL <= 32 ? 3 : 2; }
+
+// Workgroup b (one wavefront) runs on XCD b % 8 and takes group number b / 8 of that XCD's chunk.
+template <int R> __device__ __forceinline__ bool fetch_group(const bpt_plan &P, GroupHead<R> &gh) {
+    const int x = blockIdx.x & 7, w = blockIdx.x >> 3;
+    const int g = __builtin_amdgcn_readfirstlane(P.grp_chunks[x]) + w;
+    if (g >= __builtin_amdgcn_readfirstlane(P.grp_chunks[x + 1])) return false;
+    const int lane = threadIdx.x;
+    const int mem = P.grp_members[(size_t)g * (2 * R) + (lane & (2 * R - 1))];
+    const int ptr = P.grp_ptr[g + (lane & 1)];
 #pragma unroll
     for (int m = 0; m < R; ++m) {
-        gh.rows[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)g * R + m) * 2]);
-        gh.slots[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)g * R + m) * 2 + 1]);
+        gh.rows[m] = __builtin_amdgcn_readlane(mem, 2 * m);
+        gh.slots[m] = __builtin_amdgcn_readlane(mem, 2 * m + 1);
     }
-    gh.begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[g]);
-    gh.end = __builtin_amdgcn_readfirstlane(P.grp_ptr[g + 1]);
-    return gh;
+    gh.begin = __builtin_amdgcn_readlane(ptr, 0);
+    gh.end = __builtin_amdgcn_readlane(ptr, 1);
+    return true;
 }
 
-// Persistent walk over the groups of one XCD chunk.  Workgroup b (one wavefront) runs on XCD b % 8; it
-// takes the groups first + b/8, + stride, + 2*stride, ... of that XCD's chunk, stride = gridDim.x / 8.
-// A group costs a chain of dependent loads before its first FMA (header -> entries -> rows); the walk
-// hides it by fetching the header two groups ahead and the first 64 entries one group ahead.  With
-// gridDim.x = 8 * (largest chunk) every wavefront gets exactly one group.
-template <int R, class Body>
-__device__ __forceinline__ void walk_groups(const bpt_plan &P, Body &&body) {
-    const int x = blockIdx.x & 7, w = blockIdx.x >> 3, stride = gridDim.x >> 3;
-    const int first = __builtin_amdgcn_readfirstlane(P.grp_chunks[x]), last = __builtin_amdgcn_readfirstlane(P.grp_chunks[x + 1]);
-    int g = first + w;
-    if (g >= last) return;
-    const int lane = threadIdx.x;
-    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
-    GroupHead<R> cur = fetch_group<R>(P, g);
-    GroupHead<R> nxt = fetch_group<R>(P, min(g + stride, last - 1));
-    int4 ent_cur = lane < min(WAVE, cur.end - cur.begin) ? entries[cur.begin + lane] : make_int4(0, 0, 0, 0);
-    for (; g < last; g += stride) {
-        const GroupHead<R> nn = fetch_group<R>(P, min(g + 2 * stride, last - 1));
-        const int ncnt = g + stride < last ? min(WAVE, nxt.end - nxt.begin) : 0;
-        const int4 ent_nxt = lane < ncnt ? entries[nxt.begin + lane] : make_int4(0, 0, 0, 0);
-        body(cur, ent_cur);
-        cur = nxt;
-        nxt = nn;
-        ent_cur = ent_nxt;
+// Row `row` of a node tensor through a uniform base pointer, a uniform 32-bit row offset and this lane's
+// constant byte offset `loff` (global_load with scalar base + 32-bit vector offset + immediate).
+template <typename T, int H, int D>
+__device__ __forceinline__ void load_row32(const T *__restrict__ base, uint32_t row, uint32_t loff, float (&out)[Lay<T, H, D>::EPL]) {
+    using L = Lay<T, H, D>;
+    const char *p = reinterpret_cast<const char *>(base) + (size_t)(row * (uint32_t)(L::C * sizeof(T)));
+#pragma unroll
+    for (int i = 0; i < L::NV; ++i) {
+        const char *pi = p + (size_t)(loff + (uint32_t)(i * L::LPH * 16));
+        if constexpr (sizeof(T) == 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(pi);
+            out[4 * i] = v.x; out[4 * i + 1] = v.y; out[4 * i + 2] = v.z; out[4 * i + 3] = v.w;
+        } else {
+            const uint4 v = *reinterpret_cast<const uint4 *>(pi);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                out[8 * i + 2 * c] = __uint_as_float(w[c] << 16);
+                out[8 * i + 2 * c + 1] = __uint_as_float(w[c] & 0xffff0000u);
+            }
+        }
     }
 }
 
-// All three kernels run the same two-stage software pipeline over a group's entries: while the rows
-// of batch i are being used, the loads of batch i+1 are already in flight (two register buffers,
-// unconditional loads: a batch past the end re-reads the chunk's first row with an empty mask).
-template <typename T, int H, int D, int R, int BATCH, int WPE>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_fwd_grp(
-    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
-    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+// The same row as loaded, not yet converted: the software pipeline keeps rows in flight in this form, and
+// converts them where they are used, after the wait (bf16 to f32 costs a shift or a mask per element).
+template <typename T, int H, int D> struct RawRow { uint32_t w[Lay<T, H, D>::EPL * sizeof(T) / 4]; };
+
+template <typename T, int H, int D>
+__device__ __forceinline__ void load_row32_raw(const T *__restrict__ base, uint32_t row, uint32_t loff, RawRow<T, H, D> &out) {
     using L = Lay<T, H, D>;
-    const int lane = threadIdx.x, head = lane / L::LPH;
-    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
-    struct Batch {
-        float kv[BATCH][L::EPL], vv[BATCH][L::EPL];
-        int mk[BATCH], any;
-    };
-    walk_groups<R>(P, [&](const GroupHead<R> &gh, const int4 &ent0) {
-        float qv[R][L::EPL], acc[R][L::EPL], mrun[R], lrun[R];
+    const char *p = reinterpret_cast<const char *>(base) + (size_t)(row * (uint32_t)(L::C * sizeof(T)));
 #pragma unroll
-        for (int m = 0; m < R; ++m) {
-            load_row<T, H, D>(q + (size_t)max(gh.rows[m], 0) * L::C, lane, qv[m]);
-            mrun[m] = M_INIT_LOG2;
-            lrun[m] = 0.f;
-#pragma unroll
-            for (int i = 0; i < L::EPL; ++i) { qv[m][i] *= scale_log2e; acc[m][i] = 0.f; }
-        }
-        for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
-            const int cnt = min(WAVE, gh.end - p0);
-            int4 ent = ent0;
-            if (p0 != gh.begin) ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
-            auto load_batch = [&](Batch &B, int b) {
-                B.any = 0;
-#pragma unroll
-                for (int e = 0; e < BATCH; ++e) {
-                    const bool ok = b + e < cnt;
-                    const int j = ok ? b + e : 0;
-                    const int src = __builtin_amdgcn_readlane(ent.x, j);
-                    B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
-                    B.any |= B.mk[e];
-#ifdef BPT_PROBE_NO_LOADS
-#pragma unroll
-                    for (int i = 0; i < L::EPL; ++i) { B.kv[e][i] = qv[0][i] + (float)src; B.vv[e][i] = qv[1][i] - (float)src; }
-#else
-                    load_row<T, H, D>(k + (size_t)src * L::C, lane, B.kv[e]);
-                    load_row<T, H, D>(v + (size_t)src * L::C, lane, B.vv[e]);
-#endif
-                }
-            };
-            auto compute = [&](const Batch &B) {
-#ifdef BPT_PROBE_NO_MATH
-#pragma unroll
-                for (int e = 0; e < BATCH; ++e) acc[0][0] += B.kv[e][0] + B.vv[e][0] + B.kv[e][L::EPL - 1] + B.vv[e][L::EPL - 1];
-                return;
-#endif
-#pragma unroll
-                for (int m = 0; m < R; ++m) {
-                    const int bit = 1 << m;
-                    if ((B.any & bit) == 0) continue;
-                    float s[BATCH], mx = mrun[m];
-#pragma unroll
-                    for (int e = 0; e < BATCH; ++e) {
-                        s[e] = -INFINITY;
-                        if (B.mk[e] & bit) {
-                            s[e] = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], B.kv[e]));
-                            mx = fmaxf(mx, s[e]);
-                        }
-                    }
-                    const float alpha = __builtin_amdgcn_exp2f(mrun[m] - mx);
-                    lrun[m] *= alpha;
-#pragma unroll
-                    for (int i = 0; i < L::EPL; ++i) acc[m][i] *= alpha;
-#pragma unroll
-                    for (int e = 0; e < BATCH; ++e) {
-                        if (B.mk[e] & bit) {
-                            const float pe = __builtin_amdgcn_exp2f(s[e] - mx);
-                            lrun[m] += pe;
-#pragma unroll
-                            for (int i = 0; i < L::EPL; ++i) acc[m][i] = fmaf(pe, B.vv[e][i], acc[m][i]);
-                        }
-                    }
-                    mrun[m] = mx;
-                }
-            };
-            Batch A, B;
-            load_batch(A, 0);
-            for (int b = 0; b < cnt; b += 2 * BATCH) {
-                load_batch(B, b + BATCH);
-                issue_loads_first();
-                compute(A);
-                issue_loads_first();
-                load_batch(A, b + 2 * BATCH);
-                issue_loads_first();
-                compute(B);
-                issue_loads_first();
-            }
-        }
-#pragma unroll
-        for (int m = 0; m < R; ++m) {
-            if (gh.rows[m] < 0) continue;
-            if (gh.slots[m] < 0) {
-                const float inv = lrun[m] > 0.f ? 1.f / lrun[m] : 0.f;
-#pragma unroll
-                for (int i = 0; i < L::EPL; ++i) acc[m][i] *= inv;
-                store_row<T, H, D>(o + (size_t)gh.rows[m] * L::C, lane, acc[m]);
-                if (lane % L::LPH == 0) lse[(size_t)gh.rows[m] * H + head] = lrun[m] > 0.f ? mrun[m] + log2f(lrun[m]) : 0.f;
-            } else {
-                store_row_ws<T, H, D>(ws_acc + (size_t)gh.slots[m] * L::C, lane, acc[m]);
-                if (lane % L::LPH == 0) {
-                    ws_ml[((size_t)gh.slots[m] * H + head) * 2] = mrun[m];
-                    ws_ml[((size_t)gh.slots[m] * H + head) * 2 + 1] = lrun[m];
-                }
-            }
-        }
-    });
+    for (int i = 0; i < L::NV; ++i) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p + (size_t)(loff + (uint32_t)(i * L::LPH * 16)));
+        out.w[4 * i] = v.x; out.w[4 * i + 1] = v.y; out.w[4 * i + 2] = v.z; out.w[4 * i + 3] = v.w;
+    }
 }
 
-// Backward, destination side, row groups.  pds[(pair, head)] = (p, ds) in the pair order of the
-// source-side plan (P.grp_pairs maps this plan's pairs to it).
-template <typename T, int H, int D, int R, int BATCH, int WPE>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_dst_grp(
-    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
-    const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
-    float *__restrict__ ws_dq, float scale, float scale_log2e) {
+template <typename T, int H, int D>
+__device__ __forceinline__ void unpack_row(const RawRow<T, H, D> &in, float (&out)[Lay<T, H, D>::EPL]) {
     using L = Lay<T, H, D>;
-    const int lane = threadIdx.x, head = lane / L::LPH;
-    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
-    const int last_pair = (int)P.n_edges - 1;
-    struct Batch {
-        float kv[BATCH][L::EPL], vv[BATCH][L::EPL];
-        int mk[BATCH], xp[BATCH], any;
-    };
-    walk_groups<R>(P, [&](const GroupHead<R> &gh, const int4 &ent0) {
-        float qv[R][L::EPL], dov[R][L::EPL], dqa[R][L::EPL], delta[R], lse2[R];
+    if constexpr (sizeof(T) == 4) {
 #pragma unroll
-        for (int m = 0; m < R; ++m) {
-            const size_t row = (size_t)max(gh.rows[m], 0);
-            float ov[L::EPL];
-            load_row<T, H, D>(o + row * L::C, lane, ov);
-            load_row<T, H, D>(d_o + row * L::C, lane, dov[m]);
-            load_row<T, H, D>(q + row * L::C, lane, qv[m]);
-            delta[m] = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], ov));
-            lse2[m] = lse[row * H + head];
+        for (int i = 0; i < L::EPL; ++i) out[i] = __uint_as_float(in.w[i]);
+    } else {
 #pragma unroll
-            for (int i = 0; i < L::EPL; ++i) dqa[m][i] = 0.f;
+        for (int j = 0; j < L::EPL / 2; ++j) {
+            out[2 * j] = __uint_as_float(in.w[j] << 16);
+            out[2 * j + 1] = __uint_as_float(in.w[j] & 0xffff0000u);
         }
-        for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
-            const int cnt = min(WAVE, gh.end - p0);
-            int4 ent = ent0;
-            if (p0 != gh.begin) ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
-            auto load_batch = [&](Batch &B, int b) {
-                B.any = 0;
-#pragma unroll
-                for (int e = 0; e < BATCH; ++e) {
-                    const bool ok = b + e < cnt;
-                    const int j = ok ? b + e : 0;
-                    const int src = __builtin_amdgcn_readlane(ent.x, j);
-                    B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
-                    B.any |= B.mk[e];
-                    // lane r (< R) fetches the scratch position of this entry's r-th pair
-                    B.xp[e] = P.grp_pairs[min(__builtin_amdgcn_readlane(ent.z, j) + (lane & (R - 1)), last_pair)];
-                    load_row<T, H, D>(k + (size_t)src * L::C, lane, B.kv[e]);
-                    load_row<T, H, D>(v + (size_t)src * L::C, lane, B.vv[e]);
-                }
-            };
-            auto compute = [&](const Batch &B) {
-#pragma unroll
-                for (int m = 0; m < R; ++m) {
-                    const int bit = 1 << m;
-                    if ((B.any & bit) == 0) continue;
-#pragma unroll
-                    for (int e = 0; e < BATCH; ++e) {
-                        if (B.mk[e] & bit) {
-                            const int pos = __builtin_amdgcn_readlane(B.xp[e], __builtin_popcount(B.mk[e] & (bit - 1)));
-                            const float s = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], B.kv[e]));
-                            const float dp = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], B.vv[e]));
-                            const float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
-                            const float ds = pe * (dp - delta[m]) * scale;
-#pragma unroll
-                            for (int i = 0; i < L::EPL; ++i) dqa[m][i] = fmaf(ds, B.kv[e][i], dqa[m][i]);
-                            if (lane % L::LPH == 0) pds[(size_t)pos * H + head] = make_float2(pe, ds);
-                        }
-                    }
-                }
-            };
-            Batch A, B;
-            load_batch(A, 0);
-            for (int b = 0; b < cnt; b += 2 * BATCH) {
-                load_batch(B, b + BATCH);
-                issue_loads_first();
-                compute(A);
-                issue_loads_first();
-                load_batch(A, b + 2 * BATCH);
-                issue_loads_first();
-                compute(B);
-                issue_loads_first();
-            }
-        }
-#pragma unroll
-        for (int m = 0; m < R; ++m) {
-            if (gh.rows[m] < 0) continue;
-            if (gh.slots[m] < 0) store_row<T, H, D>(dq + (size_t)gh.rows[m] * L::C, lane, dqa[m]);
-            else store_row_ws<T, H, D>(ws_dq + (size_t)gh.slots[m] * L::C, lane, dqa[m]);
-        }
-    });
+    }
 }
 
-// Backward, source side, row groups: dK[src] = sum ds * q[dst], dV[src] = sum p * dO[dst]; the (p, ds)
-// of this plan's pair number n sits at pds[n].
-template <typename T, int H, int D, int R, int BATCH, int WPE>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_src_grp(
-    bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o, const float2 *__restrict__ pds, T *__restrict__ dk,
-    T *__restrict__ dv, float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
-    using L = Lay<T, H, D>;
-    const int lane = threadIdx.x, head = lane / L::LPH;
-    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
-    struct Batch {
-        float qr[BATCH][L::EPL], dr[BATCH][L::EPL];
-        float2 w[BATCH][R];
-        int mk[BATCH];
-    };
-    walk_groups<R>(P, [&](const GroupHead<R> &gh, const int4 &ent0) {
-        float ak[R][L::EPL], av[R][L::EPL];
-#pragma unroll
-        for (int m = 0; m < R; ++m)
-#pragma unroll
-            for (int i = 0; i < L::EPL; ++i) { ak[m][i] = 0.f; av[m][i] = 0.f; }
-        for (int p0 = gh.begin; p0 < gh.end; p0 += WAVE) {
-            const int cnt = min(WAVE, gh.end - p0);
-            int4 ent = ent0;
-            if (p0 != gh.begin) ent = lane < cnt ? entries[p0 + lane] : make_int4(0, 0, 0, 0);
-            auto load_batch = [&](Batch &B, int b) {
-#pragma unroll
-                for (int e = 0; e < BATCH; ++e) {
-                    const bool ok = b + e < cnt;
-                    const int j = ok ? b + e : 0;
-                    const int dst = __builtin_amdgcn_readlane(ent.x, j);
-                    B.mk[e] = ok ? __builtin_amdgcn_readlane(ent.y, j) : 0;
-                    const int pb = __builtin_amdgcn_readlane(ent.z, j);
-                    load_row<T, H, D>(q + (size_t)dst * L::C, lane, B.qr[e]);
-                    load_row<T, H, D>(d_o + (size_t)dst * L::C, lane, B.dr[e]);
-#pragma unroll
-                    for (int m = 0; m < R; ++m) {
-                        B.w[e][m] = make_float2(0.f, 0.f);
-                        if (B.mk[e] & (1 << m))
-                            B.w[e][m] = pds[(size_t)(pb + __builtin_popcount(B.mk[e] & ((1 << m) - 1))) * H + head];
-                    }
-                }
-            };
-            auto compute = [&](const Batch &B) {
-#pragma unroll
-                for (int e = 0; e < BATCH; ++e) {
-#pragma unroll
-                    for (int m = 0; m < R; ++m) {
-                        if (B.mk[e] & (1 << m)) {
-#pragma unroll
-                            for (int i = 0; i < L::EPL; ++i) {
-                                ak[m][i] = fmaf(B.w[e][m].y, B.qr[e][i], ak[m][i]);
-                                av[m][i] = fmaf(B.w[e][m].x, B.dr[e][i], av[m][i]);
-                            }
-                        }
-                    }
-                }
-            };
-            Batch A, B;
-            load_batch(A, 0);
-            for (int b = 0; b < cnt; b += 2 * BATCH) {
-                load_batch(B, b + BATCH);
-                issue_loads_first();
-                compute(A);
-                issue_loads_first();
-                load_batch(A, b + 2 * BATCH);
-                issue_loads_first();
-                compute(B);
-                issue_loads_first();
-            }
-        }
-#pragma unroll
-        for (int m = 0; m < R; ++m) {
-            if (gh.rows[m] < 0) continue;
-            if (gh.slots[m] < 0) {
-                store_row<T, H, D>(dk + (size_t)gh.rows[m] * L::C, lane, ak[m]);
-                store_row<T, H, D>(dv + (size_t)gh.rows[m] * L::C, lane, av[m]);
-            } else {
-                store_row_ws<T, H, D>(ws_dk + (size_t)gh.slots[m] * L::C, lane, ak[m]);
-                store_row_ws<T, H, D>(ws_dv + (size_t)gh.slots[m] * L::C, lane, av[m]);
-            }
-        }
-    });
-}
-
-// ------------------------------------------------------------------------------------------
-// team kernels of the fused path.  A team = one group of up to 16 rows (grp_R == 16) handled by a
-// workgroup of 4 wavefronts; wavefront w keeps the state of members 4w .. 4w+3 in registers.  The
-// team's neighbour rows are fetched from global memory ONCE per team: at every stage of TEAM_S = 4
-// entries wavefront w loads the two rows of entry 4*stage + w into registers (one stage ahead),
-// writes them to LDS in lane-major order (float4 slot c*64 + lane, conflict free), and after one
-// barrier every wavefront reads the rows its own members need (nibble w of the entry's 16-bit
-// mask).  LDS is double buffered, so there is one barrier per stage.  This turns the L2->L1
-// traffic of the single-wavefront row groups (each wavefront fetching its own union) into LDS reads.
-// ------------------------------------------------------------------------------------------
-constexpr int TEAM_WAVES = 4, TEAM_RW = 4, TEAM_R = TEAM_WAVES * TEAM_RW, TEAM_S = 4;
-
-// Workgroup b runs on XCD b % 8 and takes the (b / 8)-th team of that XCD's chunk (-1: none).
-__device__ __forceinline__ int team_index(const bpt_plan &P) {
-    const int x = blockIdx.x & 7, kk = blockIdx.x >> 3;
-    const int first = P.grp_chunks[x], last = P.grp_chunks[x + 1];
-    return first + kk < last ? first + kk : -1;
-}
-
+// A wavefront-private row in LDS, lane-major (float4 c of lane l at slot c * 64 + l: conflict free).
 template <int EPL> __device__ __forceinline__ void lds_put_row(float4 *slot, int lane, const float (&r)[EPL]) {
 #pragma unroll
     for (int c = 0; c < EPL / 4; ++c) slot[c * WAVE + lane] = make_float4(r[4 * c], r[4 * c + 1], r[4 * c + 2], r[4 * c + 3]);
@@ -1036,385 +775,374 @@ template <int EPL> __device__ __forceinline__ void lds_put_row(float4 *slot, int
 template <int EPL> __device__ __forceinline__ void lds_get_row(const float4 *slot, int lane, float (&r)[EPL]) {
 #pragma unroll
     for (int c = 0; c < EPL / 4; ++c) {
-        const float4 v = slot[c * WAVE + lane];
-        r[4 * c] = v.x; r[4 * c + 1] = v.y; r[4 * c + 2] = v.z; r[4 * c + 3] = v.w;
+        const float4 t = slot[c * WAVE + lane];
+        r[4 * c] = t.x; r[4 * c + 1] = t.y; r[4 * c + 2] = t.z; r[4 * c + 3] = t.w;
     }
 }
 
-// Entry descriptors of up to 128 consecutive entries, two per lane (fetched with two vector loads per
-// wavefront); field f of entry j is read with v_readlane, so no memory access sits between stages.
-struct TeamDesc {
-    int4 lo, hi;
-    __device__ __forceinline__ void fetch(const int4 *ent, int count, int lane) {
-        lo = lane < count ? ent[lane] : make_int4(0, 0, 0, 0);
-        hi = lane + WAVE < count ? ent[lane + WAVE] : make_int4(0, 0, 0, 0);
+// value of lane (4 * (lane / 4) + m) for every lane (m is a constant after unrolling)
+__device__ __forceinline__ float quad_bcast(float x, int m) {
+    switch (m & 3) {
+        case 0: return dpp_mov<0x00>(x);
+        case 1: return dpp_mov<0x55>(x);
+        case 2: return dpp_mov<0xAA>(x);
+        default: return dpp_mov<0xFF>(x);
     }
-    __device__ __forceinline__ int idx(int j) const { return j < WAVE ? __builtin_amdgcn_readlane(lo.x, j) : __builtin_amdgcn_readlane(hi.x, j - WAVE); }
-    __device__ __forceinline__ int mask(int j) const { return j < WAVE ? __builtin_amdgcn_readlane(lo.y, j) : __builtin_amdgcn_readlane(hi.y, j - WAVE); }
-    __device__ __forceinline__ int pair0(int j) const { return j < WAVE ? __builtin_amdgcn_readlane(lo.z, j) : __builtin_amdgcn_readlane(hi.z, j - WAVE); }
-};
-constexpr int TEAM_SPAN = 2 * WAVE;      // entries per descriptor fetch
+}
 
-template <typename T, int H, int D>
-__global__ __launch_bounds__(BLOCK) void k_attn_fwd_team(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k,
-                                                         const T *__restrict__ v, T *__restrict__ o, float *__restrict__ lse,
-                                                         float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+// two independent head sums, interleaved so that one hides the other's DPP wait states
+template <int LPH> __device__ __forceinline__ void head_sum2(float &a, float &b) {
+    if constexpr (LPH >= 2) { a += dpp_mov<0xB1>(a); b += dpp_mov<0xB1>(b); }
+    if constexpr (LPH >= 4) { a += dpp_mov<0x4E>(a); b += dpp_mov<0x4E>(b); }
+    if constexpr (LPH >= 8) { a += dpp_mov<0x141>(a); b += dpp_mov<0x141>(b); }
+    if constexpr (LPH >= 16) { a += dpp_mov<0x140>(a); b += dpp_mov<0x140>(b); }
+    if constexpr (LPH >= 32) { a += __shfl_xor(a, 16); b += __shfl_xor(b, 16); }
+    if constexpr (LPH >= 64) { a += __shfl_xor(a, 32); b += __shfl_xor(b, 32); }
+}
+
+// max of three finite-or-minus-infinity values (no NaN canonicalisation of the operands)
+__device__ __forceinline__ float max3f(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Forward: online softmax in base 2 over the group's entries, two entries per step.  The members' q rows
+// (pre-scaled) live in LDS and are re-read for every use, which keeps the kernel at three wavefronts per SIMD.
+template <typename T, int H, int D, int R>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H, D>::EPL, R>()))) void k_attn_fwd_grp(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
+    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
     using L = Lay<T, H, D>;
-    constexpr int S = TEAM_S, RW = TEAM_RW, F4 = L::EPL / 4;
-    __shared__ float4 lds[2][S][2][F4 * WAVE];
-    const int t = team_index(P);
-    if (t < 0) return;
-    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), head = lane / L::LPH;
-    int rows[RW], slots[RW];
+    constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
+    static_assert(R % 4 == 0 && R <= 2 * L::LPH, "members are handled in quads inside the lanes of one head");
+    GroupHead<R> gh;
+    if (!fetch_group<R>(P, gh)) return;
+    const int lane = threadIdx.x, head = lane / L::LPH;
+    const uint32_t loff = (uint32_t)(L::off(lane, 0) * sizeof(T));
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    struct Batch {
+        RawRow<T, H, D> kr[GRP_BATCH], vr[GRP_BATCH];
+        int mk[GRP_BATCH];
+    };
+    struct Rows {
+        float kv[GRP_BATCH][EPL], vv[GRP_BATCH][EPL];
+        int mk[GRP_BATCH];
+    };
+    __shared__ float4 q_lds[R * (EPL / 4) * WAVE];
+    float acc[R][EPL], mrun[R], lrun[R];
 #pragma unroll
-    for (int m = 0; m < RW; ++m) {
-        rows[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2]);
-        slots[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2 + 1]);
-    }
-    const int begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[t]);
-    const int n = __builtin_amdgcn_readfirstlane(P.grp_ptr[t + 1]) - begin;
-    const int4 *ent = reinterpret_cast<const int4 *>(P.grp_entries) + begin;
-
-    float qv[RW][L::EPL], acc[RW][L::EPL], mrun[RW], lrun[RW];
-#pragma unroll
-    for (int m = 0; m < RW; ++m) {
-        load_row<T, H, D>(q + (size_t)max(rows[m], 0) * L::C, lane, qv[m]);
+    for (int m = 0; m < R; ++m) {
+        float qr[EPL];
+        load_row32<T, H, D>(q, (uint32_t)max(gh.rows[m], 0), loff, qr);
         mrun[m] = M_INIT_LOG2;
         lrun[m] = 0.f;
 #pragma unroll
-        for (int i = 0; i < L::EPL; ++i) { qv[m][i] *= scale_log2e; acc[m][i] = 0.f; }
+        for (int i = 0; i < EPL; ++i) { qr[i] *= scale_log2e; acc[m][i] = 0.f; }
+        lds_put_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qr);
     }
-    // two stages of row loads are in flight per wavefront: register set A holds even stages, B odd ones
-    struct StageRegs { float ra[L::EPL], rb[L::EPL]; };
-    for (int c0 = 0; c0 < n; c0 += TEAM_SPAN) {
-        const int cnt = min(TEAM_SPAN, n - c0);
-        const int n_stage = (cnt + S - 1) / S;
-        TeamDesc dsc;
-        dsc.fetch(ent + c0, cnt, lane);
-        auto stage_load = [&](StageRegs &R, int st) {
-            const int j = st * S + w;
-            const int idx = j < cnt ? dsc.idx(j) : 0;
-            load_row<T, H, D>(k + (size_t)idx * L::C, lane, R.ra);
-            load_row<T, H, D>(v + (size_t)idx * L::C, lane, R.rb);
+    for (int p0 = gh.begin; p0 < gh.end; p0 += GRP_CHUNK) {
+        const int cnt = min(GRP_CHUNK, gh.end - p0);
+        // lanes past the end repeat the last entry with an empty mask
+        int4 ent = entries[p0 + min(lane, cnt - 1)];
+        ent.y = lane < cnt ? ent.y : 0;
+        auto load_batch = [&](Batch &B, int b) {
+#pragma unroll
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
+                B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
+                load_row32_raw<T, H, D>(k, src, loff, B.kr[e]);
+                load_row32_raw<T, H, D>(v, src, loff, B.vr[e]);
+            }
         };
-        auto stage_write = [&](const StageRegs &R, int buf) {
-            lds_put_row<L::EPL>(lds[buf][w][0], lane, R.ra);
-            lds_put_row<L::EPL>(lds[buf][w][1], lane, R.rb);
+        auto one = [&](int m, const float (&kr)[EPL], const float (&vr)[EPL]) {
+            float qm[EPL];
+            lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
+            const float s = head_sum<L::LPH>(dot_n<EPL>(qm, kr));
+            const float mx = fmaxf(mrun[m], s);
+            const float al = __builtin_amdgcn_exp2f(mrun[m] - mx), pe = __builtin_amdgcn_exp2f(s - mx);
+            lrun[m] = fmaf(lrun[m], al, pe);
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) acc[m][i] = fmaf(pe, vr[i], acc[m][i] * al);
+            mrun[m] = mx;
         };
-        auto stage_compute = [&](int st, int buf) {
-            int mk[S], any = 0;
+        auto compute = [&](const Batch &raw) {
+            Rows B;
 #pragma unroll
-            for (int e = 0; e < S; ++e) {
-                const int j = st * S + e;
-                mk[e] = j < cnt ? (dsc.mask(j) >> (w * RW)) & ((1 << RW) - 1) : 0;
-                any |= mk[e];
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                unpack_row<T, H, D>(raw.kr[e], B.kv[e]);
+                unpack_row<T, H, D>(raw.vr[e], B.vv[e]);
+                B.mk[e] = raw.mk[e];
             }
-            if (any == 0) return;
-            float sc[RW][S];
-            // K phase: scores of this stage
 #pragma unroll
-            for (int e = 0; e < S; ++e) {
-                if (mk[e] == 0) continue;
-                float kr[L::EPL];
-                lds_get_row<L::EPL>(lds[buf][e][0], lane, kr);
+            for (int m = 0; m < R; ++m) {
+                const bool h0 = (B.mk[0] >> m) & 1, h1 = (B.mk[GRP_BATCH - 1] >> m) & 1;
+                if constexpr (GRP_BATCH == 1) {
+                    if (h0) one(m, B.kv[0], B.vv[0]);
+                } else if (h0 && h1) {
+                    float qm[EPL];
+                    lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
+                    float s0 = dot_n<EPL>(qm, B.kv[0]), s1 = dot_n<EPL>(qm, B.kv[GRP_BATCH - 1]);
+                    head_sum2<L::LPH>(s0, s1);
+                    const float mx = max3f(mrun[m], s0, s1);
+                    const float al = __builtin_amdgcn_exp2f(mrun[m] - mx);
+                    const float p0e = __builtin_amdgcn_exp2f(s0 - mx), p1e = __builtin_amdgcn_exp2f(s1 - mx);
+                    lrun[m] = fmaf(lrun[m], al, p0e + p1e);
 #pragma unroll
-                for (int m = 0; m < RW; ++m)
-                    if (mk[e] & (1 << m)) sc[m][e] = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], kr));
-            }
-            // one running-maximum update (and accumulator rescale) per member and stage
-#pragma unroll
-            for (int m = 0; m < RW; ++m) {
-                if ((any & (1 << m)) == 0) continue;
-                float mx = mrun[m];
-#pragma unroll
-                for (int e = 0; e < S; ++e)
-                    if (mk[e] & (1 << m)) mx = fmaxf(mx, sc[m][e]);
-                const float alpha = __builtin_amdgcn_exp2f(mrun[m] - mx);
-                lrun[m] *= alpha;
-#pragma unroll
-                for (int i = 0; i < L::EPL; ++i) acc[m][i] *= alpha;
-                mrun[m] = mx;
-            }
-            // V phase
-#pragma unroll
-            for (int e = 0; e < S; ++e) {
-                if (mk[e] == 0) continue;
-                float vr[L::EPL];
-                lds_get_row<L::EPL>(lds[buf][e][1], lane, vr);
-#pragma unroll
-                for (int m = 0; m < RW; ++m) {
-                    if (mk[e] & (1 << m)) {
-                        const float pe = __builtin_amdgcn_exp2f(sc[m][e] - mrun[m]);
-                        lrun[m] += pe;
-#pragma unroll
-                        for (int i = 0; i < L::EPL; ++i) acc[m][i] = fmaf(pe, vr[i], acc[m][i]);
-                    }
+                    for (int i = 0; i < EPL; ++i) acc[m][i] = fmaf(p1e, B.vv[GRP_BATCH - 1][i], fmaf(p0e, B.vv[0][i], acc[m][i] * al));
+                    mrun[m] = mx;
+                } else if (h0) {
+                    one(m, B.kv[0], B.vv[0]);
+                } else if (h1) {
+                    one(m, B.kv[GRP_BATCH - 1], B.vv[GRP_BATCH - 1]);
                 }
             }
         };
-        StageRegs A, B;
-        stage_load(A, 0);
-        stage_load(B, 1);
-        stage_write(A, 0);
-        stage_load(A, 2);
-        __syncthreads();
-        for (int st = 0; st < n_stage; st += 2) {
-            stage_compute(st, 0);
+        // two-stage software pipeline: the rows of the next batch are in flight while one is used.  The loads
+        // are unconditional (a branch around them would make the compiler drain the load queue at the join);
+        // look-ahead past the end re-reads the chunk's last entry with an empty mask.
+        Batch A, B;
+        load_batch(A, 0);
+        for (int b = 0; b < cnt; b += 2 * GRP_BATCH) {
+            load_batch(B, b + GRP_BATCH);
             issue_loads_first();
-            stage_write(B, 1);         // B holds stage st + 1
-            stage_load(B, st + 3);
-            __syncthreads();
-            stage_compute(st + 1, 1);  // masks are empty past the last stage
+            compute(A);
             issue_loads_first();
-            stage_write(A, 0);         // A holds stage st + 2
-            stage_load(A, st + 4);
-            __syncthreads();
+            load_batch(A, b + 2 * GRP_BATCH);
+            issue_loads_first();
+            compute(B);
+            issue_loads_first();
         }
     }
 #pragma unroll
-    for (int m = 0; m < RW; ++m) {
-        if (rows[m] < 0) continue;
-        if (slots[m] < 0) {
+    for (int m = 0; m < R; ++m) {
+        if (gh.rows[m] < 0) continue;
+        if (gh.slots[m] < 0) {
             const float inv = lrun[m] > 0.f ? 1.f / lrun[m] : 0.f;
 #pragma unroll
-            for (int i = 0; i < L::EPL; ++i) acc[m][i] *= inv;
-            store_row<T, H, D>(o + (size_t)rows[m] * L::C, lane, acc[m]);
-            if (lane % L::LPH == 0) lse[(size_t)rows[m] * H + head] = lrun[m] > 0.f ? mrun[m] + log2f(lrun[m]) : 0.f;
+            for (int i = 0; i < EPL; ++i) acc[m][i] *= inv;
+            store_row<T, H, D>(o + (size_t)gh.rows[m] * L::C, lane, acc[m]);
+            if (lane % L::LPH == 0) lse[(size_t)gh.rows[m] * H + head] = lrun[m] > 0.f ? mrun[m] + log2f(lrun[m]) : 0.f;
         } else {
-            store_row_ws<T, H, D>(ws_acc + (size_t)slots[m] * L::C, lane, acc[m]);
+            store_row_ws<T, H, D>(ws_acc + (size_t)gh.slots[m] * L::C, lane, acc[m]);
             if (lane % L::LPH == 0) {
-                ws_ml[((size_t)slots[m] * H + head) * 2] = mrun[m];
-                ws_ml[((size_t)slots[m] * H + head) * 2 + 1] = lrun[m];
+                ws_ml[((size_t)gh.slots[m] * H + head) * 2] = mrun[m];
+                ws_ml[((size_t)gh.slots[m] * H + head) * 2 + 1] = lrun[m];
             }
         }
     }
 }
 
-// Backward, destination side, teams.  pds[(pair, head)] = (p, ds) in the pair order of the source-side plan.
-template <typename T, int H, int D>
-__global__ __launch_bounds__(BLOCK) void k_attn_bwd_dst_team(bpt_plan P, const T *__restrict__ q, const T *__restrict__ k,
-                                                             const T *__restrict__ v, const T *__restrict__ o, const T *__restrict__ d_o,
-                                                             const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
-                                                             float *__restrict__ ws_dq, float scale, float scale_log2e) {
+// Backward, destination side.  Writes (p, ds) of every pair to pds[(t * H + head)], t = the pair's
+// position (entry * R + member) in the SOURCE-side plan, which P.grp_pairs gives for every
+// (entry, member) of this plan (a spare position for members the entry does not have).  One store per
+// entry and quad of members: lane l carries the pair of member 4c + l % 4.  The members' q rows live in LDS.
+template <typename T, int H, int D, int R>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H, D>::EPL, R>()))) void k_attn_bwd_dst_grp(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
+    const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
+    float *__restrict__ ws_dq, float scale, float scale_log2e) {
     using L = Lay<T, H, D>;
-    constexpr int S = TEAM_S, RW = TEAM_RW, F4 = L::EPL / 4;
-    static_assert(S * TEAM_R == WAVE, "one lane per (entry of the stage, pair of the entry)");
-    __shared__ float4 lds[2][S][2][F4 * WAVE];
-    const int t = team_index(P);
-    if (t < 0) return;
-    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), head = lane / L::LPH;
-    int rows[RW], slots[RW];
+    constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
+    static_assert(R % 4 == 0 && R <= 2 * L::LPH, "members are handled in quads inside the lanes of one head");
+    GroupHead<R> gh;
+    if (!fetch_group<R>(P, gh)) return;
+    const int lane = threadIdx.x, head = lane / L::LPH;
+    const uint32_t loff = (uint32_t)(L::off(lane, 0) * sizeof(T));
+    const int mine = lane & 3;
+    const uint32_t hoff = (uint32_t)head * 8u, poff = (uint32_t)mine * 4u;
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    struct Batch {
+        RawRow<T, H, D> kr[GRP_BATCH], vr[GRP_BATCH];
+        int mk[GRP_BATCH], xp[GRP_BATCH][NQ];
+    };
+    __shared__ float4 q_lds[R * (EPL / 4) * WAVE];
+    float dov[R][EPL], dqa[R][EPL], delta_s[R], lse2[R];
 #pragma unroll
-    for (int m = 0; m < RW; ++m) {
-        rows[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2]);
-        slots[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2 + 1]);
+    for (int m = 0; m < R; ++m) {
+        const uint32_t row = (uint32_t)max(gh.rows[m], 0);
+        float ov[EPL], qr[EPL];
+        load_row32<T, H, D>(o, row, loff, ov);
+        load_row32<T, H, D>(d_o, row, loff, dov[m]);
+        load_row32<T, H, D>(q, row, loff, qr);
+        lds_put_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qr);
+        delta_s[m] = head_sum<L::LPH>(dot_n<EPL>(dov[m], ov)) * scale;
+        lse2[m] = lse[(size_t)row * H + head];
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) dqa[m][i] = 0.f;
     }
-    const int begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[t]);
-    const int n = __builtin_amdgcn_readfirstlane(P.grp_ptr[t + 1]) - begin;
-    const int4 *ent = reinterpret_cast<const int4 *>(P.grp_entries) + begin;
-    const int last_pair = (int)P.n_edges - 1;
-
-    float qv[RW][L::EPL], dov[RW][L::EPL], dqa[RW][L::EPL], delta[RW], lse2[RW];
+    for (int p0 = gh.begin; p0 < gh.end; p0 += GRP_CHUNK) {
+        const int cnt = min(GRP_CHUNK, gh.end - p0);
+        // lanes past the end repeat the last entry with an empty mask
+        int4 ent = entries[p0 + min(lane, cnt - 1)];
+        ent.y = lane < cnt ? ent.y : 0;
+        auto load_batch = [&](Batch &B, int b) {
 #pragma unroll
-    for (int m = 0; m < RW; ++m) {
-        const size_t row = (size_t)max(rows[m], 0);
-        float ov[L::EPL];
-        load_row<T, H, D>(o + row * L::C, lane, ov);
-        load_row<T, H, D>(d_o + row * L::C, lane, dov[m]);
-        load_row<T, H, D>(q + row * L::C, lane, qv[m]);
-        delta[m] = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], ov));
-        lse2[m] = lse[row * H + head];
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
+                B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
+                // lane l fetches the scratch positions of the pairs of members l % 4, 4 + l % 4, ... with this entry
+                const char *pp = reinterpret_cast<const char *>(P.grp_pairs) + (size_t)((uint32_t)(p0 + b + e) * (uint32_t)(R * 4));
 #pragma unroll
-        for (int i = 0; i < L::EPL; ++i) dqa[m][i] = 0.f;
-    }
-    // xp: lane e*16 + r holds the scratch position of pair r of entry e of the stage
-    struct StageRegs { float ra[L::EPL], rb[L::EPL]; int xp; };
-    for (int c0 = 0; c0 < n; c0 += TEAM_SPAN) {
-        const int cnt = min(TEAM_SPAN, n - c0);
-        const int n_stage = (cnt + S - 1) / S;
-        TeamDesc dsc;
-        dsc.fetch(ent + c0, cnt, lane);
-        auto stage_load = [&](StageRegs &R, int st) {
-            const int j = st * S + w;
-            const int idx = j < cnt ? dsc.idx(j) : 0;
-            // first pair of entry st*S + lane/16, fetched from the lane that holds that descriptor
-            const int je = min(st * S + (lane >> 4), cnt - 1);
-            const int pb = je < WAVE ? __shfl(dsc.lo.z, je) : __shfl(dsc.hi.z, je - WAVE);
-            R.xp = P.grp_pairs[min(pb + (lane & 15), last_pair)];
-            load_row<T, H, D>(k + (size_t)idx * L::C, lane, R.ra);
-            load_row<T, H, D>(v + (size_t)idx * L::C, lane, R.rb);
+                for (int c = 0; c < NQ; ++c) B.xp[e][c] = *reinterpret_cast<const int *>(pp + (size_t)(poff + (uint32_t)(c * 16)));
+                load_row32_raw<T, H, D>(k, src, loff, B.kr[e]);
+                load_row32_raw<T, H, D>(v, src, loff, B.vr[e]);
+            }
         };
-        auto stage_write = [&](const StageRegs &R, int buf) {
-            lds_put_row<L::EPL>(lds[buf][w][0], lane, R.ra);
-            lds_put_row<L::EPL>(lds[buf][w][1], lane, R.rb);
-        };
-        auto stage_compute = [&](int st, int buf, int xp) {
+        auto compute = [&](const Batch &B) {
 #pragma unroll
-            for (int e = 0; e < S; ++e) {
-                const int j = st * S + e;
-                const int mask16 = j < cnt ? dsc.mask(j) : 0;
-                const int mk = (mask16 >> (w * RW)) & ((1 << RW) - 1);
-                if (mk == 0) continue;
-                float kr[L::EPL], vr[L::EPL];
-                lds_get_row<L::EPL>(lds[buf][e][0], lane, kr);
-                lds_get_row<L::EPL>(lds[buf][e][1], lane, vr);
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                float kv[EPL], vv[EPL];
+                unpack_row<T, H, D>(B.kr[e], kv);
+                unpack_row<T, H, D>(B.vr[e], vv);
+                float wp[NQ], wd[NQ];
 #pragma unroll
-                for (int m = 0; m < RW; ++m) {
-                    if (mk & (1 << m)) {
-                        const int rank = __builtin_popcount(mask16 & ((1 << (w * RW + m)) - 1));
-                        const unsigned pos = (unsigned)__builtin_amdgcn_readlane(xp, e * TEAM_R + rank);
-                        const float sdot = head_sum<L::LPH>(dot_n<L::EPL>(qv[m], kr));
-                        const float dp = head_sum<L::LPH>(dot_n<L::EPL>(dov[m], vr));
-                        const float pe = __builtin_amdgcn_exp2f(fmaf(sdot, scale_log2e, -lse2[m]));
-                        const float ds = pe * (dp - delta[m]) * scale;
+                for (int c = 0; c < NQ; ++c) { wp[c] = 0.f; wd[c] = 0.f; }
 #pragma unroll
-                        for (int i = 0; i < L::EPL; ++i) dqa[m][i] = fmaf(ds, kr[i], dqa[m][i]);
-                        pds[(size_t)pos * H + head] = make_float2(pe, ds);     // all lanes of a head write the same value
+                for (int m = 0; m < R; ++m) {
+                    if ((B.mk[e] >> m) & 1) {
+                        float qm[EPL];
+                        lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
+                        float s = dot_n<EPL>(qm, kv), dp = dot_n<EPL>(dov[m], vv);
+                        head_sum2<L::LPH>(s, dp);
+                        const float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
+                        const float ds = pe * fmaf(dp, scale, -delta_s[m]);
+#pragma unroll
+                        for (int i = 0; i < EPL; ++i) dqa[m][i] = fmaf(ds, kv[i], dqa[m][i]);
+                        wp[m / 4] = mine == (m & 3) ? pe : wp[m / 4];
+                        wd[m / 4] = mine == (m & 3) ? ds : wd[m / 4];
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < NQ; ++c) {
+                    if ((B.mk[e] >> (4 * c)) & 15) {      // (look-ahead batches past the group's end have empty masks)
+                        char *w = reinterpret_cast<char *>(pds);
+                        *reinterpret_cast<float2 *>(w + (size_t)((uint32_t)B.xp[e][c] * (uint32_t)(H * 8) + hoff)) = make_float2(wp[c], wd[c]);
                     }
                 }
             }
         };
-        StageRegs A, B;
-        stage_load(A, 0);
-        stage_load(B, 1);
-        stage_write(A, 0);
-        int xp_even = A.xp, xp_odd = B.xp;
-        stage_load(A, 2);
-        __syncthreads();
-        for (int st = 0; st < n_stage; st += 2) {
-            stage_compute(st, 0, xp_even);
+        // two-stage software pipeline: the rows of the next batch are in flight while one is used.  The loads
+        // are unconditional (a branch around them would make the compiler drain the load queue at the join);
+        // look-ahead past the end re-reads the chunk's last entry with an empty mask.
+        Batch A, B;
+        load_batch(A, 0);
+        for (int b = 0; b < cnt; b += 2 * GRP_BATCH) {
+            load_batch(B, b + GRP_BATCH);
             issue_loads_first();
-            stage_write(B, 1);         // B holds stage st + 1
-            xp_odd = B.xp;
-            stage_load(B, st + 3);
-            __syncthreads();
-            stage_compute(st + 1, 1, xp_odd);
+            compute(A);
             issue_loads_first();
-            stage_write(A, 0);         // A holds stage st + 2
-            xp_even = A.xp;
-            stage_load(A, st + 4);
-            __syncthreads();
+            load_batch(A, b + 2 * GRP_BATCH);
+            issue_loads_first();
+            compute(B);
+            issue_loads_first();
         }
     }
 #pragma unroll
-    for (int m = 0; m < RW; ++m) {
-        if (rows[m] < 0) continue;
-        if (slots[m] < 0) store_row<T, H, D>(dq + (size_t)rows[m] * L::C, lane, dqa[m]);
-        else store_row_ws<T, H, D>(ws_dq + (size_t)slots[m] * L::C, lane, dqa[m]);
+    for (int m = 0; m < R; ++m) {
+        if (gh.rows[m] < 0) continue;
+        if (gh.slots[m] < 0) store_row<T, H, D>(dq + (size_t)gh.rows[m] * L::C, lane, dqa[m]);
+        else store_row_ws<T, H, D>(ws_dq + (size_t)gh.slots[m] * L::C, lane, dqa[m]);
     }
 }
 
-// Backward, source side, teams: dK[src] = sum ds * q[dst], dV[src] = sum p * dO[dst].  The (p, ds) of
-// this plan's pairs are contiguous per stage; the workgroup copies them to LDS with one 16-byte
-// load per thread.
-template <typename T, int H, int D>
-__global__ __launch_bounds__(BLOCK) void k_attn_bwd_src_team(bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o,
-                                                             const float2 *__restrict__ pds, T *__restrict__ dk, T *__restrict__ dv,
-                                                             float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
+// Backward, source side: dK[src] = sum ds * q[dst], dV[src] = sum p * dO[dst]; the (p, ds) of the pair
+// (entry u, member m) of this plan sits at pds[(u * R + m) * H + head].  One load per entry and quad of
+// members: lane l fetches the pair of member 4c + l % 4 for its head.  That is the A operand of
+// v_mfma_f32_4x4x1 (16 blocks of 4 lanes: A_b[i] in lane 4b+i, B_b[j] in lane 4b+j, D_b[i][j] in register i
+// of lane 4b+j): with a register of the entry's row as B, one instruction adds weight[member i] * row[..]
+// to that register's slice of all four members' accumulators (register i of the result = member i).
+template <typename T, int H, int D, int R>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H, D>::EPL, R>()))) void k_attn_bwd_src_grp(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o, const float2 *__restrict__ pds, T *__restrict__ dk,
+    T *__restrict__ dv, float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
     using L = Lay<T, H, D>;
-    constexpr int S = TEAM_S, RW = TEAM_RW, F4 = L::EPL / 4;
-    constexpr int WF4 = S * TEAM_R * H / 2;                 // float4 per stage of weights (at most S*16 pairs)
-    constexpr int WPT = (WF4 + BLOCK - 1) / BLOCK;          // float4 per thread
-    __shared__ float4 lds[2][S][2][F4 * WAVE];
-    __shared__ float4 wts[2][WPT * BLOCK];
-    const int t = team_index(P);
-    if (t < 0) return;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), head = lane / L::LPH;
-    int rows[RW], slots[RW];
+    constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
+    static_assert(R % 4 == 0 && R <= 2 * L::LPH, "members are handled in quads inside the lanes of one head");
+    GroupHead<R> gh;
+    if (!fetch_group<R>(P, gh)) return;
+    const int lane = threadIdx.x, head = lane / L::LPH;
+    const uint32_t loff = (uint32_t)(L::off(lane, 0) * sizeof(T));
+    const uint32_t woff = (uint32_t)(((lane & 3) * H + head) * 8);
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    struct Batch {
+        RawRow<T, H, D> qr[GRP_BATCH], dr[GRP_BATCH];
+        float2 w[GRP_BATCH][NQ];
+        int mk[GRP_BATCH];
+    };
+    floatx4 ak[NQ][EPL], av[NQ][EPL];          // [quad c][row register t][member 4c + i]
 #pragma unroll
-    for (int m = 0; m < RW; ++m) {
-        rows[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2]);
-        slots[m] = __builtin_amdgcn_readfirstlane(P.grp_members[((size_t)t * TEAM_R + w * RW + m) * 2 + 1]);
-    }
-    const int begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[t]);
-    const int n = __builtin_amdgcn_readfirstlane(P.grp_ptr[t + 1]) - begin;
-    const int4 *ent = reinterpret_cast<const int4 *>(P.grp_entries) + begin;
-    const float4 *pds4 = reinterpret_cast<const float4 *>(pds);
-    const int n_f4 = (int)(P.n_edges * H / 2);              // float4 in the whole scratch
-
-    float ak[RW][L::EPL], av[RW][L::EPL];
+    for (int c = 0; c < NQ; ++c)
 #pragma unroll
-    for (int m = 0; m < RW; ++m)
+        for (int t = 0; t < EPL; ++t) { ak[c][t] = floatx4{0.f, 0.f, 0.f, 0.f}; av[c][t] = floatx4{0.f, 0.f, 0.f, 0.f}; }
+    for (int p0 = gh.begin; p0 < gh.end; p0 += GRP_CHUNK) {
+        const int cnt = min(GRP_CHUNK, gh.end - p0);
+        // lanes past the end repeat the last entry with an empty mask
+        int4 ent = entries[p0 + min(lane, cnt - 1)];
+        ent.y = lane < cnt ? ent.y : 0;
+        auto load_batch = [&](Batch &B, int b) {
 #pragma unroll
-        for (int i = 0; i < L::EPL; ++i) { ak[m][i] = 0.f; av[m][i] = 0.f; }
-    struct StageRegs { float ra[L::EPL], rb[L::EPL]; float4 wreg[WPT]; };
-    for (int c0 = 0; c0 < n; c0 += TEAM_SPAN) {
-        const int cnt = min(TEAM_SPAN, n - c0);
-        const int n_stage = (cnt + S - 1) / S;
-        TeamDesc dsc;
-        dsc.fetch(ent + c0, cnt, lane);
-        auto stage_load = [&](StageRegs &R, int st) {
-            const int j = st * S + w;
-            const int idx = j < cnt ? dsc.idx(j) : 0;
-            const int pb0 = dsc.pair0(min(st * S, cnt - 1));                     // first pair of the stage
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                const uint32_t dst = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
+                B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
+                load_row32_raw<T, H, D>(q, dst, loff, B.qr[e]);
+                load_row32_raw<T, H, D>(d_o, dst, loff, B.dr[e]);
+                // the entry's R pairs, present or not (absent ones are zeroed before use)
+                const char *pw = reinterpret_cast<const char *>(pds) + (size_t)((uint32_t)(p0 + b + e) * (uint32_t)(R * H * 8));
 #pragma unroll
-            for (int u = 0; u < WPT; ++u) R.wreg[u] = pds4[min(pb0 * (H / 2) + u * BLOCK + tid, n_f4 - 1)];
-            load_row<T, H, D>(q + (size_t)idx * L::C, lane, R.ra);
-            load_row<T, H, D>(d_o + (size_t)idx * L::C, lane, R.rb);
+                for (int c = 0; c < NQ; ++c) B.w[e][c] = *reinterpret_cast<const float2 *>(pw + (size_t)(woff + (uint32_t)(c * 4 * H * 8)));
+            }
         };
-        auto stage_write = [&](const StageRegs &R, int buf) {
-            lds_put_row<L::EPL>(lds[buf][w][0], lane, R.ra);
-            lds_put_row<L::EPL>(lds[buf][w][1], lane, R.rb);
+        auto compute = [&](const Batch &B) {
 #pragma unroll
-            for (int u = 0; u < WPT; ++u) wts[buf][u * BLOCK + tid] = R.wreg[u];
-        };
-        auto stage_compute = [&](int st, int buf) {
-            if (st >= n_stage) return;
-            const float2 *wbuf = reinterpret_cast<const float2 *>(wts[buf]);
-            const int pb0 = dsc.pair0(st * S);
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                float qv[EPL], dv_[EPL];
+                unpack_row<T, H, D>(B.qr[e], qv);
+                unpack_row<T, H, D>(B.dr[e], dv_);
 #pragma unroll
-            for (int e = 0; e < S; ++e) {
-                const int j = st * S + e;
-                const int mask16 = j < cnt ? dsc.mask(j) : 0;
-                const int mk = (mask16 >> (w * RW)) & ((1 << RW) - 1);
-                if (mk == 0) continue;
-                const int pbe = dsc.pair0(j) - pb0;       // first pair of the entry, relative to the stage
-                float qr[L::EPL], dr[L::EPL];
-                lds_get_row<L::EPL>(lds[buf][e][0], lane, qr);
-                lds_get_row<L::EPL>(lds[buf][e][1], lane, dr);
+                for (int c = 0; c < NQ; ++c) {
+                    if ((B.mk[e] >> (4 * c)) & 15) {
+                        // all-ones where this lane's member has the edge: the scratch of absent pairs is not initialised
+                        const int keep = __builtin_amdgcn_sbfe(B.mk[e], 4 * c + (lane & 3), 1);
+                        const float pe = __int_as_float(__float_as_int(B.w[e][c].x) & keep);
+                        const float ds = __int_as_float(__float_as_int(B.w[e][c].y) & keep);
 #pragma unroll
-                for (int m = 0; m < RW; ++m) {
-                    if (mk & (1 << m)) {
-                        const int lp = pbe + __builtin_popcount(mask16 & ((1 << (w * RW + m)) - 1));
-                        const float2 wgt = wbuf[lp * H + head];
-#pragma unroll
-                        for (int i = 0; i < L::EPL; ++i) {
-                            ak[m][i] = fmaf(wgt.y, qr[i], ak[m][i]);
-                            av[m][i] = fmaf(wgt.x, dr[i], av[m][i]);
+                        for (int t = 0; t < EPL; ++t) {
+                            ak[c][t] = __builtin_amdgcn_mfma_f32_4x4x1f32(ds, qv[t], ak[c][t], 0, 0, 0);
+                            av[c][t] = __builtin_amdgcn_mfma_f32_4x4x1f32(pe, dv_[t], av[c][t], 0, 0, 0);
                         }
                     }
                 }
             }
         };
-        StageRegs A, B;
-        stage_load(A, 0);
-        stage_load(B, 1);
-        stage_write(A, 0);
-        stage_load(A, 2);
-        __syncthreads();
-        for (int st = 0; st < n_stage; st += 2) {
-            stage_compute(st, 0);
+        // two-stage software pipeline: the rows of the next batch are in flight while one is used.  The loads
+        // are unconditional (a branch around them would make the compiler drain the load queue at the join);
+        // look-ahead past the end re-reads the chunk's last entry with an empty mask.
+        Batch A, B;
+        load_batch(A, 0);
+        for (int b = 0; b < cnt; b += 2 * GRP_BATCH) {
+            load_batch(B, b + GRP_BATCH);
             issue_loads_first();
-            stage_write(B, 1);         // B holds stage st + 1
-            stage_load(B, st + 3);
-            __syncthreads();
-            stage_compute(st + 1, 1);
+            compute(A);
             issue_loads_first();
-            stage_write(A, 0);         // A holds stage st + 2
-            stage_load(A, st + 4);
-            __syncthreads();
+            load_batch(A, b + 2 * GRP_BATCH);
+            issue_loads_first();
+            compute(B);
+            issue_loads_first();
         }
     }
 #pragma unroll
-    for (int m = 0; m < RW; ++m) {
-        if (rows[m] < 0) continue;
-        if (slots[m] < 0) {
-            store_row<T, H, D>(dk + (size_t)rows[m] * L::C, lane, ak[m]);
-            store_row<T, H, D>(dv + (size_t)rows[m] * L::C, lane, av[m]);
+    for (int m = 0; m < R; ++m) {
+        if (gh.rows[m] < 0) continue;
+        float rk[EPL], rv[EPL];
+#pragma unroll
+        for (int t = 0; t < EPL; ++t) { rk[t] = ak[m / 4][t][m & 3]; rv[t] = av[m / 4][t][m & 3]; }
+        if (gh.slots[m] < 0) {
+            store_row<T, H, D>(dk + (size_t)gh.rows[m] * L::C, lane, rk);
+            store_row<T, H, D>(dv + (size_t)gh.rows[m] * L::C, lane, rv);
         } else {
-            store_row_ws<T, H, D>(ws_dk + (size_t)slots[m] * L::C, lane, ak[m]);
-            store_row_ws<T, H, D>(ws_dv + (size_t)slots[m] * L::C, lane, av[m]);
+            store_row_ws<T, H, D>(ws_dk + (size_t)gh.slots[m] * L::C, lane, rk);
+            store_row_ws<T, H, D>(ws_dv + (size_t)gh.slots[m] * L::C, lane, rv);
         }
     }
 }
@@ -1431,7 +1159,7 @@ inline int check_plan(const bpt_plan *p, bool need_idx) {
     if (p->n_edges > 0 && (!p->eid || (need_idx && !p->idx))) return BPT_ERR_NULL;
     if (p->n_heavy > 0 && !p->heavy) return BPT_ERR_NULL;
     if (p->n_items < p->n_rows) return BPT_ERR_SIZE;     // every row owns at least one item
-    if (p->n_groups < 0 || p->grp_R < 0 || p->grp_R > 16) return BPT_ERR_SIZE;
+    if (p->n_groups < 0 || p->grp_R < 0 || p->grp_R > 16 || p->n_grp_entries < 0) return BPT_ERR_SIZE;
     if (p->n_groups > 0 && (!p->grp_members || !p->grp_ptr || !p->grp_chunks || (p->n_edges > 0 && !p->grp_entries))) return BPT_ERR_NULL;
     if (p->n_groups > 0 && (p->grp_max_chunk < 1 || p->grp_max_chunk > p->n_groups)) return BPT_ERR_SIZE;
     return BPT_OK;
@@ -1587,22 +1315,31 @@ int spmm(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int
 
 inline int64_t round16(int64_t b) { return (b + 15) & ~(int64_t)15; }
 
-constexpr int GROUP_R = 4;
+// The row-group kernels address node rows and the per-pair scratch with 32-bit byte offsets.
+inline bool fits32(int64_t n, int64_t unit) { return n >= 0 && n <= (int64_t)0xffffffffu / unit; }
 
-inline int group_grid(const bpt_plan *P, int kernel) {
-    const int64_t per_xcd = g_group_waves[kernel].load(std::memory_order_relaxed);
-    const int64_t n = (per_xcd > 0 && per_xcd < P->grp_max_chunk) ? per_xcd : P->grp_max_chunk;
-    return (int)(8 * n);
+inline int group_grid(const bpt_plan *P) { return (int)(8 * P->grp_max_chunk); }
+
+// rows per group the row-group kernels exist for, given the elements a lane holds per row
+inline bool group_rows_ok(int64_t R, int h, int d) { return R == 4 || (R == 8 && h <= 8 && h * d <= 512); }
+
+inline bool has_groups(const bpt_plan *P, int h, int d, size_t elem) {
+    return P->n_groups > 0 && group_rows_ok(P->grp_R, h, d) && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
+           P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups && P->n_grp_entries >= 0 &&
+           fits32(P->n_rows, (int64_t)h * d * (int64_t)elem) &&
+           fits32((P->n_grp_entries + GRP_PAD_ENTRIES) * P->grp_R, (int64_t)h * 8);
 }
 
-inline bool has_teams(const bpt_plan *P) {
-    return P->n_groups > 0 && P->grp_R == TEAM_R && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
-           P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups;
+inline bool grouped_backward(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {
+    return has_groups(Pin, h, d, elem) && has_groups(Pout, h, d, elem) && Pin->grp_R == Pout->grp_R && Pin->grp_pairs;
 }
 
-inline bool has_groups(const bpt_plan *P) {
-    return P->n_groups > 0 && P->grp_R == GROUP_R && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
-           P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups;
+// float2 (p, ds) scratch of the fused backward: one per (entry, member) of the source-side groups (plus the
+// look-ahead padding), or one per edge for the per-row kernels
+inline int64_t pds_bytes(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {
+    int64_t n = Pin->n_edges;
+    if (Pout && grouped_backward(Pin, Pout, h, d, elem)) n = std::max(n, (Pout->n_grp_entries + GRP_PAD_ENTRIES) * Pout->grp_R);
+    return 2 * round16(n * h * 4);
 }
 
 template <typename T, int H, int D>
@@ -1612,18 +1349,17 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
-        if (has_teams(P)) {
-            hipLaunchKernelGGL((k_attn_fwd_team<T, H, D>), dim3((int)(8 * P->grp_max_chunk)), dim3(BLOCK), 0, s, *P, (const T *)q,
-                               (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
-        } else if (has_groups(P)) {
-#define LAUNCH_FWD_GRP(B, W)                                                                                                   \
-    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, GROUP_R, B, W>), dim3(group_grid(P, 0)), dim3(WAVE), 0, s, *P, (const T *)q,   \
+        if (has_groups(P, H, D, sizeof(T))) {
+#define LAUNCH_FWD(RR)                                                                                              \
+    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR>), dim3(group_grid(P)), dim3(WAVE), 0, s, *P, (const T *)q, \
                        (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E)
-            const int var = g_group_variant[0].load(std::memory_order_relaxed);
-            if (var == 4) LAUNCH_FWD_GRP(4, 1);
-            else if (var == 3) LAUNCH_FWD_GRP(2, 3);
-            else LAUNCH_FWD_GRP(2, 1);
-#undef LAUNCH_FWD_GRP
+            if constexpr (H <= 8 && H * D <= 512) {
+                if (P->grp_R == 8) LAUNCH_FWD(8);
+                else LAUNCH_FWD(4);
+            } else {
+                LAUNCH_FWD(4);
+            }
+#undef LAUNCH_FWD
         } else {
             hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
                                (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
@@ -1637,98 +1373,33 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
 }
 
 template <typename T, int H, int D>
-int run_attn_bwd_grouped(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
-                         const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
-    const size_t EH = (size_t)Pin->n_edges * H;
-    float2 *pds = (float2 *)ws;
-    float *ws_rows = (float *)ws + 2 * (round16((int64_t)EH * 4) / 4);
-    {
-        ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
-#define LAUNCH_DST_GRP(B, W)                                                                                                       \
-    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, GROUP_R, B, W>), dim3(group_grid(Pin, 1)), dim3(WAVE), 0, s, *Pin, (const T *)q, \
-                       (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E)
-        const int var = g_group_variant[1].load(std::memory_order_relaxed);
-        if (var == 4) LAUNCH_DST_GRP(4, 1);
-        else if (var == 3) LAUNCH_DST_GRP(2, 3);
-        else LAUNCH_DST_GRP(2, 1);
-#undef LAUNCH_DST_GRP
-    }
-    int st = launch_status();
-    if (st != BPT_OK) return st;
-    if (Pin->n_heavy > 0) {
-        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, Pin->heavy,
-                           (const float *)ws_rows, (T *)dq, (T *)nullptr, H * D, (size_t)0);
-        st = launch_status();
-        if (st != BPT_OK) return st;
-    }
-    float *ws_dk = ws_rows, *ws_dv = ws_rows + (size_t)Pout->n_slots * H * D;
-    {
-        ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
-#define LAUNCH_SRC_GRP(B, W)                                                                                                          \
-    hipLaunchKernelGGL((k_attn_bwd_src_grp<T, H, D, GROUP_R, B, W>), dim3(group_grid(Pout, 2)), dim3(WAVE), 0, s, *Pout, (const T *)q, \
-                       (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv)
-        const int var = g_group_variant[2].load(std::memory_order_relaxed);
-        if (var == 4) LAUNCH_SRC_GRP(4, 1);
-        else if (var == 3) LAUNCH_SRC_GRP(2, 3);
-        else LAUNCH_SRC_GRP(2, 1);
-#undef LAUNCH_SRC_GRP
-    }
-    st = launch_status();
-    if (st != BPT_OK || Pout->n_heavy == 0) return st;
-    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pout->n_heavy, H * D / WAVE, 2), dim3(BLOCK), 0, s, Pout->heavy,
-                       (const float *)ws_dk, (T *)dk, (T *)dv, H * D, (size_t)Pout->n_slots * H * D);
-    return launch_status();
-}
-
-template <typename T, int H, int D>
-int run_attn_bwd_team(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
-                      const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
-    const size_t EH = (size_t)Pin->n_edges * H;
-    float2 *pds = (float2 *)ws;
-    float *ws_rows = (float *)ws + 2 * (round16((int64_t)EH * 4) / 4);
-    {
-        ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
-        hipLaunchKernelGGL((k_attn_bwd_dst_team<T, H, D>), dim3((int)(8 * Pin->grp_max_chunk)), dim3(BLOCK), 0, s, *Pin, (const T *)q,
-                           (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E);
-    }
-    int st = launch_status();
-    if (st != BPT_OK) return st;
-    if (Pin->n_heavy > 0) {
-        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, Pin->heavy,
-                           (const float *)ws_rows, (T *)dq, (T *)nullptr, H * D, (size_t)0);
-        st = launch_status();
-        if (st != BPT_OK) return st;
-    }
-    float *ws_dk = ws_rows, *ws_dv = ws_rows + (size_t)Pout->n_slots * H * D;
-    {
-        ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
-        hipLaunchKernelGGL((k_attn_bwd_src_team<T, H, D>), dim3((int)(8 * Pout->grp_max_chunk)), dim3(BLOCK), 0, s, *Pout, (const T *)q,
-                           (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv);
-    }
-    st = launch_status();
-    if (st != BPT_OK || Pout->n_heavy == 0) return st;
-    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pout->n_heavy, H * D / WAVE, 2), dim3(BLOCK), 0, s, Pout->heavy,
-                       (const float *)ws_dk, (T *)dk, (T *)dv, H * D, (size_t)Pout->n_slots * H * D);
-    return launch_status();
-}
-
-template <typename T, int H, int D>
 int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
                  const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
     if (Pin->n_items == 0) return BPT_OK;
-    if (has_teams(Pin) && has_teams(Pout) && Pin->grp_pairs)
-        return run_attn_bwd_team<T, H, D>(Pin, Pout, q, k, v, o, d_o, lse, dq, dk, dv, ws, scale, s);
-    if (has_groups(Pin) && has_groups(Pout) && Pin->grp_pairs)
-        return run_attn_bwd_grouped<T, H, D>(Pin, Pout, q, k, v, o, d_o, lse, dq, dk, dv, ws, scale, s);
-    const size_t EH = (size_t)Pin->n_edges * H;
-    float *pbuf = (float *)ws;
-    float *dsbuf = pbuf + round16((int64_t)EH * 4) / 4;
-    float *ws_rows = dsbuf + round16((int64_t)EH * 4) / 4;
+    const bool grouped = grouped_backward(Pin, Pout, H, D, sizeof(T));
+    const int64_t pbytes = pds_bytes(Pin, Pout, H, D, sizeof(T));
+    float *pbuf = (float *)ws;                                   // per-row kernels: p (E, H) then ds (E, H)
+    float *dsbuf = pbuf + pbytes / 8;
+    float2 *pds = (float2 *)ws;                                  // row-group kernels: interleaved (p, ds)
+    float *ws_rows = (float *)ws + pbytes / 4;
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
-        hipLaunchKernelGGL((k_attn_bwd_dst<T, H, D, FAST_BATCH>), dim3(grid_for(Pin)), dim3(BLOCK), 0, s, *Pin, (const T *)q,
-                           (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pbuf, dsbuf, ws_rows, scale,
-                           scale * LOG2E);
+        if (grouped) {
+#define LAUNCH_DST(RR)                                                                                                        \
+    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, RR>), dim3(group_grid(Pin)), dim3(WAVE), 0, s, *Pin, (const T *)q,   \
+                       (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E)
+            if constexpr (H <= 8 && H * D <= 512) {
+                if (Pin->grp_R == 8) LAUNCH_DST(8);
+                else LAUNCH_DST(4);
+            } else {
+                LAUNCH_DST(4);
+            }
+#undef LAUNCH_DST
+        } else {
+            hipLaunchKernelGGL((k_attn_bwd_dst<T, H, D, FAST_BATCH>), dim3(grid_for(Pin)), dim3(BLOCK), 0, s, *Pin, (const T *)q,
+                               (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pbuf, dsbuf, ws_rows, scale,
+                               scale * LOG2E);
+        }
     }
     int st = launch_status();
     if (st != BPT_OK) return st;
@@ -1739,7 +1410,29 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
         if (st != BPT_OK) return st;
     }
     // source side: dK[src] = sum ds * q[dst], dV[src] = sum p * dO[dst]
-    return run_spmm_fast<T, float, H, D, 2>(Pout, dsbuf, q, dk, pbuf, d_o, dv, ws_rows, s);
+    if (!grouped) {
+        ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
+        return run_spmm_fast<T, float, H, D, 2>(Pout, dsbuf, q, dk, pbuf, d_o, dv, ws_rows, s);
+    }
+    float *ws_dk = ws_rows, *ws_dv = ws_rows + (size_t)Pout->n_slots * H * D;
+    {
+        ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
+#define LAUNCH_SRC(RR)                                                                                                       \
+    hipLaunchKernelGGL((k_attn_bwd_src_grp<T, H, D, RR>), dim3(group_grid(Pout)), dim3(WAVE), 0, s, *Pout, (const T *)q, \
+                       (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv)
+        if constexpr (H <= 8 && H * D <= 512) {
+            if (Pout->grp_R == 8) LAUNCH_SRC(8);
+            else LAUNCH_SRC(4);
+        } else {
+            LAUNCH_SRC(4);
+        }
+#undef LAUNCH_SRC
+    }
+    st = launch_status();
+    if (st != BPT_OK || Pout->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pout->n_heavy, H * D / WAVE, 2), dim3(BLOCK), 0, s, Pout->heavy,
+                       (const float *)ws_dk, (T *)dk, (T *)dv, H * D, (size_t)Pout->n_slots * H * D);
+    return launch_status();
 }
 
 }  // namespace
@@ -1766,18 +1459,6 @@ const char *bpt_strerror(int status) {
 
 int bpt_set_force_generic(int on) { return g_force_generic.exchange(on ? 1 : 0); }
 
-int bpt_set_group_variant(int kernel, int variant) {
-    if (kernel < 0 || kernel > 2 || (variant != 2 && variant != 3 && variant != 4)) return BPT_ERR_SIZE;
-    g_group_variant[kernel].store(variant);
-    return BPT_OK;
-}
-
-int bpt_set_group_waves(int kernel, int waves_per_xcd) {
-    if (kernel < 0 || kernel > 2 || waves_per_xcd < 0) return BPT_ERR_SIZE;
-    g_group_waves[kernel].store(waves_per_xcd);
-    return BPT_OK;
-}
-
 int bpt_profile_kernel(int which, void *start_event, void *stop_event) {
     if (which != 0 && (!start_event || !stop_event)) return BPT_ERR_NULL;
     g_prof_start.store(start_event);
@@ -1798,7 +1479,7 @@ int64_t bpt_workspace_bytes(int op, const bpt_plan *plan, const bpt_plan *plan_t
         case BPT_OP_ATTN_FWD: return round16(s0 * (C + 2 * h) * 4);
         case BPT_OP_ATTN_BWD: {
             const int64_t rows = s0 > 2 * s1 ? s0 : 2 * s1;
-            return 2 * round16(plan->n_edges * h * 4) + round16(rows * C * 4);
+            return pds_bytes(plan, plan_t, h, d, dtype == BPT_BF16 ? 2 : 4) + round16(rows * C * 4);
         }
         default: return -1;
     }

@@ -367,20 +367,24 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
 // Greedy clustering of work items (rows / row segments) that read mostly the same neighbour rows.
 // Items are visited in locality order; an item opens a group and the next `window` unused items
 // join it while at least half of their neighbours are already in the group's union (at most R
-// members).  The groups are then cut into 8 contiguous chunks of about equal work (one per XCD) and
+// members, and at most max_pairs edges in total unless max_pairs is 0: a group is walked by one
+// wavefront from start to end, so the largest group bounds the kernel's duration from below).  The groups are then cut into 8 contiguous chunks of about equal work (one per XCD) and
 // ordered inside each chunk (order_mode 0: locality order; 1: groups with at least average work first,
 // the small ones last, each part in locality order; 2: by decreasing work).  For every group the union
 // of neighbour ids becomes a list of entries (idx, member mask, first pair); a pair = one original
-// edge = (entry, member).  Pairs are numbered entry by entry, members ascending — the order in which
-// the kernels visit them.
+// edge = (entry, member).  Pairs are numbered entry by entry, members ascending.  With order_mode + 4
+// the entries of a group are sorted by member mask (stable, larger first), which lets a kernel that
+// handles two consecutive entries per step find the same members in both most of the time.
 int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32, const int32_t *eid32,
                     int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window, int32_t order_mode,
-                    int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *chunks,
+                    int32_t max_pairs, int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *chunks,
                     int64_t *n_groups_out, int64_t *n_entries_out) {
     if (!items || !members || !grp_ptr || !chunks || !n_groups_out || !n_entries_out) return BPTG_ERR_NULL;
     if (n_edges > 0 && (!idx32 || !eid32 || !entries || !pair_eid)) return BPTG_ERR_NULL;
     if (n_items < 0 || n_edges < 0 || n_index_nodes < 0) return BPTG_ERR_SIZE;
-    if (R < 1 || R > 16 || window < 0 || order_mode < 0 || order_mode > 2) return BPTG_ERR_ARG;
+    if (R < 1 || R > 16 || window < 0 || order_mode < 0 || order_mode > 7 || max_pairs < 0) return BPTG_ERR_ARG;
+    const bool by_mask = (order_mode & 4) != 0;
+    order_mode &= 3;
     for (int64_t i = 0; i < n_items; ++i) {
         const int32_t *it = items + 4 * i;
         if (it[1] < 0 || it[2] < it[1] || it[2] > n_edges) return BPTG_ERR_RANGE;
@@ -429,7 +433,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
             if (len == 0) continue;
             int32_t hit = 0;
             for (int32_t p = it[1]; p < it[2]; ++p) hit += (stamp[(size_t)idx32[p]] == n_groups);
-            if (2 * hit >= len) {
+            if (2 * hit >= len && (max_pairs == 0 || w + len <= max_pairs)) {
                 used[(size_t)cand] = 1;
                 mem[n_mem++] = cand;
                 w += len;
@@ -461,6 +465,17 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
             auto b = gorder.begin() + chunks[x], e = gorder.begin() + chunks[x + 1];
             if (order_mode == 2) {
                 std::stable_sort(b, e, [&](int32_t a, int32_t c) { return work[(size_t)a] > work[(size_t)c]; });
+            } else if (order_mode == 3) {
+                // runs of four groups that are consecutive in locality order stay together; the runs go by decreasing work
+                const int64_t n = e - b, nq = (n + 3) / 4;
+                std::vector<int64_t> qwork((size_t)nq, 0);
+                std::vector<int32_t> qorder((size_t)nq), tmp(b, e);
+                for (int64_t i = 0; i < n; ++i) qwork[(size_t)(i / 4)] += work[(size_t)tmp[(size_t)i]];
+                for (int64_t i = 0; i < nq; ++i) qorder[(size_t)i] = (int32_t)i;
+                std::stable_sort(qorder.begin(), qorder.end(), [&](int32_t a, int32_t c) { return qwork[(size_t)a] > qwork[(size_t)c]; });
+                auto out = b;
+                for (int64_t i = 0; i < nq; ++i)
+                    for (int64_t j = 4 * (int64_t)qorder[(size_t)i]; j < std::min<int64_t>(n, 4 * (int64_t)qorder[(size_t)i] + 4); ++j) *out++ = tmp[(size_t)j];
             } else {
                 int64_t sum = 0;
                 for (auto it = b; it != e; ++it) sum += work[(size_t)*it];
@@ -472,12 +487,15 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
 
     // ---- phase 3: emit members, entries and pairs in the final group order
     struct Triple { int32_t idx, member, eid; };
+    struct Entry { int32_t idx, mask, eids[16]; };
     std::vector<Triple> tri;
+    std::vector<Entry> ents;
     int64_t n_entries = 0, n_pairs = 0;
     grp_ptr[0] = 0;
     for (int64_t gi = 0; gi < n_groups; ++gi) {
         const int32_t *gmem = &grp_items[(size_t)gorder[(size_t)gi] * R];
         tri.clear();
+        ents.clear();
         for (int32_t m = 0; m < R; ++m) {
             int32_t *mem = members + ((int64_t)gi * R + m) * 2;
             if (gmem[m] >= 0) {
@@ -507,20 +525,29 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
             int32_t mult = 0;
             for (int32_t m = 0; m < R; ++m) mult = std::max(mult, cnt[m]);
             for (int32_t t = 0; t < mult; ++t) {
-                int32_t mask = 0;
-                int32_t *en = entries + 4 * n_entries;
-                en[0] = tri[a].idx;
-                en[2] = (int32_t)n_pairs;
-                en[3] = 0;
+                Entry en;
+                en.idx = tri[a].idx;
+                en.mask = 0;
                 for (int32_t m = 0; m < R; ++m)
                     if (cnt[m] > t) {
-                        mask |= 1 << m;
-                        pair_eid[n_pairs++] = tri[start[m] + (size_t)t].eid;
+                        en.mask |= 1 << m;
+                        en.eids[m] = tri[start[m] + (size_t)t].eid;
                     }
-                en[1] = mask;
-                ++n_entries;
+                ents.push_back(en);
             }
             a = b;
+        }
+        // equal masks next to each other (larger masks first), neighbour order kept inside a mask
+        if (by_mask) std::stable_sort(ents.begin(), ents.end(), [](const Entry &x, const Entry &y) { return x.mask > y.mask; });
+        for (const Entry &e : ents) {
+            int32_t *en = entries + 4 * n_entries;
+            en[0] = e.idx;
+            en[1] = e.mask;
+            en[2] = (int32_t)n_pairs;
+            en[3] = 0;
+            for (int32_t m = 0; m < R; ++m)
+                if (e.mask >> m & 1) pair_eid[n_pairs++] = e.eids[m];
+            ++n_entries;
         }
         grp_ptr[gi + 1] = (int32_t)n_entries;
     }

@@ -74,8 +74,10 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() else None
 
 
-def _workspace(op, plan, plan_t, h, d, dt, device):
-    n = _LIB.bpt_workspace_bytes(op, plan.ref, plan_t.ref if plan_t is not None else None, h, d, dt)
+def _workspace(op, plan, plan_t, h, d, dt, device, plan_ref=None, plan_t_ref=None):
+    if plan_t_ref is None and plan_t is not None:
+        plan_t_ref = plan_t.ref
+    n = _LIB.bpt_workspace_bytes(op, plan.ref if plan_ref is None else plan_ref, plan_t_ref, h, d, dt)
     if n < 0:
         raise RuntimeError("bpt_workspace_bytes failed")
     if n == 0:
@@ -226,14 +228,13 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None):
     h, d = _hd(q)
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
-    if _USE_GROUPS:
-        plan.ensure_groups()
+    ref = ctypes.byref(plan.ensure_groups(_group_rows(q, h, d))["struct"]) if _USE_GROUPS else plan.ref
     o = torch.empty_like(q)
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
     ws, nws = _workspace(OP_ATTN_FWD, plan, None, h, d, dt, q.device)
     with torch.cuda.device_of(q):
-        check_attn(_LIB.bpt_attention_forward(plan.ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws), nws,
+        check_attn(_LIB.bpt_attention_forward(ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws), nws,
                                               scale, h, d, dt, _stream()), "attention_forward")
     return o, lse
 
@@ -250,18 +251,39 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0))
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dt = _dtype(q)
-    ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device)
-    in_ref = plan_in.ref
+    in_ref, out_ref = plan_in.ref, plan_out.ref
     if _USE_GROUPS and plan_in.covers_all_edges and plan_out.covers_all_edges:
-        in_ref = ctypes.byref(plan_in.linked_to(plan_out))
+        R = _group_rows(q, h, d)
+        in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
+        out_ref = ctypes.byref(plan_out.ensure_groups(R)["struct"])
+    ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
     with torch.cuda.device_of(q):
-        check_attn(_LIB.bpt_attention_backward(in_ref, plan_out.ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do),
+        check_attn(_LIB.bpt_attention_backward(in_ref, out_ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do),
                                                _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
                                                scale, h, d, dt, _stream()), "attention_backward")
     return dq, dk, dv
 
 
 _USE_GROUPS = True
+_GROUP_ROWS = None          # None: chosen per call from dtype and shape
+
+
+def _group_rows(q, h, d):
+    """Rows per group for the fused kernels.  Groups of 8 exist where the per-member state still fits the
+    register file (h <= 8, h*d <= 512); they measured faster than groups of 4 for float32 and slower for bfloat16."""
+    fits8 = h <= 8 and h * d <= 512
+    if _GROUP_ROWS is not None:
+        return _GROUP_ROWS if fits8 else 4
+    return 8 if (fits8 and q.dtype == torch.float32) else 4
+
+
+def set_group_rows(R):
+    """Testing / measurement hook: force groups of R (4 or 8) rows, or None for the default choice.  Returns the old value."""
+    global _GROUP_ROWS
+    if R not in (None, 4, 8):
+        raise ValueError("R must be None, 4 or 8")
+    old, _GROUP_ROWS = _GROUP_ROWS, R
+    return old
 
 
 def set_row_groups(on):
@@ -269,30 +291,6 @@ def set_row_groups(on):
     global _USE_GROUPS
     old, _USE_GROUPS = _USE_GROUPS, bool(on)
     return old
-
-
-def set_group_rows(R):
-    """Rows per group of the fused kernels: 16 = teams of 4 wavefronts sharing neighbour rows through LDS
-    (default), 4 = one wavefront per group.  Returns the previous value."""
-    from . import plan as _plan
-    if R not in (4, 16):
-        raise ValueError("R must be 4 or 16")
-    old, _plan.GROUP_R = _plan.GROUP_R, R
-    return old
-
-
-def set_group_variant(fwd=None, bwd_dst=None, bwd_src=None):
-    """Tuning of the row-group kernels (see bpt_set_group_variant): 4, 2 or 3 per kernel; None keeps the current one."""
-    for kernel, var in enumerate((fwd, bwd_dst, bwd_src)):
-        if var is not None:
-            check_attn(_LIB.bpt_set_group_variant(kernel, int(var)), "set_group_variant")
-
-
-def set_group_waves(fwd=None, bwd_dst=None, bwd_src=None):
-    """Persistent wavefronts per XCD for each row-group kernel (0: one wavefront per group); None keeps the value."""
-    for kernel, n in enumerate((fwd, bwd_dst, bwd_src)):
-        if n is not None:
-            check_attn(_LIB.bpt_set_group_waves(kernel, int(n)), "set_group_waves")
 
 
 def set_force_generic(on):

@@ -17,9 +17,11 @@ import torch
 from ._lib import PlanInfo, PlanStruct, check_graph, graph_lib
 
 DEFAULT_SEG_LEN = 64
-GROUP_R = 4            # rows per group: 4 = one wavefront per group (default, fastest measured); 16 = a team of 4 wavefronts x 4 rows sharing rows through LDS
+GROUP_R = 4            # default rows per group (the row-group kernels exist for 4 and, float32 with h <= 8 and h*d <= 512, 8)
 GROUP_WINDOW = 32      # how many following items the greedy grouping examines per group
-GROUP_ORDER = 2        # order of the groups inside an XCD chunk: 0 locality, 1 big first / small last, 2 decreasing work
+GROUP_ORDER = 2 + 4    # groups inside an XCD chunk by decreasing work (2); entries of a group sorted by member mask (+4)
+GROUP_MAX_PAIRS = 0     # cap on the edges of one group (0 = none)
+GROUP_PAD_ENTRIES = 8  # the kernels' software pipeline reads per-entry arrays this far past the end
 _CACHE_SIZE = 64
 
 
@@ -61,11 +63,13 @@ def build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len=DE
     return arrays, info
 
 
-def build_groups_host(arrays, n_index_nodes, R=None, window=GROUP_WINDOW, order_mode=None):
+def build_groups_host(arrays, n_index_nodes, R=None, window=GROUP_WINDOW, order_mode=None, max_pairs=None):
     """Pure host step: clusters the plan's items into row groups (bptg_group_plan).  Returns a dict
     with members (n_groups, R, 2), grp_ptr (n_groups + 1), entries (n_entries, 4), pair_eid (n_edges),
-    chunks (9,)."""
+    chunks (9,), and slot_eid (n_entries, R): the edge id of (entry, member), -1 where the entry's
+    mask has no such member."""
     order_mode = GROUP_ORDER if order_mode is None else order_mode
+    max_pairs = GROUP_MAX_PAIRS if max_pairs is None else max_pairs
     R = GROUP_R if R is None else R
     items = np.ascontiguousarray(arrays["items"], dtype=np.int32)
     idx = np.ascontiguousarray(arrays["idx"], dtype=np.int32)
@@ -78,11 +82,35 @@ def build_groups_host(arrays, n_index_nodes, R=None, window=GROUP_WINDOW, order_
     chunks = np.zeros(9, dtype=np.int32)
     ng, ne = ctypes.c_int64(), ctypes.c_int64()
     check_graph(graph_lib().bptg_group_plan(_ptr(items), n_items, _ptr(idx), _ptr(eid), E, int(n_index_nodes), R, window,
-                                            int(order_mode), _ptr(members), _ptr(grp_ptr), _ptr(entries), _ptr(pair_eid),
+                                            int(order_mode), int(max_pairs), _ptr(members), _ptr(grp_ptr), _ptr(entries), _ptr(pair_eid),
                                             _ptr(chunks), ctypes.byref(ng), ctypes.byref(ne)))
+    entries = entries[:ne.value].copy()
+    pair_eid = pair_eid[:E].copy()
+    present = (entries[:, 1:2] >> np.arange(R, dtype=np.int32)[None, :]) & 1 == 1      # (n_entries, R)
+    slot_eid = np.full((ne.value, R), -1, dtype=np.int32)
+    slot_eid[present] = pair_eid          # pairs are numbered entry by entry, members ascending
     return {"members": members[:ng.value].copy(), "grp_ptr": grp_ptr[:ng.value + 1].copy(),
-            "entries": entries[:ne.value].copy(), "entries_padded": entries[:ne.value + 1].copy(),
-            "pair_eid": pair_eid[:E].copy(), "chunks": chunks, "R": R}
+            "entries": entries, "pair_eid": pair_eid, "slot_eid": slot_eid, "chunks": chunks, "R": R}
+
+
+def link_groups_host(grp_dst, grp_src, n_edges):
+    """Pure host step: for every (entry, member) of the destination-side groups, the position
+    entry' * R + member' of the same edge in the source-side groups; where the entry has no such member, and in
+    the GROUP_PAD_ENTRIES * R elements of padding, the spare position (n_entries_src + GROUP_PAD_ENTRIES) * R - 1
+    (the last one of the source side's padding, which no kernel uses).  int32, length
+    (n_entries_dst + GROUP_PAD_ENTRIES) * R."""
+    R = grp_dst["R"]
+    src_slots = grp_src["slot_eid"].reshape(-1)
+    valid = np.flatnonzero(src_slots >= 0)
+    if len(valid) != n_edges:
+        raise ValueError("the source-side groups do not cover every edge exactly once")
+    pos_of_eid = np.zeros(max(n_edges, 1), dtype=np.int32)
+    pos_of_eid[src_slots[valid]] = valid.astype(np.int32)
+    dst_slots = grp_dst["slot_eid"].reshape(-1)
+    spare = (len(grp_src["entries"]) + GROUP_PAD_ENTRIES) * R - 1
+    out = np.full((len(grp_dst["entries"]) + GROUP_PAD_ENTRIES) * R, spare, dtype=np.int32)
+    out[:len(dst_slots)] = np.where(dst_slots >= 0, pos_of_eid[np.maximum(dst_slots, 0)], spare)
+    return out
 
 
 class Plan:
@@ -98,7 +126,7 @@ class Plan:
         self.device = torch.device(device)
         self.n_index_nodes = int(n_index_nodes)
         self._host = arrays                  # kept for the (lazy) row-group construction
-        self._groups = None
+        self._groups = {}
         self._links = {}
         self._lock = threading.Lock()
         # one allocation, 256-byte aligned sections (the items array is read as 16-byte vectors)
@@ -115,42 +143,42 @@ class Plan:
         return ctypes.byref(self.struct)
 
     # ---- row groups for the fused attention kernels ----
-    def ensure_groups(self):
-        """Builds the row-group arrays once (host) and uploads them; returns the host dict."""
+    def ensure_groups(self, R=GROUP_R):
+        """Builds the row-group arrays for groups of R rows once (host) and uploads them.  Returns a dict with
+        the host arrays ("host") and the `bpt_plan` carrying them ("struct")."""
         with self._lock:
-            if self._groups is None or self._groups["R"] != GROUP_R:
-                self._links = {}
-                grp = build_groups_host(self._host, self.n_index_nodes)
-                self._grp_dev = {k: torch.from_numpy(grp[k]).to(self.device)
-                                 for k in ("members", "grp_ptr", "entries_padded", "chunks")}
-                d = self._grp_dev
-                self.n_groups = len(grp["members"])
-                self.struct.grp_members = d["members"].data_ptr() if self.n_groups else None
-                self.struct.grp_ptr = d["grp_ptr"].data_ptr()
-                self.struct.grp_entries = d["entries_padded"].data_ptr()
-                self.struct.grp_pairs = None
-                self.struct.grp_chunks = d["chunks"].data_ptr()
-                self.struct.grp_max_chunk = int(np.diff(grp["chunks"]).max()) if self.n_groups else 0
-                self.struct.n_groups = self.n_groups
-                self.struct.grp_R = grp["R"]
-                self._groups = grp
-        return self._groups
+            hit = self._groups.get(R)
+            if hit is None:
+                grp = build_groups_host(self._host, self.n_index_nodes, R=R)
+                dev = {k: torch.from_numpy(grp[k]).to(self.device) for k in ("members", "grp_ptr", "entries", "chunks")}
+                n_groups = len(grp["members"])
+                st = PlanStruct.from_buffer_copy(self.struct)
+                st.grp_members = dev["members"].data_ptr() if n_groups else None
+                st.grp_ptr = dev["grp_ptr"].data_ptr()
+                st.grp_entries = dev["entries"].data_ptr() if len(grp["entries"]) else None
+                st.grp_pairs = None
+                st.grp_chunks = dev["chunks"].data_ptr()
+                st.grp_max_chunk = int(np.diff(grp["chunks"]).max()) if n_groups else 0
+                st.n_groups = n_groups
+                st.grp_R = R
+                st.n_grp_entries = len(grp["entries"])
+                hit = {"host": grp, "dev": dev, "struct": st}
+                self._groups[R] = hit
+        return hit
 
-    def linked_to(self, plan_src):
-        """`bpt_plan` of this (destination-side) plan whose grp_pairs maps each of its pairs to the number of
-        the same edge's pair in `plan_src` (the source-side plan of the same graph)."""
-        mine, theirs = self.ensure_groups(), plan_src.ensure_groups()
-        key = (id(plan_src), GROUP_R)
+    def linked_to(self, plan_src, R=GROUP_R):
+        """`bpt_plan` of this (destination-side) plan whose grp_pairs maps each (entry, member) of its groups to
+        the position entry' * R + member' of the same edge in `plan_src` (the source-side plan of the same graph)."""
+        mine, theirs = self.ensure_groups(R), plan_src.ensure_groups(R)
+        key = (id(plan_src), R)
         with self._lock:
             hit = self._links.get(key)
             if hit is None:
                 if self.n_edges != plan_src.n_edges or not (self.covers_all_edges and plan_src.covers_all_edges):
                     raise ValueError("the two plans do not describe the same edge set")
-                pos_of_eid = np.empty(self.n_edges, dtype=np.int32)
-                pos_of_eid[theirs["pair_eid"]] = np.arange(self.n_edges, dtype=np.int32)
-                pairs = torch.from_numpy(pos_of_eid[mine["pair_eid"]]).to(self.device)
-                st = PlanStruct.from_buffer_copy(self.struct)
-                st.grp_pairs = pairs.data_ptr() if self.n_edges else None
+                pairs = torch.from_numpy(link_groups_host(mine["host"], theirs["host"], self.n_edges)).to(self.device)
+                st = PlanStruct.from_buffer_copy(mine["struct"])
+                st.grp_pairs = pairs.data_ptr()
                 hit = (st, pairs, plan_src)          # keeps the mapping and the partner alive
                 self._links[key] = hit
         return hit[0]

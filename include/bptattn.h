@@ -54,28 +54,23 @@ typedef struct {
     int64_t n_rows, n_edges, n_items, n_heavy, n_slots;
     const int32_t *grp_members;  /* n_groups * grp_R * 2 : (row, slot), row = -1 unused */
     const int32_t *grp_ptr;      /* n_groups + 1 : entry range of each group */
-    const int32_t *grp_entries;  /* n_entries * 4 : neighbour id, member mask, first pair, 0 */
-    const int32_t *grp_pairs;    /* n_edges or NULL.  On the destination-side plan of the fused backward:
-                                    for every pair of this plan, the number of the same edge's pair in the
-                                    source-side plan (the per-edge scratch is laid out in that order) */
+    const int32_t *grp_entries;  /* n_grp_entries * 4 : neighbour id, member mask, first pair, 0 */
+    const int32_t *grp_pairs;    /* (n_grp_entries + 8) * grp_R or NULL.  On the destination-side plan of the
+                                    fused backward: for (entry u, member m) of this plan, at [u * grp_R + m], the
+                                    position u' * grp_R + m' of the same edge in the source-side plan (the
+                                    per-pair scratch is laid out in that order); where the entry's mask has
+                                    no bit m, and in the 8 entries of padding, the spare position
+                                    (n_grp_entries of the source side + 8) * grp_R - 1 */
     const int32_t *grp_chunks;   /* 9 : groups grp_chunks[x] .. grp_chunks[x+1]-1 are walked by XCD x */
     int64_t n_groups, grp_R;
     int64_t grp_max_chunk;       /* largest chunk length; the row-group kernels launch 8 * grp_max_chunk workgroups */
+    int64_t n_grp_entries;       /* grp_ptr[n_groups] */
 } bpt_plan;
 
 const char *bpt_strerror(int status);
 
 /* 1: force the shape-generic kernels even where a specialised one exists (testing). Returns the old value. */
 int bpt_set_force_generic(int on);
-
-/* Tuning knob of the row-group kernels.  kernel: 0 forward, 1 backward destination side, 2 backward source
- * side.  variant: 4 = load batches of four neighbour rows, 2 = batches of two, 3 = batches of two compiled
- * for three resident wavefronts per SIMD. */
-int bpt_set_group_variant(int kernel, int variant);
-
-/* How many wavefronts per XCD walk that XCD's share of the row groups (persistent wavefronts, each
- * prefetching the next group's header and entries); 0 = one wavefront per group.  kernel as above. */
-int bpt_set_group_waves(int kernel, int waves_per_xcd);
 
 /* Measurement aid (no counterpart in the reference): while `which` is one of BPT_KERNEL_*, every launch
  * of that main kernel of the fused path is bracketed by hipEventRecord(start_event) / (stop_event) on

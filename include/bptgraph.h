@@ -91,12 +91,15 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
  *   pair_eid int32[n_edges]       edge id of every pair; pairs are numbered entry by entry, members
  *                                 ascending, and every edge of the plan appears exactly once
  *   chunks   int32[9]             groups chunks[x] .. chunks[x+1]-1 go to XCD x (contiguous, about equal work)
- * order_mode: order of the groups inside a chunk — 0 locality, 1 at-least-average work first then the
- * small ones, 2 decreasing work.
+ * order_mode: low two bits = order of the groups inside a chunk — 0 locality, 1 at-least-average work first
+ * then the small ones, 2 decreasing work; + 4 = inside a group, entries with equal member masks are made
+ * adjacent (larger masks first, neighbour order kept among equal masks) instead of plain neighbour order.
+ * max_pairs: no item joins a group whose edges would then number more than this (0 = no limit); it bounds
+ * the work of the wavefront that walks the group.
  * A neighbour that a member reaches through several parallel edges gets one entry per multiplicity. */
 int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32, const int32_t *eid32,
                     int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window, int32_t order_mode,
-                    int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *chunks,
+                    int32_t max_pairs, int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *chunks,
                     int64_t *n_groups, int64_t *n_entries);
 
 #ifdef __cplusplus

@@ -176,7 +176,7 @@ def test_single_head_2d_inputs(ops):
 # --------------------------------------------------------------------------------------------
 # the attention layer: fused kernels and the unfused op chain, forward + backward
 # --------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("fused", ["teams", "groups-4", "groups-2", "groups-3", "rows", False])
+@pytest.mark.parametrize("fused", ["groups", "groups-4", "rows", False])
 @pytest.mark.parametrize("dtype,hd", [(torch.float32, (8, 64)), (torch.float32, (16, 64)), (torch.float32, (8, 32)),
                                       (torch.bfloat16, (8, 64)), (torch.bfloat16, (16, 64)), (torch.float32, (2, 24))])
 @pytest.mark.parametrize("gname", ["bpt512_k4", "bpt300_causal_k2", "multigraph"])
@@ -188,19 +188,15 @@ def test_attention_layer(ops, gname, dtype, hd, fused):
     c = case(gname)
     q, k, v, do = (rand((c.n, h, d), dtype, s, 1.0 / 8).to(DEV) for s in (11, 12, 13, 14))   # N(0,1)/sqrt(64)
     q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
-    # fused kernels: teams of 4 wavefronts (LDS-shared rows), one wavefront per row group (variants 4 / 2 / 3), or per row
+    # fused kernels: one wavefront per group of rows that share neighbours, or one wavefront per row
     old = graphop.set_row_groups(fused != "rows")
-    old_r = graphop.set_group_rows(16 if fused == "teams" else 4)
-    var = int(fused[-1]) if str(fused).startswith("groups-") else None
-    if var:
-        graphop.set_group_variant(var, var, var)
+    old_r = graphop.set_group_rows(4 if fused == "groups-4" else None)      # None: 8 rows where the kernels allow, else 4
     try:
         o = op.bpt_attention(*c.out, *c.inn, q, k, v, fused=bool(fused))
         o.backward(do)
     finally:
         graphop.set_row_groups(old)
         graphop.set_group_rows(old_r)
-        graphop.set_group_variant(2, 2, 2)
     ro, ra = oracle.attention_forward(c.csr, f64(q), f64(k), f64(v))
     rdq, rdk, rdv = oracle.attention_backward(c.csr, f64(q), f64(k), f64(v), ra, f64(do))
     close(o, ro, TOL[dtype], "o")

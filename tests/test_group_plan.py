@@ -5,9 +5,7 @@ import pytest
 
 import oracle
 from bpt_amd import graphbuilder as gb
-from bpt_amd.plan import build_groups_host, build_plan_host
-
-from bpt_amd.plan import GROUP_R
+from bpt_amd.plan import GROUP_PAD_ENTRIES, GROUP_R, build_groups_host, build_plan_host, link_groups_host
 
 
 def bpt(L, triu, step):
@@ -39,7 +37,7 @@ def plans(name, seg=64):
 
 
 @pytest.mark.parametrize("GROUP_R", [4, 16])
-@pytest.mark.parametrize("order_mode", [0, 1, 2])
+@pytest.mark.parametrize("order_mode", [0, 1, 2, 6])
 @pytest.mark.parametrize("seg", [8, 64])
 @pytest.mark.parametrize("name", sorted(GRAPHS))
 def test_group_plan_invariants(name, seg, order_mode, GROUP_R):
@@ -47,7 +45,6 @@ def test_group_plan_invariants(name, seg, order_mode, GROUP_R):
     E = len(src)
     for arrays, rows_of, cols_of in ((pin, dst, src), (pout, src, dst)):
         grp = build_groups_host(arrays, n, R=GROUP_R, order_mode=order_mode)
-        assert grp["entries_padded"].shape[0] == grp["entries"].shape[0] + 1 and not grp["entries_padded"][-1].any()
         members, gptr, entries, pair_eid = grp["members"], grp["grp_ptr"], grp["entries"], grp["pair_eid"]
         ch = grp["chunks"]
         assert ch[0] == 0 and ch[8] == len(members) and np.all(np.diff(ch) >= 0)
@@ -64,15 +61,23 @@ def test_group_plan_invariants(name, seg, order_mode, GROUP_R):
         # entries: masks valid, pairs numbered consecutively, every pair is an edge (entry idx -> member row)
         seg_of = {(r, s): (b, e) for r, b, e, s in items.tolist()}
         eid_slot = {int(e): p for p, e in enumerate(arrays["eid"].tolist())}
+        slot_eid = grp["slot_eid"]
+        assert slot_eid.shape == (len(entries), GROUP_R)
         n_pairs = 0
         for g in range(ng):
+            masks = entries[gptr[g]:gptr[g + 1], 1]
+            if order_mode & 4:
+                assert np.all(np.diff(masks) <= 0)                # equal masks adjacent, larger first
             for u in range(gptr[g], gptr[g + 1]):
                 idx, mask, pb, _ = entries[u].tolist()
                 assert 0 < mask < (1 << GROUP_R) and pb == n_pairs
                 for m in range(GROUP_R):
-                    if mask >> m & 1:
+                    if not mask >> m & 1:
+                        assert slot_eid[u, m] == -1
+                    else:
                         row, slot = members[g, m].tolist()
                         e = int(pair_eid[n_pairs]); n_pairs += 1
+                        assert slot_eid[u, m] == e
                         assert rows_of[e] == row and cols_of[e] == idx
                         b, en = seg_of[(row, slot)]
                         assert b <= eid_slot[e] < en              # the edge lies in this member's segment
@@ -126,8 +131,10 @@ def test_emulated_group_walk_matches_oracle(name, seg):
     assert np.allclose(o, ro, rtol=1e-10, atol=1e-12)
     # backward walk: destination side writes (p, ds) at the source side's pair numbers, source side reads them in order
     gout = build_groups_host(pout, n)
-    pos_of_eid = np.empty(len(src), dtype=np.int64); pos_of_eid[gout["pair_eid"]] = np.arange(len(src))
-    xpos = pos_of_eid[gin["pair_eid"]]
+    xpos = link_groups_host(gin, gout, len(src))
+    spare = (len(gout["entries"]) + GROUP_PAD_ENTRIES) * GROUP_R - 1
+    assert len(xpos) == (len(gin["entries"]) + GROUP_PAD_ENTRIES) * GROUP_R and np.all(xpos[len(gin["entries"]) * GROUP_R:] == spare)
+    assert np.all(xpos[:len(gin["entries"]) * GROUP_R][gin["slot_eid"].reshape(-1) < 0] == spare)
     rdq, rdk, rdv = oracle.attention_backward(csr, q, k, v, ra, do)
     scale = 1 / np.sqrt(d)
     delta = (do * ro).sum(-1)
@@ -138,33 +145,30 @@ def test_emulated_group_walk_matches_oracle(name, seg):
     np.add.at(z, dst, np.exp(sc - mrow[dst]))
     has = z > 0
     lse[has] = mrow[has] + np.log(z[has])
-    pds = np.full((len(src), h, 2), np.nan)
+    pds = np.full((len(gout["entries"]) * GROUP_R, h, 2), np.nan)     # scratch indexed by source-side (entry, member)
     dq = np.zeros_like(q)
-    n_pair = 0
     for g in range(len(gin["members"])):
         for u in range(gin["grp_ptr"][g], gin["grp_ptr"][g + 1]):
-            idx, mask, pb, _ = gin["entries"][u].tolist()
-            assert pb == n_pair
+            idx, mask, _, _ = gin["entries"][u].tolist()
             for m in range(GROUP_R):
                 if mask >> m & 1:
                     row = gin["members"][g, m, 0]
                     p = np.exp((q[row] * k[idx]).sum(-1) * scale - lse[row])
                     ds = p * ((do[row] * v[idx]).sum(-1) - delta[row]) * scale
                     dq[row] += ds[:, None] * k[idx]
-                    pds[xpos[n_pair], :, 0] = p; pds[xpos[n_pair], :, 1] = ds
-                    n_pair += 1
-    assert not np.isnan(pds).any() and np.allclose(dq, rdq, rtol=1e-9, atol=1e-12)
+                    t = xpos[u * GROUP_R + m]
+                    assert np.isnan(pds[t]).all()                      # every position written once
+                    pds[t, :, 0] = p; pds[t, :, 1] = ds
+    assert np.isnan(pds[:, 0, 0]).sum() == len(pds) - len(src) and np.allclose(dq, rdq, rtol=1e-9, atol=1e-12)
     dk = np.zeros_like(k); dv = np.zeros_like(v)
-    n_pair = 0
     for g in range(len(gout["members"])):
         for u in range(gout["grp_ptr"][g], gout["grp_ptr"][g + 1]):
-            idx, mask, pb, _ = gout["entries"][u].tolist()
+            idx, mask, _, _ = gout["entries"][u].tolist()
             for m in range(GROUP_R):
                 if mask >> m & 1:
                     row = gout["members"][g, m, 0]
-                    dk[row] += pds[n_pair, :, 1][:, None] * q[idx]
-                    dv[row] += pds[n_pair, :, 0][:, None] * do[idx]
-                    n_pair += 1
+                    dk[row] += pds[u * GROUP_R + m, :, 1][:, None] * q[idx]
+                    dv[row] += pds[u * GROUP_R + m, :, 0][:, None] * do[idx]
     assert np.allclose(dk, rdk, rtol=1e-9, atol=1e-12) and np.allclose(dv, rdv, rtol=1e-9, atol=1e-12)
 
 
