@@ -57,13 +57,13 @@ def make_workload(name):
 
 
 def algorithmic_bytes(N, E, H, D, s):
-    """Compulsory HBM traffic of the fused fwd+bwd step (every distinct input read once, every output
-    written once): 12*N*C*s + 2*N*H*4 + 3*E*4 + 2*(N+1)*4, split over the three main kernels so the parts
-    add up to the total."""
+    """Compulsory HBM traffic of the fused fwd+bwd step (every distinct input read once per pass, every
+    output written once): 12*N*C*s + 2*N*H*4 + 3*E*4 + 2*(N+1)*4, split over the three main kernels so that
+    the parts add up to the total: q and dO, which both backward kernels read, are charged half to each."""
     C = H * D
     fwd = 4 * N * C * s + N * H * 4 + E * 4 + (N + 1) * 4          # read q,k,v; write o, lse; in-CSR
-    bwd_dst = 6 * N * C * s + N * H * 4 + E * 4                    # read q,k,v,o,dO, lse; write dq; in-CSR
-    bwd_src = 2 * N * C * s + E * 4 + (N + 1) * 4                  # write dk,dv; out-CSR (q, dO counted above)
+    bwd_dst = 5 * N * C * s + N * H * 4 + E * 4                    # read k,v,o + half of (q,dO), lse; write dq; in-CSR
+    bwd_src = 3 * N * C * s + E * 4 + (N + 1) * 4                  # half of (q,dO); write dk,dv; out-CSR
     return {"attn_fwd": fwd, "attn_bwd_dst": bwd_dst, "attn_bwd_src": bwd_src, "total": fwd + bwd_dst + bwd_src}
 
 

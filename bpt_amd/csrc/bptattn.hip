@@ -936,7 +936,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 // Backward, destination side.  Writes (p, ds) of every pair to pds[(t * H + head)], t = the pair's
 // position (entry * R + member) in the SOURCE-side plan, which P.grp_pairs gives for every
 // (entry, member) of this plan (a spare position for members the entry does not have).  One store per
-// entry and quad of members: lane l carries the pair of member 4c + l % 4.  The members' q rows live in LDS.
+// entry and quad of members: lane l carries the pair of member 4c + l % 4; the same register of ds values is
+// the A operand of the MFMA that accumulates dq.  The members' q rows live in LDS.
 template <typename T, int H, int D, int R>
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H, D>::EPL, R>()))) void k_attn_bwd_dst_grp(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
@@ -957,7 +958,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
         int mk[GRP_BATCH], xp[GRP_BATCH][NQ];
     };
     __shared__ float4 q_lds[R * (EPL / 4) * WAVE];
-    float dov[R][EPL], dqa[R][EPL], delta_s[R], lse2[R];
+    float dov[R][EPL], delta_s[R], lse2[R];
+    floatx4 dqa[NQ][EPL];                       // [quad c][row register t][member 4c + i], as the source-side kernel's accumulators
 #pragma unroll
     for (int m = 0; m < R; ++m) {
         const uint32_t row = (uint32_t)max(gh.rows[m], 0);
@@ -968,9 +970,11 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
         lds_put_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qr);
         delta_s[m] = head_sum<L::LPH>(dot_n<EPL>(dov[m], ov)) * scale;
         lse2[m] = lse[(size_t)row * H + head];
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) dqa[m][i] = 0.f;
     }
+#pragma unroll
+    for (int c = 0; c < NQ; ++c)
+#pragma unroll
+        for (int t = 0; t < EPL; ++t) dqa[c][t] = floatx4{0.f, 0.f, 0.f, 0.f};
     for (int p0 = gh.begin; p0 < gh.end; p0 += GRP_CHUNK) {
         const int cnt = min(GRP_CHUNK, gh.end - p0);
         // lanes past the end repeat the last entry with an empty mask
@@ -1007,8 +1011,6 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                         head_sum2<L::LPH>(s, dp);
                         const float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
                         const float ds = pe * fmaf(dp, scale, -delta_s[m]);
-#pragma unroll
-                        for (int i = 0; i < EPL; ++i) dqa[m][i] = fmaf(ds, kv[i], dqa[m][i]);
                         wp[m / 4] = mine == (m & 3) ? pe : wp[m / 4];
                         wd[m / 4] = mine == (m & 3) ? ds : wd[m / 4];
                     }
@@ -1018,6 +1020,9 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                     if ((B.mk[e] >> (4 * c)) & 15) {      // (look-ahead batches past the group's end have empty masks)
                         char *w = reinterpret_cast<char *>(pds);
                         *reinterpret_cast<float2 *>(w + (size_t)((uint32_t)B.xp[e][c] * (uint32_t)(H * 8) + hoff)) = make_float2(wp[c], wd[c]);
+                        // dq[member 4c + i] += ds[member] * k row: wd (0 for absent members) is the A operand
+#pragma unroll
+                        for (int t = 0; t < EPL; ++t) dqa[c][t] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd[c], kv[t], dqa[c][t], 0, 0, 0);
                     }
                 }
             }
@@ -1041,8 +1046,11 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 #pragma unroll
     for (int m = 0; m < R; ++m) {
         if (gh.rows[m] < 0) continue;
-        if (gh.slots[m] < 0) store_row<T, H, D>(dq + (size_t)gh.rows[m] * L::C, lane, dqa[m]);
-        else store_row_ws<T, H, D>(ws_dq + (size_t)gh.slots[m] * L::C, lane, dqa[m]);
+        float rq[EPL];
+#pragma unroll
+        for (int t = 0; t < EPL; ++t) rq[t] = dqa[m / 4][t][m & 3];
+        if (gh.slots[m] < 0) store_row<T, H, D>(dq + (size_t)gh.rows[m] * L::C, lane, rq);
+        else store_row_ws<T, H, D>(ws_dq + (size_t)gh.slots[m] * L::C, lane, rq);
     }
 }
 

@@ -228,7 +228,7 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None):
     h, d = _hd(q)
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
-    ref = ctypes.byref(plan.ensure_groups(_group_rows(q, h, d))["struct"]) if _USE_GROUPS else plan.ref
+    ref = ctypes.byref(plan.ensure_groups(_group_rows(q, h, d, plan))["struct"]) if _USE_GROUPS else plan.ref
     o = torch.empty_like(q)
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
@@ -253,7 +253,7 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref
     if _USE_GROUPS and plan_in.covers_all_edges and plan_out.covers_all_edges:
-        R = _group_rows(q, h, d)
+        R = _group_rows(q, h, d, plan_in)
         in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
         out_ref = ctypes.byref(plan_out.ensure_groups(R)["struct"])
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
@@ -268,13 +268,16 @@ _USE_GROUPS = True
 _GROUP_ROWS = None          # None: chosen per call from dtype and shape
 
 
-def _group_rows(q, h, d):
+def _group_rows(q, h, d, plan):
     """Rows per group for the fused kernels.  Groups of 8 exist where the per-member state still fits the
-    register file (h <= 8, h*d <= 512); they measured faster than groups of 4 for float32 and slower for bfloat16."""
+    register file (h <= 8, h*d <= 512).  They halve the row fetches but double the work of the longest
+    wavefront, which measured as a gain only for float32 on graphs with enough groups to fill the GPU twice
+    or with long rows (average degree >= 64)."""
     fits8 = h <= 8 and h * d <= 512
     if _GROUP_ROWS is not None:
         return _GROUP_ROWS if fits8 else 4
-    return 8 if (fits8 and q.dtype == torch.float32) else 4
+    big = plan.n_items >= 16384 or plan.n_edges >= 64 * max(plan.n_rows, 1)
+    return 8 if (fits8 and q.dtype == torch.float32 and big) else 4
 
 
 def set_group_rows(R):

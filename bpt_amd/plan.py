@@ -20,7 +20,7 @@ DEFAULT_SEG_LEN = 64
 GROUP_R = 4            # default rows per group (the row-group kernels exist for 4 and, float32 with h <= 8 and h*d <= 512, 8)
 GROUP_WINDOW = 32      # how many following items the greedy grouping examines per group
 GROUP_ORDER = 2 + 4    # groups inside an XCD chunk by decreasing work (2); entries of a group sorted by member mask (+4)
-GROUP_MAX_PAIRS = 0     # cap on the edges of one group (0 = none)
+GROUP_MAX_PAIRS = None  # cap on the edges of one group: None = 48 per member row, 0 = no cap
 GROUP_PAD_ENTRIES = 8  # the kernels' software pipeline reads per-entry arrays this far past the end
 _CACHE_SIZE = 64
 
@@ -69,8 +69,9 @@ def build_groups_host(arrays, n_index_nodes, R=None, window=GROUP_WINDOW, order_
     chunks (9,), and slot_eid (n_entries, R): the edge id of (entry, member), -1 where the entry's
     mask has no such member."""
     order_mode = GROUP_ORDER if order_mode is None else order_mode
-    max_pairs = GROUP_MAX_PAIRS if max_pairs is None else max_pairs
     R = GROUP_R if R is None else R
+    if max_pairs is None:
+        max_pairs = 48 * R if GROUP_MAX_PAIRS is None else GROUP_MAX_PAIRS
     items = np.ascontiguousarray(arrays["items"], dtype=np.int32)
     idx = np.ascontiguousarray(arrays["idx"], dtype=np.int32)
     eid = np.ascontiguousarray(arrays["eid"], dtype=np.int32)
