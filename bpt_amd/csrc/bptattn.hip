@@ -695,9 +695,12 @@ template <int R> struct GroupHead {
 // wavefronts per SIMD the row-group kernels are compiled for: the members' state has to stay in registers
 template <typename T, int EPL, int R> constexpr int grp_wpe() { return R * EPL <= 32 ? 3 : 2; }
 
-// Workgroup b (one wavefront) runs on XCD b % 8 and takes group number b / 8 of that XCD's chunk.
-template <int R> __device__ __forceinline__ bool fetch_group(const bpt_plan &P, GroupHead<R> &gh) {
-    const int x = blockIdx.x & 7, w = blockIdx.x >> 3;
+// Workgroup b (one wavefront) runs on XCD b % 8 and takes head slice (b / 8) % HS of group number (b / 8) / HS of
+// that XCD's chunk: HS wavefronts share a group, each handling H / HS of the heads of every row.  (Dispatching all
+// first slices before the second ones, to halve the rows an XCD's L2 has to hold at a time, measured slower.)
+template <int R, int HS> __device__ __forceinline__ int group_slice() { return (int)((blockIdx.x >> 3) % HS); }
+template <int R, int HS> __device__ __forceinline__ bool fetch_group(const bpt_plan &P, GroupHead<R> &gh) {
+    const int x = blockIdx.x & 7, w = (blockIdx.x >> 3) / HS;
     const int g = __builtin_amdgcn_readfirstlane(P.grp_chunks[x]) + w;
     if (g >= __builtin_amdgcn_readfirstlane(P.grp_chunks[x + 1])) return false;
     const int lane = threadIdx.x;
@@ -713,12 +716,12 @@ template <int R> __device__ __forceinline__ bool fetch_group(const bpt_plan &P, 
     return true;
 }
 
-// Row `row` of a node tensor through a uniform base pointer, a uniform 32-bit row offset and this lane's
-// constant byte offset `loff` (global_load with scalar base + 32-bit vector offset + immediate).
-template <typename T, int H, int D>
+// Row `row` of a node tensor (PITCH elements per row; the layout may cover a slice of the row's heads) through a
+// uniform base pointer, a uniform 32-bit row offset and this lane's constant byte offset `loff` (global_load with scalar base + 32-bit vector offset + immediate).
+template <typename T, int H, int D, int PITCH = Lay<T, H, D>::C>
 __device__ __forceinline__ void load_row32(const T *__restrict__ base, uint32_t row, uint32_t loff, float (&out)[Lay<T, H, D>::EPL]) {
     using L = Lay<T, H, D>;
-    const char *p = reinterpret_cast<const char *>(base) + (size_t)(row * (uint32_t)(L::C * sizeof(T)));
+    const char *p = reinterpret_cast<const char *>(base) + (size_t)(row * (uint32_t)(PITCH * sizeof(T)));
 #pragma unroll
     for (int i = 0; i < L::NV; ++i) {
         const char *pi = p + (size_t)(loff + (uint32_t)(i * L::LPH * 16));
@@ -741,10 +744,10 @@ __device__ __forceinline__ void load_row32(const T *__restrict__ base, uint32_t 
 // converts them where they are used, after the wait (bf16 to f32 costs a shift or a mask per element).
 template <typename T, int H, int D> struct RawRow { uint32_t w[Lay<T, H, D>::EPL * sizeof(T) / 4]; };
 
-template <typename T, int H, int D>
+template <typename T, int H, int D, int PITCH = Lay<T, H, D>::C>
 __device__ __forceinline__ void load_row32_raw(const T *__restrict__ base, uint32_t row, uint32_t loff, RawRow<T, H, D> &out) {
     using L = Lay<T, H, D>;
-    const char *p = reinterpret_cast<const char *>(base) + (size_t)(row * (uint32_t)(L::C * sizeof(T)));
+    const char *p = reinterpret_cast<const char *>(base) + (size_t)(row * (uint32_t)(PITCH * sizeof(T)));
 #pragma unroll
     for (int i = 0; i < L::NV; ++i) {
         const uint4 v = *reinterpret_cast<const uint4 *>(p + (size_t)(loff + (uint32_t)(i * L::LPH * 16)));
@@ -809,20 +812,22 @@ __device__ __forceinline__ float max3f(float a, float b, float c) {
 
 // Forward: online softmax in base 2 over the group's entries, two entries per step.  The members' q rows
 // (pre-scaled) live in LDS and are re-read for every use, which keeps the kernel at three wavefronts per SIMD.
-template <typename T, int H, int D, int R>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H, D>::EPL, R>()))) void k_attn_fwd_grp(
+template <typename T, int H, int D, int R, int HS>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_attn_fwd_grp(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
     float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
-    using L = Lay<T, H, D>;
+    constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
+    using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
-    static_assert(R % 4 == 0 && R <= 2 * L::LPH, "members are handled in quads inside the lanes of one head");
+    static_assert(H % HS == 0 && R % 4 == 0 && L::LPH >= 4, "members are handled in quads inside the lanes of one head");
     GroupHead<R> gh;
-    if (!fetch_group<R>(P, gh)) return;
-    const int lane = threadIdx.x, head = lane / L::LPH;
-    const uint32_t loff = (uint32_t)(L::off(lane, 0) * sizeof(T));
+    if (!fetch_group<R, HS>(P, gh)) return;
+    const int slice = group_slice<R, HS>(), coff = slice * HL * D;
+    const int lane = threadIdx.x, head = slice * HL + lane / L::LPH;
+    const uint32_t loff = (uint32_t)((coff + L::off(lane, 0)) * sizeof(T));
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     struct Batch {
-        RawRow<T, H, D> kr[GRP_BATCH], vr[GRP_BATCH];
+        RawRow<T, HL, D> kr[GRP_BATCH], vr[GRP_BATCH];
         int mk[GRP_BATCH];
     };
     struct Rows {
@@ -834,7 +839,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 #pragma unroll
     for (int m = 0; m < R; ++m) {
         float qr[EPL];
-        load_row32<T, H, D>(q, (uint32_t)max(gh.rows[m], 0), loff, qr);
+        load_row32<T, HL, D, CF>(q, (uint32_t)max(gh.rows[m], 0), loff, qr);
         mrun[m] = M_INIT_LOG2;
         lrun[m] = 0.f;
 #pragma unroll
@@ -851,8 +856,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             for (int e = 0; e < GRP_BATCH; ++e) {
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
-                load_row32_raw<T, H, D>(k, src, loff, B.kr[e]);
-                load_row32_raw<T, H, D>(v, src, loff, B.vr[e]);
+                load_row32_raw<T, HL, D, CF>(k, src, loff, B.kr[e]);
+                load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
             }
         };
         auto one = [&](int m, const float (&kr)[EPL], const float (&vr)[EPL]) {
@@ -870,8 +875,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             Rows B;
 #pragma unroll
             for (int e = 0; e < GRP_BATCH; ++e) {
-                unpack_row<T, H, D>(raw.kr[e], B.kv[e]);
-                unpack_row<T, H, D>(raw.vr[e], B.vv[e]);
+                unpack_row<T, HL, D>(raw.kr[e], B.kv[e]);
+                unpack_row<T, HL, D>(raw.vr[e], B.vv[e]);
                 B.mk[e] = raw.mk[e];
             }
 #pragma unroll
@@ -921,10 +926,10 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             const float inv = lrun[m] > 0.f ? 1.f / lrun[m] : 0.f;
 #pragma unroll
             for (int i = 0; i < EPL; ++i) acc[m][i] *= inv;
-            store_row<T, H, D>(o + (size_t)gh.rows[m] * L::C, lane, acc[m]);
+            store_row<T, HL, D>(o + (size_t)gh.rows[m] * CF + coff, lane, acc[m]);
             if (lane % L::LPH == 0) lse[(size_t)gh.rows[m] * H + head] = lrun[m] > 0.f ? mrun[m] + log2f(lrun[m]) : 0.f;
         } else {
-            store_row_ws<T, H, D>(ws_acc + (size_t)gh.slots[m] * L::C, lane, acc[m]);
+            store_row_ws<T, HL, D>(ws_acc + (size_t)gh.slots[m] * CF + coff, lane, acc[m]);
             if (lane % L::LPH == 0) {
                 ws_ml[((size_t)gh.slots[m] * H + head) * 2] = mrun[m];
                 ws_ml[((size_t)gh.slots[m] * H + head) * 2 + 1] = lrun[m];
@@ -938,23 +943,25 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 // (entry, member) of this plan (a spare position for members the entry does not have).  One store per
 // entry and quad of members: lane l carries the pair of member 4c + l % 4; the same register of ds values is
 // the A operand of the MFMA that accumulates dq.  The members' q rows live in LDS.
-template <typename T, int H, int D, int R>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H, D>::EPL, R>()))) void k_attn_bwd_dst_grp(
+template <typename T, int H, int D, int R, int HS>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_attn_bwd_dst_grp(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
     const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
     float *__restrict__ ws_dq, float scale, float scale_log2e) {
-    using L = Lay<T, H, D>;
+    constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
+    using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
-    static_assert(R % 4 == 0 && R <= 2 * L::LPH, "members are handled in quads inside the lanes of one head");
+    static_assert(H % HS == 0 && R % 4 == 0 && L::LPH >= 4, "members are handled in quads inside the lanes of one head");
     GroupHead<R> gh;
-    if (!fetch_group<R>(P, gh)) return;
-    const int lane = threadIdx.x, head = lane / L::LPH;
-    const uint32_t loff = (uint32_t)(L::off(lane, 0) * sizeof(T));
+    if (!fetch_group<R, HS>(P, gh)) return;
+    const int slice = group_slice<R, HS>(), coff = slice * HL * D;
+    const int lane = threadIdx.x, head = slice * HL + lane / L::LPH;
+    const uint32_t loff = (uint32_t)((coff + L::off(lane, 0)) * sizeof(T));
     const int mine = lane & 3;
     const uint32_t hoff = (uint32_t)head * 8u, poff = (uint32_t)mine * 4u;
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     struct Batch {
-        RawRow<T, H, D> kr[GRP_BATCH], vr[GRP_BATCH];
+        RawRow<T, HL, D> kr[GRP_BATCH], vr[GRP_BATCH];
         int mk[GRP_BATCH], xp[GRP_BATCH][NQ];
     };
     __shared__ float4 q_lds[R * (EPL / 4) * WAVE];
@@ -964,9 +971,9 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
     for (int m = 0; m < R; ++m) {
         const uint32_t row = (uint32_t)max(gh.rows[m], 0);
         float ov[EPL], qr[EPL];
-        load_row32<T, H, D>(o, row, loff, ov);
-        load_row32<T, H, D>(d_o, row, loff, dov[m]);
-        load_row32<T, H, D>(q, row, loff, qr);
+        load_row32<T, HL, D, CF>(o, row, loff, ov);
+        load_row32<T, HL, D, CF>(d_o, row, loff, dov[m]);
+        load_row32<T, HL, D, CF>(q, row, loff, qr);
         lds_put_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qr);
         delta_s[m] = head_sum<L::LPH>(dot_n<EPL>(dov[m], ov)) * scale;
         lse2[m] = lse[(size_t)row * H + head];
@@ -989,16 +996,16 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                 const char *pp = reinterpret_cast<const char *>(P.grp_pairs) + (size_t)((uint32_t)(p0 + b + e) * (uint32_t)(R * 4));
 #pragma unroll
                 for (int c = 0; c < NQ; ++c) B.xp[e][c] = *reinterpret_cast<const int *>(pp + (size_t)(poff + (uint32_t)(c * 16)));
-                load_row32_raw<T, H, D>(k, src, loff, B.kr[e]);
-                load_row32_raw<T, H, D>(v, src, loff, B.vr[e]);
+                load_row32_raw<T, HL, D, CF>(k, src, loff, B.kr[e]);
+                load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
             }
         };
         auto compute = [&](const Batch &B) {
 #pragma unroll
             for (int e = 0; e < GRP_BATCH; ++e) {
                 float kv[EPL], vv[EPL];
-                unpack_row<T, H, D>(B.kr[e], kv);
-                unpack_row<T, H, D>(B.vr[e], vv);
+                unpack_row<T, HL, D>(B.kr[e], kv);
+                unpack_row<T, HL, D>(B.vr[e], vv);
                 float wp[NQ], wd[NQ];
 #pragma unroll
                 for (int c = 0; c < NQ; ++c) { wp[c] = 0.f; wd[c] = 0.f; }
@@ -1049,8 +1056,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
         float rq[EPL];
 #pragma unroll
         for (int t = 0; t < EPL; ++t) rq[t] = dqa[m / 4][t][m & 3];
-        if (gh.slots[m] < 0) store_row<T, H, D>(dq + (size_t)gh.rows[m] * L::C, lane, rq);
-        else store_row_ws<T, H, D>(ws_dq + (size_t)gh.slots[m] * L::C, lane, rq);
+        if (gh.slots[m] < 0) store_row<T, HL, D>(dq + (size_t)gh.rows[m] * CF + coff, lane, rq);
+        else store_row_ws<T, HL, D>(ws_dq + (size_t)gh.slots[m] * CF + coff, lane, rq);
     }
 }
 
@@ -1060,21 +1067,23 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 // v_mfma_f32_4x4x1 (16 blocks of 4 lanes: A_b[i] in lane 4b+i, B_b[j] in lane 4b+j, D_b[i][j] in register i
 // of lane 4b+j): with a register of the entry's row as B, one instruction adds weight[member i] * row[..]
 // to that register's slice of all four members' accumulators (register i of the result = member i).
-template <typename T, int H, int D, int R>
-__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H, D>::EPL, R>()))) void k_attn_bwd_src_grp(
+template <typename T, int H, int D, int R, int HS>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_attn_bwd_src_grp(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o, const float2 *__restrict__ pds, T *__restrict__ dk,
     T *__restrict__ dv, float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
-    using L = Lay<T, H, D>;
+    constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
+    using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
-    static_assert(R % 4 == 0 && R <= 2 * L::LPH, "members are handled in quads inside the lanes of one head");
+    static_assert(H % HS == 0 && R % 4 == 0 && L::LPH >= 4, "members are handled in quads inside the lanes of one head");
     GroupHead<R> gh;
-    if (!fetch_group<R>(P, gh)) return;
-    const int lane = threadIdx.x, head = lane / L::LPH;
-    const uint32_t loff = (uint32_t)(L::off(lane, 0) * sizeof(T));
+    if (!fetch_group<R, HS>(P, gh)) return;
+    const int slice = group_slice<R, HS>(), coff = slice * HL * D;
+    const int lane = threadIdx.x, head = slice * HL + lane / L::LPH;
+    const uint32_t loff = (uint32_t)((coff + L::off(lane, 0)) * sizeof(T));
     const uint32_t woff = (uint32_t)(((lane & 3) * H + head) * 8);
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     struct Batch {
-        RawRow<T, H, D> qr[GRP_BATCH], dr[GRP_BATCH];
+        RawRow<T, HL, D> qr[GRP_BATCH], dr[GRP_BATCH];
         float2 w[GRP_BATCH][NQ];
         int mk[GRP_BATCH];
     };
@@ -1093,8 +1102,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             for (int e = 0; e < GRP_BATCH; ++e) {
                 const uint32_t dst = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
-                load_row32_raw<T, H, D>(q, dst, loff, B.qr[e]);
-                load_row32_raw<T, H, D>(d_o, dst, loff, B.dr[e]);
+                load_row32_raw<T, HL, D, CF>(q, dst, loff, B.qr[e]);
+                load_row32_raw<T, HL, D, CF>(d_o, dst, loff, B.dr[e]);
                 // the entry's R pairs, present or not (absent ones are zeroed before use)
                 const char *pw = reinterpret_cast<const char *>(pds) + (size_t)((uint32_t)(p0 + b + e) * (uint32_t)(R * H * 8));
 #pragma unroll
@@ -1105,8 +1114,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 #pragma unroll
             for (int e = 0; e < GRP_BATCH; ++e) {
                 float qv[EPL], dv_[EPL];
-                unpack_row<T, H, D>(B.qr[e], qv);
-                unpack_row<T, H, D>(B.dr[e], dv_);
+                unpack_row<T, HL, D>(B.qr[e], qv);
+                unpack_row<T, HL, D>(B.dr[e], dv_);
 #pragma unroll
                 for (int c = 0; c < NQ; ++c) {
                     if ((B.mk[e] >> (4 * c)) & 15) {
@@ -1146,11 +1155,11 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 #pragma unroll
         for (int t = 0; t < EPL; ++t) { rk[t] = ak[m / 4][t][m & 3]; rv[t] = av[m / 4][t][m & 3]; }
         if (gh.slots[m] < 0) {
-            store_row<T, H, D>(dk + (size_t)gh.rows[m] * L::C, lane, rk);
-            store_row<T, H, D>(dv + (size_t)gh.rows[m] * L::C, lane, rv);
+            store_row<T, HL, D>(dk + (size_t)gh.rows[m] * CF + coff, lane, rk);
+            store_row<T, HL, D>(dv + (size_t)gh.rows[m] * CF + coff, lane, rv);
         } else {
-            store_row_ws<T, H, D>(ws_dk + (size_t)gh.slots[m] * L::C, lane, rk);
-            store_row_ws<T, H, D>(ws_dv + (size_t)gh.slots[m] * L::C, lane, rv);
+            store_row_ws<T, HL, D>(ws_dk + (size_t)gh.slots[m] * CF + coff, lane, rk);
+            store_row_ws<T, HL, D>(ws_dv + (size_t)gh.slots[m] * CF + coff, lane, rv);
         }
     }
 }
@@ -1328,11 +1337,19 @@ inline bool fits32(int64_t n, int64_t unit) { return n >= 0 && n <= (int64_t)0xf
 
 inline int group_grid(const bpt_plan *P) { return (int)(8 * P->grp_max_chunk); }
 
-// rows per group the row-group kernels exist for, given the elements a lane holds per row
-inline bool group_rows_ok(int64_t R, int h, int d) { return R == 4 || (R == 8 && h <= 8 && h * d <= 512); }
+// The row-group kernels split a group's heads over wavefronts so that one wavefront handles at most 512 columns of
+// every row (8 registers per lane and row: the members' state has to fit the register file).  Slices of 256
+// float32 columns were also measured: faster on small graphs, slower at the benchmark sizes.
+template <typename T, int H, int D> constexpr int head_slices() {
+    constexpr int CS = 512, C = H * D;
+    return (C > CS && C % CS == 0 && H % (C / CS) == 0) ? C / CS : 1;
+}
+
+// rows per group the row-group kernels exist for
+inline bool group_rows_ok(int64_t R) { return R == 4 || R == 8; }
 
 inline bool has_groups(const bpt_plan *P, int h, int d, size_t elem) {
-    return P->n_groups > 0 && group_rows_ok(P->grp_R, h, d) && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
+    return P->n_groups > 0 && group_rows_ok(P->grp_R) && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
            P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups && P->n_grp_entries >= 0 &&
            fits32(P->n_rows, (int64_t)h * d * (int64_t)elem) &&
            fits32((P->n_grp_entries + GRP_PAD_ENTRIES) * P->grp_R, (int64_t)h * 8);
@@ -1358,15 +1375,12 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
         if (has_groups(P, H, D, sizeof(T))) {
-#define LAUNCH_FWD(RR)                                                                                              \
-    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR>), dim3(group_grid(P)), dim3(WAVE), 0, s, *P, (const T *)q, \
+#define LAUNCH_FWD(RR)                                                                                                   \
+    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR, HS>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)q, \
                        (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E)
-            if constexpr (H <= 8 && H * D <= 512) {
-                if (P->grp_R == 8) LAUNCH_FWD(8);
-                else LAUNCH_FWD(4);
-            } else {
-                LAUNCH_FWD(4);
-            }
+            constexpr int HS = head_slices<T, H, D>();
+            if (P->grp_R == 8) LAUNCH_FWD(8);
+            else LAUNCH_FWD(4);
 #undef LAUNCH_FWD
         } else {
             hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
@@ -1393,15 +1407,12 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
         if (grouped) {
-#define LAUNCH_DST(RR)                                                                                                        \
-    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, RR>), dim3(group_grid(Pin)), dim3(WAVE), 0, s, *Pin, (const T *)q,   \
+#define LAUNCH_DST(RR)                                                                                                             \
+    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, RR, HS>), dim3(group_grid(Pin) * HS), dim3(WAVE), 0, s, *Pin, (const T *)q,   \
                        (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E)
-            if constexpr (H <= 8 && H * D <= 512) {
-                if (Pin->grp_R == 8) LAUNCH_DST(8);
-                else LAUNCH_DST(4);
-            } else {
-                LAUNCH_DST(4);
-            }
+            constexpr int HS = head_slices<T, H, D>();
+            if (Pin->grp_R == 8) LAUNCH_DST(8);
+            else LAUNCH_DST(4);
 #undef LAUNCH_DST
         } else {
             hipLaunchKernelGGL((k_attn_bwd_dst<T, H, D, FAST_BATCH>), dim3(grid_for(Pin)), dim3(BLOCK), 0, s, *Pin, (const T *)q,
@@ -1425,15 +1436,12 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     float *ws_dk = ws_rows, *ws_dv = ws_rows + (size_t)Pout->n_slots * H * D;
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
-#define LAUNCH_SRC(RR)                                                                                                       \
-    hipLaunchKernelGGL((k_attn_bwd_src_grp<T, H, D, RR>), dim3(group_grid(Pout)), dim3(WAVE), 0, s, *Pout, (const T *)q, \
+#define LAUNCH_SRC(RR)                                                                                                            \
+    hipLaunchKernelGGL((k_attn_bwd_src_grp<T, H, D, RR, HS>), dim3(group_grid(Pout) * HS), dim3(WAVE), 0, s, *Pout, (const T *)q, \
                        (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv)
-        if constexpr (H <= 8 && H * D <= 512) {
-            if (Pout->grp_R == 8) LAUNCH_SRC(8);
-            else LAUNCH_SRC(4);
-        } else {
-            LAUNCH_SRC(4);
-        }
+        constexpr int HS = head_slices<T, H, D>();
+        if (Pout->grp_R == 8) LAUNCH_SRC(8);
+        else LAUNCH_SRC(4);
 #undef LAUNCH_SRC
     }
     st = launch_status();

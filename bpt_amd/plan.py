@@ -16,7 +16,8 @@ import torch
 
 from ._lib import PlanInfo, PlanStruct, check_graph, graph_lib
 
-DEFAULT_SEG_LEN = 64
+DEFAULT_SEG_LEN = None  # edges per work item: None = chosen per plan by auto_seg_len
+FORCE_SEG_LEN = None    # testing hook: when set, replaces the automatic choice for plans built from now on
 GROUP_R = 4            # default rows per group (the row-group kernels exist for 4 and, float32 with h <= 8 and h*d <= 512, 8)
 GROUP_WINDOW = 32      # how many following items the greedy grouping examines per group
 GROUP_ORDER = 2 + 4    # groups inside an XCD chunk by decreasing work (2); entries of a group sorted by member mask (+4)
@@ -37,12 +38,32 @@ def _host_i64(t):
     return np.ascontiguousarray(t, dtype=np.int64)
 
 
+def auto_seg_len(row, indptr, n_rows):
+    """Edges per work item.  Rows longer than this are cut into segments whose partial results cost a workspace
+    round trip and a combine pass, so on graphs with enough rows to keep every wavefront slot of the GPU busy
+    with whole rows (8 rows per slot) it is the smallest of 64, 128, 256 that leaves 90 % of the non-empty rows
+    whole; on smaller graphs the extra wavefronts that segments of 64 provide are worth more (both measured)."""
+    if len(row) == 0 or n_rows < 8 * 3072:
+        return 64
+    r = np.asarray(row)
+    if r.min() < 0 or r.max() >= max(n_rows, 1):
+        return 64                                   # malformed: the C validation reports it
+    deg = np.bincount(r, weights=np.diff(np.asarray(indptr)).astype(np.float64), minlength=max(n_rows, 1))
+    deg = deg[deg > 0]
+    if len(deg) == 0:
+        return 64
+    q90 = float(np.quantile(deg, 0.9))
+    return 64 if q90 <= 64 else (128 if q90 <= 128 else 256)
+
+
 def build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len=DEFAULT_SEG_LEN):
     """Pure host step (no GPU): returns (arrays, info) with arrays = dict of int32 numpy arrays
     rowptr, idx, eid, items (n_items, 4), heavy (n_heavy, 3).  Raises ValueError on malformed input."""
     row, indptr, eid, indices = map(_host_i64, (row, indptr, eid, indices))
     if len(indptr) != len(row) + 1:
         raise ValueError("indptr must have len(row) + 1 entries")
+    if seg_len is None:
+        seg_len = FORCE_SEG_LEN if FORCE_SEG_LEN is not None else auto_seg_len(row, indptr, int(n_rows))
     if indices is not None and len(indices) != len(eid):
         raise ValueError("indices and eid must have the same length")
     lib = graph_lib()
