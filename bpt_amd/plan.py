@@ -81,6 +81,7 @@ def build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len=DE
                                    int(n_rows), int(n_index_nodes), int(seg_len),
                                    _ptr(arrays["rowptr"]), _ptr(arrays["idx"]), _ptr(arrays["eid"]),
                                    _ptr(arrays["items"]), _ptr(arrays["heavy"]), ctypes.byref(info)))
+    arrays["seg_len"] = int(seg_len)
     return arrays, info
 
 
@@ -91,8 +92,8 @@ def build_groups_host(arrays, n_index_nodes, R=None, window=GROUP_WINDOW, order_
     mask has no such member."""
     order_mode = GROUP_ORDER if order_mode is None else order_mode
     R = GROUP_R if R is None else R
-    if max_pairs is None:
-        max_pairs = 48 * R if GROUP_MAX_PAIRS is None else GROUP_MAX_PAIRS
+    if max_pairs is None:      # 48 edges per member row, more where the work items themselves are longer than 64 edges
+        max_pairs = 48 * R * max(1, arrays.get("seg_len", 64) // 64) if GROUP_MAX_PAIRS is None else GROUP_MAX_PAIRS
     items = np.ascontiguousarray(arrays["items"], dtype=np.int32)
     idx = np.ascontiguousarray(arrays["idx"], dtype=np.int32)
     eid = np.ascontiguousarray(arrays["eid"], dtype=np.int32)
@@ -152,7 +153,8 @@ class Plan:
         self._links = {}
         self._lock = threading.Lock()
         # one allocation, 256-byte aligned sections (the items array is read as 16-byte vectors)
-        self._dev = {k: torch.from_numpy(v).to(self.device) for k, v in arrays.items()}
+        self.seg_len = arrays["seg_len"]
+        self._dev = {k: torch.from_numpy(v).to(self.device) for k, v in arrays.items() if isinstance(v, np.ndarray)}
         d = self._dev
         self.struct = PlanStruct(
             d["rowptr"].data_ptr(), d["idx"].data_ptr() if self.n_edges else None,
