@@ -104,6 +104,8 @@ def main():
     ap.add_argument("--group-rows", type=int, default=None, choices=[4, 8], help="rows per wavefront group of the fused kernels (default: 8 where available, else 4)")
     ap.add_argument("--rows", action="store_true", help="fused kernels with one wavefront per row (no row groups)")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
+    ap.add_argument("--block-layers", type=int, default=0,
+                    help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the workload's graph")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -222,6 +224,30 @@ def main():
             b.copy_(a)                    # reads 256 MiB and writes 256 MiB per launch
         torch.cuda.synchronize()
 
+    block = None
+    if args.block_layers > 0 and not args.unfused:
+        # the reference's layer (modules/attention.py:22-81) around the attention core, dropout off, no rel_pos
+        from bpt_amd.block import BPTBlock
+        dm = H * D
+        csr_dev = (tuple(t.to(dev) for t in out_csr), tuple(t.to(dev) for t in in_csr), *(x.to(dev) for x in (ROW, IR, COL, IC)))
+        torch.manual_seed(2345)
+        layers = torch.nn.ModuleList([BPTBlock(dm, H, 4 * dm, rel_pos=False, drop_h=0.0, drop_a=0.0) for _ in range(args.block_layers)])
+        layers = layers.to(dev).to(tdtype)
+        h0 = (torch.randn(N, dm, generator=torch.Generator().manual_seed(1)) / 8).to(tdtype).to(dev).requires_grad_(True)
+        gh = (torch.randn(N, dm, generator=torch.Generator().manual_seed(2)) / 8).to(tdtype).to(dev)
+
+        def stack_step():
+            x = h0
+            for blk in layers:
+                x = blk(x, csr_dev)
+            x.backward(gh)
+            return x
+
+        t_stack = timed(stack_step, max(5, min(args.steps, 30)), 3)
+        block = {"layers": args.block_layers, "d_model": dm, "d_ff": 4 * dm, "ms_per_layer_fwd_bwd": round(t_stack / args.block_layers * 1e3, 4),
+                 "attention_ms_per_layer": round(t_step * 1e3, 4), "attention_share": round(t_step * args.block_layers / t_stack, 3)}
+        log(f"block stack: {block}")
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(src, dst, N, H, D, 2345)
@@ -243,6 +269,8 @@ def main():
         "ms_per_step_graph": None if t_graph_replay is None else t_graph_replay * 1e3,
         "kernel_ms": {k_: round(v_, 5) for k_, v_ in kernels.items()},
     }
+    if block is not None:
+        out["block_stack"] = block
     log(json.dumps(out, indent=1))
     print(json.dumps(out), flush=True)
 

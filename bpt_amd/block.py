@@ -1,0 +1,85 @@
+"""The transformer block of the reference (modules/attention.py:22-81) on the HIP attention kernels.
+
+Same sub-modules, parameter names and initialisation as the reference's `BPTBlock`, so its
+`state_dict` loads here unchanged: `norm_in`, `norm_inter`, `proj_q/k/v/o` (bias-free), `embed_ak`
+(when `rel_pos`), `ffn.0.w_1`, `ffn.0.w_2`.  The reference keeps node features and edge types in a
+DGL graph object (`g.ndata['h']`, `g.edata['etype']`) and writes the result back into it; here
+`forward(h, csr, etype)` takes and returns plain tensors, `csr` being the 6-tuple that
+`graph/base.py:71-86` (`bpt_amd.graphbuilder.get_csrs`) produces.
+
+Attention core: with `rel_pos` off and no attention dropout in effect the fused kernels run
+(`op.bpt_attention`); otherwise the four operators are composed exactly as attention.py:66-77 does.
+Projections, LayerNorm and the feed-forward are torch modules (rocBLAS GEMMs).
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+from .op import bpt_attention, masked_mm, node_mul_edge, sparse_softmax, vec_spmm
+
+__all__ = ["PositionwiseFeedForward", "BPTBlock"]
+
+
+class PositionwiseFeedForward(nn.Module):
+    """FFN(x) = max(0, x W_1 + b_1) W_2 + b_2   (modules/attention.py:8-19)"""
+
+    def __init__(self, dim_model, dim_ff, dropout=0.1):
+        super().__init__()
+        self.w_1 = nn.Linear(dim_model, dim_ff)
+        self.w_2 = nn.Linear(dim_ff, dim_model)
+        self.dropout = nn.Dropout(dropout)
+
+    def forward(self, x):
+        return self.w_2(self.dropout(torch.relu(self.w_1(x))))
+
+
+class BPTBlock(nn.Module):
+    MAX_ETYPE = 1000        # modules/attention.py:23
+
+    def __init__(self, dim_model, h, dim_ff, rel_pos=False, drop_h=0.1, drop_a=0.1):
+        super().__init__()
+        self.dim_model, self.h, self.dim_ff = dim_model, h, dim_ff
+        self.d_k = dim_model // h
+        self.rel_pos = rel_pos
+        self.drop_h = nn.Dropout(drop_h)
+        self.drop_att = nn.Dropout(drop_a)
+        self.norm_in = nn.LayerNorm(dim_model)
+        self.norm_inter = nn.LayerNorm(dim_model)
+        self.proj_q = nn.Linear(dim_model, self.d_k * h, bias=False)
+        self.proj_k = nn.Linear(dim_model, self.d_k * h, bias=False)
+        self.proj_v = nn.Linear(dim_model, self.d_k * h, bias=False)
+        self.proj_o = nn.Linear(self.d_k * h, dim_model, bias=False)
+        if rel_pos:
+            self.embed_ak = nn.Embedding(self.MAX_ETYPE, self.d_k)
+        self.ffn = nn.Sequential(PositionwiseFeedForward(dim_model, dim_ff, dropout=drop_h), nn.Dropout(drop_h))
+
+    def reset_parameters(self):
+        # modules/attention.py:49-52
+        for p in self.parameters():
+            if p.dim() > 1:
+                nn.init.xavier_uniform_(p)
+
+    def attention(self, q, k, v, csr, etype=None):
+        """attention.py:66-77: (n, h, d_k) q, k, v -> (n, h * d_k)."""
+        out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C = csr
+        graph = (ROW, INDPTR_R, out_csr[2], out_csr[1], COL, INDPTR_C, in_csr[2], in_csr[1])
+        att_dropout = self.training and self.drop_att.p > 0
+        if not self.rel_pos and not att_dropout:
+            return bpt_attention(*graph, q, k, v).view(-1, self.d_k * self.h)
+        e = masked_mm(*graph, k, q)
+        if self.rel_pos:
+            if etype is None:
+                raise ValueError("rel_pos=True needs the edge types (etype)")
+            e = e + node_mul_edge(COL, INDPTR_C, in_csr[2], q, self.embed_ak(etype))
+        e = self.drop_att(sparse_softmax(COL, INDPTR_C, in_csr[2], e / math.sqrt(self.d_k)))
+        return vec_spmm(COL, INDPTR_C, in_csr[2], in_csr[1], ROW, INDPTR_R, out_csr[2], out_csr[1], e, v).view(
+            -1, self.d_k * self.h)
+
+    def forward(self, h, csr, etype=None):
+        q = self.proj_q(h).view(-1, self.h, self.d_k)
+        k = self.proj_k(h).view(-1, self.h, self.d_k)
+        v = self.proj_v(h).view(-1, self.h, self.d_k)
+        a = self.attention(q, k, v, csr, etype)
+        h = self.norm_in(h + self.drop_h(self.proj_o(a)))
+        return self.norm_inter(h + self.ffn(h))
