@@ -104,6 +104,8 @@ def main():
     ap.add_argument("--group-rows", type=int, default=None, choices=[4, 8], help="rows per wavefront group of the fused kernels (default: 8 where available, else 4)")
     ap.add_argument("--rows", action="store_true", help="fused kernels with one wavefront per row (no row groups)")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
+    ap.add_argument("--rel-pos", action="store_true",
+                    help="add the relative-position score term q[dst].table[etype[e]] (table (1000, d_head), modules/attention.py:23,42,69-71)")
     ap.add_argument("--block-layers", type=int, default=0,
                     help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the workload's graph")
     args = ap.parse_args()
@@ -126,7 +128,7 @@ def main():
     esize = {"f32": 4, "bf16": 2}[dtype_name]
 
     t0 = time.perf_counter()
-    src, dst, _, _, N = gb.merge_graphs(graphs)
+    src, dst, etype, _, N = gb.merge_graphs(graphs)
     E = len(src)
     out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, N)
     t_graph = time.perf_counter() - t0
@@ -135,7 +137,21 @@ def main():
     q, k, v, do = ((torch.randn(N, H, D, generator=gen) / 8).to(tdtype).to(dev) for _ in range(4))
     log(f"{desc}: N={N} E={E} dtype={dtype_name}; host graph+CSR build {t_graph * 1e3:.1f} ms")
 
-    if args.unfused:
+    if args.rel_pos:
+        # the op sequence of modules/attention.py:66-77 with rel_pos on; the (E, d) rows of the table are
+        # gathered per step as the reference's nn.Embedding does
+        from bpt_amd import op
+        table = (torch.randn(1000, D, generator=gen) / 8).to(tdtype).to(dev)
+        et = torch.from_numpy(np.asarray(etype, dtype=np.int64)).to(dev)
+
+        def step():
+            qq, kk, vv, tt = (x.detach().requires_grad_(True) for x in (q, k, v, table))
+            e = op.masked_mm(*gargs, kk, qq) + op.node_mul_edge(*gargs[4:7], qq, torch.nn.functional.embedding(et, tt))
+            a = op.sparse_softmax(*gargs[4:7], e / math.sqrt(D))
+            o = op.vec_spmm(*gargs[4:], *gargs[:4], a, vv)
+            o.backward(do)
+            return o, qq.grad, kk.grad, vv.grad
+    elif args.unfused:
         from bpt_amd import op
 
         def step():
@@ -165,7 +181,7 @@ def main():
     t_eager = timed(step, args.steps, args.warmup)
     t_step, mode = t_eager, "eager"
     t_graph_replay = None
-    if not args.no_graph and not args.unfused:
+    if not args.no_graph and not args.unfused and not args.rel_pos:
         try:
             side = torch.cuda.Stream()
             with torch.cuda.stream(side):
@@ -191,7 +207,7 @@ def main():
     # ---- per-kernel durations, HIP events recorded by the library around the kernel on its launch stream
     lib = attn_lib()
     kernels = {}
-    if not args.unfused:
+    if not args.unfused and not args.rel_pos:
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record(); ev1.record(); torch.cuda.synchronize()
         for which, name in ((1, "attn_fwd"), (2, "attn_bwd_dst"), (3, "attn_bwd_src")):
@@ -258,7 +274,7 @@ def main():
         "value": E / t_step, "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype_name, "data": "synthetic",
-        "config": {"workload": desc + (" (unfused op chain)" if args.unfused else " (fused fwd+bwd)"), "n_nodes": N,
+        "config": {"workload": desc + (" (op chain with rel_pos)" if args.rel_pos else " (unfused op chain)" if args.unfused else " (fused fwd+bwd)"), "n_nodes": N,
                    "n_edges": E, "heads": H, "d_head": D, "launch": mode,
                    "kernels": "per-row" if args.rows else f"row-groups({args.group_rows or 'auto'} rows per wavefront)"},
         "roofline": roofline,

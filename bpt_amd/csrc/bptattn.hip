@@ -303,6 +303,148 @@ __global__ __launch_bounds__(BLOCK) void k_softmax_bwd(bpt_plan P, const T *__re
     }
 }
 
+// Row softmax with the heads side by side: thread t handles head t % H of edge slot t / H, so a wavefront reads
+// 64 / H whole (E, H) rows per step (H must divide 64).  NW == 1: one wavefront per whole-row item; NW > 1: one
+// block of NW wavefronts per split row (grid = n_heavy).  Rows of up to SM_CACHE steps keep their values in
+// registers and read memory once; longer rows re-read.  Loads are issued SM_CACHE at a time.
+constexpr int SM_CACHE = 8;
+constexpr int SM_HEAVY_WAVES = 16;
+
+// reduction over the threads of a block that share t % H (H divides 64): first inside each wavefront, then over LDS
+template <typename A, int NW, bool IS_MAX> __device__ __forceinline__ A head_reduce(A x, int H, int h, A *smem) {
+    for (int off = H; off < WAVE; off <<= 1) {
+        const A o = __shfl_xor(x, off);
+        x = IS_MAX ? (x > o ? x : o) : x + o;
+    }
+    if (NW == 1) return x;
+    const int w = threadIdx.x >> 6;
+    __syncthreads();                       // smem may still be read from the previous reduction
+    if ((int)(threadIdx.x & 63) < H) smem[w * WAVE + h] = x;
+    __syncthreads();
+    A r = smem[h];
+    for (int i = 1; i < NW; ++i) r = IS_MAX ? (r > smem[i * WAVE + h] ? r : smem[i * WAVE + h]) : r + smem[i * WAVE + h];
+    return r;
+}
+
+template <int NW> __device__ __forceinline__ bool softmax_range(const bpt_plan &P, int &begin, int &end) {
+    if (NW == 1) {
+        Item it;
+        if (!fetch_item(P, it) || it.slot >= 0) return false;
+        begin = it.begin; end = it.end;
+    } else {
+        const int row = P.heavy[3 * blockIdx.x];
+        begin = P.rowptr[row]; end = P.rowptr[row + 1];
+    }
+    return true;
+}
+
+template <typename T, int NW>
+__global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_fwd_heads(bpt_plan P, const T *__restrict__ x, T *__restrict__ y, int H) {
+    using acc_t = typename Elem<T>::acc_t;
+    __shared__ acc_t smem[NW == 1 ? 1 : NW * WAVE];
+    int begin, end;
+    if (!softmax_range<NW>(P, begin, end)) return;
+    const int tid = NW == 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
+    const int h = tid % H, slot = tid / H, nslots = NW * WAVE / H;
+    const bool cached = end - begin <= SM_CACHE * nslots;
+    acc_t vc[SM_CACHE];
+    size_t oc[SM_CACHE];
+#pragma unroll
+    for (int u = 0; u < SM_CACHE; ++u) { vc[u] = (acc_t)-INFINITY; oc[u] = (size_t)-1; }    // threads past a short row's end
+    acc_t m = (acc_t)-1e9;
+    for (int p0 = begin + slot; p0 < end; p0 += SM_CACHE * nslots) {
+        int e[SM_CACHE];
+#pragma unroll
+        for (int u = 0; u < SM_CACHE; ++u) { const int p = p0 + u * nslots; e[u] = p < end ? P.eid[p] : -1; }
+#pragma unroll
+        for (int u = 0; u < SM_CACHE; ++u) {
+            oc[u] = (size_t)(e[u] < 0 ? 0 : e[u]) * H + h;
+            vc[u] = e[u] < 0 ? (acc_t)-INFINITY : (acc_t)Elem<T>::ld(x + oc[u]);
+            m = vc[u] > m ? vc[u] : m;
+            if (e[u] < 0) oc[u] = (size_t)-1;
+        }
+    }
+    m = head_reduce<acc_t, NW, true>(m, H, h, smem);
+    acc_t s = 0;
+    if (cached) {
+#pragma unroll
+        for (int u = 0; u < SM_CACHE; ++u) { vc[u] = exp_acc(vc[u] - m); s += vc[u]; }      // exp(-inf) = 0 for the empty slots
+    } else {
+        for (int p = begin + slot; p < end; p += nslots) s += exp_acc((acc_t)Elem<T>::ld(x + (size_t)P.eid[p] * H + h) - m);
+    }
+    s = head_reduce<acc_t, NW, false>(s, H, h, smem);
+    if (cached) {
+#pragma unroll
+        for (int u = 0; u < SM_CACHE; ++u)
+            if (oc[u] != (size_t)-1) Elem<T>::st(y + oc[u], vc[u] / s);
+    } else {
+        for (int p0 = begin + slot; p0 < end; p0 += SM_CACHE * nslots) {
+            int e[SM_CACHE];
+#pragma unroll
+            for (int u = 0; u < SM_CACHE; ++u) { const int p = p0 + u * nslots; e[u] = p < end ? P.eid[p] : -1; }
+            acc_t v[SM_CACHE];
+#pragma unroll
+            for (int u = 0; u < SM_CACHE; ++u) v[u] = e[u] < 0 ? (acc_t)0 : (acc_t)Elem<T>::ld(x + (size_t)e[u] * H + h);
+#pragma unroll
+            for (int u = 0; u < SM_CACHE; ++u)
+                if (e[u] >= 0) Elem<T>::st(y + (size_t)e[u] * H + h, exp_acc(v[u] - m) / s);
+        }
+    }
+}
+
+template <typename T, int NW>
+__global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_bwd_heads(bpt_plan P, const T *__restrict__ y, const T *__restrict__ dy,
+                                                                                   T *__restrict__ dx, int H) {
+    using acc_t = typename Elem<T>::acc_t;
+    __shared__ acc_t smem[NW == 1 ? 1 : NW * WAVE];
+    int begin, end;
+    if (!softmax_range<NW>(P, begin, end)) return;
+    const int tid = NW == 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
+    const int h = tid % H, slot = tid / H, nslots = NW * WAVE / H;
+    const bool cached = end - begin <= SM_CACHE * nslots;
+    acc_t yc[SM_CACHE], dc[SM_CACHE];
+    size_t oc[SM_CACHE];
+#pragma unroll
+    for (int u = 0; u < SM_CACHE; ++u) { yc[u] = 0; dc[u] = 0; oc[u] = (size_t)-1; }
+    acc_t s = 0;
+    for (int p0 = begin + slot; p0 < end; p0 += SM_CACHE * nslots) {
+        int e[SM_CACHE];
+#pragma unroll
+        for (int u = 0; u < SM_CACHE; ++u) { const int p = p0 + u * nslots; e[u] = p < end ? P.eid[p] : -1; }
+#pragma unroll
+        for (int u = 0; u < SM_CACHE; ++u) {
+            oc[u] = (size_t)(e[u] < 0 ? 0 : e[u]) * H + h;
+            yc[u] = e[u] < 0 ? (acc_t)0 : (acc_t)Elem<T>::ld(y + oc[u]);
+            dc[u] = e[u] < 0 ? (acc_t)0 : (acc_t)Elem<T>::ld(dy + oc[u]);
+            if (e[u] < 0) oc[u] = (size_t)-1;
+        }
+#pragma unroll
+        for (int u = 0; u < SM_CACHE; ++u) s += dc[u] * yc[u];
+    }
+    s = head_reduce<acc_t, NW, false>(s, H, h, smem);
+    if (cached) {
+#pragma unroll
+        for (int u = 0; u < SM_CACHE; ++u)
+            if (oc[u] != (size_t)-1) Elem<T>::st(dx + oc[u], dc[u] * yc[u] - s * yc[u]);
+    } else {
+        for (int p0 = begin + slot; p0 < end; p0 += SM_CACHE * nslots) {
+            int e[SM_CACHE];
+#pragma unroll
+            for (int u = 0; u < SM_CACHE; ++u) { const int p = p0 + u * nslots; e[u] = p < end ? P.eid[p] : -1; }
+            acc_t yv[SM_CACHE], dv[SM_CACHE];
+#pragma unroll
+            for (int u = 0; u < SM_CACHE; ++u) {
+                const size_t o = (size_t)(e[u] < 0 ? 0 : e[u]) * H + h;
+                yv[u] = e[u] < 0 ? (acc_t)0 : (acc_t)Elem<T>::ld(y + o);
+                dv[u] = e[u] < 0 ? (acc_t)0 : (acc_t)Elem<T>::ld(dy + o);
+            }
+#pragma unroll
+            for (int u = 0; u < SM_CACHE; ++u)
+                if (e[u] >= 0) Elem<T>::st(dx + (size_t)e[u] * H + h, dv[u] * yv[u] - s * yv[u]);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // fast family: compile-time (H, D), f32 / bf16
 // ------------------------------------------------------------------------------------------
@@ -783,16 +925,6 @@ template <int EPL> __device__ __forceinline__ void lds_get_row(const float4 *slo
     }
 }
 
-// value of lane (4 * (lane / 4) + m) for every lane (m is a constant after unrolling)
-__device__ __forceinline__ float quad_bcast(float x, int m) {
-    switch (m & 3) {
-        case 0: return dpp_mov<0x00>(x);
-        case 1: return dpp_mov<0x55>(x);
-        case 2: return dpp_mov<0xAA>(x);
-        default: return dpp_mov<0xFF>(x);
-    }
-}
-
 // two independent head sums, interleaved so that one hides the other's DPP wait states
 template <int LPH> __device__ __forceinline__ void head_sum2(float &a, float &b) {
     if constexpr (LPH >= 2) { a += dpp_mov<0xB1>(a); b += dpp_mov<0xB1>(b); }
@@ -1234,6 +1366,14 @@ int run_spmm_generic(const bpt_plan *P, const void *W, const void *X, void *Y, v
 template <typename T>
 int run_softmax_fwd(const bpt_plan *P, const void *x, void *y, int h, hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
+    if (WAVE % h == 0) {       // heads side by side
+        hipLaunchKernelGGL((k_softmax_fwd_heads<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)x, (T *)y, h);
+        int st = launch_status();
+        if (st != BPT_OK || P->n_heavy == 0) return st;
+        hipLaunchKernelGGL((k_softmax_fwd_heads<T, SM_HEAVY_WAVES>), dim3((int)P->n_heavy), dim3(SM_HEAVY_WAVES * WAVE), 0, s, *P,
+                           (const T *)x, (T *)y, h);
+        return launch_status();
+    }
     hipLaunchKernelGGL((k_softmax_fwd<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)x, (T *)y, h);
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
@@ -1244,6 +1384,14 @@ int run_softmax_fwd(const bpt_plan *P, const void *x, void *y, int h, hipStream_
 template <typename T>
 int run_softmax_bwd(const bpt_plan *P, const void *y, const void *dy, void *dx, int h, hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
+    if (WAVE % h == 0) {       // heads side by side
+        hipLaunchKernelGGL((k_softmax_bwd_heads<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)y, (const T *)dy, (T *)dx, h);
+        int st = launch_status();
+        if (st != BPT_OK || P->n_heavy == 0) return st;
+        hipLaunchKernelGGL((k_softmax_bwd_heads<T, SM_HEAVY_WAVES>), dim3((int)P->n_heavy), dim3(SM_HEAVY_WAVES * WAVE), 0, s, *P,
+                           (const T *)y, (const T *)dy, (T *)dx, h);
+        return launch_status();
+    }
     hipLaunchKernelGGL((k_softmax_bwd<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)y, (const T *)dy, (T *)dx, h);
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
