@@ -139,14 +139,14 @@ def main():
 
     if args.rel_pos:
         # the op sequence of modules/attention.py:66-77 with rel_pos on; the (E, d) rows of the table are
-        # gathered per step as the reference's nn.Embedding does
+        # gathered per step as the reference's nn.Embedding does (backward: segment sums per edge type)
         from bpt_amd import op
         table = (torch.randn(1000, D, generator=gen) / 8).to(tdtype).to(dev)
         et = torch.from_numpy(np.asarray(etype, dtype=np.int64)).to(dev)
 
         def step():
             qq, kk, vv, tt = (x.detach().requires_grad_(True) for x in (q, k, v, table))
-            e = op.masked_mm(*gargs, kk, qq) + op.node_mul_edge(*gargs[4:7], qq, torch.nn.functional.embedding(et, tt))
+            e = op.masked_mm(*gargs, kk, qq) + op.node_mul_edge(*gargs[4:7], qq, op.edge_type_embedding(tt, et))
             a = op.sparse_softmax(*gargs[4:7], e / math.sqrt(D))
             o = op.vec_spmm(*gargs[4:], *gargs[:4], a, vv)
             o.backward(do)

@@ -16,7 +16,7 @@ import math
 import torch
 import torch.nn as nn
 
-from .op import bpt_attention, masked_mm, node_mul_edge, sparse_softmax, vec_spmm
+from .op import bpt_attention, edge_type_embedding, masked_mm, node_mul_edge, sparse_softmax, vec_spmm
 
 __all__ = ["PositionwiseFeedForward", "BPTBlock"]
 
@@ -71,7 +71,7 @@ class BPTBlock(nn.Module):
         if self.rel_pos:
             if etype is None:
                 raise ValueError("rel_pos=True needs the edge types (etype)")
-            e = e + node_mul_edge(COL, INDPTR_C, in_csr[2], q, self.embed_ak(etype))
+            e = e + node_mul_edge(COL, INDPTR_C, in_csr[2], q, edge_type_embedding(self.embed_ak.weight, etype))
         e = self.drop_att(sparse_softmax(COL, INDPTR_C, in_csr[2], e / math.sqrt(self.d_k)))
         return vec_spmm(COL, INDPTR_C, in_csr[2], in_csr[1], ROW, INDPTR_R, out_csr[2], out_csr[1], e, v).view(
             -1, self.d_k * self.h)

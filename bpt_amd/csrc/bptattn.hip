@@ -500,6 +500,29 @@ __device__ __forceinline__ void store_row(T *__restrict__ row, int lane, const f
     }
 }
 
+// The D elements of an (E, D) edge-feature row that go with this lane's slice of a head (every head's lanes read
+// the same D elements).
+template <typename T, int H, int D>
+__device__ __forceinline__ void load_head_row(const T *__restrict__ row, int lane, float (&out)[Lay<T, H, D>::EPL]) {
+    using L = Lay<T, H, D>;
+#pragma unroll
+    for (int i = 0; i < L::NV; ++i) {
+        const int off = (i * L::LPH + lane % L::LPH) * L::VE;
+        if constexpr (sizeof(T) == 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(row) + off);
+            out[4 * i] = v.x; out[4 * i + 1] = v.y; out[4 * i + 2] = v.z; out[4 * i + 3] = v.w;
+        } else {
+            const uint4 v = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(row) + off);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                out[8 * i + 2 * c] = __uint_as_float(w[c] << 16);
+                out[8 * i + 2 * c + 1] = __uint_as_float(w[c] & 0xffff0000u);
+            }
+        }
+    }
+}
+
 // f32 partial rows in the workspace are stored in natural column order (the combine kernels
 // index them by column), whatever the element type of the node tensors
 template <typename T, int H, int D>
@@ -543,8 +566,8 @@ __device__ __forceinline__ void issue_loads_first() { __builtin_amdgcn_sched_bar
 // weight loads for the fast SpMM: the unfused API passes T-typed edge data, the fused backward f32
 template <typename WT> __device__ __forceinline__ float ld_w(const WT *p) { return Elem<WT>::ld(p); }
 
-// y[eid[p], head] = A[row, head, :] . B[idx[p], head, :]
-template <typename T, int H, int D, int BATCH>
+// y[eid[p], head] = A[row, head, :] . B[idx[p], head, :]   (MODE 1: . B[eid[p], :], B an (E, D) edge feature)
+template <typename T, int H, int D, int BATCH, int MODE = 0>
 __global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ y) {
     using L = Lay<T, H, D>;
     Item it;
@@ -554,7 +577,7 @@ __global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__res
     load_row<T, H, D>(A + (size_t)it.row * L::C, lane, a);
     for (int p0 = it.begin; p0 < it.end; p0 += WAVE) {
         const int cnt = min(WAVE, it.end - p0);
-        const int my_idx = lane < cnt ? P.idx[p0 + lane] : 0;
+        const int my_idx = (MODE == 0 && lane < cnt) ? P.idx[p0 + lane] : 0;
         const int my_eid = lane < cnt ? P.eid[p0 + lane] : 0;
         for (int b = 0; b < cnt; b += BATCH) {
             float bv[BATCH][L::EPL];
@@ -563,7 +586,8 @@ __global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__res
             for (int e = 0; e < BATCH; ++e) {
                 const int j = (b + e < cnt) ? b + e : b;
                 ee[e] = __builtin_amdgcn_readlane(my_eid, j);
-                load_row<T, H, D>(B + (size_t)__builtin_amdgcn_readlane(my_idx, j) * L::C, lane, bv[e]);
+                if constexpr (MODE == 0) load_row<T, H, D>(B + (size_t)__builtin_amdgcn_readlane(my_idx, j) * L::C, lane, bv[e]);
+                else load_head_row<T, H, D>(B + (size_t)ee[e] * D, lane, bv[e]);
             }
             issue_loads_first();
 #pragma unroll
@@ -575,8 +599,9 @@ __global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__res
     }
 }
 
-// Y0[row] = sum_p W0[eid[p], head] * X0[idx[p]]  (and the same with W1, X1 -> Y1 when NOUT == 2)
-template <typename T, typename WT, int H, int D, int BATCH, int NOUT>
+// Y0[row] = sum_p W0[eid[p], head] * X0[idx[p]]  (and the same with W1, X1 -> Y1 when NOUT == 2);
+// MODE 1: * X0[eid[p], :], X0 an (E, D) edge feature shared by the heads
+template <typename T, typename WT, int H, int D, int BATCH, int NOUT, int MODE = 0>
 __global__ __launch_bounds__(BLOCK) void k_spmm_fast(bpt_plan P, const WT *__restrict__ W0, const T *__restrict__ X0, T *__restrict__ Y0,
                                                      const WT *__restrict__ W1, const T *__restrict__ X1, T *__restrict__ Y1,
                                                      float *__restrict__ ws0, float *__restrict__ ws1) {
@@ -589,7 +614,7 @@ __global__ __launch_bounds__(BLOCK) void k_spmm_fast(bpt_plan P, const WT *__res
     for (int i = 0; i < L::EPL; ++i) { acc0[i] = 0.f; acc1[i] = 0.f; }
     for (int p0 = it.begin; p0 < it.end; p0 += WAVE) {
         const int cnt = min(WAVE, it.end - p0);
-        const int my_idx = lane < cnt ? P.idx[p0 + lane] : 0;
+        const int my_idx = (MODE == 0 && lane < cnt) ? P.idx[p0 + lane] : 0;
         const int my_eid = lane < cnt ? P.eid[p0 + lane] : 0;
         for (int b = 0; b < cnt; b += BATCH) {
             float x0[BATCH][L::EPL], x1[NOUT == 2 ? BATCH : 1][L::EPL];
@@ -600,7 +625,8 @@ __global__ __launch_bounds__(BLOCK) void k_spmm_fast(bpt_plan P, const WT *__res
                 const int j = ok ? b + e : b;
                 const int src = __builtin_amdgcn_readlane(my_idx, j);
                 const int ed = __builtin_amdgcn_readlane(my_eid, j);
-                load_row<T, H, D>(X0 + (size_t)src * L::C, lane, x0[e]);
+                if constexpr (MODE == 0) load_row<T, H, D>(X0 + (size_t)src * L::C, lane, x0[e]);
+                else load_head_row<T, H, D>(X0 + (size_t)ed * D, lane, x0[e]);
                 w0[e] = ok ? ld_w(W0 + (size_t)ed * H + head) : 0.f;
                 if constexpr (NOUT == 2) {
                     load_row<T, H, D>(X1 + (size_t)src * L::C, lane, x1[e]);
@@ -624,6 +650,41 @@ __global__ __launch_bounds__(BLOCK) void k_spmm_fast(bpt_plan P, const WT *__res
     } else {
         store_row_ws<T, H, D>(ws0 + (size_t)it.slot * L::C, lane, acc0);
         if constexpr (NOUT == 2) store_row_ws<T, H, D>(ws1 + (size_t)it.slot * L::C, lane, acc1);
+    }
+}
+
+// dB[eid[p], d] = sum_h dy[eid[p], h] * A[row, h, d]   (graphop_kernel.cu:79-94), lane = column d (D <= 64):
+// the row's H head vectors stay in registers, each edge costs one 4*H-byte load, H FMAs and one D-element store.
+template <typename T, int H, int D, int BATCH>
+__global__ __launch_bounds__(BLOCK) void k_nme_dB_fast(bpt_plan P, const T *__restrict__ A, const T *__restrict__ dy, T *__restrict__ dB) {
+    static_assert(D <= WAVE && H <= WAVE, "one lane per column");
+    Item it;
+    if (!fetch_item(P, it)) return;
+    const int lane = threadIdx.x & 63;
+    const int col = lane < D ? lane : 0;
+    float a[H];
+#pragma unroll
+    for (int h = 0; h < H; ++h) a[h] = Elem<T>::ld(A + (size_t)it.row * H * D + h * D + col);
+    for (int p0 = it.begin; p0 < it.end; p0 += WAVE) {
+        const int cnt = min(WAVE, it.end - p0);
+        const int my_eid = lane < cnt ? P.eid[p0 + lane] : 0;
+        for (int b = 0; b < cnt; b += BATCH) {
+            int ee[BATCH];
+            float g[BATCH];
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                ee[e] = __builtin_amdgcn_readlane(my_eid, (b + e < cnt) ? b + e : b);
+                g[e] = Elem<T>::ld(dy + (size_t)ee[e] * H + (lane < H ? lane : 0));     // lane h holds dy[e, h]
+            }
+            issue_loads_first();
+#pragma unroll
+            for (int e = 0; e < BATCH; ++e) {
+                float s = 0.f;
+#pragma unroll
+                for (int h = 0; h < H; ++h) s = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(g[e]), h)), a[h], s);
+                if (b + e < cnt && lane < D) Elem<T>::st(dB + (size_t)ee[e] * D + lane, s);
+            }
+        }
     }
 }
 
@@ -1452,6 +1513,48 @@ int run_spmm_fast(const bpt_plan *P, const void *W0, const void *X0, void *Y0, c
     return launch_status();
 }
 
+// node_mul_edge with the specialised kernels: y = A . B[e] (forward), dA = sum dy * B[e], dB[e] = sum_h dy * A
+template <typename T, int H, int D>
+int run_nme_fwd_fast(const bpt_plan *P, const void *A, const void *B, void *y, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_sddmm_fast<T, H, D, FAST_BATCH, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)B, (T *)y);
+    return launch_status();
+}
+
+template <typename T, int H, int D>
+int run_nme_bwd_fast(const bpt_plan *P, const void *A, const void *B, const void *dy, void *dA, void *dB, float *ws, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_spmm_fast<T, T, H, D, FAST_BATCH, 1, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)dy, (const T *)B,
+                       (T *)dA, (const T *)nullptr, (const T *)nullptr, (T *)nullptr, ws, (float *)nullptr);
+    int st = launch_status();
+    if (st != BPT_OK) return st;
+    if (P->n_heavy > 0) {
+        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
+                           (T *)dA, (T *)nullptr, H * D, (size_t)0);
+        st = launch_status();
+        if (st != BPT_OK) return st;
+    }
+    hipLaunchKernelGGL((k_nme_dB_fast<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)dy, (T *)dB);
+    return launch_status();
+}
+
+int nme_fwd_fast(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s) {
+#define X(HH, DD) if (h == HH && d == DD) return run_nme_fwd_fast<T, HH, DD>(P, A, B, y, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
+int nme_bwd_fast(const bpt_plan *P, const void *A, const void *B, const void *dy, void *dA, void *dB, void *ws, int h, int d, int dtype,
+                 hipStream_t s) {
+#define X(HH, DD) if (h == HH && d == DD) return run_nme_bwd_fast<T, HH, DD>(P, A, B, dy, dA, dB, (float *)ws, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
 int sddmm_fast(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s) {
 #define X(HH, DD) if (h == HH && d == DD) return run_sddmm_fast<T, HH, DD>(P, A, B, y, s);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
@@ -1675,6 +1778,7 @@ int bpt_node_mul_edge_forward(const bpt_plan *plan, const void *A, const void *B
     CHECK(check_plan(plan, false));
     CHECK(check_shape(h, d, dtype));
     if (plan->n_edges > 0 && (!A || !B || !y)) return BPT_ERR_NULL;
+    if (fast_shape(h, d, dtype) && aligned16(A) && aligned16(B)) return nme_fwd_fast(plan, A, B, y, h, d, dtype, (hipStream_t)stream);
     return sddmm_edge_generic(plan, A, B, y, h, d, dtype, (hipStream_t)stream);
 }
 
@@ -1685,6 +1789,8 @@ int bpt_node_mul_edge_backward(const bpt_plan *plan, const void *A, const void *
     if (!dA || (plan->n_edges > 0 && (!A || !B || !dy || !dB))) return BPT_ERR_NULL;
     const int64_t need = bpt_workspace_bytes(BPT_OP_NODE_MUL_EDGE_BWD, plan, nullptr, h, d, dtype);
     if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    if (fast_shape(h, d, dtype) && aligned16(B) && aligned16(dA) && aligned16(workspace))
+        return nme_bwd_fast(plan, A, B, dy, dA, dB, workspace, h, d, dtype, (hipStream_t)stream);
     CHECK(spmm_edge_generic(plan, dy, B, dA, workspace, h, d, dtype, (hipStream_t)stream));
     DISPATCH_DTYPE(dtype, (run_nme_dB<T>(plan, A, dy, dB, h, d, (hipStream_t)stream)))
 }

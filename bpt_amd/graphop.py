@@ -176,15 +176,19 @@ def sparse_softmax_backward(row, indptr, eid, y, dy):
     return dx
 
 
-def vector_spmm_forward(row, indptr, eid, indices, edata, x):
-    """y[row] = sum_p edata[eid[p]] * x[indices[p]] (graphop.cpp:79-95, graphop_kernel.cu:509-542)."""
+def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None):
+    """y[row] = sum_p edata[eid[p]] * x[indices[p]] (graphop.cpp:79-95, graphop_kernel.cu:509-542).
+
+    n_rows (keyword only, not in the reference): number of rows of y when it differs from x.size(0) — a
+    rectangular operator, used for the segment sums of the relative-position table's gradient."""
     _check_all(row=row, indptr=indptr, eid=eid, indices=indices, edata=edata, x=x)
     _same_dtype(edata, x)
     h, d = _hd(x)
     if _edge_h(edata) != h:
         raise RuntimeError("edata and x disagree on the number of heads")
-    plan = plan_cache.get(row, indptr, eid, indices, x.size(0), x.size(0))
-    y = torch.empty_like(x)
+    n_out = x.size(0) if n_rows is None else int(n_rows)
+    plan = plan_cache.get(row, indptr, eid, indices, n_out, x.size(0))
+    y = torch.empty_like(x) if n_rows is None else torch.empty((n_out,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
     dt = _dtype(x)
     ws, nws = _workspace(OP_SPMM_FWD, plan, None, h, d, dt, x.device)
     with torch.cuda.device_of(x):

@@ -11,8 +11,8 @@ from . import graphop as _g
 from .graphop import (maskedmm_csr_backward, maskedmm_csr_forward, node_mul_edge_backward, node_mul_edge_forward,
                       sparse_softmax_backward, sparse_softmax_forward, vector_spmm_backward, vector_spmm_forward)
 
-__all__ = ["SparseSoftmax", "MaskedMMCSR", "NodeMulEdge", "VectorSPMM", "BPTAttention",
-           "sparse_softmax", "masked_mm", "node_mul_edge", "vec_spmm", "bpt_attention"]
+__all__ = ["SparseSoftmax", "MaskedMMCSR", "NodeMulEdge", "VectorSPMM", "BPTAttention", "EdgeTypeEmbedding",
+           "sparse_softmax", "masked_mm", "node_mul_edge", "vec_spmm", "bpt_attention", "edge_type_embedding"]
 
 
 class SparseSoftmax(Function):
@@ -106,6 +106,55 @@ def node_mul_edge(row, indptr, eid, A, B):
 
 def vec_spmm(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x):
     return VectorSPMM.apply(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x)
+
+
+class EdgeTypeEmbedding(Function):
+    """table[etype] -> (E, d): what `self.embed_ak(g.edata['etype'])` computes (modules/attention.py:57), with a
+    deterministic backward: the (E, d) gradient rows are summed per edge type by the SpMM kernels over a CSR whose
+    rows are the edge types (torch's embedding backward scatters with atomics, about 1 ms at E = 430 k)."""
+
+    @staticmethod
+    def forward(ctx, table, etype, type_csr):
+        ctx.type_csr = type_csr
+        ctx.n_types = table.size(0)
+        return table.index_select(0, etype)
+
+    @staticmethod
+    def backward(ctx, grad):
+        row, indptr, order = ctx.type_csr
+        grad = grad.contiguous()
+        ones = torch.ones(grad.size(0), dtype=grad.dtype, device=grad.device)
+        return vector_spmm_forward(row, indptr, order, order, ones, grad, n_rows=ctx.n_types), None, None
+
+
+_type_csr_cache = {}
+
+
+def _type_csr(etype, n_types):
+    """(row, indptr, order) of the CSR whose row t lists the edges of type t (ascending edge id), chunked like the
+    reference's other CSRs; cached per etype tensor."""
+    from .graphbuilder import partition_csr
+    key = (etype.data_ptr(), etype.numel(), etype._version, str(etype.device), n_types)
+    hit = _type_csr_cache.get(key)
+    if hit is None:
+        et = etype.detach().cpu().numpy()
+        if et.size and (et.min() < 0 or et.max() >= n_types):
+            raise ValueError("edge type out of range")
+        import numpy as np
+        order = np.argsort(et, kind="stable").astype(np.int64)
+        indptr = np.zeros(n_types + 1, dtype=np.int64)
+        np.cumsum(np.bincount(et, minlength=n_types), out=indptr[1:])
+        row, indptr_units = partition_csr(indptr)
+        hit = tuple(torch.as_tensor(np.asarray(a), dtype=torch.int64).to(etype.device) for a in (row, indptr_units, order)) + (etype,)
+        if len(_type_csr_cache) > 16:
+            _type_csr_cache.clear()
+        _type_csr_cache[key] = hit          # holds etype so that its data_ptr is not reused while cached
+    return hit[:3]
+
+
+def edge_type_embedding(table, etype):
+    """Rows of `table` for every edge, differentiable w.r.t. `table` (deterministic segment-sum backward)."""
+    return EdgeTypeEmbedding.apply(table, etype, _type_csr(etype, table.size(0)))
 
 
 def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale=None, fused=None):
