@@ -104,6 +104,7 @@ def main():
     ap.add_argument("--group-rows", type=int, default=None, choices=[4, 8], help="rows per wavefront group of the fused kernels (default: 8 where available, else 4)")
     ap.add_argument("--rows", action="store_true", help="fused kernels with one wavefront per row (no row groups)")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
+    ap.add_argument("--dropout", type=float, default=0.0, help="dropout on the attention probabilities inside the fused kernels (attention.py:73)")
     ap.add_argument("--rel-pos", action="store_true",
                     help="add the relative-position score term q[dst].table[etype[e]] (table (1000, d_head), modules/attention.py:23,42,69-71)")
     ap.add_argument("--block-layers", type=int, default=0,
@@ -161,8 +162,8 @@ def main():
             return o, qq.grad, kk.grad, vv.grad
     else:
         def step():
-            o, lse = graphop.attention_forward(*gargs[4:], q, k, v)
-            dq, dk, dv = graphop.attention_backward(*gargs, q, k, v, o, lse, do)
+            o, lse = graphop.attention_forward(*gargs[4:], q, k, v, dropout_p=args.dropout, seed=2345)
+            dq, dk, dv = graphop.attention_backward(*gargs, q, k, v, o, lse, do, dropout_p=args.dropout, seed=2345)
             return o, dq, dk, dv
 
     ref = step()                                   # builds + caches the plans
@@ -274,7 +275,8 @@ def main():
         "value": E / t_step, "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype_name, "data": "synthetic",
-        "config": {"workload": desc + (" (op chain with rel_pos)" if args.rel_pos else " (unfused op chain)" if args.unfused else " (fused fwd+bwd)"), "n_nodes": N,
+        "config": {"workload": desc + (" (op chain with rel_pos)" if args.rel_pos else " (unfused op chain)" if args.unfused else
+                                       f" (fused fwd+bwd, attention dropout {args.dropout})" if args.dropout > 0 else " (fused fwd+bwd)"), "n_nodes": N,
                    "n_edges": E, "heads": H, "d_head": D, "launch": mode,
                    "kernels": "per-row" if args.rows else f"row-groups({args.group_rows or 'auto'} rows per wavefront)"},
         "roofline": roofline,

@@ -56,9 +56,10 @@ ATTN_API = {
     "bpt_sparse_softmax_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, ctypes.c_int, ctypes.c_int, c_vp]),
     "bpt_vector_spmm_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_vector_spmm_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
-    "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float] + _tail),
+    "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float, ctypes.c_float,
+                                            ctypes.c_uint64] + _tail),
     "bpt_attention_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
-                                             ctypes.c_float] + _tail),
+                                             ctypes.c_float, ctypes.c_float, ctypes.c_uint64] + _tail),
 }
 
 _graph = None

@@ -7,8 +7,8 @@ DGL graph object (`g.ndata['h']`, `g.edata['etype']`) and writes the result back
 `forward(h, csr, etype)` takes and returns plain tensors, `csr` being the 6-tuple that
 `graph/base.py:71-86` (`bpt_amd.graphbuilder.get_csrs`) produces.
 
-Attention core: with `rel_pos` off and no attention dropout in effect the fused kernels run
-(`op.bpt_attention`); otherwise the four operators are composed exactly as attention.py:66-77 does.
+Attention core: with `rel_pos` off the fused kernels run (`op.bpt_attention`, attention dropout included);
+otherwise the four operators are composed exactly as attention.py:66-77 does.
 Projections, LayerNorm and the feed-forward are torch modules (rocBLAS GEMMs).
 """
 import math
@@ -64,9 +64,9 @@ class BPTBlock(nn.Module):
         """attention.py:66-77: (n, h, d_k) q, k, v -> (n, h * d_k)."""
         out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C = csr
         graph = (ROW, INDPTR_R, out_csr[2], out_csr[1], COL, INDPTR_C, in_csr[2], in_csr[1])
-        att_dropout = self.training and self.drop_att.p > 0
-        if not self.rel_pos and not att_dropout:
-            return bpt_attention(*graph, q, k, v).view(-1, self.d_k * self.h)
+        att_dropout = self.drop_att.p if self.training else 0.0
+        if not self.rel_pos:
+            return bpt_attention(*graph, q, k, v, dropout_p=att_dropout).view(-1, self.d_k * self.h)
         e = masked_mm(*graph, k, q)
         if self.rel_pos:
             if etype is None:

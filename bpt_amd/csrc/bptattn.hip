@@ -986,6 +986,16 @@ template <int EPL> __device__ __forceinline__ void lds_get_row(const float4 *slo
     }
 }
 
+// Dropout on the attention probabilities (modules/attention.py:73): the keep / drop decision of (pair n, head h) is
+// a hash of n * H + h and the call's seed, so that forward and backward agree without storing a mask.  n is the
+// pair's number in the destination-side groups (entry's first pair + rank of the member in the entry's mask).
+// Returns the multiplier 1 / (1 - p) or 0.
+__device__ __forceinline__ float dropout_keep(uint32_t key, uint32_t seed, uint32_t thr, float inv_keep) {
+    uint32_t x = key ^ seed;
+    x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+    return x >= thr ? inv_keep : 0.f;
+}
+
 // two independent head sums, interleaved so that one hides the other's DPP wait states
 template <int LPH> __device__ __forceinline__ void head_sum2(float &a, float &b) {
     if constexpr (LPH >= 2) { a += dpp_mov<0xB1>(a); b += dpp_mov<0xB1>(b); }
@@ -1005,10 +1015,11 @@ __device__ __forceinline__ float max3f(float a, float b, float c) {
 
 // Forward: online softmax in base 2 over the group's entries, two entries per step.  The members' q rows
 // (pre-scaled) live in LDS and are re-read for every use, which keeps the kernel at three wavefronts per SIMD.
-template <typename T, int H, int D, int R, int HS>
+template <typename T, int H, int D, int R, int HS, bool DROP>
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_attn_fwd_grp(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
-    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr,
+    uint32_t drop_seed, float drop_inv) {
     constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
     using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
@@ -1021,11 +1032,11 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     struct Batch {
         RawRow<T, HL, D> kr[GRP_BATCH], vr[GRP_BATCH];
-        int mk[GRP_BATCH];
+        int mk[GRP_BATCH], pz[GRP_BATCH];
     };
     struct Rows {
         float kv[GRP_BATCH][EPL], vv[GRP_BATCH][EPL];
-        int mk[GRP_BATCH];
+        int mk[GRP_BATCH], pz[GRP_BATCH];
     };
     __shared__ float4 q_lds[R * (EPL / 4) * WAVE];
     float acc[R][EPL], mrun[R], lrun[R];
@@ -1049,19 +1060,27 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             for (int e = 0; e < GRP_BATCH; ++e) {
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
+                B.pz[e] = DROP ? __builtin_amdgcn_readlane(ent.z, b + e) : 0;
                 load_row32_raw<T, HL, D, CF>(k, src, loff, B.kr[e]);
                 load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
             }
         };
-        auto one = [&](int m, const float (&kr)[EPL], const float (&vr)[EPL]) {
+        // multiplier of the pair (member m, entry with mask mk and first pair pz): 1 without dropout
+        auto keep = [&](int m, int mk, int pz) -> float {
+            if constexpr (!DROP) return 1.f;
+            const int n = pz + __builtin_popcount(mk & ((1 << m) - 1));
+            return dropout_keep((uint32_t)(n * H + head), drop_seed, drop_thr, drop_inv);
+        };
+        auto one = [&](int m, const float (&kr)[EPL], const float (&vr)[EPL], int mk, int pz) {
             float qm[EPL];
             lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
             const float s = head_sum<L::LPH>(dot_n<EPL>(qm, kr));
             const float mx = fmaxf(mrun[m], s);
             const float al = __builtin_amdgcn_exp2f(mrun[m] - mx), pe = __builtin_amdgcn_exp2f(s - mx);
-            lrun[m] = fmaf(lrun[m], al, pe);
+            lrun[m] = fmaf(lrun[m], al, pe);                       // the softmax denominator ignores dropout
+            const float pk = pe * keep(m, mk, pz);
 #pragma unroll
-            for (int i = 0; i < EPL; ++i) acc[m][i] = fmaf(pe, vr[i], acc[m][i] * al);
+            for (int i = 0; i < EPL; ++i) acc[m][i] = fmaf(pk, vr[i], acc[m][i] * al);
             mrun[m] = mx;
         };
         auto compute = [&](const Batch &raw) {
@@ -1071,12 +1090,13 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                 unpack_row<T, HL, D>(raw.kr[e], B.kv[e]);
                 unpack_row<T, HL, D>(raw.vr[e], B.vv[e]);
                 B.mk[e] = raw.mk[e];
+                B.pz[e] = raw.pz[e];
             }
 #pragma unroll
             for (int m = 0; m < R; ++m) {
                 const bool h0 = (B.mk[0] >> m) & 1, h1 = (B.mk[GRP_BATCH - 1] >> m) & 1;
                 if constexpr (GRP_BATCH == 1) {
-                    if (h0) one(m, B.kv[0], B.vv[0]);
+                    if (h0) one(m, B.kv[0], B.vv[0], B.mk[0], B.pz[0]);
                 } else if (h0 && h1) {
                     float qm[EPL];
                     lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
@@ -1086,13 +1106,14 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                     const float al = __builtin_amdgcn_exp2f(mrun[m] - mx);
                     const float p0e = __builtin_amdgcn_exp2f(s0 - mx), p1e = __builtin_amdgcn_exp2f(s1 - mx);
                     lrun[m] = fmaf(lrun[m], al, p0e + p1e);
+                    const float k0 = p0e * keep(m, B.mk[0], B.pz[0]), k1 = p1e * keep(m, B.mk[GRP_BATCH - 1], B.pz[GRP_BATCH - 1]);
 #pragma unroll
-                    for (int i = 0; i < EPL; ++i) acc[m][i] = fmaf(p1e, B.vv[GRP_BATCH - 1][i], fmaf(p0e, B.vv[0][i], acc[m][i] * al));
+                    for (int i = 0; i < EPL; ++i) acc[m][i] = fmaf(k1, B.vv[GRP_BATCH - 1][i], fmaf(k0, B.vv[0][i], acc[m][i] * al));
                     mrun[m] = mx;
                 } else if (h0) {
-                    one(m, B.kv[0], B.vv[0]);
+                    one(m, B.kv[0], B.vv[0], B.mk[0], B.pz[0]);
                 } else if (h1) {
-                    one(m, B.kv[GRP_BATCH - 1], B.vv[GRP_BATCH - 1]);
+                    one(m, B.kv[GRP_BATCH - 1], B.vv[GRP_BATCH - 1], B.mk[GRP_BATCH - 1], B.pz[GRP_BATCH - 1]);
                 }
             }
         };
@@ -1136,11 +1157,11 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 // (entry, member) of this plan (a spare position for members the entry does not have).  One store per
 // entry and quad of members: lane l carries the pair of member 4c + l % 4; the same register of ds values is
 // the A operand of the MFMA that accumulates dq.  The members' q rows live in LDS.
-template <typename T, int H, int D, int R, int HS>
+template <typename T, int H, int D, int R, int HS, bool DROP>
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_attn_bwd_dst_grp(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
     const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
-    float *__restrict__ ws_dq, float scale, float scale_log2e) {
+    float *__restrict__ ws_dq, float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv) {
     constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
     using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
@@ -1155,7 +1176,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     struct Batch {
         RawRow<T, HL, D> kr[GRP_BATCH], vr[GRP_BATCH];
-        int mk[GRP_BATCH], xp[GRP_BATCH][NQ];
+        int mk[GRP_BATCH], pz[GRP_BATCH], xp[GRP_BATCH][NQ];
     };
     __shared__ float4 q_lds[R * (EPL / 4) * WAVE];
     float dov[R][EPL], delta_s[R], lse2[R];
@@ -1185,6 +1206,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             for (int e = 0; e < GRP_BATCH; ++e) {
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
+                B.pz[e] = DROP ? __builtin_amdgcn_readlane(ent.z, b + e) : 0;
                 // lane l fetches the scratch positions of the pairs of members l % 4, 4 + l % 4, ... with this entry
                 const char *pp = reinterpret_cast<const char *>(P.grp_pairs) + (size_t)((uint32_t)(p0 + b + e) * (uint32_t)(R * 4));
 #pragma unroll
@@ -1209,8 +1231,14 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                         lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
                         float s = dot_n<EPL>(qm, kv), dp = dot_n<EPL>(dov[m], vv);
                         head_sum2<L::LPH>(s, dp);
-                        const float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
-                        const float ds = pe * fmaf(dp, scale, -delta_s[m]);
+                        float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
+                        float mt = 1.f;                   // dropout multiplier of this pair (as in the forward kernel)
+                        if constexpr (DROP) {
+                            const int n = B.pz[e] + __builtin_popcount(B.mk[e] & ((1 << m) - 1));
+                            mt = dropout_keep((uint32_t)(n * H + head), drop_seed, drop_thr, drop_inv);
+                        }
+                        const float ds = pe * fmaf(dp * mt, scale, -delta_s[m]);
+                        pe *= mt;                         // what multiplies v (forward) and dO (dV)
                         wp[m / 4] = mine == (m & 3) ? pe : wp[m / 4];
                         wd[m / 4] = mine == (m & 3) ? ds : wd[m / 4];
                     }
@@ -1583,6 +1611,17 @@ int spmm(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int
 
 inline int64_t round16(int64_t b) { return (b + 15) & ~(int64_t)15; }
 
+// dropout of the fused path: threshold on the 32-bit hash (0 = off), seed, 1 / (1 - p)
+struct Dropout {
+    uint32_t thr, seed;
+    float inv;
+};
+inline Dropout make_dropout(float p, uint64_t seed) {
+    if (!(p > 0.f)) return Dropout{0u, 0u, 1.f};
+    const double t = (double)p * 4294967296.0;
+    return Dropout{(uint32_t)(t >= 4294967295.0 ? 4294967295.0 : (t < 1.0 ? 1.0 : t)), (uint32_t)(seed ^ (seed >> 32)), 1.f / (1.f - p)};
+}
+
 // The row-group kernels address node rows and the per-pair scratch with 32-bit byte offsets.
 inline bool fits32(int64_t n, int64_t unit) { return n >= 0 && n <= (int64_t)0xffffffffu / unit; }
 
@@ -1619,19 +1658,25 @@ inline int64_t pds_bytes(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d
 }
 
 template <typename T, int H, int D>
-int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v, void *o, float *lse, void *ws, float scale, hipStream_t s) {
+int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v, void *o, float *lse, void *ws, float scale, Dropout drop,
+                 hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
     float *ws_acc = (float *)ws;
     float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
         if (has_groups(P, H, D, sizeof(T))) {
-#define LAUNCH_FWD(RR)                                                                                                   \
-    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR, HS>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)q, \
-                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E)
+#define LAUNCH_FWD(RR, DR)                                                                                                   \
+    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR, HS, DR>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)q, \
+                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv)
             constexpr int HS = head_slices<T, H, D>();
-            if (P->grp_R == 8) LAUNCH_FWD(8);
-            else LAUNCH_FWD(4);
+            if (drop.thr == 0) {
+                if (P->grp_R == 8) LAUNCH_FWD(8, false);
+                else LAUNCH_FWD(4, false);
+            } else {
+                if (P->grp_R == 8) LAUNCH_FWD(8, true);
+                else LAUNCH_FWD(4, true);
+            }
 #undef LAUNCH_FWD
         } else {
             hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
@@ -1647,7 +1692,7 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
 
 template <typename T, int H, int D>
 int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
-                 const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, hipStream_t s) {
+                 const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, Dropout drop, hipStream_t s) {
     if (Pin->n_items == 0) return BPT_OK;
     const bool grouped = grouped_backward(Pin, Pout, H, D, sizeof(T));
     const int64_t pbytes = pds_bytes(Pin, Pout, H, D, sizeof(T));
@@ -1658,12 +1703,18 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
         if (grouped) {
-#define LAUNCH_DST(RR)                                                                                                             \
-    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, RR, HS>), dim3(group_grid(Pin) * HS), dim3(WAVE), 0, s, *Pin, (const T *)q,   \
-                       (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E)
+#define LAUNCH_DST(RR, DR)                                                                                                           \
+    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, RR, HS, DR>), dim3(group_grid(Pin) * HS), dim3(WAVE), 0, s, *Pin, (const T *)q, \
+                       (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E,  \
+                       drop.thr, drop.seed, drop.inv)
             constexpr int HS = head_slices<T, H, D>();
-            if (Pin->grp_R == 8) LAUNCH_DST(8);
-            else LAUNCH_DST(4);
+            if (drop.thr == 0) {
+                if (Pin->grp_R == 8) LAUNCH_DST(8, false);
+                else LAUNCH_DST(4, false);
+            } else {
+                if (Pin->grp_R == 8) LAUNCH_DST(8, true);
+                else LAUNCH_DST(4, true);
+            }
 #undef LAUNCH_DST
         } else {
             hipLaunchKernelGGL((k_attn_bwd_dst<T, H, D, FAST_BATCH>), dim3(grid_for(Pin)), dim3(BLOCK), 0, s, *Pin, (const T *)q,
@@ -1833,16 +1884,20 @@ int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const
 }
 
 int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v, void *o, float *lse,
-                          void *workspace, int64_t workspace_bytes, float scale, int h, int d, int dtype, void *stream) {
+                          void *workspace, int64_t workspace_bytes, float scale, float dropout_p, uint64_t dropout_seed, int h, int d,
+                          int dtype, void *stream) {
     CHECK(check_plan(plan_in, true));
     CHECK(check_shape(h, d, dtype));
     if (!q || !k || !v || !o || !lse) return BPT_ERR_NULL;
+    if (!(dropout_p >= 0.f && dropout_p < 1.f)) return BPT_ERR_SIZE;
+    const Dropout drop = make_dropout(dropout_p, dropout_seed);
+    if (drop.thr != 0 && !has_groups(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;   // row-group kernels only
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(workspace))
         return BPT_ERR_UNSUPPORTED;
     const int64_t need = bpt_workspace_bytes(BPT_OP_ATTN_FWD, plan_in, nullptr, h, d, dtype);
     if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
-#define X(HH, DD) if (h == HH && d == DD) return run_attn_fwd<T, HH, DD>(plan_in, q, k, v, o, lse, workspace, scale, s);
+#define X(HH, DD) if (h == HH && d == DD) return run_attn_fwd<T, HH, DD>(plan_in, q, k, v, o, lse, workspace, scale, drop, s);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
 #undef X
@@ -1851,10 +1906,14 @@ int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k,
 
 int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, const void *q, const void *k, const void *v,
                            const void *o, const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *workspace,
-                           int64_t workspace_bytes, float scale, int h, int d, int dtype, void *stream) {
+                           int64_t workspace_bytes, float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype,
+                           void *stream) {
     CHECK(check_plan(plan_in, true));
     CHECK(check_plan(plan_out, true));
     CHECK(check_shape(h, d, dtype));
+    if (!(dropout_p >= 0.f && dropout_p < 1.f)) return BPT_ERR_SIZE;
+    const Dropout drop = make_dropout(dropout_p, dropout_seed);
+    if (drop.thr != 0 && !grouped_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
     if (plan_in->n_edges != plan_out->n_edges || plan_in->n_rows != plan_out->n_rows) return BPT_ERR_PLAN;
     if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return BPT_ERR_NULL;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) ||
@@ -1864,7 +1923,7 @@ int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, co
     if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
 #define X(HH, DD) \
-    if (h == HH && d == DD) return run_attn_bwd<T, HH, DD>(plan_in, plan_out, q, k, v, o, d_o, lse, dq, dk, dv, workspace, scale, s);
+    if (h == HH && d == DD) return run_attn_bwd<T, HH, DD>(plan_in, plan_out, q, k, v, o, d_o, lse, dq, dk, dv, workspace, scale, drop, s);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
 #undef X

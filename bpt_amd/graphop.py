@@ -224,9 +224,11 @@ def attention_supported(q):
     return q.dim() == 3 and (h, d) in fast.get(q.dtype, ())
 
 
-def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None):
-    """o[dst] = sum over in-edges softmax(q[dst].k[src]*scale) v[src]; returns (o, lse) with lse (n, h) float32
-    in base-2 units.  Arithmetic of modules/attention.py:66-77 (no dropout, no rel-pos) in one pass."""
+def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, dropout_p=0.0, seed=0):
+    """o[dst] = sum over in-edges drop(softmax(q[dst].k[src]*scale)) v[src]; returns (o, lse) with lse (n, h)
+    float32 in base-2 units.  Arithmetic of modules/attention.py:66-77 (no rel-pos) in one pass.  dropout_p > 0
+    drops attention probabilities as attention.py:73 does; the mask is a function of (seed, graph), see
+    attention_dropout_mask."""
     _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v)
     _same_dtype(q, k, v)
     h, d = _hd(q)
@@ -239,12 +241,14 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None):
     ws, nws = _workspace(OP_ATTN_FWD, plan, None, h, d, dt, q.device)
     with torch.cuda.device_of(q):
         check_attn(_LIB.bpt_attention_forward(ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws), nws,
-                                              scale, h, d, dt, _stream()), "attention_forward")
+                                              scale, float(dropout_p), int(seed) & (2 ** 64 - 1), h, d, dt, _stream()),
+                   "attention_forward")
     return o, lse
 
 
-def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, do, scale=None):
-    """(dq, dk, dv) of attention_forward."""
+def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, do, scale=None,
+                       dropout_p=0.0, seed=0):
+    """(dq, dk, dv) of attention_forward (same dropout_p and seed)."""
     _check_all(row=row, indptr_r=indptr_r, eid_r=eid_r, indices_r=indices_r, col=col, indptr_c=indptr_c,
                eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v, o=o, lse=lse)
     do = do.contiguous()
@@ -264,8 +268,35 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     with torch.cuda.device_of(q):
         check_attn(_LIB.bpt_attention_backward(in_ref, out_ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do),
                                                _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
-                                               scale, h, d, dt, _stream()), "attention_backward")
+                                               scale, float(dropout_p), int(seed) & (2 ** 64 - 1), h, d, dt, _stream()),
+                   "attention_backward")
     return dq, dk, dv
+
+
+def attention_dropout_mask(col, indptr_c, eid_c, indices_c, q, k, dropout_p, seed):
+    """The (E, h) float32 multipliers (0 or 1 / (1 - p)) that attention_forward(..., dropout_p, seed) applies to the
+    attention probabilities of these tensors, computed on the host from the plan (testing and debugging aid)."""
+    import numpy as np
+    h, d = _hd(q)
+    plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
+    grp = plan.ensure_groups(_group_rows(q, h, d, plan))["host"]
+    E = plan.n_edges
+    p = float(dropout_p)
+    if not p > 0.0:
+        return torch.ones((E, h), dtype=torch.float32)
+    t = p * 4294967296.0
+    thr = np.uint32(min(max(t, 1.0), 4294967295.0))
+    seed = int(seed) & (2 ** 64 - 1)
+    s32 = np.uint32((seed ^ (seed >> 32)) & 0xffffffff)
+    key = (np.arange(E, dtype=np.uint64)[:, None] * np.uint64(h) + np.arange(h, dtype=np.uint64)[None, :]).astype(np.uint32)
+    x = key ^ s32
+    x ^= x >> np.uint32(16); x = (x.astype(np.uint64) * np.uint64(0x7feb352d)).astype(np.uint32)
+    x ^= x >> np.uint32(15); x = (x.astype(np.uint64) * np.uint64(0x846ca68b)).astype(np.uint32)
+    x ^= x >> np.uint32(16)
+    keep_pair = np.where(x >= thr, np.float32(1.0 / (1.0 - np.float32(p))), np.float32(0.0)).astype(np.float32)   # by pair number
+    out = np.empty((E, h), dtype=np.float32)
+    out[grp["pair_eid"]] = keep_pair
+    return torch.from_numpy(out)
 
 
 _USE_GROUPS = True
@@ -289,6 +320,10 @@ def set_group_rows(R):
         raise ValueError("R must be None, 4 or 8")
     old, _GROUP_ROWS = _GROUP_ROWS, R
     return old
+
+
+def row_groups_enabled():
+    return _USE_GROUPS
 
 
 def set_row_groups(on):

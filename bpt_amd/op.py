@@ -73,23 +73,23 @@ class VectorSPMM(Function):
 
 
 class BPTAttention(Function):
-    """Fused masked_mm -> scale -> sparse_softmax -> vec_spmm (modules/attention.py:66-77 with
-    rel_pos off and dropout 0).  Saves q, k, v, o and the per-(node, head) log-sum-exp instead of
-    the (E, h) score and probability tensors."""
+    """Fused masked_mm -> scale -> sparse_softmax -> dropout -> vec_spmm (modules/attention.py:66-77 with
+    rel_pos off).  Saves q, k, v, o and the per-(node, head) log-sum-exp instead of the (E, h) score and
+    probability tensors; the dropout mask is regenerated in backward from (dropout_p, seed)."""
 
     @staticmethod
-    def forward(ctx, row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale):
-        o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale)
+    def forward(ctx, row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p=0.0, seed=0):
+        o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed)
         ctx.save_for_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse)
-        ctx.scale = scale
+        ctx.scale, ctx.dropout_p, ctx.seed = scale, dropout_p, seed
         return o
 
     @staticmethod
     def backward(ctx, do):
         row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse = ctx.saved_tensors
         dq, dk, dv = _g.attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c,
-                                           q, k, v, o, lse, do, ctx.scale)
-        return None, None, None, None, None, None, None, None, dq, dk, dv, None
+                                           q, k, v, o, lse, do, ctx.scale, ctx.dropout_p, ctx.seed)
+        return None, None, None, None, None, None, None, None, dq, dk, dv, None, None, None
 
 
 def sparse_softmax(row, indptr, eid, x):
@@ -157,18 +157,28 @@ def edge_type_embedding(table, etype):
     return EdgeTypeEmbedding.apply(table, etype, _type_csr(etype, table.size(0)))
 
 
-def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale=None, fused=None):
+def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale=None, fused=None,
+                  dropout_p=0.0, seed=None):
     """Attention over the graph: (ROW, INDPTR_R, out_eid, out_idx) is the out-CSR side (rows =
     sources), (COL, INDPTR_C, in_eid, in_idx) the in-CSR side (rows = destinations), exactly the
     eight graph arguments modules/attention.py:66-67 passes to masked_mm.
 
     fused=None picks the fused kernels when they cover (h, d, dtype) and otherwise composes the
-    unfused HIP ops in the reference's order; both run on the GPU."""
+    unfused HIP ops in the reference's order; both run on the GPU.
+
+    dropout_p > 0 applies dropout to the attention probabilities (attention.py:73).  The fused path hashes
+    (seed, edge, head); seed=None draws one from torch's CPU generator (reproducible under torch.manual_seed).  The
+    unfused path uses torch's dropout, so the two paths drop different elements."""
     scale = 1.0 / math.sqrt(q.size(-1)) if scale is None else float(scale)
     if fused is None:
         fused = _g.attention_supported(q) and q.size(0) == k.size(0)
+        if dropout_p > 0 and not _g.row_groups_enabled():
+            fused = False                       # only the row-group kernels implement dropout
     if fused:
-        return BPTAttention.apply(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale)
+        if dropout_p > 0 and seed is None:
+            seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+        return BPTAttention.apply(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale,
+                                  float(dropout_p), int(seed or 0))
     e = masked_mm(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, k, q)
-    a = sparse_softmax(col, indptr_c, eid_c, e * scale)
+    a = torch.nn.functional.dropout(sparse_softmax(col, indptr_c, eid_c, e * scale), p=float(dropout_p), training=dropout_p > 0)
     return vec_spmm(col, indptr_c, eid_c, indices_c, row, indptr_r, eid_r, indices_r, a, v)

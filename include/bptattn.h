@@ -128,19 +128,23 @@ int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const
                              const void *x, void *dedata, void *dx, void *workspace, int64_t workspace_bytes,
                              int h, int d, int dtype, void *stream);
 
-/* Fused attention layer core = modules/attention.py:66-77 without dropout / rel-pos:
- *   o[dst] = sum_{e: src->dst} softmax_dst( q[dst].k[src] * scale ) * v[src]
+/* Fused attention layer core = modules/attention.py:66-77 without rel-pos:
+ *   o[dst] = sum_{e: src->dst} drop( softmax_dst( q[dst].k[src] * scale ) )[e] * v[src]
  * plan_in: rows = destinations (the reference's COL/INDPTR_C/in_csr), plan_out: rows = sources.
  * lse (n, h) float32 receives the base-2 log-sum-exp of the scaled scores, needed by backward.
- * f32 and bf16 only (accumulation in f32). */
+ * f32 and bf16 only (accumulation in f32).
+ * dropout_p in [0, 1): dropout on the attention probabilities (attention.py:73); 0 = none.  Each (edge, head) is
+ * kept with probability 1 - p and scaled by 1 / (1 - p); the decision is a hash of dropout_seed and the edge's pair
+ * number in plan_in's row groups, so backward must get the same plan, p and seed.  Needs the row groups
+ * (BPT_ERR_UNSUPPORTED without them). */
 int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v,
                           void *o, float *lse, void *workspace, int64_t workspace_bytes,
-                          float scale, int h, int d, int dtype, void *stream);
+                          float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype, void *stream);
 
 int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, const void *q, const void *k,
                            const void *v, const void *o, const void *d_o, const float *lse,
                            void *dq, void *dk, void *dv, void *workspace, int64_t workspace_bytes,
-                           float scale, int h, int d, int dtype, void *stream);
+                           float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype, void *stream);
 
 #ifdef __cplusplus
 }

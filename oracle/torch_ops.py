@@ -11,10 +11,12 @@ import math
 import torch
 
 
-def attention(src, dst, q, k, v, ak=None):
+def attention(src, dst, q, k, v, ak=None, drop=None):
     """src, dst: (E,) int64 edge endpoints (edge e: src[e] -> dst[e]); q,k,v: (N,H,D).
 
-    Returns o (N,H,D) with o[dst] = sum_e softmax_dst(q[dst].k[src]/sqrt(D)) * v[src]."""
+    Returns o (N,H,D) with o[dst] = sum_e softmax_dst(q[dst].k[src]/sqrt(D)) * v[src].  ak (E,D): rows of the
+    relative-position table per edge (attention.py:69-71).  drop (E,H): multipliers that dropout applies to the
+    attention probabilities, 0 or 1/(1-p) (attention.py:73)."""
     n, h, d = q.shape
     s = (k[src] * q[dst]).sum(-1)                              # (E,H)   attention.py:66-67
     if ak is not None:
@@ -25,11 +27,13 @@ def attention(src, dst, q, k, v, ak=None):
     p = torch.exp(s - m[dst])                                  # graphop_kernel.cu:180-192
     z = torch.zeros((n, h), dtype=s.dtype).index_add_(0, dst, p)
     a = p / z[dst]                                             # graphop_kernel.cu:194-202
+    if drop is not None:
+        a = a * drop                                           # attention.py:73
     o = torch.zeros_like(v).index_add_(0, dst, a.unsqueeze(-1) * v[src])   # attention.py:74-77
     return o
 
 
-def attention_fwd_bwd(src, dst, q, k, v, do, ak=None):
+def attention_fwd_bwd(src, dst, q, k, v, do, ak=None, drop=None):
     q = q.detach().clone().requires_grad_(True)
     k = k.detach().clone().requires_grad_(True)
     v = v.detach().clone().requires_grad_(True)
@@ -37,6 +41,6 @@ def attention_fwd_bwd(src, dst, q, k, v, do, ak=None):
     if ak is not None:
         ak = ak.detach().clone().requires_grad_(True)
         leaves.append(ak)
-    o = attention(src, dst, q, k, v, ak)
+    o = attention(src, dst, q, k, v, ak, drop)
     grads = torch.autograd.grad(o, leaves, do)
     return (o.detach(),) + tuple(grads)

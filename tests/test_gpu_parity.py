@@ -359,3 +359,61 @@ def test_zero_degree_rows_are_zero(ops):
     assert torch.all(y[0] == 0)
     o, lse = graphop.attention_forward(*c.inn, x, x, x)
     assert torch.all(o[0] == 0)
+
+
+# --------------------------------------------------------------------------------------------
+# dropout on the attention probabilities inside the fused kernels (modules/attention.py:73)
+# --------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,hd", [(torch.float32, (8, 64)), (torch.float32, (16, 64)), (torch.bfloat16, (8, 64))])
+@pytest.mark.parametrize("gname,rows", [("bpt512_k4", 4), ("bpt512_k4", 8), ("multigraph", 4), ("fc_w100", 8)])
+def test_fused_attention_dropout_matches_oracle_with_the_same_mask(ops, gname, rows, dtype, hd):
+    from oracle import torch_ops
+    graphop, op = ops
+    h, d = hd
+    p, seed = 0.25, 1234567890123
+    c = case(gname)
+    q, k, v, do = (rand((c.n, h, d), dtype, s, 1.0 / 8).to(DEV) for s in (21, 22, 23, 24))
+    q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+    old_r = graphop.set_group_rows(rows)
+    ctx = long_items(gname)
+    ctx.__enter__()
+    try:
+        mask = graphop.attention_dropout_mask(*c.inn, q, k, p, seed)          # (E, h): 0 or 1 / (1 - p)
+        o = op.bpt_attention(*c.out, *c.inn, q, k, v, dropout_p=p, seed=seed)
+        o.backward(do)
+        o2 = op.bpt_attention(*c.out, *c.inn, q, k, v, dropout_p=p, seed=seed)
+        o3 = op.bpt_attention(*c.out, *c.inn, q, k, v, dropout_p=p, seed=seed + 1)
+    finally:
+        ctx.__exit__()
+        graphop.set_group_rows(old_r)
+    vals = mask.numpy()
+    assert np.all((vals == 0) | (np.abs(vals - 1 / (1 - p)) < 1e-6))
+    kept = float((mask > 0).float().mean())
+    assert abs(kept - (1 - p)) < 4 * np.sqrt(p * (1 - p) / mask.numel()) + 1e-3, kept      # Bernoulli(1 - p) per (edge, head)
+    assert torch.equal(o, o2) and not torch.equal(o, o3)                                  # a function of the seed
+    t64 = lambda x: x.detach().cpu().double()
+    src, dst = torch.from_numpy(c.src), torch.from_numpy(c.dst)
+    ro, rdq, rdk, rdv = torch_ops.attention_fwd_bwd(src, dst, t64(q), t64(k), t64(v), t64(do), drop=mask.double())
+    close(o, ro.numpy(), TOL[dtype], "o", c.max_deg)
+    close(q.grad, rdq.numpy(), GTOL[dtype], "dq", c.max_deg)
+    close(k.grad, rdk.numpy(), GTOL[dtype], "dk", c.max_deg)
+    close(v.grad, rdv.numpy(), GTOL[dtype], "dv", c.max_deg)
+
+
+def test_block_uses_fused_dropout_in_training(ops):
+    from bpt_amd.block import BPTBlock
+    from bpt_amd import graphbuilder as gb
+    c = case("bpt300_causal_k2")
+    csr = gb.get_csrs(c.src, c.dst, c.n)
+    csr_dev = tuple(tuple(t.to(DEV) for t in x) if isinstance(x, (tuple, list)) else x.to(DEV) for x in csr)
+    torch.manual_seed(3)
+    blk = BPTBlock(512, 8, 128, rel_pos=False, drop_h=0.0, drop_a=0.3).to(DEV)
+    h0 = torch.randn(c.n, 512, device=DEV)
+    blk.train()
+    torch.manual_seed(11); a = blk(h0, csr_dev)
+    torch.manual_seed(11); b = blk(h0, csr_dev)
+    torch.manual_seed(12); d_ = blk(h0, csr_dev)
+    blk.eval()
+    e = blk(h0, csr_dev)
+    assert torch.equal(a, b) and not torch.equal(a, d_) and not torch.equal(a, e)
+    assert torch.isfinite(a).all()
