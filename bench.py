@@ -271,7 +271,7 @@ def main():
 
     step_gbs = alg["total"] / t_step / 1e9
     out = {
-        "metric": "attention edges/s fwd+bwd at n=8192 k=4 8h x64; % of HBM roofline",
+        "metric": "attention edges/s fwd+bwd at n=8192 k=4 8h\u00d764; % of HBM roofline",
         "value": E / t_step, "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype_name, "data": "synthetic",
