@@ -29,7 +29,7 @@ def attention(src, dst, q, k, v, ak=None, drop=None):
     a = p / z[dst]                                             # graphop_kernel.cu:194-202
     if drop is not None:
         a = a * drop                                           # attention.py:73
-    o = torch.zeros_like(v).index_add_(0, dst, a.unsqueeze(-1) * v[src])   # attention.py:74-77
+    o = torch.zeros((n,) + tuple(v.shape[1:]), dtype=v.dtype).index_add_(0, dst, a.unsqueeze(-1) * v[src])   # attention.py:74-77
     return o
 
 

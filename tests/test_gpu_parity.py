@@ -417,3 +417,46 @@ def test_block_uses_fused_dropout_in_training(ops):
     e = blk(h0, csr_dev)
     assert torch.equal(a, b) and not torch.equal(a, d_) and not torch.equal(a, e)
     assert torch.isfinite(a).all()
+
+
+# --------------------------------------------------------------------------------------------
+# attention to memory over an inter graph (modules/attention.py:144-168, graph/mt.py:318-347): bipartite blocks
+# from encoder nodes to decoder nodes in one index space of max(n_enc, n_dec) nodes, most rows without edges
+# --------------------------------------------------------------------------------------------
+def inter_graph(n_enc, n_dec, seg_enc, seg_dec):
+    rows, cols = [], []
+    e0 = d0 = 0
+    for le, ld in zip(seg_enc, seg_dec):
+        src = np.arange(e0, e0 + le); dst = np.arange(d0, d0 + ld)
+        rows.append(np.repeat(src, ld)); cols.append(np.tile(dst, le))     # graph/mt.py:318-321
+        e0 += le + 3; d0 += ld + 2                                          # internal (span) nodes in between have no inter edges
+    assert e0 <= n_enc + 3 and d0 <= n_dec + 2
+    return np.concatenate(rows).astype(np.int64), np.concatenate(cols).astype(np.int64), max(n_enc, n_dec)
+
+
+@pytest.mark.parametrize("n_enc,n_dec", [(200, 120), (150, 150)])     # the reference needs n_dec <= n_enc: y = zeros_like(v)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_to_memory_over_an_inter_graph(ops, n_enc, n_dec, dtype):
+    from bpt_amd import graphbuilder as gb
+    from oracle import torch_ops
+    graphop, op = ops
+    h, d = 8, 64
+    src, dst, n = inter_graph(n_enc, n_dec, [40, 70, 25], [30, 20, 45])
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, n)
+    t = lambda a: a.to(DEV)
+    graph = (t(ROW), t(IR), t(out_csr[2]), t(out_csr[1]), t(COL), t(IC), t(in_csr[2]), t(in_csr[1]))
+    # queries: decoder states padded to the memory's length when shorter (attention.py:148-149); keys/values: the memory
+    nq = max(n_dec, n_enc)
+    q = rand((nq, h, d), dtype, 31, 1.0 / 8).to(DEV).requires_grad_(True)
+    k = rand((n_enc, h, d), dtype, 32, 1.0 / 8).to(DEV).requires_grad_(True)
+    v = rand((n_enc, h, d), dtype, 33, 1.0 / 8).to(DEV).requires_grad_(True)
+    do = rand((nq, h, d), dtype, 34, 1.0 / 8).to(DEV)
+    o = op.bpt_attention(*graph, q, k, v)          # fused when q and k have the same number of rows, else the op chain
+    o.backward(do)
+    t64 = lambda x: x.detach().cpu().double()
+    ro, rdq, rdk, rdv = torch_ops.attention_fwd_bwd(torch.from_numpy(src), torch.from_numpy(dst), t64(q), t64(k), t64(v), t64(do))
+    close(o, ro.numpy(), TOL[dtype], "o", 70)
+    close(q.grad, rdq.numpy(), GTOL[dtype], "dq", 70)
+    close(k.grad, rdk.numpy(), GTOL[dtype], "dk", 70)
+    close(v.grad, rdv.numpy(), GTOL[dtype], "dv", 70)
+    assert not o[min(n_dec, 101):].any()             # rows without in-edges (span nodes, padding) stay zero
