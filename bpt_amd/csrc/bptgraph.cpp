@@ -382,8 +382,9 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
     if (!items || !members || !grp_ptr || !chunks || !n_groups_out || !n_entries_out) return BPTG_ERR_NULL;
     if (n_edges > 0 && (!idx32 || !eid32 || !entries || !pair_eid)) return BPTG_ERR_NULL;
     if (n_items < 0 || n_edges < 0 || n_index_nodes < 0) return BPTG_ERR_SIZE;
-    if (R < 1 || R > 16 || window < 0 || order_mode < 0 || order_mode > 7 || max_pairs < 0) return BPTG_ERR_ARG;
-    const bool by_mask = (order_mode & 4) != 0;
+    if (R < 1 || R > 16 || window < 0 || order_mode < 0 || order_mode > 15 || max_pairs < 0) return BPTG_ERR_ARG;
+    const bool aligned = (order_mode & 8) != 0;
+    const bool by_mask = (order_mode & 4) != 0 && !aligned;
     order_mode &= 3;
     for (int64_t i = 0; i < n_items; ++i) {
         const int32_t *it = items + 4 * i;
@@ -489,25 +490,16 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
     struct Triple { int32_t idx, member, eid; };
     struct Entry { int32_t idx, mask, eids[16]; };
     std::vector<Triple> tri;
-    std::vector<Entry> ents;
-    int64_t n_entries = 0, n_pairs = 0;
-    grp_ptr[0] = 0;
-    for (int64_t gi = 0; gi < n_groups; ++gi) {
-        const int32_t *gmem = &grp_items[(size_t)gorder[(size_t)gi] * R];
+    std::vector<Entry> ents, placed;
+    // the entries of one group in neighbour order
+    auto collect = [&](const int32_t *gmem) {
         tri.clear();
         ents.clear();
-        for (int32_t m = 0; m < R; ++m) {
-            int32_t *mem = members + ((int64_t)gi * R + m) * 2;
+        for (int32_t m = 0; m < R; ++m)
             if (gmem[m] >= 0) {
                 const int32_t *it = items + 4 * (int64_t)gmem[m];
-                mem[0] = it[0];
-                mem[1] = it[3];
                 for (int32_t p = it[1]; p < it[2]; ++p) tri.push_back({idx32[p], m, eid32[p]});
-            } else {
-                mem[0] = -1;
-                mem[1] = -1;
             }
-        }
         std::stable_sort(tri.begin(), tri.end(), [](const Triple &a, const Triple &b) {
             return a.idx != b.idx ? a.idx < b.idx : a.member < b.member;
         });
@@ -536,6 +528,64 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
                 ents.push_back(en);
             }
             a = b;
+        }
+    };
+    // Aligned order: walking the groups in locality order, a neighbour keeps the position (the time step) it had
+    // in the last group that read it whenever that position is free, and the other entries fill the gaps.  Wavefronts
+    // that run side by side at the same pace then ask for a shared row at about the same time.
+    std::vector<int32_t> pos_of;                 // per group (locality order): position of each entry
+    std::vector<int64_t> pos_ptr;
+    if (aligned) {
+        std::vector<int32_t> lastpos((size_t)n_index_nodes, -1);
+        std::vector<uint8_t> taken;
+        pos_ptr.assign((size_t)n_groups + 1, 0);
+        for (int64_t g = 0; g < n_groups; ++g) {
+            collect(&grp_items[(size_t)g * R]);
+            const int32_t n = (int32_t)ents.size();
+            const size_t base = pos_of.size();
+            pos_of.resize(base + (size_t)n, -1);
+            taken.assign((size_t)n, 0);
+            for (int32_t e = 0; e < n; ++e) {
+                if (e > 0 && ents[(size_t)e].idx == ents[(size_t)e - 1].idx) continue;      // repeats only fill gaps
+                const int32_t lp = lastpos[(size_t)ents[(size_t)e].idx];
+                if (lp >= 0 && lp < n && !taken[(size_t)lp]) {
+                    pos_of[base + (size_t)e] = lp;
+                    taken[(size_t)lp] = 1;
+                }
+            }
+            int32_t f = 0;
+            for (int32_t e = 0; e < n; ++e) {
+                if (pos_of[base + (size_t)e] < 0) {
+                    while (taken[(size_t)f]) ++f;
+                    pos_of[base + (size_t)e] = f;
+                    taken[(size_t)f] = 1;
+                }
+                lastpos[(size_t)ents[(size_t)e].idx] = pos_of[base + (size_t)e];
+            }
+            pos_ptr[(size_t)g + 1] = (int64_t)pos_of.size();
+        }
+    }
+    int64_t n_entries = 0, n_pairs = 0;
+    grp_ptr[0] = 0;
+    for (int64_t gi = 0; gi < n_groups; ++gi) {
+        const int32_t *gmem = &grp_items[(size_t)gorder[(size_t)gi] * R];
+        for (int32_t m = 0; m < R; ++m) {
+            int32_t *mem = members + ((int64_t)gi * R + m) * 2;
+            if (gmem[m] >= 0) {
+                const int32_t *it = items + 4 * (int64_t)gmem[m];
+                mem[0] = it[0];
+                mem[1] = it[3];
+            } else {
+                mem[0] = -1;
+                mem[1] = -1;
+            }
+        }
+        collect(gmem);
+        if (aligned) {
+            const int64_t base = pos_ptr[(size_t)gorder[(size_t)gi]];
+            placed.resize(ents.size());
+            for (size_t e = 0; e < ents.size(); ++e) placed[(size_t)pos_of[(size_t)base + e]] = ents[e];
+            ents.swap(placed);
         }
         // equal masks next to each other (larger masks first), neighbour order kept inside a mask
         if (by_mask) std::stable_sort(ents.begin(), ents.end(), [](const Entry &x, const Entry &y) { return x.mask > y.mask; });

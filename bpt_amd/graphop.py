@@ -16,7 +16,7 @@ import math
 import torch
 
 from ._lib import attn_lib, check_attn
-from .plan import plan_cache
+from .plan import GROUP_ORDER_SRC, plan_cache
 
 __all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forward", "node_mul_edge_backward",
            "sparse_softmax_forward", "sparse_softmax_backward", "vector_spmm_forward", "vector_spmm_backward"]
@@ -263,7 +263,7 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     if _USE_GROUPS and plan_in.covers_all_edges and plan_out.covers_all_edges:
         R = _group_rows(q, h, d, plan_in)
         in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
-        out_ref = ctypes.byref(plan_out.ensure_groups(R)["struct"])
+        out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
     with torch.cuda.device_of(q):
         check_attn(_LIB.bpt_attention_backward(in_ref, out_ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do),

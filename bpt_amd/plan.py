@@ -21,6 +21,7 @@ FORCE_SEG_LEN = None    # testing hook: when set, replaces the automatic choice 
 GROUP_R = 4            # default rows per group (the row-group kernels exist for 4 and, float32 with h <= 8 and h*d <= 512, 8)
 GROUP_WINDOW = 32      # how many following items the greedy grouping examines per group
 GROUP_ORDER = 2 + 4    # groups inside an XCD chunk by decreasing work (2); entries of a group sorted by member mask (+4)
+GROUP_ORDER_SRC = 2 + 8  # source-side groups of the fused backward: aligned entry order (+8), which lowers that kernel's HBM reads
 GROUP_MAX_PAIRS = None  # cap on the edges of one group: None = 48 per member row, 0 = no cap
 GROUP_PAD_ENTRIES = 8  # the kernels' software pipeline reads per-entry arrays this far past the end
 _CACHE_SIZE = 64
@@ -167,13 +168,14 @@ class Plan:
         return ctypes.byref(self.struct)
 
     # ---- row groups for the fused attention kernels ----
-    def ensure_groups(self, R=GROUP_R):
+    def ensure_groups(self, R=GROUP_R, order_mode=None):
         """Builds the row-group arrays for groups of R rows once (host) and uploads them.  Returns a dict with
         the host arrays ("host") and the `bpt_plan` carrying them ("struct")."""
+        order_mode = GROUP_ORDER if order_mode is None else order_mode
         with self._lock:
-            hit = self._groups.get(R)
+            hit = self._groups.get((R, order_mode))
             if hit is None:
-                grp = build_groups_host(self._host, self.n_index_nodes, R=R)
+                grp = build_groups_host(self._host, self.n_index_nodes, R=R, order_mode=order_mode)
                 dev = {k: torch.from_numpy(grp[k]).to(self.device) for k in ("members", "grp_ptr", "entries", "chunks")}
                 n_groups = len(grp["members"])
                 st = PlanStruct.from_buffer_copy(self.struct)
@@ -187,13 +189,13 @@ class Plan:
                 st.grp_R = R
                 st.n_grp_entries = len(grp["entries"])
                 hit = {"host": grp, "dev": dev, "struct": st}
-                self._groups[R] = hit
+                self._groups[(R, order_mode)] = hit
         return hit
 
     def linked_to(self, plan_src, R=GROUP_R):
         """`bpt_plan` of this (destination-side) plan whose grp_pairs maps each (entry, member) of its groups to
         the position entry' * R + member' of the same edge in `plan_src` (the source-side plan of the same graph)."""
-        mine, theirs = self.ensure_groups(R), plan_src.ensure_groups(R)
+        mine, theirs = self.ensure_groups(R), plan_src.ensure_groups(R, GROUP_ORDER_SRC)
         key = (id(plan_src), R)
         with self._lock:
             hit = self._links.get(key)

@@ -93,7 +93,10 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
  *   chunks   int32[9]             groups chunks[x] .. chunks[x+1]-1 go to XCD x (contiguous, about equal work)
  * order_mode: low two bits = order of the groups inside a chunk — 0 locality, 1 at-least-average work first
  * then the small ones, 2 decreasing work; + 4 = inside a group, entries with equal member masks are made
- * adjacent (larger masks first, neighbour order kept among equal masks) instead of plain neighbour order.
+ * adjacent (larger masks first, neighbour order kept among equal masks) instead of plain neighbour order;
+ * + 8 = aligned order (overrides + 4): going through the groups in locality order, a neighbour keeps the position
+ * it had in the last group that read it whenever that position is free and the rest fill the gaps, so that
+ * wavefronts running side by side ask for a shared row at about the same time.
  * max_pairs: no item joins a group whose edges would then number more than this (0 = no limit); it bounds
  * the work of the wavefront that walks the group.
  * A neighbour that a member reaches through several parallel edges gets one entry per multiplicity. */

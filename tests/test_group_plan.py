@@ -37,7 +37,7 @@ def plans(name, seg=64):
 
 
 @pytest.mark.parametrize("GROUP_R", [4, 16])
-@pytest.mark.parametrize("order_mode", [0, 1, 2, 6])
+@pytest.mark.parametrize("order_mode", [0, 1, 2, 6, 10])
 @pytest.mark.parametrize("seg", [8, 64])
 @pytest.mark.parametrize("name", sorted(GRAPHS))
 def test_group_plan_invariants(name, seg, order_mode, GROUP_R):
@@ -66,7 +66,7 @@ def test_group_plan_invariants(name, seg, order_mode, GROUP_R):
         n_pairs = 0
         for g in range(ng):
             masks = entries[gptr[g]:gptr[g + 1], 1]
-            if order_mode & 4:
+            if order_mode & 4 and not order_mode & 8:
                 assert np.all(np.diff(masks) <= 0)                # equal masks adjacent, larger first
             for u in range(gptr[g], gptr[g + 1]):
                 idx, mask, pb, _ = entries[u].tolist()
