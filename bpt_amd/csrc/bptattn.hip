@@ -1152,6 +1152,234 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
     }
 }
 
+// ---- matrix-core forward for groups of 8 rows -------------------------------------------------------------------
+// v_mfma_f32_4x4x1 works on 16 blocks of 4 lanes: D_b[i][j] += A_b[i] * B_b[j] with A_b[i] taken from lane 4b+i,
+// B_b[j] from lane 4b+j and D_b[i][j] held in register i of lane 4b+j.  Block b owns the 4 * EPL columns that its
+// four lanes hold in the row layout (all of one head).
+//   scores   S^T = K Q^T: lane 4b+i supplies column c of the row of entry i (of a batch of four), lane 4b+j column c
+//            of the q row of member j; after one instruction per column of the block and a sum over the blocks of a
+//            head, register i of lane 4b+j holds (entry i, member j).  The rows reach this "one row per lane of a
+//            block" arrangement through LDS: written as loaded, read back by (row, block).
+//   output   O += P V: A = the lane's own probability (member j = lane % 4, entry e), B = register r of the V row
+//            of entry e in the row layout; D is the accumulator of (member i, this lane's r-th column).
+// A wavefront issues at most one instruction every eight cycles, so the time of a group is its instruction count:
+// the matrix-core form needs about a third of the instructions per (entry, member) of the vector form.
+// The exponent reference of a (member, head) is raised only when a score exceeds it by more than MFMA_TAU (base-2
+// units), so the accumulators are rescaled rarely; probabilities stay below 2^MFMA_TAU times the usual ones, and
+// o and lse come out the same up to rounding.
+constexpr float MFMA_TAU = 8.f;
+constexpr int MFMA_NB = 4;                          // entries per batch = rows of the A operand
+
+// sum over the blocks (quads of lanes) that hold one head; the result is in all of them.  Every lane has to take
+// part: a lane switched off by a branch would hand zero to its partners.
+template <int BPH> __device__ __forceinline__ float block_sum(float x) {
+    if constexpr (BPH >= 2) x += dpp_mov<0x1B>(dpp_mov<0x141>(x));     // lane ^ 4: row_half_mirror, then quad_perm [3,2,1,0]
+    if constexpr (BPH >= 4) x += dpp_mov<0x141>(dpp_mov<0x140>(x));    // lane ^ 8: row_mirror, then row_half_mirror
+    return x;
+}
+template <int I> __device__ __forceinline__ float quad_lane(float x) { return dpp_mov<I * 0x55>(x); }   // value of lane I of the quad
+
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// 16-byte vector as VE floats
+template <typename T> __device__ __forceinline__ void unpack_vec(const uint4 &w, float *out) {
+    const uint32_t x[4] = {w.x, w.y, w.z, w.w};
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) out[c] = __uint_as_float(x[c]);
+    } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            out[2 * c] = __uint_as_float(x[c] << 16);
+            out[2 * c + 1] = __uint_as_float(x[c] & 0xffff0000u);
+        }
+    }
+}
+
+// Two wavefronts per group of 8 rows: wavefront w owns members 4 w .. 4 w + 3 (one quad: the B operand of the
+// score products), both share the staged rows.  Each wavefront loads and stages half of a batch; the staging area
+// is double buffered, so one workgroup barrier per batch orders the writes of batch b + 1 after the reads of
+// batch b - 1.
+template <typename T, int H, int D, int HS, bool DROP>
+__global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) void k_attn_fwd_mfma(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
+    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr,
+    uint32_t drop_seed, float drop_inv) {
+    constexpr int R = 8, NB = MFMA_NB, HL = H / HS, CF = H * D, NE = NB / 2;      // NE: entries a wavefront loads per batch
+    using L = Lay<T, HL, D>;
+    constexpr int EPL = L::EPL, NV = L::NV, VE = L::VE, BPH = L::LPH / 4, CB = 4 * EPL, PITCH = NV * WAVE + 1;
+    static_assert(EPL % VE == 0 && EPL <= 8 && (BPH == 1 || BPH == 2 || BPH == 4), "shape not covered by the matrix-core kernels");
+    const int lane = threadIdx.x & (WAVE - 1), wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // the group of this workgroup (as fetch_group, for workgroups of two wavefronts)
+    int rows[4], slots[4], g_begin, g_end;
+    {
+        const int x = blockIdx.x & 7, w = (blockIdx.x >> 3) / HS;
+        const int g = __builtin_amdgcn_readfirstlane(P.grp_chunks[x]) + w;
+        if (g >= __builtin_amdgcn_readfirstlane(P.grp_chunks[x + 1])) return;
+        const int mem = P.grp_members[(size_t)g * (2 * R) + (lane & (2 * R - 1))];
+        const int ptr = P.grp_ptr[g + (lane & 1)];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            rows[i] = __builtin_amdgcn_readlane(mem, 8 * wv + 2 * i);
+            slots[i] = __builtin_amdgcn_readlane(mem, 8 * wv + 2 * i + 1);
+        }
+        g_begin = __builtin_amdgcn_readlane(ptr, 0);
+        g_end = __builtin_amdgcn_readlane(ptr, 1);
+    }
+    const int slice = (int)((blockIdx.x >> 3) % HS), coff = slice * HL * D;
+    const int head = slice * HL + lane / L::LPH, j = lane & 3, blk = lane >> 2;
+    const uint32_t loff = (uint32_t)((coff + L::off(lane, 0)) * sizeof(T));
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    __shared__ uint4 kst[2][NB * PITCH];              // rows as loaded, one spare vector per row against bank conflicts
+    __shared__ uint4 vst[2][NB * NV * WAVE];
+    float qb[CB];                                      // q row of member 4 wv + j, the columns of this lane's block, pre-scaled
+    {
+        // wavefront 0 stages its q rows through the K area, wavefront 1 through the V area
+        uint4 *qst = wv == 0 ? &kst[0][0] : &vst[0][0];
+        constexpr int QP = NV * WAVE;                  // unpadded: four rows fill either area exactly
+        RawRow<T, HL, D> qr[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_row32_raw<T, HL, D, CF>(q, (uint32_t)max(rows[i], 0), loff, qr[i]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int c = 0; c < NV; ++c) qst[i * QP + c * WAVE + lane] = make_uint4(qr[i].w[4 * c], qr[i].w[4 * c + 1], qr[i].w[4 * c + 2], qr[i].w[4 * c + 3]);
+        wave_lds_fence();
+#pragma unroll
+        for (int t = 0; t < NV * 4; ++t) unpack_vec<T>(qst[j * QP + (t / 4) * WAVE + 4 * blk + (t % 4)], &qb[t * VE]);
+#pragma unroll
+        for (int c = 0; c < CB; ++c) qb[c] *= scale_log2e;
+    }
+    floatx4 acc[EPL];                                  // [row register r][member 4 wv + i]
+    float mref = M_INIT_LOG2, lrun = 0.f;
+#pragma unroll
+    for (int r = 0; r < EPL; ++r) acc[r] = floatx4{0.f, 0.f, 0.f, 0.f};
+    struct Raw { RawRow<T, HL, D> kr[NE], vr[NE]; };
+    for (int p0 = g_begin; p0 < g_end; p0 += GRP_CHUNK) {
+        const int cnt = min(GRP_CHUNK, g_end - p0);
+        int4 ent = entries[p0 + min(lane, cnt - 1)];    // lanes past the end repeat the last entry with an empty mask
+        ent.y = lane < cnt ? ent.y : 0;
+        auto load_half = [&](Raw &B, int b) {          // this wavefront's entries of batch b
+#pragma unroll
+            for (int e = 0; e < NE; ++e) {
+                const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + NE * wv + e);
+                load_row32_raw<T, HL, D, CF>(k, src, loff, B.kr[e]);
+                load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
+            }
+        };
+        auto stage_half = [&](const Raw &B, int buf) {
+#pragma unroll
+            for (int e = 0; e < NE; ++e)
+#pragma unroll
+                for (int c = 0; c < NV; ++c) {
+                    kst[buf][(NE * wv + e) * PITCH + c * WAVE + lane] = make_uint4(B.kr[e].w[4 * c], B.kr[e].w[4 * c + 1], B.kr[e].w[4 * c + 2], B.kr[e].w[4 * c + 3]);
+                    vst[buf][((NE * wv + e) * NV + c) * WAVE + lane] = make_uint4(B.vr[e].w[4 * c], B.vr[e].w[4 * c + 1], B.vr[e].w[4 * c + 2], B.vr[e].w[4 * c + 3]);
+                }
+        };
+        Raw raw;
+        load_half(raw, 0);
+        __syncthreads();                               // the staging area is free (q rows, the previous chunk's last batch)
+        stage_half(raw, 0);
+        load_half(raw, NB);
+        __syncthreads();
+        for (int b = 0, buf = 0; b < cnt; b += NB, buf ^= 1) {
+            int mk[NB], pz[NB];
+#pragma unroll
+            for (int e = 0; e < NB; ++e) {
+                mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
+                pz[e] = DROP ? __builtin_amdgcn_readlane(ent.z, b + e) : 0;
+            }
+            // all LDS reads of the batch go out first: the K rows of this lane's entry by block, the V rows as loaded
+            uint4 kv[NV * 4], vv[NB][NV];
+#pragma unroll
+            for (int t = 0; t < NV * 4; ++t) kv[t] = kst[buf][j * PITCH + (t / 4) * WAVE + 4 * blk + (t % 4)];
+#pragma unroll
+            for (int e = 0; e < NB; ++e)
+#pragma unroll
+                for (int c = 0; c < NV; ++c) vv[e][c] = vst[buf][(e * NV + c) * WAVE + lane];
+            issue_loads_first();
+            // scores: register e of lane 4 blk + j = (entry e, member 4 wv + j), head of the block
+            floatx4 st[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) st[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < NV * 4; ++t) {
+                float kf[VE];
+                unpack_vec<T>(kv[t], kf);
+#pragma unroll
+                for (int c = 0; c < VE; ++c) st[c & 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(kf[c], qb[t * VE + c], st[c & 3], 0, 0, 0);
+            }
+            float sc[NB];
+#pragma unroll
+            for (int e = 0; e < NB; ++e) sc[e] = block_sum<BPH>((st[0][e] + st[1][e]) + (st[2][e] + st[3][e]));
+#pragma unroll
+            for (int e = 0; e < NB; ++e) sc[e] = ((mk[e] >> (4 * wv + j)) & 1) ? sc[e] : -INFINITY;
+            const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
+                const float mn = fmaxf(mref, mb);
+                const float al = __builtin_amdgcn_exp2f(mref - mn);
+                mref = mn;
+                lrun *= al;
+                const float a0 = quad_lane<0>(al), a1 = quad_lane<1>(al), a2 = quad_lane<2>(al), a3 = quad_lane<3>(al);
+#pragma unroll
+                for (int r = 0; r < EPL; ++r) {
+                    acc[r][0] *= a0; acc[r][1] *= a1; acc[r][2] *= a2; acc[r][3] *= a3;
+                }
+            }
+            float pk[NB];
+#pragma unroll
+            for (int e = 0; e < NB; ++e) {
+                const float pe = __builtin_amdgcn_exp2f(sc[e] - mref);
+                lrun += pe;                                          // the softmax denominator ignores dropout
+                if constexpr (DROP) {
+                    const int n = pz[e] + __builtin_popcount(mk[e] & ((1 << (4 * wv + j)) - 1));
+                    pk[e] = pe * dropout_keep((uint32_t)(n * H + head), drop_seed, drop_thr, drop_inv);
+                } else {
+                    pk[e] = pe;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < NB; ++e) {
+                float vf[EPL];
+#pragma unroll
+                for (int c = 0; c < NV; ++c) unpack_vec<T>(vv[e][c], &vf[c * VE]);
+#pragma unroll
+                for (int r = 0; r < EPL; ++r) acc[r] = __builtin_amdgcn_mfma_f32_4x4x1f32(pk[e], vf[r], acc[r], 0, 0, 0);
+            }
+            // the other buffer was last read one batch ago, before the previous barrier
+            stage_half(raw, buf ^ 1);
+            load_half(raw, b + 2 * NB);                // look-ahead (past the end: the last entry again, unused)
+            __syncthreads();
+        }
+    }
+    const float ls[4] = {quad_lane<0>(lrun), quad_lane<1>(lrun), quad_lane<2>(lrun), quad_lane<3>(lrun)};
+    const float ms[4] = {quad_lane<0>(mref), quad_lane<1>(mref), quad_lane<2>(mref), quad_lane<3>(mref)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (rows[i] < 0) continue;
+        float out[EPL];
+        if (slots[i] < 0) {
+            const float inv = ls[i] > 0.f ? 1.f / ls[i] : 0.f;
+#pragma unroll
+            for (int r = 0; r < EPL; ++r) out[r] = acc[r][i] * inv;
+            store_row<T, HL, D>(o + (size_t)rows[i] * CF + coff, lane, out);
+            if (lane % L::LPH == 0) lse[(size_t)rows[i] * H + head] = ls[i] > 0.f ? ms[i] + log2f(ls[i]) : 0.f;
+        } else {
+#pragma unroll
+            for (int r = 0; r < EPL; ++r) out[r] = acc[r][i];
+            store_row_ws<T, HL, D>(ws_acc + (size_t)slots[i] * CF + coff, lane, out);
+            if (lane % L::LPH == 0) {
+                ws_ml[((size_t)slots[i] * H + head) * 2] = ms[i];
+                ws_ml[((size_t)slots[i] * H + head) * 2 + 1] = ls[i];
+            }
+        }
+    }
+}
+
 // Backward, destination side.  Writes (p, ds) of every pair to pds[(t * H + head)], t = the pair's
 // position (entry * R + member) in the SOURCE-side plan, which P.grp_pairs gives for every
 // (entry, member) of this plan (a spare position for members the entry does not have).  One store per
@@ -1635,6 +1863,21 @@ template <typename T, int H, int D> constexpr int head_slices() {
     return (C > CS && C % CS == 0 && H % (C / CS) == 0) ? C / CS : 1;
 }
 
+// The matrix-core forward gives a wavefront at most 512 columns of every row.  0 slices = shape not covered.
+template <typename T, int H, int D> constexpr int mfma_slices() {
+    constexpr int CS = 512, C = H * D;
+    if (C <= CS) return 1;
+    return (C % CS == 0 && H % (C / CS) == 0) ? C / CS : 0;
+}
+template <typename T, int H, int D> constexpr bool mfma_ok() {
+    constexpr int HS = mfma_slices<T, H, D>();
+    if (HS == 0) return false;
+    constexpr int HL = H / HS, CS = HL * D, VE = 16 / (int)sizeof(T);
+    if (64 % HL != 0 || CS % 64 != 0) return false;
+    constexpr int LPH = 64 / HL, EPL = CS / 64;
+    return (LPH == 4 || LPH == 8 || LPH == 16) && EPL % VE == 0 && EPL <= 8;
+}
+
 // rows per group the row-group kernels exist for
 inline bool group_rows_ok(int64_t R) { return R == 4 || R == 8; }
 
@@ -1669,15 +1912,22 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
 #define LAUNCH_FWD(RR, DR)                                                                                                   \
     hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR, HS, DR>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)q, \
                        (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv)
+#define LAUNCH_FWD_MFMA(DR)                                                                                                  \
+    hipLaunchKernelGGL((k_attn_fwd_mfma<T, H, D, HSM, DR>), dim3(group_grid(P) * HSM), dim3(2 * WAVE), 0, s, *P, (const T *)q, \
+                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv)
             constexpr int HS = head_slices<T, H, D>();
-            if (drop.thr == 0) {
-                if (P->grp_R == 8) LAUNCH_FWD(8, false);
-                else LAUNCH_FWD(4, false);
+            if (P->grp_R == 8) {
+                // every compile-time shape has the matrix-core form for groups of 8
+                static_assert(mfma_ok<T, H, D>(), "groups of 8 rows need the matrix-core forward");
+                constexpr int HSM = mfma_slices<T, H, D>();
+                if (drop.thr == 0) LAUNCH_FWD_MFMA(false);
+                else LAUNCH_FWD_MFMA(true);
             } else {
-                if (P->grp_R == 8) LAUNCH_FWD(8, true);
+                if (drop.thr == 0) LAUNCH_FWD(4, false);
                 else LAUNCH_FWD(4, true);
             }
 #undef LAUNCH_FWD
+#undef LAUNCH_FWD_MFMA
         } else {
             hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
                                (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);

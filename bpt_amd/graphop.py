@@ -234,7 +234,7 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     h, d = _hd(q)
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
-    ref = ctypes.byref(plan.ensure_groups(_group_rows(q, h, d, plan))["struct"]) if _USE_GROUPS else plan.ref
+    ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, dropout_p))["struct"]) if _USE_GROUPS else plan.ref
     o = torch.empty_like(q)
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
@@ -311,6 +311,17 @@ def _group_rows(q, h, d, plan):
         return _GROUP_ROWS
     big = plan.n_items >= 16384 or plan.n_edges >= 64 * max(plan.n_rows, 1)
     return 8 if (big and (q.dtype == torch.float32 or h * d > 512)) else 4
+
+
+def _forward_rows(q, h, d, plan, dropout_p=0.0):
+    """Rows per group for the forward kernel.  Groups of 8 run on the matrix cores (two wavefronts per group), which
+    measured faster than the vector kernels at every float32 size, and for bfloat16 on rows of more than 512 columns
+    and on dense graphs.  With dropout the forward and the backward number the pairs by the same groups."""
+    if _GROUP_ROWS is not None or dropout_p > 0.0:
+        return _group_rows(q, h, d, plan)
+    if q.dtype == torch.float32 or h * d > 512 or plan.n_edges >= 64 * max(plan.n_rows, 1):
+        return 8
+    return _group_rows(q, h, d, plan)
 
 
 def set_group_rows(R):
