@@ -138,7 +138,18 @@ def main():
     q, k, v, do = ((torch.randn(N, H, D, generator=gen) / 8).to(tdtype).to(dev) for _ in range(4))
     log(f"{desc}: N={N} E={E} dtype={dtype_name}; host graph+CSR build {t_graph * 1e3:.1f} ms")
 
-    if args.rel_pos:
+    if args.rel_pos and not args.unfused:
+        # rel_pos inside the fused kernels: per-edge score term from the (1000, d) table, table gradient by SpMMs
+        from bpt_amd import op
+        table = (torch.randn(1000, D, generator=gen) / 8).to(tdtype).to(dev)
+        et = torch.from_numpy(np.asarray(etype, dtype=np.int64)).to(dev)
+
+        def step():
+            qq, kk, vv, tt = (x.detach().requires_grad_(True) for x in (q, k, v, table))
+            o = op.bpt_attention(*gargs, qq, kk, vv, dropout_p=args.dropout, seed=2345, rel_table=tt, etype=et)
+            o.backward(do)
+            return o, qq.grad, kk.grad, vv.grad
+    elif args.rel_pos:
         # the op sequence of modules/attention.py:66-77 with rel_pos on; the (E, d) rows of the table are
         # gathered per step as the reference's nn.Embedding does (backward: segment sums per edge type)
         from bpt_amd import op
@@ -275,7 +286,7 @@ def main():
         "value": E / t_step, "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype_name, "data": "synthetic",
-        "config": {"workload": desc + (" (op chain with rel_pos)" if args.rel_pos else " (unfused op chain)" if args.unfused else
+        "config": {"workload": desc + (" (op chain with rel_pos)" if args.rel_pos and args.unfused else " (fused fwd+bwd with rel_pos)" if args.rel_pos else " (unfused op chain)" if args.unfused else
                                        f" (fused fwd+bwd, attention dropout {args.dropout})" if args.dropout > 0 else " (fused fwd+bwd)"), "n_nodes": N,
                    "n_edges": E, "heads": H, "d_head": D, "launch": mode,
                    "kernels": "per-row" if args.rows else f"row-groups({args.group_rows or 'auto'} rows per wavefront)"},

@@ -18,7 +18,7 @@ class PlanStruct(ctypes.Structure):
                 ("n_rows", c_i64), ("n_edges", c_i64), ("n_items", c_i64), ("n_heavy", c_i64), ("n_slots", c_i64),
                 ("grp_members", c_vp), ("grp_ptr", c_vp), ("grp_entries", c_vp), ("grp_pairs", c_vp),
                 ("grp_chunks", c_vp), ("n_groups", c_i64), ("grp_R", c_i64), ("grp_max_chunk", c_i64),
-                ("n_grp_entries", c_i64)]
+                ("n_grp_entries", c_i64), ("grp_eids", c_vp)]
 
 
 class PlanInfo(ctypes.Structure):
@@ -56,10 +56,11 @@ ATTN_API = {
     "bpt_sparse_softmax_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, ctypes.c_int, ctypes.c_int, c_vp]),
     "bpt_vector_spmm_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_vector_spmm_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
-    "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float, ctypes.c_float,
+    "bpt_rel_bias_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp] + _tail),
+    "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float, ctypes.c_float,
                                             ctypes.c_uint64] + _tail),
-    "bpt_attention_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64,
-                                             ctypes.c_float, ctypes.c_float, ctypes.c_uint64] + _tail),
+    "bpt_attention_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
+                                             c_i64, ctypes.c_float, ctypes.c_float, ctypes.c_uint64] + _tail),
 }
 
 _graph = None

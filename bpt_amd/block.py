@@ -7,8 +7,8 @@ DGL graph object (`g.ndata['h']`, `g.edata['etype']`) and writes the result back
 `forward(h, csr, etype)` takes and returns plain tensors, `csr` being the 6-tuple that
 `graph/base.py:71-86` (`bpt_amd.graphbuilder.get_csrs`) produces.
 
-Attention core: with `rel_pos` off the fused kernels run (`op.bpt_attention`, attention dropout included);
-otherwise the four operators are composed exactly as attention.py:66-77 does.
+Attention core: the fused kernels (`op.bpt_attention`: rel_pos term and attention dropout included), or with
+`fused=False` the four operators composed exactly as attention.py:66-77 does.
 Projections, LayerNorm and the feed-forward are torch modules (rocBLAS GEMMs).
 """
 import math
@@ -37,8 +37,9 @@ class PositionwiseFeedForward(nn.Module):
 class BPTBlock(nn.Module):
     MAX_ETYPE = 1000        # modules/attention.py:23
 
-    def __init__(self, dim_model, h, dim_ff, rel_pos=False, drop_h=0.1, drop_a=0.1):
+    def __init__(self, dim_model, h, dim_ff, rel_pos=False, drop_h=0.1, drop_a=0.1, fused=True):
         super().__init__()
+        self.fused = fused          # False: the four operators composed exactly as attention.py:66-77 does
         self.dim_model, self.h, self.dim_ff = dim_model, h, dim_ff
         self.d_k = dim_model // h
         self.rel_pos = rel_pos
@@ -65,12 +66,13 @@ class BPTBlock(nn.Module):
         out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C = csr
         graph = (ROW, INDPTR_R, out_csr[2], out_csr[1], COL, INDPTR_C, in_csr[2], in_csr[1])
         att_dropout = self.drop_att.p if self.training else 0.0
-        if not self.rel_pos:
-            return bpt_attention(*graph, q, k, v, dropout_p=att_dropout).view(-1, self.d_k * self.h)
+        if self.rel_pos and etype is None:
+            raise ValueError("rel_pos=True needs the edge types (etype)")
+        if self.fused:
+            rel = dict(rel_table=self.embed_ak.weight, etype=etype) if self.rel_pos else {}
+            return bpt_attention(*graph, q, k, v, dropout_p=att_dropout, **rel).view(-1, self.d_k * self.h)
         e = masked_mm(*graph, k, q)
         if self.rel_pos:
-            if etype is None:
-                raise ValueError("rel_pos=True needs the edge types (etype)")
             e = e + node_mul_edge(COL, INDPTR_C, in_csr[2], q, edge_type_embedding(self.embed_ak.weight, etype))
         e = self.drop_att(sparse_softmax(COL, INDPTR_C, in_csr[2], e / math.sqrt(self.d_k)))
         return vec_spmm(COL, INDPTR_C, in_csr[2], in_csr[1], ROW, INDPTR_R, out_csr[2], out_csr[1], e, v).view(

@@ -540,6 +540,16 @@ template <int CTRL> __device__ __forceinline__ float dpp_mov(float x) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
 }
 
+template <int I> __device__ __forceinline__ float quad_lane(float x) { return dpp_mov<I * 0x55>(x); }   // value of lane I of the quad
+__device__ __forceinline__ float quad_bcast(float x, int i) {      // the same for an index that is constant after unrolling
+    switch (i & 3) {
+    case 0: return quad_lane<0>(x);
+    case 1: return quad_lane<1>(x);
+    case 2: return quad_lane<2>(x);
+    default: return quad_lane<3>(x);
+    }
+}
+
 // Sum over the LPH lanes that hold one head; the result is in all of them.
 template <int LPH> __device__ __forceinline__ float head_sum(float x) {
     if constexpr (LPH >= 2) x += dpp_mov<0xB1>(x);    // quad_perm [1,0,3,2]
@@ -566,9 +576,10 @@ __device__ __forceinline__ void issue_loads_first() { __builtin_amdgcn_sched_bar
 // weight loads for the fast SpMM: the unfused API passes T-typed edge data, the fused backward f32
 template <typename WT> __device__ __forceinline__ float ld_w(const WT *p) { return Elem<WT>::ld(p); }
 
-// y[eid[p], head] = A[row, head, :] . B[idx[p], head, :]   (MODE 1: . B[eid[p], :], B an (E, D) edge feature)
-template <typename T, int H, int D, int BATCH, int MODE = 0>
-__global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ y) {
+// y[eid[p], head] = A[row, head, :] . B[idx[p], head, :]   (MODE 1: . B[eid[p], :], B an (E, D) edge feature;
+// MODE 2: . B[idx[p], :], B a (n_index, D) table shared by the heads).  YT: element type of y.
+template <typename T, int H, int D, int BATCH, int MODE = 0, typename YT = T>
+__global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__restrict__ A, const T *__restrict__ B, YT *__restrict__ y) {
     using L = Lay<T, H, D>;
     Item it;
     if (!fetch_item(P, it)) return;
@@ -577,7 +588,7 @@ __global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__res
     load_row<T, H, D>(A + (size_t)it.row * L::C, lane, a);
     for (int p0 = it.begin; p0 < it.end; p0 += WAVE) {
         const int cnt = min(WAVE, it.end - p0);
-        const int my_idx = (MODE == 0 && lane < cnt) ? P.idx[p0 + lane] : 0;
+        const int my_idx = (MODE != 1 && lane < cnt) ? P.idx[p0 + lane] : 0;
         const int my_eid = lane < cnt ? P.eid[p0 + lane] : 0;
         for (int b = 0; b < cnt; b += BATCH) {
             float bv[BATCH][L::EPL];
@@ -587,13 +598,14 @@ __global__ __launch_bounds__(BLOCK) void k_sddmm_fast(bpt_plan P, const T *__res
                 const int j = (b + e < cnt) ? b + e : b;
                 ee[e] = __builtin_amdgcn_readlane(my_eid, j);
                 if constexpr (MODE == 0) load_row<T, H, D>(B + (size_t)__builtin_amdgcn_readlane(my_idx, j) * L::C, lane, bv[e]);
-                else load_head_row<T, H, D>(B + (size_t)ee[e] * D, lane, bv[e]);
+                else if constexpr (MODE == 1) load_head_row<T, H, D>(B + (size_t)ee[e] * D, lane, bv[e]);
+                else load_head_row<T, H, D>(B + (size_t)__builtin_amdgcn_readlane(my_idx, j) * D, lane, bv[e]);
             }
             issue_loads_first();
 #pragma unroll
             for (int e = 0; e < BATCH; ++e) {
                 const float s = head_sum<L::LPH>(dot_n<L::EPL>(a, bv[e]));
-                if (b + e < cnt && lane % L::LPH == 0) Elem<T>::st(y + (size_t)ee[e] * H + head, s);
+                if (b + e < cnt && lane % L::LPH == 0) Elem<YT>::st(y + (size_t)ee[e] * H + head, s);
             }
         }
     }
@@ -1015,14 +1027,14 @@ __device__ __forceinline__ float max3f(float a, float b, float c) {
 
 // Forward: online softmax in base 2 over the group's entries, two entries per step.  The members' q rows
 // (pre-scaled) live in LDS and are re-read for every use, which keeps the kernel at three wavefronts per SIMD.
-template <typename T, int H, int D, int R, int HS, bool DROP>
+template <typename T, int H, int D, int R, int HS, bool DROP, bool BIAS>
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_attn_fwd_grp(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
     float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr,
-    uint32_t drop_seed, float drop_inv) {
+    uint32_t drop_seed, float drop_inv, const float *__restrict__ bias) {
     constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
     using L = Lay<T, HL, D>;
-    constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
+    constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = BIAS ? 1 : grp_batch<L::EPL>()   /* the score term's registers take the place of a second entry */;
     static_assert(H % HS == 0 && R % 4 == 0 && L::LPH >= 4, "members are handled in quads inside the lanes of one head");
     GroupHead<R> gh;
     if (!fetch_group<R, HS>(P, gh)) return;
@@ -1033,11 +1045,13 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
     struct Batch {
         RawRow<T, HL, D> kr[GRP_BATCH], vr[GRP_BATCH];
         int mk[GRP_BATCH], pz[GRP_BATCH];
+        float bz[GRP_BATCH][BIAS ? R / 4 : 1];      // score term of (entry, member 4c + lane % 4), this lane's head
     };
     struct Rows {
         float kv[GRP_BATCH][EPL], vv[GRP_BATCH][EPL];
         int mk[GRP_BATCH], pz[GRP_BATCH];
     };
+    const int4 *eids4 = reinterpret_cast<const int4 *>(P.grp_eids);
     __shared__ float4 q_lds[R * (EPL / 4) * WAVE];
     float acc[R][EPL], mrun[R], lrun[R];
 #pragma unroll
@@ -1055,12 +1069,28 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
         // lanes past the end repeat the last entry with an empty mask
         int4 ent = entries[p0 + min(lane, cnt - 1)];
         ent.y = lane < cnt ? ent.y : 0;
+        // edge ids of the lane's entry, four members per vector (the list is padded like the entries)
+        int4 xe[R / 4];
+        if constexpr (BIAS) {
+#pragma unroll
+            for (int c = 0; c < R / 4; ++c) xe[c] = eids4[(size_t)(p0 + min(lane, cnt - 1)) * (R / 4) + c];
+        }
         auto load_batch = [&](Batch &B, int b) {
 #pragma unroll
             for (int e = 0; e < GRP_BATCH; ++e) {
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
                 B.pz[e] = DROP ? __builtin_amdgcn_readlane(ent.z, b + e) : 0;
+                if constexpr (BIAS) {
+#pragma unroll
+                    for (int c = 0; c < R / 4; ++c) {
+                        // lane l fetches the term of member 4c + l % 4; the quad's lanes hand it round when it is used
+                        const uint32_t e0 = (uint32_t)__builtin_amdgcn_readlane(xe[c].x, b + e), e1 = (uint32_t)__builtin_amdgcn_readlane(xe[c].y, b + e);
+                        const uint32_t e2 = (uint32_t)__builtin_amdgcn_readlane(xe[c].z, b + e), e3 = (uint32_t)__builtin_amdgcn_readlane(xe[c].w, b + e);
+                        const uint32_t el = (lane & 3) == 0 ? e0 : (lane & 3) == 1 ? e1 : (lane & 3) == 2 ? e2 : e3;
+                        B.bz[e][c] = bias[(size_t)(el * (uint32_t)H) + head];
+                    }
+                }
                 load_row32_raw<T, HL, D, CF>(k, src, loff, B.kr[e]);
                 load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
             }
@@ -1071,10 +1101,10 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             const int n = pz + __builtin_popcount(mk & ((1 << m) - 1));
             return dropout_keep((uint32_t)(n * H + head), drop_seed, drop_thr, drop_inv);
         };
-        auto one = [&](int m, const float (&kr)[EPL], const float (&vr)[EPL], int mk, int pz) {
+        auto one = [&](int m, const float (&kr)[EPL], const float (&vr)[EPL], int mk, int pz, float bz) {
             float qm[EPL];
             lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
-            const float s = head_sum<L::LPH>(dot_n<EPL>(qm, kr));
+            const float s = head_sum<L::LPH>(dot_n<EPL>(qm, kr)) + bz;
             const float mx = fmaxf(mrun[m], s);
             const float al = __builtin_amdgcn_exp2f(mrun[m] - mx), pe = __builtin_amdgcn_exp2f(s - mx);
             lrun[m] = fmaf(lrun[m], al, pe);                       // the softmax denominator ignores dropout
@@ -1095,13 +1125,18 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 #pragma unroll
             for (int m = 0; m < R; ++m) {
                 const bool h0 = (B.mk[0] >> m) & 1, h1 = (B.mk[GRP_BATCH - 1] >> m) & 1;
+                // the score term in the units of the scaled scores
+                const float z0 = BIAS ? quad_bcast(raw.bz[0][BIAS ? m / 4 : 0], m) * scale_log2e : 0.f;
+                const float z1 = BIAS ? quad_bcast(raw.bz[GRP_BATCH - 1][BIAS ? m / 4 : 0], m) * scale_log2e : 0.f;
                 if constexpr (GRP_BATCH == 1) {
-                    if (h0) one(m, B.kv[0], B.vv[0], B.mk[0], B.pz[0]);
+                    if (h0) one(m, B.kv[0], B.vv[0], B.mk[0], B.pz[0], z0);
                 } else if (h0 && h1) {
                     float qm[EPL];
                     lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
                     float s0 = dot_n<EPL>(qm, B.kv[0]), s1 = dot_n<EPL>(qm, B.kv[GRP_BATCH - 1]);
                     head_sum2<L::LPH>(s0, s1);
+                    s0 += z0;
+                    s1 += z1;
                     const float mx = max3f(mrun[m], s0, s1);
                     const float al = __builtin_amdgcn_exp2f(mrun[m] - mx);
                     const float p0e = __builtin_amdgcn_exp2f(s0 - mx), p1e = __builtin_amdgcn_exp2f(s1 - mx);
@@ -1111,9 +1146,9 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                     for (int i = 0; i < EPL; ++i) acc[m][i] = fmaf(k1, B.vv[GRP_BATCH - 1][i], fmaf(k0, B.vv[0][i], acc[m][i] * al));
                     mrun[m] = mx;
                 } else if (h0) {
-                    one(m, B.kv[0], B.vv[0], B.mk[0], B.pz[0]);
+                    one(m, B.kv[0], B.vv[0], B.mk[0], B.pz[0], z0);
                 } else if (h1) {
-                    one(m, B.kv[GRP_BATCH - 1], B.vv[GRP_BATCH - 1], B.mk[GRP_BATCH - 1], B.pz[GRP_BATCH - 1]);
+                    one(m, B.kv[GRP_BATCH - 1], B.vv[GRP_BATCH - 1], B.mk[GRP_BATCH - 1], B.pz[GRP_BATCH - 1], z1);
                 }
             }
         };
@@ -1177,7 +1212,6 @@ template <int BPH> __device__ __forceinline__ float block_sum(float x) {
     if constexpr (BPH >= 4) x += dpp_mov<0x141>(dpp_mov<0x140>(x));    // lane ^ 8: row_mirror, then row_half_mirror
     return x;
 }
-template <int I> __device__ __forceinline__ float quad_lane(float x) { return dpp_mov<I * 0x55>(x); }   // value of lane I of the quad
 
 __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -1204,11 +1238,11 @@ template <typename T> __device__ __forceinline__ void unpack_vec(const uint4 &w,
 // score products), both share the staged rows.  Each wavefront loads and stages half of a batch; the staging area
 // is double buffered, so one workgroup barrier per batch orders the writes of batch b + 1 after the reads of
 // batch b - 1.
-template <typename T, int H, int D, int HS, bool DROP>
+template <typename T, int H, int D, int HS, bool DROP, bool BIAS>
 __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) void k_attn_fwd_mfma(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
     float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr,
-    uint32_t drop_seed, float drop_inv) {
+    uint32_t drop_seed, float drop_inv, const float *__restrict__ bias) {
     constexpr int R = 8, NB = MFMA_NB, HL = H / HS, CF = H * D, NE = NB / 2;      // NE: entries a wavefront loads per batch
     using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, NV = L::NV, VE = L::VE, BPH = L::LPH / 4, CB = 4 * EPL, PITCH = NV * WAVE + 1;
@@ -1258,7 +1292,10 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     float mref = M_INIT_LOG2, lrun = 0.f;
 #pragma unroll
     for (int r = 0; r < EPL; ++r) acc[r] = floatx4{0.f, 0.f, 0.f, 0.f};
-    struct Raw { RawRow<T, HL, D> kr[NE], vr[NE]; };
+    struct Raw {
+        RawRow<T, HL, D> kr[NE], vr[NE];
+        int xe[BIAS ? NB : 1];                         // edge ids of this lane's member with the batch's entries
+    };
     for (int p0 = g_begin; p0 < g_end; p0 += GRP_CHUNK) {
         const int cnt = min(GRP_CHUNK, g_end - p0);
         int4 ent = entries[p0 + min(lane, cnt - 1)];    // lanes past the end repeat the last entry with an empty mask
@@ -1269,6 +1306,18 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + NE * wv + e);
                 load_row32_raw<T, HL, D, CF>(k, src, loff, B.kr[e]);
                 load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
+            }
+            if constexpr (BIAS) {
+#pragma unroll
+                for (int e = 0; e < NB; ++e) B.xe[e] = P.grp_eids[(size_t)(p0 + b + e) * R + 4 * wv + j];
+            }
+        };
+        // the score terms of a batch are fetched one batch ahead, with the edge ids that came in the batch before
+        float bz[NB];
+        auto load_bias = [&](const Raw &B) {
+            if constexpr (BIAS) {
+#pragma unroll
+                for (int e = 0; e < NB; ++e) bz[e] = bias[(size_t)((uint32_t)B.xe[e] * (uint32_t)H) + head];
             }
         };
         auto stage_half = [&](const Raw &B, int buf) {
@@ -1284,6 +1333,7 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         load_half(raw, 0);
         __syncthreads();                               // the staging area is free (q rows, the previous chunk's last batch)
         stage_half(raw, 0);
+        load_bias(raw);
         load_half(raw, NB);
         __syncthreads();
         for (int b = 0, buf = 0; b < cnt; b += NB, buf ^= 1) {
@@ -1317,7 +1367,7 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
             for (int e = 0; e < NB; ++e) sc[e] = block_sum<BPH>((st[0][e] + st[1][e]) + (st[2][e] + st[3][e]));
 #pragma unroll
-            for (int e = 0; e < NB; ++e) sc[e] = ((mk[e] >> (4 * wv + j)) & 1) ? sc[e] : -INFINITY;
+            for (int e = 0; e < NB; ++e) sc[e] = ((mk[e] >> (4 * wv + j)) & 1) ? (BIAS ? fmaf(bz[e], scale_log2e, sc[e]) : sc[e]) : -INFINITY;
             const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
             if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
                 const float mn = fmaxf(mref, mb);
@@ -1352,6 +1402,7 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
             }
             // the other buffer was last read one batch ago, before the previous barrier
             stage_half(raw, buf ^ 1);
+            load_bias(raw);
             load_half(raw, b + 2 * NB);                // look-ahead (past the end: the last entry again, unused)
             __syncthreads();
         }
@@ -1385,14 +1436,15 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 // (entry, member) of this plan (a spare position for members the entry does not have).  One store per
 // entry and quad of members: lane l carries the pair of member 4c + l % 4; the same register of ds values is
 // the A operand of the MFMA that accumulates dq.  The members' q rows live in LDS.
-template <typename T, int H, int D, int R, int HS, bool DROP>
+template <typename T, int H, int D, int R, int HS, bool DROP, bool BIAS>
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_attn_bwd_dst_grp(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
     const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds,
-    float *__restrict__ ws_dq, float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv) {
+    float *__restrict__ ws_dq, float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv,
+    const float *__restrict__ bias, float *__restrict__ ds_out) {
     constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
     using L = Lay<T, HL, D>;
-    constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
+    constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = BIAS ? 1 : grp_batch<L::EPL>()   /* the score term's registers take the place of a second entry */;
     static_assert(H % HS == 0 && R % 4 == 0 && L::LPH >= 4, "members are handled in quads inside the lanes of one head");
     GroupHead<R> gh;
     if (!fetch_group<R, HS>(P, gh)) return;
@@ -1405,7 +1457,10 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
     struct Batch {
         RawRow<T, HL, D> kr[GRP_BATCH], vr[GRP_BATCH];
         int mk[GRP_BATCH], pz[GRP_BATCH], xp[GRP_BATCH][NQ];
+        int xl[GRP_BATCH][BIAS ? NQ : 1];           // edge id of (entry, member 4c + lane % 4): where ds_out gets this lane's ds
+        float bz[GRP_BATCH][BIAS ? NQ : 1];         // score term of (entry, member 4c + lane % 4), this lane's head
     };
+    const int4 *eids4 = reinterpret_cast<const int4 *>(P.grp_eids);
     __shared__ float4 q_lds[R * (EPL / 4) * WAVE];
     float dov[R][EPL], delta_s[R], lse2[R];
     floatx4 dqa[NQ][EPL];                       // [quad c][row register t][member 4c + i], as the source-side kernel's accumulators
@@ -1429,12 +1484,28 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
         // lanes past the end repeat the last entry with an empty mask
         int4 ent = entries[p0 + min(lane, cnt - 1)];
         ent.y = lane < cnt ? ent.y : 0;
+        // edge ids of the lane's entry, four members per vector (the list is padded like the entries)
+        int4 xe[R / 4];
+        if constexpr (BIAS) {
+#pragma unroll
+            for (int c = 0; c < R / 4; ++c) xe[c] = eids4[(size_t)(p0 + min(lane, cnt - 1)) * (R / 4) + c];
+        }
         auto load_batch = [&](Batch &B, int b) {
 #pragma unroll
             for (int e = 0; e < GRP_BATCH; ++e) {
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
                 B.pz[e] = DROP ? __builtin_amdgcn_readlane(ent.z, b + e) : 0;
+                if constexpr (BIAS) {
+#pragma unroll
+                    for (int c = 0; c < R / 4; ++c) {
+                        const uint32_t e0 = (uint32_t)__builtin_amdgcn_readlane(xe[c].x, b + e), e1 = (uint32_t)__builtin_amdgcn_readlane(xe[c].y, b + e);
+                        const uint32_t e2 = (uint32_t)__builtin_amdgcn_readlane(xe[c].z, b + e), e3 = (uint32_t)__builtin_amdgcn_readlane(xe[c].w, b + e);
+                        // lane l fetches the term of member 4c + l % 4; the quad's lanes hand it round when it is used
+                        B.xl[e][c] = (int)(mine == 0 ? e0 : mine == 1 ? e1 : mine == 2 ? e2 : e3);
+                        B.bz[e][c] = bias[(size_t)((uint32_t)B.xl[e][c] * (uint32_t)H) + head];
+                    }
+                }
                 // lane l fetches the scratch positions of the pairs of members l % 4, 4 + l % 4, ... with this entry
                 const char *pp = reinterpret_cast<const char *>(P.grp_pairs) + (size_t)((uint32_t)(p0 + b + e) * (uint32_t)(R * 4));
 #pragma unroll
@@ -1459,6 +1530,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                         lds_get_row<EPL>(q_lds + m * (EPL / 4) * WAVE, lane, qm);
                         float s = dot_n<EPL>(qm, kv), dp = dot_n<EPL>(dov[m], vv);
                         head_sum2<L::LPH>(s, dp);
+                        if constexpr (BIAS) s += quad_bcast(B.bz[e][BIAS ? m / 4 : 0], m);
                         float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
                         float mt = 1.f;                   // dropout multiplier of this pair (as in the forward kernel)
                         if constexpr (DROP) {
@@ -1476,6 +1548,8 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                     if ((B.mk[e] >> (4 * c)) & 15) {      // (look-ahead batches past the group's end have empty masks)
                         char *w = reinterpret_cast<char *>(pds);
                         *reinterpret_cast<float2 *>(w + (size_t)((uint32_t)B.xp[e][c] * (uint32_t)(H * 8) + hoff)) = make_float2(wp[c], wd[c]);
+                        // dL/d(score before scaling) in edge order (absent members write the spare row n_edges)
+                        if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.xl[e][c] * (uint32_t)H) + head] = wd[c];
                         // dq[member 4c + i] += ds[member] * k row: wd (0 for absent members) is the A operand
 #pragma unroll
                         for (int t = 0; t < EPL; ++t) dqa[c][t] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd[c], kv[t], dqa[c][t], 0, 0, 0);
@@ -1769,6 +1843,15 @@ int run_spmm_fast(const bpt_plan *P, const void *W0, const void *X0, void *Y0, c
     return launch_status();
 }
 
+// score term of the relative positions: bias[eid[p], head] = A[row, head, :] . table[idx[p], :], float32
+template <typename T, int H, int D>
+int run_rel_bias(const bpt_plan *P, const void *A, const void *table, float *bias, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    hipLaunchKernelGGL((k_sddmm_fast<T, H, D, FAST_BATCH, 2, float>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)table,
+                       bias);
+    return launch_status();
+}
+
 // node_mul_edge with the specialised kernels: y = A . B[e] (forward), dA = sum dy * B[e], dB[e] = sum_h dy * A
 template <typename T, int H, int D>
 int run_nme_fwd_fast(const bpt_plan *P, const void *A, const void *B, void *y, hipStream_t s) {
@@ -1902,29 +1985,38 @@ inline int64_t pds_bytes(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d
 
 template <typename T, int H, int D>
 int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v, void *o, float *lse, void *ws, float scale, Dropout drop,
-                 hipStream_t s) {
+                 const float *bias, hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
     float *ws_acc = (float *)ws;
     float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
         if (has_groups(P, H, D, sizeof(T))) {
-#define LAUNCH_FWD(RR, DR)                                                                                                   \
-    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR, HS, DR>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)q, \
-                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv)
-#define LAUNCH_FWD_MFMA(DR)                                                                                                  \
-    hipLaunchKernelGGL((k_attn_fwd_mfma<T, H, D, HSM, DR>), dim3(group_grid(P) * HSM), dim3(2 * WAVE), 0, s, *P, (const T *)q, \
-                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv)
+#define LAUNCH_FWD(RR, DR, BI)                                                                                                   \
+    hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR, HS, DR, BI>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)q, \
+                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv, bias)
+#define LAUNCH_FWD_MFMA(DR, BI)                                                                                                      \
+    hipLaunchKernelGGL((k_attn_fwd_mfma<T, H, D, HSM, DR, BI>), dim3(group_grid(P) * HSM), dim3(2 * WAVE), 0, s, *P, (const T *)q, \
+                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv, bias)
             constexpr int HS = head_slices<T, H, D>();
+            const int variant = (drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0);
             if (P->grp_R == 8) {
                 // every compile-time shape has the matrix-core form for groups of 8
                 static_assert(mfma_ok<T, H, D>(), "groups of 8 rows need the matrix-core forward");
                 constexpr int HSM = mfma_slices<T, H, D>();
-                if (drop.thr == 0) LAUNCH_FWD_MFMA(false);
-                else LAUNCH_FWD_MFMA(true);
+                switch (variant) {
+                case 0: LAUNCH_FWD_MFMA(false, false); break;
+                case 1: LAUNCH_FWD_MFMA(true, false); break;
+                case 2: LAUNCH_FWD_MFMA(false, true); break;
+                default: LAUNCH_FWD_MFMA(true, true); break;
+                }
             } else {
-                if (drop.thr == 0) LAUNCH_FWD(4, false);
-                else LAUNCH_FWD(4, true);
+                switch (variant) {
+                case 0: LAUNCH_FWD(4, false, false); break;
+                case 1: LAUNCH_FWD(4, true, false); break;
+                case 2: LAUNCH_FWD(4, false, true); break;
+                default: LAUNCH_FWD(4, true, true); break;
+                }
             }
 #undef LAUNCH_FWD
 #undef LAUNCH_FWD_MFMA
@@ -1942,7 +2034,8 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
 
 template <typename T, int H, int D>
 int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const void *k, const void *v, const void *o,
-                 const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, Dropout drop, hipStream_t s) {
+                 const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *ws, float scale, Dropout drop, const float *bias,
+                 float *ds_out, hipStream_t s) {
     if (Pin->n_items == 0) return BPT_OK;
     const bool grouped = grouped_backward(Pin, Pout, H, D, sizeof(T));
     const int64_t pbytes = pds_bytes(Pin, Pout, H, D, sizeof(T));
@@ -1953,17 +2046,21 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
         if (grouped) {
-#define LAUNCH_DST(RR, DR)                                                                                                           \
-    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, RR, HS, DR>), dim3(group_grid(Pin) * HS), dim3(WAVE), 0, s, *Pin, (const T *)q, \
-                       (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E,  \
-                       drop.thr, drop.seed, drop.inv)
+#define LAUNCH_DST(RR, DR, BI)                                                                                                           \
+    hipLaunchKernelGGL((k_attn_bwd_dst_grp<T, H, D, RR, HS, DR, BI>), dim3(group_grid(Pin) * HS), dim3(WAVE), 0, s, *Pin, (const T *)q, \
+                       (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale, scale * LOG2E,      \
+                       drop.thr, drop.seed, drop.inv, bias, ds_out)
             constexpr int HS = head_slices<T, H, D>();
-            if (drop.thr == 0) {
-                if (Pin->grp_R == 8) LAUNCH_DST(8, false);
-                else LAUNCH_DST(4, false);
-            } else {
-                if (Pin->grp_R == 8) LAUNCH_DST(8, true);
-                else LAUNCH_DST(4, true);
+            const int variant = (drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0) + (Pin->grp_R == 8 ? 4 : 0);
+            switch (variant) {
+            case 0: LAUNCH_DST(4, false, false); break;
+            case 1: LAUNCH_DST(4, true, false); break;
+            case 2: LAUNCH_DST(4, false, true); break;
+            case 3: LAUNCH_DST(4, true, true); break;
+            case 4: LAUNCH_DST(8, false, false); break;
+            case 5: LAUNCH_DST(8, true, false); break;
+            case 6: LAUNCH_DST(8, false, true); break;
+            default: LAUNCH_DST(8, true, true); break;
             }
 #undef LAUNCH_DST
         } else {
@@ -2075,6 +2172,19 @@ int bpt_maskedmm_csr_backward(const bpt_plan *plan_r, const bpt_plan *plan_c, co
     return spmm(plan_c, dy, A, dB, workspace, h, d, dtype, (hipStream_t)stream);
 }
 
+int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, float *bias, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan, true));
+    CHECK(check_shape(h, d, dtype));
+    if (plan->n_edges > 0 && (!q || !table || !bias)) return BPT_ERR_NULL;
+    if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(table)) return BPT_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+#define X(HH, DD) if (h == HH && d == DD) return run_rel_bias<T, HH, DD>(plan, q, table, bias, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
 int bpt_node_mul_edge_forward(const bpt_plan *plan, const void *A, const void *B, void *y, int h, int d, int dtype, void *stream) {
     CHECK(check_plan(plan, false));
     CHECK(check_shape(h, d, dtype));
@@ -2133,21 +2243,23 @@ int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const
     return spmm(plan_t, edata, dy, dx, workspace, h, d, dtype, (hipStream_t)stream);
 }
 
-int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v, void *o, float *lse,
-                          void *workspace, int64_t workspace_bytes, float scale, float dropout_p, uint64_t dropout_seed, int h, int d,
-                          int dtype, void *stream) {
+int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v, const float *bias, void *o,
+                          float *lse, void *workspace, int64_t workspace_bytes, float scale, float dropout_p, uint64_t dropout_seed,
+                          int h, int d, int dtype, void *stream) {
     CHECK(check_plan(plan_in, true));
     CHECK(check_shape(h, d, dtype));
     if (!q || !k || !v || !o || !lse) return BPT_ERR_NULL;
     if (!(dropout_p >= 0.f && dropout_p < 1.f)) return BPT_ERR_SIZE;
     const Dropout drop = make_dropout(dropout_p, dropout_seed);
-    if (drop.thr != 0 && !has_groups(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;   // row-group kernels only
+    // dropout and the score term exist in the row-group kernels only
+    if ((drop.thr != 0 || bias) && !has_groups(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
+    if (bias && !plan_in->grp_eids) return BPT_ERR_PLAN;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(workspace))
         return BPT_ERR_UNSUPPORTED;
     const int64_t need = bpt_workspace_bytes(BPT_OP_ATTN_FWD, plan_in, nullptr, h, d, dtype);
     if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
-#define X(HH, DD) if (h == HH && d == DD) return run_attn_fwd<T, HH, DD>(plan_in, q, k, v, o, lse, workspace, scale, drop, s);
+#define X(HH, DD) if (h == HH && d == DD) return run_attn_fwd<T, HH, DD>(plan_in, q, k, v, o, lse, workspace, scale, drop, bias, s);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
 #undef X
@@ -2155,15 +2267,17 @@ int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k,
 }
 
 int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, const void *q, const void *k, const void *v,
-                           const void *o, const void *d_o, const float *lse, void *dq, void *dk, void *dv, void *workspace,
-                           int64_t workspace_bytes, float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype,
-                           void *stream) {
+                           const float *bias, const void *o, const void *d_o, const float *lse, void *dq, void *dk, void *dv,
+                           float *ds_out, void *workspace, int64_t workspace_bytes, float scale, float dropout_p,
+                           uint64_t dropout_seed, int h, int d, int dtype, void *stream) {
     CHECK(check_plan(plan_in, true));
     CHECK(check_plan(plan_out, true));
     CHECK(check_shape(h, d, dtype));
     if (!(dropout_p >= 0.f && dropout_p < 1.f)) return BPT_ERR_SIZE;
     const Dropout drop = make_dropout(dropout_p, dropout_seed);
-    if (drop.thr != 0 && !grouped_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
+    if ((drop.thr != 0 || bias) && !grouped_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
+    if ((bias != nullptr) != (ds_out != nullptr)) return BPT_ERR_NULL;       // the score term and its gradient go together
+    if (bias && !plan_in->grp_eids) return BPT_ERR_PLAN;
     if (plan_in->n_edges != plan_out->n_edges || plan_in->n_rows != plan_out->n_rows) return BPT_ERR_PLAN;
     if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return BPT_ERR_NULL;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) ||
@@ -2173,7 +2287,7 @@ int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, co
     if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
 #define X(HH, DD) \
-    if (h == HH && d == DD) return run_attn_bwd<T, HH, DD>(plan_in, plan_out, q, k, v, o, d_o, lse, dq, dk, dv, workspace, scale, drop, s);
+    if (h == HH && d == DD) return run_attn_bwd<T, HH, DD>(plan_in, plan_out, q, k, v, o, d_o, lse, dq, dk, dv, workspace, scale, drop, bias, ds_out, s);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
 #undef X

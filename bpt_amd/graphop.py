@@ -224,12 +224,42 @@ def attention_supported(q):
     return q.dim() == 3 and (h, d) in fast.get(q.dtype, ())
 
 
-def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, dropout_p=0.0, seed=0):
-    """o[dst] = sum over in-edges drop(softmax(q[dst].k[src]*scale)) v[src]; returns (o, lse) with lse (n, h)
-    float32 in base-2 units.  Arithmetic of modules/attention.py:66-77 (no rel-pos) in one pass.  dropout_p > 0
+def rel_bias_forward(col, indptr_c, eid_c, etype_slot, q, table):
+    """The rel_pos score term of modules/attention.py:69-71 without the (E, d) embedding rows:
+    bias[eid_c[p], head] = q[row(p), head, :] . table[etype_slot[p], :], where etype_slot[p] is the type of the edge
+    in slot p of the in-CSR (etype[eid_c]).  Returns float32 (E + 1, h); the last row is a zero spare row that the
+    fused kernels read for absent pairs."""
+    _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, etype_slot=etype_slot, q=q, table=table)
+    _same_dtype(q, table)
+    h, d = _hd(q)
+    if table.dim() != 2 or table.size(1) != d:
+        raise ValueError(f"table must be (n_types, {d})")
+    plan = plan_cache.get(col, indptr_c, eid_c, etype_slot, q.size(0), table.size(0))
+    E = eid_c.size(0)
+    bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
+    bias[E].zero_()
+    with torch.cuda.device_of(q):
+        check_attn(_LIB.bpt_rel_bias_forward(plan.ref, _ptr(q), _ptr(table), _ptr(bias), h, d, _dtype(q), _stream()),
+                   "rel_bias_forward")
+    return bias
+
+
+def _check_bias(bias, n_edges, h, device):
+    if bias is None:
+        return
+    if bias.dtype != torch.float32 or tuple(bias.shape) != (n_edges + 1, h) or not bias.is_contiguous() or bias.device != device:
+        raise ValueError(f"bias must be a contiguous float32 ({n_edges + 1}, {h}) tensor on {device}")
+    if not _USE_GROUPS:
+        raise RuntimeError("the per-edge score term needs the row-group kernels")
+
+
+def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, dropout_p=0.0, seed=0, bias=None):
+    """o[dst] = sum over in-edges drop(softmax((q[dst].k[src] + bias[e])*scale)) v[src]; returns (o, lse) with lse
+    (n, h) float32 in base-2 units.  Arithmetic of modules/attention.py:66-77 in one pass.  dropout_p > 0
     drops attention probabilities as attention.py:73 does; the mask is a function of (seed, graph), see
-    attention_dropout_mask."""
+    attention_dropout_mask.  bias: None or the float32 (E + 1, h) score term of rel_bias_forward."""
     _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v)
+    _check_bias(bias, eid_c.size(0), _hd(q)[0], q.device)
     _same_dtype(q, k, v)
     h, d = _hd(q)
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
@@ -240,15 +270,16 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     dt = _dtype(q)
     ws, nws = _workspace(OP_ATTN_FWD, plan, None, h, d, dt, q.device)
     with torch.cuda.device_of(q):
-        check_attn(_LIB.bpt_attention_forward(ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(ws), nws,
+        check_attn(_LIB.bpt_attention_forward(ref, _ptr(q), _ptr(k), _ptr(v), _ptr(bias), _ptr(o), _ptr(lse), _ptr(ws), nws,
                                               scale, float(dropout_p), int(seed) & (2 ** 64 - 1), h, d, dt, _stream()),
                    "attention_forward")
     return o, lse
 
 
 def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, do, scale=None,
-                       dropout_p=0.0, seed=0):
-    """(dq, dk, dv) of attention_forward (same dropout_p and seed)."""
+                       dropout_p=0.0, seed=0, bias=None):
+    """(dq, dk, dv) of attention_forward (same dropout_p, seed and bias).  With bias a fourth result: ds, float32
+    (E, h), the gradient with respect to q.k + bias of every edge and head (= the gradient of bias)."""
     _check_all(row=row, indptr_r=indptr_r, eid_r=eid_r, indices_r=indices_r, col=col, indptr_c=indptr_c,
                eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v, o=o, lse=lse)
     do = do.contiguous()
@@ -258,6 +289,8 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
     plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0))
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    _check_bias(bias, eid_c.size(0), h, q.device)
+    ds = torch.empty((eid_c.size(0) + 1, h), dtype=torch.float32, device=q.device) if bias is not None else None
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref
     if _USE_GROUPS and plan_in.covers_all_edges and plan_out.covers_all_edges:
@@ -266,10 +299,12 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
         out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
     with torch.cuda.device_of(q):
-        check_attn(_LIB.bpt_attention_backward(in_ref, out_ref, _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do),
-                                               _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), nws,
+        check_attn(_LIB.bpt_attention_backward(in_ref, out_ref, _ptr(q), _ptr(k), _ptr(v), _ptr(bias), _ptr(o), _ptr(do),
+                                               _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ds), _ptr(ws), nws,
                                                scale, float(dropout_p), int(seed) & (2 ** 64 - 1), h, d, dt, _stream()),
                    "attention_backward")
+    if bias is not None:
+        return dq, dk, dv, ds[:-1]
     return dq, dk, dv
 
 

@@ -92,6 +92,61 @@ class BPTAttention(Function):
         return None, None, None, None, None, None, None, None, dq, dk, dv, None, None, None
 
 
+class BPTRelAttention(Function):
+    """BPTAttention with the rel_pos score term of modules/attention.py:69-71, s = (q.k + q.table[etype]) * scale,
+    without the (E, d) rows of the embedding lookup: a small kernel writes the (E, h) term q[dst].table[etype], the
+    fused kernels add it to the scores, and the backward kernel returns ds = dL/d(q.k + term) per edge and head,
+    from which two SpMMs form the term's gradients: dq += sum_e ds[e] table[etype[e]] over the in-CSR with the edge
+    types as column indices, and dtable[t] = sum_h sum_{e of type t} ds[e, h] q[dst(e), h] over a CSR whose rows
+    are the edge types.  All sums are row-owned (no atomics)."""
+
+    @staticmethod
+    def forward(ctx, row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed,
+                table, etype):
+        aux = _rel_aux(etype, col, indptr_c, eid_c, table.size(0))
+        table = table.contiguous()
+        bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux[0], q, table)
+        o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed, bias=bias)
+        ctx.save_for_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, bias, table)
+        ctx.scale, ctx.dropout_p, ctx.seed, ctx.aux = scale, dropout_p, seed, aux
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, bias, table = ctx.saved_tensors
+        etype_slot, t_row, t_indptr, t_order, t_dst = ctx.aux
+        dq, dk, dv, ds = _g.attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c,
+                                               q, k, v, o, lse, do, ctx.scale, ctx.dropout_p, ctx.seed, bias=bias)
+        h = q.size(1)
+        ds = ds.to(q.dtype)
+        table_h = table.unsqueeze(1).expand(-1, h, -1).contiguous()
+        dq = dq + vector_spmm_forward(col, indptr_c, eid_c, etype_slot, ds, table_h, n_rows=q.size(0))
+        dtable = vector_spmm_forward(t_row, t_indptr, t_order, t_dst, ds, q, n_rows=table.size(0))
+        dtable = dtable.float().sum(1).to(table.dtype)
+        return None, None, None, None, None, None, None, None, dq, dk, dv, None, None, None, dtable, None
+
+
+_rel_aux_cache = {}
+
+
+def _rel_aux(etype, col, indptr_c, eid_c, n_types):
+    """Index tensors of the rel_pos term, cached per (etype, in-CSR): the edge type of every in-CSR slot, and the
+    CSR whose row t lists the edges of type t (_type_csr) together with the destination node of each of its slots."""
+    key = tuple((t.data_ptr(), t.numel(), t._version) for t in (etype, col, indptr_c, eid_c)) + (str(etype.device), n_types)
+    hit = _rel_aux_cache.get(key)
+    if hit is None:
+        t_row, t_indptr, t_order = _type_csr(etype, n_types)
+        etype_slot = etype.index_select(0, eid_c).contiguous()
+        slot_dst = torch.repeat_interleave(col, indptr_c[1:] - indptr_c[:-1])          # destination of every in-CSR slot
+        dst_of_eid = torch.empty_like(slot_dst)
+        dst_of_eid[eid_c] = slot_dst
+        hit = (etype_slot, t_row, t_indptr, t_order, dst_of_eid.index_select(0, t_order).contiguous(), (etype, col, indptr_c, eid_c))
+        if len(_rel_aux_cache) > 16:
+            _rel_aux_cache.clear()
+        _rel_aux_cache[key] = hit           # holds the tensors so that their data_ptrs are not reused while cached
+    return hit[:5]
+
+
 def sparse_softmax(row, indptr, eid, x):
     return SparseSoftmax.apply(row, indptr, eid, x)
 
@@ -158,7 +213,7 @@ def edge_type_embedding(table, etype):
 
 
 def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale=None, fused=None,
-                  dropout_p=0.0, seed=None):
+                  dropout_p=0.0, seed=None, rel_table=None, etype=None):
     """Attention over the graph: (ROW, INDPTR_R, out_eid, out_idx) is the out-CSR side (rows =
     sources), (COL, INDPTR_C, in_eid, in_idx) the in-CSR side (rows = destinations), exactly the
     eight graph arguments modules/attention.py:66-67 passes to masked_mm.
@@ -168,17 +223,27 @@ def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices
 
     dropout_p > 0 applies dropout to the attention probabilities (attention.py:73).  The fused path hashes
     (seed, edge, head); seed=None draws one from torch's CPU generator (reproducible under torch.manual_seed).  The
-    unfused path uses torch's dropout, so the two paths drop different elements."""
+    unfused path uses torch's dropout, so the two paths drop different elements.
+
+    rel_table (n_types, d) and etype (E,) int64 add the rel_pos term q[dst] . rel_table[etype[e]] to the score of
+    edge e (attention.py:69-71); the gradient of rel_table is returned like any other."""
     scale = 1.0 / math.sqrt(q.size(-1)) if scale is None else float(scale)
+    if (rel_table is None) != (etype is None):
+        raise ValueError("rel_table and etype go together")
     if fused is None:
         fused = _g.attention_supported(q) and q.size(0) == k.size(0)
-        if dropout_p > 0 and not _g.row_groups_enabled():
-            fused = False                       # only the row-group kernels implement dropout
+        if (dropout_p > 0 or rel_table is not None) and not _g.row_groups_enabled():
+            fused = False                       # only the row-group kernels implement dropout and the rel_pos term
     if fused:
         if dropout_p > 0 and seed is None:
             seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+        if rel_table is not None:
+            return BPTRelAttention.apply(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale,
+                                         float(dropout_p), int(seed or 0), rel_table, etype)
         return BPTAttention.apply(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale,
                                   float(dropout_p), int(seed or 0))
     e = masked_mm(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, k, q)
+    if rel_table is not None:
+        e = e + node_mul_edge(col, indptr_c, eid_c, q, edge_type_embedding(rel_table, etype))
     a = torch.nn.functional.dropout(sparse_softmax(col, indptr_c, eid_c, e * scale), p=float(dropout_p), training=dropout_p > 0)
     return vec_spmm(col, indptr_c, eid_c, indices_c, row, indptr_r, eid_r, indices_r, a, v)

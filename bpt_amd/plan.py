@@ -176,7 +176,12 @@ class Plan:
             hit = self._groups.get((R, order_mode))
             if hit is None:
                 grp = build_groups_host(self._host, self.n_index_nodes, R=R, order_mode=order_mode)
-                dev = {k: torch.from_numpy(grp[k]).to(self.device) for k in ("members", "grp_ptr", "entries", "chunks")}
+                # edge id of every (entry, member); absent members and the padding point at the spare row n_edges
+                eids = np.full((len(grp["entries"]) + GROUP_PAD_ENTRIES, R), self.n_edges, dtype=np.int32)
+                se = grp["slot_eid"]
+                eids[:len(se)] = np.where(se >= 0, se, self.n_edges)
+                grp["eids"] = eids
+                dev = {k: torch.from_numpy(grp[k]).to(self.device) for k in ("members", "grp_ptr", "entries", "chunks", "eids")}
                 n_groups = len(grp["members"])
                 st = PlanStruct.from_buffer_copy(self.struct)
                 st.grp_members = dev["members"].data_ptr() if n_groups else None
@@ -188,6 +193,7 @@ class Plan:
                 st.n_groups = n_groups
                 st.grp_R = R
                 st.n_grp_entries = len(grp["entries"])
+                st.grp_eids = dev["eids"].data_ptr()
                 hit = {"host": grp, "dev": dev, "struct": st}
                 self._groups[(R, order_mode)] = hit
         return hit

@@ -65,6 +65,9 @@ typedef struct {
     int64_t n_groups, grp_R;
     int64_t grp_max_chunk;       /* largest chunk length; the row-group kernels launch 8 * grp_max_chunk workgroups */
     int64_t n_grp_entries;       /* grp_ptr[n_groups] */
+    const int32_t *grp_eids;     /* (n_grp_entries + 8) * grp_R or NULL: edge id of (entry u, member m) at
+                                    [u * grp_R + m]; n_edges where the entry's mask has no bit m and in the 8
+                                    entries of padding.  Needed by the calls that take a per-edge score term */
 } bpt_plan;
 
 const char *bpt_strerror(int status);
@@ -128,22 +131,37 @@ int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const
                              const void *x, void *dedata, void *dx, void *workspace, int64_t workspace_bytes,
                              int h, int d, int dtype, void *stream);
 
-/* Fused attention layer core = modules/attention.py:66-77 without rel-pos:
- *   o[dst] = sum_{e: src->dst} drop( softmax_dst( q[dst].k[src] * scale ) )[e] * v[src]
+/* Score term of the relative positions, modules/attention.py:69-71 (embed_ak looked up per edge, then
+ * node_mul_edge): bias[eid[p], head] = sum_d q[row, head, d] * table[idx[p], d] over `plan`, whose rows are the
+ * destinations and whose idx[p] is the edge TYPE of the edge in slot p (a plan built with the edge types as
+ * `indices`, n_index_nodes = rows of table).  bias is float32 (n_edges, h) or larger; the (n_edges, d) rows of the
+ * reference's nn.Embedding lookup are never materialised.  Compile-time shapes only (BPT_ERR_UNSUPPORTED else). */
+int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, float *bias,
+                         int h, int d, int dtype, void *stream);
+
+/* Fused attention layer core = modules/attention.py:66-77:
+ *   o[dst] = sum_{e: src->dst} drop( softmax_dst( (q[dst].k[src] + bias[e]) * scale ) )[e] * v[src]
  * plan_in: rows = destinations (the reference's COL/INDPTR_C/in_csr), plan_out: rows = sources.
  * lse (n, h) float32 receives the base-2 log-sum-exp of the scaled scores, needed by backward.
  * f32 and bf16 only (accumulation in f32).
+ * bias: NULL, or float32 (n_edges + 1, h): per edge and head, added to q.k before scaling (the rel_pos term,
+ * bpt_rel_bias_forward); row n_edges is a spare row that is read for absent pairs and never used.  Needs the row
+ * groups with grp_eids (BPT_ERR_UNSUPPORTED / BPT_ERR_PLAN without them).
  * dropout_p in [0, 1): dropout on the attention probabilities (attention.py:73); 0 = none.  Each (edge, head) is
  * kept with probability 1 - p and scaled by 1 / (1 - p); the decision is a hash of dropout_seed and the edge's pair
  * number in plan_in's row groups, so backward must get the same plan, p and seed.  Needs the row groups
  * (BPT_ERR_UNSUPPORTED without them). */
-int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v,
+int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v, const float *bias,
                           void *o, float *lse, void *workspace, int64_t workspace_bytes,
                           float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype, void *stream);
 
+/* Backward of bpt_attention_forward.  With bias, ds_out (float32 (n_edges + 1, h), row n_edges spare) receives
+ * dL/d(q.k + bias) of every edge and head, from which the caller forms the gradients of what produced the bias
+ * (for rel_pos: dq += sum_e ds[e] * table[type(e)], dtable[t] = sum_{e of type t} sum_h ds[e, h] * q[dst(e), h]);
+ * bias and ds_out are both given or both NULL. */
 int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, const void *q, const void *k,
-                           const void *v, const void *o, const void *d_o, const float *lse,
-                           void *dq, void *dk, void *dv, void *workspace, int64_t workspace_bytes,
+                           const void *v, const float *bias, const void *o, const void *d_o, const float *lse,
+                           void *dq, void *dk, void *dv, float *ds_out, void *workspace, int64_t workspace_bytes,
                            float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype, void *stream);
 
 #ifdef __cplusplus

@@ -400,6 +400,47 @@ def test_fused_attention_dropout_matches_oracle_with_the_same_mask(ops, gname, r
     close(v.grad, rdv.numpy(), GTOL[dtype], "dv", c.max_deg)
 
 
+# --------------------------------------------------------------------------------------------
+# the rel_pos score term inside the fused kernels (modules/attention.py:69-71), with and without dropout
+# --------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("p", [0.0, 0.25])
+@pytest.mark.parametrize("dtype,hd", [(torch.float32, (8, 64)), (torch.float32, (16, 64)), (torch.float32, (4, 64)), (torch.bfloat16, (8, 64))])
+@pytest.mark.parametrize("gname,rows", [("bpt512_k4", 4), ("bpt512_k4", 8), ("bpt300_causal_k2", None), ("multigraph", 4), ("fc_w100", 8),
+                                        ("bpt256_k24", 8)])
+def test_fused_attention_with_rel_pos_matches_oracle(ops, gname, rows, dtype, hd, p):
+    from oracle import torch_ops
+    graphop, op = ops
+    h, d = hd
+    n_types, seed = 37, 987654321
+    c = case(gname)
+    q, k, v, do = (rand((c.n, h, d), dtype, s, 1.0 / 8).to(DEV) for s in (31, 32, 33, 34))
+    table = rand((n_types, d), dtype, 35, 1.0 / 8).to(DEV)
+    etype = torch.from_numpy(np.random.default_rng(36).integers(0, n_types, c.E)).to(DEV)
+    for t in (q, k, v, table):
+        t.requires_grad_(True)
+    old_r = graphop.set_group_rows(rows)
+    ctx = long_items(gname)
+    ctx.__enter__()
+    try:
+        mask = graphop.attention_dropout_mask(*c.inn, q, k, p, seed) if p > 0 else None
+        o = op.bpt_attention(*c.out, *c.inn, q, k, v, dropout_p=p, seed=seed, rel_table=table, etype=etype)
+        o.backward(do)
+    finally:
+        ctx.__exit__()
+        graphop.set_group_rows(old_r)
+    t64 = lambda x: x.detach().cpu().double()
+    src, dst, et = torch.from_numpy(c.src), torch.from_numpy(c.dst), etype.cpu()
+    ro, rdq, rdk, rdv, rdak = torch_ops.attention_fwd_bwd(src, dst, t64(q), t64(k), t64(v), t64(do), ak=t64(table)[et],
+                                                          drop=mask.double() if mask is not None else None)
+    rdt = torch.zeros(n_types, d, dtype=torch.float64).index_add_(0, et, rdak)
+    close(o, ro.numpy(), TOL[dtype], "o", c.max_deg)
+    close(q.grad, rdq.numpy(), GTOL[dtype], "dq", c.max_deg)
+    close(k.grad, rdk.numpy(), GTOL[dtype], "dk", c.max_deg)
+    close(v.grad, rdv.numpy(), GTOL[dtype], "dv", c.max_deg)
+    # a table row sums over all edges of its type and all heads
+    close(table.grad, rdt.numpy(), GTOL[dtype], "dtable", h * c.E / n_types)
+
+
 def test_block_uses_fused_dropout_in_training(ops):
     from bpt_amd.block import BPTBlock
     from bpt_amd import graphbuilder as gb
