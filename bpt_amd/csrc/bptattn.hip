@@ -1219,6 +1219,13 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+typedef short bf16x4_t __attribute__((ext_vector_type(4)));
+// two registers of bfloat16 pairs as the four-element operand of the bfloat16 matrix instructions
+__device__ __forceinline__ bf16x4_t as_bf16x4(uint32_t a, uint32_t b) {
+    const uint2 u = make_uint2(a, b);
+    return __builtin_bit_cast(bf16x4_t, u);
+}
+
 // 16-byte vector as VE floats
 template <typename T> __device__ __forceinline__ void unpack_vec(const uint4 &w, float *out) {
     const uint32_t x[4] = {w.x, w.y, w.z, w.w};
@@ -1270,7 +1277,11 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     __shared__ uint4 kst[2][NB * PITCH];              // rows as loaded, one spare vector per row against bank conflicts
     __shared__ uint4 vst[2][NB * NV * WAVE];
-    float qb[CB];                                      // q row of member 4 wv + j, the columns of this lane's block, pre-scaled
+    // q row of member 4 wv + j, the columns of this lane's block: float32 pre-scaled, or (bfloat16) as loaded, the
+    // scale then being applied to the scores
+    constexpr bool B16 = sizeof(T) == 2;
+    float qb[B16 ? 1 : CB];
+    uint4 qraw[B16 ? NV * 4 : 1];
     {
         // wavefront 0 stages its q rows through the K area, wavefront 1 through the V area
         uint4 *qst = wv == 0 ? &kst[0][0] : &vst[0][0];
@@ -1283,10 +1294,15 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
             for (int c = 0; c < NV; ++c) qst[i * QP + c * WAVE + lane] = make_uint4(qr[i].w[4 * c], qr[i].w[4 * c + 1], qr[i].w[4 * c + 2], qr[i].w[4 * c + 3]);
         wave_lds_fence();
+        if constexpr (B16) {
 #pragma unroll
-        for (int t = 0; t < NV * 4; ++t) unpack_vec<T>(qst[j * QP + (t / 4) * WAVE + 4 * blk + (t % 4)], &qb[t * VE]);
+            for (int t = 0; t < NV * 4; ++t) qraw[t] = qst[j * QP + (t / 4) * WAVE + 4 * blk + (t % 4)];
+        } else {
 #pragma unroll
-        for (int c = 0; c < CB; ++c) qb[c] *= scale_log2e;
+            for (int t = 0; t < NV * 4; ++t) unpack_vec<T>(qst[j * QP + (t / 4) * WAVE + 4 * blk + (t % 4)], &qb[t * VE]);
+#pragma unroll
+            for (int c = 0; c < CB; ++c) qb[c] *= scale_log2e;
+        }
     }
     floatx4 acc[EPL];                                  // [row register r][member 4 wv + i]
     float mref = M_INIT_LOG2, lrun = 0.f;
@@ -1356,16 +1372,25 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
             floatx4 st[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) st[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+            if constexpr (B16) {
+                // four columns per instruction, operands as loaded (v_mfma_f32_4x4x4 on bfloat16)
 #pragma unroll
-            for (int t = 0; t < NV * 4; ++t) {
-                float kf[VE];
-                unpack_vec<T>(kv[t], kf);
+                for (int t = 0; t < NV * 4; ++t) {
+                    st[0] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(as_bf16x4(kv[t].x, kv[t].y), as_bf16x4(qraw[t].x, qraw[t].y), st[0], 0, 0, 0);
+                    st[1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(as_bf16x4(kv[t].z, kv[t].w), as_bf16x4(qraw[t].z, qraw[t].w), st[1], 0, 0, 0);
+                }
+            } else {
 #pragma unroll
-                for (int c = 0; c < VE; ++c) st[c & 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(kf[c], qb[t * VE + c], st[c & 3], 0, 0, 0);
+                for (int t = 0; t < NV * 4; ++t) {
+                    float kf[VE];
+                    unpack_vec<T>(kv[t], kf);
+#pragma unroll
+                    for (int c = 0; c < VE; ++c) st[c & 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(kf[c], qb[t * VE + c], st[c & 3], 0, 0, 0);
+                }
             }
             float sc[NB];
 #pragma unroll
-            for (int e = 0; e < NB; ++e) sc[e] = block_sum<BPH>((st[0][e] + st[1][e]) + (st[2][e] + st[3][e]));
+            for (int e = 0; e < NB; ++e) sc[e] = block_sum<BPH>((st[0][e] + st[1][e]) + (st[2][e] + st[3][e])) * (B16 ? scale_log2e : 1.f);
 #pragma unroll
             for (int e = 0; e < NB; ++e) sc[e] = ((mk[e] >> (4 * wv + j)) & 1) ? (BIAS ? fmaf(bz[e], scale_log2e, sc[e]) : sc[e]) : -INFINITY;
             const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
@@ -1392,13 +1417,30 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                     pk[e] = pe;
                 }
             }
+            if constexpr (B16) {
+                // A = the lane's four probabilities (one per entry of the batch) rounded to bfloat16; B = column r of
+                // the four V rows, gathered from the rows' registers by byte permutes
+                const uint32_t p01 = (uint32_t)f32_to_bf16(pk[0]) | ((uint32_t)f32_to_bf16(pk[1]) << 16);
+                const uint32_t p23 = (uint32_t)f32_to_bf16(pk[2]) | ((uint32_t)f32_to_bf16(pk[3]) << 16);
+                static_assert(NV == 1 && NB == 4, "one 16-byte vector per row and lane");
+                const uint32_t v0[4] = {vv[0][0].x, vv[0][0].y, vv[0][0].z, vv[0][0].w}, v1[4] = {vv[1][0].x, vv[1][0].y, vv[1][0].z, vv[1][0].w};
+                const uint32_t v2[4] = {vv[2][0].x, vv[2][0].y, vv[2][0].z, vv[2][0].w}, v3[4] = {vv[3][0].x, vv[3][0].y, vv[3][0].z, vv[3][0].w};
 #pragma unroll
-            for (int e = 0; e < NB; ++e) {
-                float vf[EPL];
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t lo01 = __builtin_amdgcn_perm(v1[c], v0[c], 0x05040100u), lo23 = __builtin_amdgcn_perm(v3[c], v2[c], 0x05040100u);
+                    const uint32_t hi01 = __builtin_amdgcn_perm(v1[c], v0[c], 0x07060302u), hi23 = __builtin_amdgcn_perm(v3[c], v2[c], 0x07060302u);
+                    acc[2 * c] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(as_bf16x4(p01, p23), as_bf16x4(lo01, lo23), acc[2 * c], 0, 0, 0);
+                    acc[2 * c + 1] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(as_bf16x4(p01, p23), as_bf16x4(hi01, hi23), acc[2 * c + 1], 0, 0, 0);
+                }
+            } else {
 #pragma unroll
-                for (int c = 0; c < NV; ++c) unpack_vec<T>(vv[e][c], &vf[c * VE]);
+                for (int e = 0; e < NB; ++e) {
+                    float vf[EPL];
 #pragma unroll
-                for (int r = 0; r < EPL; ++r) acc[r] = __builtin_amdgcn_mfma_f32_4x4x1f32(pk[e], vf[r], acc[r], 0, 0, 0);
+                    for (int c = 0; c < NV; ++c) unpack_vec<T>(vv[e][c], &vf[c * VE]);
+#pragma unroll
+                    for (int r = 0; r < EPL; ++r) acc[r] = __builtin_amdgcn_mfma_f32_4x4x1f32(pk[e], vf[r], acc[r], 0, 0, 0);
+                }
             }
             // the other buffer was last read one batch ago, before the previous barrier
             stage_half(raw, buf ^ 1);

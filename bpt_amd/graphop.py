@@ -349,14 +349,12 @@ def _group_rows(q, h, d, plan):
 
 
 def _forward_rows(q, h, d, plan, dropout_p=0.0):
-    """Rows per group for the forward kernel.  Groups of 8 run on the matrix cores (two wavefronts per group), which
-    measured faster than the vector kernels at every float32 size, and for bfloat16 on rows of more than 512 columns
-    and on dense graphs.  With dropout the forward and the backward number the pairs by the same groups."""
+    """Rows per group for the forward kernel.  Groups of 8 run on the matrix cores (two wavefronts per group; bfloat16
+    rows go through the bfloat16 matrix instructions as loaded), which measured faster than the vector kernels at every
+    size and both dtypes.  With dropout the forward and the backward number the pairs by the same groups."""
     if _GROUP_ROWS is not None or dropout_p > 0.0:
         return _group_rows(q, h, d, plan)
-    if q.dtype == torch.float32 or h * d > 512 or plan.n_edges >= 64 * max(plan.n_rows, 1):
-        return 8
-    return _group_rows(q, h, d, plan)
+    return 8
 
 
 def set_group_rows(R):
