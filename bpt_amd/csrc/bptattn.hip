@@ -188,18 +188,16 @@ __global__ __launch_bounds__(BLOCK) void k_spmm_generic(bpt_plan P, const T *__r
 // workspace).  Wave w adds slots w, w+4, ... (eight independent loads per step); the four wave sums
 // are then added in wave order, so the result is a fixed function of the plan.
 template <typename T>
-__global__ __launch_bounds__(BLOCK) void k_combine_sum(const int32_t *__restrict__ heavy,
-                                                       const typename Elem<T>::acc_t *__restrict__ ws, T *__restrict__ Y0,
-                                                       T *__restrict__ Y1, int C, size_t ws_stride) {
+__device__ __forceinline__ void combine_sum_block(const int32_t *__restrict__ hv, const typename Elem<T>::acc_t *__restrict__ ws,
+                                                  T *__restrict__ Y, int C) {
     using acc_t = typename Elem<T>::acc_t;
     __shared__ acc_t part[WAVES_PER_BLOCK][WAVE];
-    const int row = heavy[3 * blockIdx.x], s0 = heavy[3 * blockIdx.x + 1], ns = heavy[3 * blockIdx.x + 2];
+    const int row = hv[0], s0 = hv[1], ns = hv[2];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int j = blockIdx.y * WAVE + lane;
-    T *Y = blockIdx.z == 0 ? Y0 : Y1;
     acc_t s = 0;
     if (j < C) {
-        const acc_t *col = ws + (size_t)blockIdx.z * ws_stride + (size_t)s0 * C + j;
+        const acc_t *col = ws + (size_t)s0 * C + j;
         int k = w;
         for (; k + 7 * WAVES_PER_BLOCK < ns; k += 8 * WAVES_PER_BLOCK) {
             acc_t t[8];
@@ -217,6 +215,27 @@ __global__ __launch_bounds__(BLOCK) void k_combine_sum(const int32_t *__restrict
 #pragma unroll
         for (int i = 1; i < WAVES_PER_BLOCK; ++i) r += part[i][lane];
         Elem<T>::st(Y + (size_t)row * C + j, r);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_combine_sum(const int32_t *__restrict__ heavy,
+                                                       const typename Elem<T>::acc_t *__restrict__ ws, T *__restrict__ Y0,
+                                                       T *__restrict__ Y1, int C, size_t ws_stride) {
+    combine_sum_block<T>(heavy + 3 * blockIdx.x, ws + (size_t)blockIdx.z * ws_stride, blockIdx.z == 0 ? Y0 : Y1, C);
+}
+
+// The three sums of the fused backward in one launch: blocks x < n_a combine rows of list A into YA (z = 0 only),
+// the others rows of list B into YB0 (z = 0) and YB1 (z = 1).
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_combine_sum3(const int32_t *__restrict__ heavy_a, int n_a, const float *__restrict__ ws_a,
+                                                        T *__restrict__ YA, const int32_t *__restrict__ heavy_b,
+                                                        const float *__restrict__ ws_b, T *__restrict__ YB0, T *__restrict__ YB1, int C,
+                                                        size_t ws_stride_b) {
+    if ((int)blockIdx.x < n_a) {
+        if (blockIdx.z == 0) combine_sum_block<T>(heavy_a + 3 * blockIdx.x, ws_a, YA, C);
+    } else {
+        combine_sum_block<T>(heavy_b + 3 * (blockIdx.x - n_a), ws_b + (size_t)blockIdx.z * ws_stride_b, blockIdx.z == 0 ? YB0 : YB1, C);
     }
 }
 
@@ -2113,7 +2132,7 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     }
     int st = launch_status();
     if (st != BPT_OK) return st;
-    if (Pin->n_heavy > 0) {
+    if (Pin->n_heavy > 0 && !grouped) {
         hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, Pin->heavy,
                            (const float *)ws_rows, (T *)dq, (T *)nullptr, H * D, (size_t)0);
         st = launch_status();
@@ -2124,7 +2143,7 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
         ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
         return run_spmm_fast<T, float, H, D, 2>(Pout, dsbuf, q, dk, pbuf, d_o, dv, ws_rows, s);
     }
-    float *ws_dk = ws_rows, *ws_dv = ws_rows + (size_t)Pout->n_slots * H * D;
+    float *ws_dk = ws_rows + (size_t)Pin->n_slots * H * D, *ws_dv = ws_dk + (size_t)Pout->n_slots * H * D;
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
 #define LAUNCH_SRC(RR)                                                                                                            \
@@ -2136,9 +2155,11 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
 #undef LAUNCH_SRC
     }
     st = launch_status();
-    if (st != BPT_OK || Pout->n_heavy == 0) return st;
-    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pout->n_heavy, H * D / WAVE, 2), dim3(BLOCK), 0, s, Pout->heavy,
-                       (const float *)ws_dk, (T *)dk, (T *)dv, H * D, (size_t)Pout->n_slots * H * D);
+    if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;
+    // partial rows of dq (destination side) and of dk, dv (source side) in one launch
+    hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / WAVE, 2), dim3(BLOCK), 0, s, Pin->heavy,
+                       (int)Pin->n_heavy, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
+                       (size_t)Pout->n_slots * H * D);
     return launch_status();
 }
 
@@ -2185,8 +2206,8 @@ int64_t bpt_workspace_bytes(int op, const bpt_plan *plan, const bpt_plan *plan_t
         case BPT_OP_SPMM_BWD: return round16(s1 * C * a);
         case BPT_OP_ATTN_FWD: return round16(s0 * (C + 2 * h) * 4);
         case BPT_OP_ATTN_BWD: {
-            const int64_t rows = s0 > 2 * s1 ? s0 : 2 * s1;
-            return pds_bytes(plan, plan_t, h, d, dtype == BPT_BF16 ? 2 : 4) + round16(rows * C * 4);
+            // partial rows of dq, then of dk and dv (the three are merged by one launch after the source-side kernel)
+            return pds_bytes(plan, plan_t, h, d, dtype == BPT_BF16 ? 2 : 4) + round16((s0 + 2 * s1) * C * 4);
         }
         default: return -1;
     }
