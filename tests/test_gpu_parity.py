@@ -441,6 +441,29 @@ def test_fused_attention_with_rel_pos_matches_oracle(ops, gname, rows, dtype, hd
     close(table.grad, rdt.numpy(), GTOL[dtype], "dtable", h * c.E / n_types)
 
 
+def test_rel_pos_without_row_groups_takes_the_op_chain_and_the_raw_call_refuses(ops):
+    graphop, op = ops
+    c = case("bpt300_causal_k2")
+    h, d, n_types = 8, 64, 11
+    q, k, v = (rand((c.n, h, d), torch.float32, s, 1.0 / 8).to(DEV) for s in (41, 42, 43))
+    table = rand((n_types, d), torch.float32, 44, 1.0 / 8).to(DEV)
+    etype = torch.from_numpy(np.random.default_rng(45).integers(0, n_types, c.E)).to(DEV)
+    want = op.bpt_attention(*c.out, *c.inn, q, k, v, rel_table=table, etype=etype)
+    old = graphop.set_row_groups(False)
+    try:
+        got = op.bpt_attention(*c.out, *c.inn, q, k, v, rel_table=table, etype=etype)          # op chain
+        bias = torch.zeros((c.E + 1, h), dtype=torch.float32, device=DEV)
+        with pytest.raises(RuntimeError):
+            graphop.attention_forward(*c.inn, q, k, v, bias=bias)
+    finally:
+        graphop.set_row_groups(old)
+    close(got, f64(want), TOL[torch.float32], "chain vs fused", c.max_deg)
+    with pytest.raises(ValueError):
+        graphop.attention_forward(*c.inn, q, k, v, bias=torch.zeros((c.E, h), dtype=torch.float32, device=DEV))   # no spare row
+    with pytest.raises(ValueError):
+        op.bpt_attention(*c.out, *c.inn, q, k, v, rel_table=table)                                                  # etype missing
+
+
 def test_block_uses_fused_dropout_in_training(ops):
     from bpt_amd.block import BPTBlock
     from bpt_amd import graphbuilder as gb
