@@ -38,7 +38,8 @@ GRAPH_API = {
     "bptg_plan_fill": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i64, c_i64, c_i64,
                                       c_vp, c_vp, c_vp, c_vp, c_vp, ctypes.POINTER(PlanInfo)]),
     "bptg_group_plan": (ctypes.c_int, [c_vp, c_i64, c_vp, c_vp, c_i64, c_i64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
-                                       ctypes.c_int32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
+                                       ctypes.c_int32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
+    "bptg_link_groups": (ctypes.c_int, [c_vp, c_i64, ctypes.c_int32, c_vp, c_i64, ctypes.c_int32, c_i64, ctypes.c_int32, c_vp]),
 }
 
 _PP = ctypes.POINTER(PlanStruct)

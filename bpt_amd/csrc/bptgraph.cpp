@@ -377,8 +377,8 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
 // handles two consecutive entries per step find the same members in both most of the time.
 int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32, const int32_t *eid32,
                     int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window, int32_t order_mode,
-                    int32_t max_pairs, int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *chunks,
-                    int64_t *n_groups_out, int64_t *n_entries_out) {
+                    int32_t max_pairs, int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *slot_eid,
+                    int32_t *chunks, int64_t *n_groups_out, int64_t *n_entries_out) {
     if (!items || !members || !grp_ptr || !chunks || !n_groups_out || !n_entries_out) return BPTG_ERR_NULL;
     if (n_edges > 0 && (!idx32 || !eid32 || !entries || !pair_eid)) return BPTG_ERR_NULL;
     if (n_items < 0 || n_edges < 0 || n_index_nodes < 0) return BPTG_ERR_SIZE;
@@ -492,7 +492,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
     std::vector<Triple> tri;
     std::vector<Entry> ents, placed;
     // the entries of one group in neighbour order
-    auto collect = [&](const int32_t *gmem) {
+    auto collect_sorted = [&](const int32_t *gmem) {        // general path: handles parallel edges
         tri.clear();
         ents.clear();
         for (int32_t m = 0; m < R; ++m)
@@ -529,6 +529,43 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
             }
             a = b;
         }
+    };
+    // Fast path (no member reaches a neighbour twice): the distinct neighbours are found through a stamped map and
+    // only they are sorted, not every edge of the group.
+    std::vector<int64_t> seen_in((size_t)n_index_nodes, -1);
+    std::vector<int32_t> local_of((size_t)n_index_nodes, 0);
+    std::vector<Entry> found;
+    std::vector<int32_t> by_idx;
+    int64_t collect_id = 0;
+    auto collect = [&](const int32_t *gmem) {
+        found.clear();
+        ++collect_id;
+        bool repeated = false;
+        for (int32_t m = 0; m < R && !repeated; ++m)
+            if (gmem[m] >= 0) {
+                const int32_t *it = items + 4 * (int64_t)gmem[m];
+                for (int32_t p = it[1]; p < it[2]; ++p) {
+                    const int32_t v = idx32[p];
+                    if (seen_in[(size_t)v] != collect_id) {
+                        seen_in[(size_t)v] = collect_id;
+                        local_of[(size_t)v] = (int32_t)found.size();
+                        Entry en;
+                        en.idx = v;
+                        en.mask = 0;
+                        found.push_back(en);
+                    }
+                    Entry &en = found[(size_t)local_of[(size_t)v]];
+                    if (en.mask >> m & 1) { repeated = true; break; }
+                    en.mask |= 1 << m;
+                    en.eids[m] = eid32[p];
+                }
+            }
+        if (repeated) { collect_sorted(gmem); return; }
+        by_idx.resize(found.size());
+        for (size_t i = 0; i < found.size(); ++i) by_idx[i] = (int32_t)i;
+        std::sort(by_idx.begin(), by_idx.end(), [&](int32_t a, int32_t b) { return found[(size_t)a].idx < found[(size_t)b].idx; });
+        ents.resize(found.size());
+        for (size_t i = 0; i < found.size(); ++i) ents[i] = found[(size_t)by_idx[i]];
     };
     // Aligned order: walking the groups in locality order, a neighbour keeps the position (the time step) it had
     // in the last group that read it whenever that position is free, and the other entries fill the gaps.  Wavefronts
@@ -595,14 +632,44 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
             en[1] = e.mask;
             en[2] = (int32_t)n_pairs;
             en[3] = 0;
-            for (int32_t m = 0; m < R; ++m)
-                if (e.mask >> m & 1) pair_eid[n_pairs++] = e.eids[m];
+            for (int32_t m = 0; m < R; ++m) {
+                const bool has = e.mask >> m & 1;
+                if (has) pair_eid[n_pairs++] = e.eids[m];
+                if (slot_eid) slot_eid[n_entries * R + m] = has ? e.eids[m] : -1;
+            }
             ++n_entries;
         }
         grp_ptr[gi + 1] = (int32_t)n_entries;
     }
     *n_groups_out = n_groups;
     *n_entries_out = n_entries;
+    return BPTG_OK;
+}
+
+int bptg_link_groups(const int32_t *slot_eid_dst, int64_t n_entries_dst, int32_t R_dst, const int32_t *slot_eid_src,
+                     int64_t n_entries_src, int32_t R_src, int64_t n_edges, int32_t pad_entries, int32_t *pairs) {
+    if (!pairs || (n_entries_dst > 0 && !slot_eid_dst) || (n_entries_src > 0 && !slot_eid_src)) return BPTG_ERR_NULL;
+    if (n_entries_dst < 0 || n_entries_src < 0 || n_edges < 0 || pad_entries < 0) return BPTG_ERR_SIZE;
+    if (R_dst < 1 || R_dst > 16 || R_src < 1 || R_src > 16) return BPTG_ERR_ARG;
+    if ((n_entries_src + pad_entries) * R_src >= INT32_MAX) return BPTG_ERR_SIZE;
+    std::vector<int32_t> pos_of((size_t)n_edges, -1);
+    int64_t covered = 0;
+    for (int64_t i = 0; i < n_entries_src * R_src; ++i) {
+        const int32_t e = slot_eid_src[i];
+        if (e < 0) continue;
+        if (e >= n_edges || pos_of[(size_t)e] >= 0) return BPTG_ERR_RANGE;          // not an edge, or an edge twice
+        pos_of[(size_t)e] = (int32_t)i;
+        ++covered;
+    }
+    if (covered != n_edges) return BPTG_ERR_RANGE;
+    const int32_t spare = (int32_t)((n_entries_src + pad_entries) * R_src - 1);
+    const int64_t n_real = n_entries_dst * R_dst, n_all = (n_entries_dst + pad_entries) * R_dst;
+    for (int64_t i = 0; i < n_real; ++i) {
+        const int32_t e = slot_eid_dst[i];
+        if (e >= n_edges) return BPTG_ERR_RANGE;
+        pairs[i] = e >= 0 ? pos_of[(size_t)e] : spare;
+    }
+    for (int64_t i = n_real; i < n_all; ++i) pairs[i] = spare;
     return BPTG_OK;
 }
 

@@ -101,39 +101,34 @@ def build_groups_host(arrays, n_index_nodes, R=None, window=GROUP_WINDOW, order_
     n_items, E = len(items), len(eid)
     members = np.empty((max(n_items, 1), R, 2), dtype=np.int32)
     grp_ptr = np.empty(n_items + 1, dtype=np.int32)
-    entries = np.zeros((E + 1, 4), dtype=np.int32)      # one zero row of padding: kernels may peek at entries[n_entries]
+    entries = np.empty((E + 1, 4), dtype=np.int32)
     pair_eid = np.empty(max(E, 1), dtype=np.int32)
+    slot_eid = np.empty((max(E, 1), R), dtype=np.int32)
     chunks = np.zeros(9, dtype=np.int32)
     ng, ne = ctypes.c_int64(), ctypes.c_int64()
     check_graph(graph_lib().bptg_group_plan(_ptr(items), n_items, _ptr(idx), _ptr(eid), E, int(n_index_nodes), R, window,
                                             int(order_mode), int(max_pairs), _ptr(members), _ptr(grp_ptr), _ptr(entries), _ptr(pair_eid),
-                                            _ptr(chunks), ctypes.byref(ng), ctypes.byref(ne)))
-    entries = entries[:ne.value].copy()
-    pair_eid = pair_eid[:E].copy()
-    present = (entries[:, 1:2] >> np.arange(R, dtype=np.int32)[None, :]) & 1 == 1      # (n_entries, R)
-    slot_eid = np.full((ne.value, R), -1, dtype=np.int32)
-    slot_eid[present] = pair_eid          # pairs are numbered entry by entry, members ascending
+                                            _ptr(slot_eid), _ptr(chunks), ctypes.byref(ng), ctypes.byref(ne)))
+    entries[ne.value] = 0                  # one zero row of padding: kernels may peek at entries[n_entries]
     return {"members": members[:ng.value].copy(), "grp_ptr": grp_ptr[:ng.value + 1].copy(),
-            "entries": entries, "pair_eid": pair_eid, "slot_eid": slot_eid, "chunks": chunks, "R": R}
+            "entries": entries[:ne.value].copy(), "pair_eid": pair_eid[:E].copy(), "slot_eid": slot_eid[:ne.value].copy(),
+            "chunks": chunks, "R": R}
 
 
 def link_groups_host(grp_dst, grp_src, n_edges):
-    """Pure host step: for every (entry, member) of the destination-side groups, the position
+    """Pure host step (bptg_link_groups): for every (entry, member) of the destination-side groups, the position
     entry' * R + member' of the same edge in the source-side groups; where the entry has no such member, and in
     the GROUP_PAD_ENTRIES * R elements of padding, the spare position (n_entries_src + GROUP_PAD_ENTRIES) * R - 1
     (the last one of the source side's padding, which no kernel uses).  int32, length
     (n_entries_dst + GROUP_PAD_ENTRIES) * R."""
-    R = grp_dst["R"]
-    src_slots = grp_src["slot_eid"].reshape(-1)
-    valid = np.flatnonzero(src_slots >= 0)
-    if len(valid) != n_edges:
+    sd = np.ascontiguousarray(grp_dst["slot_eid"], dtype=np.int32)
+    ss = np.ascontiguousarray(grp_src["slot_eid"], dtype=np.int32)
+    out = np.empty((len(sd) + GROUP_PAD_ENTRIES) * grp_dst["R"], dtype=np.int32)
+    st = graph_lib().bptg_link_groups(_ptr(sd), len(sd), grp_dst["R"], _ptr(ss), len(ss), grp_src["R"], int(n_edges),
+                                      GROUP_PAD_ENTRIES, _ptr(out))
+    if st == -4:          # BPTG_ERR_RANGE
         raise ValueError("the source-side groups do not cover every edge exactly once")
-    pos_of_eid = np.zeros(max(n_edges, 1), dtype=np.int32)
-    pos_of_eid[src_slots[valid]] = valid.astype(np.int32)
-    dst_slots = grp_dst["slot_eid"].reshape(-1)
-    spare = (len(grp_src["entries"]) + GROUP_PAD_ENTRIES) * R - 1
-    out = np.full((len(grp_dst["entries"]) + GROUP_PAD_ENTRIES) * R, spare, dtype=np.int32)
-    out[:len(dst_slots)] = np.where(dst_slots >= 0, pos_of_eid[np.maximum(dst_slots, 0)], spare)
+    check_graph(st)
     return out
 
 

@@ -90,6 +90,8 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
  *   entries  int32[n_edges*4]     (neighbour id, member bit mask, first pair, 0)
  *   pair_eid int32[n_edges]       edge id of every pair; pairs are numbered entry by entry, members
  *                                 ascending, and every edge of the plan appears exactly once
+ *   slot_eid int32[n_edges*R]     or NULL: edge id of (entry, member) at [entry*R + member], -1 where the
+ *                                 entry's mask has no such member (the first n_entries*R elements are written)
  *   chunks   int32[9]             groups chunks[x] .. chunks[x+1]-1 go to XCD x (contiguous, about equal work)
  * order_mode: low two bits = order of the groups inside a chunk — 0 locality, 1 at-least-average work first
  * then the small ones, 2 decreasing work; + 4 = inside a group, entries with equal member masks are made
@@ -102,8 +104,16 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
  * A neighbour that a member reaches through several parallel edges gets one entry per multiplicity. */
 int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32, const int32_t *eid32,
                     int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window, int32_t order_mode,
-                    int32_t max_pairs, int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *chunks,
-                    int64_t *n_groups, int64_t *n_entries);
+                    int32_t max_pairs, int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *slot_eid,
+                    int32_t *chunks, int64_t *n_groups, int64_t *n_entries);
+
+/* For every (entry, member) of the destination-side groups (slot_eid_dst: n_entries_dst * R_dst edge ids, -1 = absent)
+ * the position entry' * R_src + member' of the same edge in the source-side groups; where absent, and in the
+ * pad_entries * R_dst elements of padding, the spare position (n_entries_src + pad_entries) * R_src - 1.
+ * pairs: int32[(n_entries_dst + pad_entries) * R_dst].  BPTG_ERR_RANGE unless the source side holds every edge
+ * 0 .. n_edges-1 exactly once. */
+int bptg_link_groups(const int32_t *slot_eid_dst, int64_t n_entries_dst, int32_t R_dst, const int32_t *slot_eid_src,
+                     int64_t n_entries_src, int32_t R_src, int64_t n_edges, int32_t pad_entries, int32_t *pairs);
 
 #ifdef __cplusplus
 }

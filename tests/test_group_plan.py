@@ -189,3 +189,18 @@ def test_grouping_reduces_row_loads_on_the_headline_graph():
         ch = grp["chunks"]
         per = [cum[grp["grp_ptr"][ch[x + 1]]] - cum[grp["grp_ptr"][ch[x]]] for x in range(8)]
         assert max(per) < 1.10 * min(per)      # balanced on pairs + a fixed cost per group
+
+
+def test_link_groups_rejects_incomplete_source_side():
+    """bptg_link_groups: the source-side groups must hold every edge exactly once."""
+    src, dst, n, csr, pin, pout = plans(sorted(GRAPHS)[0], 64)
+    gd = build_groups_host(pin, n, R=4)
+    gs = build_groups_host(pout, n, R=4)
+    pairs = link_groups_host(gd, gs, len(src))
+    assert pairs.dtype == np.int32 and len(pairs) == (len(gd["entries"]) + 8) * 4
+    broken = dict(gs)
+    broken["slot_eid"] = gs["slot_eid"].copy()
+    r, c = np.argwhere(broken["slot_eid"] >= 0)[0]
+    broken["slot_eid"][r, c] = -1                      # one edge missing
+    with pytest.raises(ValueError):
+        link_groups_host(gd, broken, len(src))
