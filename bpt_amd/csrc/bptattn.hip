@@ -327,7 +327,6 @@ __global__ __launch_bounds__(BLOCK) void k_softmax_bwd(bpt_plan P, const T *__re
 // block of NW wavefronts per split row (grid = n_heavy).  Rows of up to SM_CACHE steps keep their values in
 // registers and read memory once; longer rows re-read.  Loads are issued SM_CACHE at a time.
 constexpr int SM_CACHE = 8;
-constexpr int SM_HEAVY_WAVES = 16;
 
 // reduction over the threads of a block that share t % H (H divides 64): first inside each wavefront, then over LDS
 template <typename A, int NW, bool IS_MAX> __device__ __forceinline__ A head_reduce(A x, int H, int h, A *smem) {
@@ -345,11 +344,13 @@ template <typename A, int NW, bool IS_MAX> __device__ __forceinline__ A head_red
     return r;
 }
 
-template <int NW> __device__ __forceinline__ bool softmax_range(const bpt_plan &P, int &begin, int &end) {
+// seg_slot: NULL = whole rows only (segments of split rows are skipped); else it receives the item's slot (-1 = whole row)
+template <int NW> __device__ __forceinline__ bool softmax_range(const bpt_plan &P, int &begin, int &end, int *seg_slot = nullptr) {
     if (NW == 1) {
         Item it;
-        if (!fetch_item(P, it) || it.slot >= 0) return false;
+        if (!fetch_item(P, it) || (it.slot >= 0 && !seg_slot)) return false;
         begin = it.begin; end = it.end;
+        if (seg_slot) *seg_slot = it.slot;
     } else {
         const int row = P.heavy[3 * blockIdx.x];
         begin = P.rowptr[row]; end = P.rowptr[row + 1];
@@ -358,11 +359,12 @@ template <int NW> __device__ __forceinline__ bool softmax_range(const bpt_plan &
 }
 
 template <typename T, int NW>
-__global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_fwd_heads(bpt_plan P, const T *__restrict__ x, T *__restrict__ y, int H) {
+__global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_fwd_heads(bpt_plan P, const T *__restrict__ x, T *__restrict__ y, int H,
+                                                                                   typename Elem<T>::acc_t *__restrict__ seg) {
     using acc_t = typename Elem<T>::acc_t;
     __shared__ acc_t smem[NW == 1 ? 1 : NW * WAVE];
-    int begin, end;
-    if (!softmax_range<NW>(P, begin, end)) return;
+    int begin, end, seg_slot = -1;
+    if (!softmax_range<NW>(P, begin, end, seg ? &seg_slot : nullptr)) return;
     const int tid = NW == 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
     const int h = tid % H, slot = tid / H, nslots = NW * WAVE / H;
     const bool cached = end - begin <= SM_CACHE * nslots;
@@ -392,6 +394,12 @@ __global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_fwd_hea
         for (int p = begin + slot; p < end; p += nslots) s += exp_acc((acc_t)Elem<T>::ld(x + (size_t)P.eid[p] * H + h) - m);
     }
     s = head_reduce<acc_t, NW, false>(s, H, h, smem);
+    if (seg_slot >= 0) {
+        // a segment of a split row: y gets exp(x - m) of the segment; its (m, s) go to the workspace, from which
+        // k_softmax_seg_rows forms the factor exp(m - M) / S that k_softmax_seg_scale applies
+        if (slot == 0) { seg[((size_t)seg_slot * H + h) * 2] = m; seg[((size_t)seg_slot * H + h) * 2 + 1] = s; }
+        s = 1;
+    }
     if (cached) {
 #pragma unroll
         for (int u = 0; u < SM_CACHE; ++u)
@@ -413,11 +421,12 @@ __global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_fwd_hea
 
 template <typename T, int NW>
 __global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_bwd_heads(bpt_plan P, const T *__restrict__ y, const T *__restrict__ dy,
-                                                                                   T *__restrict__ dx, int H) {
+                                                                                   T *__restrict__ dx, int H,
+                                                                                   typename Elem<T>::acc_t *__restrict__ seg) {
     using acc_t = typename Elem<T>::acc_t;
     __shared__ acc_t smem[NW == 1 ? 1 : NW * WAVE];
-    int begin, end;
-    if (!softmax_range<NW>(P, begin, end)) return;
+    int begin, end, seg_slot = -1;
+    if (!softmax_range<NW>(P, begin, end, seg ? &seg_slot : nullptr)) return;
     const int tid = NW == 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
     const int h = tid % H, slot = tid / H, nslots = NW * WAVE / H;
     const bool cached = end - begin <= SM_CACHE * nslots;
@@ -441,6 +450,12 @@ __global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_bwd_hea
         for (int u = 0; u < SM_CACHE; ++u) s += dc[u] * yc[u];
     }
     s = head_reduce<acc_t, NW, false>(s, H, h, smem);
+    if (seg_slot >= 0) {
+        // a segment of a split row: only its part of sum(dy * y); k_softmax_seg_rows adds the parts up and
+        // k_softmax_bwd_seg_finish writes dx
+        if (slot == 0) seg[(size_t)seg_slot * H + h] = s;
+        return;
+    }
     if (cached) {
 #pragma unroll
         for (int u = 0; u < SM_CACHE; ++u)
@@ -461,6 +476,64 @@ __global__ __launch_bounds__(NW == 1 ? BLOCK : NW * WAVE) void k_softmax_bwd_hea
             for (int u = 0; u < SM_CACHE; ++u)
                 if (e[u] >= 0) Elem<T>::st(dx + (size_t)e[u] * H + h, dv[u] * yv[u] - s * yv[u]);
         }
+    }
+}
+
+// Split rows of the softmax, second step: one block per split row.  Forward (PAIR): the segments' (m_i, s_i) become the
+// factors exp(m_i - M) / S with M = max(-1e9, m_i), S = sum s_i exp(m_i - M) (stored over m_i); backward: the segments'
+// partial sums are replaced by their total.  Thread t handles head t % H of slots t / H, t / H + n, ...
+template <typename A, bool PAIR>
+__global__ __launch_bounds__(BLOCK) void k_softmax_seg_rows(const int32_t *__restrict__ heavy, A *__restrict__ seg, int H) {
+    __shared__ A smem[WAVES_PER_BLOCK * WAVE];
+    const int s0 = heavy[3 * blockIdx.x + 1], ns = heavy[3 * blockIdx.x + 2];
+    const int h = threadIdx.x % H, j0 = threadIdx.x / H, nj = BLOCK / H;
+    constexpr int ST = PAIR ? 2 : 1;
+    if constexpr (PAIR) {
+        A m = (A)-1e9;
+        for (int j = j0; j < ns; j += nj) { const A v = seg[((size_t)(s0 + j) * H + h) * ST]; m = v > m ? v : m; }
+        m = head_reduce<A, WAVES_PER_BLOCK, true>(m, H, h, smem);
+        A s = 0;
+        for (int j = j0; j < ns; j += nj) s += seg[((size_t)(s0 + j) * H + h) * ST + 1] * exp_acc(seg[((size_t)(s0 + j) * H + h) * ST] - m);
+        s = head_reduce<A, WAVES_PER_BLOCK, false>(s, H, h, smem);
+        for (int j = j0; j < ns; j += nj) {
+            A *q = seg + ((size_t)(s0 + j) * H + h) * ST;
+            q[0] = exp_acc(q[0] - m) / s;
+        }
+    } else {
+        A s = 0;
+        for (int j = j0; j < ns; j += nj) s += seg[(size_t)(s0 + j) * H + h];
+        s = head_reduce<A, WAVES_PER_BLOCK, false>(s, H, h, smem);
+        for (int j = j0; j < ns; j += nj) seg[(size_t)(s0 + j) * H + h] = s;
+    }
+}
+
+// third step, one wavefront per item, segments only.  Forward: y *= factor of the segment.
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_softmax_seg_scale(bpt_plan P, T *__restrict__ y, int H, const typename Elem<T>::acc_t *__restrict__ seg) {
+    using acc_t = typename Elem<T>::acc_t;
+    Item it;
+    if (!fetch_item(P, it) || it.slot < 0) return;
+    const int tid = threadIdx.x & 63, h = tid % H, nslots = WAVE / H;
+    const acc_t f = seg[((size_t)it.slot * H + h) * 2];
+    for (int p = it.begin + tid / H; p < it.end; p += nslots) {
+        const size_t o = (size_t)P.eid[p] * H + h;
+        Elem<T>::st(y + o, (acc_t)Elem<T>::ld(y + o) * f);
+    }
+}
+
+// Backward: dx = y * (dy - total) on the segments.
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_softmax_bwd_seg_finish(bpt_plan P, const T *__restrict__ y, const T *__restrict__ dy, T *__restrict__ dx,
+                                                                  int H, const typename Elem<T>::acc_t *__restrict__ seg) {
+    using acc_t = typename Elem<T>::acc_t;
+    Item it;
+    if (!fetch_item(P, it) || it.slot < 0) return;
+    const int tid = threadIdx.x & 63, h = tid % H, nslots = WAVE / H;
+    const acc_t t = seg[(size_t)it.slot * H + h];
+    for (int p = it.begin + tid / H; p < it.end; p += nslots) {
+        const size_t o = (size_t)P.eid[p] * H + h;
+        const acc_t yv = (acc_t)Elem<T>::ld(y + o);
+        Elem<T>::st(dx + o, yv * ((acc_t)Elem<T>::ld(dy + o) - t));
     }
 }
 
@@ -1820,14 +1893,18 @@ int run_spmm_generic(const bpt_plan *P, const void *W, const void *X, void *Y, v
 }
 
 template <typename T>
-int run_softmax_fwd(const bpt_plan *P, const void *x, void *y, int h, hipStream_t s) {
+int run_softmax_fwd(const bpt_plan *P, const void *x, void *y, void *ws, int h, hipStream_t s) {
+    using acc_t = typename Elem<T>::acc_t;
     if (P->n_items == 0) return BPT_OK;
-    if (WAVE % h == 0) {       // heads side by side
-        hipLaunchKernelGGL((k_softmax_fwd_heads<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)x, (T *)y, h);
+    if (WAVE % h == 0) {       // heads side by side; split rows in three steps over their segments
+        acc_t *seg = P->n_heavy > 0 ? (acc_t *)ws : nullptr;
+        hipLaunchKernelGGL((k_softmax_fwd_heads<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)x, (T *)y, h, seg);
         int st = launch_status();
         if (st != BPT_OK || P->n_heavy == 0) return st;
-        hipLaunchKernelGGL((k_softmax_fwd_heads<T, SM_HEAVY_WAVES>), dim3((int)P->n_heavy), dim3(SM_HEAVY_WAVES * WAVE), 0, s, *P,
-                           (const T *)x, (T *)y, h);
+        hipLaunchKernelGGL((k_softmax_seg_rows<acc_t, true>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, seg, h);
+        st = launch_status();
+        if (st != BPT_OK) return st;
+        hipLaunchKernelGGL((k_softmax_seg_scale<T>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (T *)y, h, (const acc_t *)seg);
         return launch_status();
     }
     hipLaunchKernelGGL((k_softmax_fwd<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)x, (T *)y, h);
@@ -1838,14 +1915,19 @@ int run_softmax_fwd(const bpt_plan *P, const void *x, void *y, int h, hipStream_
 }
 
 template <typename T>
-int run_softmax_bwd(const bpt_plan *P, const void *y, const void *dy, void *dx, int h, hipStream_t s) {
+int run_softmax_bwd(const bpt_plan *P, const void *y, const void *dy, void *dx, void *ws, int h, hipStream_t s) {
+    using acc_t = typename Elem<T>::acc_t;
     if (P->n_items == 0) return BPT_OK;
-    if (WAVE % h == 0) {       // heads side by side
-        hipLaunchKernelGGL((k_softmax_bwd_heads<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)y, (const T *)dy, (T *)dx, h);
+    if (WAVE % h == 0) {       // heads side by side; split rows in three steps over their segments
+        acc_t *seg = P->n_heavy > 0 ? (acc_t *)ws : nullptr;
+        hipLaunchKernelGGL((k_softmax_bwd_heads<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)y, (const T *)dy, (T *)dx, h, seg);
         int st = launch_status();
         if (st != BPT_OK || P->n_heavy == 0) return st;
-        hipLaunchKernelGGL((k_softmax_bwd_heads<T, SM_HEAVY_WAVES>), dim3((int)P->n_heavy), dim3(SM_HEAVY_WAVES * WAVE), 0, s, *P,
-                           (const T *)y, (const T *)dy, (T *)dx, h);
+        hipLaunchKernelGGL((k_softmax_seg_rows<acc_t, false>), dim3((int)P->n_heavy), dim3(BLOCK), 0, s, P->heavy, seg, h);
+        st = launch_status();
+        if (st != BPT_OK) return st;
+        hipLaunchKernelGGL((k_softmax_bwd_seg_finish<T>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)y, (const T *)dy, (T *)dx, h,
+                           (const acc_t *)seg);
         return launch_status();
     }
     hipLaunchKernelGGL((k_softmax_bwd<T, 1>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)y, (const T *)dy, (T *)dx, h);
@@ -2209,6 +2291,8 @@ int64_t bpt_workspace_bytes(int op, const bpt_plan *plan, const bpt_plan *plan_t
         case BPT_OP_SPMM_FWD: return round16(s0 * C * a);
         case BPT_OP_SPMM_BWD: return round16(s1 * C * a);
         case BPT_OP_ATTN_FWD: return round16(s0 * (C + 2 * h) * 4);
+        case BPT_OP_SOFTMAX_FWD: return WAVE % h == 0 ? round16(s0 * h * 2 * a) : 0;      // (m, s) of every segment and head
+        case BPT_OP_SOFTMAX_BWD: return WAVE % h == 0 ? round16(s0 * h * a) : 0;
         case BPT_OP_ATTN_BWD: {
             // partial rows of dq, then of dk and dv (the three are merged by one launch after the source-side kernel)
             return pds_bytes(plan, plan_t, h, d, dtype == BPT_BF16 ? 2 : 4) + round16((s0 + 2 * s1) * C * 4);
@@ -2273,18 +2357,24 @@ int bpt_node_mul_edge_backward(const bpt_plan *plan, const void *A, const void *
     DISPATCH_DTYPE(dtype, (run_nme_dB<T>(plan, A, dy, dB, h, d, (hipStream_t)stream)))
 }
 
-int bpt_sparse_softmax_forward(const bpt_plan *plan, const void *x, void *y, int h, int dtype, void *stream) {
+int bpt_sparse_softmax_forward(const bpt_plan *plan, const void *x, void *y, void *workspace, int64_t workspace_bytes, int h,
+                               int dtype, void *stream) {
     CHECK(check_plan(plan, false));
     CHECK(check_shape(h, 1, dtype));
     if (plan->n_edges > 0 && (!x || !y)) return BPT_ERR_NULL;
-    DISPATCH_DTYPE(dtype, (run_softmax_fwd<T>(plan, x, y, h, (hipStream_t)stream)))
+    const int64_t need = bpt_workspace_bytes(BPT_OP_SOFTMAX_FWD, plan, nullptr, h, 1, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    DISPATCH_DTYPE(dtype, (run_softmax_fwd<T>(plan, x, y, workspace, h, (hipStream_t)stream)))
 }
 
-int bpt_sparse_softmax_backward(const bpt_plan *plan, const void *y, const void *dy, void *dx, int h, int dtype, void *stream) {
+int bpt_sparse_softmax_backward(const bpt_plan *plan, const void *y, const void *dy, void *dx, void *workspace,
+                                int64_t workspace_bytes, int h, int dtype, void *stream) {
     CHECK(check_plan(plan, false));
     CHECK(check_shape(h, 1, dtype));
     if (plan->n_edges > 0 && (!y || !dy || !dx)) return BPT_ERR_NULL;
-    DISPATCH_DTYPE(dtype, (run_softmax_bwd<T>(plan, y, dy, dx, h, (hipStream_t)stream)))
+    const int64_t need = bpt_workspace_bytes(BPT_OP_SOFTMAX_BWD, plan, nullptr, h, 1, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    DISPATCH_DTYPE(dtype, (run_softmax_bwd<T>(plan, y, dy, dx, workspace, h, (hipStream_t)stream)))
 }
 
 int bpt_vector_spmm_forward(const bpt_plan *plan, const void *edata, const void *x, void *y, void *workspace,

@@ -24,7 +24,7 @@ __all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forwa
 _LIB = attn_lib()          # fail at import time if the HIP library is missing
 
 _DTYPE = {torch.float32: 0, torch.float64: 1, torch.bfloat16: 2}
-OP_MASKEDMM_BWD, OP_NME_BWD, OP_SPMM_FWD, OP_SPMM_BWD, OP_ATTN_FWD, OP_ATTN_BWD = 1, 2, 3, 4, 5, 6
+OP_MASKEDMM_BWD, OP_NME_BWD, OP_SPMM_FWD, OP_SPMM_BWD, OP_ATTN_FWD, OP_ATTN_BWD, OP_SOFTMAX_FWD, OP_SOFTMAX_BWD = 1, 2, 3, 4, 5, 6, 7, 8
 
 
 def _check_input(t, name):
@@ -158,8 +158,9 @@ def sparse_softmax_forward(row, indptr, eid, x):
     _check_all(row=row, indptr=indptr, eid=eid, x=x)
     plan = plan_cache.get(row, indptr, eid, None, None, None)
     y = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(x)
+    ws, nws = _workspace(OP_SOFTMAX_FWD, plan, None, _edge_h(x), 1, _dtype(x), x.device)
     with torch.cuda.device_of(x):
-        check_attn(_LIB.bpt_sparse_softmax_forward(plan.ref, _ptr(x), _ptr(y), _edge_h(x), _dtype(x), _stream()),
+        check_attn(_LIB.bpt_sparse_softmax_forward(plan.ref, _ptr(x), _ptr(y), _ptr(ws), nws, _edge_h(x), _dtype(x), _stream()),
                    "sparse_softmax_forward")
     return y
 
@@ -170,8 +171,10 @@ def sparse_softmax_backward(row, indptr, eid, y, dy):
     _same_dtype(y, dy)
     plan = plan_cache.get(row, indptr, eid, None, None, None)
     dx = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(dy)
+    ws, nws = _workspace(OP_SOFTMAX_BWD, plan, None, _edge_h(dy), 1, _dtype(y), y.device)
     with torch.cuda.device_of(y):
-        check_attn(_LIB.bpt_sparse_softmax_backward(plan.ref, _ptr(y), _ptr(dy), _ptr(dx), _edge_h(dy), _dtype(y), _stream()),
+        check_attn(_LIB.bpt_sparse_softmax_backward(plan.ref, _ptr(y), _ptr(dy), _ptr(dx), _ptr(ws), nws, _edge_h(dy), _dtype(y),
+                                                    _stream()),
                    "sparse_softmax_backward")
     return dx
 

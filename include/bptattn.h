@@ -84,7 +84,7 @@ int bpt_profile_kernel(int which, void *start_event, void *stop_event);
 /* Bytes of workspace the call needs (0 possible).  op: one of the BPT_OP_* below. */
 enum {
     BPT_OP_MASKEDMM_BWD = 1, BPT_OP_NODE_MUL_EDGE_BWD = 2, BPT_OP_SPMM_FWD = 3, BPT_OP_SPMM_BWD = 4,
-    BPT_OP_ATTN_FWD = 5, BPT_OP_ATTN_BWD = 6
+    BPT_OP_ATTN_FWD = 5, BPT_OP_ATTN_BWD = 6, BPT_OP_SOFTMAX_FWD = 7, BPT_OP_SOFTMAX_BWD = 8
 };
 int64_t bpt_workspace_bytes(int op, const bpt_plan *plan, const bpt_plan *plan_t, int h, int d, int dtype);
 
@@ -110,12 +110,14 @@ int bpt_node_mul_edge_backward(const bpt_plan *plan, const void *A, const void *
                                int h, int d, int dtype, void *stream);
 
 /* graphop.cpp:59  sparse_softmax_forward(row, indptr, eid, x) -> y   (softmax over each row's slots;
- * the running maximum starts at -1e9 as in graphop_kernel.cu:428) */
-int bpt_sparse_softmax_forward(const bpt_plan *plan, const void *x, void *y, int h, int dtype, void *stream);
+ * the running maximum starts at -1e9 as in graphop_kernel.cu:428).  The workspace (bpt_workspace_bytes with
+ * BPT_OP_SOFTMAX_FWD, d = 1) holds the per-segment maxima and sums of the rows that the plan splits. */
+int bpt_sparse_softmax_forward(const bpt_plan *plan, const void *x, void *y, void *workspace, int64_t workspace_bytes,
+                               int h, int dtype, void *stream);
 
-/* graphop.cpp:163 sparse_softmax_backward(row, indptr, eid, y, dy) -> dx */
-int bpt_sparse_softmax_backward(const bpt_plan *plan, const void *y, const void *dy, void *dx,
-                                int h, int dtype, void *stream);
+/* graphop.cpp:163 sparse_softmax_backward(row, indptr, eid, y, dy) -> dx   (workspace: BPT_OP_SOFTMAX_BWD) */
+int bpt_sparse_softmax_backward(const bpt_plan *plan, const void *y, const void *dy, void *dx, void *workspace,
+                                int64_t workspace_bytes, int h, int dtype, void *stream);
 
 /* graphop.cpp:79  vector_spmm_forward(row, indptr, eid, indices, edata, x) -> y
  * y[r] = sum_p edata[eid[p]] * x[idx[p]];  every row of y is written (zero for empty rows). */

@@ -40,10 +40,10 @@ def test_error_strings_and_argument_errors_without_gpu():
     # argument errors are detected before anything touches the device
     assert alib.bpt_maskedmm_csr_forward(None, None, None, None, 8, 64, 0, None) == -1
     plan = _lib.PlanStruct(None, None, None, None, None, 0, 0, 0, 0, 0)
-    assert alib.bpt_sparse_softmax_forward(ctypes.byref(plan), None, None, 8, 7, None) == -3          # dtype
+    assert alib.bpt_sparse_softmax_forward(ctypes.byref(plan), None, None, None, 0, 8, 7, None) == -3          # dtype
     assert alib.bpt_vector_spmm_forward(ctypes.byref(plan), None, None, None, None, 0, 0, 64, 0, None) == -4   # h = 0
     plan_bad = _lib.PlanStruct(None, None, None, None, None, 0, -1, 0, 0, 0)
-    assert alib.bpt_sparse_softmax_forward(ctypes.byref(plan_bad), None, None, 8, 0, None) == -2
+    assert alib.bpt_sparse_softmax_forward(ctypes.byref(plan_bad), None, None, None, 0, 8, 0, None) == -2
     assert alib.bpt_workspace_bytes(5, ctypes.byref(plan), None, 8, 64, 0) == 0
     assert _lib.graph_lib().bptg_strerror(-4).startswith(b"row id")
 
