@@ -145,7 +145,8 @@ SHAPES = [(8, 64), (1, 40), (3, 20), (4, 64)]   # (8,64)/(4,64) have specialised
 @pytest.mark.parametrize("force_generic", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
 @pytest.mark.parametrize("hd", SHAPES)
-@pytest.mark.parametrize("gname,chunk", [("blocks8x30", 32), ("blocks8x30", 7), ("bpt512_k4", 32), ("multigraph", 8), ("fc_w100", 32)])
+@pytest.mark.parametrize("gname,chunk", [("blocks8x30", 32), ("blocks8x30", 7), ("bpt512_k4", 32), ("multigraph", 8), ("fc_w100", 32),
+                                         ("bpt256_k24", 32)])
 def test_ops_match_oracle(ops, gname, chunk, hd, dtype, force_generic):
     graphop, _ = ops
     h, d = hd
