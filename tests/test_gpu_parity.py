@@ -465,6 +465,32 @@ def test_rel_pos_without_row_groups_takes_the_op_chain_and_the_raw_call_refuses(
         op.bpt_attention(*c.out, *c.inn, q, k, v, rel_table=table)                                                  # etype missing
 
 
+@pytest.mark.parametrize("rows", [4, 8])
+def test_fused_attention_with_large_scores(ops, rows):
+    """Scores of +-60 (q, k four times the usual size): nearly one-hot softmax rows, exponent references that move by
+    large steps.  Errors are measured against the largest element (rounding of a score of 60 moves its exponential
+    by 4e-6 relative in float32)."""
+    from oracle import torch_ops
+    graphop, op = ops
+    c = case("bpt512_k4")
+    h, d = 8, 64
+    q, k = (rand((c.n, h, d), torch.float32, s, 4.0).to(DEV).requires_grad_(True) for s in (51, 52))
+    v = rand((c.n, h, d), torch.float32, 53).to(DEV).requires_grad_(True)
+    do = rand((c.n, h, d), torch.float32, 54).to(DEV)
+    old_r = graphop.set_group_rows(rows)
+    try:
+        o = op.bpt_attention(*c.out, *c.inn, q, k, v)
+        o.backward(do)
+    finally:
+        graphop.set_group_rows(old_r)
+    t64 = lambda x: x.detach().cpu().double()
+    ro, rdq, rdk, rdv = torch_ops.attention_fwd_bwd(torch.from_numpy(c.src), torch.from_numpy(c.dst), t64(q), t64(k), t64(v), t64(do))
+    assert torch.isfinite(o).all()
+    for got, want, nm in ((o, ro, "o"), (q.grad, rdq, "dq"), (k.grad, rdk, "dk"), (v.grad, rdv, "dv")):
+        err = float((t64(got) - want).abs().max() / want.abs().max())
+        assert err < 5e-5, (nm, err)
+
+
 def test_block_uses_fused_dropout_in_training(ops):
     from bpt_amd.block import BPTBlock
     from bpt_amd import graphbuilder as gb
