@@ -1334,9 +1334,9 @@ template <typename T> __device__ __forceinline__ void unpack_vec(const uint4 &w,
 }
 
 // Two wavefronts per group of 8 rows: wavefront w owns members 4 w .. 4 w + 3 (one quad: the B operand of the
-// score products), both share the staged rows.  Each wavefront loads and stages half of a batch; the staging area
-// is double buffered, so one workgroup barrier per batch orders the writes of batch b + 1 after the reads of
-// batch b - 1.
+// score products), both share the staged rows.  Each wavefront loads and stages half of a batch.  With two staging
+// buffers one workgroup barrier per batch orders the writes of batch b + 1 after the reads of batch b - 1; where V
+// has a single buffer (W3 below) a second barrier separates the reads of batch b from the writes of batch b + 1.
 template <typename T, int H, int D, int HS, bool DROP, bool BIAS>
 __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 && !BIAS ? 3 : 2))) void k_attn_fwd_mfma(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
