@@ -1,7 +1,8 @@
-"""Compiles the two native libraries in-tree:
+"""Compiles the three native libraries in-tree:
 
   bpt_amd/csrc/libbptgraph.so  host C++ (g++)            <- bptgraph.cpp
   bpt_amd/csrc/libbptattn.so   gfx950 HIP (hipcc)        <- bptattn.hip
+  bpt_amd/csrc/libbptplan.so   gfx950 HIP (hipcc)        <- bptplan.hip  (plans built on the GPU; rocPRIM headers)
 
 hipcc cross-compiles for gfx950 without a GPU.  Run `python -m bpt_amd._build`.
 """
@@ -12,6 +13,7 @@ import sys
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 GRAPH_SO = os.path.join(CSRC, "libbptgraph.so")
 ATTN_SO = os.path.join(CSRC, "libbptattn.so")
+PLAN_SO = os.path.join(CSRC, "libbptplan.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
@@ -39,8 +41,16 @@ def build_attn(verbose=True, extra=(), out=None):
     return ATTN_SO
 
 
+def build_plan(verbose=True):
+    cmd = [HIPCC] + HIP_FLAGS + [os.path.join(CSRC, "bptplan.hip"), "-o", PLAN_SO]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return PLAN_SO
+
+
 def build_all(verbose=True):
-    return build_graph(verbose), build_attn(verbose)
+    return build_graph(verbose), build_attn(verbose), build_plan(verbose)
 
 
 if __name__ == "__main__":

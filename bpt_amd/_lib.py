@@ -6,7 +6,7 @@ There is no Python or CPU fallback for the device ops: if libbptattn.so is missi
 import ctypes
 import os
 
-from ._build import ATTN_SO, GRAPH_SO
+from ._build import ATTN_SO, GRAPH_SO, PLAN_SO
 
 c_i64 = ctypes.c_int64
 c_vp = ctypes.c_void_p
@@ -64,8 +64,20 @@ ATTN_API = {
                                              c_i64, ctypes.c_float, ctypes.c_float, ctypes.c_uint64] + _tail),
 }
 
+c_i32 = ctypes.c_int32
+# libbptplan (include/bptplan.h): plans built on the GPU
+PLAN_API = {
+    "bpt_plan_device_bounds": (ctypes.c_int, [c_i64, c_i64, c_i64, c_i32, c_i32, ctypes.POINTER(c_i64 * 4)]),
+    "bpt_plan_build_device": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32,
+                                             c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp]),
+    "bpt_plan_group_device": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32,
+                                             c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp]),
+    "bpt_plan_link_device": (ctypes.c_int, [c_vp, c_vp, c_i32, c_vp, c_vp, c_i32, c_i64, c_i32, c_vp, c_vp, c_i64, c_vp]),
+}
+
 _graph = None
 _attn = None
+_plan = None
 
 
 def _load(path, api, what):
@@ -92,6 +104,13 @@ def attn_lib():
         # BPT_ATTN_SO: load another build of the same library (kernel experiments); default = the in-tree build
         _attn = _load(os.environ.get("BPT_ATTN_SO", ATTN_SO), ATTN_API, "libbptattn (HIP kernels)")
     return _attn
+
+
+def plan_lib():
+    global _plan
+    if _plan is None:
+        _plan = _load(PLAN_SO, PLAN_API, "libbptplan (plans built on the GPU)")
+    return _plan
 
 
 def check_graph(status):

@@ -1,0 +1,708 @@
+// libbptplan — launch plans and row groups built on the GPU (gfx950), C ABI of include/bptplan.h.
+//
+// The host builder (bptgraph.cpp) needs the index arrays on the host and tens of milliseconds per new graph.  Here the
+// same plan comes out of sorts and prefix sums over the device arrays: every step is a data-parallel kernel or a
+// rocPRIM primitive on the caller's stream, sizes that depend on the data stay on the device (kernels are launched
+// for the upper bounds and read the actual counts from the info blocks), and all integer results are independent of
+// the execution order (the only atomics are integer max / or / add whose results do not depend on their order).
+//
+// The reference has no plans: its kernels take the chunked CSR arrays of graph/base.py:71-86 as they are.
+#include <cstring>
+
+#include <hip/hip_runtime.h>
+
+#include <rocprim/rocprim.hpp>
+
+#include <cstdint>
+
+#include "../../include/bptattn.h"
+#include "../../include/bptplan.h"
+
+namespace {
+
+constexpr int TPB = 256;
+constexpr int FIXED_WORK = 24;        // cost of a group beyond its pairs, in pair equivalents (as the host builder)
+constexpr uint32_t PAD32 = 0xFFFFFFFFu;
+constexpr uint64_t PAD64 = ~uint64_t(0);
+
+inline unsigned blocks_for(int64_t n) { return (unsigned)((n + TPB - 1) / TPB); }
+
+inline unsigned bits_for(uint64_t max_value) {      // bits needed to hold values 0 .. max_value
+    unsigned b = 1;
+    while (b < 64 && (max_value >> b) != 0) ++b;
+    return b;
+}
+
+// Carves 256-byte aligned arrays out of the caller's workspace; with a null base it only adds up the sizes.
+struct Bump {
+    char *base;
+    size_t off;
+    template <typename T> T *take(int64_t n) {
+        off = (off + 255) & ~size_t(255);
+        T *p = base ? reinterpret_cast<T *>(base + off) : nullptr;
+        off += (size_t)(n > 0 ? n : 1) * sizeof(T);
+        return p;
+    }
+};
+
+// ---- rocPRIM wrappers (temporary storage = one shared region of the workspace) ------------------------------------
+template <typename K>
+hipError_t sort_pairs(void *tmp, size_t &bytes, const K *kin, K *kout, const int32_t *vin, int32_t *vout, int64_t n,
+                      unsigned end_bit, hipStream_t s) {
+    return rocprim::radix_sort_pairs(tmp, bytes, kin, kout, vin, vout, (size_t)n, 0u, end_bit, s, false);
+}
+
+hipError_t scan_i32(void *tmp, size_t &bytes, const int32_t *in, int32_t *out, int64_t n, hipStream_t s) {
+    return rocprim::exclusive_scan(tmp, bytes, in, out, (int32_t)0, (size_t)n, rocprim::plus<int32_t>(), s, false);
+}
+
+// largest temporary storage any primitive of the three entry points asks for
+hipError_t temp_bytes(int64_t max_items, int64_t max_groups, int64_t n_edges, int64_t n_rows, size_t *out) {
+    size_t best = 0, b = 0;
+    hipError_t e;
+    if ((e = sort_pairs<uint32_t>(nullptr, b, nullptr, nullptr, nullptr, nullptr, max_items + 1, 32, nullptr)) != hipSuccess) return e;
+    best = b > best ? b : best;
+    if ((e = sort_pairs<uint32_t>(nullptr, b, nullptr, nullptr, nullptr, nullptr, max_groups + 1, 32, nullptr)) != hipSuccess) return e;
+    best = b > best ? b : best;
+    if ((e = sort_pairs<uint64_t>(nullptr, b, nullptr, nullptr, nullptr, nullptr, n_edges + 1, 64, nullptr)) != hipSuccess) return e;
+    best = b > best ? b : best;
+    int64_t ns = n_rows + 1;
+    ns = ns > n_edges + 1 ? ns : n_edges + 1;
+    ns = ns > max_groups + 1 ? ns : max_groups + 1;
+    if ((e = scan_i32(nullptr, b, nullptr, nullptr, ns, nullptr)) != hipSuccess) return e;
+    best = b > best ? b : best;
+    *out = best + 256;
+    return hipSuccess;
+}
+
+// ---- small helpers ---------------------------------------------------------------------------------------------------
+__global__ void k_fill_i32(int32_t *p, int64_t n, int32_t v) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+__global__ void k_iota_i32(int32_t *p, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i < n) p[i] = (int32_t)i;
+}
+
+// ---- base plan ---------------------------------------------------------------------------------------------------------
+struct BaseWs {
+    int32_t *c_items, *c_heavy, *c_slots, *b_items, *b_heavy, *b_slots, *seen, *items_tmp, *iota, *perm;
+    uint32_t *key, *key_s;
+    void *tmp;
+};
+
+BaseWs base_layout(Bump &b, int64_t n_rows, int64_t n_edges, int64_t max_items, size_t tmp_bytes) {
+    BaseWs w;
+    w.c_items = b.take<int32_t>(n_rows + 1);
+    w.c_heavy = b.take<int32_t>(n_rows + 1);
+    w.c_slots = b.take<int32_t>(n_rows + 1);
+    w.b_items = b.take<int32_t>(n_rows + 1);
+    w.b_heavy = b.take<int32_t>(n_rows + 1);
+    w.b_slots = b.take<int32_t>(n_rows + 1);
+    w.seen = b.take<int32_t>(n_edges);
+    w.items_tmp = b.take<int32_t>(4 * max_items);
+    w.iota = b.take<int32_t>(max_items);
+    w.perm = b.take<int32_t>(max_items);
+    w.key = b.take<uint32_t>(max_items);
+    w.key_s = b.take<uint32_t>(max_items);
+    w.tmp = b.take<char>((int64_t)tmp_bytes);
+    return w;
+}
+
+__global__ void k_base_init(int32_t *info, const int64_t *ipu, int64_t n_units, int64_t n_edges) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    for (int i = 0; i < 16; ++i) info[i] = 0;
+    int err = 0;
+    bool covers = (n_edges == 0);
+    if (n_units > 0) {
+        const int64_t first = ipu[0], last = ipu[n_units];
+        if (first < 0 || last >= INT32_MAX) err = 3;
+        else if (last > n_edges) err = 1;
+        covers = (first == 0 && last == n_edges);
+    }
+    info[BPT_PI_ERR] = err;
+    info[BPT_PI_FLAGS] = covers ? 1 : 0;
+}
+
+__global__ void k_check_units(const int64_t *row, const int64_t *ipu, int64_t n_units, int64_t n_rows, int32_t *info) {
+    const int64_t u = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (u >= n_units) return;
+    int err = 0;
+    if (row[u] < 0 || row[u] >= n_rows) err = 1;
+    if (u > 0 && row[u] < row[u - 1]) err = err > 2 ? err : 2;
+    if (ipu[u + 1] < ipu[u]) err = err > 2 ? err : 2;
+    if (err) atomicMax(&info[BPT_PI_ERR], err);
+}
+
+// rowptr[r] = start of the first unit whose row is >= r (rows without a unit are empty)
+__global__ void k_rowptr(const int64_t *row, const int64_t *ipu, int64_t n_units, int64_t n_rows, const int32_t *info,
+                         int32_t *rowptr) {
+    const int64_t r = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (r > n_rows || info[BPT_PI_ERR]) return;
+    int64_t lo = 0, hi = n_units;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (row[mid] < r) lo = mid + 1; else hi = mid;
+    }
+    rowptr[r] = n_units > 0 ? (int32_t)ipu[lo] : 0;
+}
+
+__global__ void k_row_counts(const int32_t *rowptr, int64_t n_rows, int32_t seg_len, int32_t *info, int32_t *c_items,
+                             int32_t *c_heavy, int32_t *c_slots) {
+    const int64_t r = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (r > n_rows || info[BPT_PI_ERR]) return;
+    int32_t ni = 0, nh = 0, ns = 0;
+    if (r < n_rows) {
+        const int32_t deg = rowptr[r + 1] - rowptr[r];
+        ni = 1;
+        if (deg > seg_len) {
+            nh = 1;
+            ni = ns = (deg + seg_len - 1) / seg_len;
+        }
+        atomicMax(&info[BPT_PI_MAX_DEGREE], deg);
+    }
+    c_items[r] = ni;
+    c_heavy[r] = nh;
+    c_slots[r] = ns;
+}
+
+__global__ void k_emit_items(const int32_t *rowptr, int64_t n_rows, int32_t seg_len, const int32_t *b_items,
+                             const int32_t *b_heavy, const int32_t *b_slots, int32_t *info, int32_t *items, int32_t *heavy) {
+    const int64_t r = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (r > n_rows || info[BPT_PI_ERR]) return;
+    if (r == n_rows) {
+        info[BPT_PI_N_ITEMS] = b_items[n_rows];
+        info[BPT_PI_N_HEAVY] = b_heavy[n_rows];
+        info[BPT_PI_N_SLOTS] = b_slots[n_rows];
+        return;
+    }
+    const int32_t begin = rowptr[r], end = rowptr[r + 1], deg = end - begin;
+    int4 *out = reinterpret_cast<int4 *>(items) + b_items[r];
+    if (deg <= seg_len) {
+        *out = make_int4((int32_t)r, begin, end, -1);
+        return;
+    }
+    const int32_t n_seg = (deg + seg_len - 1) / seg_len, s0 = b_slots[r];
+    int32_t *hv = heavy + 3 * (int64_t)b_heavy[r];
+    hv[0] = (int32_t)r;
+    hv[1] = s0;
+    hv[2] = n_seg;
+    for (int32_t s = 0; s < n_seg; ++s) {
+        const int32_t b = begin + s * seg_len;
+        out[s] = make_int4((int32_t)r, b, min(end, b + seg_len), s0 + s);
+    }
+}
+
+__global__ void k_narrow(const int64_t *eid, const int64_t *indices, int64_t n_edges, int64_t n_index_nodes, int32_t *info,
+                         int32_t *idx32, int32_t *eid32, int32_t *seen) {
+    const int64_t p = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (p >= n_edges) return;
+    const int64_t e = eid[p], c = indices ? indices[p] : 0;
+    if (e < 0 || e >= n_edges || c < 0 || (indices && c >= n_index_nodes)) {
+        atomicMax(&info[BPT_PI_ERR], 1);
+        eid32[p] = 0;
+        idx32[p] = 0;
+        return;
+    }
+    eid32[p] = (int32_t)e;
+    idx32[p] = (int32_t)c;
+    if (atomicAdd(&seen[e], 1) != 0) atomicAnd(&info[BPT_PI_FLAGS], ~1);
+}
+
+// Sort key of every item: smallest (LARGEST = false) or largest neighbour id; an empty item takes its own row id,
+// clipped to n_index_nodes.  Positions past n_items get the padding key, which sorts behind every real one.
+template <bool LARGEST>
+__global__ void k_item_keys(const int32_t *items, const int32_t *idx32, const int32_t *info, int64_t max_items,
+                            int64_t n_index_nodes, uint32_t *key) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= max_items) return;
+    if (info[BPT_PI_ERR] || i >= info[BPT_PI_N_ITEMS]) {
+        key[i] = PAD32;
+        return;
+    }
+    const int4 it = reinterpret_cast<const int4 *>(items)[i];
+    int32_t k = it.x < n_index_nodes ? it.x : (int32_t)n_index_nodes;
+    if (it.z > it.y) {
+        k = idx32[it.y];
+        for (int32_t p = it.y + 1; p < it.z; ++p) k = LARGEST ? max(k, idx32[p]) : min(k, idx32[p]);
+    }
+    key[i] = (uint32_t)k;
+}
+
+__global__ void k_gather_items(const int32_t *items_tmp, const int32_t *perm, const int32_t *info, int64_t max_items,
+                               int32_t *items) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= max_items || info[BPT_PI_ERR] || i >= info[BPT_PI_N_ITEMS]) return;
+    reinterpret_cast<int4 *>(items)[i] = reinterpret_cast<const int4 *>(items_tmp)[perm[i]];
+}
+
+// ---- row groups --------------------------------------------------------------------------------------------------------
+struct GroupWs {
+    uint32_t *key, *key_s;            // item keys, then group keys
+    int32_t *iota, *jorder;           // items in the order of their largest neighbour
+    int32_t *work, *prefix;           // per group (locality numbering), max_groups + 1
+    int32_t *gorder, *inv;            // final group order and its inverse
+    uint64_t *ekey, *ekey_s;          // one record per edge slot: (group, neighbour, member), unsorted and sorted
+    uint64_t *mkey_s;                 // sorted (group, mask) keys of the entries (ekey is reused for the unsorted ones)
+    int32_t *eval, *eval_s;           // the slot of a record; later the entry permutation
+    int32_t *rank, *head, *run, *mult, *ebase, *ent_of;   // per record
+    int32_t *ent_idx, *ent_g, *ent_mask, *newpos, *pop, *first;   // per entry
+    void *tmp;
+};
+
+GroupWs group_layout(Bump &b, int64_t max_items, int64_t max_groups, int64_t n_edges, size_t tmp_bytes) {
+    GroupWs w;
+    const int64_t nk = max_items > max_groups ? max_items : max_groups;
+    w.key = b.take<uint32_t>(nk);
+    w.key_s = b.take<uint32_t>(nk);
+    w.iota = b.take<int32_t>(nk > n_edges ? nk : n_edges);
+    w.jorder = b.take<int32_t>(max_items);
+    w.work = b.take<int32_t>(max_groups + 1);
+    w.prefix = b.take<int32_t>(max_groups + 1);
+    w.gorder = b.take<int32_t>(max_groups);
+    w.inv = b.take<int32_t>(max_groups);
+    w.ekey = b.take<uint64_t>(n_edges);
+    w.ekey_s = b.take<uint64_t>(n_edges);
+    w.mkey_s = b.take<uint64_t>(n_edges);
+    w.eval = b.take<int32_t>(n_edges);
+    w.eval_s = b.take<int32_t>(n_edges);
+    w.rank = b.take<int32_t>(n_edges);
+    w.head = b.take<int32_t>(n_edges + 1);
+    w.run = b.take<int32_t>(n_edges + 1);
+    w.mult = b.take<int32_t>(n_edges + 1);
+    w.ebase = b.take<int32_t>(n_edges + 1);
+    w.ent_of = b.take<int32_t>(n_edges);
+    w.ent_idx = b.take<int32_t>(n_edges);
+    w.ent_g = b.take<int32_t>(n_edges);
+    w.ent_mask = b.take<int32_t>(n_edges);
+    w.newpos = b.take<int32_t>(n_edges);
+    w.pop = b.take<int32_t>(n_edges + 1);
+    w.first = b.take<int32_t>(n_edges + 1);
+    w.tmp = b.take<char>((int64_t)tmp_bytes);
+    return w;
+}
+
+__device__ inline bool plan_usable(const int32_t *pinfo) { return pinfo[BPT_PI_ERR] == 0 && (pinfo[BPT_PI_FLAGS] & 1); }
+
+__device__ inline int32_t n_groups_of(const int32_t *pinfo, int32_t R) {
+    return plan_usable(pinfo) ? (pinfo[BPT_PI_N_ITEMS] + R - 1) / R : 0;
+}
+
+__global__ void k_group_work(const int32_t *items, const int32_t *jorder, const int32_t *pinfo, int64_t max_groups, int32_t R,
+                             int32_t *work, int32_t *ginfo) {
+    const int64_t g = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (g > max_groups) return;
+    const int32_t ng = n_groups_of(pinfo, R), n_items = pinfo[BPT_PI_N_ITEMS];
+    if (g == 0) {
+        for (int i = 0; i < 16; ++i) ginfo[i] = 0;
+        ginfo[BPT_GI_N_GROUPS] = ng;
+    }
+    int32_t w = 0;
+    if (g < ng) {
+        w = FIXED_WORK;
+        for (int32_t m = 0; m < R; ++m) {
+            const int64_t j = g * R + m;
+            if (j < n_items) {
+                const int4 it = reinterpret_cast<const int4 *>(items)[jorder[j]];
+                w += it.z - it.y;
+            }
+        }
+    }
+    work[g] = w;
+}
+
+// 8 contiguous ranges of about equal work: chunks[x] = number of groups whose midpoint lies before x/8 of the total
+__global__ void k_chunks(const int32_t *work, const int32_t *prefix, const int32_t *pinfo, int32_t R, int32_t *chunks,
+                         int32_t *ginfo) {
+    __shared__ int32_t sh[9];
+    const int x = threadIdx.x;
+    const int32_t ng = n_groups_of(pinfo, R);
+    if (x <= 8) {
+        int32_t c = (x == 8) ? ng : 0;
+        if (x >= 1 && x <= 7 && ng > 0) {
+            const int64_t total = (int64_t)prefix[ng - 1] + work[ng - 1];
+            const int64_t target = total * x / 8;
+            int32_t lo = 0, hi = ng;                      // first group with prefix + work / 2 >= target
+            while (lo < hi) {
+                const int32_t mid = (lo + hi) >> 1;
+                if ((int64_t)prefix[mid] + work[mid] / 2 < target) lo = mid + 1; else hi = mid;
+            }
+            c = lo;
+        }
+        sh[x] = c;
+        chunks[x] = c;
+    }
+    __syncthreads();
+    if (x == 0) {
+        int32_t mx = 0;
+        for (int i = 0; i < 8; ++i) mx = max(mx, sh[i + 1] - sh[i]);
+        ginfo[BPT_GI_MAX_CHUNK] = mx;
+    }
+}
+
+__global__ void k_group_keys(const int32_t *work, const int32_t *chunks, const int32_t *pinfo, int64_t max_groups, int32_t R,
+                             uint32_t *key) {
+    const int64_t g = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (g >= max_groups) return;
+    if (g >= n_groups_of(pinfo, R)) {
+        key[g] = PAD32;
+        return;
+    }
+    uint32_t c = 0;
+    for (int x = 1; x <= 7; ++x) c += (chunks[x] <= g) ? 1u : 0u;
+    key[g] = (c << 16) | (0xFFFFu - (uint32_t)work[g]);
+}
+
+__global__ void k_invert(const int32_t *order, const int32_t *count, int idx_of_count, int64_t max_n, int32_t *inv) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= max_n || i >= count[idx_of_count]) return;
+    inv[order[i]] = (int32_t)i;
+}
+
+// members of the groups in their final order, and one sort record per edge slot
+__global__ void k_members_and_records(const int32_t *items, const int32_t *idx32, const int32_t *jorder, const int32_t *inv,
+                                      const int32_t *pinfo, int64_t max_groups, int32_t R, int32_t *members, uint64_t *ekey,
+                                      int32_t *eval) {
+    const int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (j >= max_groups * R) return;
+    const int32_t ng = n_groups_of(pinfo, R), n_items = pinfo[BPT_PI_N_ITEMS];
+    const int64_t g0 = j / R;
+    const int32_t m = (int32_t)(j % R);
+    if (g0 >= ng) return;
+    const int32_t gi = inv[g0];
+    int32_t *mem = members + ((int64_t)gi * R + m) * 2;
+    if (j >= n_items) {
+        mem[0] = -1;
+        mem[1] = -1;
+        return;
+    }
+    const int4 it = reinterpret_cast<const int4 *>(items)[jorder[j]];
+    mem[0] = it.x;
+    mem[1] = it.w;
+    for (int32_t p = it.y; p < it.z; ++p) {
+        ekey[p] = ((uint64_t)(uint32_t)gi << 35) | ((uint64_t)(uint32_t)idx32[p] << 4) | (uint64_t)m;
+        eval[p] = p;
+    }
+}
+
+__global__ void k_pad_records(uint64_t *ekey, int32_t *eval, int64_t n_edges, const int32_t *pinfo) {
+    const int64_t p = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (p >= n_edges) return;
+    if (!plan_usable(pinfo)) {
+        ekey[p] = PAD64;
+        eval[p] = (int32_t)p;
+    }
+}
+
+// rank of a record among the equal ones before it (an edge that a member holds several times), and the starts of the
+// runs of equal (group, neighbour)
+__global__ void k_rank(const uint64_t *skey, int64_t n_edges, const int32_t *pinfo, int32_t *rank, int32_t *head) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i > n_edges) return;
+    if (i == n_edges || !plan_usable(pinfo)) {
+        head[i] = 0;
+        if (i < n_edges) rank[i] = 0;
+        return;
+    }
+    const uint64_t k = skey[i];
+    int32_t t = 0;
+    for (int64_t b = i - 1; b >= 0 && skey[b] == k; --b) ++t;
+    rank[i] = t;
+    head[i] = (i == 0 || (skey[i - 1] >> 4) != (k >> 4)) ? 1 : 0;
+}
+
+__global__ void k_multiplicity(const int32_t *rank, const int32_t *head, const int32_t *run_excl, int64_t n_edges,
+                               const int32_t *pinfo, int32_t *run, int32_t *mult) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n_edges || !plan_usable(pinfo)) return;
+    const int32_t r = run_excl[i] + head[i] - 1;
+    run[i] = r;
+    atomicMax(&mult[r], rank[i] + 1);
+}
+
+__global__ void k_entry_fill(const uint64_t *skey, const int32_t *rank, const int32_t *run, const int32_t *ebase,
+                             int64_t n_edges, const int32_t *pinfo, int32_t *ent_of, int32_t *ent_idx, int32_t *ent_g,
+                             int32_t *ent_mask, int32_t *ginfo) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n_edges || !plan_usable(pinfo)) return;
+    if (i == 0) ginfo[BPT_GI_N_ENTRIES] = ebase[n_edges];
+    const uint64_t k = skey[i];
+    const int32_t u = ebase[run[i]] + rank[i];
+    ent_of[i] = u;
+    ent_idx[u] = (int32_t)((k >> 4) & 0x7FFFFFFFu);
+    ent_g[u] = (int32_t)(k >> 35);
+    atomicOr(&ent_mask[u], 1 << (int)(k & 15));
+}
+
+__global__ void k_entry_keys(const int32_t *ent_g, const int32_t *ent_mask, int64_t n_edges, const int32_t *ginfo,
+                             uint64_t *ekey) {
+    const int64_t u = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (u >= n_edges) return;
+    ekey[u] = (u < ginfo[BPT_GI_N_ENTRIES]) ? (((uint64_t)(uint32_t)ent_g[u] << 16) | (uint64_t)(0xFFFF ^ ent_mask[u])) : PAD64;
+}
+
+__global__ void k_popcounts(const int32_t *ent_mask, const int32_t *perm, int64_t n_edges, const int32_t *ginfo, int32_t *pop) {
+    const int64_t u = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (u > n_edges) return;
+    pop[u] = (u < ginfo[BPT_GI_N_ENTRIES]) ? __popc((uint32_t)ent_mask[perm[u]]) : 0;
+}
+
+__global__ void k_entries_out(const int32_t *ent_idx, const int32_t *ent_mask, const int32_t *perm, const int32_t *first,
+                              int64_t n_edges, const int32_t *ginfo, int32_t *entries) {
+    const int64_t u = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    const int32_t ne = ginfo[BPT_GI_N_ENTRIES];
+    if (u > n_edges || u > ne) return;
+    int4 e = make_int4(0, 0, 0, 0);                   // the row behind the last entry is zero
+    if (u < ne) e = make_int4(ent_idx[perm[u]], ent_mask[perm[u]], first[u], 0);
+    reinterpret_cast<int4 *>(entries)[u] = e;
+}
+
+__global__ void k_group_ptr(const int32_t *ent_g, const int32_t *perm, int64_t max_groups, const int32_t *ginfo, int32_t *grp_ptr) {
+    const int64_t g = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    const int32_t ng = ginfo[BPT_GI_N_GROUPS], ne = ginfo[BPT_GI_N_ENTRIES];
+    if (g > max_groups || g > ng) return;
+    int32_t lo = 0, hi = ne;                          // first entry whose group is >= g
+    while (lo < hi) {
+        const int32_t mid = (lo + hi) >> 1;
+        if (ent_g[perm[mid]] < g) lo = mid + 1; else hi = mid;
+    }
+    grp_ptr[g] = lo;
+}
+
+__global__ void k_edge_ids(const uint64_t *skey, const int32_t *slot_of, const int32_t *ent_of, const int32_t *newpos,
+                           const int32_t *ent_mask, const int32_t *first, const int32_t *eid32, int64_t n_edges,
+                           const int32_t *pinfo, int32_t R, int32_t *grp_eids, int32_t *pair_eid) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= n_edges || !plan_usable(pinfo)) return;
+    const int32_t m = (int32_t)(skey[i] & 15), old = ent_of[i], u = newpos[old];
+    const int32_t e = eid32[slot_of[i]];
+    grp_eids[(int64_t)u * R + m] = e;
+    pair_eid[first[u] + __popc((uint32_t)ent_mask[old] & ((1u << m) - 1u))] = e;
+}
+
+// ---- link -----------------------------------------------------------------------------------------------------------------
+__global__ void k_positions(const int32_t *eids_src, const int32_t *ginfo_src, int32_t R_src, int64_t n_edges, int32_t *pos) {
+    const int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (j >= (int64_t)ginfo_src[BPT_GI_N_ENTRIES] * R_src) return;
+    const int32_t e = eids_src[j];
+    if (e >= 0 && e < n_edges) pos[e] = (int32_t)j;
+}
+
+__global__ void k_pairs(const int32_t *eids_dst, const int32_t *ginfo_dst, int32_t R_dst, const int32_t *ginfo_src,
+                        int32_t R_src, int64_t n_edges, int32_t pad, const int32_t *pos, int32_t *pairs) {
+    const int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    const int64_t n_real = (int64_t)ginfo_dst[BPT_GI_N_ENTRIES] * R_dst;
+    if (j >= n_real + (int64_t)pad * R_dst) return;
+    const int32_t spare = (ginfo_src[BPT_GI_N_ENTRIES] + pad) * R_src - 1;
+    int32_t out = spare;
+    if (j < n_real) {
+        const int32_t e = eids_dst[j];
+        if (e >= 0 && e < n_edges) out = pos[e];
+    }
+    pairs[j] = out;
+}
+
+int sizes_ok(int64_t n_units, int64_t n_edges, int64_t n_rows, int64_t n_index_nodes, int32_t seg_len) {
+    if (n_units < 0 || n_edges < 0 || n_rows < 0 || n_index_nodes < 0) return BPT_ERR_SIZE;
+    if (n_rows >= INT32_MAX || n_edges >= INT32_MAX || n_index_nodes >= INT32_MAX || n_units > n_edges + n_rows) return BPT_ERR_SIZE;
+    if (seg_len < 1) return BPT_ERR_SHAPE;
+    return BPT_OK;
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        const hipError_t e_ = (expr);                   \
+        if (e_ != hipSuccess) return (int)e_;           \
+    } while (0)
+
+#define LAUNCH(kernel, n, ...)                                                         \
+    do {                                                                               \
+        if ((n) > 0) {                                                                 \
+            hipLaunchKernelGGL(kernel, dim3(blocks_for(n)), dim3(TPB), 0, s, __VA_ARGS__); \
+            HIP_TRY(hipGetLastError());                                                \
+        }                                                                              \
+    } while (0)
+
+}  // namespace
+
+extern "C" {
+
+int bpt_plan_device_bounds(int64_t n_units, int64_t n_edges, int64_t n_rows, int32_t seg_len, int32_t R, int64_t bounds[4]) {
+    if (!bounds) return BPT_ERR_NULL;
+    const int st = sizes_ok(n_units, n_edges, n_rows, 0, seg_len);
+    if (st != BPT_OK) return st;
+    if (R < 0 || R > 16) return BPT_ERR_SHAPE;
+    const int64_t max_items = n_rows + n_edges / seg_len;
+    const int64_t max_heavy = n_edges / ((int64_t)seg_len + 1);
+    const int64_t max_groups = R > 0 ? (max_items + R - 1) / R : 0;
+    if (max_items >= INT32_MAX || (R > 0 && (n_edges + 8) * R >= INT32_MAX)) return BPT_ERR_SIZE;
+    size_t tmp = 0;
+    HIP_TRY(temp_bytes(max_items, max_groups, n_edges, n_rows, &tmp));
+    Bump a{nullptr, 0}, b{nullptr, 0}, c{nullptr, 0};
+    base_layout(a, n_rows, n_edges, max_items, tmp);
+    group_layout(b, max_items, max_groups, n_edges, tmp);
+    c.take<int32_t>(n_edges);
+    size_t ws = a.off > b.off ? a.off : b.off;
+    ws = ws > c.off ? ws : c.off;
+    bounds[0] = max_items;
+    bounds[1] = max_heavy;
+    bounds[2] = max_groups;
+    bounds[3] = (int64_t)ws + 256;
+    return BPT_OK;
+}
+
+int bpt_plan_build_device(const int64_t *row, const int64_t *indptr_units, int64_t n_units, const int64_t *eid,
+                          const int64_t *indices, int64_t n_edges, int64_t n_rows, int64_t n_index_nodes, int32_t seg_len,
+                          int32_t *rowptr, int32_t *idx32, int32_t *eid32, int32_t *items, int32_t *heavy, int32_t *info,
+                          void *workspace, int64_t workspace_bytes, void *stream) {
+    int64_t bounds[4];
+    const int st = sizes_ok(n_units, n_edges, n_rows, n_index_nodes, seg_len);
+    if (st != BPT_OK) return st;
+    if (!rowptr || !items || !info || !workspace) return BPT_ERR_NULL;
+    if (n_units > 0 && (!row || !indptr_units)) return BPT_ERR_NULL;
+    if (n_edges > 0 && (!eid || !idx32 || !eid32)) return BPT_ERR_NULL;
+    const int bs = bpt_plan_device_bounds(n_units, n_edges, n_rows, seg_len, 0, bounds);
+    if (bs != BPT_OK) return bs;
+    if (bounds[1] > 0 && !heavy) return BPT_ERR_NULL;
+    if (workspace_bytes < bounds[3]) return BPT_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t max_items = bounds[0];
+    size_t tmp = 0;
+    HIP_TRY(temp_bytes(max_items, 0, n_edges, n_rows, &tmp));
+    Bump bump{(char *)workspace, 0};
+    BaseWs w = base_layout(bump, n_rows, n_edges, max_items, tmp);
+
+    hipLaunchKernelGGL(k_base_init, dim3(1), dim3(1), 0, s, info, indptr_units, n_units, n_edges);
+    HIP_TRY(hipGetLastError());
+    LAUNCH(k_check_units, n_units, row, indptr_units, n_units, n_rows, info);
+    LAUNCH(k_fill_i32, n_edges, w.seen, n_edges, 0);
+    LAUNCH(k_narrow, n_edges, eid, indices, n_edges, n_index_nodes, info, idx32, eid32, w.seen);
+    LAUNCH(k_rowptr, n_rows + 1, row, indptr_units, n_units, n_rows, info, rowptr);
+    LAUNCH(k_row_counts, n_rows + 1, rowptr, n_rows, seg_len, info, w.c_items, w.c_heavy, w.c_slots);
+    size_t tb = tmp;
+    HIP_TRY(scan_i32(w.tmp, tb, w.c_items, w.b_items, n_rows + 1, s));
+    tb = tmp;
+    HIP_TRY(scan_i32(w.tmp, tb, w.c_heavy, w.b_heavy, n_rows + 1, s));
+    tb = tmp;
+    HIP_TRY(scan_i32(w.tmp, tb, w.c_slots, w.b_slots, n_rows + 1, s));
+    LAUNCH(k_emit_items, n_rows + 1, rowptr, n_rows, seg_len, w.b_items, w.b_heavy, w.b_slots, info, w.items_tmp, heavy);
+    if (max_items > 0) {
+        // locality order: by smallest neighbour id (without indices the items stay in row order, as on the host)
+        LAUNCH(k_iota_i32, max_items, w.iota, max_items);
+        const int32_t *perm = w.iota;
+        if (indices) {
+            LAUNCH(k_item_keys<false>, max_items, w.items_tmp, idx32, info, max_items, n_index_nodes, w.key);
+            tb = tmp;
+            HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key, w.key_s, w.iota, w.perm, max_items, 32, s));
+            perm = w.perm;
+        }
+        LAUNCH(k_gather_items, max_items, w.items_tmp, perm, info, max_items, items);
+    }
+    return BPT_OK;
+}
+
+int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int32_t *eid32, const int32_t *plan_info,
+                          int64_t max_items, int64_t n_edges, int64_t n_index_nodes, int32_t seg_len, int32_t R,
+                          int32_t by_mask, int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid,
+                          int32_t *grp_eids, int32_t *chunks, int32_t *group_info, void *workspace,
+                          int64_t workspace_bytes, void *stream) {
+    if (max_items < 0 || n_edges < 0 || n_index_nodes < 0 || max_items >= INT32_MAX || n_edges >= INT32_MAX ||
+        n_index_nodes >= INT32_MAX)
+        return BPT_ERR_SIZE;
+    if (R < 1 || R > 16 || seg_len < 1) return BPT_ERR_SHAPE;
+    if ((int64_t)R * seg_len + FIXED_WORK > 0xFFFF) return BPT_ERR_UNSUPPORTED;       // the work of a group is a 16-bit sort key
+    if ((n_edges + 8) * R >= INT32_MAX) return BPT_ERR_SIZE;
+    if (!plan_info || !grp_ptr || !entries || !grp_eids || !chunks || !group_info || !workspace) return BPT_ERR_NULL;
+    if (max_items > 0 && (!items || !members)) return BPT_ERR_NULL;
+    if (n_edges > 0 && (!idx32 || !eid32 || !pair_eid)) return BPT_ERR_NULL;
+    const int64_t max_groups = (max_items + R - 1) / R;
+    if (max_groups >= (int64_t)1 << 28) return BPT_ERR_UNSUPPORTED;                    // group numbers are 28-bit sort keys
+    size_t tmp = 0;
+    HIP_TRY(temp_bytes(max_items, max_groups, n_edges, 0, &tmp));
+    Bump dry{nullptr, 0};
+    group_layout(dry, max_items, max_groups, n_edges, tmp);
+    if (workspace_bytes < (int64_t)dry.off) return BPT_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    Bump bump{(char *)workspace, 0};
+    GroupWs w = group_layout(bump, max_items, max_groups, n_edges, tmp);
+    size_t tb;
+
+    // the items in the order of their largest neighbour; R consecutive ones are a group
+    if (max_items > 0) {
+        LAUNCH(k_item_keys<true>, max_items, items, idx32, plan_info, max_items, n_index_nodes, w.key);
+        LAUNCH(k_iota_i32, max_items, w.iota, max_items);
+        tb = tmp;
+        HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key, w.key_s, w.iota, w.jorder, max_items, 32, s));
+    }
+    LAUNCH(k_group_work, max_groups + 1, items, w.jorder, plan_info, max_groups, R, w.work, group_info);
+    tb = tmp;
+    HIP_TRY(scan_i32(w.tmp, tb, w.work, w.prefix, max_groups + 1, s));
+    hipLaunchKernelGGL(k_chunks, dim3(1), dim3(64), 0, s, w.work, w.prefix, plan_info, R, chunks, group_info);
+    HIP_TRY(hipGetLastError());
+    if (max_groups > 0) {
+        LAUNCH(k_group_keys, max_groups, w.work, chunks, plan_info, max_groups, R, w.key);
+        LAUNCH(k_iota_i32, max_groups, w.iota, max_groups);
+        tb = tmp;
+        HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key, w.key_s, w.iota, w.gorder, max_groups, 32, s));
+        LAUNCH(k_invert, max_groups, w.gorder, group_info, (int)BPT_GI_N_GROUPS, max_groups, w.inv);
+        LAUNCH(k_members_and_records, max_groups * R, items, idx32, w.jorder, w.inv, plan_info, max_groups, R, members,
+               w.ekey, w.eval);
+    }
+    // entries: distinct (group, neighbour, multiplicity) of the records sorted by (group, neighbour, member)
+    LAUNCH(k_fill_i32, (n_edges + 8) * R, grp_eids, (n_edges + 8) * R, (int32_t)n_edges);
+    if (n_edges > 0) {
+        LAUNCH(k_pad_records, n_edges, w.ekey, w.eval, n_edges, plan_info);
+        tb = tmp;
+        HIP_TRY(sort_pairs<uint64_t>(w.tmp, tb, w.ekey, w.ekey_s, w.eval, w.eval_s, n_edges, 35 + bits_for((uint64_t)max_groups), s));
+    }
+    LAUNCH(k_rank, n_edges + 1, w.ekey_s, n_edges, plan_info, w.rank, w.head);
+    tb = tmp;
+    HIP_TRY(scan_i32(w.tmp, tb, w.head, w.run, n_edges + 1, s));       // w.run = exclusive scan for now
+    LAUNCH(k_fill_i32, n_edges + 1, w.mult, n_edges + 1, 0);
+    LAUNCH(k_fill_i32, n_edges, w.ent_mask, n_edges, 0);
+    LAUNCH(k_multiplicity, n_edges, w.rank, w.head, w.run, n_edges, plan_info, w.run, w.mult);
+    tb = tmp;
+    HIP_TRY(scan_i32(w.tmp, tb, w.mult, w.ebase, n_edges + 1, s));
+    LAUNCH(k_entry_fill, n_edges, w.ekey_s, w.rank, w.run, w.ebase, n_edges, plan_info, w.ent_of, w.ent_idx, w.ent_g,
+           w.ent_mask, group_info);
+    // entry order inside a group: neighbour order, or by member mask (larger first, neighbour order inside a mask)
+    int32_t *perm = w.iota;                               // new position -> entry as numbered above
+    LAUNCH(k_iota_i32, n_edges, w.iota, n_edges);
+    if (by_mask && n_edges > 0) {
+        LAUNCH(k_entry_keys, n_edges, w.ent_g, w.ent_mask, n_edges, group_info, w.ekey);
+        tb = tmp;
+        HIP_TRY(sort_pairs<uint64_t>(w.tmp, tb, w.ekey, w.mkey_s, w.iota, w.eval, n_edges, 16 + bits_for((uint64_t)max_groups), s));
+        perm = w.eval;
+    }
+    LAUNCH(k_invert, n_edges, perm, group_info, (int)BPT_GI_N_ENTRIES, n_edges, w.newpos);
+    LAUNCH(k_popcounts, n_edges + 1, w.ent_mask, perm, n_edges, group_info, w.pop);
+    tb = tmp;
+    HIP_TRY(scan_i32(w.tmp, tb, w.pop, w.first, n_edges + 1, s));
+    LAUNCH(k_entries_out, n_edges + 1, w.ent_idx, w.ent_mask, perm, w.first, n_edges, group_info, entries);
+    LAUNCH(k_group_ptr, max_groups + 1, w.ent_g, perm, max_groups, group_info, grp_ptr);
+    LAUNCH(k_edge_ids, n_edges, w.ekey_s, w.eval_s, w.ent_of, w.newpos, w.ent_mask, w.first, eid32, n_edges, plan_info, R, grp_eids,
+           pair_eid);
+    return BPT_OK;
+}
+
+int bpt_plan_link_device(const int32_t *grp_eids_dst, const int32_t *group_info_dst, int32_t R_dst,
+                         const int32_t *grp_eids_src, const int32_t *group_info_src, int32_t R_src, int64_t n_edges,
+                         int32_t pad_entries, int32_t *pairs, void *workspace, int64_t workspace_bytes, void *stream) {
+    if (n_edges < 0 || n_edges >= INT32_MAX || pad_entries < 0) return BPT_ERR_SIZE;
+    if (R_dst < 1 || R_dst > 16 || R_src < 1 || R_src > 16) return BPT_ERR_SHAPE;
+    if (((int64_t)n_edges + pad_entries) * (R_dst > R_src ? R_dst : R_src) >= INT32_MAX) return BPT_ERR_SIZE;
+    if (!grp_eids_dst || !group_info_dst || !grp_eids_src || !group_info_src || !pairs || !workspace) return BPT_ERR_NULL;
+    if (workspace_bytes < (int64_t)((n_edges > 0 ? n_edges : 1) * sizeof(int32_t) + 256)) return BPT_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    Bump bump{(char *)workspace, 0};
+    int32_t *pos = bump.take<int32_t>(n_edges);
+    LAUNCH(k_fill_i32, n_edges, pos, n_edges, 0);
+    LAUNCH(k_positions, n_edges * R_src, grp_eids_src, group_info_src, R_src, n_edges, pos);
+    LAUNCH(k_pairs, (n_edges + pad_entries) * R_dst, grp_eids_dst, group_info_dst, R_dst, group_info_src, R_src, n_edges,
+           pad_entries, pos, pairs);
+    return BPT_OK;
+}
+
+}  // extern "C"

@@ -14,7 +14,7 @@ import threading
 import numpy as np
 import torch
 
-from ._lib import PlanInfo, PlanStruct, check_graph, graph_lib
+from ._lib import PlanInfo, PlanStruct, check_graph, graph_lib, plan_lib
 
 DEFAULT_SEG_LEN = None  # edges per work item: None = chosen per plan by auto_seg_len
 FORCE_SEG_LEN = None    # testing hook: when set, replaces the automatic choice for plans built from now on
@@ -25,6 +25,7 @@ GROUP_ORDER_SRC = 2 + 8  # source-side groups of the fused backward: aligned ent
 GROUP_MAX_PAIRS = None  # cap on the edges of one group: None = 48 per member row, 0 = no cap
 GROUP_PAD_ENTRIES = 8  # the kernels' software pipeline reads per-entry arrays this far past the end
 _CACHE_SIZE = 64
+DEVICE_BUILD = False    # build new plans on the GPU (libbptplan) instead of on the host; see set_device_build
 
 
 def _ptr(a):
@@ -211,6 +212,175 @@ class Plan:
         return hit[0]
 
 
+def set_device_build(on):
+    """Plans of graphs seen from now on are built on the GPU (DevicePlan) or on the host (Plan, the default).
+    Returns the old setting."""
+    global DEVICE_BUILD
+    old, DEVICE_BUILD = DEVICE_BUILD, bool(on)
+    return old
+
+
+_PLAN_ERRORS = {1: "row id, column id or edge id out of range", 2: "row / indptr not sorted", 3: "sizes out of the int32 range"}
+
+
+def _check_plan(status, what):
+    if status != 0:
+        raise RuntimeError(f"{what}: status {status}" + (" (HIP error)" if status > 0 else ""))
+
+
+class _Groups(dict):
+    """Row-group record of a DevicePlan; the host copies ("host") are downloaded when first asked for."""
+
+    def __missing__(self, key):
+        if key != "host":
+            raise KeyError(key)
+        dev, R = self["dev"], self["R"]
+        ne = self["struct"].n_grp_entries
+        eids = dev["eids"][:ne * R].view(ne, R).cpu().numpy()
+        host = {"members": dev["members"].cpu().numpy(), "grp_ptr": dev["grp_ptr"].cpu().numpy(),
+                "entries": dev["entries"][:ne].cpu().numpy(), "pair_eid": dev["pair_eid"].cpu().numpy(),
+                "slot_eid": np.where(eids < self["n_edges"], eids, -1).astype(np.int32),
+                "chunks": dev["chunks"].cpu().numpy(), "R": R}
+        self["host"] = host
+        return host
+
+
+class DevicePlan:
+    """Plan of one CSR side built on the GPU from the reference's int64 device tensors (include/bptplan.h): no copy
+    of the index arrays to the host, only the 16-int size blocks come back.  Same interface as Plan."""
+
+    def __init__(self, row, indptr, eid, indices, n_rows, n_index_nodes, device, seg_len=DEFAULT_SEG_LEN):
+        self.device = torch.device(device)
+        self.n_rows, self.n_edges, self.n_index_nodes = int(n_rows), int(eid.numel()), int(n_index_nodes)
+        self.has_indices = indices is not None
+        if indptr.numel() != row.numel() + 1:
+            raise ValueError("indptr must have len(row) + 1 entries")
+        if indices is not None and indices.numel() != eid.numel():
+            raise ValueError("indices and eid must have the same length")
+        if seg_len is None:
+            seg_len = FORCE_SEG_LEN if FORCE_SEG_LEN is not None else self._auto_seg_len(row, indptr)
+        self.seg_len = int(seg_len)
+        self._groups, self._links, self._lock = {}, {}, threading.Lock()
+        lib = plan_lib()
+        U, E = int(row.numel()), self.n_edges
+        b = (ctypes.c_int64 * 4)()
+        _check_plan(lib.bpt_plan_device_bounds(U, E, self.n_rows, self.seg_len, 0, ctypes.byref(b)), "bpt_plan_device_bounds")
+        self._max_items, max_heavy = int(b[0]), int(b[1])
+        i32 = lambda *shape: torch.empty(shape, dtype=torch.int32, device=self.device)
+        rowptr, idx, eid32 = i32(self.n_rows + 1), i32(max(E, 1)), i32(max(E, 1))
+        items, heavy, info = i32(max(self._max_items, 1), 4), i32(max(max_heavy, 1), 3), i32(16)
+        ws = torch.empty(int(b[3]), dtype=torch.uint8, device=self.device)
+        with torch.cuda.device(self.device):
+            st = lib.bpt_plan_build_device(row.data_ptr() if U else None, indptr.data_ptr() if U else None, U,
+                                           eid.data_ptr() if E else None,
+                                           indices.data_ptr() if (indices is not None and E) else None, E, self.n_rows,
+                                           self.n_index_nodes, self.seg_len, rowptr.data_ptr(), idx.data_ptr(),
+                                           eid32.data_ptr(), items.data_ptr(), heavy.data_ptr(), info.data_ptr(),
+                                           ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+        _check_plan(st, "bpt_plan_build_device")
+        h = info.cpu().tolist()                       # the one synchronisation of the build
+        if h[0] != 0:
+            raise ValueError("bptplan: " + _PLAN_ERRORS.get(h[0], f"error {h[0]}"))
+        self.n_items, self.n_heavy, self.n_slots, self.max_degree = h[1], h[2], h[3], h[4]
+        self.covers_all_edges = bool(h[5] & 1)
+        self._info = info
+        self._dev = {"rowptr": rowptr, "idx": idx, "eid": eid32, "items": items, "heavy": heavy}   # items / heavy: upper-bound sized
+        d = self._dev
+        self.struct = PlanStruct(
+            d["rowptr"].data_ptr(), d["idx"].data_ptr() if E else None, d["eid"].data_ptr() if E else None,
+            d["items"].data_ptr() if self.n_items else None, d["heavy"].data_ptr() if self.n_heavy else None,
+            self.n_rows, E, self.n_items, self.n_heavy, self.n_slots)
+
+    def _auto_seg_len(self, row, indptr):
+        """auto_seg_len on the device: the 90 % quantile of the non-empty rows' degrees."""
+        if row.numel() == 0 or self.n_rows < 8 * 3072:
+            return 64
+        if int(row.min()) < 0 or int(row.max()) >= self.n_rows:
+            return 64                                   # malformed: the validation kernels report it
+        deg = torch.zeros(self.n_rows, dtype=torch.int64, device=row.device).index_add_(0, row, indptr[1:] - indptr[:-1])
+        deg = deg[deg > 0]
+        if deg.numel() == 0:
+            return 64
+        q90 = float(np.quantile(deg.cpu().numpy(), 0.9))
+        return 64 if q90 <= 64 else (128 if q90 <= 128 else 256)
+
+    @property
+    def ref(self):
+        return ctypes.byref(self.struct)
+
+    def ensure_groups(self, R=GROUP_R, order_mode=None):
+        """Row groups of R rows built on the GPU (bpt_plan_group_device).  Of order_mode only the entry order counts:
+        by member mask (+4) or ascending neighbour (the aligned order of the host builder has no parallel form)."""
+        order_mode = GROUP_ORDER if order_mode is None else order_mode
+        by_mask = bool(order_mode & 4) and not (order_mode & 8)
+        with self._lock:
+            hit = self._groups.get((R, by_mask))
+            if hit is None:
+                lib = plan_lib()
+                E = self.n_edges
+                b = (ctypes.c_int64 * 4)()
+                _check_plan(lib.bpt_plan_device_bounds(0, E, self.n_rows, self.seg_len, R, ctypes.byref(b)),
+                            "bpt_plan_device_bounds")
+                max_groups = (self._max_items + R - 1) // R
+                i32 = lambda *shape: torch.empty(shape, dtype=torch.int32, device=self.device)
+                members, grp_ptr, entries = i32(max(max_groups, 1), R, 2), i32(max_groups + 1), i32(E + 1, 4)
+                pair_eid, eids, chunks, ginfo = i32(max(E, 1)), i32((E + GROUP_PAD_ENTRIES) * R), i32(9), i32(16)
+                ws = torch.empty(int(b[3]), dtype=torch.uint8, device=self.device)
+                d = self._dev
+                with torch.cuda.device(self.device):
+                    st = lib.bpt_plan_group_device(d["items"].data_ptr(), d["idx"].data_ptr(), d["eid"].data_ptr(),
+                                                   self._info.data_ptr(), self._max_items, E, self.n_index_nodes,
+                                                   self.seg_len, R, int(by_mask), members.data_ptr(), grp_ptr.data_ptr(),
+                                                   entries.data_ptr(), pair_eid.data_ptr(), eids.data_ptr(),
+                                                   chunks.data_ptr(), ginfo.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                   torch.cuda.current_stream().cuda_stream)
+                _check_plan(st, "bpt_plan_group_device")
+                ng, ne, max_chunk = ginfo.cpu().tolist()[:3]
+                dev = {"members": members[:ng].clone(), "grp_ptr": grp_ptr[:ng + 1].clone(),
+                       "entries": entries[:ne + 1].clone(), "pair_eid": pair_eid[:E].clone(),
+                       "eids": eids[:(ne + GROUP_PAD_ENTRIES) * R].clone(), "chunks": chunks, "ginfo": ginfo}
+                st = PlanStruct.from_buffer_copy(self.struct)
+                st.grp_members = dev["members"].data_ptr() if ng else None
+                st.grp_ptr = dev["grp_ptr"].data_ptr()
+                st.grp_entries = dev["entries"].data_ptr()
+                st.grp_pairs = None
+                st.grp_chunks = dev["chunks"].data_ptr()
+                st.grp_max_chunk = max_chunk
+                st.n_groups = ng
+                st.grp_R = R
+                st.n_grp_entries = ne
+                st.grp_eids = dev["eids"].data_ptr()
+                hit = _Groups(dev=dev, struct=st, R=R, n_edges=E)
+                self._groups[(R, by_mask)] = hit
+        return hit
+
+    def linked_to(self, plan_src, R=GROUP_R):
+        """As Plan.linked_to, with the pair mapping computed on the GPU (bpt_plan_link_device)."""
+        mine, theirs = self.ensure_groups(R), plan_src.ensure_groups(R, GROUP_ORDER_SRC)
+        key = (id(plan_src), R)
+        with self._lock:
+            hit = self._links.get(key)
+            if hit is None:
+                if self.n_edges != plan_src.n_edges or not (self.covers_all_edges and plan_src.covers_all_edges):
+                    raise ValueError("the two plans do not describe the same edge set")
+                E = self.n_edges
+                n_pairs = (mine["struct"].n_grp_entries + GROUP_PAD_ENTRIES) * R
+                pairs = torch.empty((E + GROUP_PAD_ENTRIES) * R, dtype=torch.int32, device=self.device)
+                ws = torch.empty(4 * max(E, 1) + 512, dtype=torch.uint8, device=self.device)
+                with torch.cuda.device(self.device):
+                    st = plan_lib().bpt_plan_link_device(mine["dev"]["eids"].data_ptr(), mine["dev"]["ginfo"].data_ptr(), R,
+                                                         theirs["dev"]["eids"].data_ptr(), theirs["dev"]["ginfo"].data_ptr(), R,
+                                                         E, GROUP_PAD_ENTRIES, pairs.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                         torch.cuda.current_stream().cuda_stream)
+                _check_plan(st, "bpt_plan_link_device")
+                pairs = pairs[:n_pairs].clone()
+                st = PlanStruct.from_buffer_copy(mine["struct"])
+                st.grp_pairs = pairs.data_ptr()
+                hit = (st, pairs, plan_src)
+                self._links[key] = hit
+        return hit[0]
+
+
 class PlanCache:
     def __init__(self, capacity=_CACHE_SIZE):
         self._d = collections.OrderedDict()
@@ -221,7 +391,7 @@ class PlanCache:
     @staticmethod
     def _key(tensors, n_rows, n_index, seg_len):
         return tuple((t.data_ptr(), t.numel(), t._version, str(t.device)) if t is not None else None
-                     for t in tensors) + (n_rows, n_index, seg_len)
+                     for t in tensors) + (n_rows, n_index, seg_len, DEVICE_BUILD)
 
     def get(self, row, indptr, eid, indices, n_rows=None, n_index_nodes=None, seg_len=DEFAULT_SEG_LEN):
         """n_rows None: as many rows as `row` mentions (ops that only produce edge outputs)."""
@@ -234,10 +404,15 @@ class PlanCache:
                 self.hits += 1
                 return hit[0]
         self.misses += 1
-        row_h = _host_i64(row)
-        nr = n_rows if n_rows is not None else (int(row_h[-1]) + 1 if len(row_h) else 0)
-        ni = n_index_nodes if n_index_nodes is not None else nr
-        plan = Plan(row_h, indptr, eid, indices, nr, ni, eid.device, seg_len)
+        if DEVICE_BUILD and eid.is_cuda:
+            nr = n_rows if n_rows is not None else (int(row[-1]) + 1 if row.numel() else 0)
+            ni = n_index_nodes if n_index_nodes is not None else nr
+            plan = DevicePlan(row, indptr, eid, indices, nr, ni, eid.device, seg_len)
+        else:
+            row_h = _host_i64(row)
+            nr = n_rows if n_rows is not None else (int(row_h[-1]) + 1 if len(row_h) else 0)
+            ni = n_index_nodes if n_index_nodes is not None else nr
+            plan = Plan(row_h, indptr, eid, indices, nr, ni, eid.device, seg_len)
         with self._lock:
             self._d[key] = (plan, tensors)          # tensors kept alive with the entry
             while len(self._d) > self._cap:

@@ -1,0 +1,256 @@
+"""Plans built on the GPU (libbptplan): bit for bit against the numpy model of the same construction (and, for the
+base plan, against the host builder), rejection of malformed arrays without a fault, and the attention kernels
+running on such plans against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import parallel_plan_model as model
+from test_gpu_parity import GTOL, TOL, Case, close, f64, rand
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _graphs():
+    from bpt_amd import graphbuilder as gb
+
+    def bpt(L, triu, step):
+        g = gb.BinaryPartition(L, triu, step, 10)
+        src, dst, _ = g.get_edges()
+        return src, dst, g.number_of_nodes
+
+    def multigraph(n=40, E=600, seed=3):
+        rng = np.random.default_rng(seed)
+        src = rng.integers(0, n, E); dst = rng.integers(0, n, E)
+        dst[: E // 3] = 1; src[E // 3: E // 2] = 2
+        src[src == 0] = 3; dst[dst == 0] = 3
+        src[-3:] = src[-4]; dst[-3:] = dst[-4]            # an edge with multiplicity 4
+        return src.astype(np.int64), dst.astype(np.int64), n
+
+    def batch():
+        parts = [bpt(L, True, 4) for L in (171, 99, 260, 64)]
+        shift, srcs, dsts = 0, [], []
+        for s, d, n in parts:
+            srcs.append(s + shift); dsts.append(d + shift); shift += n
+        return np.concatenate(srcs), np.concatenate(dsts), shift
+
+    return {"bpt64c": lambda: bpt(64, True, 4), "bpt37": lambda: bpt(37, False, 2), "bpt300c": lambda: bpt(300, True, 2),
+            "multi": multigraph, "bpt1": lambda: bpt(1, False, 1), "bpt2048c": lambda: bpt(2048, True, 4), "batch": batch}
+
+
+GRAPHS = _graphs()
+_cache = {}
+
+
+def sides(name):
+    """(src, dst, n, csr, host arrays of the in side, of the out side, the same as device tensors)."""
+    if name not in _cache:
+        from bpt_amd import graphbuilder as gb
+        src, dst, n = GRAPHS[name]()
+        csr = gb.get_csrs(src, dst, n, as_torch=False)
+        out_csr, in_csr, ROW, IR, COL, IC = csr
+        a_in, a_out = (COL, IC, in_csr[2], in_csr[1]), (ROW, IR, out_csr[2], out_csr[1])
+        t = lambda arrs: tuple(torch.from_numpy(a).to(DEV) for a in arrs)
+        _cache[name] = (src, dst, n, csr, a_in, a_out, t(a_in), t(a_out))
+    return _cache[name]
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def check_base(dp, arrays, info):
+    d = dp._dev
+    assert (dp.n_items, dp.n_heavy, dp.n_slots, dp.max_degree, dp.covers_all_edges) == \
+           (info["n_items"], info["n_heavy"], info["n_slots"], info["max_degree"], info["perm"])
+    assert np.array_equal(host(d["rowptr"]), arrays["rowptr"])
+    E = len(arrays["eid"])
+    assert np.array_equal(host(d["idx"])[:E], arrays["idx"]) and np.array_equal(host(d["eid"])[:E], arrays["eid"])
+    assert np.array_equal(host(d["items"])[:dp.n_items], arrays["items"])
+    assert np.array_equal(host(d["heavy"])[:dp.n_heavy], arrays["heavy"])
+
+
+def check_groups(hit, grp, n_edges):
+    from bpt_amd.plan import GROUP_PAD_ENTRIES
+    st, dev, R = hit["struct"], hit["dev"], grp["R"]
+    ng, ne = len(grp["members"]), len(grp["entries"])
+    assert (st.n_groups, st.n_grp_entries, st.grp_R) == (ng, ne, R)
+    assert st.grp_max_chunk == (int(np.diff(grp["chunks"]).max()) if ng else 0)
+    assert np.array_equal(host(dev["chunks"]), grp["chunks"])
+    assert np.array_equal(host(dev["members"]), grp["members"])
+    assert np.array_equal(host(dev["grp_ptr"]), grp["grp_ptr"])
+    ent = host(dev["entries"])
+    assert np.array_equal(ent[:ne], grp["entries"]) and np.all(ent[ne] == 0)
+    assert np.array_equal(host(dev["pair_eid"])[:n_edges], grp["pair_eid"])
+    eids = host(dev["eids"])
+    want = np.full((ne + GROUP_PAD_ENTRIES, R), n_edges, dtype=np.int32)
+    want[:ne] = np.where(grp["slot_eid"] >= 0, grp["slot_eid"], n_edges)
+    assert np.array_equal(eids, want.reshape(-1))
+
+
+@pytest.mark.parametrize("seg", [8, 64])
+@pytest.mark.parametrize("name", sorted(GRAPHS))
+def test_device_plan_equals_model_and_host(name, seg):
+    from bpt_amd.plan import GROUP_PAD_ENTRIES, DevicePlan, build_plan_host
+    src, dst, n, csr, a_in, a_out, t_in, t_out = sides(name)
+    plans = []
+    for arrs, tens in ((a_in, t_in), (a_out, t_out)):
+        dp = DevicePlan(*tens, n, n, DEV, seg)
+        arrays, info = model.base_plan(*arrs, n, n, seg)
+        check_base(dp, arrays, info)
+        harr, _ = build_plan_host(*arrs, n, n, seg)
+        assert np.array_equal(host(dp._dev["items"])[:dp.n_items], harr["items"])       # and the host builder's
+        plans.append((dp, arrays))
+    for R in (4, 8, 16):
+        grps = []
+        for (dp, arrays), by_mask in zip(plans, (True, False)):
+            hit = dp.ensure_groups(R, 6 if by_mask else 10)
+            grp = model.group_plan(arrays, n, R, by_mask)
+            check_groups(hit, grp, len(src))
+            grps.append(grp)
+        if R != 16:
+            st = plans[0][0].linked_to(plans[1][0], R)
+            want = model.link_groups(grps[0], grps[1], len(src), GROUP_PAD_ENTRIES)
+            got = host(plans[0][0]._links[(id(plans[1][0]), R)][1])
+            assert np.array_equal(got, want) and st.grp_pairs
+
+
+def test_device_plan_without_indices_and_with_uncovered_slots():
+    """Plans of the ops that take no indices keep the row order; units that leave edge slots out give a plan that
+    is valid for the per-row kernels and has no groups."""
+    from bpt_amd.plan import DevicePlan
+    src, dst, n, csr, a_in, a_out, t_in, t_out = sides("bpt37")
+    dp = DevicePlan(t_in[0], t_in[1], t_in[2], None, n, n, DEV, 8)
+    arrays, info = model.base_plan(a_in[0], a_in[1], a_in[2], None, n, n, 8)
+    rowsorted = arrays["items"][np.argsort(arrays["items"][:, 1], kind="stable")]       # the model always sorts by locality
+    assert np.array_equal(host(dp._dev["items"])[:dp.n_items][:, :3], rowsorted[:, :3])
+    # drop the last unit: the slots it covered belong to no row any more
+    row, ip = a_in[0][:-1], a_in[1][:-1]
+    dp = DevicePlan(torch.from_numpy(row).to(DEV), torch.from_numpy(ip).to(DEV), t_in[2], t_in[3], n, n, DEV, 8)
+    arrays, info = model.base_plan(row, ip, a_in[2], a_in[3], n, n, 8)
+    assert not dp.covers_all_edges and not info["perm"]
+    check_base(dp, arrays, info)
+    assert dp.ensure_groups(4)["struct"].n_groups == 0
+
+
+def test_device_plan_rejects_malformed_arrays():
+    from bpt_amd.plan import DevicePlan
+    src, dst, n, csr, a_in, a_out, t_in, t_out = sides("bpt64c")
+    row, ip, eid, idx = (t.clone() for t in t_in)
+    bad = idx.clone(); bad[5] = n
+    with pytest.raises(ValueError, match="out of range"):
+        DevicePlan(row, ip, eid, bad, n, n, DEV, 64)
+    bad = idx.clone(); bad[7] = -1
+    with pytest.raises(ValueError, match="out of range"):
+        DevicePlan(row, ip, eid, bad, n, n, DEV, 64)
+    bad = eid.clone(); bad[0] = len(eid)
+    with pytest.raises(ValueError, match="out of range"):
+        DevicePlan(row, ip, bad, idx, n, n, DEV, 64)
+    bad = row.clone(); bad[3], bad[4] = row[4] + 1, row[3]
+    with pytest.raises(ValueError, match="not sorted"):
+        DevicePlan(bad, ip, eid, idx, n, n, DEV, 64)
+    bad = ip.clone(); bad[2] = bad[3] + 1
+    with pytest.raises(ValueError, match="not sorted"):
+        DevicePlan(row, bad, eid, idx, n, n, DEV, 64)
+    bad = row.clone(); bad[-1] = n
+    with pytest.raises(ValueError, match="out of range"):
+        DevicePlan(bad, ip, eid, idx, n, n, DEV, 64)
+    # a repeated edge id is no error, but such a plan gets no groups (as on the host)
+    dup = eid.clone(); dup[1] = dup[0]
+    dp = DevicePlan(row, ip, dup, idx, n, n, DEV, 64)
+    assert not dp.covers_all_edges and dp.ensure_groups(4)["struct"].n_groups == 0
+    torch.cuda.synchronize()
+
+
+@pytest.fixture
+def device_plans():
+    from bpt_amd import plan
+    plan.plan_cache.clear()
+    old = plan.set_device_build(True)
+    yield plan
+    plan.set_device_build(old)
+    plan.plan_cache.clear()
+
+
+@pytest.mark.parametrize("R", [4, 8])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("gname", ["bpt512_k4", "bpt300_causal_k2", "multigraph", "fc_w100"])
+def test_fused_attention_on_device_plans_matches_oracle(device_plans, gname, dtype, R):
+    from bpt_amd import graphop
+    c = Case(gname)
+    h, d = 8, 64
+    q, k, v, do = (rand((c.n, h, d), dtype, s, 0.125 if s < 3 else 1.0) for s in range(4))
+    old = graphop.set_group_rows(R)
+    try:
+        qd, kd, vd, dod = (x.to(DEV) for x in (q, k, v, do))
+        o, lse = graphop.attention_forward(*c.inn, qd, kd, vd)
+        dq, dk, dv = graphop.attention_backward(*c.out, *c.inn, qd, kd, vd, o, lse, dod)
+        torch.cuda.synchronize()
+        assert isinstance(device_plans.plan_cache.get(*c.inn, c.n, c.n), device_plans.DevicePlan)
+    finally:
+        graphop.set_group_rows(old)
+    ro, ra = oracle.attention_forward(c.csr, f64(q), f64(k), f64(v))
+    rdq, rdk, rdv = oracle.attention_backward(c.csr, f64(q), f64(k), f64(v), ra, f64(do))
+    close(o, ro, TOL[dtype], "o")
+    for got, want, nm in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv")):
+        close(got, want, GTOL[dtype], nm, terms=c.max_deg)
+
+
+def test_ops_and_rel_pos_on_device_plans_match_host_plans(device_plans):
+    """The unfused ops and the fused path with rel_pos and dropout give the same results on device-built plans as on
+    host-built ones (the ops bit for bit: their base plans are identical)."""
+    from bpt_amd import graphop, op, plan
+    c = Case("bpt512_k4")
+    h, d = 8, 64
+    q, k, v = (rand((c.n, h, d), torch.float32, s, 0.125).to(DEV) for s in range(3))
+    table = rand((30, d), torch.float32, 7, 0.125).to(DEV)
+    etype = torch.from_numpy(np.random.default_rng(0).integers(0, 30, c.E)).to(DEV)
+
+    def run():
+        e = graphop.maskedmm_csr_forward(*c.out, k, q)
+        a = graphop.sparse_softmax_forward(*c.inn[:3], e)
+        y = graphop.vector_spmm_forward(*c.inn, a, v)
+        qq, kk, vv, tt = (x.clone().requires_grad_(True) for x in (q, k, v, table))
+        o = op.bpt_attention(*c.out, *c.inn, qq, kk, vv, rel_table=tt, etype=etype)
+        o.sum().backward()
+        torch.cuda.synchronize()
+        return e, a, y, o.detach(), qq.grad, kk.grad, vv.grad, tt.grad
+
+    dev = run()
+    assert isinstance(plan.plan_cache.get(*c.inn, c.n, c.n), plan.DevicePlan)
+    plan.set_device_build(False)
+    plan.plan_cache.clear()
+    hst = run()
+    assert isinstance(plan.plan_cache.get(*c.inn, c.n, c.n), plan.Plan)
+    for i in range(3):
+        assert torch.equal(dev[i], hst[i])
+    for got, want in zip(dev[3:], hst[3:]):
+        assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
+
+
+def test_device_plan_at_headline_size_and_its_build_time():
+    """cfg 3 (L = 8192, k = 4, causal): the device-built plans equal the model, and the kernels accept them."""
+    import time
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd.plan import DevicePlan
+    g = gb.BinaryPartition(8192, True, 4, 10)
+    src, dst, _ = g.get_edges()
+    n = g.number_of_nodes
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, n, as_torch=False)
+    a_in, a_out = (COL, IC, in_csr[2], in_csr[1]), (ROW, IR, out_csr[2], out_csr[1])
+    t_in, t_out = (tuple(torch.from_numpy(a).to(DEV) for a in arrs) for arrs in (a_in, a_out))
+    for rep in range(2):                                   # the second pass is warm
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        pin, pout = DevicePlan(*t_in, n, n, DEV), DevicePlan(*t_out, n, n, DEV)
+        pin.linked_to(pout, 8)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    print(f"device plan build (both sides, groups of 8, pair mapping) at cfg 3: {dt * 1e3:.2f} ms")
+    for dp, arrs, by_mask in ((pin, a_in, True), (pout, a_out, False)):
+        arrays, info = model.base_plan(*arrs, n, n, 64)
+        check_base(dp, arrays, info)
+        check_groups(dp.ensure_groups(8, 6 if by_mask else 10), model.group_plan(arrays, n, 8, by_mask), len(src))

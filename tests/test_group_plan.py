@@ -36,6 +36,46 @@ def plans(name, seg=64):
     return src, dst, n, csr, pin, pout
 
 
+def check_group_invariants(arrays, grp, rows_of, cols_of, E, GROUP_R, masks_sorted):
+    members, gptr, entries, pair_eid = grp["members"], grp["grp_ptr"], grp["entries"], grp["pair_eid"]
+    ch = grp["chunks"]
+    assert ch[0] == 0 and ch[8] == len(members) and np.all(np.diff(ch) >= 0)
+    items = arrays["items"]
+    ng = len(members)
+    assert members.shape == (ng, GROUP_R, 2) and len(gptr) == ng + 1
+    assert gptr[0] == 0 and gptr[-1] == len(entries) and np.all(np.diff(gptr) >= 0)
+    # every item is a member of exactly one group
+    used = [(r, s) for r, s in members.reshape(-1, 2).tolist() if r >= 0]
+    assert sorted(used) == sorted((r, s) for r, _, _, s in items.tolist())
+    assert np.all(members[:, 0, 0] >= 0)                      # no empty group
+    # every edge is exactly one pair
+    assert sorted(pair_eid.tolist()) == list(range(E))
+    # entries: masks valid, pairs numbered consecutively, every pair is an edge (entry idx -> member row)
+    seg_of = {(r, s): (b, e) for r, b, e, s in items.tolist()}
+    eid_slot = {int(e): p for p, e in enumerate(arrays["eid"].tolist())}
+    slot_eid = grp["slot_eid"]
+    assert slot_eid.shape == (len(entries), GROUP_R)
+    n_pairs = 0
+    for g in range(ng):
+        masks = entries[gptr[g]:gptr[g + 1], 1]
+        if masks_sorted:
+            assert np.all(np.diff(masks) <= 0)                # equal masks adjacent, larger first
+        for u in range(gptr[g], gptr[g + 1]):
+            idx, mask, pb, _ = entries[u].tolist()
+            assert 0 < mask < (1 << GROUP_R) and pb == n_pairs
+            for m in range(GROUP_R):
+                if not mask >> m & 1:
+                    assert slot_eid[u, m] == -1
+                else:
+                    row, slot = members[g, m].tolist()
+                    e = int(pair_eid[n_pairs]); n_pairs += 1
+                    assert slot_eid[u, m] == e
+                    assert rows_of[e] == row and cols_of[e] == idx
+                    b, en = seg_of[(row, slot)]
+                    assert b <= eid_slot[e] < en              # the edge lies in this member's segment
+    assert n_pairs == E
+
+
 @pytest.mark.parametrize("GROUP_R", [4, 16])
 @pytest.mark.parametrize("order_mode", [0, 1, 2, 6, 10])
 @pytest.mark.parametrize("seg", [8, 64])
@@ -45,43 +85,7 @@ def test_group_plan_invariants(name, seg, order_mode, GROUP_R):
     E = len(src)
     for arrays, rows_of, cols_of in ((pin, dst, src), (pout, src, dst)):
         grp = build_groups_host(arrays, n, R=GROUP_R, order_mode=order_mode)
-        members, gptr, entries, pair_eid = grp["members"], grp["grp_ptr"], grp["entries"], grp["pair_eid"]
-        ch = grp["chunks"]
-        assert ch[0] == 0 and ch[8] == len(members) and np.all(np.diff(ch) >= 0)
-        items = arrays["items"]
-        ng = len(members)
-        assert members.shape == (ng, GROUP_R, 2) and len(gptr) == ng + 1
-        assert gptr[0] == 0 and gptr[-1] == len(entries) and np.all(np.diff(gptr) >= 0)
-        # every item is a member of exactly one group
-        used = [(r, s) for r, s in members.reshape(-1, 2).tolist() if r >= 0]
-        assert sorted(used) == sorted((r, s) for r, _, _, s in items.tolist())
-        assert np.all(members[:, 0, 0] >= 0)                      # no empty group
-        # every edge is exactly one pair
-        assert sorted(pair_eid.tolist()) == list(range(E))
-        # entries: masks valid, pairs numbered consecutively, every pair is an edge (entry idx -> member row)
-        seg_of = {(r, s): (b, e) for r, b, e, s in items.tolist()}
-        eid_slot = {int(e): p for p, e in enumerate(arrays["eid"].tolist())}
-        slot_eid = grp["slot_eid"]
-        assert slot_eid.shape == (len(entries), GROUP_R)
-        n_pairs = 0
-        for g in range(ng):
-            masks = entries[gptr[g]:gptr[g + 1], 1]
-            if order_mode & 4 and not order_mode & 8:
-                assert np.all(np.diff(masks) <= 0)                # equal masks adjacent, larger first
-            for u in range(gptr[g], gptr[g + 1]):
-                idx, mask, pb, _ = entries[u].tolist()
-                assert 0 < mask < (1 << GROUP_R) and pb == n_pairs
-                for m in range(GROUP_R):
-                    if not mask >> m & 1:
-                        assert slot_eid[u, m] == -1
-                    else:
-                        row, slot = members[g, m].tolist()
-                        e = int(pair_eid[n_pairs]); n_pairs += 1
-                        assert slot_eid[u, m] == e
-                        assert rows_of[e] == row and cols_of[e] == idx
-                        b, en = seg_of[(row, slot)]
-                        assert b <= eid_slot[e] < en              # the edge lies in this member's segment
-        assert n_pairs == E
+        check_group_invariants(arrays, grp, rows_of, cols_of, E, GROUP_R, bool(order_mode & 4 and not order_mode & 8))
 
 
 def emulate_forward(arrays, grp, q, k, v, scale):
@@ -89,6 +93,7 @@ def emulate_forward(arrays, grp, q, k, v, scale):
     n, h, d = q.shape
     o = np.zeros_like(q); lse = np.zeros((n, h))
     part = {}
+    GROUP_R = grp["R"]
     for g in range(len(grp["members"])):
         st = [dict(m=np.full(h, -np.inf), l=np.zeros(h), acc=np.zeros((h, d))) for _ in range(GROUP_R)]
         for u in range(grp["grp_ptr"][g], grp["grp_ptr"][g + 1]):
@@ -119,19 +124,17 @@ def emulate_forward(arrays, grp, q, k, v, scale):
     return o
 
 
-@pytest.mark.parametrize("name,seg", [("bpt64c", 64), ("bpt37", 8), ("multi", 8), ("bpt300c", 64)])
-def test_emulated_group_walk_matches_oracle(name, seg):
-    src, dst, n, csr, pin, pout = plans(name, seg)
+def check_emulated_walks(src, dst, n, csr, pin, gin, gout, xpos):
+    """Forward walk over the destination-side groups, backward walks over both sides, against the oracle."""
+    GROUP_R = gin["R"]
+    assert gout["R"] == GROUP_R
     rng = np.random.default_rng(0)
     h, d = 2, 8
     q, k, v, do = (rng.standard_normal((n, h, d)) / 2 for _ in range(4))
     ro, ra = oracle.attention_forward(csr, q, k, v)
-    gin = build_groups_host(pin, n)
     o = emulate_forward(pin, gin, q, k, v, 1 / np.sqrt(d))
     assert np.allclose(o, ro, rtol=1e-10, atol=1e-12)
     # backward walk: destination side writes (p, ds) at the source side's pair numbers, source side reads them in order
-    gout = build_groups_host(pout, n)
-    xpos = link_groups_host(gin, gout, len(src))
     spare = (len(gout["entries"]) + GROUP_PAD_ENTRIES) * GROUP_R - 1
     assert len(xpos) == (len(gin["entries"]) + GROUP_PAD_ENTRIES) * GROUP_R and np.all(xpos[len(gin["entries"]) * GROUP_R:] == spare)
     assert np.all(xpos[:len(gin["entries"]) * GROUP_R][gin["slot_eid"].reshape(-1) < 0] == spare)
@@ -170,6 +173,13 @@ def test_emulated_group_walk_matches_oracle(name, seg):
                     dk[row] += pds[u * GROUP_R + m, :, 1][:, None] * q[idx]
                     dv[row] += pds[u * GROUP_R + m, :, 0][:, None] * do[idx]
     assert np.allclose(dk, rdk, rtol=1e-9, atol=1e-12) and np.allclose(dv, rdv, rtol=1e-9, atol=1e-12)
+
+
+@pytest.mark.parametrize("name,seg", [("bpt64c", 64), ("bpt37", 8), ("multi", 8), ("bpt300c", 64)])
+def test_emulated_group_walk_matches_oracle(name, seg):
+    src, dst, n, csr, pin, pout = plans(name, seg)
+    gin, gout = build_groups_host(pin, n), build_groups_host(pout, n)
+    check_emulated_walks(src, dst, n, csr, pin, gin, gout, link_groups_host(gin, gout, len(src)))
 
 
 def test_grouping_reduces_row_loads_on_the_headline_graph():

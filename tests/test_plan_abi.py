@@ -1,4 +1,4 @@
-"""Host logic of the launch plan, and that both shared libraries load and export every symbol
+"""Host logic of the launch plan, and that the shared libraries load and export every symbol
 their headers declare (no GPU needed, no compute calls)."""
 import ctypes
 import os
@@ -30,8 +30,13 @@ def test_libraries_export_every_declared_symbol():
         assert hasattr(glib, name), name
     for name in a:
         assert hasattr(alib, name), name
+    p = _declared("bptplan.h", "bpt_plan_")
+    assert len(p) == 4
+    plib = _lib.plan_lib()
+    for name in p:
+        assert hasattr(plib, name), name
     # the Python bindings cover exactly the declared API
-    assert sorted(_lib.GRAPH_API) == g and sorted(_lib.ATTN_API) == a
+    assert sorted(_lib.GRAPH_API) == g and sorted(_lib.ATTN_API) == a and sorted(_lib.PLAN_API) == p
 
 
 def test_error_strings_and_argument_errors_without_gpu():
@@ -46,6 +51,12 @@ def test_error_strings_and_argument_errors_without_gpu():
     assert alib.bpt_sparse_softmax_forward(ctypes.byref(plan_bad), None, None, None, 0, 8, 0, None) == -2
     assert alib.bpt_workspace_bytes(5, ctypes.byref(plan), None, 8, 64, 0) == 0
     assert _lib.graph_lib().bptg_strerror(-4).startswith(b"row id")
+    plib = _lib.plan_lib()
+    assert plib.bpt_plan_device_bounds(0, -1, 0, 64, 0, ctypes.byref((ctypes.c_int64 * 4)())) == -2            # size
+    assert plib.bpt_plan_device_bounds(0, 0, 0, 64, 0, None) == -1
+    assert plib.bpt_plan_group_device(None, None, None, None, 0, 0, 0, 64, 17, 0, None, None, None, None, None, None, None,
+                                      None, 0, None) == -4                                                    # R
+    assert plib.bpt_plan_link_device(None, None, 4, None, None, 4, 10, 8, None, None, 0, None) == -1
 
 
 def _bpt_csr(L, triu, step):
