@@ -107,6 +107,8 @@ def main():
     ap.add_argument("--dropout", type=float, default=0.0, help="dropout on the attention probabilities inside the fused kernels (attention.py:73)")
     ap.add_argument("--rel-pos", action="store_true",
                     help="add the relative-position score term q[dst].table[etype[e]] (table (1000, d_head), modules/attention.py:23,42,69-71)")
+    ap.add_argument("--device-plan", action="store_true",
+                    help="build the launch plans and row groups on the GPU (libbptplan) instead of on the host")
     ap.add_argument("--block-layers", type=int, default=0,
                     help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the workload's graph")
     args = ap.parse_args()
@@ -123,6 +125,8 @@ def main():
     dev = "cuda:0"
     graphop.set_row_groups(not args.rows)
     graphop.set_group_rows(args.group_rows)
+    from bpt_amd import plan as plan_mod
+    plan_mod.set_device_build(args.device_plan)
     desc, graphs, H, D, default_dtype = make_workload(args.workload)
     dtype_name = args.dtype or default_dtype
     tdtype = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
@@ -179,6 +183,26 @@ def main():
 
     ref = step()                                   # builds + caches the plans
     torch.cuda.synchronize()
+
+    # what a new graph costs before its first step: plans of both CSR sides, the row groups both passes use and the
+    # pair mapping, from the int64 device tensors the ops receive (warm: the libraries are loaded)
+    plan_build = None
+    if not args.rows and not args.unfused and not args.rel_pos:
+        ts = []
+        for _ in range(3):
+            plan_mod.plan_cache.clear()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            pin = plan_mod.plan_cache.get(*gargs[4:], N, N)
+            pout = plan_mod.plan_cache.get(*gargs[:4], N, N)
+            pin.ensure_groups(graphop._forward_rows(q, H, D, pin, args.dropout))
+            pin.linked_to(pout, graphop._group_rows(q, H, D, pin))
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        plan_build = {"where": "device" if args.device_plan else "host", "ms": round(min(ts) * 1e3, 3)}
+        log(f"plan build: {plan_build}")
+        ref = step()
+        torch.cuda.synchronize()
 
     def timed(fn, steps, warmup):
         for _ in range(warmup):
@@ -298,6 +322,8 @@ def main():
         "ms_per_step_graph": None if t_graph_replay is None else t_graph_replay * 1e3,
         "kernel_ms": {k_: round(v_, 5) for k_, v_ in kernels.items()},
     }
+    if plan_build is not None:
+        out["plan_build"] = plan_build
     if block is not None:
         out["block_stack"] = block
     log(json.dumps(out, indent=1))

@@ -242,8 +242,10 @@ __global__ void k_gather_items(const int32_t *items_tmp, const int32_t *perm, co
 struct GroupWs {
     uint32_t *key, *key_s;            // item keys, then group keys
     int32_t *iota, *jorder;           // items in the order of their largest neighbour
-    int32_t *work, *prefix;           // per group (locality numbering), max_groups + 1
-    int32_t *gorder, *inv;            // final group order and its inverse
+    int32_t *work0;                   // per group as formed
+    int32_t *lorder, *lpos;           // locality numbering of the groups (by smallest neighbour) and its inverse
+    int32_t *work, *prefix;           // per group in locality numbering, max_groups + 1
+    int32_t *gorder, *inv;            // final group order (positions in locality numbering) and its inverse
     uint64_t *ekey, *ekey_s;          // one record per edge slot: (group, neighbour, member), unsorted and sorted
     uint64_t *mkey_s;                 // sorted (group, mask) keys of the entries (ekey is reused for the unsorted ones)
     int32_t *eval, *eval_s;           // the slot of a record; later the entry permutation
@@ -259,6 +261,9 @@ GroupWs group_layout(Bump &b, int64_t max_items, int64_t max_groups, int64_t n_e
     w.key_s = b.take<uint32_t>(nk);
     w.iota = b.take<int32_t>(nk > n_edges ? nk : n_edges);
     w.jorder = b.take<int32_t>(max_items);
+    w.work0 = b.take<int32_t>(max_groups + 1);
+    w.lorder = b.take<int32_t>(max_groups);
+    w.lpos = b.take<int32_t>(max_groups);
     w.work = b.take<int32_t>(max_groups + 1);
     w.prefix = b.take<int32_t>(max_groups + 1);
     w.gorder = b.take<int32_t>(max_groups);
@@ -290,8 +295,10 @@ __device__ inline int32_t n_groups_of(const int32_t *pinfo, int32_t R) {
     return plan_usable(pinfo) ? (pinfo[BPT_PI_N_ITEMS] + R - 1) / R : 0;
 }
 
-__global__ void k_group_work(const int32_t *items, const int32_t *jorder, const int32_t *pinfo, int64_t max_groups, int32_t R,
-                             int32_t *work, int32_t *ginfo) {
+// work of every group as formed (its pairs plus a fixed cost) and its locality key: the smallest neighbour id any
+// member reads
+__global__ void k_group_work(const int32_t *items, const int32_t *jorder, const uint32_t *kmin, const int32_t *pinfo,
+                             int64_t max_groups, int32_t R, int32_t *work0, uint32_t *lkey, int32_t *ginfo) {
     const int64_t g = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (g > max_groups) return;
     const int32_t ng = n_groups_of(pinfo, R), n_items = pinfo[BPT_PI_N_ITEMS];
@@ -300,17 +307,27 @@ __global__ void k_group_work(const int32_t *items, const int32_t *jorder, const 
         ginfo[BPT_GI_N_GROUPS] = ng;
     }
     int32_t w = 0;
+    uint32_t key = PAD32;
     if (g < ng) {
         w = FIXED_WORK;
         for (int32_t m = 0; m < R; ++m) {
             const int64_t j = g * R + m;
             if (j < n_items) {
-                const int4 it = reinterpret_cast<const int4 *>(items)[jorder[j]];
+                const int32_t item = jorder[j];
+                const int4 it = reinterpret_cast<const int4 *>(items)[item];
                 w += it.z - it.y;
+                key = min(key, kmin[item]);
             }
         }
     }
-    work[g] = w;
+    work0[g] = w;
+    if (g < max_groups) lkey[g] = key;
+}
+
+__global__ void k_gather_work(const int32_t *work0, const int32_t *lorder, const int32_t *ginfo, int64_t max_groups, int32_t *work) {
+    const int64_t l = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (l > max_groups) return;
+    work[l] = (l < ginfo[BPT_GI_N_GROUPS]) ? work0[lorder[l]] : 0;
 }
 
 // 8 contiguous ranges of about equal work: chunks[x] = number of groups whose midpoint lies before x/8 of the total
@@ -362,8 +379,8 @@ __global__ void k_invert(const int32_t *order, const int32_t *count, int idx_of_
 }
 
 // members of the groups in their final order, and one sort record per edge slot
-__global__ void k_members_and_records(const int32_t *items, const int32_t *idx32, const int32_t *jorder, const int32_t *inv,
-                                      const int32_t *pinfo, int64_t max_groups, int32_t R, int32_t *members, uint64_t *ekey,
+__global__ void k_members_and_records(const int32_t *items, const int32_t *idx32, const int32_t *jorder, const int32_t *lpos,
+                                      const int32_t *inv, const int32_t *pinfo, int64_t max_groups, int32_t R, int32_t *members, uint64_t *ekey,
                                       int32_t *eval) {
     const int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (j >= max_groups * R) return;
@@ -371,7 +388,7 @@ __global__ void k_members_and_records(const int32_t *items, const int32_t *idx32
     const int64_t g0 = j / R;
     const int32_t m = (int32_t)(j % R);
     if (g0 >= ng) return;
-    const int32_t gi = inv[g0];
+    const int32_t gi = inv[lpos[g0]];
     int32_t *mem = members + ((int64_t)gi * R + m) * 2;
     if (j >= n_items) {
         mem[0] = -1;
@@ -636,18 +653,27 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
         tb = tmp;
         HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key, w.key_s, w.iota, w.jorder, max_items, 32, s));
     }
-    LAUNCH(k_group_work, max_groups + 1, items, w.jorder, plan_info, max_groups, R, w.work, group_info);
+    // the groups numbered by locality (smallest neighbour id), cut into 8 ranges of equal work, by decreasing work
+    // inside a range
+    if (max_items > 0) LAUNCH(k_item_keys<false>, max_items, items, idx32, plan_info, max_items, n_index_nodes, w.key);
+    LAUNCH(k_group_work, max_groups + 1, items, w.jorder, w.key, plan_info, max_groups, R, w.work0, w.key_s, group_info);
+    if (max_groups > 0) {
+        LAUNCH(k_iota_i32, max_groups, w.iota, max_groups);
+        tb = tmp;
+        HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key_s, w.key, w.iota, w.lorder, max_groups, 32, s));
+        LAUNCH(k_invert, max_groups, w.lorder, group_info, (int)BPT_GI_N_GROUPS, max_groups, w.lpos);
+    }
+    LAUNCH(k_gather_work, max_groups + 1, w.work0, w.lorder, group_info, max_groups, w.work);
     tb = tmp;
     HIP_TRY(scan_i32(w.tmp, tb, w.work, w.prefix, max_groups + 1, s));
     hipLaunchKernelGGL(k_chunks, dim3(1), dim3(64), 0, s, w.work, w.prefix, plan_info, R, chunks, group_info);
     HIP_TRY(hipGetLastError());
     if (max_groups > 0) {
-        LAUNCH(k_group_keys, max_groups, w.work, chunks, plan_info, max_groups, R, w.key);
-        LAUNCH(k_iota_i32, max_groups, w.iota, max_groups);
+        LAUNCH(k_group_keys, max_groups, w.work, chunks, plan_info, max_groups, R, w.key_s);
         tb = tmp;
-        HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key, w.key_s, w.iota, w.gorder, max_groups, 32, s));
+        HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key_s, w.key, w.iota, w.gorder, max_groups, 32, s));
         LAUNCH(k_invert, max_groups, w.gorder, group_info, (int)BPT_GI_N_GROUPS, max_groups, w.inv);
-        LAUNCH(k_members_and_records, max_groups * R, items, idx32, w.jorder, w.inv, plan_info, max_groups, R, members,
+        LAUNCH(k_members_and_records, max_groups * R, items, idx32, w.jorder, w.lpos, w.inv, plan_info, max_groups, R, members,
                w.ekey, w.eval);
     }
     // entries: distinct (group, neighbour, multiplicity) of the records sorted by (group, neighbour, member)

@@ -47,9 +47,11 @@ int bpt_plan_build_device(const int64_t *row, const int64_t *indptr_units, int64
                           int32_t *heavy, int32_t *info, void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Row groups of R rows over a base plan (the arrays bpt_plan's grp_* fields point at).  The items are taken in
- * the order of their largest neighbour id, R consecutive ones form a group; the groups are cut into 8 ranges of
- * equal work (one per XCD) and ordered by decreasing work inside a range; the entries of a group (its distinct
- * neighbours) are in ascending neighbour order, or with by_mask != 0 sorted by member mask (larger first).
+ * the order of their largest neighbour id, R consecutive ones form a group; the groups are numbered by the smallest
+ * neighbour id any member reads (groups that read the same rows end up on the same XCD at about the same time), cut
+ * into 8 ranges of equal work (one per XCD) and ordered by decreasing work inside a range; the entries of a group
+ * (its distinct neighbours) are in ascending neighbour order, or with by_mask != 0 sorted by member mask (larger
+ * first).
  * plan_info is the info block bpt_plan_build_device wrote (device memory; groups are only built when its flags
  * say that the plan covers every edge, else n_groups = 0).  max_items = bounds[0].
  *   members   (bounds[2], R, 2)    grp_ptr (bounds[2] + 1)      entries (n_edges + 1, 4)

@@ -60,16 +60,25 @@ def item_keys(items, idx32, n_index, red):
 
 
 def group_plan(arrays, n_index, R, by_mask):
-    """Row groups: the items in the order of their largest neighbour, R consecutive ones per group."""
+    """Row groups: the items in the order of their largest neighbour, R consecutive ones per group; the groups
+    numbered by locality (smallest neighbour), cut into 8 ranges of equal work, by decreasing work inside a range."""
     items, idx32, eid32 = arrays["items"], arrays["idx"], arrays["eid"]
     n_items, E = len(items), len(eid32)
     kmax = item_keys(items, idx32, n_index, np.max)
     jorder = np.argsort(kmax, kind="stable")
     ng = -(-n_items // R)
     lens = (items[:, 2] - items[:, 1]).astype(np.int64)
-    w = np.zeros(ng, dtype=np.int64)
-    np.add.at(w, np.arange(n_items) // R, lens[jorder])
-    w += FIXED_WORK
+    w0 = np.zeros(ng, dtype=np.int64)
+    np.add.at(w0, np.arange(n_items) // R, lens[jorder])
+    w0 += FIXED_WORK
+    # locality numbering of the groups: by the smallest neighbour id any member reads
+    kmin = item_keys(items, idx32, n_index, np.min)
+    gk = np.full(ng, np.iinfo(np.int64).max, dtype=np.int64)
+    np.minimum.at(gk, np.arange(n_items) // R, kmin[jorder])
+    lorder = np.argsort(gk, kind="stable")
+    lpos = np.empty(ng, dtype=np.int64)
+    lpos[lorder] = np.arange(ng)
+    w = w0[lorder]
     prefix, total = _excl(w)[:-1], int(w.sum())
     chunks = np.zeros(9, dtype=np.int32)
     for x in range(1, 8):
@@ -80,7 +89,7 @@ def group_plan(arrays, n_index, R, by_mask):
     inv = np.empty(ng, dtype=np.int64)
     inv[gorder] = np.arange(ng)
     members = np.full((ng, R, 2), -1, dtype=np.int32)
-    g_of_item, m_of_item = inv[np.arange(n_items) // R], np.arange(n_items) % R
+    g_of_item, m_of_item = inv[lpos[np.arange(n_items) // R]], np.arange(n_items) % R
     members[g_of_item, m_of_item, 0] = items[jorder, 0]
     members[g_of_item, m_of_item, 1] = items[jorder, 3]
     # one record per edge slot, sorted by (group, neighbour, member); equal records keep the slot order
