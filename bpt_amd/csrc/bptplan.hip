@@ -521,6 +521,94 @@ __global__ void k_pairs(const int32_t *eids_dst, const int32_t *ginfo_dst, int32
     pairs[j] = out;
 }
 
+// ---- CSR of an edge list ------------------------------------------------------------------------------------------------
+__global__ void k_csr_keys(const int64_t *rows, const int64_t *cols, int64_t n_edges, int64_t n_nodes, int32_t *info,
+                           uint32_t *key, int32_t *val) {
+    const int64_t e = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (e == 0) info[1] = 0;
+    if (e >= n_edges) return;
+    const int64_t r = rows[e], c = cols[e];
+    const bool ok = r >= 0 && r < n_nodes && c >= 0 && c < n_nodes;
+    if (!ok) atomicMax(&info[0], 1);
+    key[e] = ok ? (uint32_t)r : PAD32;
+    val[e] = (int32_t)e;
+}
+
+__global__ void k_csr_slots(const int64_t *cols, const int32_t *val_s, int64_t n_edges, const int32_t *info, int64_t *indices,
+                            int64_t *eid) {
+    const int64_t p = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (p >= n_edges || info[0]) return;
+    const int32_t e = val_s[p];
+    eid[p] = e;
+    indices[p] = cols[e];
+}
+
+// indptr[r] = first slot whose row is >= r; number of chunked units of every row
+__global__ void k_csr_indptr(const uint32_t *key_s, int64_t n_edges, int64_t n_nodes, int32_t chunk, const int32_t *info,
+                             int64_t *indptr, int32_t *lo_of, int32_t *n_units_of) {
+    const int64_t r = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (r > n_nodes || info[0]) return;
+    int64_t lo = 0, hi = n_edges;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (key_s[mid] < (uint32_t)r) lo = mid + 1; else hi = mid;
+    }
+    indptr[r] = lo;
+    lo_of[r] = (int32_t)lo;
+}
+
+__global__ void k_csr_unit_counts(const int32_t *lo_of, int64_t n_nodes, int32_t chunk, const int32_t *info, int32_t *n_units_of) {
+    const int64_t r = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (r > n_nodes || info[0]) return;
+    n_units_of[r] = (r < n_nodes) ? (lo_of[r + 1] - lo_of[r] + chunk - 1) / chunk : 0;
+}
+
+// the units of builder.pyx:305-321: each row's slot range in chunks of at most `chunk` slots; empty rows give no unit
+__global__ void k_csr_units(const int32_t *lo_of, const int32_t *unit_base, int64_t n_nodes, int64_t n_edges, int32_t chunk,
+                            int32_t *info, int64_t *unit_row, int64_t *unit_ptr) {
+    const int64_t r = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (r > n_nodes || info[0]) return;
+    if (r == n_nodes) {
+        info[1] = unit_base[n_nodes];
+        unit_ptr[unit_base[n_nodes]] = n_edges;
+        return;
+    }
+    const int32_t b = lo_of[r], e = lo_of[r + 1];
+    int64_t u = unit_base[r];
+    for (int32_t p = b; p < e; p += chunk, ++u) {
+        unit_row[u] = r;
+        unit_ptr[u] = p;
+    }
+}
+
+struct CsrWs {
+    uint32_t *key, *key_s;
+    int32_t *val, *val_s, *lo_of, *n_units_of, *unit_base;
+    void *tmp;
+};
+
+CsrWs csr_layout(Bump &b, int64_t n_edges, int64_t n_nodes, size_t tmp_bytes) {
+    CsrWs w;
+    w.key = b.take<uint32_t>(n_edges);
+    w.key_s = b.take<uint32_t>(n_edges);
+    w.val = b.take<int32_t>(n_edges);
+    w.val_s = b.take<int32_t>(n_edges);
+    w.lo_of = b.take<int32_t>(n_nodes + 1);
+    w.n_units_of = b.take<int32_t>(n_nodes + 1);
+    w.unit_base = b.take<int32_t>(n_nodes + 1);
+    w.tmp = b.take<char>((int64_t)tmp_bytes);
+    return w;
+}
+
+hipError_t csr_temp_bytes(int64_t n_edges, int64_t n_nodes, size_t *out) {
+    size_t a = 0, b = 0;
+    hipError_t e;
+    if ((e = sort_pairs<uint32_t>(nullptr, a, nullptr, nullptr, nullptr, nullptr, n_edges + 1, 32, nullptr)) != hipSuccess) return e;
+    if ((e = scan_i32(nullptr, b, nullptr, nullptr, n_nodes + 1, nullptr)) != hipSuccess) return e;
+    *out = (a > b ? a : b) + 256;
+    return hipSuccess;
+}
+
 int sizes_ok(int64_t n_units, int64_t n_edges, int64_t n_rows, int64_t n_index_nodes, int32_t seg_len) {
     if (n_units < 0 || n_edges < 0 || n_rows < 0 || n_index_nodes < 0) return BPT_ERR_SIZE;
     if (n_rows >= INT32_MAX || n_edges >= INT32_MAX || n_index_nodes >= INT32_MAX || n_units > n_edges + n_rows) return BPT_ERR_SIZE;
@@ -545,6 +633,50 @@ int sizes_ok(int64_t n_units, int64_t n_edges, int64_t n_rows, int64_t n_index_n
 }  // namespace
 
 extern "C" {
+
+int bpt_csr_device_bounds(int64_t n_edges, int64_t n_nodes, int32_t chunk_size, int64_t bounds[2]) {
+    if (!bounds) return BPT_ERR_NULL;
+    if (n_edges < 0 || n_nodes < 0 || n_edges >= INT32_MAX || n_nodes >= INT32_MAX) return BPT_ERR_SIZE;
+    if (chunk_size < 1) return BPT_ERR_SHAPE;
+    size_t tmp = 0;
+    HIP_TRY(csr_temp_bytes(n_edges, n_nodes, &tmp));
+    Bump dry{nullptr, 0};
+    csr_layout(dry, n_edges, n_nodes, tmp);
+    const int64_t by_rows = n_nodes + n_edges / chunk_size;
+    bounds[0] = by_rows < n_edges ? by_rows : n_edges;
+    bounds[1] = (int64_t)dry.off + 256;
+    return BPT_OK;
+}
+
+int bpt_csr_build_device(const int64_t *rows, const int64_t *cols, int64_t n_edges, int64_t n_nodes, int32_t chunk_size,
+                         int64_t *indptr, int64_t *indices, int64_t *eid, int64_t *unit_row, int64_t *unit_ptr, int32_t *info,
+                         void *workspace, int64_t workspace_bytes, void *stream) {
+    int64_t bounds[2];
+    const int st = bpt_csr_device_bounds(n_edges, n_nodes, chunk_size, bounds);
+    if (st != BPT_OK) return st;
+    if (!indptr || !unit_ptr || !info || !workspace) return BPT_ERR_NULL;
+    if (n_edges > 0 && (!rows || !cols || !indices || !eid || !unit_row)) return BPT_ERR_NULL;
+    if (workspace_bytes < bounds[1]) return BPT_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    size_t tmp = 0;
+    HIP_TRY(csr_temp_bytes(n_edges, n_nodes, &tmp));
+    Bump bump{(char *)workspace, 0};
+    CsrWs w = csr_layout(bump, n_edges, n_nodes, tmp);
+    LAUNCH(k_fill_i32, 16, info, 16, 0);
+    size_t tb;
+    if (n_edges > 0) {
+        LAUNCH(k_csr_keys, n_edges, rows, cols, n_edges, n_nodes, info, w.key, w.val);
+        tb = tmp;
+        HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key, w.key_s, w.val, w.val_s, n_edges, 32, s));
+        LAUNCH(k_csr_slots, n_edges, cols, w.val_s, n_edges, info, indices, eid);
+    }
+    LAUNCH(k_csr_indptr, n_nodes + 1, w.key_s, n_edges, n_nodes, chunk_size, info, indptr, w.lo_of, w.n_units_of);
+    LAUNCH(k_csr_unit_counts, n_nodes + 1, w.lo_of, n_nodes, chunk_size, info, w.n_units_of);
+    tb = tmp;
+    HIP_TRY(scan_i32(w.tmp, tb, w.n_units_of, w.unit_base, n_nodes + 1, s));
+    LAUNCH(k_csr_units, n_nodes + 1, w.lo_of, w.unit_base, n_nodes, n_edges, chunk_size, info, unit_row, unit_ptr);
+    return BPT_OK;
+}
 
 int bpt_plan_device_bounds(int64_t n_units, int64_t n_edges, int64_t n_rows, int32_t seg_len, int32_t R, int64_t bounds[4]) {
     if (!bounds) return BPT_ERR_NULL;

@@ -153,6 +153,48 @@ def get_csrs(src, dst, n_nodes, chunk_size=32, as_torch=True):
     return res
 
 
+def get_csrs_device(src, dst, n_nodes, chunk_size=32):
+    """get_csrs for an edge list that already lives on the GPU (int64 CUDA tensors): the same 6-tuple, built there by
+    libbptplan (bpt_csr_build_device: a stable radix sort by row, binary searches, a prefix sum) and bit for bit what
+    get_csrs returns for the same edges.  One synchronisation (the number of units of each side comes back)."""
+    import torch
+    from ._lib import plan_lib
+    if not (src.is_cuda and dst.is_cuda and src.dtype == torch.int64 and dst.dtype == torch.int64):
+        raise ValueError("src and dst must be int64 CUDA tensors")
+    if src.shape != dst.shape or src.dim() != 1:
+        raise ValueError("src and dst must be 1-D tensors of the same length")
+    src, dst = src.contiguous(), dst.contiguous()
+    lib, E, n, dev = plan_lib(), int(src.numel()), int(n_nodes), src.device
+    b = (ctypes.c_int64 * 2)()
+    st = lib.bpt_csr_device_bounds(E, n, int(chunk_size), ctypes.byref(b))
+    if st != 0:
+        raise RuntimeError(f"bpt_csr_device_bounds: status {st}")
+    i64 = lambda k: torch.empty(max(k, 1), dtype=torch.int64, device=dev)
+    sides = []
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream().cuda_stream
+        for rows, cols in ((src, dst), (dst, src)):
+            indptr, indices, eid = i64(n + 1), i64(E), i64(E)
+            unit_row, unit_ptr = i64(int(b[0])), i64(int(b[0]) + 1)
+            info = torch.empty(16, dtype=torch.int32, device=dev)
+            ws = torch.empty(int(b[1]), dtype=torch.uint8, device=dev)
+            st = lib.bpt_csr_build_device(rows.data_ptr() if E else None, cols.data_ptr() if E else None, E, n,
+                                          int(chunk_size), indptr.data_ptr(), indices.data_ptr(), eid.data_ptr(),
+                                          unit_row.data_ptr(), unit_ptr.data_ptr(), info.data_ptr(), ws.data_ptr(),
+                                          ws.numel(), stream)
+            if st != 0:
+                raise RuntimeError(f"bpt_csr_build_device: status {st}")
+            sides.append((indptr, indices[:E], eid[:E], unit_row, unit_ptr, info))
+    out = []
+    for indptr, indices, eid, unit_row, unit_ptr, info in sides:
+        err, n_units = info[:2].tolist()
+        if err:
+            raise ValueError("bptplan: row id, column id or edge id out of range")
+        out.append(((indptr, indices, eid), unit_row[:n_units].clone(), unit_ptr[:n_units + 1].clone()))
+    (out_csr, ROW, INDPTR_R), (in_csr, COL, INDPTR_C) = out
+    return out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C
+
+
 def merge_graphs(graphs):
     """Block-diagonal batch merge of graph/lm.py:53-98 / graph/text_classification.py:30-67:
     returns (src, dst, etype, pos, n_nodes); the edge id of an edge is its position."""

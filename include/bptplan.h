@@ -29,6 +29,18 @@ enum { BPT_PI_ERR = 0,        /* 0 ok, 1 id out of range, 2 row / indptr not mon
 /* indices into the int32[16] info block of bpt_plan_group_device */
 enum { BPT_GI_N_GROUPS = 0, BPT_GI_N_ENTRIES = 1, BPT_GI_MAX_CHUNK = 2 };
 
+/* One CSR side of graph/base.py:71-86 from an edge list on the device: the edges grouped by rows[e], ascending edge
+ * id inside a row (the order of bptg_build_csr, bptgraph.h), in the reference's int64 layout: indptr (n_nodes + 1),
+ * indices (n_edges: cols of the slots), eid (n_edges); and the chunked units of builder.pyx:305-321 (partition_csr):
+ * unit_row (bounds[0]), unit_ptr (bounds[0] + 1), unit_ptr[n_units] = n_edges, no unit for an empty row.
+ * bpt_csr_device_bounds: bounds[0] = most units there can be, bounds[1] = workspace bytes.
+ * info: int32[16]; info[0] = 0, or 1 when a row / column id is outside [0, n_nodes) (then nothing else is valid);
+ * info[1] = number of units. */
+int bpt_csr_device_bounds(int64_t n_edges, int64_t n_nodes, int32_t chunk_size, int64_t bounds[2]);
+int bpt_csr_build_device(const int64_t *rows, const int64_t *cols, int64_t n_edges, int64_t n_nodes, int32_t chunk_size,
+                         int64_t *indptr, int64_t *indices, int64_t *eid, int64_t *unit_row, int64_t *unit_ptr,
+                         int32_t *info, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Upper bounds of the data-dependent sizes, for the caller's allocations:
  *   bounds[0] = items      (rows of 4 int32)      n_rows + n_edges / seg_len
  *   bounds[1] = heavy rows (rows of 3 int32)      n_edges / (seg_len + 1)

@@ -254,3 +254,52 @@ def test_device_plan_at_headline_size_and_its_build_time():
         arrays, info = model.base_plan(*arrs, n, n, 64)
         check_base(dp, arrays, info)
         check_groups(dp.ensure_groups(8, 6 if by_mask else 10), model.group_plan(arrays, n, 8, by_mask), len(src))
+
+
+@pytest.mark.parametrize("chunk", [4, 32])
+@pytest.mark.parametrize("name", sorted(GRAPHS))
+def test_device_csr_equals_host_csr(name, chunk):
+    """get_csrs_device: bit for bit the arrays of get_csrs (the layout of graph/base.py:71-86 + partition_csr)."""
+    from bpt_amd import graphbuilder as gb
+    src, dst, n = GRAPHS[name]()
+    want = gb.get_csrs(src, dst, n, chunk_size=chunk, as_torch=False)
+    got = gb.get_csrs_device(torch.from_numpy(src).to(DEV), torch.from_numpy(dst).to(DEV), n, chunk_size=chunk)
+    for side in (0, 1):
+        for a, b in zip(got[side], want[side]):
+            assert a.dtype == torch.int64 and np.array_equal(host(a), b)
+    for a, b in zip(got[2:], want[2:]):
+        assert a.dtype == torch.int64 and np.array_equal(host(a), b)
+
+
+def test_device_csr_edge_cases():
+    from bpt_amd import graphbuilder as gb
+    e = torch.empty(0, dtype=torch.int64, device=DEV)
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs_device(e, e, 5)
+    assert host(out_csr[0]).tolist() == [0] * 6 and ROW.numel() == 0 and host(IR).tolist() == [0]
+    bad = torch.tensor([0, 7], dtype=torch.int64, device=DEV)
+    with pytest.raises(ValueError, match="out of range"):
+        gb.get_csrs_device(bad, torch.zeros_like(bad), 5)
+    with pytest.raises(ValueError):
+        gb.get_csrs_device(bad.cpu(), bad.cpu(), 9)
+    torch.cuda.synchronize()
+
+
+def test_edge_list_to_attention_without_leaving_the_gpu(device_plans):
+    """Edge list on the device -> CSRs -> plans -> fused attention forward and backward, against the oracle."""
+    from bpt_amd import graphbuilder as gb, graphop
+    src, dst, n = GRAPHS["batch"]()
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs_device(torch.from_numpy(src).to(DEV), torch.from_numpy(dst).to(DEV), n)
+    h, d = 8, 64
+    q, k, v, do = (rand((n, h, d), torch.float32, s, 0.125 if s < 3 else 1.0) for s in range(4))
+    qd, kd, vd, dod = (x.to(DEV) for x in (q, k, v, do))
+    inn, out = (COL, IC, in_csr[2], in_csr[1]), (ROW, IR, out_csr[2], out_csr[1])
+    o, lse = graphop.attention_forward(*inn, qd, kd, vd)
+    dq, dk, dv = graphop.attention_backward(*out, *inn, qd, kd, vd, o, lse, dod)
+    torch.cuda.synchronize()
+    csr = gb.get_csrs(src, dst, n, as_torch=False)
+    ro, ra = oracle.attention_forward(csr, f64(q), f64(k), f64(v))
+    rdq, rdk, rdv = oracle.attention_backward(csr, f64(q), f64(k), f64(v), ra, f64(do))
+    close(o, ro, TOL[torch.float32], "o")
+    deg = int(max(np.bincount(src, minlength=n).max(), np.bincount(dst, minlength=n).max()))
+    for got, want, nm in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv")):
+        close(got, want, GTOL[torch.float32], nm, terms=deg)
