@@ -1163,7 +1163,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
         ent.y = lane < cnt ? ent.y : 0;
         // edge ids of the lane's entry, four members per vector (the list is padded like the entries)
         int4 xe[R / 4];
-        if constexpr (BIAS) {
+        if constexpr (BIAS || DROP) {
 #pragma unroll
             for (int c = 0; c < R / 4; ++c) xe[c] = eids4[(size_t)(p0 + min(lane, cnt - 1)) * (R / 4) + c];
         }
@@ -1172,7 +1172,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             for (int e = 0; e < GRP_BATCH; ++e) {
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
-                B.pz[e] = DROP ? __builtin_amdgcn_readlane(ent.z, b + e) : 0;
+                B.pz[e] = DROP ? b + e : 0;                  // position of the entry in the chunk: the lane that holds its edge ids
                 if constexpr (BIAS) {
 #pragma unroll
                     for (int c = 0; c < R / 4; ++c) {
@@ -1187,11 +1187,13 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                 load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
             }
         };
-        // multiplier of the pair (member m, entry with mask mk and first pair pz): 1 without dropout
+        // multiplier of the pair (member m, entry at position pz of the chunk): 1 without dropout; keyed by the edge id
         auto keep = [&](int m, int mk, int pz) -> float {
             if constexpr (!DROP) return 1.f;
-            const int n = pz + __builtin_popcount(mk & ((1 << m) - 1));
-            return dropout_keep((uint32_t)(n * H + head), drop_seed, drop_thr, drop_inv);
+            const int4 &x = xe[m / 4];
+            const int held = (m & 3) == 0 ? x.x : (m & 3) == 1 ? x.y : (m & 3) == 2 ? x.z : x.w;
+            const uint32_t edge = (uint32_t)__builtin_amdgcn_readlane(held, pz);
+            return dropout_keep(edge * (uint32_t)H + (uint32_t)head, drop_seed, drop_thr, drop_inv);
         };
         auto one = [&](int m, const float (&kr)[EPL], const float (&vr)[EPL], int mk, int pz, float bz) {
             float qm[EPL];
@@ -1345,7 +1347,7 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
     constexpr int R = 8, NB = MFMA_NB, HL = H / HS, CF = H * D, NE = NB / 2;      // NE: entries a wavefront loads per batch
     // float32: one V area instead of two (a second barrier per batch) and no read-ahead registers, which fits three
     // wavefronts per SIMD and six workgroups per CU (measured 5 % faster); bfloat16 rows are half as large
-    constexpr bool W3 = sizeof(T) == 4 && !BIAS;          // (the score term's registers would not fit)
+    constexpr bool W3 = sizeof(T) == 4 && !BIAS && !DROP;  // (the edge ids and score terms would not fit)
     using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, NV = L::NV, VE = L::VE, BPH = L::LPH / 4, CB = 4 * EPL, PITCH = NV * WAVE + 1;
     static_assert(EPL % VE == 0 && EPL <= 8 && (BPH == 1 || BPH == 2 || BPH == 4), "shape not covered by the matrix-core kernels");
@@ -1405,7 +1407,7 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
     for (int r = 0; r < EPL; ++r) acc[r] = floatx4{0.f, 0.f, 0.f, 0.f};
     struct Raw {
         RawRow<T, HL, D> kr[NE], vr[NE];
-        int xe[BIAS ? NB : 1];                         // edge ids of this lane's member with the batch's entries
+        int xe[(BIAS || DROP) ? NB : 1];               // edge ids of this lane's member with the batch's entries
     };
     for (int p0 = g_begin; p0 < g_end; p0 += GRP_CHUNK) {
         const int cnt = min(GRP_CHUNK, g_end - p0);
@@ -1418,17 +1420,22 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
                 load_row32_raw<T, HL, D, CF>(k, src, loff, B.kr[e]);
                 load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
             }
-            if constexpr (BIAS) {
+            if constexpr (BIAS || DROP) {
 #pragma unroll
                 for (int e = 0; e < NB; ++e) B.xe[e] = P.grp_eids[(size_t)(p0 + b + e) * R + 4 * wv + j];
             }
         };
         // the score terms of a batch are fetched one batch ahead, with the edge ids that came in the batch before
         float bz[NB];
+        int xd[NB];                                    // edge ids of the batch in use (dropout is keyed by them)
         auto load_bias = [&](const Raw &B) {
             if constexpr (BIAS) {
 #pragma unroll
                 for (int e = 0; e < NB; ++e) bz[e] = bias[(size_t)((uint32_t)B.xe[e] * (uint32_t)H) + head];
+            }
+            if constexpr (DROP) {
+#pragma unroll
+                for (int e = 0; e < NB; ++e) xd[e] = B.xe[e];
             }
         };
         auto stage_half = [&](const Raw &B, int buf) {
@@ -1448,12 +1455,9 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
         load_half(raw, NB);
         __syncthreads();
         for (int b = 0, buf = 0; b < cnt; b += NB, buf ^= 1) {
-            int mk[NB], pz[NB];
+            int mk[NB];
 #pragma unroll
-            for (int e = 0; e < NB; ++e) {
-                mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
-                pz[e] = DROP ? __builtin_amdgcn_readlane(ent.z, b + e) : 0;
-            }
+            for (int e = 0; e < NB; ++e) mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
             // all LDS reads of the batch go out first: the K rows of this lane's entry by block, the V rows as loaded
             uint4 kv[NV * 4], vv[NB][NV];
 #pragma unroll
@@ -1506,8 +1510,7 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
                 const float pe = __builtin_amdgcn_exp2f(sc[e] - mref);
                 lrun += pe;                                          // the softmax denominator ignores dropout
                 if constexpr (DROP) {
-                    const int n = pz[e] + __builtin_popcount(mk[e] & ((1 << (4 * wv + j)) - 1));
-                    pk[e] = pe * dropout_keep((uint32_t)(n * H + head), drop_seed, drop_thr, drop_inv);
+                    pk[e] = pe * dropout_keep((uint32_t)xd[e] * (uint32_t)H + (uint32_t)head, drop_seed, drop_thr, drop_inv);
                 } else {
                     pk[e] = pe;
                 }
@@ -1624,7 +1627,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
         ent.y = lane < cnt ? ent.y : 0;
         // edge ids of the lane's entry, four members per vector (the list is padded like the entries)
         int4 xe[R / 4];
-        if constexpr (BIAS) {
+        if constexpr (BIAS || DROP) {
 #pragma unroll
             for (int c = 0; c < R / 4; ++c) xe[c] = eids4[(size_t)(p0 + min(lane, cnt - 1)) * (R / 4) + c];
         }
@@ -1633,7 +1636,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
             for (int e = 0; e < GRP_BATCH; ++e) {
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
-                B.pz[e] = DROP ? __builtin_amdgcn_readlane(ent.z, b + e) : 0;
+                B.pz[e] = DROP ? b + e : 0;                  // position of the entry in the chunk: the lane that holds its edge ids
                 if constexpr (BIAS) {
 #pragma unroll
                     for (int c = 0; c < R / 4; ++c) {
@@ -1672,8 +1675,10 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
                         float pe = __builtin_amdgcn_exp2f(fmaf(s, scale_log2e, -lse2[m]));
                         float mt = 1.f;                   // dropout multiplier of this pair (as in the forward kernel)
                         if constexpr (DROP) {
-                            const int n = B.pz[e] + __builtin_popcount(B.mk[e] & ((1 << m) - 1));
-                            mt = dropout_keep((uint32_t)(n * H + head), drop_seed, drop_thr, drop_inv);
+                            const int4 &x = xe[m / 4];
+                            const int held = (m & 3) == 0 ? x.x : (m & 3) == 1 ? x.y : (m & 3) == 2 ? x.z : x.w;
+                            const uint32_t edge = (uint32_t)__builtin_amdgcn_readlane(held, B.pz[e]);
+                            mt = dropout_keep(edge * (uint32_t)H + (uint32_t)head, drop_seed, drop_thr, drop_inv);
                         }
                         const float ds = pe * fmaf(dp * mt, scale, -delta_s[m]);
                         pe *= mt;                         // what multiplies v (forward) and dO (dV)
@@ -2410,7 +2415,7 @@ int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k,
     const Dropout drop = make_dropout(dropout_p, dropout_seed);
     // dropout and the score term exist in the row-group kernels only
     if ((drop.thr != 0 || bias) && !has_groups(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
-    if (bias && !plan_in->grp_eids) return BPT_ERR_PLAN;
+    if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(workspace))
         return BPT_ERR_UNSUPPORTED;
     const int64_t need = bpt_workspace_bytes(BPT_OP_ATTN_FWD, plan_in, nullptr, h, d, dtype);
@@ -2434,7 +2439,7 @@ int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, co
     const Dropout drop = make_dropout(dropout_p, dropout_seed);
     if ((drop.thr != 0 || bias) && !grouped_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
     if ((bias != nullptr) != (ds_out != nullptr)) return BPT_ERR_NULL;       // the score term and its gradient go together
-    if (bias && !plan_in->grp_eids) return BPT_ERR_PLAN;
+    if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
     if (plan_in->n_edges != plan_out->n_edges || plan_in->n_rows != plan_out->n_rows) return BPT_ERR_PLAN;
     if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return BPT_ERR_NULL;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) ||

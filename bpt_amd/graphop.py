@@ -313,12 +313,11 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
 
 def attention_dropout_mask(col, indptr_c, eid_c, indices_c, q, k, dropout_p, seed):
     """The (E, h) float32 multipliers (0 or 1 / (1 - p)) that attention_forward(..., dropout_p, seed) applies to the
-    attention probabilities of these tensors, computed on the host from the plan (testing and debugging aid)."""
+    attention probabilities, computed on the host (testing and debugging aid).  The decision is a hash of
+    (seed, edge id, head): it does not depend on the graph's plan."""
     import numpy as np
     h, d = _hd(q)
-    plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
-    grp = plan.ensure_groups(_group_rows(q, h, d, plan))["host"]
-    E = plan.n_edges
+    E = eid_c.size(0)
     p = float(dropout_p)
     if not p > 0.0:
         return torch.ones((E, h), dtype=torch.float32)
@@ -331,10 +330,8 @@ def attention_dropout_mask(col, indptr_c, eid_c, indices_c, q, k, dropout_p, see
     x ^= x >> np.uint32(16); x = (x.astype(np.uint64) * np.uint64(0x7feb352d)).astype(np.uint32)
     x ^= x >> np.uint32(15); x = (x.astype(np.uint64) * np.uint64(0x846ca68b)).astype(np.uint32)
     x ^= x >> np.uint32(16)
-    keep_pair = np.where(x >= thr, np.float32(1.0 / (1.0 - np.float32(p))), np.float32(0.0)).astype(np.float32)   # by pair number
-    out = np.empty((E, h), dtype=np.float32)
-    out[grp["pair_eid"]] = keep_pair
-    return torch.from_numpy(out)
+    keep = np.where(x >= thr, np.float32(1.0 / (1.0 - np.float32(p))), np.float32(0.0)).astype(np.float32)
+    return torch.from_numpy(keep)
 
 
 _USE_GROUPS = True
@@ -354,8 +351,8 @@ def _group_rows(q, h, d, plan):
 def _forward_rows(q, h, d, plan, dropout_p=0.0):
     """Rows per group for the forward kernel.  Groups of 8 run on the matrix cores (two wavefronts per group; bfloat16
     rows go through the bfloat16 matrix instructions as loaded), which measured faster than the vector kernels at every
-    size and both dtypes.  With dropout the forward and the backward number the pairs by the same groups."""
-    if _GROUP_ROWS is not None or dropout_p > 0.0:
+    size and both dtypes."""
+    if _GROUP_ROWS is not None:
         return _group_rows(q, h, d, plan)
     return 8
 

@@ -150,9 +150,9 @@ int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table,
  * bpt_rel_bias_forward); row n_edges is a spare row that is read for absent pairs and never used.  Needs the row
  * groups with grp_eids (BPT_ERR_UNSUPPORTED / BPT_ERR_PLAN without them).
  * dropout_p in [0, 1): dropout on the attention probabilities (attention.py:73); 0 = none.  Each (edge, head) is
- * kept with probability 1 - p and scaled by 1 / (1 - p); the decision is a hash of dropout_seed and the edge's pair
- * number in plan_in's row groups, so backward must get the same plan, p and seed.  Needs the row groups
- * (BPT_ERR_UNSUPPORTED without them). */
+ * kept with probability 1 - p and scaled by 1 / (1 - p); the decision is a hash of (dropout_seed, edge id, head),
+ * so it does not depend on the plan and backward only needs the same p and seed.  Needs the row groups with
+ * grp_eids (BPT_ERR_UNSUPPORTED / BPT_ERR_PLAN without them). */
 int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k, const void *v, const float *bias,
                           void *o, float *lse, void *workspace, int64_t workspace_bytes,
                           float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype, void *stream);
