@@ -216,8 +216,9 @@ def test_ops_and_rel_pos_on_device_plans_match_host_plans(device_plans):
         qq, kk, vv, tt = (x.clone().requires_grad_(True) for x in (q, k, v, table))
         o = op.bpt_attention(*c.out, *c.inn, qq, kk, vv, rel_table=tt, etype=etype)
         o.sum().backward()
+        od = op.bpt_attention(*c.out, *c.inn, q, k, v, dropout_p=0.2, seed=5)      # the mask is keyed by edge id, not by the plan
         torch.cuda.synchronize()
-        return e, a, y, o.detach(), qq.grad, kk.grad, vv.grad, tt.grad
+        return e, a, y, o.detach(), qq.grad, kk.grad, vv.grad, tt.grad, od
 
     dev = run()
     assert isinstance(plan.plan_cache.get(*c.inn, c.n, c.n), plan.DevicePlan)
@@ -303,3 +304,38 @@ def test_edge_list_to_attention_without_leaving_the_gpu(device_plans):
     deg = int(max(np.bincount(src, minlength=n).max(), np.bincount(dst, minlength=n).max()))
     for got, want, nm in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv")):
         close(got, want, GTOL[torch.float32], nm, terms=deg)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_device_plan_on_random_graphs(seed):
+    """Seeded random multigraphs (empty rows, rows longer than a segment, repeated edges, more index nodes than rows):
+    CSR, base plan, groups and pair mapping equal the host builders / the model."""
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd.plan import GROUP_PAD_ENTRIES, DevicePlan
+    rng = np.random.default_rng(100 + seed)
+    n = int(rng.integers(1, 300))
+    E = int(rng.integers(0, 4000))
+    hot = rng.integers(0, n, 3)
+    src = np.where(rng.random(E) < 0.3, hot[rng.integers(0, 3, E)], rng.integers(0, n, E)).astype(np.int64)
+    dst = np.where(rng.random(E) < 0.3, hot[rng.integers(0, 3, E)], rng.integers(0, max(n // 2, 1), E)).astype(np.int64)
+    if E > 10:
+        src[-5:], dst[-5:] = src[-6], dst[-6]                        # one edge six times
+    seg, R, chunk = int(rng.choice([4, 16, 64])), int(rng.choice([4, 8, 16])), int(rng.choice([3, 32]))
+    want = gb.get_csrs(src, dst, n, chunk_size=chunk, as_torch=False)
+    got = gb.get_csrs_device(torch.from_numpy(src).to(DEV), torch.from_numpy(dst).to(DEV), n, chunk_size=chunk)
+    for a, b in zip((*got[0], *got[1], *got[2:]), (*want[0], *want[1], *want[2:])):
+        assert np.array_equal(host(a), b)
+    out_csr, in_csr, ROW, IR, COL, IC = got
+    w_out, w_in = want[0], want[1]
+    sides_ = (((COL, IC, in_csr[2], in_csr[1]), (want[4], want[5], w_in[2], w_in[1]), True),
+              ((ROW, IR, out_csr[2], out_csr[1]), (want[2], want[3], w_out[2], w_out[1]), False))
+    plans, grps = [], []
+    for tens, arrs, by_mask in sides_:
+        dp = DevicePlan(*tens, n, n, DEV, seg)
+        arrays, info = model.base_plan(*arrs, n, n, seg)
+        check_base(dp, arrays, info)
+        grp = model.group_plan(arrays, n, R, by_mask)
+        check_groups(dp.ensure_groups(R, 6 if by_mask else 10), grp, E)
+        plans.append(dp); grps.append(grp)
+    plans[0].linked_to(plans[1], R)
+    assert np.array_equal(host(plans[0]._links[(id(plans[1]), R)][1]), model.link_groups(grps[0], grps[1], E, GROUP_PAD_ENTRIES))
