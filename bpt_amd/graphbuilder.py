@@ -11,7 +11,7 @@ import numpy as np
 from ._lib import check_graph, graph_lib
 
 __all__ = ["BinaryPartition", "FullyConnected", "OpenAISparse", "partition_csr",
-           "build_csr", "get_csrs", "merge_graphs"]
+           "build_csr", "get_csrs", "merge_graphs", "get_csrs_device", "merge_graphs_device"]
 
 
 def _ptr(a):
@@ -206,3 +206,37 @@ def merge_graphs(graphs):
         v_shift += g.number_of_nodes
     cat = np.concatenate
     return cat(src), cat(dst), cat(et), cat(pos), v_shift
+
+
+_DEVICE_EDGES = {}           # (graph class, constructor arguments, device) -> (src, dst, etype, pos) device tensors
+_DEVICE_EDGES_MAX = 4096
+
+
+def merge_graphs_device(graphs, device):
+    """merge_graphs with the result on the GPU: the edge lists of the single graphs are kept on the device per
+    (class, length, ...) the way the reference caches them on the host (graph/base.py:12-26), and a batch is their
+    concatenation plus the node shifts (graph/lm.py:83-98), formed there; only the shifts and counts of the batch
+    (one number per graph) cross the bus.  Returns int64 device tensors (src, dst, etype, pos) and n_nodes."""
+    import torch
+    device = torch.device(device)
+    parts, shifts, v_shift = [], [], 0
+    for g in graphs:
+        key = (type(g).__name__,) + tuple(g.__reduce__()[1]) + (str(device),)
+        hit = _DEVICE_EDGES.get(key)
+        if hit is None:
+            if len(_DEVICE_EDGES) >= _DEVICE_EDGES_MAX:
+                _DEVICE_EDGES.clear()
+            hit = tuple(torch.from_numpy(a).to(device) for a in (*g.get_edges(), g.get_pos()))
+            _DEVICE_EDGES[key] = hit
+        parts.append(hit)
+        shifts.append(v_shift)
+        v_shift += g.number_of_nodes
+    if not parts:
+        e = torch.empty(0, dtype=torch.int64, device=device)
+        return e, e.clone(), e.clone(), e.clone(), 0
+    counts = torch.tensor([p[0].numel() for p in parts], dtype=torch.int64)
+    n_edges = int(counts.sum())
+    shift = torch.repeat_interleave(torch.tensor(shifts, dtype=torch.int64).to(device), counts.to(device), output_size=n_edges)
+    src = torch.cat([p[0] for p in parts]) + shift
+    dst = torch.cat([p[1] for p in parts]) + shift
+    return src, dst, torch.cat([p[2] for p in parts]), torch.cat([p[3] for p in parts]), v_shift

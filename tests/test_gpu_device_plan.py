@@ -339,3 +339,47 @@ def test_device_plan_on_random_graphs(seed):
         plans.append(dp); grps.append(grp)
     plans[0].linked_to(plans[1], R)
     assert np.array_equal(host(plans[0]._links[(id(plans[1]), R)][1]), model.link_groups(grps[0], grps[1], E, GROUP_PAD_ENTRIES))
+
+
+def test_batch_merge_on_the_device_and_the_whole_pipeline_time():
+    """merge_graphs_device equals merge_graphs; and what a new batch costs from its lengths to plans that the fused
+    kernels can run on, on the host and on the GPU (BASELINE config 2: 32 sequences, causal, k = 4)."""
+    import time
+    from bpt_amd import graphbuilder as gb, plan
+    lengths = np.random.default_rng(2345).integers(64, 1025, 32)
+    graphs = [gb.BinaryPartition(int(L), True, 4, 10) for L in lengths]
+    want = gb.merge_graphs(graphs)
+    got = gb.merge_graphs_device(graphs, DEV)
+    for a, b in zip(got[:4], want[:4]):
+        assert np.array_equal(host(a), b)
+    assert got[4] == want[4] == 33598 and len(want[0]) == 573520
+
+    def on_host():
+        src, dst, et, pos, n = gb.merge_graphs(graphs)
+        out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, n)
+        t = [x.to(DEV) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1])]
+        pin, pout = plan.Plan(*t[4:], n, n, DEV), plan.Plan(*t[:4], n, n, DEV)
+        pin.linked_to(pout, 8)
+        return pin, pout
+
+    def on_device():
+        src, dst, et, pos, n = gb.merge_graphs_device(graphs, DEV)
+        out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs_device(src, dst, n)
+        pin = plan.DevicePlan(COL, IC, in_csr[2], in_csr[1], n, n, DEV)
+        pout = plan.DevicePlan(ROW, IR, out_csr[2], out_csr[1], n, n, DEV)
+        pin.linked_to(pout, 8)
+        return pin, pout
+
+    times = {}
+    for name, fn in (("host", on_host), ("device", on_device)):
+        best = 1e9
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            pin, pout = fn()
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        times[name] = best
+        assert pin.n_edges == 573520 and pin.covers_all_edges and pout.covers_all_edges
+    print(f"lengths -> plans with groups of 8 (cfg 2): host {times['host'] * 1e3:.1f} ms, device {times['device'] * 1e3:.2f} ms")
+    assert times["device"] < times["host"]
