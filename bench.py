@@ -217,7 +217,7 @@ def main():
     t_eager = timed(step, args.steps, args.warmup)
     t_step, mode = t_eager, "eager"
     t_graph_replay = None
-    if not args.no_graph and not args.unfused and not args.rel_pos:
+    if not args.no_graph:
         try:
             side = torch.cuda.Stream()
             with torch.cuda.stream(side):

@@ -1340,7 +1340,7 @@ template <typename T> __device__ __forceinline__ void unpack_vec(const uint4 &w,
 // buffers one workgroup barrier per batch orders the writes of batch b + 1 after the reads of batch b - 1; where V
 // has a single buffer (W3 below) a second barrier separates the reads of batch b from the writes of batch b + 1.
 template <typename T, int H, int D, int HS, bool DROP, bool BIAS>
-__global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 && !BIAS ? 3 : 2))) void k_attn_fwd_mfma(
+__global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 && !BIAS && !DROP ? 3 : 2))) void k_attn_fwd_mfma(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o,
     float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr,
     uint32_t drop_seed, float drop_inv, const float *__restrict__ bias) {
@@ -1830,6 +1830,175 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
     }
 }
 
+// Y[row] = sum over the row's edges of W[eid, head] * X[idx]: the row-group form of k_spmm_fast for the unfused ops.
+// X[idx] is loaded once per entry for every member that has the edge; the weight of (entry, member 4c + lane % 4) is
+// fetched by its edge id (grp_eids) and is the A operand of v_mfma_f32_4x4x1 exactly as in k_attn_bwd_src_grp.
+template <typename T, int H, int D, int R, int HS>
+__global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_spmm_grp(
+    bpt_plan P, const T *__restrict__ W, const T *__restrict__ X, T *__restrict__ Y, float *__restrict__ ws) {
+    constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
+    using L = Lay<T, HL, D>;
+    constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
+    static_assert(H % HS == 0 && R % 4 == 0 && L::LPH >= 4, "members are handled in quads inside the lanes of one head");
+    GroupHead<R> gh;
+    if (!fetch_group<R, HS>(P, gh)) return;
+    const int slice = group_slice<R, HS>(), coff = slice * HL * D;
+    const int lane = threadIdx.x, head = slice * HL + lane / L::LPH, mine = lane & 3;
+    const uint32_t loff = (uint32_t)((coff + L::off(lane, 0)) * sizeof(T));
+    const uint32_t last_edge = (uint32_t)max(P.n_edges, (int64_t)1) - 1u;
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    const int4 *eids4 = reinterpret_cast<const int4 *>(P.grp_eids);
+    struct Batch {
+        RawRow<T, HL, D> xr[GRP_BATCH];
+        float w[GRP_BATCH][NQ];
+        int mk[GRP_BATCH];
+    };
+    floatx4 acc[NQ][EPL];                      // [quad c][row register t][member 4c + i]
+#pragma unroll
+    for (int c = 0; c < NQ; ++c)
+#pragma unroll
+        for (int t = 0; t < EPL; ++t) acc[c][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int p0 = gh.begin; p0 < gh.end; p0 += GRP_CHUNK) {
+        const int cnt = min(GRP_CHUNK, gh.end - p0);
+        // lanes past the end repeat the last entry with an empty mask
+        int4 ent = entries[p0 + min(lane, cnt - 1)];
+        ent.y = lane < cnt ? ent.y : 0;
+        // edge ids of the lane's entry, four members per vector
+        int4 xe[R / 4];
+#pragma unroll
+        for (int c = 0; c < R / 4; ++c) xe[c] = eids4[(size_t)(p0 + min(lane, cnt - 1)) * (R / 4) + c];
+        auto load_batch = [&](Batch &B, int b) {
+#pragma unroll
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
+                B.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
+#pragma unroll
+                for (int c = 0; c < NQ; ++c) {
+                    const uint32_t e0 = (uint32_t)__builtin_amdgcn_readlane(xe[c].x, b + e), e1 = (uint32_t)__builtin_amdgcn_readlane(xe[c].y, b + e);
+                    const uint32_t e2 = (uint32_t)__builtin_amdgcn_readlane(xe[c].z, b + e), e3 = (uint32_t)__builtin_amdgcn_readlane(xe[c].w, b + e);
+                    // absent members carry the id n_edges: read the last edge instead, the mask zeroes the weight
+                    const uint32_t el = min(mine == 0 ? e0 : mine == 1 ? e1 : mine == 2 ? e2 : e3, last_edge);
+                    B.w[e][c] = ld_w(W + (size_t)el * H + head);
+                }
+                load_row32_raw<T, HL, D, CF>(X, src, loff, B.xr[e]);
+            }
+        };
+        auto compute = [&](const Batch &B) {
+#pragma unroll
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                float xv[EPL];
+                unpack_row<T, HL, D>(B.xr[e], xv);
+#pragma unroll
+                for (int c = 0; c < NQ; ++c) {
+                    if ((B.mk[e] >> (4 * c)) & 15) {
+                        const int keep = __builtin_amdgcn_sbfe(B.mk[e], 4 * c + mine, 1);     // all-ones where the member has the edge
+                        const float wt = __int_as_float(__float_as_int(B.w[e][c]) & keep);
+#pragma unroll
+                        for (int t = 0; t < EPL; ++t) acc[c][t] = __builtin_amdgcn_mfma_f32_4x4x1f32(wt, xv[t], acc[c][t], 0, 0, 0);
+                    }
+                }
+            }
+        };
+        // two-stage software pipeline as in the fused kernels (unconditional loads; look-ahead past the end re-reads
+        // the chunk's last entry with an empty mask)
+        Batch A, B;
+        load_batch(A, 0);
+        for (int b = 0; b < cnt; b += 2 * GRP_BATCH) {
+            load_batch(B, b + GRP_BATCH);
+            issue_loads_first();
+            compute(A);
+            issue_loads_first();
+            load_batch(A, b + 2 * GRP_BATCH);
+            issue_loads_first();
+            compute(B);
+            issue_loads_first();
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < R; ++m) {
+        if (gh.rows[m] < 0) continue;
+        float out[EPL];
+#pragma unroll
+        for (int t = 0; t < EPL; ++t) out[t] = acc[m / 4][t][m & 3];
+        if (gh.slots[m] < 0) store_row<T, HL, D>(Y + (size_t)gh.rows[m] * CF + coff, lane, out);
+        else store_row_ws<T, HL, D>(ws + (size_t)gh.slots[m] * CF + coff, lane, out);
+    }
+}
+
+// y[eid, head] = <A[row, head, :], B[idx, head, :]> for every edge: the row-group form of k_sddmm_fast.  The
+// members' A rows stay in registers, B[idx] is loaded once per entry and every member that has the edge takes its
+// dot products with it; the edge id of (entry, member) comes from grp_eids.
+template <typename T, int H, int D, int R, int HS>
+__global__ __launch_bounds__(WAVE) void k_sddmm_grp(bpt_plan P, const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ y) {
+    constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
+    using L = Lay<T, HL, D>;
+    constexpr int EPL = L::EPL, GRP_BATCH = 2;
+    static_assert(H % HS == 0 && R % 4 == 0, "edge ids come four members per vector");
+    GroupHead<R> gh;
+    if (!fetch_group<R, HS>(P, gh)) return;
+    const int slice = group_slice<R, HS>(), coff = slice * HL * D;
+    const int lane = threadIdx.x, head = slice * HL + lane / L::LPH;
+    const uint32_t loff = (uint32_t)((coff + L::off(lane, 0)) * sizeof(T));
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    const int4 *eids4 = reinterpret_cast<const int4 *>(P.grp_eids);
+    float a[R][EPL];
+#pragma unroll
+    for (int m = 0; m < R; ++m) load_row32<T, HL, D, CF>(A, (uint32_t)max(gh.rows[m], 0), loff, a[m]);
+    struct Batch {
+        RawRow<T, HL, D> br[GRP_BATCH];
+        int mk[GRP_BATCH], pz[GRP_BATCH];
+    };
+    for (int p0 = gh.begin; p0 < gh.end; p0 += GRP_CHUNK) {
+        const int cnt = min(GRP_CHUNK, gh.end - p0);
+        // lanes past the end repeat the last entry with an empty mask
+        int4 ent = entries[p0 + min(lane, cnt - 1)];
+        ent.y = lane < cnt ? ent.y : 0;
+        int4 xe[R / 4];                                     // edge ids of the lane's entry, four members per vector
+#pragma unroll
+        for (int c = 0; c < R / 4; ++c) xe[c] = eids4[(size_t)(p0 + min(lane, cnt - 1)) * (R / 4) + c];
+        auto load_batch = [&](Batch &Bt, int b) {
+#pragma unroll
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
+                Bt.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
+                Bt.pz[e] = b + e;
+                load_row32_raw<T, HL, D, CF>(B, src, loff, Bt.br[e]);
+            }
+        };
+        auto compute = [&](const Batch &Bt) {
+#pragma unroll
+            for (int e = 0; e < GRP_BATCH; ++e) {
+                float bv[EPL];
+                unpack_row<T, HL, D>(Bt.br[e], bv);
+#pragma unroll
+                for (int m = 0; m < R; ++m) {
+                    if ((Bt.mk[e] >> m) & 1) {
+                        const float s = head_sum<L::LPH>(dot_n<EPL>(a[m], bv));
+                        const int4 &x = xe[m / 4];
+                        const int held = (m & 3) == 0 ? x.x : (m & 3) == 1 ? x.y : (m & 3) == 2 ? x.z : x.w;
+                        const uint32_t edge = (uint32_t)__builtin_amdgcn_readlane(held, Bt.pz[e]);
+                        if (lane % L::LPH == 0) Elem<T>::st(y + (size_t)edge * H + head, s);
+                    }
+                }
+            }
+        };
+        // two-stage software pipeline as in the fused kernels (unconditional loads; look-ahead past the end re-reads
+        // the chunk's last entry with an empty mask)
+        Batch X0, X1;
+        load_batch(X0, 0);
+        for (int b = 0; b < cnt; b += 2 * GRP_BATCH) {
+            load_batch(X1, b + GRP_BATCH);
+            issue_loads_first();
+            compute(X0);
+            issue_loads_first();
+            load_batch(X0, b + 2 * GRP_BATCH);
+            issue_loads_first();
+            compute(X1);
+            issue_loads_first();
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
@@ -2063,12 +2232,22 @@ int spmm_fast(const bpt_plan *P, const void *W, const void *Xp, void *Y, void *w
 }
 
 // SDDMM / SpMM with automatic family choice
+bool spmm_grp_ok(const bpt_plan *P, int h, int d, int dtype);
+int sddmm_grp(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s);
 int sddmm(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s) {
-    if (fast_shape(h, d, dtype) && aligned16(A) && aligned16(B)) return sddmm_fast(P, A, B, y, h, d, dtype, s);
+    if (fast_shape(h, d, dtype) && aligned16(A) && aligned16(B)) {
+        if (spmm_grp_ok(P, h, d, dtype)) return sddmm_grp(P, A, B, y, h, d, dtype, s);
+        return sddmm_fast(P, A, B, y, h, d, dtype, s);
+    }
     return sddmm_generic(P, A, B, y, h, d, dtype, s);
 }
+int spmm_grp(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, int dtype, hipStream_t s);
 int spmm(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, int dtype, hipStream_t s) {
-    if (fast_shape(h, d, dtype) && aligned16(X) && aligned16(Y) && aligned16(ws)) return spmm_fast(P, W, X, Y, ws, h, d, dtype, s);
+    if (fast_shape(h, d, dtype) && aligned16(X) && aligned16(Y) && aligned16(ws)) {
+        // a plan that carries row groups and their edge ids: one row load per entry instead of one per edge
+        if (spmm_grp_ok(P, h, d, dtype)) return spmm_grp(P, W, X, Y, ws, h, d, dtype, s);
+        return spmm_fast(P, W, X, Y, ws, h, d, dtype, s);
+    }
     return spmm_generic(P, W, X, Y, ws, h, d, dtype, s);
 }
 
@@ -2121,6 +2300,50 @@ inline bool has_groups(const bpt_plan *P, int h, int d, size_t elem) {
            P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups && P->n_grp_entries >= 0 &&
            fits32(P->n_rows, (int64_t)h * d * (int64_t)elem) &&
            fits32((P->n_grp_entries + GRP_PAD_ENTRIES) * P->grp_R, (int64_t)h * 8);
+}
+
+bool spmm_grp_ok(const bpt_plan *P, int h, int d, int dtype) {
+    return has_groups(P, h, d, dtype == BPT_BF16 ? 2 : 4) && P->grp_eids && P->n_edges > 0;
+}
+
+template <typename T, int H, int D>
+int run_spmm_grp(const bpt_plan *P, const void *W, const void *X, void *Y, float *ws, hipStream_t s) {
+    constexpr int HS = head_slices<T, H, D>();
+#define LAUNCH_SPMM(RR)                                                                                                     \
+    hipLaunchKernelGGL((k_spmm_grp<T, H, D, RR, HS>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)W, (const T *)X, \
+                       (T *)Y, ws)
+    if (P->grp_R == 8) LAUNCH_SPMM(8);
+    else LAUNCH_SPMM(4);
+#undef LAUNCH_SPMM
+    int st = launch_status();
+    if (st != BPT_OK || P->n_heavy == 0) return st;
+    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
+                       (T *)Y, (T *)nullptr, H * D, (size_t)0);
+    return launch_status();
+}
+
+template <typename T, int H, int D>
+int run_sddmm_grp(const bpt_plan *P, const void *A, const void *B, void *y, hipStream_t s) {
+    constexpr int HS = head_slices<T, H, D>();
+    if (P->grp_R == 8) hipLaunchKernelGGL((k_sddmm_grp<T, H, D, 8, HS>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)A, (const T *)B, (T *)y);
+    else hipLaunchKernelGGL((k_sddmm_grp<T, H, D, 4, HS>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)A, (const T *)B, (T *)y);
+    return launch_status();
+}
+
+int sddmm_grp(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d, int dtype, hipStream_t s) {
+#define X(HH, DD) if (h == HH && d == DD) return run_sddmm_grp<T, HH, DD>(P, A, B, y, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
+int spmm_grp(const bpt_plan *P, const void *W, const void *Xp, void *Y, void *ws, int h, int d, int dtype, hipStream_t s) {
+#define X(HH, DD) if (h == HH && d == DD) return run_spmm_grp<T, HH, DD>(P, W, Xp, Y, (float *)ws, s);
+    if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
+    if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
 }
 
 inline bool grouped_backward(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {

@@ -85,6 +85,15 @@ def _workspace(op, plan, plan_t, h, d, dt, device, plan_ref=None, plan_t_ref=Non
     return torch.empty(n, dtype=torch.uint8, device=device), n
 
 
+def _spmm_ref(plan, x, h, d):
+    """The plan to hand a SpMM- or SDDMM-shaped op: with row groups (one load of a neighbour row per group entry instead of one
+    per edge) where the row-group kernels apply, else the plain plan."""
+    if not (_USE_GROUPS and _GROUPED_OPS and attention_supported(x) and plan.covers_all_edges and plan.has_indices
+            and plan.n_edges > 0 and max(plan.n_rows, plan.n_index_nodes) * h * d * x.element_size() < 2 ** 32):
+        return plan.ref
+    return ctypes.byref(plan.ensure_groups(_group_rows(x, h, d, plan), GROUP_ORDER_SRC)["struct"])
+
+
 def _edge_out(plan, shape, like):
     # kernels write every edge id the plan covers; zero-fill only when some edge is not covered
     return (torch.empty if plan.covers_all_edges else torch.zeros)(shape, dtype=like.dtype, device=like.device)
@@ -99,7 +108,7 @@ def maskedmm_csr_forward(row, indptr, eid, indices, A, B):
     e = eid.size(0)
     y = _edge_out(plan, (e,) if A.dim() == 2 else (e, h), A)
     with torch.cuda.device_of(A):
-        check_attn(_LIB.bpt_maskedmm_csr_forward(plan.ref, _ptr(A), _ptr(B), _ptr(y), h, d, _dtype(A), _stream()),
+        check_attn(_LIB.bpt_maskedmm_csr_forward(_spmm_ref(plan, A, h, d), _ptr(A), _ptr(B), _ptr(y), h, d, _dtype(A), _stream()),
                    "maskedmm_csr_forward")
     return y
 
@@ -117,7 +126,7 @@ def maskedmm_csr_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c,
     dt = _dtype(A)
     ws, nws = _workspace(OP_MASKEDMM_BWD, plan_r, plan_c, h, d, dt, A.device)
     with torch.cuda.device_of(A):
-        check_attn(_LIB.bpt_maskedmm_csr_backward(plan_r.ref, plan_c.ref, _ptr(A), _ptr(B), _ptr(dy), _ptr(dA), _ptr(dB),
+        check_attn(_LIB.bpt_maskedmm_csr_backward(_spmm_ref(plan_r, A, h, d), _spmm_ref(plan_c, A, h, d), _ptr(A), _ptr(B), _ptr(dy), _ptr(dA), _ptr(dB),
                                                   _ptr(ws), nws, h, d, dt, _stream()), "maskedmm_csr_backward")
     return [dA, dB]
 
@@ -195,7 +204,8 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None):
     dt = _dtype(x)
     ws, nws = _workspace(OP_SPMM_FWD, plan, None, h, d, dt, x.device)
     with torch.cuda.device_of(x):
-        check_attn(_LIB.bpt_vector_spmm_forward(plan.ref, _ptr(edata), _ptr(x), _ptr(y), _ptr(ws), nws, h, d, dt, _stream()),
+        ref = _spmm_ref(plan, x, h, d) if n_rows is None else plan.ref
+        check_attn(_LIB.bpt_vector_spmm_forward(ref, _ptr(edata), _ptr(x), _ptr(y), _ptr(ws), nws, h, d, dt, _stream()),
                    "vector_spmm_forward")
     return y
 
@@ -214,7 +224,7 @@ def vector_spmm_backward(row, indptr, eid, indices, col, indptr_t, eid_t, indice
     dt = _dtype(x)
     ws, nws = _workspace(OP_SPMM_BWD, plan, plan_t, h, d, dt, x.device)
     with torch.cuda.device_of(x):
-        check_attn(_LIB.bpt_vector_spmm_backward(plan.ref, plan_t.ref, _ptr(edata), _ptr(dy), _ptr(x), _ptr(dedata), _ptr(dx),
+        check_attn(_LIB.bpt_vector_spmm_backward(_spmm_ref(plan, x, h, d), _spmm_ref(plan_t, x, h, d), _ptr(edata), _ptr(dy), _ptr(x), _ptr(dedata), _ptr(dx),
                                                  _ptr(ws), nws, h, d, dt, _stream()), "vector_spmm_backward")
     return [dedata, dx]
 
@@ -335,6 +345,7 @@ def attention_dropout_mask(col, indptr_c, eid_c, indices_c, q, k, dropout_p, see
 
 
 _USE_GROUPS = True
+_GROUPED_OPS = True         # row groups also in the unfused SpMM / SDDMM ops (set_grouped_ops)
 _GROUP_ROWS = None          # None: chosen per call from dtype and shape
 
 
@@ -374,6 +385,14 @@ def set_row_groups(on):
     """Fused attention: let one wavefront own several rows that share neighbours (default) or one row each."""
     global _USE_GROUPS
     old, _USE_GROUPS = _USE_GROUPS, bool(on)
+    return old
+
+
+def set_grouped_ops(on):
+    """Testing / measurement hook: let the unfused SpMM- and SDDMM-shaped ops (masked_mm and vector_spmm, forward and
+    backward) use the row groups (default) or one wavefront per row.  Returns the old setting."""
+    global _GROUPED_OPS
+    old, _GROUPED_OPS = _GROUPED_OPS, bool(on)
     return old
 
 

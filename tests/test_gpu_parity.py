@@ -142,16 +142,21 @@ def close(got, want, tol, what, terms=1):
 SHAPES = [(8, 64), (1, 40), (3, 20), (4, 64)]   # (8,64)/(4,64) have specialised kernels, the others are generic
 
 
-@pytest.mark.parametrize("force_generic", [False, True])
+@pytest.mark.parametrize("kernels", ["groups-4", "groups-8", "rows", "generic"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
 @pytest.mark.parametrize("hd", SHAPES)
 @pytest.mark.parametrize("gname,chunk", [("blocks8x30", 32), ("blocks8x30", 7), ("bpt512_k4", 32), ("multigraph", 8), ("fc_w100", 32),
                                          ("bpt256_k24", 32)])
-def test_ops_match_oracle(ops, gname, chunk, hd, dtype, force_generic):
+def test_ops_match_oracle(ops, gname, chunk, hd, dtype, kernels):
+    """kernels: which family the SpMM / SDDMM ops run in: row groups of 4 or 8 rows, one wavefront per row
+    (specialised shapes), or the shape-generic kernels."""
     graphop, _ = ops
     h, d = hd
-    if force_generic and (hd not in ((8, 64), (4, 64)) or dtype == torch.float64):
+    force_generic = kernels == "generic"
+    if kernels != "groups-4" and (hd not in ((8, 64), (4, 64)) or dtype == torch.float64):
         pytest.skip("already generic")
+    if kernels != "groups-4" and dtype == torch.bfloat16 and hd == (4, 64):
+        pytest.skip("no specialised bfloat16 kernels for this shape")
     c = case(gname, chunk)
     n, E = c.n, c.E
     A = rand((n, h, d), dtype, 1, 0.5).to(DEV)
@@ -161,6 +166,8 @@ def test_ops_match_oracle(ops, gname, chunk, hd, dtype, force_generic):
     Be = rand((E, d), dtype, 5, 0.5).to(DEV)
     tol, gtol = TOL[dtype], GTOL[dtype]
     graphop.set_force_generic(force_generic)
+    old_grouped = graphop.set_grouped_ops(kernels.startswith("groups"))
+    old_rows = graphop.set_group_rows(8 if kernels == "groups-8" else 4)
     ctx = long_items(gname)
     ctx.__enter__()
     try:
@@ -190,6 +197,8 @@ def test_ops_match_oracle(ops, gname, chunk, hd, dtype, force_generic):
         close(dAn, rAn, gtol, "node_mul_edge dA", c.max_deg); close(dBe, rBe, gtol, "node_mul_edge dB")
     finally:
         graphop.set_force_generic(False)
+        graphop.set_grouped_ops(old_grouped)
+        graphop.set_group_rows(old_rows)
         ctx.__exit__()
 
 
