@@ -453,11 +453,19 @@ __global__ void k_entry_fill(const uint64_t *skey, const int32_t *rank, const in
     atomicOr(&ent_mask[u], 1 << (int)(k & 15));
 }
 
-__global__ void k_entry_keys(const int32_t *ent_g, const int32_t *ent_mask, int64_t n_edges, const int32_t *ginfo,
-                             uint64_t *ekey) {
+// sort keys of the entries inside their groups.  mode 1: by member mask, larger first; mode 2: by (neighbour mod 16,
+// neighbour), which spreads a group's walk over the id range the same way in every group, so that groups running
+// side by side ask for a shared row at about the same step
+__global__ void k_entry_keys(const int32_t *ent_g, const int32_t *ent_mask, const int32_t *ent_idx, int64_t n_edges,
+                             const int32_t *ginfo, int mode, uint64_t *ekey) {
     const int64_t u = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (u >= n_edges) return;
-    ekey[u] = (u < ginfo[BPT_GI_N_ENTRIES]) ? (((uint64_t)(uint32_t)ent_g[u] << 16) | (uint64_t)(0xFFFF ^ ent_mask[u])) : PAD64;
+    uint64_t k = PAD64;
+    if (u < ginfo[BPT_GI_N_ENTRIES]) {
+        const uint64_t g = (uint64_t)(uint32_t)ent_g[u], x = (uint64_t)(uint32_t)ent_idx[u];
+        k = (mode == 1) ? ((g << 16) | (uint64_t)(0xFFFF ^ ent_mask[u])) : ((g << 35) | ((x & 15) << 31) | x);
+    }
+    ekey[u] = k;
 }
 
 __global__ void k_popcounts(const int32_t *ent_mask, const int32_t *perm, int64_t n_edges, const int32_t *ginfo, int32_t *pop) {
@@ -760,7 +768,7 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
     if (max_items < 0 || n_edges < 0 || n_index_nodes < 0 || max_items >= INT32_MAX || n_edges >= INT32_MAX ||
         n_index_nodes >= INT32_MAX)
         return BPT_ERR_SIZE;
-    if (R < 1 || R > 16 || seg_len < 1) return BPT_ERR_SHAPE;
+    if (R < 1 || R > 16 || seg_len < 1 || by_mask < 0 || by_mask > 2) return BPT_ERR_SHAPE;
     if ((int64_t)R * seg_len + FIXED_WORK > 0xFFFF) return BPT_ERR_UNSUPPORTED;       // the work of a group is a 16-bit sort key
     if ((n_edges + 8) * R >= INT32_MAX) return BPT_ERR_SIZE;
     if (!plan_info || !grp_ptr || !entries || !grp_eids || !chunks || !group_info || !workspace) return BPT_ERR_NULL;
@@ -828,10 +836,11 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
     // entry order inside a group: neighbour order, or by member mask (larger first, neighbour order inside a mask)
     int32_t *perm = w.iota;                               // new position -> entry as numbered above
     LAUNCH(k_iota_i32, n_edges, w.iota, n_edges);
-    if (by_mask && n_edges > 0) {
-        LAUNCH(k_entry_keys, n_edges, w.ent_g, w.ent_mask, n_edges, group_info, w.ekey);
+    if (by_mask != 0 && n_edges > 0) {
+        LAUNCH(k_entry_keys, n_edges, w.ent_g, w.ent_mask, w.ent_idx, n_edges, group_info, (int)by_mask, w.ekey);
         tb = tmp;
-        HIP_TRY(sort_pairs<uint64_t>(w.tmp, tb, w.ekey, w.mkey_s, w.iota, w.eval, n_edges, 16 + bits_for((uint64_t)max_groups), s));
+        HIP_TRY(sort_pairs<uint64_t>(w.tmp, tb, w.ekey, w.mkey_s, w.iota, w.eval, n_edges,
+                                     (by_mask == 1 ? 16 : 35) + bits_for((uint64_t)max_groups), s));
         perm = w.eval;
     }
     LAUNCH(k_invert, n_edges, perm, group_info, (int)BPT_GI_N_ENTRIES, n_edges, w.newpos);

@@ -310,9 +310,10 @@ class DevicePlan:
 
     def ensure_groups(self, R=GROUP_R, order_mode=None):
         """Row groups of R rows built on the GPU (bpt_plan_group_device).  Of order_mode only the entry order counts:
-        by member mask (+4) or ascending neighbour (the aligned order of the host builder has no parallel form)."""
+        by member mask (+4), or for the aligned order of the host builder (+8), which is sequential by construction, its
+        parallel stand-in (entries by neighbour id mod 16, then id); else ascending neighbour."""
         order_mode = GROUP_ORDER if order_mode is None else order_mode
-        by_mask = bool(order_mode & 4) and not (order_mode & 8)
+        by_mask = 2 if order_mode & 8 else (1 if order_mode & 4 else 0)
         with self._lock:
             hit = self._groups.get((R, by_mask))
             if hit is None:

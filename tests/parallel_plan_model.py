@@ -61,7 +61,8 @@ def item_keys(items, idx32, n_index, red):
 
 def group_plan(arrays, n_index, R, by_mask):
     """Row groups: the items in the order of their largest neighbour, R consecutive ones per group; the groups
-    numbered by locality (smallest neighbour), cut into 8 ranges of equal work, by decreasing work inside a range."""
+    numbered by locality (smallest neighbour), cut into 8 ranges of equal work, by decreasing work inside a range.
+    by_mask: entry order inside a group: 0 / False ascending neighbour, 1 / True by member mask, 2 interleaved."""
     items, idx32, eid32 = arrays["items"], arrays["idx"], arrays["eid"]
     n_items, E = len(items), len(eid32)
     kmax = item_keys(items, idx32, n_index, np.max)
@@ -119,8 +120,11 @@ def group_plan(arrays, n_index, R, by_mask):
     ent_g[u] = skey >> 35
     np.bitwise_or.at(mask, u, 1 << mem)
     slot_eid[u, mem] = eid32[order]
-    if by_mask:
+    if int(by_mask) == 1:        # by member mask, larger first
         perm = np.argsort((ent_g << 16) | (0xFFFF ^ mask), kind="stable")
+        ent_idx, ent_g, mask, slot_eid = ent_idx[perm], ent_g[perm], mask[perm], slot_eid[perm]
+    elif int(by_mask) == 2:      # by (neighbour mod 16, neighbour): groups that share rows read them at about the same step
+        perm = np.argsort((ent_g << 35) | ((ent_idx & 15) << 31) | ent_idx, kind="stable")
         ent_idx, ent_g, mask, slot_eid = ent_idx[perm], ent_g[perm], mask[perm], slot_eid[perm]
     grp_ptr = np.searchsorted(ent_g, np.arange(ng + 1), side="left").astype(np.int32)
     pop = np.array([bin(int(m)).count("1") for m in mask], dtype=np.int64)

@@ -106,8 +106,8 @@ def test_device_plan_equals_model_and_host(name, seg):
         plans.append((dp, arrays))
     for R in (4, 8, 16):
         grps = []
-        for (dp, arrays), by_mask in zip(plans, (True, False)):
-            hit = dp.ensure_groups(R, 6 if by_mask else 10)
+        for (dp, arrays), by_mask in zip(plans, (1, 2) if R != 16 else (0, 0)):
+            hit = dp.ensure_groups(R, {0: 2, 1: 6, 2: 10}[by_mask])
             grp = model.group_plan(arrays, n, R, by_mask)
             check_groups(hit, grp, len(src))
             grps.append(grp)
@@ -201,7 +201,8 @@ def test_fused_attention_on_device_plans_matches_oracle(device_plans, gname, dty
 
 def test_ops_and_rel_pos_on_device_plans_match_host_plans(device_plans):
     """The unfused ops and the fused path with rel_pos and dropout give the same results on device-built plans as on
-    host-built ones (the ops bit for bit: their base plans are identical)."""
+    host-built ones: edge outputs bit for bit (a dot product or a row's softmax does not depend on the grouping), row
+    sums up to their order of summation."""
     from bpt_amd import graphop, op, plan
     c = Case("bpt512_k4")
     h, d = 8, 64
@@ -226,9 +227,9 @@ def test_ops_and_rel_pos_on_device_plans_match_host_plans(device_plans):
     plan.plan_cache.clear()
     hst = run()
     assert isinstance(plan.plan_cache.get(*c.inn, c.n, c.n), plan.Plan)
-    for i in range(3):
+    for i in range(2):
         assert torch.equal(dev[i], hst[i])
-    for got, want in zip(dev[3:], hst[3:]):
+    for got, want in zip(dev[2:], hst[2:]):
         assert torch.allclose(got, want, rtol=1e-4, atol=1e-5)
 
 
@@ -251,10 +252,10 @@ def test_device_plan_at_headline_size_and_its_build_time():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
     print(f"device plan build (both sides, groups of 8, pair mapping) at cfg 3: {dt * 1e3:.2f} ms")
-    for dp, arrs, by_mask in ((pin, a_in, True), (pout, a_out, False)):
+    for dp, arrs, by_mask in ((pin, a_in, 1), (pout, a_out, 2)):
         arrays, info = model.base_plan(*arrs, n, n, 64)
         check_base(dp, arrays, info)
-        check_groups(dp.ensure_groups(8, 6 if by_mask else 10), model.group_plan(arrays, n, 8, by_mask), len(src))
+        check_groups(dp.ensure_groups(8, {0: 2, 1: 6, 2: 10}[by_mask]), model.group_plan(arrays, n, 8, by_mask), len(src))
 
 
 @pytest.mark.parametrize("chunk", [4, 32])
@@ -327,15 +328,15 @@ def test_device_plan_on_random_graphs(seed):
         assert np.array_equal(host(a), b)
     out_csr, in_csr, ROW, IR, COL, IC = got
     w_out, w_in = want[0], want[1]
-    sides_ = (((COL, IC, in_csr[2], in_csr[1]), (want[4], want[5], w_in[2], w_in[1]), True),
-              ((ROW, IR, out_csr[2], out_csr[1]), (want[2], want[3], w_out[2], w_out[1]), False))
+    sides_ = (((COL, IC, in_csr[2], in_csr[1]), (want[4], want[5], w_in[2], w_in[1]), 1),
+              ((ROW, IR, out_csr[2], out_csr[1]), (want[2], want[3], w_out[2], w_out[1]), 2))
     plans, grps = [], []
     for tens, arrs, by_mask in sides_:
         dp = DevicePlan(*tens, n, n, DEV, seg)
         arrays, info = model.base_plan(*arrs, n, n, seg)
         check_base(dp, arrays, info)
         grp = model.group_plan(arrays, n, R, by_mask)
-        check_groups(dp.ensure_groups(R, 6 if by_mask else 10), grp, E)
+        check_groups(dp.ensure_groups(R, {0: 2, 1: 6, 2: 10}[by_mask]), grp, E)
         plans.append(dp); grps.append(grp)
     plans[0].linked_to(plans[1], R)
     assert np.array_equal(host(plans[0]._links[(id(plans[1]), R)][1]), model.link_groups(grps[0], grps[1], E, GROUP_PAD_ENTRIES))

@@ -30,7 +30,7 @@ def test_model_base_plan_equals_host_plan(name, seg):
 
 
 @pytest.mark.parametrize("R", [4, 8, 16])
-@pytest.mark.parametrize("by_mask", [False, True])
+@pytest.mark.parametrize("by_mask", [0, 1, 2])
 @pytest.mark.parametrize("seg", [8, 64])
 @pytest.mark.parametrize("name", sorted(GRAPHS))
 def test_model_group_plan_invariants(name, seg, by_mask, R):
@@ -38,7 +38,7 @@ def test_model_group_plan_invariants(name, seg, by_mask, R):
     for (row, ip, eid, idx), rows_of, cols_of in ((a_in, dst, src), (a_out, src, dst)):
         arrays, _ = model.base_plan(row, ip, eid, idx, n, n, seg)
         grp = model.group_plan(arrays, n, R, by_mask)
-        check_group_invariants(arrays, grp, rows_of, cols_of, len(src), R, by_mask)
+        check_group_invariants(arrays, grp, rows_of, cols_of, len(src), R, by_mask == 1)
 
 
 @pytest.mark.parametrize("name,seg,R", [("bpt64c", 64, 4), ("bpt37", 8, 8), ("multi", 8, 4), ("bpt300c", 64, 8)])
@@ -46,7 +46,7 @@ def test_model_group_walk_matches_oracle(name, seg, R):
     src, dst, n, csr, a_in, a_out = sides(name, seg)
     pin, _ = model.base_plan(*a_in, n, n, seg)
     pout, _ = model.base_plan(*a_out, n, n, seg)
-    gin, gout = model.group_plan(pin, n, R, True), model.group_plan(pout, n, R, False)
+    gin, gout = model.group_plan(pin, n, R, 1), model.group_plan(pout, n, R, 2)
     check_emulated_walks(src, dst, n, csr, pin, gin, gout, model.link_groups(gin, gout, len(src), GROUP_PAD_ENTRIES))
 
 
