@@ -107,8 +107,9 @@ def main():
     ap.add_argument("--dropout", type=float, default=0.0, help="dropout on the attention probabilities inside the fused kernels (attention.py:73)")
     ap.add_argument("--rel-pos", action="store_true",
                     help="add the relative-position score term q[dst].table[etype[e]] (table (1000, d_head), modules/attention.py:23,42,69-71)")
-    ap.add_argument("--device-plan", action="store_true",
-                    help="build the launch plans and row groups on the GPU (libbptplan) instead of on the host")
+    ap.add_argument("--plan", default="auto", choices=["auto", "host", "device"],
+                    help="where launch plans and row groups are built: on the host (libbptgraph), on the GPU (libbptplan), "
+                         "or by graph size (the library's default: on the GPU from 24576 rows)")
     ap.add_argument("--block-layers", type=int, default=0,
                     help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the workload's graph")
     args = ap.parse_args()
@@ -126,7 +127,7 @@ def main():
     graphop.set_row_groups(not args.rows)
     graphop.set_group_rows(args.group_rows)
     from bpt_amd import plan as plan_mod
-    plan_mod.set_device_build(args.device_plan)
+    plan_mod.set_device_build({"auto": None, "host": False, "device": True}[args.plan])
     desc, graphs, H, D, default_dtype = make_workload(args.workload)
     dtype_name = args.dtype or default_dtype
     tdtype = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
@@ -199,7 +200,7 @@ def main():
             pin.linked_to(pout, graphop._group_rows(q, H, D, pin))
             torch.cuda.synchronize()
             ts.append(time.perf_counter() - t0)
-        plan_build = {"where": "device" if args.device_plan else "host", "ms": round(min(ts) * 1e3, 3)}
+        plan_build = {"where": "device" if isinstance(pin, plan_mod.DevicePlan) else "host", "ms": round(min(ts) * 1e3, 3)}
         log(f"plan build: {plan_build}")
         ref = step()
         torch.cuda.synchronize()
