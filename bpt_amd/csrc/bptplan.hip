@@ -215,7 +215,7 @@ __global__ void k_narrow(const int64_t *eid, const int64_t *indices, int64_t n_e
 // clipped to n_index_nodes.  Positions past n_items get the padding key, which sorts behind every real one.
 template <bool LARGEST>
 __global__ void k_item_keys(const int32_t *items, const int32_t *idx32, const int32_t *info, int64_t max_items,
-                            int64_t n_index_nodes, uint32_t *key) {
+                            int64_t n_index_nodes, int64_t n_edges, uint32_t *key) {
     const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= max_items) return;
     if (info[BPT_PI_ERR] || i >= info[BPT_PI_N_ITEMS]) {
@@ -223,8 +223,8 @@ __global__ void k_item_keys(const int32_t *items, const int32_t *idx32, const in
         return;
     }
     const int4 it = reinterpret_cast<const int4 *>(items)[i];
-    int32_t k = it.x < n_index_nodes ? it.x : (int32_t)n_index_nodes;
-    if (it.z > it.y) {
+    int32_t k = (it.x >= 0 && it.x < n_index_nodes) ? it.x : (int32_t)n_index_nodes;
+    if (it.z > it.y && it.y >= 0 && it.z <= n_edges) {          // (an item list from elsewhere is not trusted with addresses)
         k = idx32[it.y];
         for (int32_t p = it.y + 1; p < it.z; ++p) k = LARGEST ? max(k, idx32[p]) : min(k, idx32[p]);
     }
@@ -380,8 +380,8 @@ __global__ void k_invert(const int32_t *order, const int32_t *count, int idx_of_
 
 // members of the groups in their final order, and one sort record per edge slot
 __global__ void k_members_and_records(const int32_t *items, const int32_t *idx32, const int32_t *jorder, const int32_t *lpos,
-                                      const int32_t *inv, const int32_t *pinfo, int64_t max_groups, int32_t R, int32_t *members, uint64_t *ekey,
-                                      int32_t *eval) {
+                                      const int32_t *inv, const int32_t *pinfo, int64_t max_groups, int64_t n_edges, int32_t R,
+                                      int32_t *members, uint64_t *ekey, int32_t *eval) {
     const int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (j >= max_groups * R) return;
     const int32_t ng = n_groups_of(pinfo, R), n_items = pinfo[BPT_PI_N_ITEMS];
@@ -398,7 +398,8 @@ __global__ void k_members_and_records(const int32_t *items, const int32_t *idx32
     const int4 it = reinterpret_cast<const int4 *>(items)[jorder[j]];
     mem[0] = it.x;
     mem[1] = it.w;
-    for (int32_t p = it.y; p < it.z; ++p) {
+    const int32_t p_end = it.z < n_edges ? it.z : (int32_t)n_edges;
+    for (int32_t p = it.y > 0 ? it.y : 0; p < p_end; ++p) {
         ekey[p] = ((uint64_t)(uint32_t)gi << 35) | ((uint64_t)(uint32_t)idx32[p] << 4) | (uint64_t)m;
         eval[p] = p;
     }
@@ -502,6 +503,7 @@ __global__ void k_edge_ids(const uint64_t *skey, const int32_t *slot_of, const i
     const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (i >= n_edges || !plan_usable(pinfo)) return;
     const int32_t m = (int32_t)(skey[i] & 15), old = ent_of[i], u = newpos[old];
+    if (m >= R) return;                                   // (only with an item list that does not cover the edge slots)
     const int32_t e = eid32[slot_of[i]];
     grp_eids[(int64_t)u * R + m] = e;
     pair_eid[first[u] + __popc((uint32_t)ent_mask[old] & ((1u << m) - 1u))] = e;
@@ -750,7 +752,7 @@ int bpt_plan_build_device(const int64_t *row, const int64_t *indptr_units, int64
         LAUNCH(k_iota_i32, max_items, w.iota, max_items);
         const int32_t *perm = w.iota;
         if (indices) {
-            LAUNCH(k_item_keys<false>, max_items, w.items_tmp, idx32, info, max_items, n_index_nodes, w.key);
+            LAUNCH(k_item_keys<false>, max_items, w.items_tmp, idx32, info, max_items, n_index_nodes, n_edges, w.key);
             tb = tmp;
             HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key, w.key_s, w.iota, w.perm, max_items, 32, s));
             perm = w.perm;
@@ -788,14 +790,14 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
 
     // the items in the order of their largest neighbour; R consecutive ones are a group
     if (max_items > 0) {
-        LAUNCH(k_item_keys<true>, max_items, items, idx32, plan_info, max_items, n_index_nodes, w.key);
+        LAUNCH(k_item_keys<true>, max_items, items, idx32, plan_info, max_items, n_index_nodes, n_edges, w.key);
         LAUNCH(k_iota_i32, max_items, w.iota, max_items);
         tb = tmp;
         HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key, w.key_s, w.iota, w.jorder, max_items, 32, s));
     }
     // the groups numbered by locality (smallest neighbour id), cut into 8 ranges of equal work, by decreasing work
     // inside a range
-    if (max_items > 0) LAUNCH(k_item_keys<false>, max_items, items, idx32, plan_info, max_items, n_index_nodes, w.key);
+    if (max_items > 0) LAUNCH(k_item_keys<false>, max_items, items, idx32, plan_info, max_items, n_index_nodes, n_edges, w.key);
     LAUNCH(k_group_work, max_groups + 1, items, w.jorder, w.key, plan_info, max_groups, R, w.work0, w.key_s, group_info);
     if (max_groups > 0) {
         LAUNCH(k_iota_i32, max_groups, w.iota, max_groups);
@@ -813,7 +815,7 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
         tb = tmp;
         HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key_s, w.key, w.iota, w.gorder, max_groups, 32, s));
         LAUNCH(k_invert, max_groups, w.gorder, group_info, (int)BPT_GI_N_GROUPS, max_groups, w.inv);
-        LAUNCH(k_members_and_records, max_groups * R, items, idx32, w.jorder, w.lpos, w.inv, plan_info, max_groups, R, members,
+        LAUNCH(k_members_and_records, max_groups * R, items, idx32, w.jorder, w.lpos, w.inv, plan_info, max_groups, n_edges, R, members,
                w.ekey, w.eval);
     }
     // entries: distinct (group, neighbour, multiplicity) of the records sorted by (group, neighbour, member)
