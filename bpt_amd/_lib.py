@@ -67,6 +67,8 @@ ATTN_API = {
 c_i32 = ctypes.c_int32
 # libbptplan (include/bptplan.h): plans built on the GPU
 PLAN_API = {
+    "bpt_graph_count_device": (ctypes.c_int, [ctypes.c_int, c_i64, ctypes.c_int, c_i64, c_i64, c_vp, c_vp, c_i64, c_vp]),
+    "bpt_graph_fill_device": (ctypes.c_int, [ctypes.c_int, c_i64, ctypes.c_int, c_i64, c_i64, c_i64, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp]),
     "bpt_csr_device_bounds": (ctypes.c_int, [c_i64, c_i64, c_i32, ctypes.POINTER(c_i64 * 2)]),
     "bpt_csr_build_device": (ctypes.c_int, [c_vp, c_vp, c_i64, c_i64, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp]),
     "bpt_plan_device_bounds": (ctypes.c_int, [c_i64, c_i64, c_i64, c_i32, c_i32, ctypes.POINTER(c_i64 * 4)]),

@@ -531,6 +531,121 @@ __global__ void k_pairs(const int32_t *eids_dst, const int32_t *ginfo_dst, int32
     pairs[j] = out;
 }
 
+// ---- edge lists of the reference's graph builder --------------------------------------------------------------------
+// builder.pyx:41-116 (binary partition), :243-274 (fully connected), :171-199 (strided sparse) emit the edges token by
+// token, so one thread walks one token: a first pass counts its edges, a prefix sum gives every token its place in
+// the list, a second pass writes them there — the same list, in the same order, as the host walk (bptgraph.cpp).
+constexpr int MAX_LEVELS = 48;
+struct LevelTable {
+    int64_t size[MAX_LEVELS], offset[MAX_LEVELS];
+    int n;
+};
+
+struct EdgeCount {
+    int64_t n = 0;
+    __device__ void operator()(int64_t, int64_t, int64_t) { ++n; }
+};
+struct EdgeWrite {
+    int64_t *src, *dst, *etype;
+    int64_t shift, at;
+    __device__ void operator()(int64_t s, int64_t d, int64_t t) {
+        src[at] = s + shift;
+        dst[at] = d + shift;
+        etype[at] = t;
+        ++at;
+    }
+};
+
+// One token of builder.pyx:64-116: two cursors walk outwards, `step` nodes per side per level, then move one level
+// up; a cursor that stops on a node whose sibling was taken continues with that child on the next level (the
+// right-hand bound is checked against the current level even then, as the reference does).
+template <class Sink>
+__device__ void token_binary_partition(const LevelTable &lv, int64_t tok, bool causal, int64_t step, int64_t clip, Sink &out) {
+    int64_t left = tok - 1, right = tok + 1, ancestor = tok;
+    bool left_child = false, right_child = false;
+    for (int j = 0; j < lv.n; ++j) {
+        const int64_t type0 = (2 * step + 1) * (j < clip ? j : clip);
+        for (int64_t s = 0; s < step; ++s) {
+            if (!causal && right < lv.size[j]) {
+                out(right_child ? lv.offset[j - 1] + 2 * right + 1 : lv.offset[j] + right, tok, type0 + 2 * (s + 1));
+                right_child = false;
+            }
+            ++right;
+            if (left >= 0) {
+                out(left_child ? lv.offset[j - 1] + 2 * left : lv.offset[j] + left, tok, type0 + 2 * s + 1);
+                left_child = false;
+            }
+            --left;
+        }
+        if ((left & 1) == 0) left_child = true;
+        if ((right & 1) == 1) right_child = true;
+        right >>= 1;
+        left >>= 1;                           // arithmetic shift: stays negative once it is
+        out(tok, lv.offset[j] + ancestor, type0);
+        ancestor >>= 1;
+    }
+}
+
+template <class Sink>
+__device__ void token_edges(int kind, const LevelTable &lv, int64_t length, int64_t i, bool causal, int64_t a, int64_t b, Sink &out) {
+    if (kind == 0) {
+        token_binary_partition(lv, i, causal, a, b, out);
+    } else if (kind == 1) {                   // builder.pyx:243-274: a = window
+        const int64_t reach = length < a + 1 ? length : a + 1;
+        out(i, i, 0);
+        for (int64_t j = 1; j < reach; ++j) {
+            if (i >= j) out(i - j, i, 2 * j - 1);
+            if (!causal && i + j < length) out(i + j, i, 2 * j);
+        }
+        out(i, length, 0);
+    } else {                                  // builder.pyx:171-199: a = stride, b = c
+        for (int64_t j = (i / a) * a; j <= i; ++j) out(j, i, 0);
+        for (int64_t blk = 1; blk <= i / a; ++blk)
+            for (int64_t k = a * blk - b; k < a * blk; ++k) out(k, i, 0);
+        out(i, length, 0);
+    }
+}
+
+__global__ void k_graph_count(int kind, LevelTable lv, int64_t length, int causal, int64_t a, int64_t b, int32_t *counts) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i > length) return;
+    EdgeCount c;
+    if (i < length) token_edges(kind, lv, length, i, causal != 0, a, b, c);
+    counts[i] = (int32_t)c.n;
+}
+
+__global__ void k_graph_fill(int kind, LevelTable lv, int64_t length, int causal, int64_t a, int64_t b, int64_t shift,
+                             const int32_t *offsets, int64_t n_edges, int64_t *src, int64_t *dst, int64_t *etype) {
+    const int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (i >= length || offsets[length] != n_edges) return;     // the caller's edge count must be the list's
+    EdgeWrite w{src, dst, etype, shift, offsets[i]};
+    token_edges(kind, lv, length, i, causal != 0, a, b, w);
+}
+
+bool level_table(int kind, int64_t length, LevelTable &lv) {
+    lv.n = 0;
+    if (kind != 0) return true;
+    int64_t n = length, nodes = 0;
+    while (n >= 2) {
+        if (lv.n >= MAX_LEVELS - 1) return false;
+        lv.size[lv.n] = n;
+        lv.offset[lv.n++] = nodes;
+        nodes += n;
+        n = (n + 1) >> 1;
+    }
+    lv.size[lv.n] = 1;
+    lv.offset[lv.n++] = nodes;
+    return true;
+}
+
+bool graph_args_ok(int kind, int64_t length, int64_t a, int64_t b) {
+    if (length < 1 || length >= INT32_MAX) return false;
+    if (kind == 0) return a >= 1 && b >= 0;
+    if (kind == 1) return a >= 0;
+    if (kind == 2) return a >= 1 && b >= 0 && b <= a;
+    return false;
+}
+
 // ---- CSR of an edge list ------------------------------------------------------------------------------------------------
 __global__ void k_csr_keys(const int64_t *rows, const int64_t *cols, int64_t n_edges, int64_t n_nodes, int32_t *info,
                            uint32_t *key, int32_t *val) {
@@ -643,6 +758,36 @@ int sizes_ok(int64_t n_units, int64_t n_edges, int64_t n_rows, int64_t n_index_n
 }  // namespace
 
 extern "C" {
+
+int bpt_graph_count_device(int kind, int64_t length, int triu, int64_t a, int64_t b, int32_t *offsets, void *workspace,
+                           int64_t workspace_bytes, void *stream) {
+    if (!graph_args_ok(kind, length, a, b)) return BPT_ERR_SIZE;
+    if (!offsets || !workspace) return BPT_ERR_NULL;
+    LevelTable lv;
+    if (!level_table(kind, length, lv)) return BPT_ERR_SIZE;
+    size_t tmp = 0, tb = 0;
+    HIP_TRY(scan_i32(nullptr, tmp, nullptr, nullptr, length + 1, nullptr));
+    Bump bump{(char *)workspace, 0};
+    int32_t *counts = bump.take<int32_t>(length + 1);
+    void *scratch = bump.take<char>((int64_t)tmp + 256);
+    if (workspace_bytes < (int64_t)bump.off) return BPT_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    LAUNCH(k_graph_count, length + 1, kind, lv, length, triu, a, b, counts);
+    tb = tmp + 256;
+    HIP_TRY(scan_i32(scratch, tb, counts, offsets, length + 1, s));
+    return BPT_OK;
+}
+
+int bpt_graph_fill_device(int kind, int64_t length, int triu, int64_t a, int64_t b, int64_t v_shift, const int32_t *offsets,
+                          int64_t n_edges, int64_t *src, int64_t *dst, int64_t *etype, void *stream) {
+    if (!graph_args_ok(kind, length, a, b) || n_edges < 0) return BPT_ERR_SIZE;
+    if (!offsets || (n_edges > 0 && (!src || !dst || !etype))) return BPT_ERR_NULL;
+    LevelTable lv;
+    if (!level_table(kind, length, lv)) return BPT_ERR_SIZE;
+    hipStream_t s = (hipStream_t)stream;
+    LAUNCH(k_graph_fill, length, kind, lv, length, triu, a, b, v_shift, offsets, n_edges, src, dst, etype);
+    return BPT_OK;
+}
 
 int bpt_csr_device_bounds(int64_t n_edges, int64_t n_nodes, int32_t chunk_size, int64_t bounds[2]) {
     if (!bounds) return BPT_ERR_NULL;

@@ -59,6 +59,31 @@ class _Graph:
                                                 _ptr(src), _ptr(dst), _ptr(et), None, None))
         return src, dst, et
 
+    def get_edges_device(self, device, v_shift=0):
+        """get_edges built on the GPU (libbptplan: one thread per token, count / prefix sum / write): int64 device
+        tensors (src, dst, etype), bit for bit the arrays of get_edges.  One synchronisation (the edge count)."""
+        import torch
+        from ._lib import plan_lib
+        lib, device = plan_lib(), torch.device(device)
+        L = self._length
+        offsets = torch.empty(L + 1, dtype=torch.int32, device=device)
+        ws = torch.empty(8 * (L + 1) + (1 << 20), dtype=torch.uint8, device=device)
+        with torch.cuda.device(device):
+            stream = torch.cuda.current_stream().cuda_stream
+            st = lib.bpt_graph_count_device(self._kind, L, int(self._triu), self._a, self._b, offsets.data_ptr(),
+                                            ws.data_ptr(), ws.numel(), stream)
+            if st != 0:
+                raise RuntimeError(f"bpt_graph_count_device: status {st}")
+            n_edges = int(offsets[L])
+            if n_edges != self._n_edges:
+                raise RuntimeError("device and host edge counts differ")
+            src, dst, et = (torch.empty(n_edges, dtype=torch.int64, device=device) for _ in range(3))
+            st = lib.bpt_graph_fill_device(self._kind, L, int(self._triu), self._a, self._b, int(v_shift),
+                                           offsets.data_ptr(), n_edges, src.data_ptr(), dst.data_ptr(), et.data_ptr(), stream)
+            if st != 0:
+                raise RuntimeError(f"bpt_graph_fill_device: status {st}")
+        return src, dst, et
+
     # builder.pyx:142-149
     def leaf_ids(self, v_shift=0, start=0):
         return np.arange(v_shift + start, v_shift + self._length)
@@ -226,7 +251,7 @@ def merge_graphs_device(graphs, device):
         if hit is None:
             if len(_DEVICE_EDGES) >= _DEVICE_EDGES_MAX:
                 _DEVICE_EDGES.clear()
-            hit = tuple(torch.from_numpy(a).to(device) for a in (*g.get_edges(), g.get_pos()))
+            hit = (*g.get_edges_device(device), torch.from_numpy(g.get_pos()).to(device))
             _DEVICE_EDGES[key] = hit
         parts.append(hit)
         shifts.append(v_shift)

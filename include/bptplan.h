@@ -29,6 +29,19 @@ enum { BPT_PI_ERR = 0,        /* 0 ok, 1 id out of range, 2 row / indptr not mon
 /* indices into the int32[16] info block of bpt_plan_group_device */
 enum { BPT_GI_N_GROUPS = 0, BPT_GI_N_ENTRIES = 1, BPT_GI_MAX_CHUNK = 2 };
 
+/* Edge lists of the reference's graph builder on the device, in the reference's order (kind 0: BinaryPartition,
+ * builder.pyx:41-116, a = step, b = clip_dist; 1: FullyConnected, :243-274, a = window; 2: OpenAISparse, :171-199,
+ * a = stride, b = c; same arguments as bptg_graph_fill, bptgraph.h).  Two calls: bpt_graph_count_device writes
+ * offsets (length + 1 int32: offsets[i] = position of token i's first edge, offsets[length] = number of edges; the
+ * caller reads that one number to size the lists; workspace: 8 * (length + 1) bytes + 1 MiB are enough), then
+ * bpt_graph_fill_device writes src / dst (+ v_shift) and etype (n_edges int64 each; nothing is written unless n_edges
+ * equals offsets[length]). */
+int bpt_graph_count_device(int kind, int64_t length, int triu, int64_t a, int64_t b, int32_t *offsets, void *workspace,
+                           int64_t workspace_bytes, void *stream);
+int bpt_graph_fill_device(int kind, int64_t length, int triu, int64_t a, int64_t b, int64_t v_shift,
+                          const int32_t *offsets, int64_t n_edges, int64_t *src, int64_t *dst, int64_t *etype,
+                          void *stream);
+
 /* One CSR side of graph/base.py:71-86 from an edge list on the device: the edges grouped by rows[e], ascending edge
  * id inside a row (the order of bptg_build_csr, bptgraph.h), in the reference's int64 layout: indptr (n_nodes + 1),
  * indices (n_edges: cols of the slots), eid (n_edges); and the chunked units of builder.pyx:305-321 (partition_csr):

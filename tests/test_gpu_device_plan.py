@@ -384,3 +384,20 @@ def test_batch_merge_on_the_device_and_the_whole_pipeline_time():
         assert pin.n_edges == 573520 and pin.covers_all_edges and pout.covers_all_edges
     print(f"lengths -> plans with groups of 8 (cfg 2): host {times['host'] * 1e3:.1f} ms, device {times['device'] * 1e3:.2f} ms")
     assert times["device"] < times["host"]
+
+
+def test_device_graph_builder_equals_host_builder():
+    """Edge lists built on the GPU, bit for bit those of the host builder (itself pinned by the reference's own
+    module through tests/golden): all three graph kinds, causal and not, odd sizes, shifts."""
+    from bpt_amd import graphbuilder as gb
+    graphs = [gb.BinaryPartition(L, triu, step, clip) for L in (1, 2, 3, 5, 6, 7, 13, 33, 100, 511, 512, 1000)
+              for triu in (False, True) for step, clip in ((1, 10), (2, 3), (4, 10))]
+    graphs += [gb.BinaryPartition(8192, True, 4, 10), gb.BinaryPartition(4097, False, 8, 2)]
+    graphs += [gb.FullyConnected(L, triu, w) for L in (1, 2, 17, 260) for triu in (False, True) for w in (0, 1, 5, 8192)]
+    graphs += [gb.OpenAISparse(L, stride, c) for L, stride, c in ((1, 4, 2), (50, 8, 3), (257, 16, 16), (64, 64, 0))]
+    for i, g in enumerate(graphs):
+        shift = 7 * (i % 3)
+        want = g.get_edges(v_shift=shift)
+        got = g.get_edges_device(DEV, v_shift=shift)
+        for a, b in zip(got, want):
+            assert a.dtype == torch.int64 and np.array_equal(host(a), b), (type(g).__name__, g.__reduce__()[1])

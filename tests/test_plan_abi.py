@@ -30,8 +30,8 @@ def test_libraries_export_every_declared_symbol():
         assert hasattr(glib, name), name
     for name in a:
         assert hasattr(alib, name), name
-    p = sorted(_declared("bptplan.h", "bpt_plan_") + _declared("bptplan.h", "bpt_csr_"))
-    assert len(p) == 6
+    p = sorted(_declared("bptplan.h", "bpt_plan_") + _declared("bptplan.h", "bpt_csr_") + _declared("bptplan.h", "bpt_graph_"))
+    assert len(p) == 8
     plib = _lib.plan_lib()
     for name in p:
         assert hasattr(plib, name), name
@@ -59,6 +59,8 @@ def test_error_strings_and_argument_errors_without_gpu():
     assert plib.bpt_plan_link_device(None, None, 4, None, None, 4, 10, 8, None, None, 0, None) == -1
     assert plib.bpt_csr_device_bounds(10, 10, 0, ctypes.byref((ctypes.c_int64 * 2)())) == -4                  # chunk size
     assert plib.bpt_csr_build_device(None, None, -1, 0, 32, None, None, None, None, None, None, None, 0, None) == -2
+    assert plib.bpt_graph_count_device(0, 0, 1, 4, 10, None, None, 0, None) == -2                             # length < 1
+    assert plib.bpt_graph_fill_device(2, 8, 1, 4, 5, 0, None, 0, None, None, None, None) == -2                # c > stride
 
 
 def _bpt_csr(L, triu, step):
