@@ -1927,9 +1927,10 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 
 // y[eid, head] = <A[row, head, :], B[idx, head, :]> for every edge: the row-group form of k_sddmm_fast.  The
 // members' A rows stay in registers, B[idx] is loaded once per entry and every member that has the edge takes its
-// dot products with it; the edge id of (entry, member) comes from grp_eids.
-template <typename T, int H, int D, int R, int HS>
-__global__ __launch_bounds__(WAVE) void k_sddmm_grp(bpt_plan P, const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ y) {
+// dot products with it; the edge id of (entry, member) comes from grp_eids.  TABLE: B is a (n, D) table whose rows
+// all heads share (the rel_pos score term q[row] . table[idx], written as float32).
+template <typename T, int H, int D, int R, int HS, bool TABLE = false, typename YT = T>
+__global__ __launch_bounds__(WAVE) void k_sddmm_grp(bpt_plan P, const T *__restrict__ A, const T *__restrict__ B, YT *__restrict__ y) {
     constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
     using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, GRP_BATCH = 2;
@@ -1939,6 +1940,7 @@ __global__ __launch_bounds__(WAVE) void k_sddmm_grp(bpt_plan P, const T *__restr
     const int slice = group_slice<R, HS>(), coff = slice * HL * D;
     const int lane = threadIdx.x, head = slice * HL + lane / L::LPH;
     const uint32_t loff = (uint32_t)((coff + L::off(lane, 0)) * sizeof(T));
+    const uint32_t toff = (uint32_t)((lane % L::LPH) * L::VE * sizeof(T));      // the lane's columns inside a table row
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     const int4 *eids4 = reinterpret_cast<const int4 *>(P.grp_eids);
     float a[R][EPL];
@@ -1962,7 +1964,8 @@ __global__ __launch_bounds__(WAVE) void k_sddmm_grp(bpt_plan P, const T *__restr
                 const uint32_t src = (uint32_t)__builtin_amdgcn_readlane(ent.x, b + e);
                 Bt.mk[e] = __builtin_amdgcn_readlane(ent.y, b + e);
                 Bt.pz[e] = b + e;
-                load_row32_raw<T, HL, D, CF>(B, src, loff, Bt.br[e]);
+                if constexpr (TABLE) load_row32_raw<T, HL, D, D>(B, src, toff, Bt.br[e]);
+                else load_row32_raw<T, HL, D, CF>(B, src, loff, Bt.br[e]);
             }
         };
         auto compute = [&](const Batch &Bt) {
@@ -1977,7 +1980,7 @@ __global__ __launch_bounds__(WAVE) void k_sddmm_grp(bpt_plan P, const T *__restr
                         const int4 &x = xe[m / 4];
                         const int held = (m & 3) == 0 ? x.x : (m & 3) == 1 ? x.y : (m & 3) == 2 ? x.z : x.w;
                         const uint32_t edge = (uint32_t)__builtin_amdgcn_readlane(held, Bt.pz[e]);
-                        if (lane % L::LPH == 0) Elem<T>::st(y + (size_t)edge * H + head, s);
+                        if (lane % L::LPH == 0) Elem<YT>::st(y + (size_t)edge * H + head, s);
                     }
                 }
             }
@@ -2165,9 +2168,23 @@ int run_spmm_fast(const bpt_plan *P, const void *W0, const void *X0, void *Y0, c
 }
 
 // score term of the relative positions: bias[eid[p], head] = A[row, head, :] . table[idx[p], :], float32
+bool spmm_grp_ok(const bpt_plan *P, int h, int d, int dtype);
+template <typename T, int H, int D> constexpr int head_slices();
+inline int group_grid(const bpt_plan *P);
+
 template <typename T, int H, int D>
 int run_rel_bias(const bpt_plan *P, const void *A, const void *table, float *bias, hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
+    if (spmm_grp_ok(P, H, D, sizeof(T) == 2 ? BPT_BF16 : BPT_F32)) {      // row groups: one load of a table row per group entry
+        constexpr int HS = head_slices<T, H, D>();
+        if (P->grp_R == 8)
+            hipLaunchKernelGGL((k_sddmm_grp<T, H, D, 8, HS, true, float>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)A,
+                               (const T *)table, bias);
+        else
+            hipLaunchKernelGGL((k_sddmm_grp<T, H, D, 4, HS, true, float>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)A,
+                               (const T *)table, bias);
+        return launch_status();
+    }
     hipLaunchKernelGGL((k_sddmm_fast<T, H, D, FAST_BATCH, 2, float>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)table,
                        bias);
     return launch_status();

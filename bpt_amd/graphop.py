@@ -204,7 +204,7 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None):
     dt = _dtype(x)
     ws, nws = _workspace(OP_SPMM_FWD, plan, None, h, d, dt, x.device)
     with torch.cuda.device_of(x):
-        ref = _spmm_ref(plan, x, h, d) if n_rows is None else plan.ref
+        ref = _spmm_ref(plan, x, h, d)
         check_attn(_LIB.bpt_vector_spmm_forward(ref, _ptr(edata), _ptr(x), _ptr(y), _ptr(ws), nws, h, d, dt, _stream()),
                    "vector_spmm_forward")
     return y
@@ -252,7 +252,7 @@ def rel_bias_forward(col, indptr_c, eid_c, etype_slot, q, table):
     bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
     bias[E].zero_()
     with torch.cuda.device_of(q):
-        check_attn(_LIB.bpt_rel_bias_forward(plan.ref, _ptr(q), _ptr(table), _ptr(bias), h, d, _dtype(q), _stream()),
+        check_attn(_LIB.bpt_rel_bias_forward(_spmm_ref(plan, q, h, d), _ptr(q), _ptr(table), _ptr(bias), h, d, _dtype(q), _stream()),
                    "rel_bias_forward")
     return bias
 
