@@ -44,7 +44,9 @@ typedef enum {
 
 /* Device-resident plan of one CSR side (see bptg_plan_fill / bptg_group_plan for the array contents).
  * The grp_* fields are optional (n_groups == 0: none); the fused attention entries use them to let one
- * wavefront own up to grp_R rows that share neighbours, loading each neighbour row once for all. */
+ * wavefront own up to grp_R rows that share neighbours, loading each neighbour row once for all, and so do the
+ * SDDMM / SpMM-shaped ops (maskedmm_csr, vector_spmm, rel_bias) when the plan also carries grp_eids and the shape
+ * has specialised kernels; without groups every row (segment) has a wavefront of its own. */
 typedef struct {
     const int32_t *rowptr;   /* n_rows + 1 */
     const int32_t *idx;      /* n_edges : other endpoint of the edge in slot p */
@@ -67,7 +69,8 @@ typedef struct {
     int64_t n_grp_entries;       /* grp_ptr[n_groups] */
     const int32_t *grp_eids;     /* (n_grp_entries + 8) * grp_R or NULL: edge id of (entry u, member m) at
                                     [u * grp_R + m]; n_edges where the entry's mask has no bit m and in the 8
-                                    entries of padding.  Needed by the calls that take a per-edge score term */
+                                    entries of padding.  Needed by the attention calls that take a per-edge score
+                                    term or dropout and by the row-group kernels of the SDDMM / SpMM-shaped ops */
 } bpt_plan;
 
 const char *bpt_strerror(int status);
