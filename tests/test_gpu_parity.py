@@ -325,6 +325,23 @@ def test_stress_graph_properties(ops):
     # 4. run-to-run bit reproducibility (no atomics)
     o2 = op.bpt_attention(*args, q, k, ones)
     assert torch.equal(o, o2)
+    # 5. the op chain (row-group SDDMM / SpMM, segmented softmax) agrees with the fused kernels on random v
+    vr = ((torch.randn(n, 16, 64, generator=gen) / 8).to(torch.bfloat16)).to(DEV)
+    of = op.bpt_attention(*args, q, k, vr)
+    oc = op.bpt_attention(*args, q, k, vr, fused=False)
+    assert torch.allclose(of.float(), oc.float(), rtol=2e-2, atol=2e-2)
+    # 6. plans built on the host and on the GPU (this size takes the GPU by default) give the same result up to rounding
+    from bpt_amd import plan
+    assert isinstance(plan.plan_cache.get(*args[4:], n, n), plan.DevicePlan)
+    old = plan.set_device_build(False)
+    plan.plan_cache.clear()
+    try:
+        oh = op.bpt_attention(*args, q, k, vr)
+        assert isinstance(plan.plan_cache.get(*args[4:], n, n), plan.Plan)
+    finally:
+        plan.set_device_build(old)
+        plan.plan_cache.clear()
+    assert torch.allclose(of.float(), oh.float(), rtol=2e-2, atol=2e-2)
 
 
 def test_determinism_and_cache(ops):
