@@ -143,21 +143,27 @@ SHAPES = [(8, 64), (1, 40), (3, 20), (4, 64), (16, 64), (8, 32)]   # (1,40) and 
 FAST = {torch.float32: {(8, 64), (4, 64), (16, 64), (8, 32)}, torch.bfloat16: {(8, 64), (16, 64)}, torch.float64: set()}
 
 
-@pytest.mark.parametrize("kernels", ["groups-4", "groups-8", "rows", "generic"])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
-@pytest.mark.parametrize("hd", SHAPES)
-@pytest.mark.parametrize("gname,chunk", [("blocks8x30", 32), ("blocks8x30", 7), ("bpt512_k4", 32), ("multigraph", 8), ("fc_w100", 32),
-                                         ("bpt256_k24", 32)])
+def _ops_cases():
+    """(graph, chunk, shape, dtype, kernel family): every family a shape and dtype have, the wide (16x64) and the
+    narrow (8x32) shape on three of the graphs."""
+    out = []
+    for gname, chunk in (("blocks8x30", 32), ("blocks8x30", 7), ("bpt512_k4", 32), ("multigraph", 8), ("fc_w100", 32), ("bpt256_k24", 32)):
+        for hd in SHAPES:
+            if hd in ((16, 64), (8, 32)) and gname not in ("bpt512_k4", "multigraph", "bpt256_k24"):
+                continue
+            for dtype in (torch.float32, torch.float64, torch.bfloat16):
+                families = ["groups-4", "groups-8", "rows", "generic"] if hd in FAST[dtype] else ["groups-4"]
+                out += [pytest.param(gname, chunk, hd, dtype, f, id=f"{gname}-{chunk}-{hd[0]}x{hd[1]}-{str(dtype)[6:]}-{f}") for f in families]
+    return out
+
+
+@pytest.mark.parametrize("gname,chunk,hd,dtype,kernels", _ops_cases())
 def test_ops_match_oracle(ops, gname, chunk, hd, dtype, kernels):
     """kernels: which family the SpMM / SDDMM ops run in: row groups of 4 or 8 rows, one wavefront per row
-    (specialised shapes), or the shape-generic kernels."""
+    (specialised shapes), or the shape-generic kernels (the only family of the other shapes and of float64)."""
     graphop, _ = ops
     h, d = hd
     force_generic = kernels == "generic"
-    if kernels != "groups-4" and hd not in FAST[dtype]:
-        pytest.skip("already generic")
-    if hd in ((16, 64), (8, 32)) and gname not in ("bpt512_k4", "multigraph", "bpt256_k24"):
-        pytest.skip("the wide and the narrow shape run on three of the graphs")
     c = case(gname, chunk)
     n, E = c.n, c.E
     A = rand((n, h, d), dtype, 1, 0.5).to(DEV)
@@ -223,15 +229,20 @@ def test_single_head_2d_inputs(ops):
 # --------------------------------------------------------------------------------------------
 # the attention layer: fused kernels and the unfused op chain, forward + backward
 # --------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("fused", ["groups-4", "groups-8", "rows", False])
-@pytest.mark.parametrize("dtype,hd", [(torch.float32, (8, 64)), (torch.float32, (16, 64)), (torch.float32, (8, 32)),
-                                      (torch.bfloat16, (8, 64)), (torch.bfloat16, (16, 64)), (torch.float32, (2, 24))])
-@pytest.mark.parametrize("gname", ["bpt512_k4", "bpt300_causal_k2", "multigraph", "fc_w100", "bpt256_k24"])
+def _layer_cases():
+    """(graph, dtype, shape, path): the fused kernels over groups of 4 / 8 rows and per row, and the op chain; (2, 24)
+    has no fused instantiation and runs the op chain only."""
+    shapes = [(torch.float32, (8, 64)), (torch.float32, (16, 64)), (torch.float32, (8, 32)),
+              (torch.bfloat16, (8, 64)), (torch.bfloat16, (16, 64)), (torch.float32, (2, 24))]
+    return [pytest.param(g, dt, hd, f, id=f"{g}-{str(dt)[6:]}-{hd[0]}x{hd[1]}-{f or 'chain'}")
+            for g in ("bpt512_k4", "bpt300_causal_k2", "multigraph", "fc_w100", "bpt256_k24") for dt, hd in shapes
+            for f in (("groups-4", "groups-8", "rows", False) if hd != (2, 24) else (False,))]
+
+
+@pytest.mark.parametrize("gname,dtype,hd,fused", _layer_cases())
 def test_attention_layer(ops, gname, dtype, hd, fused):
     graphop, op = ops
     h, d = hd
-    if fused and hd == (2, 24):
-        pytest.skip("no fused instantiation; covered by the unfused chain")
     c = case(gname)
     q, k, v, do = (rand((c.n, h, d), dtype, s, 1.0 / 8).to(DEV) for s in (11, 12, 13, 14))   # N(0,1)/sqrt(64)
     q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
