@@ -375,6 +375,15 @@ class DevicePlan:
                 if self.n_edges != plan_src.n_edges or not (self.covers_all_edges and plan_src.covers_all_edges):
                     raise ValueError("the two plans do not describe the same edge set")
                 E = self.n_edges
+                if not isinstance(plan_src, DevicePlan):
+                    # the partner was planned on the host (the two sides of a bipartite graph can fall on either side
+                    # of the size rule): map the pairs there, from the downloaded group arrays
+                    pairs = torch.from_numpy(link_groups_host(mine["host"], theirs["host"], E)).to(self.device)
+                    st = PlanStruct.from_buffer_copy(mine["struct"])
+                    st.grp_pairs = pairs.data_ptr()
+                    hit = (st, pairs, plan_src)
+                    self._links[key] = hit
+                    return hit[0]
                 n_pairs = (mine["struct"].n_grp_entries + GROUP_PAD_ENTRIES) * R
                 pairs = torch.empty((E + GROUP_PAD_ENTRIES) * R, dtype=torch.int32, device=self.device)
                 ws = torch.empty(4 * max(E, 1) + 512, dtype=torch.uint8, device=self.device)

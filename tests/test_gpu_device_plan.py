@@ -401,3 +401,45 @@ def test_device_graph_builder_equals_host_builder():
         got = g.get_edges_device(DEV, v_shift=shift)
         for a, b in zip(got, want):
             assert a.dtype == torch.int64 and np.array_equal(host(a), b), (type(g).__name__, g.__reduce__()[1])
+
+
+@pytest.mark.parametrize("device_side", ["in", "out"])
+def test_one_side_planned_on_the_gpu_and_the_other_on_the_host(device_side):
+    """The two CSR sides of a graph can be planned in different places (a bipartite graph whose sides fall on either
+    side of the size rule): the pair mapping and the backward pass still work."""
+    from bpt_amd import graphop, plan
+    c = Case("bpt300_causal_k2")
+    h, d = 8, 64
+    q, k, v, do = (rand((c.n, h, d), torch.float32, s, 0.125 if s < 3 else 1.0).to(DEV) for s in range(4))
+    plan.plan_cache.clear()
+    old = plan.set_device_build(device_side == "in")
+    try:
+        p_in = plan.plan_cache.get(*c.inn, c.n, c.n)
+        plan.set_device_build(device_side != "in")
+        p_out = plan.plan_cache.get(*c.out, c.n, c.n)
+        assert isinstance(p_in, plan.DevicePlan) != isinstance(p_out, plan.DevicePlan)
+        # the cache key carries the setting: look the plans up under the setting they were built with
+        plan.set_device_build(device_side == "in")
+        o, lse = graphop.attention_forward(*c.inn, q, k, v)
+        st = p_in.linked_to(p_out, 4)
+        assert st.grp_pairs
+        import ctypes
+        from bpt_amd._lib import attn_lib
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        out_st = p_out.ensure_groups(4, plan.GROUP_ORDER_SRC)["struct"]
+        lib = attn_lib()
+        nws = lib.bpt_workspace_bytes(6, ctypes.byref(st), ctypes.byref(out_st), h, d, 0)
+        ws = torch.empty(nws, dtype=torch.uint8, device=DEV)
+        status = lib.bpt_attention_backward(ctypes.byref(st), ctypes.byref(out_st), q.data_ptr(), k.data_ptr(), v.data_ptr(), None,
+                                            o.data_ptr(), do.data_ptr(), lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                            None, ws.data_ptr(), nws, 0.125, 0.0, 0, h, d, 0, torch.cuda.current_stream().cuda_stream)
+        assert status == 0
+        torch.cuda.synchronize()
+    finally:
+        plan.set_device_build(old)
+        plan.plan_cache.clear()
+    ro, ra = oracle.attention_forward(c.csr, f64(q), f64(k), f64(v))
+    rdq, rdk, rdv = oracle.attention_backward(c.csr, f64(q), f64(k), f64(v), ra, f64(do))
+    close(o, ro, TOL[torch.float32], "o")
+    for got, want, nm in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv")):
+        close(got, want, GTOL[torch.float32], nm, terms=c.max_deg)
