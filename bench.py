@@ -2,8 +2,8 @@
 """Benchmark of the BPT graph-attention hot path on one MI355X.
 
 A step = one fused attention layer forward + backward (SDDMM -> edge softmax -> SpMM and their
-gradients) over one synthetic graph batch, inputs resident in HBM.  Default workload: BASELINE
-config 3, L=8192 tokens, k=4, causal binary-partition graph, 8 heads x 64, fp32.
+gradients) over one synthetic graph batch, inputs resident in HBM.  Default workload: the headline
+configuration (cfg3), L=8192 tokens, k=4, causal binary-partition graph, 8 heads x 64, fp32.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg1|cfg2|cfg5|cfg4-kN|cfg4-w128]
                   [--dtype f32|bf16] [--no-cpu-baseline] [--no-graph]

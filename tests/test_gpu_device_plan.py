@@ -344,7 +344,7 @@ def test_device_plan_on_random_graphs(seed):
 
 def test_batch_merge_on_the_device_and_the_whole_pipeline_time():
     """merge_graphs_device equals merge_graphs; and what a new batch costs from its lengths to plans that the fused
-    kernels can run on, on the host and on the GPU (BASELINE config 2: 32 sequences, causal, k = 4)."""
+    kernels can run on, on the host and on the GPU (benchmark configuration 2: 32 sequences, causal, k = 4)."""
     import time
     from bpt_amd import graphbuilder as gb, plan
     lengths = np.random.default_rng(2345).integers(64, 1025, 32)

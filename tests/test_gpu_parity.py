@@ -56,7 +56,7 @@ def random_multigraph(n, E, seed=1):
 
 GRAPHS = {
     "blocks8x30": lambda: block_graph(8, 30),
-    "bpt512_k4": lambda: bpt_graph(512, False, 4),          # BASELINE config 1 (non-causal: duplicate edges, deg 512 row)
+    "bpt512_k4": lambda: bpt_graph(512, False, 4),          # benchmark configuration 1 (non-causal: duplicate edges, deg 512 row)
     "bpt300_causal_k2": lambda: bpt_graph(300, True, 2),
     "multigraph": lambda: random_multigraph(97, 3000),      # zero-degree node, heavy rows both sides, duplicates
     "fc_w100": lambda: fc_graph(260, 100),                  # every row longer than 64 edges
@@ -284,7 +284,7 @@ def test_attention_with_rel_pos_chain(ops):
 
 
 def test_headline_graph_full_parity(ops):
-    """BASELINE config 3 at full size (L=8192, k=4, causal, 8x64 fp32) directly against the oracle."""
+    """benchmark configuration 3 at full size (L=8192, k=4, causal, 8x64 fp32) directly against the oracle."""
     _, op = ops
     from bpt_amd import graphbuilder as gb
     g = gb.BinaryPartition(8192, True, 4, 10)
@@ -310,7 +310,7 @@ def test_headline_graph_full_parity(ops):
 
 
 def test_stress_graph_properties(ops):
-    """BASELINE config 5 (L=32768, k=8, causal, 16x64, bf16): size-independent properties."""
+    """benchmark configuration 5 (L=32768, k=8, causal, 16x64, bf16): size-independent properties."""
     _, op = ops
     from bpt_amd import graphbuilder as gb
     g = gb.BinaryPartition(32768, True, 8, 10)

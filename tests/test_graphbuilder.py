@@ -120,7 +120,7 @@ def test_build_csr_rejects_out_of_range():
 
 
 def test_batch_merge_cfg2_shape():
-    """BASELINE config 2: 32 causal graphs with seeded lengths merged block-diagonally."""
+    """benchmark configuration 2: 32 causal graphs with seeded lengths merged block-diagonally."""
     lengths = np.random.default_rng(2345).integers(64, 1025, 32)
     assert lengths[:4].tolist() == [171, 550, 518, 514] and lengths.sum() == 16736
     cache = {}
