@@ -392,7 +392,7 @@ def test_device_graph_builder_equals_host_builder():
     from bpt_amd import graphbuilder as gb
     graphs = [gb.BinaryPartition(L, triu, step, clip) for L in (1, 2, 3, 5, 6, 7, 13, 33, 100, 511, 512, 1000)
               for triu in (False, True) for step, clip in ((1, 10), (2, 3), (4, 10))]
-    graphs += [gb.BinaryPartition(8192, True, 4, 10), gb.BinaryPartition(4097, False, 8, 2)]
+    graphs += [gb.BinaryPartition(8192, True, 4, 10), gb.BinaryPartition(4097, False, 8, 2), gb.BinaryPartition(32768, True, 8, 10)]
     graphs += [gb.FullyConnected(L, triu, w) for L in (1, 2, 17, 260) for triu in (False, True) for w in (0, 1, 5, 8192)]
     graphs += [gb.OpenAISparse(L, stride, c) for L, stride, c in ((1, 4, 2), (50, 8, 3), (257, 16, 16), (64, 64, 0))]
     for i, g in enumerate(graphs):
