@@ -56,6 +56,7 @@ ATTN_API = {
     "bpt_sparse_softmax_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_i64, ctypes.c_int, ctypes.c_int, c_vp]),
     "bpt_sparse_softmax_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_int, ctypes.c_int, c_vp]),
     "bpt_vector_spmm_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
+    "bpt_vector_spmm_accumulate": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_vector_spmm_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_rel_bias_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp] + _tail),
     "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float, ctypes.c_float,

@@ -189,7 +189,7 @@ __global__ __launch_bounds__(BLOCK) void k_spmm_generic(bpt_plan P, const T *__r
 // are then added in wave order, so the result is a fixed function of the plan.
 template <typename T>
 __device__ __forceinline__ void combine_sum_block(const int32_t *__restrict__ hv, const typename Elem<T>::acc_t *__restrict__ ws,
-                                                  T *__restrict__ Y, int C) {
+                                                  T *__restrict__ Y, int C, bool accumulate = false) {
     using acc_t = typename Elem<T>::acc_t;
     __shared__ acc_t part[WAVES_PER_BLOCK][WAVE];
     const int row = hv[0], s0 = hv[1], ns = hv[2];
@@ -214,6 +214,7 @@ __device__ __forceinline__ void combine_sum_block(const int32_t *__restrict__ hv
         acc_t r = part[0][lane];
 #pragma unroll
         for (int i = 1; i < WAVES_PER_BLOCK; ++i) r += part[i][lane];
+        if (accumulate) r += Elem<T>::ld(Y + (size_t)row * C + j);
         Elem<T>::st(Y + (size_t)row * C + j, r);
     }
 }
@@ -221,8 +222,8 @@ __device__ __forceinline__ void combine_sum_block(const int32_t *__restrict__ hv
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void k_combine_sum(const int32_t *__restrict__ heavy,
                                                        const typename Elem<T>::acc_t *__restrict__ ws, T *__restrict__ Y0,
-                                                       T *__restrict__ Y1, int C, size_t ws_stride) {
-    combine_sum_block<T>(heavy + 3 * blockIdx.x, ws + (size_t)blockIdx.z * ws_stride, blockIdx.z == 0 ? Y0 : Y1, C);
+                                                       T *__restrict__ Y1, int C, size_t ws_stride, int accumulate = 0) {
+    combine_sum_block<T>(heavy + 3 * blockIdx.x, ws + (size_t)blockIdx.z * ws_stride, blockIdx.z == 0 ? Y0 : Y1, C, accumulate != 0);
 }
 
 // The three sums of the fused backward in one launch: blocks x < n_a combine rows of list A into YA (z = 0 only),
@@ -1835,7 +1836,7 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
 // fetched by its edge id (grp_eids) and is the A operand of v_mfma_f32_4x4x1 exactly as in k_attn_bwd_src_grp.
 template <typename T, int H, int D, int R, int HS>
 __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T, Lay<T, H / HS, D>::EPL, R>()))) void k_spmm_grp(
-    bpt_plan P, const T *__restrict__ W, const T *__restrict__ X, T *__restrict__ Y, float *__restrict__ ws) {
+    bpt_plan P, const T *__restrict__ W, const T *__restrict__ X, T *__restrict__ Y, float *__restrict__ ws, int accumulate) {
     constexpr int HL = H / HS, CF = H * D;                  // heads of this wavefront's slice; elements of a full row
     using L = Lay<T, HL, D>;
     constexpr int EPL = L::EPL, NQ = R / 4, GRP_BATCH = grp_batch<L::EPL>();
@@ -1920,8 +1921,17 @@ __global__ __launch_bounds__(WAVE) __attribute__((amdgpu_waves_per_eu(grp_wpe<T,
         float out[EPL];
 #pragma unroll
         for (int t = 0; t < EPL; ++t) out[t] = acc[m / 4][t][m & 3];
-        if (gh.slots[m] < 0) store_row<T, HL, D>(Y + (size_t)gh.rows[m] * CF + coff, lane, out);
-        else store_row_ws<T, HL, D>(ws + (size_t)gh.slots[m] * CF + coff, lane, out);
+        if (gh.slots[m] < 0) {
+            if (accumulate) {                 // Y += the sum (rows in segments get theirs when the segments are combined)
+                float old[EPL];
+                load_row32<T, HL, D, CF>(Y, (uint32_t)gh.rows[m], loff, old);
+#pragma unroll
+                for (int t = 0; t < EPL; ++t) out[t] += old[t];
+            }
+            store_row<T, HL, D>(Y + (size_t)gh.rows[m] * CF + coff, lane, out);
+        } else {
+            store_row_ws<T, HL, D>(ws + (size_t)gh.slots[m] * CF + coff, lane, out);
+        }
     }
 }
 
@@ -2258,7 +2268,7 @@ int sddmm(const bpt_plan *P, const void *A, const void *B, void *y, int h, int d
     }
     return sddmm_generic(P, A, B, y, h, d, dtype, s);
 }
-int spmm_grp(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, int dtype, hipStream_t s);
+int spmm_grp(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, int dtype, hipStream_t s, int accumulate = 0);
 int spmm(const bpt_plan *P, const void *W, const void *X, void *Y, void *ws, int h, int d, int dtype, hipStream_t s) {
     if (fast_shape(h, d, dtype) && aligned16(X) && aligned16(Y) && aligned16(ws)) {
         // a plan that carries row groups and their edge ids: one row load per entry instead of one per edge
@@ -2324,18 +2334,18 @@ bool spmm_grp_ok(const bpt_plan *P, int h, int d, int dtype) {
 }
 
 template <typename T, int H, int D>
-int run_spmm_grp(const bpt_plan *P, const void *W, const void *X, void *Y, float *ws, hipStream_t s) {
+int run_spmm_grp(const bpt_plan *P, const void *W, const void *X, void *Y, float *ws, hipStream_t s, int accumulate = 0) {
     constexpr int HS = head_slices<T, H, D>();
 #define LAUNCH_SPMM(RR)                                                                                                     \
     hipLaunchKernelGGL((k_spmm_grp<T, H, D, RR, HS>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)W, (const T *)X, \
-                       (T *)Y, ws)
+                       (T *)Y, ws, accumulate)
     if (P->grp_R == 8) LAUNCH_SPMM(8);
     else LAUNCH_SPMM(4);
 #undef LAUNCH_SPMM
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
     hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
-                       (T *)Y, (T *)nullptr, H * D, (size_t)0);
+                       (T *)Y, (T *)nullptr, H * D, (size_t)0, accumulate);
     return launch_status();
 }
 
@@ -2355,8 +2365,8 @@ int sddmm_grp(const bpt_plan *P, const void *A, const void *B, void *y, int h, i
     return BPT_ERR_UNSUPPORTED;
 }
 
-int spmm_grp(const bpt_plan *P, const void *W, const void *Xp, void *Y, void *ws, int h, int d, int dtype, hipStream_t s) {
-#define X(HH, DD) if (h == HH && d == DD) return run_spmm_grp<T, HH, DD>(P, W, Xp, Y, (float *)ws, s);
+int spmm_grp(const bpt_plan *P, const void *W, const void *Xp, void *Y, void *ws, int h, int d, int dtype, hipStream_t s, int accumulate) {
+#define X(HH, DD) if (h == HH && d == DD) return run_spmm_grp<T, HH, DD>(P, W, Xp, Y, (float *)ws, s, accumulate);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
 #undef X
@@ -2630,6 +2640,20 @@ int bpt_vector_spmm_forward(const bpt_plan *plan, const void *edata, const void 
     const int64_t need = bpt_workspace_bytes(BPT_OP_SPMM_FWD, plan, nullptr, h, d, dtype);
     if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
     return spmm(plan, edata, x, y, workspace, h, d, dtype, (hipStream_t)stream);
+}
+
+int bpt_vector_spmm_accumulate(const bpt_plan *plan, const void *edata, const void *x, void *y, void *workspace,
+                               int64_t workspace_bytes, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan, true));
+    CHECK(check_shape(h, d, dtype));
+    if (!y || (plan->n_edges > 0 && (!edata || !x))) return BPT_ERR_NULL;
+    if (plan->n_edges == 0) return BPT_OK;
+    const int64_t need = bpt_workspace_bytes(BPT_OP_SPMM_FWD, plan, nullptr, h, d, dtype);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return BPT_ERR_WORKSPACE;
+    // exists in the row-group kernels only
+    if (!(fast_shape(h, d, dtype) && aligned16(x) && aligned16(y) && aligned16(workspace) && spmm_grp_ok(plan, h, d, dtype)))
+        return BPT_ERR_UNSUPPORTED;
+    return spmm_grp(plan, edata, x, y, workspace, h, d, dtype, (hipStream_t)stream, 1);
 }
 
 int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const void *edata, const void *dy, const void *x,

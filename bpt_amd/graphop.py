@@ -188,11 +188,13 @@ def sparse_softmax_backward(row, indptr, eid, y, dy):
     return dx
 
 
-def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None):
+def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None, out=None):
     """y[row] = sum_p edata[eid[p]] * x[indices[p]] (graphop.cpp:79-95, graphop_kernel.cu:509-542).
 
     n_rows (keyword only, not in the reference): number of rows of y when it differs from x.size(0) — a
-    rectangular operator, used for the segment sums of the relative-position table's gradient."""
+    rectangular operator, used for the segment sums of the relative-position table's gradient.
+    out (keyword only, not in the reference): a contiguous tensor of y's shape that the sum is ADDED to and that is
+    returned (in the kernel's store where the row-group kernels apply, else by a separate addition)."""
     _check_all(row=row, indptr=indptr, eid=eid, indices=indices, edata=edata, x=x)
     _same_dtype(edata, x)
     h, d = _hd(x)
@@ -203,11 +205,19 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None):
     y = torch.empty_like(x) if n_rows is None else torch.empty((n_out,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
     dt = _dtype(x)
     ws, nws = _workspace(OP_SPMM_FWD, plan, None, h, d, dt, x.device)
+    if out is not None and (out.shape != y.shape or out.dtype != y.dtype or out.device != y.device or not out.is_contiguous()):
+        raise ValueError("out must be a contiguous tensor of the result's shape, dtype and device")
     with torch.cuda.device_of(x):
         ref = _spmm_ref(plan, x, h, d)
+        if out is not None:
+            st = _LIB.bpt_vector_spmm_accumulate(ref, _ptr(edata), _ptr(x), _ptr(out), _ptr(ws), nws, h, d, dt, _stream())
+            if st == 0:
+                return out
+            if st != -7:                      # BPT_ERR_UNSUPPORTED: no row-group kernel for this call
+                check_attn(st, "vector_spmm_accumulate")
         check_attn(_LIB.bpt_vector_spmm_forward(ref, _ptr(edata), _ptr(x), _ptr(y), _ptr(ws), nws, h, d, dt, _stream()),
                    "vector_spmm_forward")
-    return y
+    return y if out is None else out.add_(y)
 
 
 def vector_spmm_backward(row, indptr, eid, indices, col, indptr_t, eid_t, indices_t, edata, dy, x):

@@ -120,7 +120,7 @@ class BPTRelAttention(Function):
         h = q.size(1)
         ds = ds.to(q.dtype)
         table_h = table.unsqueeze(1).expand(-1, h, -1).contiguous()
-        dq = dq + vector_spmm_forward(col, indptr_c, eid_c, etype_slot, ds, table_h, n_rows=q.size(0))
+        dq = vector_spmm_forward(col, indptr_c, eid_c, etype_slot, ds, table_h, n_rows=q.size(0), out=dq)
         dtable = vector_spmm_forward(t_row, t_indptr, t_order, t_dst, ds, q, n_rows=table.size(0))
         dtable = dtable.float().sum(1).to(table.dtype)
         return None, None, None, None, None, None, None, None, dq, dk, dv, None, None, None, dtable, None

@@ -127,6 +127,12 @@ int bpt_sparse_softmax_backward(const bpt_plan *plan, const void *y, const void 
 int bpt_vector_spmm_forward(const bpt_plan *plan, const void *edata, const void *x, void *y,
                             void *workspace, int64_t workspace_bytes, int h, int d, int dtype, void *stream);
 
+/* y[r] += sum_p edata[eid[p]] * x[idx[p]]: bpt_vector_spmm_forward accumulating into y.  No counterpart in the reference
+ * (it serves the q gradient of the fused rel_pos term).  Row-group kernels only: BPT_ERR_UNSUPPORTED unless the plan
+ * carries row groups with grp_eids and the shape has specialised kernels; the caller then adds the plain result. */
+int bpt_vector_spmm_accumulate(const bpt_plan *plan, const void *edata, const void *x, void *y,
+                               void *workspace, int64_t workspace_bytes, int h, int d, int dtype, void *stream);
+
 /* graphop.cpp:190 vector_spmm_backward(row.., col.., edata, dy, x) -> [dedata, dx]
  * dedata[eid[p]] = <dy[row], x[idx[p]]> over `plan`; dx[c] = sum over ALL rows c of `plan_t` of
  * edata[eid_t[p]] * dy[idx_t[p]].  (The reference launches the dx kernel with the grid of the

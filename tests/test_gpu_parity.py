@@ -589,3 +589,26 @@ def test_attention_to_memory_over_an_inter_graph(ops, n_enc, n_dec, dtype):
     close(k.grad, rdk.numpy(), GTOL[dtype], "dk", 70)
     close(v.grad, rdv.numpy(), GTOL[dtype], "dv", 70)
     assert not o[min(n_dec, 101):].any()             # rows without in-edges (span nodes, padding) stay zero
+
+
+@pytest.mark.parametrize("grouped", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_vector_spmm_accumulates_into_out(ops, dtype, grouped):
+    """vector_spmm_forward(out=y0) returns y0 + the product: in the row-group kernel's store, or by a separate addition
+    where there is none (one wavefront per row; 2-D inputs)."""
+    graphop, _ = ops
+    c = case("bpt512_k4")
+    w = rand((c.E, 8), dtype, 1).to(DEV)
+    x = rand((c.n, 8, 64), dtype, 2, 0.5).to(DEV)
+    y0 = rand((c.n, 8, 64), dtype, 3).to(DEV)
+    old = graphop.set_grouped_ops(grouped)
+    try:
+        want = oracle.vector_spmm_forward(*c.np_in, f64(w), f64(x)) + f64(y0)
+        out = y0.clone()
+        got = graphop.vector_spmm_forward(*c.inn, w, x, out=out)
+        assert got is out
+        close(got, want, GTOL[dtype] if dtype == torch.float32 else TOL[dtype], "spmm accumulate", c.max_deg)
+        with pytest.raises(ValueError):
+            graphop.vector_spmm_forward(*c.inn, w, x, out=y0[:-1])
+    finally:
+        graphop.set_grouped_ops(old)
