@@ -373,10 +373,11 @@ _GROUP_ROWS = None          # None: chosen per call from dtype and shape
 def _group_rows(q, h, d, plan):
     """Rows per group for the fused kernels.  Groups of 8 nearly halve the row fetches of groups of 4 but double
     the work of the longest wavefront, which measured as a gain only on graphs with enough groups to fill the
-    GPU twice or with long rows (average degree >= 64), and not for bfloat16 rows of up to 512 columns."""
+    GPU twice or with long rows (average degree >= 48: at L = 4096, k = 8 (37) groups of 4 win, at k = 16 (59) groups of 8),
+    and not for bfloat16 rows of up to 512 columns."""
     if _GROUP_ROWS is not None:
         return _GROUP_ROWS
-    big = plan.n_items >= 16384 or plan.n_edges >= 64 * max(plan.n_rows, 1)
+    big = plan.n_items >= 16384 or plan.n_edges >= 48 * max(plan.n_rows, 1)
     return 8 if (big and (q.dtype == torch.float32 or h * d > 512)) else 4
 
 
