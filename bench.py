@@ -109,7 +109,7 @@ def main():
                     help="add the relative-position score term q[dst].table[etype[e]] (table (1000, d_head), modules/attention.py:23,42,69-71)")
     ap.add_argument("--plan", default="auto", choices=["auto", "host", "device"],
                     help="where launch plans and row groups are built: on the host (libbptgraph), on the GPU (libbptplan), "
-                         "or by graph size (the library's default: on the GPU from 24576 rows)")
+                         "or by graph size and density (the library's default)")
     ap.add_argument("--block-layers", type=int, default=0,
                     help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the workload's graph")
     args = ap.parse_args()

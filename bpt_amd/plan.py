@@ -27,7 +27,9 @@ GROUP_PAD_ENTRIES = 8  # the kernels' software pipeline reads per-entry arrays t
 _CACHE_SIZE = 64
 DEVICE_BUILD = None     # where new plans are built: True = on the GPU (libbptplan), False = on the host, None = by size
 DEVICE_BUILD_MIN_ROWS = 24576   # None: graphs with at least this many rows are planned on the GPU (measured: their
-                                # simpler grouping runs the fused kernels 4-9 % faster there and builds 10-30 x faster)
+                                # simpler grouping runs the fused kernels 4-9 % faster there and builds 10-30 x faster),
+DEVICE_BUILD_MIN_DEGREE = 32    # and so are graphs of at least 2^17 edges with this average degree (L = 4096: k = 8, 16,
+                                # 32 run 5, 3 and 18 % faster on GPU-built groups, k = 1 and 4 run 8 and 1 % slower)
 
 
 def _ptr(a):
@@ -216,7 +218,8 @@ class Plan:
 
 def set_device_build(on):
     """Plans of graphs seen from now on are built on the GPU (True: DevicePlan), on the host (False: Plan), or where
-    their size says (None, the default: on the GPU from DEVICE_BUILD_MIN_ROWS rows).  Returns the old setting."""
+    their size says (None, the default: on the GPU from DEVICE_BUILD_MIN_ROWS rows, or from 2^17 edges at an average
+    degree of DEVICE_BUILD_MIN_DEGREE).  Returns the old setting."""
     global DEVICE_BUILD
     old, DEVICE_BUILD = DEVICE_BUILD, (None if on is None else bool(on))
     return old
@@ -226,7 +229,10 @@ def _build_on_device(eid, n_rows):
     if not eid.is_cuda:
         return False
     if DEVICE_BUILD is None:
-        return n_rows is not None and n_rows >= DEVICE_BUILD_MIN_ROWS
+        if n_rows is None:
+            return False
+        n_edges = int(eid.numel())
+        return n_rows >= DEVICE_BUILD_MIN_ROWS or (n_edges >= (1 << 17) and n_edges >= DEVICE_BUILD_MIN_DEGREE * n_rows)
     return DEVICE_BUILD
 
 
