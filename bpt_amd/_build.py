@@ -24,28 +24,35 @@ HIP_FLAGS = [
 ]
 
 
-def build_graph(verbose=True):
-    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
-           os.path.join(CSRC, "bptgraph.cpp"), "-o", GRAPH_SO]
+# The target feature above only exists for the GPU; hipcc also hands it to its host pass, which reports it once per
+# internal step with exactly this line and ignores it.  The line is dropped so that real diagnostics stand out.
+_HOST_PASS_NOTE = "'-packed-fp32-ops' is not a recognized feature for this target (ignoring feature)"
+
+
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(line for line in proc.stdout.splitlines() if line.strip() != _HOST_PASS_NOTE)
+    if out.strip():
+        print(out, flush=True)
+    if proc.returncode != 0:
+        raise subprocess.CalledProcessError(proc.returncode, cmd)
+
+
+def build_graph(verbose=True):
+    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+          os.path.join(CSRC, "bptgraph.cpp"), "-o", GRAPH_SO], verbose)
     return GRAPH_SO
 
 
-def build_attn(verbose=True, extra=(), out=None):
-    cmd = [HIPCC] + HIP_FLAGS + list(extra) + [os.path.join(CSRC, "bptattn.hip"), "-o", out or ATTN_SO]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+def build_attn(verbose=True):
+    _run([HIPCC] + HIP_FLAGS + [os.path.join(CSRC, "bptattn.hip"), "-o", ATTN_SO], verbose)
     return ATTN_SO
 
 
 def build_plan(verbose=True):
-    cmd = [HIPCC] + HIP_FLAGS + [os.path.join(CSRC, "bptplan.hip"), "-o", PLAN_SO]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+    _run([HIPCC] + HIP_FLAGS + [os.path.join(CSRC, "bptplan.hip"), "-o", PLAN_SO], verbose)
     return PLAN_SO
 
 

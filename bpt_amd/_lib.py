@@ -106,8 +106,7 @@ def graph_lib():
 def attn_lib():
     global _attn
     if _attn is None:
-        # BPT_ATTN_SO: load another build of the same library (kernel experiments); default = the in-tree build
-        _attn = _load(os.environ.get("BPT_ATTN_SO", ATTN_SO), ATTN_API, "libbptattn (HIP kernels)")
+        _attn = _load(ATTN_SO, ATTN_API, "libbptattn (HIP kernels)")
     return _attn
 
 
