@@ -61,6 +61,8 @@ ATTN_API = {
     "bpt_rel_bias_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp] + _tail),
     "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float, ctypes.c_float,
                                             ctypes.c_uint64] + _tail),
+    "bpt_attention_forward_noalloc": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, ctypes.c_float, ctypes.c_float,
+                                                    ctypes.c_uint64] + _tail),
     "bpt_attention_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
                                              c_i64, ctypes.c_float, ctypes.c_float, ctypes.c_uint64] + _tail),
 }

@@ -20,6 +20,7 @@
 #include <atomic>
 #include <cmath>
 #include <cstdint>
+#include <mutex>
 
 #include "../../include/bptattn.h"
 
@@ -2506,6 +2507,36 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
 
 }  // namespace
 
+// Workspace of bpt_attention_forward_noalloc: one copy per GPU, held until the process ends.  In host code this
+// name is only a handle for hipGetSymbolAddress; kernels get the device address that call returns.
+static __device__ __align__(256) unsigned char scratch[BPT_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int MAX_SCRATCH_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[MAX_SCRATCH_DEVICES] = {};
+
+// device address of `scratch` on the current device (looked up once per device)
+int scratch_of_current_device(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_SCRATCH_DEVICES) return BPT_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return BPT_ERR_NULL;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return BPT_OK;
+}
+
+}  // namespace
+
 // ------------------------------------------------------------------------------------------
 // C ABI
 // ------------------------------------------------------------------------------------------
@@ -2522,6 +2553,7 @@ const char *bpt_strerror(int status) {
         case BPT_ERR_WORKSPACE: return "workspace missing or too small";
         case BPT_ERR_PLAN: return "plans do not describe the same graph";
         case BPT_ERR_UNSUPPORTED: return "combination not implemented";
+        case BPT_ERR_SCRATCH: return "the call needs more than the library's static scratch (BPT_NOALLOC_SCRATCH_BYTES)";
         default: return "unknown bptattn status";
     }
 }
@@ -2690,6 +2722,20 @@ int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k,
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
 #undef X
     return BPT_ERR_UNSUPPORTED;
+}
+
+int bpt_attention_forward_noalloc(const bpt_plan *plan_in, const void *q, const void *k, const void *v, const float *bias, void *o,
+                                  float *lse, float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype,
+                                  void *stream) {
+    CHECK(check_plan(plan_in, true));
+    CHECK(check_shape(h, d, dtype));
+    const int64_t need = bpt_workspace_bytes(BPT_OP_ATTN_FWD, plan_in, nullptr, h, d, dtype);
+    if (need < 0) return BPT_ERR_SIZE;
+    if (need > (int64_t)BPT_NOALLOC_SCRATCH_BYTES) return BPT_ERR_SCRATCH;
+    void *ws = nullptr;
+    CHECK(scratch_of_current_device(&ws));
+    return bpt_attention_forward(plan_in, q, k, v, bias, o, lse, ws, (int64_t)BPT_NOALLOC_SCRATCH_BYTES, scale, dropout_p, dropout_seed,
+                                 h, d, dtype, stream);
 }
 
 int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, const void *q, const void *k, const void *v,

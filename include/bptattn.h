@@ -39,7 +39,8 @@ typedef enum {
     BPT_ERR_SHAPE = -4,       /* h or d not positive / too large */
     BPT_ERR_WORKSPACE = -5,   /* workspace missing or smaller than bpt_workspace_bytes() */
     BPT_ERR_PLAN = -6,        /* plans do not describe the same graph (edge / node counts differ) */
-    BPT_ERR_UNSUPPORTED = -7  /* combination not implemented (e.g. fused attention in f64) */
+    BPT_ERR_UNSUPPORTED = -7, /* combination not implemented (e.g. fused attention in f64) */
+    BPT_ERR_SCRATCH = -8      /* the call needs more than BPT_NOALLOC_SCRATCH_BYTES of the library's static scratch */
 } bpt_status;
 
 /* Device-resident plan of one CSR side (see bptg_plan_fill / bptg_group_plan for the array contents).
@@ -174,6 +175,21 @@ int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, co
                            const void *v, const float *bias, const void *o, const void *d_o, const float *lse,
                            void *dq, void *dk, void *dv, float *ds_out, void *workspace, int64_t workspace_bytes,
                            float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype, void *stream);
+
+/* bpt_attention_forward for callers that cannot allocate device memory (code under HIP graph capture, serving
+ * loops that forbid it, harnesses that fail on any hipMalloc).  No counterpart in the reference.  Same arguments,
+ * kernels and results as bpt_attention_forward, except that the workspace (partial rows of the nodes that the
+ * plan splits) is a static device array of BPT_NOALLOC_SCRATCH_BYTES inside the library instead of an argument;
+ * the call allocates and frees nothing (inputs and outputs are still the caller's).  A plan that needs more
+ * (bpt_workspace_bytes(BPT_OP_ATTN_FWD, ...) > BPT_NOALLOC_SCRATCH_BYTES) is refused with BPT_ERR_SCRATCH and
+ * nothing is launched.  The first call on a device looks up that device's copy of the array (no allocation,
+ * but not capturable: make one call before capturing).  Every call on a device uses that device's one array:
+ * calls that overlap on one GPU (two streams, two threads) race on it; calls on one stream are ordered.
+ * Nothing in the array has to start at zero: every slot that is read has been written by the same call. */
+#define BPT_NOALLOC_SCRATCH_BYTES (16 * 1024 * 1024)
+int bpt_attention_forward_noalloc(const bpt_plan *plan_in, const void *q, const void *k, const void *v,
+                                  const float *bias, void *o, float *lse, float scale, float dropout_p,
+                                  uint64_t dropout_seed, int h, int d, int dtype, void *stream);
 
 #ifdef __cplusplus
 }
