@@ -1374,6 +1374,7 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
     const int head = slice * HL + lane / L::LPH, j = lane & 3, blk = lane >> 2;
     const uint32_t loff = (uint32_t)((coff + L::off(lane, 0)) * sizeof(T));
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    const int eid_last = (int)P.n_grp_entries + GRP_PAD_ENTRIES - 1;      // last entry of grp_eids, padding included
     __shared__ uint4 kst[2][NB * PITCH];              // rows as loaded, one spare vector per row against bank conflicts
     __shared__ uint4 vst[W3 ? 1 : 2][NB * NV * WAVE];
     // q row of member 4 wv + j, the columns of this lane's block: float32 pre-scaled, or (bfloat16) as loaded, the
@@ -1423,8 +1424,10 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
                 load_row32_raw<T, HL, D, CF>(v, src, loff, B.vr[e]);
             }
             if constexpr (BIAS || DROP) {
+                // the look-ahead reaches up to 2 * NB + NB - 1 entries past the group's last one: clamped to the last
+                // entry of the list's padding (all values there are the spare edge id)
 #pragma unroll
-                for (int e = 0; e < NB; ++e) B.xe[e] = P.grp_eids[(size_t)(p0 + b + e) * R + 4 * wv + j];
+                for (int e = 0; e < NB; ++e) B.xe[e] = P.grp_eids[(size_t)min(p0 + b + e, eid_last) * R + 4 * wv + j];
             }
         };
         // the score terms of a batch are fetched one batch ahead, with the edge ids that came in the batch before

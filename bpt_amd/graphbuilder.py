@@ -162,12 +162,26 @@ def build_csr(rows, cols, n_nodes):
     return indptr, indices, eid
 
 
-def get_csrs(src, dst, n_nodes, chunk_size=32, as_torch=True):
+def get_csrs(src, dst, n_nodes, chunk_size=32, as_torch=True, in_order="eid"):
     """Replacement of graph/base.py:71-86 without DGL: returns
     (out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C) with csr = (indptr, indices, eid), all int64
-    (torch CPU tensors by default, numpy with as_torch=False)."""
+    (torch CPU tensors by default, numpy with as_torch=False).
+
+    The reference takes both CSRs from DGL 0.4 (`adjacency_matrix_scipy`), which fixes `indptr` and the set of
+    (index, edge id) pairs of every row but whose order INSIDE a row is not specified by anything in the reference.
+    in_order picks it for the in-CSR: "eid" (default) = ascending edge id, the order of a stable counting sort of the
+    edge list by destination; "src_eid" = ascending (source, edge id), the order a transpose of the out-CSR gives.
+    The out-CSR is in ascending edge id either way.  Every op result is the same for both up to float rounding, and
+    edge-addressed results do not depend on it at all."""
+    if in_order not in ("eid", "src_eid"):
+        raise ValueError('in_order must be "eid" or "src_eid"')
     out_csr = build_csr(src, dst, n_nodes)
     in_csr = build_csr(dst, src, n_nodes)
+    if in_order == "src_eid":
+        indptr, indices, eid = in_csr
+        row_of_slot = np.repeat(np.arange(n_nodes, dtype=np.int64), np.diff(indptr))
+        order = np.lexsort((eid, indices, row_of_slot))
+        in_csr = (indptr, np.ascontiguousarray(indices[order]), np.ascontiguousarray(eid[order]))
     ROW, INDPTR_R = partition_csr(out_csr[0], chunk_size)
     COL, INDPTR_C = partition_csr(in_csr[0], chunk_size)
     res = (out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C)

@@ -64,6 +64,27 @@ def _same_dtype(*ts):
     for t in ts[1:]:
         if t.dtype != ts[0].dtype:
             raise RuntimeError("all floating point arguments must share one dtype")
+        if t.device != ts[0].device:
+            raise ValueError("all tensors of a call must be on one device")
+
+
+# The kernels take raw pointers and trust the sizes of the plan, so every tensor's shape is checked here, before
+# anything is launched: a mismatch raises ValueError instead of reading or writing out of bounds on the GPU.
+def _expect_shape(t, shape, name):
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+def _expect_edges(t, n_edges, h, name, two_d_node):
+    """Edge tensors are (E,) next to (n, d) node tensors and (E, h) next to (n, h, d) ones (graphop_kernel.cu:247-248)."""
+    if h == 1 and tuple(t.shape) in ((n_edges,), (n_edges, 1)):
+        return                                   # one head: the two spellings are the same memory
+    _expect_shape(t, (n_edges,) if two_d_node else (n_edges, h), name)
+
+
+def _expect_index(eid, indices):
+    if eid.dim() != 1 or (indices is not None and tuple(indices.shape) != tuple(eid.shape)):
+        raise ValueError("eid and indices must be 1-D tensors of the same length")
 
 
 def _stream():
@@ -104,6 +125,8 @@ def maskedmm_csr_forward(row, indptr, eid, indices, A, B):
     _check_all(row=row, indptr=indptr, eid=eid, indices=indices, A=A, B=B)
     _same_dtype(A, B)
     h, d = _hd(A)
+    _expect_index(eid, indices)
+    _expect_shape(B, (B.size(0),) + tuple(A.shape[1:]), "B")
     plan = plan_cache.get(row, indptr, eid, indices, A.size(0), B.size(0))
     e = eid.size(0)
     y = _edge_out(plan, (e,) if A.dim() == 2 else (e, h), A)
@@ -120,6 +143,11 @@ def maskedmm_csr_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c,
     dy = dy.contiguous()
     _same_dtype(A, B, dy)
     h, d = _hd(A)
+    _expect_index(eid_r, indices_r)
+    _expect_index(eid_c, indices_c)
+    _expect_shape(B, (B.size(0),) + tuple(A.shape[1:]), "B")
+    _expect_shape(eid_c, eid_r.shape, "eid_c")
+    _expect_edges(dy, eid_r.size(0), h, "dy", A.dim() == 2)
     plan_r = plan_cache.get(row, indptr_r, eid_r, indices_r, A.size(0), B.size(0))
     plan_c = plan_cache.get(col, indptr_c, eid_c, indices_c, B.size(0), A.size(0))
     dA, dB = torch.empty_like(A), torch.empty_like(B)
@@ -136,6 +164,8 @@ def node_mul_edge_forward(row, indptr, eid, A, B):
     _check_all(row=row, indptr=indptr, eid=eid, A=A, B=B)
     _same_dtype(A, B)
     h, d = _hd(A)
+    _expect_index(eid, None)
+    _expect_shape(B, (eid.size(0), d), "B")
     plan = plan_cache.get(row, indptr, eid, None, A.size(0), None)
     e = eid.size(0)
     y = _edge_out(plan, (e,) if A.dim() == 2 else (e, h), A)
@@ -151,6 +181,9 @@ def node_mul_edge_backward(row, indptr, eid, A, B, dy):
     dy = dy.contiguous()
     _same_dtype(A, B, dy)
     h, d = _hd(A)
+    _expect_index(eid, None)
+    _expect_shape(B, (eid.size(0), d), "B")
+    _expect_edges(dy, eid.size(0), h, "dy", A.dim() == 2)
     plan = plan_cache.get(row, indptr, eid, None, A.size(0), None)
     dA = torch.empty_like(A)
     dB = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(B)
@@ -165,6 +198,9 @@ def node_mul_edge_backward(row, indptr, eid, A, B, dy):
 def sparse_softmax_forward(row, indptr, eid, x):
     """softmax of x over the slots of each row (graphop.cpp:59-71, graphop_kernel.cu:411-463)."""
     _check_all(row=row, indptr=indptr, eid=eid, x=x)
+    _expect_index(eid, None)
+    if x.dim() not in (1, 2) or x.size(0) != eid.size(0):
+        raise ValueError(f"x must be ({eid.size(0)},) or ({eid.size(0)}, h), got {tuple(x.shape)}")
     plan = plan_cache.get(row, indptr, eid, None, None, None)
     y = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(x)
     ws, nws = _workspace(OP_SOFTMAX_FWD, plan, None, _edge_h(x), 1, _dtype(x), x.device)
@@ -178,6 +214,10 @@ def sparse_softmax_backward(row, indptr, eid, y, dy):
     """dx = y * (dy - sum_row dy*y) (graphop.cpp:163-177, graphop_kernel.cu:465-507)."""
     _check_all(row=row, indptr=indptr, eid=eid, y=y, dy=dy)
     _same_dtype(y, dy)
+    _expect_index(eid, None)
+    if y.dim() not in (1, 2) or y.size(0) != eid.size(0):
+        raise ValueError(f"y must be ({eid.size(0)},) or ({eid.size(0)}, h), got {tuple(y.shape)}")
+    _expect_shape(dy, y.shape, "dy")
     plan = plan_cache.get(row, indptr, eid, None, None, None)
     dx = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(dy)
     ws, nws = _workspace(OP_SOFTMAX_BWD, plan, None, _edge_h(dy), 1, _dtype(y), y.device)
@@ -198,8 +238,8 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None, out
     _check_all(row=row, indptr=indptr, eid=eid, indices=indices, edata=edata, x=x)
     _same_dtype(edata, x)
     h, d = _hd(x)
-    if _edge_h(edata) != h:
-        raise RuntimeError("edata and x disagree on the number of heads")
+    _expect_index(eid, indices)
+    _expect_edges(edata, eid.size(0), h, "edata", x.dim() == 2)
     n_out = x.size(0) if n_rows is None else int(n_rows)
     plan = plan_cache.get(row, indptr, eid, indices, n_out, x.size(0))
     y = torch.empty_like(x) if n_rows is None else torch.empty((n_out,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
@@ -227,6 +267,11 @@ def vector_spmm_backward(row, indptr, eid, indices, col, indptr_t, eid_t, indice
     dy = dy.contiguous()
     _same_dtype(edata, dy, x)
     h, d = _hd(x)
+    _expect_index(eid, indices)
+    _expect_index(eid_t, indices_t)
+    _expect_shape(eid_t, eid.shape, "eid_t")
+    _expect_edges(edata, eid.size(0), h, "edata", x.dim() == 2)
+    _expect_shape(dy, x.shape, "dy")
     plan = plan_cache.get(row, indptr, eid, indices, x.size(0), x.size(0))
     plan_t = plan_cache.get(col, indptr_t, eid_t, indices_t, x.size(0), x.size(0))
     dedata = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(edata)
@@ -257,6 +302,7 @@ def rel_bias_forward(col, indptr_c, eid_c, etype_slot, q, table):
     h, d = _hd(q)
     if table.dim() != 2 or table.size(1) != d:
         raise ValueError(f"table must be (n_types, {d})")
+    _expect_index(eid_c, etype_slot)
     plan = plan_cache.get(col, indptr_c, eid_c, etype_slot, q.size(0), table.size(0))
     E = eid_c.size(0)
     bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
@@ -285,10 +331,13 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     _check_bias(bias, eid_c.size(0), _hd(q)[0], q.device)
     _same_dtype(q, k, v)
     h, d = _hd(q)
+    _expect_index(eid_c, indices_c)
+    _expect_shape(k, (k.size(0),) + tuple(q.shape[1:]), "k")
+    _expect_shape(v, k.shape, "v")
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
     ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, dropout_p))["struct"]) \
-        if _attention_groups(plan, dropout_p, bias) else plan.ref
+        if _attention_groups(plan, dropout_p, bias, q, k) else plan.ref
     o = torch.empty_like(q)
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
@@ -309,6 +358,16 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     do = do.contiguous()
     _same_dtype(q, k, v, o, do)
     h, d = _hd(q)
+    _expect_index(eid_c, indices_c)
+    _expect_index(eid_r, indices_r)
+    _expect_shape(eid_r, eid_c.shape, "eid_r")
+    _expect_shape(k, (k.size(0),) + tuple(q.shape[1:]), "k")
+    _expect_shape(v, k.shape, "v")
+    _expect_shape(o, q.shape, "o")
+    _expect_shape(do, q.shape, "do")
+    if lse.dtype != torch.float32 or lse.device != q.device:
+        raise ValueError("lse must be the float32 tensor that attention_forward returned")
+    _expect_shape(lse, (q.size(0), h), "lse")
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
     plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0))
@@ -317,7 +376,7 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     ds = torch.empty((eid_c.size(0) + 1, h), dtype=torch.float32, device=q.device) if bias is not None else None
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref
-    if _attention_groups(plan_in, dropout_p, bias) and plan_in.covers_all_edges and plan_out.covers_all_edges:
+    if _attention_groups(plan_in, dropout_p, bias, q, k) and plan_in.covers_all_edges and plan_out.covers_all_edges:
         R = _group_rows(q, h, d, plan_in)
         in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
         out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
@@ -359,11 +418,16 @@ _USE_GROUPS = True
 _MIN_GROUP_ITEMS = 1536     # graphs with fewer work items run one wavefront per row (unless set_group_rows forces groups)
 
 
-def _attention_groups(plan, dropout_p, bias):
+def _attention_groups(plan, dropout_p, bias, q, k):
     """Whether the fused kernels take the row groups for this graph.  Very small graphs do not fill the GPU with one
     wavefront per group of rows and run faster with one per row (measured: L = 512, 0.055 against 0.070 ms per step;
-    even at L = 1024); dropout and the score term exist in the row-group kernels only."""
+    even at L = 1024); dropout and the score term exist in the row-group kernels only.  The row-group kernels address
+    the rows of q AND of k / v with 32-bit byte offsets, so both node tensors have to stay below 4 GiB."""
     if not _USE_GROUPS:
+        return False
+    if max(q.size(0), k.size(0)) * q.size(1) * q.size(2) * q.element_size() >= 2 ** 32:
+        if dropout_p > 0.0 or bias is not None:
+            raise RuntimeError("dropout and the score term need the row-group kernels, which address node tensors below 4 GiB")
         return False
     return plan.n_items >= _MIN_GROUP_ITEMS or _GROUP_ROWS is not None or dropout_p > 0.0 or bias is not None
 _GROUPED_OPS = True         # row groups also in the unfused SpMM / SDDMM ops (set_grouped_ops)

@@ -1,0 +1,88 @@
+"""The benchmark configurations at their full sizes: fused attention forward + backward on the GPU against the
+float64 CPU oracle on the same seeded inputs (q, k, v, grad-out = N(0,1) / sqrt(64) drawn in that order from seed
+2345, all nodes), with the stated tolerances applied as they stand: float32 outputs rtol 1e-5 / atol 1e-5, gradients
+rtol 1e-4 (atol 1e-5); bfloat16 rtol 2e-2 (atol 2e-2).
+
+  configuration 2: 32 causal graphs, lengths uniform in [64, 1024] (seed 2345), k = 4, merged block-diagonally
+  configuration 3 in bfloat16: L = 8192, k = 4, causal (float32: tests/test_gpu_parity.py::test_headline_graph_full_parity)
+  configuration 4: L = 4096, causal, k in {1, 2, 4, 8, 16, 32}, and the window-128 graph (FullyConnected)
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL = {torch.float32: dict(rtol=1e-5, atol=1e-5), torch.bfloat16: dict(rtol=2e-2, atol=2e-2)}
+GTOL = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=2e-2, atol=2e-2)}
+
+
+def f64(t):
+    return t.detach().cpu().to(torch.float64).numpy()
+
+
+def check(got, want, tol, what):
+    got = f64(got)
+    err = np.abs(got - want)
+    bound = tol["atol"] + tol["rtol"] * np.abs(want)
+    assert got.shape == want.shape and np.all(err <= bound), f"{what}: max err {err.max():.3e}, worst excess {(err - bound).max():.3e}"
+
+
+def run_layer(src, dst, n, h, d, dtype):
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd import op
+    csr = gb.get_csrs(src, dst, n, as_torch=False)
+    out_csr, in_csr, ROW, IR, COL, IC = csr
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    args = (t(ROW), t(IR), t(out_csr[2]), t(out_csr[1]), t(COL), t(IC), t(in_csr[2]), t(in_csr[1]))
+    gen = torch.Generator().manual_seed(2345)
+    q, k, v, do = ((torch.randn(n, h, d, generator=gen) / 8).to(dtype) for _ in range(4))
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    o = op.bpt_attention(*args, qd, kd, vd, fused=True)
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    ro, ra = oracle.attention_forward(csr, f64(q), f64(k), f64(v))
+    rdq, rdk, rdv = oracle.attention_backward(csr, f64(q), f64(k), f64(v), ra, f64(do))
+    check(o, ro, TOL[dtype], "o")
+    for got, want, nm in ((qd.grad, rdq, "dq"), (kd.grad, rdk, "dk"), (vd.grad, rdv, "dv")):
+        check(got, want, GTOL[dtype], nm)
+    return o
+
+
+def test_cfg2_batch_of_32_graphs_fp32():
+    from bpt_amd import graphbuilder as gb
+    lengths = np.random.default_rng(2345).integers(64, 1025, 32)
+    assert int(lengths.sum()) == 16736 and lengths[0] == 171 and lengths[-1] == 105
+    cache = {}
+    graphs = [cache.setdefault(int(L), gb.BinaryPartition(int(L), True, 4, 10)) for L in lengths]
+    src, dst, _, _, n = gb.merge_graphs(graphs)
+    assert (n, len(src)) == (33598, 573520)
+    run_layer(src, dst, n, 8, 64, torch.float32)
+
+
+def test_cfg3_bf16_full_size():
+    from bpt_amd import graphbuilder as gb
+    g = gb.BinaryPartition(8192, True, 4, 10)
+    src, dst, _ = g.get_edges()
+    assert (g.number_of_nodes, len(src)) == (16383, 430237)
+    run_layer(src, dst, g.number_of_nodes, 8, 64, torch.bfloat16)
+
+
+@pytest.mark.parametrize("k,n_edges", [(1, 98305), (2, 133148), (4, 194705), (8, 301659), (16, 483591), (32, 784687)])
+def test_cfg4_partition_width_sweep_fp32(k, n_edges):
+    from bpt_amd import graphbuilder as gb
+    g = gb.BinaryPartition(4096, True, k, 10)
+    src, dst, _ = g.get_edges()
+    assert (g.number_of_nodes, len(src)) == (8191, n_edges)
+    run_layer(src, dst, g.number_of_nodes, 8, 64, torch.float32)
+
+
+def test_cfg4_window_128_fp32():
+    from bpt_amd import graphbuilder as gb
+    g = gb.FullyConnected(4096, True, 128)
+    src, dst, _ = g.get_edges()
+    assert (g.number_of_nodes, len(src)) == (4097, 524224)
+    run_layer(src, dst, g.number_of_nodes, 8, 64, torch.float32)

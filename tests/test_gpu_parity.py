@@ -126,9 +126,11 @@ GTOL = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.float64: dict(rtol=1e-1
 
 
 def close(got, want, tol, what, terms=1):
-    """|got - want| <= atol * max(1, terms / 64) + rtol * |want|.  `terms` = the longest sum behind an element: the
-    absolute floor of a float32 (or bf16-stored) sum of unnormalised N(0,1) products grows with its length, while
-    the stated atol is for attention-like sums of up to 64 terms."""
+    """|got - want| <= atol * max(1, terms / 64) + rtol * |want|.  The stated tolerances are applied literally
+    (terms = 1) to every output of the attention layer, normalised or not: o, dq, dk, dv, the softmax and the SpMM
+    of softmax weights.  `terms` is passed only where a test feeds an op UNNORMALISED N(0,1) edge weights, so that
+    an element is a raw sum of up to `terms` products of size ~1 whose float32 rounding floor grows with its length
+    (the stated atol is for attention-like sums); every such call says so."""
     got = f64(got)
     assert got.shape == want.shape, (what, got.shape, want.shape)
     err = np.abs(got - want)
@@ -183,6 +185,7 @@ def test_ops_match_oracle(ops, gname, chunk, hd, dtype, kernels):
         close(y, oracle.maskedmm_csr_forward(*c.np_out, f64(A), f64(B)), tol, "maskedmm fwd")
         dA, dB = graphop.maskedmm_csr_backward(*c.out, *c.inn, A, B, w)
         rA, rB = oracle.maskedmm_csr_backward(*c.np_out, *c.np_in, f64(A), f64(B), f64(w))
+        # dy = unnormalised N(0,1) per edge: dA / dB are raw sums of up to max_deg such products (terms)
         close(dA, rA, gtol, "maskedmm dA", c.max_deg); close(dB, rB, gtol, "maskedmm dB", c.max_deg)
         # edge softmax over in-edges
         a = graphop.sparse_softmax_forward(*c.inn[:3], w)
@@ -190,17 +193,20 @@ def test_ops_match_oracle(ops, gname, chunk, hd, dtype, kernels):
         close(a, ra, tol, "softmax fwd")
         dx = graphop.sparse_softmax_backward(*c.inn[:3], a, w)
         close(dx, oracle.sparse_softmax_backward(*c.np_in[:3], f64(a), f64(w), n_nodes=n), gtol, "softmax bwd")
-        # SpMM over the in-CSR
-        o = graphop.vector_spmm_forward(*c.inn, w, A)
-        close(o, oracle.vector_spmm_forward(*c.np_in, f64(w), f64(A)), tol if dtype != torch.float32 else gtol, "spmm fwd", c.max_deg)
+        # SpMM over the in-CSR, as the layer calls it: the edge weights are the softmax output (rows sum to 1), so
+        # the forward is held to the stated output tolerance as it stands
+        o = graphop.vector_spmm_forward(*c.inn, a, A)
+        close(o, oracle.vector_spmm_forward(*c.np_in, f64(a), f64(A)), tol, "spmm fwd")
         dw, dxx = graphop.vector_spmm_backward(*c.inn, *c.out, w, gy, A)
         rdw, rdx = oracle.vector_spmm_backward(*c.np_in, *c.np_out, f64(w), f64(gy), f64(A))
+        # dedata is one dot product per edge; dx sums up to max_deg products of unnormalised N(0,1) weights: terms
         close(dw, rdw, gtol, "spmm dedata"); close(dxx, rdx, gtol, "spmm dx", c.max_deg)
         # node . edge (rel-pos term), in-CSR, A = q
         yn = graphop.node_mul_edge_forward(*c.inn[:3], A, Be)
         close(yn, oracle.node_mul_edge_forward(*c.np_in[:3], f64(A), f64(Be)), tol, "node_mul_edge fwd")
         dAn, dBe = graphop.node_mul_edge_backward(*c.inn[:3], A, Be, w)
         rAn, rBe = oracle.node_mul_edge_backward(*c.np_in[:3], f64(A), f64(Be), f64(w))
+        # dA: raw sum of up to max_deg products of unnormalised N(0,1) edge gradients (terms); dB: h products
         close(dAn, rAn, gtol, "node_mul_edge dA", c.max_deg); close(dBe, rBe, gtol, "node_mul_edge dB")
     finally:
         graphop.set_force_generic(False)
@@ -433,10 +439,10 @@ def test_fused_attention_dropout_matches_oracle_with_the_same_mask(ops, gname, r
     t64 = lambda x: x.detach().cpu().double()
     src, dst = torch.from_numpy(c.src), torch.from_numpy(c.dst)
     ro, rdq, rdk, rdv = torch_ops.attention_fwd_bwd(src, dst, t64(q), t64(k), t64(v), t64(do), drop=mask.double())
-    close(o, ro.numpy(), TOL[dtype], "o", c.max_deg)
-    close(q.grad, rdq.numpy(), GTOL[dtype], "dq", c.max_deg)
-    close(k.grad, rdk.numpy(), GTOL[dtype], "dk", c.max_deg)
-    close(v.grad, rdv.numpy(), GTOL[dtype], "dv", c.max_deg)
+    close(o, ro.numpy(), TOL[dtype], "o")
+    close(q.grad, rdq.numpy(), GTOL[dtype], "dq")
+    close(k.grad, rdk.numpy(), GTOL[dtype], "dk")
+    close(v.grad, rdv.numpy(), GTOL[dtype], "dv")
 
 
 # --------------------------------------------------------------------------------------------
@@ -472,11 +478,11 @@ def test_fused_attention_with_rel_pos_matches_oracle(ops, gname, rows, dtype, hd
     ro, rdq, rdk, rdv, rdak = torch_ops.attention_fwd_bwd(src, dst, t64(q), t64(k), t64(v), t64(do), ak=t64(table)[et],
                                                           drop=mask.double() if mask is not None else None)
     rdt = torch.zeros(n_types, d, dtype=torch.float64).index_add_(0, et, rdak)
-    close(o, ro.numpy(), TOL[dtype], "o", c.max_deg)
-    close(q.grad, rdq.numpy(), GTOL[dtype], "dq", c.max_deg)
-    close(k.grad, rdk.numpy(), GTOL[dtype], "dk", c.max_deg)
-    close(v.grad, rdv.numpy(), GTOL[dtype], "dv", c.max_deg)
-    # a table row sums over all edges of its type and all heads
+    close(o, ro.numpy(), TOL[dtype], "o")
+    close(q.grad, rdq.numpy(), GTOL[dtype], "dq")
+    close(k.grad, rdk.numpy(), GTOL[dtype], "dk")
+    close(v.grad, rdv.numpy(), GTOL[dtype], "dv")
+    # a table row is a raw sum over all edges of its type and all heads (h * E / n_types products): terms
     close(table.grad, rdt.numpy(), GTOL[dtype], "dtable", h * c.E / n_types)
 
 
@@ -496,7 +502,7 @@ def test_rel_pos_without_row_groups_takes_the_op_chain_and_the_raw_call_refuses(
             graphop.attention_forward(*c.inn, q, k, v, bias=bias)
     finally:
         graphop.set_row_groups(old)
-    close(got, f64(want), TOL[torch.float32], "chain vs fused", c.max_deg)
+    close(got, f64(want), TOL[torch.float32], "chain vs fused")
     with pytest.raises(ValueError):
         graphop.attention_forward(*c.inn, q, k, v, bias=torch.zeros((c.E, h), dtype=torch.float32, device=DEV))   # no spare row
     with pytest.raises(ValueError):
@@ -584,10 +590,10 @@ def test_attention_to_memory_over_an_inter_graph(ops, n_enc, n_dec, dtype):
     o.backward(do)
     t64 = lambda x: x.detach().cpu().double()
     ro, rdq, rdk, rdv = torch_ops.attention_fwd_bwd(torch.from_numpy(src), torch.from_numpy(dst), t64(q), t64(k), t64(v), t64(do))
-    close(o, ro.numpy(), TOL[dtype], "o", 70)
-    close(q.grad, rdq.numpy(), GTOL[dtype], "dq", 70)
-    close(k.grad, rdk.numpy(), GTOL[dtype], "dk", 70)
-    close(v.grad, rdv.numpy(), GTOL[dtype], "dv", 70)
+    close(o, ro.numpy(), TOL[dtype], "o")
+    close(q.grad, rdq.numpy(), GTOL[dtype], "dq")
+    close(k.grad, rdk.numpy(), GTOL[dtype], "dk")
+    close(v.grad, rdv.numpy(), GTOL[dtype], "dv")
     assert not o[min(n_dec, 101):].any()             # rows without in-edges (span nodes, padding) stay zero
 
 
@@ -607,6 +613,7 @@ def test_vector_spmm_accumulates_into_out(ops, dtype, grouped):
         out = y0.clone()
         got = graphop.vector_spmm_forward(*c.inn, w, x, out=out)
         assert got is out
+        # unnormalised N(0,1) edge weights: an element is a raw sum of up to max_deg products (terms)
         close(got, want, GTOL[dtype] if dtype == torch.float32 else TOL[dtype], "spmm accumulate", c.max_deg)
         with pytest.raises(ValueError):
             graphop.vector_spmm_forward(*c.inn, w, x, out=y0[:-1])

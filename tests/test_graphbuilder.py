@@ -131,3 +131,32 @@ def test_batch_merge_cfg2_shape():
     osrc, odst, oet, opos, on = oracle.merge_graphs(ogs)
     assert np.array_equal(src[:len(osrc)], osrc) and np.array_equal(dst[:len(osrc)], odst)
     assert np.array_equal(et[:len(osrc)], oet) and np.array_equal(pos[:on], opos)
+
+
+@pytest.mark.parametrize("L,triu,step", [(37, False, 2), (100, True, 4), (5, False, 1)])
+def test_get_csrs_src_ordered_in_csr(L, triu, step):
+    """The opt-in in-CSR order (source, edge id): same indptr, same (index, edge id) pairs per row as the default,
+    rows sorted by (source, edge id), which is what scipy's transpose of the out-CSR produces; out-CSR unchanged."""
+    import scipy.sparse as sp
+    g = gb.BinaryPartition(L, triu, step, 10)        # the non-causal graphs carry duplicate edges
+    src, dst, _ = g.get_edges()
+    n = g.number_of_nodes
+    base = gb.get_csrs(src, dst, n, as_torch=False)
+    alt = gb.get_csrs(src, dst, n, as_torch=False, in_order="src_eid")
+    for a, b in zip(base[0] + base[2:], alt[0] + alt[2:]):
+        assert np.array_equal(a, b)                                       # out-CSR and the units of both sides
+    (ip0, ix0, e0), (ip1, ix1, e1) = base[1], alt[1]
+    assert np.array_equal(ip0, ip1)
+    for r in range(n):
+        a, b = slice(ip0[r], ip0[r + 1]), slice(ip1[r], ip1[r + 1])
+        assert sorted(zip(ix0[a], e0[a])) == list(zip(ix1[b], e1[b]))      # same pairs, (source, edge id) ascending
+        assert np.all(np.diff(e0[a]) > 0)                                  # default: ascending edge id
+    assert np.array_equal(src[e1], ix1) and np.array_equal(dst[e1], np.repeat(np.arange(n), np.diff(ip1)))
+    # independent construction: CSR of (dst, src) with data = edge id + 1, duplicates kept, columns sorted stably
+    m = sp.csr_matrix((np.arange(len(src)) + 1, (dst, src)), shape=(n, n))
+    assert m.nnz == len(src) or not triu          # scipy sums duplicates in the constructor: only compare without them
+    if m.nnz == len(src):
+        m.sort_indices()
+        assert np.array_equal(m.indptr, ip1) and np.array_equal(m.indices, ix1) and np.array_equal(m.data - 1, e1)
+    with pytest.raises(ValueError):
+        gb.get_csrs(src, dst, n, in_order="random")

@@ -37,7 +37,7 @@ def _both_entries(n, args, h, d, dtype, seed):
     gen = torch.Generator().manual_seed(seed)
     q, k, v = ((torch.randn(n, h, d, generator=gen) / 8).to(dtype).to(DEV) for _ in range(3))
     plan = plan_cache.get(*args, n, n)
-    if graphop._attention_groups(plan, 0.0, None):
+    if graphop._attention_groups(plan, 0.0, None, q, k):
         ref = ctypes.byref(plan.ensure_groups(graphop._forward_rows(q, h, d, plan))["struct"])
     else:
         ref = plan.ref
