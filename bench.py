@@ -6,7 +6,7 @@ gradients) over one synthetic graph batch, inputs resident in HBM.  Default work
 configuration (cfg3), L=8192 tokens, k=4, causal binary-partition graph, 8 heads x 64, fp32.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg1|cfg2|cfg5|cfg4-kN|cfg4-w128]
-                  [--dtype f32|bf16] [--no-cpu-baseline] [--no-graph]
+                  [--dtype f32|bf16] [--no-cpu-baseline] [--no-graph] [--block-layers N]
 
 Prints ONE JSON line on stdout (details go to stderr).  `value` = graph edges per second of the
 whole fwd+bwd step; `roofline` describes the dominant kernel, timed live with HIP events on the
@@ -100,7 +100,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only (no HIP graph replay)")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run three 256 MiB device-to-device copies (known HBM bytes) so counter runs can be scaled")
+                    help="accepted for older command lines: the 256 MiB device-to-device copies (known HBM bytes, by which "
+                         "counter runs are scaled) now run every time")
     ap.add_argument("--group-rows", type=int, default=None, choices=[4, 8], help="rows per wavefront group of the fused kernels (default: 8 where available, else 4)")
     ap.add_argument("--rows", action="store_true", help="fused kernels with one wavefront per row (no row groups)")
     ap.add_argument("--unfused", action="store_true", help="time the unfused op chain of the reference's surface")
@@ -110,11 +111,14 @@ def main():
     ap.add_argument("--plan", default="auto", choices=["auto", "host", "device"],
                     help="where launch plans and row groups are built: on the host (libbptgraph), on the GPU (libbptplan), "
                          "or by graph size and density (the library's default)")
-    ap.add_argument("--block-layers", type=int, default=0,
-                    help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the workload's graph")
+    ap.add_argument("--block-layers", type=int, default=None,
+                    help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the "
+                         "workload's graph, a few steps, reported as block_stack; default: 12 for the headline workload, else 0")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.block_layers is None:
+        args.block_layers = 12 if (args.workload == "cfg3" and not args.unfused and not args.rel_pos and not args.rows) else 0
 
     import numpy as np
     import torch
@@ -270,12 +274,24 @@ def main():
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                     "algorithmic_bytes": alg[dom], "avg_launch_ms": round(kernels[dom], 5)}
 
-    if args.calibrate_copy:
-        a = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
-        b = torch.empty_like(a)
-        for _ in range(3):
-            b.copy_(a)                    # reads 256 MiB and writes 256 MiB per launch
-        torch.cuda.synchronize()
+    # what this GPU's memory system delivers to a plain streaming kernel: device-to-device copies of 256 MiB (read +
+    # write = 512 MiB of HBM traffic per launch, far larger than the caches), timed with events on the current stream
+    a = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+    b = torch.empty_like(a)
+    for _ in range(3):
+        b.copy_(a)
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    for _ in range(10):
+        b.copy_(a)
+    c1.record()
+    torch.cuda.synchronize()
+    copy_gbs = 10 * 2 * a.numel() * 4 / (c0.elapsed_time(c1) * 1e-3) / 1e9
+    del a, b
+    log(f"measured device copy bandwidth: {copy_gbs:.0f} GB/s (read + write)")
+    if roofline is not None:
+        roofline["measured_copy_GBps"] = round(copy_gbs, 1)
+        roofline["frac_of_measured_copy"] = round(roofline["achieved"] / copy_gbs, 4)
 
     block = None
     if args.block_layers > 0 and not args.unfused:
@@ -296,7 +312,7 @@ def main():
             x.backward(gh)
             return x
 
-        t_stack = timed(stack_step, max(5, min(args.steps, 30)), 3)
+        t_stack = timed(stack_step, 5, 2)
         block = {"layers": args.block_layers, "d_model": dm, "d_ff": 4 * dm, "ms_per_layer_fwd_bwd": round(t_stack / args.block_layers * 1e3, 4),
                  "attention_ms_per_layer": round(t_step * 1e3, 4), "attention_share": round(t_step * args.block_layers / t_stack, 3)}
         log(f"block stack: {block}")
@@ -318,7 +334,8 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "step_roofline": {"algorithmic_bytes": alg["total"], "achieved_GBps": round(step_gbs, 1),
-                          "frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4)},
+                          "frac_of_hbm_peak": round(step_gbs / HBM_PEAK_GBS, 4),
+                          "measured_copy_GBps": round(copy_gbs, 1), "frac_of_measured_copy": round(step_gbs / copy_gbs, 4)},
         "ms_per_step_eager": t_eager * 1e3,
         "ms_per_step_graph": None if t_graph_replay is None else t_graph_replay * 1e3,
         "kernel_ms": {k_: round(v_, 5) for k_, v_ in kernels.items()},

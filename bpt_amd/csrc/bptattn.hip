@@ -2753,7 +2753,8 @@ int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, co
     if ((drop.thr != 0 || bias) && !grouped_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
     if ((bias != nullptr) != (ds_out != nullptr)) return BPT_ERR_NULL;       // the score term and its gradient go together
     if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
-    if (plan_in->n_edges != plan_out->n_edges || plan_in->n_rows != plan_out->n_rows) return BPT_ERR_PLAN;
+    // (the two sides may have different row counts: attention to a memory of another length, attention.py:144-168)
+    if (plan_in->n_edges != plan_out->n_edges) return BPT_ERR_PLAN;
     if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return BPT_ERR_NULL;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) ||
         !aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !aligned16(workspace))

@@ -11,7 +11,8 @@ import numpy as np
 from ._lib import check_graph, graph_lib
 
 __all__ = ["BinaryPartition", "FullyConnected", "OpenAISparse", "partition_csr",
-           "build_csr", "get_csrs", "merge_graphs", "get_csrs_device", "merge_graphs_device"]
+           "build_csr", "get_csrs", "merge_graphs", "get_csrs_device", "merge_graphs_device",
+           "inter_graph_edges", "nli_inter_graph_edges", "get_csrs_bipartite"]
 
 
 def _ptr(a):
@@ -190,6 +191,91 @@ def get_csrs(src, dst, n_nodes, chunk_size=32, as_torch=True, in_order="eid"):
         t = torch.from_numpy
         res = (tuple(map(t, out_csr)), tuple(map(t, in_csr)), t(ROW), t(INDPTR_R), t(COL), t(INDPTR_C))
     return res
+
+
+def get_csrs_bipartite(src, dst, n_src, n_dst, chunk_size=32, as_torch=True):
+    """get_csrs for a bipartite graph whose two sides have index spaces of their own (sources 0 .. n_src - 1, the
+    keys / values of an attention to memory; destinations 0 .. n_dst - 1, its queries): the out-CSR has n_src rows,
+    the in-CSR n_dst.  The reference stores such a graph in one square index space of max(n_src, n_dst) nodes
+    (graph/mt.py:340-344) and pads the shorter node tensor (modules/attention.py:148-149); get_csrs(src, dst,
+    max(n_src, n_dst)) gives that form, and the ops accept both."""
+    src = np.ascontiguousarray(src, dtype=np.int64)
+    dst = np.ascontiguousarray(dst, dtype=np.int64)
+    if src.shape != dst.shape or src.ndim != 1:
+        raise ValueError("src and dst must be 1-D arrays of the same length")
+    if len(src) and (src.min() < 0 or dst.min() < 0 or src.max() >= n_src or dst.max() >= n_dst):
+        raise ValueError("node id out of range")
+
+    def side(rows, cols, n_rows):          # stable sort by row = ascending edge id inside a row, as build_csr
+        eid = np.argsort(rows, kind="stable").astype(np.int64)
+        indptr = np.zeros(n_rows + 1, dtype=np.int64)
+        np.cumsum(np.bincount(rows, minlength=n_rows), out=indptr[1:])
+        return indptr, np.ascontiguousarray(cols[eid]), eid
+
+    out_csr = side(src, dst, int(n_src))
+    in_csr = side(dst, src, int(n_dst))
+    ROW, INDPTR_R = partition_csr(out_csr[0], chunk_size)
+    COL, INDPTR_C = partition_csr(in_csr[0], chunk_size)
+    res = (out_csr, in_csr, ROW, INDPTR_R, COL, INDPTR_C)
+    if as_torch:
+        import torch
+        t = torch.from_numpy
+        res = (tuple(map(t, out_csr)), tuple(map(t, in_csr)), t(ROW), t(INDPTR_R), t(COL), t(INDPTR_C))
+    return res
+
+
+def _segments(seg, length):
+    seg = [0, length] if seg is None else [int(x) for x in seg]
+    if len(seg) < 2 or seg[0] < 0 or seg[-1] > length or any(b < a for a, b in zip(seg, seg[1:])):
+        raise ValueError("segment boundaries must be non-decreasing positions inside the sequence")
+    return seg
+
+
+def inter_graph_edges(enc_graphs, dec_graphs, enc_segments=None, dec_segments=None):
+    """Edges of the encoder -> decoder graph of a batch of sequence pairs, graph/mt.py:286-321: for pair b and
+    segment i, every token (leaf node) of the source sentence's segment i is connected to every token of the target
+    sentence's segment i; node ids are those of the merged encoder graph (sources) and of the merged decoder graph
+    (destinations), i.e. the sequences' leaf ids shifted by the node counts of the graphs before them.
+    enc_segments / dec_segments: per pair a list of boundaries [s_0, s_1, ...] (segment i = tokens s_i .. s_{i+1} - 1),
+    or None for one segment covering the whole sentence (mt.py:260-262).
+    Returns (src, dst, n_enc, n_dec): int64 edge list in the reference's order and the two node counts; the
+    reference's square form is get_csrs(src, dst, max(n_enc, n_dec)) (mt.py:340-344)."""
+    if len(enc_graphs) != len(dec_graphs):
+        raise ValueError("one encoder graph per decoder graph")
+    enc_segments = enc_segments or [None] * len(enc_graphs)
+    dec_segments = dec_segments or [None] * len(dec_graphs)
+    rows, cols, ve, vd = [], [], 0, 0
+    for ge, gd, se, sd in zip(enc_graphs, dec_graphs, enc_segments, dec_segments):
+        se, sd = _segments(se, len(ge.leaf_ids())), _segments(sd, len(gd.leaf_ids()))
+        if len(se) != len(sd):
+            raise ValueError("source and target must have the same number of segments")
+        for i in range(1, len(se)):
+            a = np.arange(ve + se[i - 1], ve + se[i], dtype=np.int64)
+            b = np.arange(vd + sd[i - 1], vd + sd[i], dtype=np.int64)
+            rows.append(np.repeat(a, len(b)))
+            cols.append(np.tile(b, len(a)))
+        ve += ge.number_of_nodes
+        vd += gd.number_of_nodes
+    cat = lambda xs: np.concatenate(xs) if xs else np.empty(0, dtype=np.int64)
+    return cat(rows), cat(cols), ve, vd
+
+
+def nli_inter_graph_edges(premise_graphs, hypo_graphs):
+    """Edges of the inter graph of graph/nli.py:60-99: premise and hypothesis of a pair are laid out one after the other
+    in ONE node index space; every premise token is connected to every hypothesis token and back.
+    Returns (src, dst, n_nodes)."""
+    if len(premise_graphs) != len(hypo_graphs):
+        raise ValueError("one premise graph per hypothesis graph")
+    rows, cols, v = [], [], 0
+    for gp, gh in zip(premise_graphs, hypo_graphs):
+        a = gp.leaf_ids(v_shift=v).astype(np.int64)
+        v += gp.number_of_nodes
+        b = gh.leaf_ids(v_shift=v).astype(np.int64)
+        v += gh.number_of_nodes
+        rows += [np.repeat(a, len(b)), np.repeat(b, len(a))]
+        cols += [np.tile(b, len(a)), np.tile(a, len(b))]
+    cat = lambda xs: np.concatenate(xs) if xs else np.empty(0, dtype=np.int64)
+    return cat(rows), cat(cols), v
 
 
 def get_csrs_device(src, dst, n_nodes, chunk_size=32):

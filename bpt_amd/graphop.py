@@ -271,9 +271,10 @@ def vector_spmm_backward(row, indptr, eid, indices, col, indptr_t, eid_t, indice
     _expect_index(eid_t, indices_t)
     _expect_shape(eid_t, eid.shape, "eid_t")
     _expect_edges(edata, eid.size(0), h, "edata", x.dim() == 2)
-    _expect_shape(dy, x.shape, "dy")
-    plan = plan_cache.get(row, indptr, eid, indices, x.size(0), x.size(0))
-    plan_t = plan_cache.get(col, indptr_t, eid_t, indices_t, x.size(0), x.size(0))
+    # y = dy may have another number of rows than x (a rectangular operator: attention to a memory of another length)
+    _expect_shape(dy, (dy.size(0),) + tuple(x.shape[1:]), "dy")
+    plan = plan_cache.get(row, indptr, eid, indices, dy.size(0), x.size(0))
+    plan_t = plan_cache.get(col, indptr_t, eid_t, indices_t, x.size(0), dy.size(0))
     dedata = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(edata)
     dx = torch.empty_like(x)
     dt = _dtype(x)

@@ -60,8 +60,9 @@ class NodeMulEdge(Function):
 class VectorSPMM(Function):
     # modules/op.py:47-58
     @staticmethod
-    def forward(ctx, row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x):
-        y = vector_spmm_forward(row, indptr, eid, indices, edata, x)
+    def forward(ctx, row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x, n_rows=None):
+        # n_rows (not in the reference): rows of y when the operator is rectangular (y = zeros_like(x) there, :527)
+        y = vector_spmm_forward(row, indptr, eid, indices, edata, x, n_rows=n_rows)
         ctx.save_for_backward(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x)
         return y
 
@@ -69,7 +70,7 @@ class VectorSPMM(Function):
     def backward(ctx, dy):
         row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x = ctx.saved_tensors
         dedata, dx = vector_spmm_backward(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, dy, x)
-        return None, None, None, None, None, None, None, None, dedata, dx
+        return None, None, None, None, None, None, None, None, dedata, dx, None
 
 
 class BPTAttention(Function):
@@ -159,8 +160,8 @@ def node_mul_edge(row, indptr, eid, A, B):
     return NodeMulEdge.apply(row, indptr, eid, A, B)
 
 
-def vec_spmm(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x):
-    return VectorSPMM.apply(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x)
+def vec_spmm(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x, n_rows=None):
+    return VectorSPMM.apply(row, indptr, eid, indices, col, ptr_t, eid_t, indices_t, edata, x, n_rows)
 
 
 class EdgeTypeEmbedding(Function):
@@ -231,7 +232,7 @@ def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices
     if (rel_table is None) != (etype is None):
         raise ValueError("rel_table and etype go together")
     if fused is None:
-        fused = _g.attention_supported(q) and q.size(0) == k.size(0)
+        fused = _g.attention_supported(q)
         if (dropout_p > 0 or rel_table is not None) and not _g.row_groups_enabled():
             fused = False                       # only the row-group kernels implement dropout and the rel_pos term
     if fused:
@@ -246,4 +247,5 @@ def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices
     if rel_table is not None:
         e = e + node_mul_edge(col, indptr_c, eid_c, q, edge_type_embedding(rel_table, etype))
     a = torch.nn.functional.dropout(sparse_softmax(col, indptr_c, eid_c, e * scale), p=float(dropout_p), training=dropout_p > 0)
-    return vec_spmm(col, indptr_c, eid_c, indices_c, row, indptr_r, eid_r, indices_r, a, v)
+    return vec_spmm(col, indptr_c, eid_c, indices_c, row, indptr_r, eid_r, indices_r, a, v,
+                    n_rows=None if q.size(0) == v.size(0) else q.size(0))

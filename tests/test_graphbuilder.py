@@ -160,3 +160,51 @@ def test_get_csrs_src_ordered_in_csr(L, triu, step):
         assert np.array_equal(m.indptr, ip1) and np.array_equal(m.indices, ix1) and np.array_equal(m.data - 1, e1)
     with pytest.raises(ValueError):
         gb.get_csrs(src, dst, n, in_order="random")
+
+
+def test_inter_graph_edges_follow_the_reference_construction():
+    """graph/mt.py:286-321: per sentence pair and segment, np.repeat(source tokens, #target) / np.tile(target tokens,
+    #source), node ids shifted by the node counts of the graphs before; graph/nli.py:60-87 for the two-way form."""
+    enc = [gb.BinaryPartition(7, False, 2, 10), gb.BinaryPartition(12, False, 2, 10), gb.BinaryPartition(3, False, 2, 10)]
+    dec = [gb.BinaryPartition(5, True, 2, 10), gb.BinaryPartition(9, True, 2, 10), gb.BinaryPartition(4, True, 2, 10)]
+    seg_e = [None, [0, 4, 12], None]
+    seg_d = [None, [0, 6, 9], None]
+    src, dst, n_enc, n_dec = gb.inter_graph_edges(enc, dec, seg_e, seg_d)
+    assert n_enc == sum(g.number_of_nodes for g in enc) and n_dec == sum(g.number_of_nodes for g in dec)
+    # brute force from the definition: (s, t) for every source token s and target token t of the same pair and segment
+    want, ve, vd = [], 0, 0
+    for ge, gd, se, sd in zip(enc, dec, seg_e, seg_d):
+        le, ld = len(ge.leaf_ids()), len(gd.leaf_ids())
+        se, sd = se or [0, le], sd or [0, ld]
+        for i in range(1, len(se)):
+            for s in range(se[i - 1], se[i]):
+                for t in range(sd[i - 1], sd[i]):
+                    want.append((ve + s, vd + t))
+        ve += ge.number_of_nodes
+        vd += gd.number_of_nodes
+    assert list(zip(src.tolist(), dst.tolist())) == want
+    assert len(src) == 7 * 5 + 4 * 6 + 8 * 3 + 3 * 4
+    # only tokens carry inter edges: span nodes of both sides have none
+    leaf_e = np.concatenate([g.leaf_ids(v_shift=s) for g, s in zip(enc, np.cumsum([0] + [g.number_of_nodes for g in enc[:-1]]))])
+    assert set(src.tolist()) <= set(leaf_e.tolist())
+    # square (reference) and bipartite CSR forms describe the same edges
+    sq = gb.get_csrs(src, dst, max(n_enc, n_dec), as_torch=False)
+    bi = gb.get_csrs_bipartite(src, dst, n_enc, n_dec, as_torch=False)
+    assert len(bi[0][0]) == n_enc + 1 and len(bi[1][0]) == n_dec + 1
+    assert np.array_equal(sq[0][0][:n_enc + 1], bi[0][0]) and np.array_equal(sq[1][0][:n_dec + 1], bi[1][0])
+    assert np.array_equal(sq[0][1], bi[0][1]) and np.array_equal(sq[1][2], bi[1][2])
+    with pytest.raises(ValueError):
+        gb.inter_graph_edges(enc, dec[:2])
+    with pytest.raises(ValueError):
+        gb.inter_graph_edges(enc[:1], dec[:1], [[0, 3, 7]], [[0, 5]])
+    with pytest.raises(ValueError):
+        gb.get_csrs_bipartite(src, dst, n_enc, int(dst.max()))
+
+    prem = [gb.BinaryPartition(4, False, 1, 10), gb.BinaryPartition(6, False, 1, 10)]
+    hypo = [gb.BinaryPartition(3, False, 1, 10), gb.BinaryPartition(2, False, 1, 10)]
+    s2, d2, n2 = gb.nli_inter_graph_edges(prem, hypo)
+    assert n2 == sum(g.number_of_nodes for g in prem + hypo) and len(s2) == 2 * (4 * 3 + 6 * 2)
+    pairs = set(zip(s2.tolist(), d2.tolist()))
+    assert len(pairs) == len(s2) and all((b, a) in pairs for a, b in pairs)                  # two-way, no duplicates
+    v0 = prem[0].number_of_nodes
+    assert (0, v0) in pairs and (v0 + 2, 3) in pairs and (4, v0) not in pairs                  # node 4 is a span node

@@ -80,7 +80,7 @@ def test_vector_spmm_checks(g):
     with pytest.raises(ValueError):
         g.vector_spmm_forward(*INN, torch.zeros(E), node())                   # (E,) goes with (n, d) tensors only
     with pytest.raises(ValueError):
-        g.vector_spmm_backward(*INN, *OUT, edge(), node(n=N - 1), node())     # dy has a row less than x
+        g.vector_spmm_backward(*INN, *OUT, edge(), node(d=32), node())        # dy has another head size than x
     with pytest.raises(ValueError):
         g.vector_spmm_backward(*INN, *OUT, edge(e=E - 1), node(), node())
 
@@ -113,3 +113,5 @@ def test_well_formed_calls_get_past_the_checks(g):
         g.attention_backward(*OUT, *INN, node(), node(n=N + 3), node(n=N + 3), node(), torch.zeros(N, H), node())
     with pytest.raises(AssertionError):
         g.vector_spmm_forward(*INN, torch.zeros(E), torch.zeros(N, D))        # single head: (E,) with (n, d)
+    with pytest.raises(AssertionError):
+        g.vector_spmm_backward(*INN, *OUT, edge(), node(n=N - 1), node())     # rectangular: y has other rows than x
