@@ -200,7 +200,7 @@ def main():
             t0 = time.perf_counter()
             pin = plan_mod.plan_cache.get(*gargs[4:], N, N)
             pout = plan_mod.plan_cache.get(*gargs[:4], N, N)
-            pin.ensure_groups(graphop._forward_rows(q, H, D, pin, args.dropout))
+            pin.ensure_groups(graphop._forward_rows(q, H, D, pin))
             pin.linked_to(pout, graphop._group_rows(q, H, D, pin))
             torch.cuda.synchronize()
             ts.append(time.perf_counter() - t0)

@@ -79,6 +79,8 @@ class BPTBlock(nn.Module):
             -1, self.d_k * self.h)
 
     def forward(self, h, csr, etype=None):
+        # three GEMMs: one strided-batched GEMM over the stacked weights (its (3, n, h * d_k) result holds q, k, v as the
+        # contiguous tensors the kernels need) measured slower, 3.38 against 3.17 ms per layer fwd+bwd at n = 16 383 in float32
         q = self.proj_q(h).view(-1, self.h, self.d_k)
         k = self.proj_k(h).view(-1, self.h, self.d_k)
         v = self.proj_v(h).view(-1, self.h, self.d_k)

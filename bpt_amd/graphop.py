@@ -10,8 +10,10 @@ Beyond the reference: bf16 tensors are accepted, `attention_forward/backward` ex
 SDDMM -> edge-softmax -> SpMM pass, and vector_spmm_backward returns the complete dx (the
 reference's launch drops trailing units of the transposed side, graphop_kernel.cu:566,588).
 """
+import collections
 import ctypes
 import math
+import threading
 
 import torch
 
@@ -22,6 +24,28 @@ __all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forwa
            "sparse_softmax_forward", "sparse_softmax_backward", "vector_spmm_forward", "vector_spmm_backward"]
 
 _LIB = attn_lib()          # fail at import time if the HIP library is missing
+
+
+class _Settings(collections.namedtuple("_Settings", "use_groups grouped_ops group_rows")):
+    """Which kernel family the ops take: use_groups (fused attention: one wavefront per group of rows that share
+    neighbours, or per row), grouped_ops (the same for the unfused SpMM / SDDMM ops), group_rows (None: chosen per call
+    from dtype and shape; 4 or 8: forced).  Immutable: the set_* hooks below replace the whole tuple under a lock, and
+    every op reads it ONCE on entry, so a call (forward on the Python thread, backward on autograd's) works with one
+    consistent set even if another thread flips a hook meanwhile.  The hooks are process-wide testing / measurement
+    aids, not per-thread state; every family computes the same results."""
+    __slots__ = ()
+
+
+_SETTINGS = _Settings(True, True, None)
+_SETTINGS_LOCK = threading.Lock()
+
+
+def _replace_setting(**kw):
+    global _SETTINGS
+    with _SETTINGS_LOCK:
+        old = _SETTINGS
+        _SETTINGS = old._replace(**kw)
+    return old
 
 _DTYPE = {torch.float32: 0, torch.float64: 1, torch.bfloat16: 2}
 OP_MASKEDMM_BWD, OP_NME_BWD, OP_SPMM_FWD, OP_SPMM_BWD, OP_ATTN_FWD, OP_ATTN_BWD, OP_SOFTMAX_FWD, OP_SOFTMAX_BWD = 1, 2, 3, 4, 5, 6, 7, 8
@@ -106,13 +130,13 @@ def _workspace(op, plan, plan_t, h, d, dt, device, plan_ref=None, plan_t_ref=Non
     return torch.empty(n, dtype=torch.uint8, device=device), n
 
 
-def _spmm_ref(plan, x, h, d):
+def _spmm_ref(plan, x, h, d, cfg):
     """The plan to hand a SpMM- or SDDMM-shaped op: with row groups (one load of a neighbour row per group entry instead of one
     per edge) where the row-group kernels apply, else the plain plan."""
-    if not (_USE_GROUPS and _GROUPED_OPS and attention_supported(x) and plan.covers_all_edges and plan.has_indices
+    if not (cfg.use_groups and cfg.grouped_ops and attention_supported(x) and plan.covers_all_edges and plan.has_indices
             and plan.n_edges > 0 and max(plan.n_rows, plan.n_index_nodes) * h * d * x.element_size() < 2 ** 32):
         return plan.ref
-    return ctypes.byref(plan.ensure_groups(_group_rows(x, h, d, plan), GROUP_ORDER_SRC)["struct"])
+    return ctypes.byref(plan.ensure_groups(_group_rows(x, h, d, plan, cfg), GROUP_ORDER_SRC)["struct"])
 
 
 def _edge_out(plan, shape, like):
@@ -122,6 +146,7 @@ def _edge_out(plan, shape, like):
 
 def maskedmm_csr_forward(row, indptr, eid, indices, A, B):
     """y[eid[p]] = <A[row], B[indices[p]]> per head (graphop.cpp:16-31, graphop_kernel.cu:269-304)."""
+    cfg = _SETTINGS
     _check_all(row=row, indptr=indptr, eid=eid, indices=indices, A=A, B=B)
     _same_dtype(A, B)
     h, d = _hd(A)
@@ -131,13 +156,14 @@ def maskedmm_csr_forward(row, indptr, eid, indices, A, B):
     e = eid.size(0)
     y = _edge_out(plan, (e,) if A.dim() == 2 else (e, h), A)
     with torch.cuda.device_of(A):
-        check_attn(_LIB.bpt_maskedmm_csr_forward(_spmm_ref(plan, A, h, d), _ptr(A), _ptr(B), _ptr(y), h, d, _dtype(A), _stream()),
+        check_attn(_LIB.bpt_maskedmm_csr_forward(_spmm_ref(plan, A, h, d, cfg), _ptr(A), _ptr(B), _ptr(y), h, d, _dtype(A), _stream()),
                    "maskedmm_csr_forward")
     return y
 
 
 def maskedmm_csr_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, A, B, dy):
     """[dA, dB] (graphop.cpp:108-139, graphop_kernel.cu:355-409)."""
+    cfg = _SETTINGS
     _check_all(row=row, indptr_r=indptr_r, eid_r=eid_r, indices_r=indices_r, col=col, indptr_c=indptr_c,
                eid_c=eid_c, indices_c=indices_c, A=A, B=B)
     dy = dy.contiguous()
@@ -154,7 +180,7 @@ def maskedmm_csr_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c,
     dt = _dtype(A)
     ws, nws = _workspace(OP_MASKEDMM_BWD, plan_r, plan_c, h, d, dt, A.device)
     with torch.cuda.device_of(A):
-        check_attn(_LIB.bpt_maskedmm_csr_backward(_spmm_ref(plan_r, A, h, d), _spmm_ref(plan_c, A, h, d), _ptr(A), _ptr(B), _ptr(dy), _ptr(dA), _ptr(dB),
+        check_attn(_LIB.bpt_maskedmm_csr_backward(_spmm_ref(plan_r, A, h, d, cfg), _spmm_ref(plan_c, A, h, d, cfg), _ptr(A), _ptr(B), _ptr(dy), _ptr(dA), _ptr(dB),
                                                   _ptr(ws), nws, h, d, dt, _stream()), "maskedmm_csr_backward")
     return [dA, dB]
 
@@ -235,6 +261,7 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None, out
     rectangular operator, used for the segment sums of the relative-position table's gradient.
     out (keyword only, not in the reference): a contiguous tensor of y's shape that the sum is ADDED to and that is
     returned (in the kernel's store where the row-group kernels apply, else by a separate addition)."""
+    cfg = _SETTINGS
     _check_all(row=row, indptr=indptr, eid=eid, indices=indices, edata=edata, x=x)
     _same_dtype(edata, x)
     h, d = _hd(x)
@@ -248,7 +275,7 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None, out
     if out is not None and (out.shape != y.shape or out.dtype != y.dtype or out.device != y.device or not out.is_contiguous()):
         raise ValueError("out must be a contiguous tensor of the result's shape, dtype and device")
     with torch.cuda.device_of(x):
-        ref = _spmm_ref(plan, x, h, d)
+        ref = _spmm_ref(plan, x, h, d, cfg)
         if out is not None:
             st = _LIB.bpt_vector_spmm_accumulate(ref, _ptr(edata), _ptr(x), _ptr(out), _ptr(ws), nws, h, d, dt, _stream())
             if st == 0:
@@ -262,6 +289,7 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None, out
 
 def vector_spmm_backward(row, indptr, eid, indices, col, indptr_t, eid_t, indices_t, edata, dy, x):
     """[dedata, dx] (graphop.cpp:190-214, graphop_kernel.cu:544-600; dx over all units of the transposed side)."""
+    cfg = _SETTINGS
     _check_all(row=row, indptr=indptr, eid=eid, indices=indices, col=col, indptr_t=indptr_t, eid_t=eid_t,
                indices_t=indices_t, edata=edata, x=x)
     dy = dy.contiguous()
@@ -280,7 +308,7 @@ def vector_spmm_backward(row, indptr, eid, indices, col, indptr_t, eid_t, indice
     dt = _dtype(x)
     ws, nws = _workspace(OP_SPMM_BWD, plan, plan_t, h, d, dt, x.device)
     with torch.cuda.device_of(x):
-        check_attn(_LIB.bpt_vector_spmm_backward(_spmm_ref(plan, x, h, d), _spmm_ref(plan_t, x, h, d), _ptr(edata), _ptr(dy), _ptr(x), _ptr(dedata), _ptr(dx),
+        check_attn(_LIB.bpt_vector_spmm_backward(_spmm_ref(plan, x, h, d, cfg), _spmm_ref(plan_t, x, h, d, cfg), _ptr(edata), _ptr(dy), _ptr(x), _ptr(dedata), _ptr(dx),
                                                  _ptr(ws), nws, h, d, dt, _stream()), "vector_spmm_backward")
     return [dedata, dx]
 
@@ -298,6 +326,7 @@ def rel_bias_forward(col, indptr_c, eid_c, etype_slot, q, table):
     bias[eid_c[p], head] = q[row(p), head, :] . table[etype_slot[p], :], where etype_slot[p] is the type of the edge
     in slot p of the in-CSR (etype[eid_c]).  Returns float32 (E + 1, h); the last row is a zero spare row that the
     fused kernels read for absent pairs."""
+    cfg = _SETTINGS
     _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, etype_slot=etype_slot, q=q, table=table)
     _same_dtype(q, table)
     h, d = _hd(q)
@@ -309,17 +338,17 @@ def rel_bias_forward(col, indptr_c, eid_c, etype_slot, q, table):
     bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
     bias[E].zero_()
     with torch.cuda.device_of(q):
-        check_attn(_LIB.bpt_rel_bias_forward(_spmm_ref(plan, q, h, d), _ptr(q), _ptr(table), _ptr(bias), h, d, _dtype(q), _stream()),
+        check_attn(_LIB.bpt_rel_bias_forward(_spmm_ref(plan, q, h, d, cfg), _ptr(q), _ptr(table), _ptr(bias), h, d, _dtype(q), _stream()),
                    "rel_bias_forward")
     return bias
 
 
-def _check_bias(bias, n_edges, h, device):
+def _check_bias(bias, n_edges, h, device, cfg):
     if bias is None:
         return
     if bias.dtype != torch.float32 or tuple(bias.shape) != (n_edges + 1, h) or not bias.is_contiguous() or bias.device != device:
         raise ValueError(f"bias must be a contiguous float32 ({n_edges + 1}, {h}) tensor on {device}")
-    if not _USE_GROUPS:
+    if not cfg.use_groups:
         raise RuntimeError("the per-edge score term needs the row-group kernels")
 
 
@@ -328,8 +357,9 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     (n, h) float32 in base-2 units.  Arithmetic of modules/attention.py:66-77 in one pass.  dropout_p > 0
     drops attention probabilities as attention.py:73 does; the mask is a function of (seed, graph), see
     attention_dropout_mask.  bias: None or the float32 (E + 1, h) score term of rel_bias_forward."""
+    cfg = _SETTINGS
     _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v)
-    _check_bias(bias, eid_c.size(0), _hd(q)[0], q.device)
+    _check_bias(bias, eid_c.size(0), _hd(q)[0], q.device, cfg)
     _same_dtype(q, k, v)
     h, d = _hd(q)
     _expect_index(eid_c, indices_c)
@@ -337,8 +367,8 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     _expect_shape(v, k.shape, "v")
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
-    ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, dropout_p))["struct"]) \
-        if _attention_groups(plan, dropout_p, bias, q, k) else plan.ref
+    ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, cfg))["struct"]) \
+        if _attention_groups(plan, dropout_p, bias, q, k, cfg) else plan.ref
     o = torch.empty_like(q)
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
@@ -354,6 +384,7 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
                        dropout_p=0.0, seed=0, bias=None):
     """(dq, dk, dv) of attention_forward (same dropout_p, seed and bias).  With bias a fourth result: ds, float32
     (E, h), the gradient with respect to q.k + bias of every edge and head (= the gradient of bias)."""
+    cfg = _SETTINGS
     _check_all(row=row, indptr_r=indptr_r, eid_r=eid_r, indices_r=indices_r, col=col, indptr_c=indptr_c,
                eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v, o=o, lse=lse)
     do = do.contiguous()
@@ -373,12 +404,12 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
     plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0))
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    _check_bias(bias, eid_c.size(0), h, q.device)
+    _check_bias(bias, eid_c.size(0), h, q.device, cfg)
     ds = torch.empty((eid_c.size(0) + 1, h), dtype=torch.float32, device=q.device) if bias is not None else None
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref
-    if _attention_groups(plan_in, dropout_p, bias, q, k) and plan_in.covers_all_edges and plan_out.covers_all_edges:
-        R = _group_rows(q, h, d, plan_in)
+    if _attention_groups(plan_in, dropout_p, bias, q, k, cfg) and plan_in.covers_all_edges and plan_out.covers_all_edges:
+        R = _group_rows(q, h, d, plan_in, cfg)
         in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
         out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
@@ -415,74 +446,70 @@ def attention_dropout_mask(col, indptr_c, eid_c, indices_c, q, k, dropout_p, see
     return torch.from_numpy(keep)
 
 
-_USE_GROUPS = True
 _MIN_GROUP_ITEMS = 1536     # graphs with fewer work items run one wavefront per row (unless set_group_rows forces groups)
 
 
-def _attention_groups(plan, dropout_p, bias, q, k):
+def _attention_groups(plan, dropout_p, bias, q, k, cfg=None):
     """Whether the fused kernels take the row groups for this graph.  Very small graphs do not fill the GPU with one
     wavefront per group of rows and run faster with one per row (measured: L = 512, 0.055 against 0.070 ms per step;
     even at L = 1024); dropout and the score term exist in the row-group kernels only.  The row-group kernels address
     the rows of q AND of k / v with 32-bit byte offsets, so both node tensors have to stay below 4 GiB."""
-    if not _USE_GROUPS:
+    cfg = _SETTINGS if cfg is None else cfg
+    if not cfg.use_groups:
         return False
     if max(q.size(0), k.size(0)) * q.size(1) * q.size(2) * q.element_size() >= 2 ** 32:
         if dropout_p > 0.0 or bias is not None:
             raise RuntimeError("dropout and the score term need the row-group kernels, which address node tensors below 4 GiB")
         return False
-    return plan.n_items >= _MIN_GROUP_ITEMS or _GROUP_ROWS is not None or dropout_p > 0.0 or bias is not None
-_GROUPED_OPS = True         # row groups also in the unfused SpMM / SDDMM ops (set_grouped_ops)
-_GROUP_ROWS = None          # None: chosen per call from dtype and shape
+    return plan.n_items >= _MIN_GROUP_ITEMS or cfg.group_rows is not None or dropout_p > 0.0 or bias is not None
 
 
-def _group_rows(q, h, d, plan):
+def _group_rows(q, h, d, plan, cfg=None):
     """Rows per group for the fused kernels.  Groups of 8 nearly halve the row fetches of groups of 4 but double
     the work of the longest wavefront, which measured as a gain only on graphs with enough groups to fill the
     GPU twice or with long rows (average degree >= 48: at L = 4096, k = 8 (37) groups of 4 win, at k = 16 (59) groups of 8),
     and not for bfloat16 rows of up to 512 columns."""
-    if _GROUP_ROWS is not None:
-        return _GROUP_ROWS
+    cfg = _SETTINGS if cfg is None else cfg
+    if cfg.group_rows is not None:
+        return cfg.group_rows
     big = plan.n_items >= 16384 or plan.n_edges >= 48 * max(plan.n_rows, 1)
     return 8 if (big and (q.dtype == torch.float32 or h * d > 512)) else 4
 
 
-def _forward_rows(q, h, d, plan, dropout_p=0.0):
+def _forward_rows(q, h, d, plan, cfg=None):
     """Rows per group for the forward kernel.  Groups of 8 run on the matrix cores (two wavefronts per group; bfloat16
     rows go through the bfloat16 matrix instructions as loaded), which measured faster than the vector kernels at every
     size and both dtypes."""
-    if _GROUP_ROWS is not None:
-        return _group_rows(q, h, d, plan)
+    cfg = _SETTINGS if cfg is None else cfg
+    if cfg.group_rows is not None:
+        return cfg.group_rows
     return 8
 
 
 def set_group_rows(R):
-    """Testing / measurement hook: force groups of R (4 or 8) rows, or None for the default choice.  Returns the old value."""
-    global _GROUP_ROWS
+    """Testing / measurement hook (process-wide): force groups of R (4 or 8) rows, or None for the default choice.
+    Returns the old value."""
     if R not in (None, 4, 8):
         raise ValueError("R must be None, 4 or 8")
-    old, _GROUP_ROWS = _GROUP_ROWS, R
-    return old
+    return _replace_setting(group_rows=R).group_rows
 
 
 def row_groups_enabled():
-    return _USE_GROUPS
+    return _SETTINGS.use_groups
 
 
 def set_row_groups(on):
-    """Fused attention: let one wavefront own several rows that share neighbours (default) or one row each."""
-    global _USE_GROUPS
-    old, _USE_GROUPS = _USE_GROUPS, bool(on)
-    return old
+    """Testing / measurement hook (process-wide): fused attention lets one wavefront own several rows that share
+    neighbours (default) or one row each.  Returns the old setting."""
+    return _replace_setting(use_groups=bool(on)).use_groups
 
 
 def set_grouped_ops(on):
-    """Testing / measurement hook: let the unfused SpMM- and SDDMM-shaped ops (masked_mm and vector_spmm, forward and
-    backward) use the row groups (default) or one wavefront per row.  Returns the old setting."""
-    global _GROUPED_OPS
-    old, _GROUPED_OPS = _GROUPED_OPS, bool(on)
-    return old
+    """Testing / measurement hook (process-wide): let the unfused SpMM- and SDDMM-shaped ops (masked_mm and vector_spmm,
+    forward and backward) use the row groups (default) or one wavefront per row.  Returns the old setting."""
+    return _replace_setting(grouped_ops=bool(on)).grouped_ops
 
 
 def set_force_generic(on):
-    """Testing hook: route every op through the shape-generic kernels."""
+    """Testing hook (process-wide, an atomic flag inside the library): route every op through the shape-generic kernels."""
     return bool(_LIB.bpt_set_force_generic(1 if on else 0))

@@ -138,7 +138,7 @@ def _rel_aux(etype, col, indptr_c, eid_c, n_types):
     if hit is None:
         t_row, t_indptr, t_order = _type_csr(etype, n_types)
         etype_slot = etype.index_select(0, eid_c).contiguous()
-        slot_dst = torch.repeat_interleave(col, indptr_c[1:] - indptr_c[:-1])          # destination of every in-CSR slot
+        slot_dst = torch.repeat_interleave(col, indptr_c[1:] - indptr_c[:-1], output_size=eid_c.numel())   # destination of every in-CSR slot
         dst_of_eid = torch.empty_like(slot_dst)
         dst_of_eid[eid_c] = slot_dst
         hit = (etype_slot, t_row, t_indptr, t_order, dst_of_eid.index_select(0, t_order).contiguous(), (etype, col, indptr_c, eid_c))
@@ -186,22 +186,33 @@ class EdgeTypeEmbedding(Function):
 _type_csr_cache = {}
 
 
-def _type_csr(etype, n_types):
+def _type_csr(etype, n_types, chunk_size=32):
     """(row, indptr, order) of the CSR whose row t lists the edges of type t (ascending edge id), chunked like the
-    reference's other CSRs; cached per etype tensor."""
-    from .graphbuilder import partition_csr
+    reference's other CSRs (builder.pyx:305-321); cached per etype tensor.  Built where etype lives: on the GPU a stable
+    sort, a histogram and prefix sums, with two scalars read back (the range check and the number of units), so the
+    edge types never travel to the host."""
     key = (etype.data_ptr(), etype.numel(), etype._version, str(etype.device), n_types)
     hit = _type_csr_cache.get(key)
     if hit is None:
-        et = etype.detach().cpu().numpy()
-        if et.size and (et.min() < 0 or et.max() >= n_types):
+        et = etype.detach()
+        if et.dim() != 1 or et.dtype != torch.int64:
+            raise ValueError("etype must be a 1-D int64 tensor")
+        if et.numel() and (int(et.min()) < 0 or int(et.max()) >= n_types):
             raise ValueError("edge type out of range")
-        import numpy as np
-        order = np.argsort(et, kind="stable").astype(np.int64)
-        indptr = np.zeros(n_types + 1, dtype=np.int64)
-        np.cumsum(np.bincount(et, minlength=n_types), out=indptr[1:])
-        row, indptr_units = partition_csr(indptr)
-        hit = tuple(torch.as_tensor(np.asarray(a), dtype=torch.int64).to(etype.device) for a in (row, indptr_units, order)) + (etype,)
+        order = torch.argsort(et, stable=True)
+        counts = torch.bincount(et, minlength=n_types)
+        indptr = torch.zeros(n_types + 1, dtype=torch.int64, device=et.device)
+        torch.cumsum(counts, 0, out=indptr[1:])
+        # partition_csr on the device: row t gives ceil(count_t / chunk) units; unit u of row t starts at indptr[t] + u * chunk
+        units = (counts + (chunk_size - 1)) // chunk_size
+        first = torch.cumsum(units, 0) - units                           # number of the first unit of every row
+        n_units = int(units.sum())
+        row = torch.repeat_interleave(torch.arange(n_types, device=et.device), units, output_size=n_units)
+        rank = torch.arange(n_units, device=et.device) - first.index_select(0, row)
+        indptr_units = torch.empty(n_units + 1, dtype=torch.int64, device=et.device)
+        indptr_units[:n_units] = indptr.index_select(0, row) + rank * chunk_size
+        indptr_units[n_units] = et.numel()
+        hit = (row, indptr_units, order, etype)
         if len(_type_csr_cache) > 16:
             _type_csr_cache.clear()
         _type_csr_cache[key] = hit          # holds etype so that its data_ptr is not reused while cached

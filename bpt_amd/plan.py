@@ -24,7 +24,8 @@ GROUP_ORDER = 2 + 4    # groups inside an XCD chunk by decreasing work (2); entr
 GROUP_ORDER_SRC = 2 + 8  # source-side groups of the fused backward: aligned entry order (+8), which lowers that kernel's HBM reads
 GROUP_MAX_PAIRS = None  # cap on the edges of one group: None = 48 per member row, 0 = no cap
 GROUP_PAD_ENTRIES = 8  # the kernels' software pipeline reads per-entry arrays this far past the end
-_CACHE_SIZE = 64
+_CACHE_SIZE = 64                 # plans kept by the cache (PlanCache.set_limits)
+_CACHE_BYTES = 2 << 30           # and the device memory they may hold together: least recently used plans go first
 DEVICE_BUILD = None     # where new plans are built: True = on the GPU (libbptplan), False = on the host, None = by size
 DEVICE_BUILD_MIN_ROWS = 24576   # None: graphs with at least this many rows are planned on the GPU (measured: their
                                 # simpler grouping runs the fused kernels 4-9 % faster there and builds 10-30 x faster),
@@ -137,8 +138,23 @@ def link_groups_host(grp_dst, grp_src, n_edges):
     return out
 
 
+def _tensor_bytes(obj):
+    """Bytes of the torch tensors reachable from a plan's containers (dicts, tuples, lists)."""
+    if isinstance(obj, torch.Tensor):
+        return obj.numel() * obj.element_size()
+    if isinstance(obj, dict):
+        return sum(_tensor_bytes(v) for k, v in obj.items() if k != "host")
+    if isinstance(obj, (tuple, list)):
+        return sum(_tensor_bytes(v) for v in obj if not isinstance(v, (Plan, DevicePlan)))
+    return 0
+
+
 class Plan:
     """Device-resident plan of one CSR side; `.struct` is the `bpt_plan` passed to the C ABI."""
+
+    def device_bytes(self):
+        """Device memory held by this plan, its row groups and pair mappings."""
+        return _tensor_bytes(self._dev) + _tensor_bytes(list(self._groups.values())) + _tensor_bytes(list(self._links.values()))
 
     def __init__(self, row, indptr, eid, indices, n_rows, n_index_nodes, device, seg_len=DEFAULT_SEG_LEN):
         arrays, info = build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len)
@@ -265,6 +281,8 @@ class DevicePlan:
     """Plan of one CSR side built on the GPU from the reference's int64 device tensors (include/bptplan.h): no copy
     of the index arrays to the host, only the 16-int size blocks come back.  Same interface as Plan."""
 
+    device_bytes = Plan.device_bytes
+
     def __init__(self, row, indptr, eid, indices, n_rows, n_index_nodes, device, seg_len=DEFAULT_SEG_LEN):
         self.device = torch.device(device)
         self.n_rows, self.n_edges, self.n_index_nodes = int(n_rows), int(eid.numel()), int(n_index_nodes)
@@ -300,8 +318,12 @@ class DevicePlan:
         self.n_items, self.n_heavy, self.n_slots, self.max_degree = h[1], h[2], h[3], h[4]
         self.covers_all_edges = bool(h[5] & 1)
         self._info = info
-        self._dev = {"rowptr": rowptr, "idx": idx, "eid": eid32, "items": items, "heavy": heavy}   # items / heavy: upper-bound sized
+        # the work lists were allocated for their upper bounds: keep what the build produced
+        items, heavy = items[:max(self.n_items, 1)].clone(), heavy[:max(self.n_heavy, 1)].clone()
+        self._max_items = max(self.n_items, 1)
+        self._dev = {"rowptr": rowptr, "idx": idx, "eid": eid32, "items": items, "heavy": heavy}
         d = self._dev
+        torch.cuda.current_stream(self.device).synchronize()      # the plan is complete before any stream can use it
         self.struct = PlanStruct(
             d["rowptr"].data_ptr(), d["idx"].data_ptr() if E else None, d["eid"].data_ptr() if E else None,
             d["items"].data_ptr() if self.n_items else None, d["heavy"].data_ptr() if self.n_heavy else None,
@@ -368,6 +390,7 @@ class DevicePlan:
                 st.n_grp_entries = ne
                 st.grp_eids = dev["eids"].data_ptr()
                 hit = _Groups(dev=dev, struct=st, R=R, n_edges=E)
+                torch.cuda.current_stream(self.device).synchronize()      # the clones above ran on the building stream
                 self._groups[(R, by_mask)] = hit
         return hit
 
@@ -400,6 +423,7 @@ class DevicePlan:
                                                          torch.cuda.current_stream().cuda_stream)
                 _check_plan(st, "bpt_plan_link_device")
                 pairs = pairs[:n_pairs].clone()
+                torch.cuda.current_stream(self.device).synchronize()      # complete before another stream may read it
                 st = PlanStruct.from_buffer_copy(mine["struct"])
                 st.grp_pairs = pairs.data_ptr()
                 hit = (st, pairs, plan_src)
@@ -408,11 +432,41 @@ class DevicePlan:
 
 
 class PlanCache:
-    def __init__(self, capacity=_CACHE_SIZE):
+    """Least-recently-used cache of plans, bounded by a number of entries AND by the device memory the entries hold
+    (index arrays, work lists, row groups, pair mappings: about 45 MB per graph at L = 8192, k = 4).  A training loop
+    that builds a new graph per batch (graph/lm.py:53-98) therefore keeps at most `max_bytes` of plans alive."""
+
+    def __init__(self, capacity=_CACHE_SIZE, max_bytes=_CACHE_BYTES):
         self._d = collections.OrderedDict()
         self._cap = capacity
+        self._max_bytes = max_bytes
         self._lock = threading.Lock()     # forward runs on the Python thread, backward on autograd's
         self.hits = self.misses = 0
+
+    def set_limits(self, capacity=None, max_bytes=None):
+        """Change the number of plans kept and / or the device bytes they may hold together; returns the old pair."""
+        with self._lock:
+            old = (self._cap, self._max_bytes)
+            if capacity is not None:
+                self._cap = max(1, int(capacity))
+            if max_bytes is not None:
+                self._max_bytes = max(0, int(max_bytes))
+            self._evict()
+        return old
+
+    def device_bytes(self):
+        with self._lock:
+            return sum(p.device_bytes() + _tensor_bytes(list(t for t in ts if t is not None and t.is_cuda)) for p, ts in self._d.values())
+
+    def _evict(self):
+        # called with the lock held; the newest entry always stays
+        while len(self._d) > self._cap:
+            self._d.popitem(last=False)
+        if len(self._d) > 1:
+            total = sum(p.device_bytes() for p, _ in self._d.values())
+            while len(self._d) > 1 and total > self._max_bytes:
+                _, (p, _) = self._d.popitem(last=False)
+                total -= p.device_bytes()
 
     @staticmethod
     def _key(tensors, n_rows, n_index, seg_len):
@@ -428,6 +482,8 @@ class PlanCache:
             if hit is not None:
                 self._d.move_to_end(key)
                 self.hits += 1
+                if self.hits % 64 == 0:
+                    self._evict()                   # row groups and pair mappings are added to plans after insertion
                 return hit[0]
         self.misses += 1
         if _build_on_device(eid, n_rows):
@@ -441,8 +497,7 @@ class PlanCache:
             plan = Plan(row_h, indptr, eid, indices, nr, ni, eid.device, seg_len)
         with self._lock:
             self._d[key] = (plan, tensors)          # tensors kept alive with the entry
-            while len(self._d) > self._cap:
-                self._d.popitem(last=False)
+            self._evict()
         return plan
 
     def clear(self):

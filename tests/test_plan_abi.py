@@ -136,3 +136,31 @@ def test_cfg3_plan_numbers():
     assert deg_in[:8192].max() == 46 and deg_in.max() == 8192 and np.diff(out_csr[0]).max() == 3587
     arr, info = build_plan_host(COL, IC, in_csr[2], in_csr[1], 16383, 16383, 64)
     assert info.n_heavy == 127 and info.n_slots == 896
+
+
+def test_plan_cache_is_bounded_by_entries_and_by_bytes():
+    import torch
+    from bpt_amd import plan as pm
+    graphs = []
+    for L in (64, 80, 96, 112):
+        g, src, dst, (out_csr, in_csr, ROW, IR, COL, IC) = _bpt_csr(L, True, 2)
+        graphs.append((g.number_of_nodes, tuple(torch.from_numpy(a) for a in (COL, IC, in_csr[2], in_csr[1]))))
+    cache = pm.PlanCache(capacity=3, max_bytes=1 << 30)
+    plans = [cache.get(*args, n, n) for n, args in graphs]
+    assert len(cache._d) == 3 and cache.misses == 4                      # the oldest entry went
+    assert cache.get(*graphs[3][1], graphs[3][0], graphs[3][0]) is plans[3] and cache.hits == 1
+    one = plans[3].device_bytes()
+    plans[3].ensure_groups(8)
+    assert plans[3].device_bytes() > one                                 # row groups count towards the bytes
+    assert cache.device_bytes() >= sum(p.device_bytes() for p in plans[1:])
+    old = cache.set_limits(max_bytes=plans[3].device_bytes() + 1)
+    assert old == (3, 1 << 30) and len(cache._d) == 1                    # least recently used plans evicted, newest stays
+    cache.get(*graphs[0][1], graphs[0][0], graphs[0][0])
+    assert len(cache._d) == 1                                            # a plan larger than the budget is still usable once
+
+
+def test_noalloc_entry_refuses_a_plan_that_does_not_fit_its_scratch():
+    alib = _lib.attn_lib()
+    big = _lib.PlanStruct(None, None, None, None, None, 0, 0, 0, 0, 10 ** 6)       # a million partial rows
+    assert alib.bpt_attention_forward_noalloc(ctypes.byref(big), None, None, None, None, None, None, 0.125, 0.0, 0, 8, 64, 0, None) == -8
+    assert b"scratch" in alib.bpt_strerror(-8)
