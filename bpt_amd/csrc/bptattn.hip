@@ -1577,6 +1577,381 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
     }
 }
 
+// ---- dense tiles: groups of 16 rows, one wavefront per head ---------------------------------------------------------
+// A group of TILE_R = 16 rows (or row segments) and its entries (the union of the members' neighbours, each with a
+// 16-bit member mask) is walked in blocks of 16 entries as a dense 16 x 16 problem on the matrix cores: the pairs a
+// block does not have are computed and masked.  Adjacent rows of a BPT graph share most neighbours (35 % of a block's
+// pairs exist at L = 8192, k = 4), and a dense block costs 4 cycles per pair and head in float32 against 25-35 issue
+// slots of the gather form.  Workgroup = H wavefronts, wavefront = one head, so every lane keeps 1/64 of a
+// 16 x 64 tile per operand and nothing is exchanged between wavefronts.
+//
+// v_mfma_f32_16x16x4f32: D[i][n] += sum_k A[i][k] B[k][n], lane (c = lane % 16, g = lane / 16) supplies A[c][g] and
+// B[g][c] and holds D[4 g + r][c] in register r.  Which column of a row a (step, g) pair stands for is free as long as
+// A and B agree, so operands are loaded as 16-byte vectors:
+//   scores S^T = K Q^T : A = K[entry c][16 t + 4 g + e], B = q[member c][16 t + 4 g + e] (steps t, e = 0..3);
+//                        register r of lane (c, g) = score of (entry 4 g + r, member c);
+//   output O += P V    : A = register r of the probabilities as they stand (row = member c, k = g stands for entry
+//                        4 g + r), B = V[entry 4 g + r][4 c + nb]; register r' of accumulator nb of lane (c, g) =
+//                        O[member 4 g + r'][4 c + nb]: four consecutive columns per lane, 256 contiguous bytes per
+//                        member and 16 lanes.
+// Softmax state is per lane for member c (the four lanes of a member hold partial denominators that are added at the
+// end); the exponent reference is raised lazily as in the matrix-core forward above.
+constexpr int TILE_R = 16;
+constexpr int TILE_CHUNK = 128;                     // entries staged in LDS at a time = 8 blocks
+
+typedef float floatx4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float lane_bcast(float x, int src_lane) {
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(x)));
+}
+__device__ __forceinline__ int lane_bcast(int x, int src_lane) { return __builtin_amdgcn_ds_bpermute(src_lane << 2, x); }
+
+// Common start of the tile kernels.  HW heads (= wavefronts) per workgroup: workgroup b handles head slice
+// (b / 8) % (H / HW) of group (b / 8) / (H / HW) of XCD b % 8's range.
+struct TileCtx {
+    int lane, wv, c, g, head, p_begin, p_end;
+    int2 member;                 // (row, slot) of member c
+    uint32_t offa, offv;         // byte offsets of this lane inside a node row: its 16-column slice of the head (operands of the
+                                 // products that contract over columns, + 64 t bytes per step), and its columns 4 c .. 4 c + 3
+};
+
+template <typename T, int H, int D, int HW>
+__device__ __forceinline__ bool tile_begin(const bpt_plan &P, TileCtx &t) {
+    static_assert(D == 64 && H % HW == 0 && sizeof(T) == 4, "float32 rows, four 16-column slices per head, one per lane group");
+    constexpr int HS = H / HW;
+    t.lane = threadIdx.x & (WAVE - 1);
+    t.wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    t.c = t.lane & 15;
+    t.g = t.lane >> 4;
+    const int x = blockIdx.x & 7, w = (blockIdx.x >> 3) / HS;
+    const int grp = __builtin_amdgcn_readfirstlane(P.grp_chunks[x]) + w;
+    if (grp >= __builtin_amdgcn_readfirstlane(P.grp_chunks[x + 1])) return false;
+    t.member = reinterpret_cast<const int2 *>(P.grp_members)[(size_t)grp * TILE_R + t.c];
+    t.p_begin = __builtin_amdgcn_readfirstlane(P.grp_ptr[grp]);
+    t.p_end = __builtin_amdgcn_readfirstlane(P.grp_ptr[grp + 1]);
+    t.head = (int)((blockIdx.x >> 3) % HS) * HW + t.wv;
+    t.offa = (uint32_t)((t.head * D + 4 * t.g) * sizeof(T));
+    t.offv = (uint32_t)((t.head * D + 4 * t.c) * sizeof(T));
+    return true;
+}
+
+// The entry list of a group is staged, TILE_CHUNK entries at a time, in a wavefront-private piece of LDS as (neighbour,
+// mask) pairs: every lane needs five of them per block (its A-operand row and the four rows / masks of its lane
+// group), which would otherwise be five dependent global loads in front of every block's row loads.
+__device__ __forceinline__ void tile_stage_entries(const bpt_plan &P, int2 *lds, int p0, int cnt, int lane) {
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+#pragma unroll
+    for (int u = 0; u < TILE_CHUNK / WAVE; ++u) {
+        const int e = u * WAVE + lane;
+        const int4 x = entries[p0 + min(e, cnt - 1)];           // past the end: the last entry with an empty mask
+        lds[e] = make_int2(x.x, e < cnt ? x.y : 0);
+    }
+    wave_lds_fence();
+}
+
+// this lane's 16 columns of a node row (bytes offa + 64 t), as the A or B operand of a product over columns
+__device__ __forceinline__ void tile_load16(const char *row, float (&out)[16]) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const float4 x = *reinterpret_cast<const float4 *>(row + 64 * t);
+        out[4 * t] = x.x; out[4 * t + 1] = x.y; out[4 * t + 2] = x.z; out[4 * t + 3] = x.w;
+    }
+}
+
+// register r of the result of lane (c, g) = sum over the 64 columns of a[entry c] * b[member c] for (entry 4 g + r, member c)
+__device__ __forceinline__ floatx4v tile_dot(const float (&a)[16], const float (&b)[16]) {
+    floatx4v s0 = floatx4v{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[i], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i + 1], b[i + 1], s1, 0, 0, 0);
+    }
+    return s0 + s1;
+}
+
+// acc[nb][r'] (member 4 g + r', column 4 c + nb) += sum over the block's entries of w[member][entry] * row[entry][column]:
+// w = this lane's four weights (member c with entries 4 g + r), rows = columns 4 c .. 4 c + 3 of the rows of entries 4 g + r
+__device__ __forceinline__ void tile_axpy(const float (&w)[4], const float4 (&rows)[4], floatx4v (&acc)[4]) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].x, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].y, acc[1], 0, 0, 0);
+        acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].z, acc[2], 0, 0, 0);
+        acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].w, acc[3], 0, 0, 0);
+    }
+}
+
+// The members' result rows: whole rows go to `out` (scaled by inv[member] where given), segments of split rows to the
+// workspace in natural column order.
+template <int H, int D, bool SCALE>
+__device__ __forceinline__ void tile_store_rows(const TileCtx &t, const floatx4v (&acc)[4], float inv_c, float *__restrict__ out,
+                                                float *__restrict__ ws) {
+    constexpr int C = H * D;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int m = 4 * t.g + r;                                // the member whose row this lane stores a piece of
+        const int row = lane_bcast(t.member.x, m), slot = lane_bcast(t.member.y, m);
+        const float inv = SCALE ? lane_bcast(inv_c, m) : 1.f;
+        if (row < 0) continue;
+        float4 x = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
+        if (slot < 0) {
+            if (SCALE) { x.x *= inv; x.y *= inv; x.z *= inv; x.w *= inv; }
+            *reinterpret_cast<float4 *>(out + (size_t)row * C + t.head * D + 4 * t.c) = x;
+        } else {
+            *reinterpret_cast<float4 *>(ws + (size_t)slot * C + t.head * D + 4 * t.c) = x;
+        }
+    }
+}
+
+// Without read-ahead in registers the kernels fit four (forward, source side) or three wavefronts per SIMD, which
+// measured faster than a two-stage register pipeline at three (44.6 against 47 us, forward at L = 8192); groups of
+// 32 rows per wavefront (two member blocks sharing the K / V registers) cut the rows through the L1s by a third
+// but leave two or three wavefronts per SIMD and measured slower (56 us).
+// PIPE: the rows of the next block are loaded while one is used (two-stage register pipeline).  Pays on graphs with few,
+// tall tiles (a dense window graph: 9 blocks per tile, two wavefronts per SIMD in all), costs a wavefront per SIMD.
+template <bool PIPE, typename Blk, typename Issue, typename Compute>
+__device__ __forceinline__ void tile_walk(int nblk, Issue &&issue, Compute &&compute) {
+    if constexpr (PIPE) {
+        Blk A, B;
+        issue(A, 0);
+        for (int b = 0; b < nblk; b += 2) {
+            issue(B, min(b + 1, nblk - 1));                       // past the end: the last block again, not used
+            issue_loads_first();
+            compute(A);
+            issue_loads_first();
+            issue(A, min(b + 2, nblk - 1));
+            issue_loads_first();
+            if (b + 1 < nblk) compute(B);
+            issue_loads_first();
+        }
+    } else {
+        for (int b = 0; b < nblk; ++b) {
+            Blk A;
+            issue(A, b);
+            issue_loads_first();
+            compute(A);
+            issue_loads_first();
+        }
+    }
+}
+
+template <typename T, int H, int D, int HW, bool PIPE>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 3 : 4))) void k_attn_fwd_tile(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o, float *__restrict__ lse,
+    float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+    constexpr int C = H * D;
+    TileCtx t;
+    if (!tile_begin<T, H, D, HW>(P, t)) return;
+    __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    int2 *ent = ent_lds[t.wv];
+    const int c = t.c, g = t.g;
+    const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
+    float qb[16];
+    tile_load16(reinterpret_cast<const char *>(q) + (size_t)max(t.member.x, 0) * (C * sizeof(T)) + t.offa, qb);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) qb[i] *= scale_log2e;
+    floatx4v acc[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
+    float mref = M_INIT_LOG2, lrun = 0.f;
+    struct Blk {
+        float kr[16];
+        float4 vr[4];
+        int mk[4];
+    };
+    for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
+        const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
+        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        auto issue = [&](Blk &B, int b) {
+            const int2 ea = ent[TILE_R * b + c];
+            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
+            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
+            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+            tile_load16(kb + (size_t)((uint32_t)ea.x * (uint32_t)(C * sizeof(T))) + t.offa, B.kr);
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                B.vr[r] = *reinterpret_cast<const float4 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
+        };
+        auto compute = [&](const Blk &B) {
+            const floatx4v st = tile_dot(B.kr, qb);
+            float sc[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sc[r] = ((B.mk[r] >> c) & 1) ? st[r] : -INFINITY;
+            const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
+                float gm = fmaxf(mb, __shfl_xor(mb, 16));
+                gm = fmaxf(gm, __shfl_xor(gm, 32));              // over the four lanes of member c
+                const float mn = fmaxf(mref, gm);
+                const float al = __builtin_amdgcn_exp2f(mref - mn);
+                mref = mn;
+                lrun *= al;
+                // register r' of the accumulators belongs to member 4 g + r': its factor sits in lane 4 g + r'
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float a = lane_bcast(al, 4 * g + r);
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) acc[nb][r] *= a;
+                }
+            }
+            float pr[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                pr[r] = __builtin_amdgcn_exp2f(sc[r] - mref);
+                lrun += pr[r];
+            }
+            tile_axpy(pr, B.vr, acc);
+        };
+        tile_walk<PIPE, Blk>(nblk, issue, compute);
+        wave_lds_fence();                                         // the piece is read to the end before the next one is staged
+    }
+    float lt = lrun + __shfl_xor(lrun, 16);
+    lt += __shfl_xor(lt, 32);                                    // denominator of member c, in its four lanes
+    tile_store_rows<H, D, true>(t, acc, lt > 0.f ? 1.f / lt : 0.f, reinterpret_cast<float *>(o), ws_acc);
+    if (g == 0 && t.member.x >= 0) {                              // lanes 0 .. 15: one member each
+        if (t.member.y < 0) {
+            lse[(size_t)t.member.x * H + t.head] = lt > 0.f ? mref + log2f(lt) : 0.f;
+        } else {
+            ws_ml[((size_t)t.member.y * H + t.head) * 2] = mref;
+            ws_ml[((size_t)t.member.y * H + t.head) * 2 + 1] = lt;
+        }
+    }
+}
+
+// Backward on tiles, destination side: per block the scores and dO . v of all 16 x 16 pairs (two products over the
+// columns), p = 2^(s - lse), ds = p (dO . v - delta) scale, dq += ds K (third product; K is read a second time in the
+// column layout, which the L1 serves).  (p, ds) of the pairs that exist go to the scratch of the source side: position
+// u' * 16 + m' of the pair in the source-side groups comes from grp_pairs, and the pair is stored at
+// pds[(u' * H + head) * 16 + m'], so that the source-side wavefront of a head reads the 16 members of an entry as 128
+// contiguous bytes.  These scattered 8-byte stores are 36 of the kernel's 92 us at L = 8192, k = 4; letting the source
+// side recompute p and ds instead (two more products there, delta (n, H) handed over) measured slower on every graph
+// tried (L = 4096, k = 16: 0.166 against 0.146 ms per step; window 128: 0.134 against 0.114).
+template <typename T, int H, int D, int HW, bool PIPE>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : 3))) void k_attn_bwd_dst_tile(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
+    const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds, float *__restrict__ ws_dq,
+    float scale, float scale_log2e) {
+    constexpr int C = H * D;
+    TileCtx t;
+    if (!tile_begin<T, H, D, HW>(P, t)) return;
+    __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    int2 *ent = ent_lds[t.wv];
+    const int c = t.c, g = t.g;
+    const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
+    const size_t mrow = (size_t)max(t.member.x, 0) * (C * sizeof(T)) + t.offa;
+    float qb[16], dob[16], delta, lse_c;
+    {
+        float ob[16];
+        tile_load16(reinterpret_cast<const char *>(q) + mrow, qb);
+        tile_load16(reinterpret_cast<const char *>(d_o) + mrow, dob);
+        tile_load16(reinterpret_cast<const char *>(o) + mrow, ob);
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { part = fmaf(dob[i], ob[i], part); qb[i] *= scale_log2e; }
+        part += __shfl_xor(part, 16);
+        delta = part + __shfl_xor(part, 32);                      // dO . O of member c, this head
+        lse_c = lse[(size_t)max(t.member.x, 0) * H + t.head];
+    }
+    floatx4v acc[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
+    struct Blk {
+        float kr[16], va[16];
+        float4 kc[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 g + r
+        int pos[4], mk[4];
+    };
+    for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
+        const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
+        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        auto issue = [&](Blk &B, int b) {
+            const int2 ea = ent[TILE_R * b + c];
+            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
+            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
+            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+            const size_t arow = (size_t)((uint32_t)ea.x * (uint32_t)(C * sizeof(T))) + t.offa;
+            tile_load16(kb + arow, B.kr);
+            tile_load16(vb + arow, B.va);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                B.kc[r] = *reinterpret_cast<const float4 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
+                // (positions past the group's end are read at its last entry: their masks are empty)
+                B.pos[r] = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
+            }
+        };
+        auto compute = [&](const Blk &B) {
+            const floatx4v st = tile_dot(B.kr, qb), dp = tile_dot(B.va, dob);
+            float ds[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool has = (B.mk[r] >> c) & 1;
+                const float pe = has ? __builtin_amdgcn_exp2f(st[r] - lse_c) : 0.f;
+                ds[r] = pe * (dp[r] - delta) * scale;
+                if (has) pds[((size_t)(B.pos[r] >> 4) * H + t.head) * TILE_R + (B.pos[r] & 15)] = make_float2(pe, ds[r]);
+            }
+            tile_axpy(ds, B.kc, acc);
+        };
+        tile_walk<PIPE, Blk>(nblk, issue, compute);
+        wave_lds_fence();
+    }
+    tile_store_rows<H, D, false>(t, acc, 1.f, reinterpret_cast<float *>(dq), ws_dq);
+}
+
+// Backward on tiles, source side (groups of the out-CSR plan: members = source rows, entries = destinations):
+// dk += ds^T q, dv += p^T dO with (p, ds) read from the scratch the destination side filled.
+template <typename T, int H, int D, int HW, bool PIPE>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 3 : 4))) void k_attn_bwd_src_tile(
+    bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o, const float2 *__restrict__ pds, T *__restrict__ dk, T *__restrict__ dv,
+    float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
+    constexpr int C = H * D;
+    TileCtx t;
+    if (!tile_begin<T, H, D, HW>(P, t)) return;
+    __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    int2 *ent = ent_lds[t.wv];
+    const int c = t.c, g = t.g;
+    const char *qb = reinterpret_cast<const char *>(q), *db = reinterpret_cast<const char *>(d_o);
+    floatx4v ak[4], av[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) { ak[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; av[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; }
+    struct Blk {
+        float4 qr[4], dr[4];
+        float2 w[4];
+        int mk[4];
+    };
+    for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
+        const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
+        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        auto issue = [&](Blk &B, int b) {
+            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
+            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
+            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const size_t off = (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv;
+                B.qr[r] = *reinterpret_cast<const float4 *>(qb + off);
+                B.dr[r] = *reinterpret_cast<const float4 *>(db + off);
+                B.w[r] = pds[((size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * H + t.head) * TILE_R + c];
+            }
+        };
+        auto compute = [&](const Blk &B) {
+            float pe[4], ds[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool has = (B.mk[r] >> c) & 1;              // the scratch of pairs that do not exist is not initialised
+                pe[r] = has ? B.w[r].x : 0.f;
+                ds[r] = has ? B.w[r].y : 0.f;
+            }
+            tile_axpy(ds, B.qr, ak);
+            tile_axpy(pe, B.dr, av);
+        };
+        tile_walk<PIPE, Blk>(nblk, issue, compute);
+        wave_lds_fence();
+    }
+    tile_store_rows<H, D, false>(t, ak, 1.f, reinterpret_cast<float *>(dk), ws_dk);
+    tile_store_rows<H, D, false>(t, av, 1.f, reinterpret_cast<float *>(dv), ws_dv);
+}
+
 // Backward, destination side.  Writes (p, ds) of every pair to pds[(t * H + head)], t = the pair's
 // position (entry * R + member) in the SOURCE-side plan, which P.grp_pairs gives for every
 // (entry, member) of this plan (a spare position for members the entry does not have).  One store per
@@ -2028,7 +2403,7 @@ inline int check_plan(const bpt_plan *p, bool need_idx) {
     if (p->n_edges > 0 && (!p->eid || (need_idx && !p->idx))) return BPT_ERR_NULL;
     if (p->n_heavy > 0 && !p->heavy) return BPT_ERR_NULL;
     if (p->n_items < p->n_rows) return BPT_ERR_SIZE;     // every row owns at least one item
-    if (p->n_groups < 0 || p->grp_R < 0 || p->grp_R > 16 || p->n_grp_entries < 0) return BPT_ERR_SIZE;
+    if (p->n_groups < 0 || p->grp_R < 0 || p->grp_R > 32 || p->n_grp_entries < 0) return BPT_ERR_SIZE;
     if (p->n_groups > 0 && (!p->grp_members || !p->grp_ptr || !p->grp_chunks || (p->n_edges > 0 && !p->grp_entries))) return BPT_ERR_NULL;
     if (p->n_groups > 0 && (p->grp_max_chunk < 1 || p->grp_max_chunk > p->n_groups)) return BPT_ERR_SIZE;
     return BPT_OK;
@@ -2333,6 +2708,19 @@ inline bool has_groups(const bpt_plan *P, int h, int d, size_t elem) {
            fits32((P->n_grp_entries + GRP_PAD_ENTRIES) * P->grp_R, (int64_t)h * 8);
 }
 
+// groups of 16 rows for the dense-tile kernels (one wavefront per head: h * 64 threads per workgroup)
+inline bool has_tiles(const bpt_plan *P, int h, int d, size_t elem) {
+    return P->n_groups > 0 && P->grp_R == TILE_R && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
+           P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups && P->n_grp_entries >= 0 && d == 64 && h <= 16 && elem == 4 &&
+           fits32(P->n_rows, (int64_t)h * d * (int64_t)elem);
+}
+
+// Few and tall tiles (fewer wavefronts than three per SIMD, six or more blocks each on average): the kernels then read one
+// block ahead in registers instead of counting on other wavefronts to cover the loads.
+inline bool tall_tiles(const bpt_plan *P, int h) {
+    return P->n_groups * h < 3 * 1024 && P->n_grp_entries >= 6 * TILE_R * P->n_groups;
+}
+
 bool spmm_grp_ok(const bpt_plan *P, int h, int d, int dtype) {
     return has_groups(P, h, d, dtype == BPT_BF16 ? 2 : 4) && P->grp_eids && P->n_edges > 0;
 }
@@ -2383,9 +2771,17 @@ inline bool grouped_backward(const bpt_plan *Pin, const bpt_plan *Pout, int h, i
 
 // float2 (p, ds) scratch of the fused backward: one per (entry, member) of the source-side groups (plus the
 // look-ahead padding), or one per edge for the per-row kernels
+inline bool tiled_backward(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {
+    return has_tiles(Pin, h, d, elem) && has_tiles(Pout, h, d, elem) && Pin->grp_pairs &&
+           fits32((Pout->n_grp_entries + GRP_PAD_ENTRIES) * TILE_R, (int64_t)h * 8);
+}
+
+// float2 (p, ds) scratch of the fused backward: one per (entry, member) of the source-side groups (plus the
+// look-ahead padding), or one per edge for the per-row kernels
 inline int64_t pds_bytes(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {
     int64_t n = Pin->n_edges;
-    if (Pout && grouped_backward(Pin, Pout, h, d, elem)) n = std::max(n, (Pout->n_grp_entries + GRP_PAD_ENTRIES) * Pout->grp_R);
+    if (Pout && (grouped_backward(Pin, Pout, h, d, elem) || tiled_backward(Pin, Pout, h, d, elem)))
+        n = std::max(n, (Pout->n_grp_entries + GRP_PAD_ENTRIES) * Pout->grp_R);
     return 2 * round16(n * h * 4);
 }
 
@@ -2397,6 +2793,18 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
+        if constexpr (D == 64 && sizeof(T) == 4) {
+            if (has_tiles(P, H, D, sizeof(T)) && drop.thr == 0 && !bias) {
+                constexpr int HW = H >= 4 ? 4 : H;          // heads per workgroup
+                if (tall_tiles(P, H))
+                    hipLaunchKernelGGL((k_attn_fwd_tile<T, H, D, HW, true>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), 0, s, *P,
+                                       (const T *)q, (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+                else
+                    hipLaunchKernelGGL((k_attn_fwd_tile<T, H, D, HW, false>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), 0, s, *P,
+                                       (const T *)q, (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+                goto launched;
+            }
+        }
         if (has_groups(P, H, D, sizeof(T))) {
 #define LAUNCH_FWD(RR, DR, BI)                                                                                                   \
     hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR, HS, DR, BI>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)q, \
@@ -2430,6 +2838,7 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
             hipLaunchKernelGGL((k_attn_fwd<T, H, D, FAST_BATCH>), dim3(grid_for(P)), dim3(BLOCK), 0, s, *P, (const T *)q, (const T *)k,
                                (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
         }
+    launched:;
     }
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
@@ -2449,6 +2858,40 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     float *dsbuf = pbuf + pbytes / 8;
     float2 *pds = (float2 *)ws;                                  // row-group kernels: interleaved (p, ds)
     float *ws_rows = (float *)ws + pbytes / 4;
+    if constexpr (D == 64 && sizeof(T) == 4) {
+        if (tiled_backward(Pin, Pout, H, D, sizeof(T)) && drop.thr == 0 && !bias) {
+            constexpr int HW = H >= 4 ? 4 : H;
+            float *ws_dk = ws_rows + (size_t)Pin->n_slots * H * D, *ws_dv = ws_dk + (size_t)Pout->n_slots * H * D;
+            {
+                ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
+                if (tall_tiles(Pin, H))
+                    hipLaunchKernelGGL((k_attn_bwd_dst_tile<T, H, D, HW, true>), dim3(group_grid(Pin) * (H / HW)), dim3(HW * WAVE), 0, s, *Pin,
+                                       (const T *)q, (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows,
+                                       scale, scale * LOG2E);
+                else
+                    hipLaunchKernelGGL((k_attn_bwd_dst_tile<T, H, D, HW, false>), dim3(group_grid(Pin) * (H / HW)), dim3(HW * WAVE), 0, s, *Pin,
+                                       (const T *)q, (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows,
+                                       scale, scale * LOG2E);
+            }
+            int st = launch_status();
+            if (st != BPT_OK) return st;
+            {
+                ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
+                if (tall_tiles(Pout, H))
+                    hipLaunchKernelGGL((k_attn_bwd_src_tile<T, H, D, HW, true>), dim3(group_grid(Pout) * (H / HW)), dim3(HW * WAVE), 0, s, *Pout,
+                                       (const T *)q, (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv);
+                else
+                    hipLaunchKernelGGL((k_attn_bwd_src_tile<T, H, D, HW, false>), dim3(group_grid(Pout) * (H / HW)), dim3(HW * WAVE), 0, s, *Pout,
+                                       (const T *)q, (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv);
+            }
+            st = launch_status();
+            if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;
+            hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / WAVE, 2), dim3(BLOCK), 0, s, Pin->heavy,
+                               (int)Pin->n_heavy, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
+                               (size_t)Pout->n_slots * H * D);
+            return launch_status();
+        }
+    }
     {
         ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
         if (grouped) {

@@ -375,6 +375,8 @@ int bptg_plan_fill(const int64_t *row, const int64_t *indptr_units, int64_t n_un
 // edge = (entry, member).  Pairs are numbered entry by entry, members ascending.  With order_mode + 4
 // the entries of a group are sorted by member mask (stable, larger first), which lets a kernel that
 // handles two consecutive entries per step find the same members in both most of the time.
+constexpr int32_t MAX_GROUP_ROWS = 32;          // member masks are 32-bit
+
 int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32, const int32_t *eid32,
                     int64_t n_edges, int64_t n_index_nodes, int32_t R, int32_t window, int32_t order_mode,
                     int32_t max_pairs, int32_t *members, int32_t *grp_ptr, int32_t *entries, int32_t *pair_eid, int32_t *slot_eid,
@@ -382,7 +384,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
     if (!items || !members || !grp_ptr || !chunks || !n_groups_out || !n_entries_out) return BPTG_ERR_NULL;
     if (n_edges > 0 && (!idx32 || !eid32 || !entries || !pair_eid)) return BPTG_ERR_NULL;
     if (n_items < 0 || n_edges < 0 || n_index_nodes < 0) return BPTG_ERR_SIZE;
-    if (R < 1 || R > 16 || window < 0 || order_mode < 0 || order_mode > 15 || max_pairs < 0) return BPTG_ERR_ARG;
+    if (R < 1 || R > MAX_GROUP_ROWS || window < 0 || order_mode < 0 || order_mode > 15 || max_pairs < 0) return BPTG_ERR_ARG;
     const bool aligned = (order_mode & 8) != 0;
     const bool by_mask = (order_mode & 4) != 0 && !aligned;
     order_mode &= 3;
@@ -414,8 +416,8 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
         const int32_t first = order[(size_t)oi];
         if (used[(size_t)first]) continue;
         used[(size_t)first] = 1;
-        int32_t mem[16];
-        for (int32_t m = 0; m < 16; ++m) mem[m] = -1;
+        int32_t mem[MAX_GROUP_ROWS];
+        for (int32_t m = 0; m < MAX_GROUP_ROWS; ++m) mem[m] = -1;
         int32_t n_mem = 1;
         mem[0] = first;
         int64_t w = 0;
@@ -488,7 +490,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
 
     // ---- phase 3: emit members, entries and pairs in the final group order
     struct Triple { int32_t idx, member, eid; };
-    struct Entry { int32_t idx, mask, eids[16]; };
+    struct Entry { int32_t idx; uint32_t mask; int32_t eids[MAX_GROUP_ROWS]; };
     std::vector<Triple> tri;
     std::vector<Entry> ents, placed;
     // the entries of one group in neighbour order
@@ -507,8 +509,8 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
         size_t a = 0;
         while (a < tri.size()) {
             size_t b = a;
-            int32_t cnt[16] = {0};
-            size_t start[16] = {0};
+            int32_t cnt[MAX_GROUP_ROWS] = {0};
+            size_t start[MAX_GROUP_ROWS] = {0};
             while (b < tri.size() && tri[b].idx == tri[a].idx) {
                 if (cnt[tri[b].member] == 0) start[tri[b].member] = b;
                 ++cnt[tri[b].member];
@@ -522,7 +524,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
                 en.mask = 0;
                 for (int32_t m = 0; m < R; ++m)
                     if (cnt[m] > t) {
-                        en.mask |= 1 << m;
+                        en.mask |= 1u << m;
                         en.eids[m] = tri[start[m] + (size_t)t].eid;
                     }
                 ents.push_back(en);
@@ -556,7 +558,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
                     }
                     Entry &en = found[(size_t)local_of[(size_t)v]];
                     if (en.mask >> m & 1) { repeated = true; break; }
-                    en.mask |= 1 << m;
+                    en.mask |= 1u << m;
                     en.eids[m] = eid32[p];
                 }
             }
@@ -629,7 +631,7 @@ int bptg_group_plan(const int32_t *items, int64_t n_items, const int32_t *idx32,
         for (const Entry &e : ents) {
             int32_t *en = entries + 4 * n_entries;
             en[0] = e.idx;
-            en[1] = e.mask;
+            en[1] = (int32_t)e.mask;
             en[2] = (int32_t)n_pairs;
             en[3] = 0;
             for (int32_t m = 0; m < R; ++m) {
@@ -650,7 +652,7 @@ int bptg_link_groups(const int32_t *slot_eid_dst, int64_t n_entries_dst, int32_t
                      int64_t n_entries_src, int32_t R_src, int64_t n_edges, int32_t pad_entries, int32_t *pairs) {
     if (!pairs || (n_entries_dst > 0 && !slot_eid_dst) || (n_entries_src > 0 && !slot_eid_src)) return BPTG_ERR_NULL;
     if (n_entries_dst < 0 || n_entries_src < 0 || n_edges < 0 || pad_entries < 0) return BPTG_ERR_SIZE;
-    if (R_dst < 1 || R_dst > 16 || R_src < 1 || R_src > 16) return BPTG_ERR_ARG;
+    if (R_dst < 1 || R_dst > MAX_GROUP_ROWS || R_src < 1 || R_src > MAX_GROUP_ROWS) return BPTG_ERR_ARG;
     if ((n_entries_src + pad_entries) * R_src >= INT32_MAX) return BPTG_ERR_SIZE;
     std::vector<int32_t> pos_of((size_t)n_edges, -1);
     int64_t covered = 0;

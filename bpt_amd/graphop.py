@@ -18,7 +18,7 @@ import threading
 import torch
 
 from ._lib import attn_lib, check_attn
-from .plan import GROUP_ORDER_SRC, plan_cache
+from .plan import GROUP_ORDER_SRC, TILE_GROUP_R, plan_cache
 
 __all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forward", "node_mul_edge_backward",
            "sparse_softmax_forward", "sparse_softmax_backward", "vector_spmm_forward", "vector_spmm_backward"]
@@ -26,17 +26,17 @@ __all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forwa
 _LIB = attn_lib()          # fail at import time if the HIP library is missing
 
 
-class _Settings(collections.namedtuple("_Settings", "use_groups grouped_ops group_rows")):
+class _Settings(collections.namedtuple("_Settings", "use_groups grouped_ops group_rows use_tiles")):
     """Which kernel family the ops take: use_groups (fused attention: one wavefront per group of rows that share
     neighbours, or per row), grouped_ops (the same for the unfused SpMM / SDDMM ops), group_rows (None: chosen per call
-    from dtype and shape; 4 or 8: forced).  Immutable: the set_* hooks below replace the whole tuple under a lock, and
+    from dtype and shape; 4 or 8: forced), use_tiles (fused attention on dense 16 x 16 tiles where they exist).  Immutable: the set_* hooks below replace the whole tuple under a lock, and
     every op reads it ONCE on entry, so a call (forward on the Python thread, backward on autograd's) works with one
     consistent set even if another thread flips a hook meanwhile.  The hooks are process-wide testing / measurement
     aids, not per-thread state; every family computes the same results."""
     __slots__ = ()
 
 
-_SETTINGS = _Settings(True, True, None)
+_SETTINGS = _Settings(True, True, None, True)
 _SETTINGS_LOCK = threading.Lock()
 
 
@@ -367,8 +367,13 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     _expect_shape(v, k.shape, "v")
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
-    ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, cfg))["struct"]) \
-        if _attention_groups(plan, dropout_p, bias, q, k, cfg) else plan.ref
+    if not _attention_groups(plan, dropout_p, bias, q, k, cfg):
+        ref = plan.ref
+    elif _tiles(q, h, d, plan, dropout_p, bias, cfg):
+        plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=_tile_seg_len(plan))
+        ref = ctypes.byref(plan.ensure_groups(TILE_ROWS)["struct"])
+    else:
+        ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, cfg))["struct"])
     o = torch.empty_like(q)
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
@@ -409,9 +414,16 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref
     if _attention_groups(plan_in, dropout_p, bias, q, k, cfg) and plan_in.covers_all_edges and plan_out.covers_all_edges:
-        R = _group_rows(q, h, d, plan_in, cfg)
-        in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
-        out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
+        if _tiles(q, h, d, plan_in, dropout_p, bias, cfg) and _tiles_backward(plan_in):
+            seg = _tile_seg_len(plan_in)
+            plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg)
+            plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg)
+            in_ref = ctypes.byref(plan_in.linked_to(plan_out, TILE_ROWS))
+            out_ref = ctypes.byref(plan_out.ensure_groups(TILE_ROWS, GROUP_ORDER_SRC)["struct"])
+        else:
+            R = _group_rows(q, h, d, plan_in, cfg)
+            in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
+            out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
     with torch.cuda.device_of(q):
         check_attn(_LIB.bpt_attention_backward(in_ref, out_ref, _ptr(q), _ptr(k), _ptr(v), _ptr(bias), _ptr(o), _ptr(do),
@@ -484,6 +496,41 @@ def _forward_rows(q, h, d, plan, cfg=None):
     if cfg.group_rows is not None:
         return cfg.group_rows
     return 8
+
+
+TILE_ROWS = TILE_GROUP_R
+TILE_BACKWARD = None       # testing / measurement hook: True / False force the backward on / off tiles (None: by graph size and density)
+TILE_SEG_LEN = None        # testing / measurement hook: edges per work item of the tile plans (None: by average degree)
+
+
+def _tiles(q, h, d, plan, dropout_p, bias, cfg):
+    """Whether the fused forward runs on dense tiles (groups of 16 rows, one wavefront per head, every block of 16
+    entries a dense 16 x 16 matrix product with the missing pairs masked): float32 rows of 64 columns per head, no
+    dropout or score term, and the library's choice of rows per group not overridden."""
+    return (cfg.use_tiles and cfg.group_rows is None and q.dtype == torch.float32 and d == 64 and h <= 16
+            and dropout_p == 0.0 and bias is None)
+
+
+def _tiles_backward(plan):
+    """The backward runs on tiles where that measured faster than the row-group kernels (float32, 8 x 64): on small graphs,
+    which the row groups of 8 cannot spread over the GPU (L = 4096: k = 4 ... 32 run 7 to 27 % faster), and on dense ones
+    (window 128: 1.9 x); at L = 8192, k = 4 and on the 32-graph batch the row-group kernels win (0.203 against 0.214 ms)."""
+    if TILE_BACKWARD is not None:
+        return TILE_BACKWARD
+    return plan.n_rows < 12288 or plan.n_edges >= 64 * max(plan.n_rows, 1)
+
+
+def _tile_seg_len(plan):
+    """Edges per work item of the plans the tile kernels walk (TILE_SEG_LEN overrides when set)."""
+    if TILE_SEG_LEN is not None:
+        return TILE_SEG_LEN
+    deg = plan.n_edges / max(plan.n_rows, 1)
+    return 64 if deg < 32 else (128 if deg < 80 else 256)
+
+
+def set_tiles(on):
+    """Testing / measurement hook (process-wide): dense-tile kernels on (default) or off.  Returns the old setting."""
+    return _replace_setting(use_tiles=bool(on)).use_tiles
 
 
 def set_group_rows(R):

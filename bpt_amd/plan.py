@@ -24,6 +24,8 @@ GROUP_ORDER = 2 + 4    # groups inside an XCD chunk by decreasing work (2); entr
 GROUP_ORDER_SRC = 2 + 8  # source-side groups of the fused backward: aligned entry order (+8), which lowers that kernel's HBM reads
 GROUP_MAX_PAIRS = None  # cap on the edges of one group: None = 48 per member row, 0 = no cap
 GROUP_PAD_ENTRIES = 8  # the kernels' software pipeline reads per-entry arrays this far past the end
+TILE_GROUP_R = 16      # rows per group of the dense-tile kernels
+TILE_MAX_PAIRS = 0     # cap on the edges of such a group (0 = none, None = as the other groups)
 _CACHE_SIZE = 64                 # plans kept by the cache (PlanCache.set_limits)
 _CACHE_BYTES = 2 << 30           # and the device memory they may hold together: least recently used plans go first
 DEVICE_BUILD = None     # where new plans are built: True = on the GPU (libbptplan), False = on the host, None = by size
@@ -186,12 +188,14 @@ class Plan:
     # ---- row groups for the fused attention kernels ----
     def ensure_groups(self, R=GROUP_R, order_mode=None):
         """Builds the row-group arrays for groups of R rows once (host) and uploads them.  Returns a dict with
-        the host arrays ("host") and the `bpt_plan` carrying them ("struct")."""
+        the host arrays ("host") and the `bpt_plan` carrying them ("struct").  Groups of TILE_GROUP_R rows (the dense-tile
+        kernels) have no cap on their edges: a tile costs the same whether its pairs exist or not."""
         order_mode = GROUP_ORDER if order_mode is None else order_mode
         with self._lock:
             hit = self._groups.get((R, order_mode))
             if hit is None:
-                grp = build_groups_host(self._host, self.n_index_nodes, R=R, order_mode=order_mode)
+                grp = build_groups_host(self._host, self.n_index_nodes, R=R, order_mode=order_mode,
+                                        max_pairs=TILE_MAX_PAIRS if R == TILE_GROUP_R else None)
                 # edge id of every (entry, member); absent members and the padding point at the spare row n_edges
                 eids = np.full((len(grp["entries"]) + GROUP_PAD_ENTRIES, R), self.n_edges, dtype=np.int32)
                 se = grp["slot_eid"]
