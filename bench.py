@@ -289,9 +289,27 @@ def main():
     copy_gbs = 10 * 2 * a.numel() * 4 / (c0.elapsed_time(c1) * 1e-3) / 1e9
     del a, b
     log(f"measured device copy bandwidth: {copy_gbs:.0f} GB/s (read + write)")
+    # ... and to the access pattern of these kernels: pseudo-random 1 KB rows (a node row's share of one wavefront) of a
+    # region the size of the K and V tensors, at the occupancies the attention kernels run at (8 and 16 wavefronts per CU)
+    gather = {}
+    region = torch.zeros(max(2 * N * H * D * esize, 1 << 20), dtype=torch.uint8, device=dev)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    for waves in (8, 16, 32):
+        iters, in_flight = 100, 4
+        for rep in range(2):
+            c0.record()
+            st = lib.bpt_gather_probe(region.data_ptr(), region.numel(), waves, in_flight, iters, sink.data_ptr(),
+                                      torch.cuda.current_stream().cuda_stream)
+            c1.record()
+            torch.cuda.synchronize()
+        assert st == 0, st
+        gather[f"{waves}_waves_per_cu"] = round(256 * waves * iters * in_flight * 1024 / (c0.elapsed_time(c1) * 1e-3) / 1e9, 1)
+    del region
+    log(f"measured 1 KB row-gather bandwidth from a {2 * N * H * D * esize / 1e6:.0f} MB region, GB/s: {gather}")
     if roofline is not None:
         roofline["measured_copy_GBps"] = round(copy_gbs, 1)
         roofline["frac_of_measured_copy"] = round(roofline["achieved"] / copy_gbs, 4)
+        roofline["measured_row_gather_GBps"] = gather
 
     block = None
     if args.block_layers > 0 and not args.unfused:

@@ -48,6 +48,7 @@ ATTN_API = {
     "bpt_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "bpt_set_force_generic": (ctypes.c_int, [ctypes.c_int]),
     "bpt_profile_kernel": (ctypes.c_int, [ctypes.c_int, c_vp, c_vp]),
+    "bpt_gather_probe": (ctypes.c_int, [c_vp, c_i64, ctypes.c_int, ctypes.c_int, ctypes.c_int, c_vp, c_vp]),
     "bpt_workspace_bytes": (c_i64, [ctypes.c_int, _PP, _PP, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "bpt_maskedmm_csr_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp] + _tail),
     "bpt_maskedmm_csr_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),

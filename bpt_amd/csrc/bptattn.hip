@@ -1703,12 +1703,13 @@ __device__ __forceinline__ void tile_store_rows(const TileCtx &t, const floatx4v
     }
 }
 
-// Without read-ahead in registers the kernels fit four (forward, source side) or three wavefronts per SIMD, which
-// measured faster than a two-stage register pipeline at three (44.6 against 47 us, forward at L = 8192); groups of
-// 32 rows per wavefront (two member blocks sharing the K / V registers) cut the rows through the L1s by a third
-// but leave two or three wavefronts per SIMD and measured slower (56 us).
 // PIPE: the rows of the next block are loaded while one is used (two-stage register pipeline).  Pays on graphs with few,
-// tall tiles (a dense window graph: 9 blocks per tile, two wavefronts per SIMD in all), costs a wavefront per SIMD.
+// tall tiles (a dense window graph: 9 blocks per tile, two wavefronts per SIMD in all), costs a wavefront per SIMD:
+// at L = 8192, k = 4 (1217 tiles of 4 blocks) the forward takes 47 us with it and 44 without.
+// Other forms measured there and dropped: groups of 32 rows (two member blocks per wavefront sharing the K / V
+// registers: a third fewer rows through the L1s, two or three wavefronts per SIMD, 56 us; two wavefronts per head in step
+// on the same entries, one member block each, so that the L1 fetches a row once: 60 us: the time follows the number
+// of 16 x 16 blocks, 4716 against 6324, not the bytes), five or six wavefronts per SIMD by spilling (53 / 85 us).
 template <bool PIPE, typename Blk, typename Issue, typename Compute>
 __device__ __forceinline__ void tile_walk(int nblk, Issue &&issue, Compute &&compute) {
     if constexpr (PIPE) {
@@ -2391,6 +2392,27 @@ __global__ __launch_bounds__(WAVE) void k_sddmm_grp(bpt_plan P, const T *__restr
     }
 }
 
+// Measurement aid: what the memory system delivers to row gathers.  Every wavefront reads `iters` batches of
+// IN_FLIGHT pseudo-random 1 KB rows (16 bytes per lane, the access pattern of the attention kernels' neighbour rows)
+// of a region and keeps a checksum, so that nothing but the loads is timed.
+template <int IN_FLIGHT>
+__global__ __launch_bounds__(BLOCK) void k_gather_probe(const float4 *__restrict__ base, uint32_t n_rows, int iters, float *__restrict__ sink) {
+    const int lane = threadIdx.x & 63;
+    uint32_t r = (uint32_t)((blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6)) * 2654435761u);
+    float acc = 0.f;
+    for (int i = 0; i < iters; ++i) {
+        float4 x[IN_FLIGHT];
+#pragma unroll
+        for (int u = 0; u < IN_FLIGHT; ++u) {
+            r = r * 1664525u + 1013904223u;                       // row = high word of r * n_rows: two instructions per address
+            x[u] = base[(size_t)__umulhi(r, n_rows) * 64 + lane];
+        }
+#pragma unroll
+        for (int u = 0; u < IN_FLIGHT; ++u) acc += x[u].x + x[u].w;
+    }
+    if (acc == 12345.678f) sink[0] = acc;                      // never true for the zero / random data of the probe
+}
+
 // ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
@@ -3005,6 +3027,23 @@ const char *bpt_strerror(int status) {
 }
 
 int bpt_set_force_generic(int on) { return g_force_generic.exchange(on ? 1 : 0); }
+
+int bpt_gather_probe(const void *region, int64_t region_bytes, int waves_per_cu, int in_flight, int iters, float *sink, void *stream) {
+    if (!region || !sink) return BPT_ERR_NULL;
+    if (region_bytes < 1024 || region_bytes / 1024 > 0x7fffffff || waves_per_cu < WAVES_PER_BLOCK || waves_per_cu > 64 || iters < 1)
+        return BPT_ERR_SIZE;
+    if (!aligned16(region)) return BPT_ERR_UNSUPPORTED;
+    const int grid = 256 * (waves_per_cu / WAVES_PER_BLOCK);      // 256 compute units
+    const uint32_t n_rows = (uint32_t)(region_bytes / 1024);
+    hipStream_t s = (hipStream_t)stream;
+    switch (in_flight) {
+    case 2: hipLaunchKernelGGL((k_gather_probe<2>), dim3(grid), dim3(BLOCK), 0, s, (const float4 *)region, n_rows, iters, sink); break;
+    case 4: hipLaunchKernelGGL((k_gather_probe<4>), dim3(grid), dim3(BLOCK), 0, s, (const float4 *)region, n_rows, iters, sink); break;
+    case 8: hipLaunchKernelGGL((k_gather_probe<8>), dim3(grid), dim3(BLOCK), 0, s, (const float4 *)region, n_rows, iters, sink); break;
+    default: return BPT_ERR_SIZE;
+    }
+    return launch_status();
+}
 
 int bpt_profile_kernel(int which, void *start_event, void *stop_event) {
     if (which != 0 && (!start_event || !stop_event)) return BPT_ERR_NULL;

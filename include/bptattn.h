@@ -85,6 +85,14 @@ int bpt_set_force_generic(int on);
 enum { BPT_KERNEL_NONE = 0, BPT_KERNEL_ATTN_FWD = 1, BPT_KERNEL_ATTN_BWD_DST = 2, BPT_KERNEL_ATTN_BWD_SRC = 3 };
 int bpt_profile_kernel(int which, void *start_event, void *stop_event);
 
+/* Measurement aid (no counterpart in the reference): launches a kernel in which waves_per_cu wavefronts per compute unit
+ * (a multiple of 4, at most 64) each read `iters` batches of in_flight (2, 4 or 8) pseudo-random 1 KB rows of `region`
+ * (region_bytes of device memory, 16-byte aligned), the access pattern of the attention kernels' neighbour-row gathers.
+ * Timed with events by the caller, 256 * waves_per_cu * iters * in_flight KB / duration is the rate at which this GPU's
+ * memory system feeds such gathers: the practical ceiling of these kernels (lower than the streaming bandwidth).
+ * sink: one float of device memory (never written in practice). */
+int bpt_gather_probe(const void *region, int64_t region_bytes, int waves_per_cu, int in_flight, int iters, float *sink, void *stream);
+
 /* Bytes of workspace the call needs (0 possible).  op: one of the BPT_OP_* below. */
 enum {
     BPT_OP_MASKEDMM_BWD = 1, BPT_OP_NODE_MUL_EDGE_BWD = 2, BPT_OP_SPMM_FWD = 3, BPT_OP_SPMM_BWD = 4,
