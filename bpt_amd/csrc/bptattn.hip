@@ -1821,12 +1821,12 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 
 // Backward on tiles, destination side: per block the scores and dO . v of all 16 x 16 pairs (two products over the
 // columns), p = 2^(s - lse), ds = p (dO . v - delta) scale, dq += ds K (third product; K is read a second time in the
-// column layout, which the L1 serves).  (p, ds) of the pairs that exist go to the scratch of the source side: position
-// u' * 16 + m' of the pair in the source-side groups comes from grp_pairs, and the pair is stored at
-// pds[(u' * H + head) * 16 + m'], so that the source-side wavefront of a head reads the 16 members of an entry as 128
-// contiguous bytes.  These scattered 8-byte stores are 36 of the kernel's 92 us at L = 8192, k = 4; letting the source
-// side recompute p and ds instead (two more products there, delta (n, H) handed over) measured slower on every graph
-// tried (L = 4096, k = 16: 0.166 against 0.146 ms per step; window 128: 0.134 against 0.114).
+// column layout, which the L1 serves).  (p, ds) of the pairs that exist go to a scratch in THIS side's layout,
+// pds[(u * H + head) * 16 + m] for entry u and member m: the 16 lanes of a lane group write 128 contiguous bytes.  The
+// source side looks its pairs up there through its pair mapping (grp_pairs).  Writing in the source side's layout instead
+// (scattered 8-byte stores here, contiguous reads there) cost this kernel a third of its time (126 against 85 us at
+// L = 4096, k = 32); letting the source side recompute p and ds (two more products there, delta (n, H) handed over)
+// measured slower than either on every graph tried.
 template <typename T, int H, int D, int HW, bool PIPE>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : 3))) void k_attn_bwd_dst_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
@@ -1876,8 +1876,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 B.kc[r] = *reinterpret_cast<const float4 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
-                // (positions past the group's end are read at its last entry: their masks are empty)
-                B.pos[r] = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
+                B.pos[r] = p0 + TILE_R * b + 4 * g + r;            // (past the group's end the masks are empty)
             }
         };
         auto compute = [&](const Blk &B) {
@@ -1888,7 +1887,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 const bool has = (B.mk[r] >> c) & 1;
                 const float pe = has ? __builtin_amdgcn_exp2f(st[r] - lse_c) : 0.f;
                 ds[r] = pe * (dp[r] - delta) * scale;
-                if (has) pds[((size_t)(B.pos[r] >> 4) * H + t.head) * TILE_R + (B.pos[r] & 15)] = make_float2(pe, ds[r]);
+                if (has) pds[((size_t)B.pos[r] * H + t.head) * TILE_R + c] = make_float2(pe, ds[r]);
             }
             tile_axpy(ds, B.kc, acc);
         };
@@ -1899,7 +1898,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 }
 
 // Backward on tiles, source side (groups of the out-CSR plan: members = source rows, entries = destinations):
-// dk += ds^T q, dv += p^T dO with (p, ds) read from the scratch the destination side filled.
+// dk += ds^T q, dv += p^T dO with (p, ds) of every pair fetched from the scratch the destination side filled, at the
+// position u' * 16 + m' that this plan's grp_pairs gives for (entry, member).
 template <typename T, int H, int D, int HW, bool PIPE>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 3 : 4))) void k_attn_bwd_src_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o, const float2 *__restrict__ pds, T *__restrict__ dk, T *__restrict__ dv,
@@ -1932,7 +1932,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 const size_t off = (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv;
                 B.qr[r] = *reinterpret_cast<const float4 *>(qb + off);
                 B.dr[r] = *reinterpret_cast<const float4 *>(db + off);
-                B.w[r] = pds[((size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * H + t.head) * TILE_R + c];
+                // (positions past the group's end are read at its last entry: their masks are empty)
+                const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
+                B.w[r] = pds[((size_t)(pos >> 4) * H + t.head) * TILE_R + (pos & 15)];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -2794,16 +2796,16 @@ inline bool grouped_backward(const bpt_plan *Pin, const bpt_plan *Pout, int h, i
 // float2 (p, ds) scratch of the fused backward: one per (entry, member) of the source-side groups (plus the
 // look-ahead padding), or one per edge for the per-row kernels
 inline bool tiled_backward(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {
-    return has_tiles(Pin, h, d, elem) && has_tiles(Pout, h, d, elem) && Pin->grp_pairs &&
-           fits32((Pout->n_grp_entries + GRP_PAD_ENTRIES) * TILE_R, (int64_t)h * 8);
+    return has_tiles(Pin, h, d, elem) && has_tiles(Pout, h, d, elem) && Pout->grp_pairs &&
+           fits32((Pin->n_grp_entries + GRP_PAD_ENTRIES) * TILE_R, (int64_t)h * 8);
 }
 
 // float2 (p, ds) scratch of the fused backward: one per (entry, member) of the source-side groups (plus the
 // look-ahead padding), or one per edge for the per-row kernels
 inline int64_t pds_bytes(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {
     int64_t n = Pin->n_edges;
-    if (Pout && (grouped_backward(Pin, Pout, h, d, elem) || tiled_backward(Pin, Pout, h, d, elem)))
-        n = std::max(n, (Pout->n_grp_entries + GRP_PAD_ENTRIES) * Pout->grp_R);
+    if (Pout && grouped_backward(Pin, Pout, h, d, elem)) n = std::max(n, (Pout->n_grp_entries + GRP_PAD_ENTRIES) * Pout->grp_R);
+    if (Pout && tiled_backward(Pin, Pout, h, d, elem)) n = std::max(n, (Pin->n_grp_entries + GRP_PAD_ENTRIES) * Pin->grp_R);
     return 2 * round16(n * h * 4);
 }
 

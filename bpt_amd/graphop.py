@@ -418,8 +418,9 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
             seg = _tile_seg_len(plan_in)
             plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg)
             plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg)
-            in_ref = ctypes.byref(plan_in.linked_to(plan_out, TILE_ROWS))
-            out_ref = ctypes.byref(plan_out.ensure_groups(TILE_ROWS, GROUP_ORDER_SRC)["struct"])
+            # the destination side writes (p, ds) in its own layout; the source side finds them through its pair mapping
+            in_ref = ctypes.byref(plan_in.ensure_groups(TILE_ROWS)["struct"])
+            out_ref = ctypes.byref(plan_out.linked_to(plan_in, TILE_ROWS, partner_order=None))
         else:
             R = _group_rows(q, h, d, plan_in, cfg)
             in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
@@ -513,11 +514,12 @@ def _tiles(q, h, d, plan, dropout_p, bias, cfg):
 
 def _tiles_backward(plan):
     """The backward runs on tiles where that measured faster than the row-group kernels (float32, 8 x 64): on small graphs,
-    which the row groups of 8 cannot spread over the GPU (L = 4096: k = 4 ... 32 run 7 to 27 % faster), and on dense ones
-    (window 128: 1.9 x); at L = 8192, k = 4 and on the 32-graph batch the row-group kernels win (0.203 against 0.214 ms)."""
+    which the row groups of 8 cannot spread over the GPU (L = 4096: k = 1 ... 4 run level to 3 % faster), and on graphs of
+    mean degree 32 and more (L = 4096, k = 8 ... 32: 15 to 27 %; window 128: 1.9 x; L = 32768, k = 8, 16 heads: 3 %); at
+    L = 8192, k = 4 and on the 32-graph batch the row-group kernels win (0.203 against 0.213 ms, 0.323 against 0.329)."""
     if TILE_BACKWARD is not None:
         return TILE_BACKWARD
-    return plan.n_rows < 12288 or plan.n_edges >= 64 * max(plan.n_rows, 1)
+    return plan.n_rows < 12288 or plan.n_edges >= 32 * max(plan.n_rows, 1)
 
 
 def _tile_seg_len(plan):

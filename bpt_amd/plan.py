@@ -218,11 +218,13 @@ class Plan:
                 self._groups[(R, order_mode)] = hit
         return hit
 
-    def linked_to(self, plan_src, R=GROUP_R):
-        """`bpt_plan` of this (destination-side) plan whose grp_pairs maps each (entry, member) of its groups to
-        the position entry' * R + member' of the same edge in `plan_src` (the source-side plan of the same graph)."""
-        mine, theirs = self.ensure_groups(R), plan_src.ensure_groups(R, GROUP_ORDER_SRC)
-        key = (id(plan_src), R)
+    def linked_to(self, plan_src, R=GROUP_R, order=None, partner_order=GROUP_ORDER_SRC):
+        """`bpt_plan` of this plan whose grp_pairs maps each (entry, member) of its groups (built with `order`) to the
+        position entry' * R + member' of the same edge in the groups of `plan_src` (the plan of the other CSR side of the
+        same graph, groups built with `partner_order`).  The row-group kernels link the destination side to the source
+        side, the tile kernels the source side to the destination side."""
+        mine, theirs = self.ensure_groups(R, order), plan_src.ensure_groups(R, partner_order)
+        key = (id(plan_src), R, order, partner_order)
         with self._lock:
             hit = self._links.get(key)
             if hit is None:
@@ -398,10 +400,10 @@ class DevicePlan:
                 self._groups[(R, by_mask)] = hit
         return hit
 
-    def linked_to(self, plan_src, R=GROUP_R):
+    def linked_to(self, plan_src, R=GROUP_R, order=None, partner_order=GROUP_ORDER_SRC):
         """As Plan.linked_to, with the pair mapping computed on the GPU (bpt_plan_link_device)."""
-        mine, theirs = self.ensure_groups(R), plan_src.ensure_groups(R, GROUP_ORDER_SRC)
-        key = (id(plan_src), R)
+        mine, theirs = self.ensure_groups(R, order), plan_src.ensure_groups(R, partner_order)
+        key = (id(plan_src), R, order, partner_order)
         with self._lock:
             hit = self._links.get(key)
             if hit is None:

@@ -94,7 +94,7 @@ def check_groups(hit, grp, n_edges):
 @pytest.mark.parametrize("seg", [8, 64])
 @pytest.mark.parametrize("name", sorted(GRAPHS))
 def test_device_plan_equals_model_and_host(name, seg):
-    from bpt_amd.plan import GROUP_PAD_ENTRIES, DevicePlan, build_plan_host
+    from bpt_amd.plan import GROUP_ORDER_SRC, GROUP_PAD_ENTRIES, DevicePlan, build_plan_host
     src, dst, n, csr, a_in, a_out, t_in, t_out = sides(name)
     plans = []
     for arrs, tens in ((a_in, t_in), (a_out, t_out)):
@@ -114,7 +114,14 @@ def test_device_plan_equals_model_and_host(name, seg):
         if R != 16:
             st = plans[0][0].linked_to(plans[1][0], R)
             want = model.link_groups(grps[0], grps[1], len(src), GROUP_PAD_ENTRIES)
-            got = host(plans[0][0]._links[(id(plans[1][0]), R)][1])
+            got = host(plans[0][0]._links[(id(plans[1][0]), R, None, GROUP_ORDER_SRC)][1])
+            assert np.array_equal(got, want) and st.grp_pairs
+        else:
+            # the tile kernels link the other way round: source side -> destination side, both in the default order
+            grps = [model.group_plan(arrays, n, R, 1) for dp, arrays in plans]
+            st = plans[1][0].linked_to(plans[0][0], R, partner_order=None)
+            want = model.link_groups(grps[1], grps[0], len(src), GROUP_PAD_ENTRIES)
+            got = host(plans[1][0]._links[(id(plans[0][0]), R, None, None)][1])
             assert np.array_equal(got, want) and st.grp_pairs
 
 
@@ -312,7 +319,7 @@ def test_device_plan_on_random_graphs(seed):
     """Seeded random multigraphs (empty rows, rows longer than a segment, repeated edges, more index nodes than rows):
     CSR, base plan, groups and pair mapping equal the host builders / the model."""
     from bpt_amd import graphbuilder as gb
-    from bpt_amd.plan import GROUP_PAD_ENTRIES, DevicePlan
+    from bpt_amd.plan import GROUP_ORDER_SRC, GROUP_PAD_ENTRIES, DevicePlan
     rng = np.random.default_rng(100 + seed)
     n = int(rng.integers(1, 300))
     E = int(rng.integers(0, 4000))
@@ -339,7 +346,8 @@ def test_device_plan_on_random_graphs(seed):
         check_groups(dp.ensure_groups(R, {0: 2, 1: 6, 2: 10}[by_mask]), grp, E)
         plans.append(dp); grps.append(grp)
     plans[0].linked_to(plans[1], R)
-    assert np.array_equal(host(plans[0]._links[(id(plans[1]), R)][1]), model.link_groups(grps[0], grps[1], E, GROUP_PAD_ENTRIES))
+    assert np.array_equal(host(plans[0]._links[(id(plans[1]), R, None, GROUP_ORDER_SRC)][1]),
+                          model.link_groups(grps[0], grps[1], E, GROUP_PAD_ENTRIES))
 
 
 def test_batch_merge_on_the_device_and_the_whole_pipeline_time():
