@@ -33,6 +33,8 @@ DEVICE_BUILD_MIN_ROWS = 24576   # None: graphs with at least this many rows are 
                                 # simpler grouping runs the fused kernels 4-9 % faster there and builds 10-30 x faster),
 DEVICE_BUILD_MIN_DEGREE = 32    # and so are graphs of at least 2^17 edges with this average degree (L = 4096: k = 8, 16,
                                 # 32 run 5, 3 and 18 % faster on GPU-built groups, k = 1 and 4 run 8 and 1 % slower)
+DEVICE_BUILD_DENSE_MIN_ROWS = 2048   # if they have this many rows: the CSR of 1000 edge types over 430 k edges (the table
+                                     # gradient of the rel_pos term) runs its SpMM in 40 us on host-built groups, 130 us on GPU-built ones
 
 
 def _ptr(a):
@@ -241,7 +243,7 @@ class Plan:
 def set_device_build(on):
     """Plans of graphs seen from now on are built on the GPU (True: DevicePlan), on the host (False: Plan), or where
     their size says (None, the default: on the GPU from DEVICE_BUILD_MIN_ROWS rows, or from 2^17 edges at an average
-    degree of DEVICE_BUILD_MIN_DEGREE).  Returns the old setting."""
+    degree of DEVICE_BUILD_MIN_DEGREE and DEVICE_BUILD_DENSE_MIN_ROWS rows).  Returns the old setting."""
     global DEVICE_BUILD
     old, DEVICE_BUILD = DEVICE_BUILD, (None if on is None else bool(on))
     return old
@@ -254,7 +256,8 @@ def _build_on_device(eid, n_rows):
         if n_rows is None:
             return False
         n_edges = int(eid.numel())
-        return n_rows >= DEVICE_BUILD_MIN_ROWS or (n_edges >= (1 << 17) and n_edges >= DEVICE_BUILD_MIN_DEGREE * n_rows)
+        return n_rows >= DEVICE_BUILD_MIN_ROWS or (n_rows >= DEVICE_BUILD_DENSE_MIN_ROWS and n_edges >= (1 << 17) and
+                                                   n_edges >= DEVICE_BUILD_MIN_DEGREE * n_rows)
     return DEVICE_BUILD
 
 
