@@ -348,7 +348,8 @@ def main():
         "config": {"workload": desc + (" (op chain with rel_pos)" if args.rel_pos and args.unfused else " (fused fwd+bwd with rel_pos)" if args.rel_pos else " (unfused op chain)" if args.unfused else
                                        f" (fused fwd+bwd, attention dropout {args.dropout})" if args.dropout > 0 else " (fused fwd+bwd)"), "n_nodes": N,
                    "n_edges": E, "heads": H, "d_head": D, "launch": mode,
-                   "kernels": "per-row" if args.rows else f"row-groups({args.group_rows or 'auto'} rows per wavefront)"},
+                   "kernels": "per-row" if args.rows else f"row groups of {args.group_rows}" if args.group_rows else
+                              "auto (tiles of 16 rows or row groups of 4 / 8, by dtype and graph)"},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "step_roofline": {"algorithmic_bytes": alg["total"], "achieved_GBps": round(step_gbs, 1),
