@@ -1617,7 +1617,7 @@ struct TileCtx {
 
 template <typename T, int H, int D, int HW>
 __device__ __forceinline__ bool tile_begin(const bpt_plan &P, TileCtx &t) {
-    static_assert(D == 64 && H % HW == 0 && sizeof(T) == 4, "float32 rows, four 16-column slices per head, one per lane group");
+    static_assert(D == 64 && H % HW == 0 && (sizeof(T) == 4 || sizeof(T) == 2), "64 columns per head: one 16-column slice per lane group");
     constexpr int HS = H / HW;
     t.lane = threadIdx.x & (WAVE - 1);
     t.wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1683,8 +1683,8 @@ __device__ __forceinline__ void tile_axpy(const float (&w)[4], const float4 (&ro
 
 // The members' result rows: whole rows go to `out` (scaled by inv[member] where given), segments of split rows to the
 // workspace in natural column order.
-template <int H, int D, bool SCALE>
-__device__ __forceinline__ void tile_store_rows(const TileCtx &t, const floatx4v (&acc)[4], float inv_c, float *__restrict__ out,
+template <int H, int D, bool SCALE, typename T>
+__device__ __forceinline__ void tile_store_rows(const TileCtx &t, const floatx4v (&acc)[4], float inv_c, T *__restrict__ out,
                                                 float *__restrict__ ws) {
     constexpr int C = H * D;
 #pragma unroll
@@ -1696,7 +1696,13 @@ __device__ __forceinline__ void tile_store_rows(const TileCtx &t, const floatx4v
         float4 x = make_float4(acc[0][r], acc[1][r], acc[2][r], acc[3][r]);
         if (slot < 0) {
             if (SCALE) { x.x *= inv; x.y *= inv; x.z *= inv; x.w *= inv; }
-            *reinterpret_cast<float4 *>(out + (size_t)row * C + t.head * D + 4 * t.c) = x;
+            if constexpr (sizeof(T) == 4) {
+                *reinterpret_cast<float4 *>(out + (size_t)row * C + t.head * D + 4 * t.c) = x;
+            } else {
+                const uint2 y = make_uint2(((uint32_t)f32_to_bf16(x.x)) | ((uint32_t)f32_to_bf16(x.y) << 16),
+                               ((uint32_t)f32_to_bf16(x.z)) | ((uint32_t)f32_to_bf16(x.w) << 16));
+                *reinterpret_cast<uint2 *>(out + (size_t)row * C + t.head * D + 4 * t.c) = y;
+            }
         } else {
             *reinterpret_cast<float4 *>(ws + (size_t)slot * C + t.head * D + 4 * t.c) = x;
         }
@@ -1808,7 +1814,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     }
     float lt = lrun + __shfl_xor(lrun, 16);
     lt += __shfl_xor(lt, 32);                                    // denominator of member c, in its four lanes
-    tile_store_rows<H, D, true>(t, acc, lt > 0.f ? 1.f / lt : 0.f, reinterpret_cast<float *>(o), ws_acc);
+    tile_store_rows<H, D, true>(t, acc, lt > 0.f ? 1.f / lt : 0.f, o, ws_acc);
     if (g == 0 && t.member.x >= 0) {                              // lanes 0 .. 15: one member each
         if (t.member.y < 0) {
             lse[(size_t)t.member.x * H + t.head] = lt > 0.f ? mref + log2f(lt) : 0.f;
@@ -1894,7 +1900,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         tile_walk<PIPE, Blk>(nblk, issue, compute);
         wave_lds_fence();
     }
-    tile_store_rows<H, D, false>(t, acc, 1.f, reinterpret_cast<float *>(dq), ws_dq);
+    tile_store_rows<H, D, false>(t, acc, 1.f, dq, ws_dq);
 }
 
 // Backward on tiles, source side (groups of the out-CSR plan: members = source rows, entries = destinations):
@@ -1951,8 +1957,281 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         tile_walk<PIPE, Blk>(nblk, issue, compute);
         wave_lds_fence();
     }
-    tile_store_rows<H, D, false>(t, ak, 1.f, reinterpret_cast<float *>(dk), ws_dk);
-    tile_store_rows<H, D, false>(t, av, 1.f, reinterpret_cast<float *>(dv), ws_dv);
+    tile_store_rows<H, D, false>(t, ak, 1.f, dk, ws_dk);
+    tile_store_rows<H, D, false>(t, av, 1.f, dv, ws_dv);
+}
+
+// ---- Dense tiles for bfloat16 rows.  Same walk and the same lane roles as the float32 tile kernels above, on
+// v_mfma_f32_16x16x32_bf16 (products over the 64 columns: two instructions) and v_mfma_f32_16x16x16_bf16 (products over
+// the 16 entries of a block: one instruction per four output columns), operands as loaded, float32 accumulation:
+//   lane (c, g) loads columns 16 g .. 16 g + 15 of the row of entry c (32 contiguous bytes; slot j of step t of the product
+//   stands for column 16 g + 8 t + j in both operands) and columns 4 c .. 4 c + 3 of the rows of entries 4 g + r (8 bytes;
+//   the B operand of output columns {4 c + nb} takes element nb of each of the four, packed by byte permutes).
+// Probabilities and ds are rounded to bfloat16 where they enter a product (the softmax denominator is summed unrounded);
+// the scratch between the two backward kernels holds (p, ds) as two bfloat16 in 4 bytes, in the destination side's layout.
+// The two-stage register pipeline of tile_walk does not pay here: at six wavefronts per SIMD it spills (2.4 x slower),
+// at four it measured 5 to 10 % slower on the sparse graphs and level on the window graph.
+constexpr bool TILE_BF16_PIPE = false;
+constexpr int TILE_BF16_WPE = 6, TILE_BF16_WPE_DST = 5;     // wavefronts per SIMD the bfloat16 tile kernels are compiled for
+typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+typedef float floatx2v __attribute__((ext_vector_type(2)));
+typedef short shortx4v __attribute__((ext_vector_type(4)));
+union Bf8 { bf16x8v v; uint4 q; };
+union Bf4 { shortx4v v; uint32_t u[2]; };
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    union { bf16x2v v; uint32_t u; } r;
+    r.v = __builtin_convertvector(floatx2v{lo, hi}, bf16x2v);      // round to nearest even
+    return r.u;
+}
+__device__ __forceinline__ uint32_t pack_lo16(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }   // (a.lo, b.lo)
+__device__ __forceinline__ uint32_t pack_hi16(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }   // (a.hi, b.hi)
+
+// B operand of output columns {4 c + nb}: element nb of the 8-byte pieces of the rows of entries 4 g + r, r = 0 .. 3
+template <int NB>
+__device__ __forceinline__ Bf4 tile_cols_bf16(const uint2 (&rows)[4]) {
+    Bf4 b;
+    if constexpr (NB == 0) { b.u[0] = pack_lo16(rows[0].x, rows[1].x); b.u[1] = pack_lo16(rows[2].x, rows[3].x); }
+    if constexpr (NB == 1) { b.u[0] = pack_hi16(rows[0].x, rows[1].x); b.u[1] = pack_hi16(rows[2].x, rows[3].x); }
+    if constexpr (NB == 2) { b.u[0] = pack_lo16(rows[0].y, rows[1].y); b.u[1] = pack_lo16(rows[2].y, rows[3].y); }
+    if constexpr (NB == 3) { b.u[0] = pack_hi16(rows[0].y, rows[1].y); b.u[1] = pack_hi16(rows[2].y, rows[3].y); }
+    return b;
+}
+// acc[nb][r'] (member 4 g + r', column 4 c + nb) += sum over the block's entries of w[member c][entry 4 g + r] * row[entry][column]
+__device__ __forceinline__ void tile_axpy_bf16(const Bf4 &w, const uint2 (&rows)[4], floatx4v (&acc)[4]) {
+    acc[0] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w.v, tile_cols_bf16<0>(rows).v, acc[0], 0, 0, 0);
+    acc[1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w.v, tile_cols_bf16<1>(rows).v, acc[1], 0, 0, 0);
+    acc[2] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w.v, tile_cols_bf16<2>(rows).v, acc[2], 0, 0, 0);
+    acc[3] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w.v, tile_cols_bf16<3>(rows).v, acc[3], 0, 0, 0);
+}
+// register r of lane (c, g) = sum over the 64 columns of a[entry 4 g + r] * b[member c]
+__device__ __forceinline__ floatx4v tile_dot_bf16(const Bf8 (&a)[2], const Bf8 (&b)[2]) {
+    floatx4v s = floatx4v{0.f, 0.f, 0.f, 0.f};
+    s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[0].v, b[0].v, s, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[1].v, b[1].v, s, 0, 0, 0);
+}
+__device__ __forceinline__ void tile_load_row_bf16(const char *p, Bf8 (&out)[2]) {
+    out[0].q = *reinterpret_cast<const uint4 *>(p);
+    out[1].q = *reinterpret_cast<const uint4 *>(p + 16);
+}
+
+template <int H, int D, int HW, int WPE, bool PIPE>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_fwd_tile_bf16(
+    bpt_plan P, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v, bf16_t *__restrict__ o,
+    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+    constexpr int RB = H * D * 2;                                 // bytes of a node row
+    TileCtx t;
+    if (!tile_begin<bf16_t, H, D, HW>(P, t)) return;
+    __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    int2 *ent = ent_lds[t.wv];
+    const int c = t.c, g = t.g;
+    const uint32_t offr = (uint32_t)((t.head * D + 16 * g) * 2), offc = (uint32_t)((t.head * D + 4 * c) * 2);
+    const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
+    Bf8 qb[2];
+    tile_load_row_bf16(reinterpret_cast<const char *>(q) + (size_t)max(t.member.x, 0) * RB + offr, qb);
+    floatx4v acc[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
+    float mref = M_INIT_LOG2, lrun = 0.f;
+    struct Blk {
+        Bf8 kr[2];
+        uint2 vr[4];
+        int mk[4];
+    };
+    for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
+        const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
+        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        auto issue = [&](Blk &B, int b) {
+            const int2 ea = ent[TILE_R * b + c];
+            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
+            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
+            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+            tile_load_row_bf16(kb + (size_t)((uint32_t)ea.x * (uint32_t)RB) + offr, B.kr);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) B.vr[r] = *reinterpret_cast<const uint2 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
+        };
+        auto compute = [&](const Blk &B) {
+            const floatx4v st = tile_dot_bf16(B.kr, qb);
+            float sc[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sc[r] = ((B.mk[r] >> c) & 1) ? st[r] * scale_log2e : -INFINITY;
+            const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+            if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
+                float gm = fmaxf(mb, __shfl_xor(mb, 16));
+                gm = fmaxf(gm, __shfl_xor(gm, 32));              // over the four lanes of member c
+                const float mn = fmaxf(mref, gm);
+                const float al = __builtin_amdgcn_exp2f(mref - mn);
+                mref = mn;
+                lrun *= al;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float a = lane_bcast(al, 4 * g + r);
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) acc[nb][r] *= a;
+                }
+            }
+            float pr[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                pr[r] = __builtin_amdgcn_exp2f(sc[r] - mref);
+                lrun += pr[r];
+            }
+            Bf4 pa;
+            pa.u[0] = pack_bf16(pr[0], pr[1]);
+            pa.u[1] = pack_bf16(pr[2], pr[3]);
+            tile_axpy_bf16(pa, B.vr, acc);
+        };
+        tile_walk<PIPE, Blk>(nblk, issue, compute);
+        wave_lds_fence();
+    }
+    float lt = lrun + __shfl_xor(lrun, 16);
+    lt += __shfl_xor(lt, 32);
+    tile_store_rows<H, D, true>(t, acc, lt > 0.f ? 1.f / lt : 0.f, o, ws_acc);
+    if (g == 0 && t.member.x >= 0) {
+        if (t.member.y < 0) {
+            lse[(size_t)t.member.x * H + t.head] = lt > 0.f ? mref + log2f(lt) : 0.f;
+        } else {
+            ws_ml[((size_t)t.member.y * H + t.head) * 2] = mref;
+            ws_ml[((size_t)t.member.y * H + t.head) * 2 + 1] = lt;
+        }
+    }
+}
+
+template <int H, int D, int HW, int WPE, bool PIPE>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_dst_tile_bf16(
+    bpt_plan P, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v, const bf16_t *__restrict__ o,
+    const bf16_t *__restrict__ d_o, const float *__restrict__ lse, bf16_t *__restrict__ dq, uint32_t *__restrict__ pds,
+    float *__restrict__ ws_dq, float scale, float scale_log2e) {
+    constexpr int RB = H * D * 2;
+    TileCtx t;
+    if (!tile_begin<bf16_t, H, D, HW>(P, t)) return;
+    __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    int2 *ent = ent_lds[t.wv];
+    const int c = t.c, g = t.g;
+    const uint32_t offr = (uint32_t)((t.head * D + 16 * g) * 2), offc = (uint32_t)((t.head * D + 4 * c) * 2);
+    const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
+    const size_t mrow = (size_t)max(t.member.x, 0) * RB + offr;
+    Bf8 qb[2], dob[2];
+    float delta, lse_c;
+    {
+        Bf8 ob[2];
+        tile_load_row_bf16(reinterpret_cast<const char *>(q) + mrow, qb);
+        tile_load_row_bf16(reinterpret_cast<const char *>(d_o) + mrow, dob);
+        tile_load_row_bf16(reinterpret_cast<const char *>(o) + mrow, ob);
+        float part = 0.f;
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+            const uint32_t a[4] = {dob[h2].q.x, dob[h2].q.y, dob[h2].q.z, dob[h2].q.w}, b[4] = {ob[h2].q.x, ob[h2].q.y, ob[h2].q.z, ob[h2].q.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                part = fmaf(__uint_as_float(a[i] << 16), __uint_as_float(b[i] << 16), part);
+                part = fmaf(__uint_as_float(a[i] & 0xffff0000u), __uint_as_float(b[i] & 0xffff0000u), part);
+            }
+        }
+        part += __shfl_xor(part, 16);
+        delta = part + __shfl_xor(part, 32);                      // dO . O of member c, this head
+        lse_c = lse[(size_t)max(t.member.x, 0) * H + t.head];
+    }
+    floatx4v acc[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
+    struct Blk {
+        Bf8 kr[2], va[2];
+        uint2 kc[4];
+        int mk[4], pos0;
+    };
+    for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
+        const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
+        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        auto issue = [&](Blk &B, int b) {
+            const int2 ea = ent[TILE_R * b + c];
+            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
+            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
+            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+            const size_t arow = (size_t)((uint32_t)ea.x * (uint32_t)RB) + offr;
+            tile_load_row_bf16(kb + arow, B.kr);
+            tile_load_row_bf16(vb + arow, B.va);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) B.kc[r] = *reinterpret_cast<const uint2 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
+            B.pos0 = p0 + TILE_R * b + 4 * g;                     // (past the group's end the masks are empty)
+        };
+        auto compute = [&](const Blk &B) {
+            const floatx4v st = tile_dot_bf16(B.kr, qb), dp = tile_dot_bf16(B.va, dob);
+            float ds[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool has = (B.mk[r] >> c) & 1;
+                const float pe = has ? __builtin_amdgcn_exp2f(st[r] * scale_log2e - lse_c) : 0.f;
+                ds[r] = pe * (dp[r] - delta) * scale;
+                if (has) pds[((size_t)(B.pos0 + r) * H + t.head) * TILE_R + c] = pack_bf16(pe, ds[r]);
+            }
+            Bf4 da;
+            da.u[0] = pack_bf16(ds[0], ds[1]);
+            da.u[1] = pack_bf16(ds[2], ds[3]);
+            tile_axpy_bf16(da, B.kc, acc);
+        };
+        tile_walk<PIPE, Blk>(nblk, issue, compute);
+        wave_lds_fence();
+    }
+    tile_store_rows<H, D, false>(t, acc, 1.f, dq, ws_dq);
+}
+
+template <int H, int D, int HW, int WPE, bool PIPE>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_src_tile_bf16(
+    bpt_plan P, const bf16_t *__restrict__ q, const bf16_t *__restrict__ d_o, const uint32_t *__restrict__ pds, bf16_t *__restrict__ dk,
+    bf16_t *__restrict__ dv, float *__restrict__ ws_dk, float *__restrict__ ws_dv) {
+    constexpr int RB = H * D * 2;
+    TileCtx t;
+    if (!tile_begin<bf16_t, H, D, HW>(P, t)) return;
+    __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    int2 *ent = ent_lds[t.wv];
+    const int c = t.c, g = t.g;
+    const uint32_t offc = (uint32_t)((t.head * D + 4 * c) * 2);
+    const char *qb = reinterpret_cast<const char *>(q), *db = reinterpret_cast<const char *>(d_o);
+    floatx4v ak[4], av[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) { ak[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; av[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; }
+    struct Blk {
+        uint2 qr[4], dr[4];
+        uint32_t w[4];
+        int mk[4];
+    };
+    for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
+        const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
+        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        auto issue = [&](Blk &B, int b) {
+            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
+            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
+            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const size_t off = (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc;
+                B.qr[r] = *reinterpret_cast<const uint2 *>(qb + off);
+                B.dr[r] = *reinterpret_cast<const uint2 *>(db + off);
+                // (positions past the group's end are read at its last entry: their masks are empty)
+                const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
+                B.w[r] = pds[((size_t)(pos >> 4) * H + t.head) * TILE_R + (pos & 15)];
+            }
+        };
+        auto compute = [&](const Blk &B) {
+            uint32_t w[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) w[r] = ((B.mk[r] >> c) & 1) ? B.w[r] : 0u;     // the scratch of pairs that do not exist is not initialised
+            Bf4 pa, da;
+            pa.u[0] = pack_lo16(w[0], w[1]); pa.u[1] = pack_lo16(w[2], w[3]);
+            da.u[0] = pack_hi16(w[0], w[1]); da.u[1] = pack_hi16(w[2], w[3]);
+            tile_axpy_bf16(da, B.qr, ak);
+            tile_axpy_bf16(pa, B.dr, av);
+        };
+        tile_walk<PIPE, Blk>(nblk, issue, compute);
+        wave_lds_fence();
+    }
+    tile_store_rows<H, D, false>(t, ak, 1.f, dk, ws_dk);
+    tile_store_rows<H, D, false>(t, av, 1.f, dv, ws_dv);
 }
 
 // Backward, destination side.  Writes (p, ds) of every pair to pds[(t * H + head)], t = the pair's
@@ -2735,7 +3014,7 @@ inline bool has_groups(const bpt_plan *P, int h, int d, size_t elem) {
 // groups of 16 rows for the dense-tile kernels (one wavefront per head: h * 64 threads per workgroup)
 inline bool has_tiles(const bpt_plan *P, int h, int d, size_t elem) {
     return P->n_groups > 0 && P->grp_R == TILE_R && P->grp_members && P->grp_ptr && P->grp_entries && P->grp_chunks &&
-           P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups && P->n_grp_entries >= 0 && d == 64 && h <= 16 && elem == 4 &&
+           P->grp_max_chunk > 0 && 8 * P->grp_max_chunk >= P->n_groups && P->n_grp_entries >= 0 && d == 64 && h <= 16 && (elem == 4 || elem == 2) &&
            fits32(P->n_rows, (int64_t)h * d * (int64_t)elem);
 }
 
@@ -2829,6 +3108,14 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
                 goto launched;
             }
         }
+        if constexpr (D == 64 && sizeof(T) == 2) {
+            if (has_tiles(P, H, D, sizeof(T)) && drop.thr == 0 && !bias) {
+                constexpr int HW = H >= 4 ? 4 : H;
+                hipLaunchKernelGGL((k_attn_fwd_tile_bf16<H, D, HW, TILE_BF16_WPE, TILE_BF16_PIPE>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), 0, s, *P,
+                                   (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (bf16_t *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+                goto launched;
+            }
+        }
         if (has_groups(P, H, D, sizeof(T))) {
 #define LAUNCH_FWD(RR, DR, BI)                                                                                                   \
     hipLaunchKernelGGL((k_attn_fwd_grp<T, H, D, RR, HS, DR, BI>), dim3(group_grid(P) * HS), dim3(WAVE), 0, s, *P, (const T *)q, \
@@ -2907,6 +3194,31 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
                 else
                     hipLaunchKernelGGL((k_attn_bwd_src_tile<T, H, D, HW, false>), dim3(group_grid(Pout) * (H / HW)), dim3(HW * WAVE), 0, s, *Pout,
                                        (const T *)q, (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv);
+            }
+            st = launch_status();
+            if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;
+            hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / WAVE, 2), dim3(BLOCK), 0, s, Pin->heavy,
+                               (int)Pin->n_heavy, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
+                               (size_t)Pout->n_slots * H * D);
+            return launch_status();
+        }
+    }
+    if constexpr (D == 64 && sizeof(T) == 2) {
+        if (tiled_backward(Pin, Pout, H, D, sizeof(T)) && drop.thr == 0 && !bias) {
+            constexpr int HW = H >= 4 ? 4 : H;
+            float *ws_dk = ws_rows + (size_t)Pin->n_slots * H * D, *ws_dv = ws_dk + (size_t)Pout->n_slots * H * D;
+            {
+                ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
+                hipLaunchKernelGGL((k_attn_bwd_dst_tile_bf16<H, D, HW, TILE_BF16_WPE_DST, TILE_BF16_PIPE>), dim3(group_grid(Pin) * (H / HW)), dim3(HW * WAVE), 0, s,
+                                   *Pin, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)o, (const bf16_t *)d_o, lse,
+                                   (bf16_t *)dq, (uint32_t *)ws, ws_rows, scale, scale * LOG2E);
+            }
+            int st = launch_status();
+            if (st != BPT_OK) return st;
+            {
+                ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
+                hipLaunchKernelGGL((k_attn_bwd_src_tile_bf16<H, D, HW, TILE_BF16_WPE, TILE_BF16_PIPE>), dim3(group_grid(Pout) * (H / HW)), dim3(HW * WAVE), 0, s,
+                                   *Pout, (const bf16_t *)q, (const bf16_t *)d_o, (const uint32_t *)ws, (bf16_t *)dk, (bf16_t *)dv, ws_dk, ws_dv);
             }
             st = launch_status();
             if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;

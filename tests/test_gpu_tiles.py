@@ -105,6 +105,37 @@ def test_tile_kernels_match_the_oracle(gname, seg, heads):
         assert not o[0].any() and not qd.grad[0].any()                            # the node without edges
 
 
+BF16_TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("gname,seg,heads", [(g, s, 8) for g, s in CASES] + [(g, s, 16) for g, s in OTHER_HEADS])
+def test_tile_kernels_in_bfloat16_match_the_oracle(gname, seg, heads):
+    """bfloat16 rows on the tile kernels (operands as loaded on the bfloat16 matrix instructions, float32 accumulation,
+    (p, ds) handed from the destination to the source side as bfloat16 pairs): rtol 2e-2 / atol 2e-2 against the float64
+    oracle on the same (bfloat16-rounded) inputs; 8 heads and 16 (the two sizes the fused bfloat16 path is compiled for)."""
+    from oracle import torch_ops
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd import op
+    src, dst, n_k, n_q = graphs(gname)
+    csr = gb.get_csrs_bipartite(src, dst, n_k, n_q)
+    out_csr, in_csr, ROW, IR, COL, IC = csr
+    args = tuple(x.to(DEV) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
+    gen = torch.Generator().manual_seed(19)
+    q, do = (torch.randn(n_q, heads, 64, generator=gen).to(torch.bfloat16) for _ in range(2))
+    k, v = (torch.randn(n_k, heads, 64, generator=gen).to(torch.bfloat16) for _ in range(2))
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    with forced_tiles(seg):
+        o = op.bpt_attention(*args, qd, kd, vd, fused=True)
+        o.backward(do.to(DEV))
+        o2 = op.bpt_attention(*args, qd.detach(), kd.detach(), vd.detach(), fused=True)
+        from bpt_amd.plan import plan_cache
+        assert [p for p, _ in plan_cache._d.values() if any(key[0] == 16 for key in p._groups)], "the tile kernels did not run"
+    assert o.dtype == torch.bfloat16 and torch.equal(o.detach(), o2)
+    ro, rdq, rdk, rdv = torch_ops.attention_fwd_bwd(torch.from_numpy(src), torch.from_numpy(dst), f64(q), f64(k), f64(v), f64(do))
+    check(o, ro, BF16_TOL, "o")
+    check(qd.grad, rdq, BF16_TOL, "dq"); check(kd.grad, rdk, BF16_TOL, "dk"); check(vd.grad, rdv, BF16_TOL, "dv")
+
+
 def test_tiles_agree_with_the_row_group_kernels_on_the_headline_graph():
     """L = 8192, k = 4, causal, 8 x 64: tile forward + tile backward against the row-group kernels (themselves checked
     against the oracle in test_headline_graph_full_parity) and against the oracle's forward."""
