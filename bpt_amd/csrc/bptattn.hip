@@ -1709,6 +1709,13 @@ __device__ __forceinline__ void tile_store_rows(const TileCtx &t, const floatx4v
     }
 }
 
+// Edge ids of this lane's four pairs of a block, (entry 4 g + r, member c): what the dropout hash and the score term are
+// indexed by (n_edges, the spare row, where the pair does not exist; past the group's end the last entry is read again).
+__device__ __forceinline__ void tile_pair_eids(const bpt_plan &P, int first_entry, int p_end, int c, int (&xe)[4]) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) xe[r] = P.grp_eids[(size_t)min(first_entry + r, p_end - 1) * TILE_R + c];
+}
+
 // PIPE: the rows of the next block are loaded while one is used (two-stage register pipeline).  Pays on graphs with few,
 // tall tiles (a dense window graph: 9 blocks per tile, two wavefronts per SIMD in all), costs a wavefront per SIMD:
 // at L = 8192, k = 4 (1217 tiles of 4 blocks) the forward takes 47 us with it and 44 without.
@@ -1742,10 +1749,11 @@ __device__ __forceinline__ void tile_walk(int nblk, Issue &&issue, Compute &&com
     }
 }
 
-template <typename T, int H, int D, int HW, bool PIPE>
+template <typename T, int H, int D, int HW, bool PIPE, bool DROP, bool BIAS>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 3 : 4))) void k_attn_fwd_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o, float *__restrict__ lse,
-    float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+    float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv,
+    const float *__restrict__ bias) {
     constexpr int C = H * D;
     TileCtx t;
     if (!tile_begin<T, H, D, HW>(P, t)) return;
@@ -1765,11 +1773,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         float kr[16];
         float4 vr[4];
         int mk[4];
+        int xe[DROP || BIAS ? 4 : 1];
+        float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
         auto issue = [&](Blk &B, int b) {
+            if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -1779,12 +1790,16 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 B.vr[r] = *reinterpret_cast<const float4 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
+            if constexpr (BIAS) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
+            }
         };
         auto compute = [&](const Blk &B) {
             const floatx4v st = tile_dot(B.kr, qb);
             float sc[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sc[r] = ((B.mk[r] >> c) & 1) ? st[r] : -INFINITY;
+            for (int r = 0; r < 4; ++r) sc[r] = ((B.mk[r] >> c) & 1) ? (BIAS ? fmaf(B.bz[BIAS ? r : 0], scale_log2e, st[r]) : st[r]) : -INFINITY;
             const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
             if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
                 float gm = fmaxf(mb, __shfl_xor(mb, 16));
@@ -1805,7 +1820,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 pr[r] = __builtin_amdgcn_exp2f(sc[r] - mref);
-                lrun += pr[r];
+                lrun += pr[r];                                   // the softmax denominator ignores dropout
+                if constexpr (DROP)
+                    pr[r] *= dropout_keep((uint32_t)B.xe[DROP ? r : 0] * (uint32_t)H + (uint32_t)t.head, drop_seed, drop_thr, drop_inv);
             }
             tile_axpy(pr, B.vr, acc);
         };
@@ -1833,11 +1850,12 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 // (scattered 8-byte stores here, contiguous reads there) cost this kernel a third of its time (126 against 85 us at
 // L = 4096, k = 32); letting the source side recompute p and ds (two more products there, delta (n, H) handed over)
 // measured slower than either on every graph tried.
-template <typename T, int H, int D, int HW, bool PIPE>
+template <typename T, int H, int D, int HW, bool PIPE, bool DROP, bool BIAS>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : 3))) void k_attn_bwd_dst_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
     const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds, float *__restrict__ ws_dq,
-    float scale, float scale_log2e) {
+    float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv, const float *__restrict__ bias,
+    float *__restrict__ ds_out) {
     constexpr int C = H * D;
     TileCtx t;
     if (!tile_begin<T, H, D, HW>(P, t)) return;
@@ -1866,11 +1884,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         float kr[16], va[16];
         float4 kc[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 g + r
         int pos[4], mk[4];
+        int xe[DROP || BIAS ? 4 : 1];
+        float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
         auto issue = [&](Blk &B, int b) {
+            if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -1884,6 +1905,10 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 B.kc[r] = *reinterpret_cast<const float4 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
                 B.pos[r] = p0 + TILE_R * b + 4 * g + r;            // (past the group's end the masks are empty)
             }
+            if constexpr (BIAS) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
+            }
         };
         auto compute = [&](const Blk &B) {
             const floatx4v st = tile_dot(B.kr, qb), dp = tile_dot(B.va, dob);
@@ -1891,9 +1916,16 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const bool has = (B.mk[r] >> c) & 1;
-                const float pe = has ? __builtin_amdgcn_exp2f(st[r] - lse_c) : 0.f;
-                ds[r] = pe * (dp[r] - delta) * scale;
-                if (has) pds[((size_t)B.pos[r] * H + t.head) * TILE_R + c] = make_float2(pe, ds[r]);
+                float pe = has ? __builtin_amdgcn_exp2f((BIAS ? fmaf(B.bz[BIAS ? r : 0], scale_log2e, st[r]) : st[r]) - lse_c) : 0.f;
+                float mt = 1.f;                                   // dropout multiplier of this pair (as in the forward)
+                if constexpr (DROP)
+                    mt = dropout_keep((uint32_t)B.xe[DROP ? r : 0] * (uint32_t)H + (uint32_t)t.head, drop_seed, drop_thr, drop_inv);
+                ds[r] = pe * (dp[r] * mt - delta) * scale;
+                pe *= mt;                                         // what multiplies v (forward) and dO (dV)
+                if (has) {
+                    pds[((size_t)B.pos[r] * H + t.head) * TILE_R + c] = make_float2(pe, ds[r]);
+                    if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
+                }
             }
             tile_axpy(ds, B.kc, acc);
         };
@@ -2016,10 +2048,11 @@ __device__ __forceinline__ void tile_load_row_bf16(const char *p, Bf8 (&out)[2])
     out[1].q = *reinterpret_cast<const uint4 *>(p + 16);
 }
 
-template <int H, int D, int HW, int WPE, bool PIPE>
-__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_fwd_tile_bf16(
+template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, bool BIAS>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP || BIAS ? WPE - 1 : WPE))) void k_attn_fwd_tile_bf16(
     bpt_plan P, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v, bf16_t *__restrict__ o,
-    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e) {
+    float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr,
+    uint32_t drop_seed, float drop_inv, const float *__restrict__ bias) {
     constexpr int RB = H * D * 2;                                 // bytes of a node row
     TileCtx t;
     if (!tile_begin<bf16_t, H, D, HW>(P, t)) return;
@@ -2038,11 +2071,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
         Bf8 kr[2];
         uint2 vr[4];
         int mk[4];
+        int xe[DROP || BIAS ? 4 : 1];
+        float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
         auto issue = [&](Blk &B, int b) {
+            if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -2051,12 +2087,16 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
             tile_load_row_bf16(kb + (size_t)((uint32_t)ea.x * (uint32_t)RB) + offr, B.kr);
 #pragma unroll
             for (int r = 0; r < 4; ++r) B.vr[r] = *reinterpret_cast<const uint2 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
+            if constexpr (BIAS) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
+            }
         };
         auto compute = [&](const Blk &B) {
             const floatx4v st = tile_dot_bf16(B.kr, qb);
             float sc[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sc[r] = ((B.mk[r] >> c) & 1) ? st[r] * scale_log2e : -INFINITY;
+            for (int r = 0; r < 4; ++r) sc[r] = ((B.mk[r] >> c) & 1) ? (BIAS ? st[r] + B.bz[BIAS ? r : 0] : st[r]) * scale_log2e : -INFINITY;
             const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
             if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
                 float gm = fmaxf(mb, __shfl_xor(mb, 16));
@@ -2076,7 +2116,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 pr[r] = __builtin_amdgcn_exp2f(sc[r] - mref);
-                lrun += pr[r];
+                lrun += pr[r];                                   // the softmax denominator ignores dropout
+                if constexpr (DROP)
+                    pr[r] *= dropout_keep((uint32_t)B.xe[DROP ? r : 0] * (uint32_t)H + (uint32_t)t.head, drop_seed, drop_thr, drop_inv);
             }
             Bf4 pa;
             pa.u[0] = pack_bf16(pr[0], pr[1]);
@@ -2099,11 +2141,12 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
     }
 }
 
-template <int H, int D, int HW, int WPE, bool PIPE>
-__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_bwd_dst_tile_bf16(
+template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, bool BIAS>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP || BIAS ? WPE - 1 : WPE))) void k_attn_bwd_dst_tile_bf16(
     bpt_plan P, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v, const bf16_t *__restrict__ o,
     const bf16_t *__restrict__ d_o, const float *__restrict__ lse, bf16_t *__restrict__ dq, uint32_t *__restrict__ pds,
-    float *__restrict__ ws_dq, float scale, float scale_log2e) {
+    float *__restrict__ ws_dq, float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv,
+    const float *__restrict__ bias, float *__restrict__ ds_out) {
     constexpr int RB = H * D * 2;
     TileCtx t;
     if (!tile_begin<bf16_t, H, D, HW>(P, t)) return;
@@ -2141,11 +2184,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
         Bf8 kr[2], va[2];
         uint2 kc[4];
         int mk[4], pos0;
+        int xe[DROP || BIAS ? 4 : 1];
+        float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
         auto issue = [&](Blk &B, int b) {
+            if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -2157,6 +2203,10 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
 #pragma unroll
             for (int r = 0; r < 4; ++r) B.kc[r] = *reinterpret_cast<const uint2 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
             B.pos0 = p0 + TILE_R * b + 4 * g;                     // (past the group's end the masks are empty)
+            if constexpr (BIAS) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
+            }
         };
         auto compute = [&](const Blk &B) {
             const floatx4v st = tile_dot_bf16(B.kr, qb), dp = tile_dot_bf16(B.va, dob);
@@ -2164,9 +2214,16 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const bool has = (B.mk[r] >> c) & 1;
-                const float pe = has ? __builtin_amdgcn_exp2f(st[r] * scale_log2e - lse_c) : 0.f;
-                ds[r] = pe * (dp[r] - delta) * scale;
-                if (has) pds[((size_t)(B.pos0 + r) * H + t.head) * TILE_R + c] = pack_bf16(pe, ds[r]);
+                float pe = has ? __builtin_amdgcn_exp2f((BIAS ? st[r] + B.bz[BIAS ? r : 0] : st[r]) * scale_log2e - lse_c) : 0.f;
+                float mt = 1.f;                                   // dropout multiplier of this pair (as in the forward)
+                if constexpr (DROP)
+                    mt = dropout_keep((uint32_t)B.xe[DROP ? r : 0] * (uint32_t)H + (uint32_t)t.head, drop_seed, drop_thr, drop_inv);
+                ds[r] = pe * (dp[r] * mt - delta) * scale;
+                pe *= mt;                                         // what multiplies v (forward) and dO (dV)
+                if (has) {
+                    pds[((size_t)(B.pos0 + r) * H + t.head) * TILE_R + c] = pack_bf16(pe, ds[r]);
+                    if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
+                }
             }
             Bf4 da;
             da.u[0] = pack_bf16(ds[0], ds[1]);
@@ -3097,22 +3154,35 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
         if constexpr (D == 64 && sizeof(T) == 4) {
-            if (has_tiles(P, H, D, sizeof(T)) && drop.thr == 0 && !bias) {
+            if (has_tiles(P, H, D, sizeof(T)) && ((drop.thr == 0 && !bias) || P->grp_eids)) {
                 constexpr int HW = H >= 4 ? 4 : H;          // heads per workgroup
-                if (tall_tiles(P, H))
-                    hipLaunchKernelGGL((k_attn_fwd_tile<T, H, D, HW, true>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), 0, s, *P,
-                                       (const T *)q, (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
-                else
-                    hipLaunchKernelGGL((k_attn_fwd_tile<T, H, D, HW, false>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), 0, s, *P,
-                                       (const T *)q, (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+#define LAUNCH_FWD_TILE(PI, DR, BI)                                                                                                  \
+    hipLaunchKernelGGL((k_attn_fwd_tile<T, H, D, HW, PI, DR, BI>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), 0, s, *P, (const T *)q, \
+                       (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv, bias)
+                switch ((drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0)) {
+                case 0: if (tall_tiles(P, H)) LAUNCH_FWD_TILE(true, false, false); else LAUNCH_FWD_TILE(false, false, false); break;
+                case 1: LAUNCH_FWD_TILE(false, true, false); break;
+                case 2: LAUNCH_FWD_TILE(false, false, true); break;
+                default: LAUNCH_FWD_TILE(false, true, true); break;
+                }
+#undef LAUNCH_FWD_TILE
                 goto launched;
             }
         }
         if constexpr (D == 64 && sizeof(T) == 2) {
-            if (has_tiles(P, H, D, sizeof(T)) && drop.thr == 0 && !bias) {
+            if (has_tiles(P, H, D, sizeof(T)) && ((drop.thr == 0 && !bias) || P->grp_eids)) {
                 constexpr int HW = H >= 4 ? 4 : H;
-                hipLaunchKernelGGL((k_attn_fwd_tile_bf16<H, D, HW, TILE_BF16_WPE, TILE_BF16_PIPE>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), 0, s, *P,
-                                   (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (bf16_t *)o, lse, ws_acc, ws_ml, scale * LOG2E);
+#define LAUNCH_FWD_TILE(DR, BI)                                                                                                          \
+    hipLaunchKernelGGL((k_attn_fwd_tile_bf16<H, D, HW, TILE_BF16_WPE, TILE_BF16_PIPE, DR, BI>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), \
+                       0, s, *P, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (bf16_t *)o, lse, ws_acc, ws_ml, scale * LOG2E,   \
+                       drop.thr, drop.seed, drop.inv, bias)
+                switch ((drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0)) {
+                case 0: LAUNCH_FWD_TILE(false, false); break;
+                case 1: LAUNCH_FWD_TILE(true, false); break;
+                case 2: LAUNCH_FWD_TILE(false, true); break;
+                default: LAUNCH_FWD_TILE(true, true); break;
+                }
+#undef LAUNCH_FWD_TILE
                 goto launched;
             }
         }
@@ -3170,19 +3240,22 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     float2 *pds = (float2 *)ws;                                  // row-group kernels: interleaved (p, ds)
     float *ws_rows = (float *)ws + pbytes / 4;
     if constexpr (D == 64 && sizeof(T) == 4) {
-        if (tiled_backward(Pin, Pout, H, D, sizeof(T)) && drop.thr == 0 && !bias) {
+        if (tiled_backward(Pin, Pout, H, D, sizeof(T)) && ((drop.thr == 0 && !bias) || Pin->grp_eids)) {
             constexpr int HW = H >= 4 ? 4 : H;
             float *ws_dk = ws_rows + (size_t)Pin->n_slots * H * D, *ws_dv = ws_dk + (size_t)Pout->n_slots * H * D;
             {
                 ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
-                if (tall_tiles(Pin, H))
-                    hipLaunchKernelGGL((k_attn_bwd_dst_tile<T, H, D, HW, true>), dim3(group_grid(Pin) * (H / HW)), dim3(HW * WAVE), 0, s, *Pin,
-                                       (const T *)q, (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows,
-                                       scale, scale * LOG2E);
-                else
-                    hipLaunchKernelGGL((k_attn_bwd_dst_tile<T, H, D, HW, false>), dim3(group_grid(Pin) * (H / HW)), dim3(HW * WAVE), 0, s, *Pin,
-                                       (const T *)q, (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows,
-                                       scale, scale * LOG2E);
+#define LAUNCH_DST_TILE(PI, DR, BI)                                                                                                    \
+    hipLaunchKernelGGL((k_attn_bwd_dst_tile<T, H, D, HW, PI, DR, BI>), dim3(group_grid(Pin) * (H / HW)), dim3(HW * WAVE), 0, s, *Pin,     \
+                       (const T *)q, (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale,         \
+                       scale * LOG2E, drop.thr, drop.seed, drop.inv, bias, ds_out)
+                switch ((drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0)) {
+                case 0: if (tall_tiles(Pin, H)) LAUNCH_DST_TILE(true, false, false); else LAUNCH_DST_TILE(false, false, false); break;
+                case 1: LAUNCH_DST_TILE(false, true, false); break;
+                case 2: LAUNCH_DST_TILE(false, false, true); break;
+                default: LAUNCH_DST_TILE(false, true, true); break;
+                }
+#undef LAUNCH_DST_TILE
             }
             int st = launch_status();
             if (st != BPT_OK) return st;
@@ -3204,14 +3277,23 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
         }
     }
     if constexpr (D == 64 && sizeof(T) == 2) {
-        if (tiled_backward(Pin, Pout, H, D, sizeof(T)) && drop.thr == 0 && !bias) {
+        if (tiled_backward(Pin, Pout, H, D, sizeof(T)) && ((drop.thr == 0 && !bias) || Pin->grp_eids)) {
             constexpr int HW = H >= 4 ? 4 : H;
             float *ws_dk = ws_rows + (size_t)Pin->n_slots * H * D, *ws_dv = ws_dk + (size_t)Pout->n_slots * H * D;
             {
                 ProfScope prof(BPT_KERNEL_ATTN_BWD_DST, s);
-                hipLaunchKernelGGL((k_attn_bwd_dst_tile_bf16<H, D, HW, TILE_BF16_WPE_DST, TILE_BF16_PIPE>), dim3(group_grid(Pin) * (H / HW)), dim3(HW * WAVE), 0, s,
-                                   *Pin, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)o, (const bf16_t *)d_o, lse,
-                                   (bf16_t *)dq, (uint32_t *)ws, ws_rows, scale, scale * LOG2E);
+#define LAUNCH_DST_TILE(DR, BI)                                                                                                          \
+    hipLaunchKernelGGL((k_attn_bwd_dst_tile_bf16<H, D, HW, TILE_BF16_WPE_DST, TILE_BF16_PIPE, DR, BI>), dim3(group_grid(Pin) * (H / HW)),   \
+                       dim3(HW * WAVE), 0, s, *Pin, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)o,             \
+                       (const bf16_t *)d_o, lse, (bf16_t *)dq, (uint32_t *)ws, ws_rows, scale, scale * LOG2E, drop.thr, drop.seed,          \
+                       drop.inv, bias, ds_out)
+                switch ((drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0)) {
+                case 0: LAUNCH_DST_TILE(false, false); break;
+                case 1: LAUNCH_DST_TILE(true, false); break;
+                case 2: LAUNCH_DST_TILE(false, true); break;
+                default: LAUNCH_DST_TILE(true, true); break;
+                }
+#undef LAUNCH_DST_TILE
             }
             int st = launch_status();
             if (st != BPT_OK) return st;
@@ -3508,8 +3590,9 @@ int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k,
     if (!q || !k || !v || !o || !lse) return BPT_ERR_NULL;
     if (!(dropout_p >= 0.f && dropout_p < 1.f)) return BPT_ERR_SIZE;
     const Dropout drop = make_dropout(dropout_p, dropout_seed);
-    // dropout and the score term exist in the row-group kernels only
-    if ((drop.thr != 0 || bias) && !has_groups(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
+    // dropout and the score term exist in the row-group and the tile kernels only
+    if ((drop.thr != 0 || bias) && !has_groups(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4) && !has_tiles(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4))
+        return BPT_ERR_UNSUPPORTED;
     if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(workspace))
         return BPT_ERR_UNSUPPORTED;
@@ -3546,7 +3629,9 @@ int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, co
     CHECK(check_shape(h, d, dtype));
     if (!(dropout_p >= 0.f && dropout_p < 1.f)) return BPT_ERR_SIZE;
     const Dropout drop = make_dropout(dropout_p, dropout_seed);
-    if ((drop.thr != 0 || bias) && !grouped_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
+    if ((drop.thr != 0 || bias) && !grouped_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4) &&
+        !tiled_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4))
+        return BPT_ERR_UNSUPPORTED;
     if ((bias != nullptr) != (ds_out != nullptr)) return BPT_ERR_NULL;       // the score term and its gradient go together
     if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
     // (the two sides may have different row counts: attention to a memory of another length, attention.py:144-168)

@@ -508,9 +508,10 @@ TILE_SEG_LEN = None        # testing / measurement hook: edges per work item of 
 def _tiles(q, h, d, plan, dropout_p, bias, cfg):
     """Whether the fused forward runs on dense tiles (groups of 16 rows, one wavefront per head, every block of 16
     entries a dense 16 x 16 matrix product with the missing pairs masked): float32 or bfloat16 rows of 64 columns per
-    head, no dropout or score term, and the library's choice of rows per group not overridden."""
+    head (dropout and the score term included: their variants read the edge id of every pair), and the library's choice of
+    rows per group not overridden."""
     return (cfg.use_tiles and cfg.group_rows is None and (q.dtype == torch.float32 or (TILE_BF16 and q.dtype == torch.bfloat16))
-            and d == 64 and h <= 16 and dropout_p == 0.0 and bias is None)
+            and d == 64 and h <= 16)
 
 
 def _tiles_backward(plan, dtype):

@@ -410,7 +410,8 @@ def test_zero_degree_rows_are_zero(ops):
 # dropout on the attention probabilities inside the fused kernels (modules/attention.py:73)
 # --------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,hd", [(torch.float32, (8, 64)), (torch.float32, (16, 64)), (torch.bfloat16, (8, 64))])
-@pytest.mark.parametrize("gname,rows", [("bpt512_k4", 4), ("bpt512_k4", 8), ("multigraph", 4), ("fc_w100", 8)])
+@pytest.mark.parametrize("gname,rows", [("bpt512_k4", 4), ("bpt512_k4", 8), ("multigraph", 4), ("fc_w100", 8),
+                                        ("bpt512_k4", None), ("multigraph", None)])          # None: the library's choice (tiles of 16 rows)
 def test_fused_attention_dropout_matches_oracle_with_the_same_mask(ops, gname, rows, dtype, hd):
     from oracle import torch_ops
     graphop, op = ops
@@ -451,7 +452,7 @@ def test_fused_attention_dropout_matches_oracle_with_the_same_mask(ops, gname, r
 @pytest.mark.parametrize("p", [0.0, 0.25])
 @pytest.mark.parametrize("dtype,hd", [(torch.float32, (8, 64)), (torch.float32, (16, 64)), (torch.float32, (4, 64)), (torch.bfloat16, (8, 64))])
 @pytest.mark.parametrize("gname,rows", [("bpt512_k4", 4), ("bpt512_k4", 8), ("bpt300_causal_k2", None), ("multigraph", 4), ("fc_w100", 8),
-                                        ("bpt256_k24", 8)])
+                                        ("bpt256_k24", 8), ("multigraph", None), ("fc_w100", None)])    # None: the library's choice (tiles of 16 rows)
 def test_fused_attention_with_rel_pos_matches_oracle(ops, gname, rows, dtype, hd, p):
     from oracle import torch_ops
     graphop, op = ops

@@ -136,6 +136,46 @@ def test_tile_kernels_in_bfloat16_match_the_oracle(gname, seg, heads):
     check(qd.grad, rdq, BF16_TOL, "dq"); check(kd.grad, rdk, BF16_TOL, "dk"); check(vd.grad, rdv, BF16_TOL, "dv")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("gname,seg", [("multigraph", 64), ("bpt2048_causal", 64), ("window100", 256)])
+def test_tile_kernels_with_dropout_and_score_term(gname, seg, dtype):
+    """The DROP / BIAS variants of the tile kernels (forward and destination-side backward read the edge id of every pair):
+    dropout 0.25 with the mask attention_dropout_mask reproduces, and a rel_pos table of 23 types, together, against the
+    float64 oracle given the same mask; float32 rtol 1e-5 / atol 1e-5 (gradients rtol 1e-4), bfloat16 rtol 2e-2 / atol 2e-2."""
+    from oracle import torch_ops
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd import op, graphop
+    src, dst, n_k, n_q = graphs(gname)
+    csr = gb.get_csrs_bipartite(src, dst, n_k, n_q)
+    out_csr, in_csr, ROW, IR, COL, IC = csr
+    args = tuple(x.to(DEV) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
+    h, n_types, p, seed = 8, 23, 0.25, 424242
+    gen = torch.Generator().manual_seed(23)
+    q, do = ((torch.randn(n_q, h, 64, generator=gen) / 8).to(dtype) for _ in range(2))
+    k, v = ((torch.randn(n_k, h, 64, generator=gen) / 8).to(dtype) for _ in range(2))
+    table = (torch.randn(n_types, 64, generator=gen) / 8).to(dtype)
+    etype = torch.from_numpy(np.random.default_rng(24).integers(0, n_types, len(src))).to(DEV)
+    qd, kd, vd, td = (x.to(DEV).requires_grad_(True) for x in (q, k, v, table))
+    with forced_tiles(seg):
+        mask = graphop.attention_dropout_mask(*args[4:], qd, kd, p, seed)
+        o = op.bpt_attention(*args, qd, kd, vd, fused=True, dropout_p=p, seed=seed, rel_table=td, etype=etype)
+        o.backward(do.to(DEV))
+        from bpt_amd.plan import plan_cache
+        assert [pl for pl, _ in plan_cache._d.values() if any(key[0] == 16 for key in pl._groups)], "the tile kernels did not run"
+    et = etype.cpu()
+    ro, rdq, rdk, rdv, rdak = torch_ops.attention_fwd_bwd(torch.from_numpy(src), torch.from_numpy(dst), f64(q), f64(k), f64(v), f64(do),
+                                                          ak=f64(table)[et], drop=mask.double())
+    rdt = torch.zeros(n_types, 64, dtype=torch.float64).index_add_(0, et, rdak)
+    tol, gtol = (TOL, GTOL) if dtype == torch.float32 else (BF16_TOL, BF16_TOL)
+    check(o, ro, tol, "o")
+    check(qd.grad, rdq, gtol, "dq"); check(kd.grad, rdk, gtol, "dk"); check(vd.grad, rdv, gtol, "dv")
+    # a table row is a raw sum over all edges of its type and all heads (h * E / n_types products): atol grows with
+    # its length as in tests/test_gpu_parity.py::close
+    terms = h * len(src) / n_types
+    err = (f64(td.grad) - rdt).abs().numpy()
+    assert np.all(err <= gtol["atol"] * max(1.0, terms / 64.0) + gtol["rtol"] * rdt.abs().numpy()), err.max()
+
+
 def test_tiles_agree_with_the_row_group_kernels_on_the_headline_graph():
     """L = 8192, k = 4, causal, 8 x 64: tile forward + tile backward against the row-group kernels (themselves checked
     against the oracle in test_headline_graph_full_parity) and against the oracle's forward."""
