@@ -2002,7 +2002,10 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 // Probabilities and ds are rounded to bfloat16 where they enter a product (the softmax denominator is summed unrounded);
 // the scratch between the two backward kernels holds (p, ds) as two bfloat16 in 4 bytes, in the destination side's layout.
 // The two-stage register pipeline of tile_walk does not pay here: at six wavefronts per SIMD it spills (2.4 x slower),
-// at four it measured 5 to 10 % slower on the sparse graphs and level on the window graph.
+// at four it measured 5 to 10 % slower on the sparse graphs and level on the window graph.  Tiles of 32 rows (two member
+// blocks per wavefront on the same loaded rows, three or four wavefronts per SIMD) did not pay either: the entry lists
+// shrink by a third on the destination side but only by an eighth on the source side (L = 8192, k = 4: 67 k -> 46 k and
+// 71 k -> 62 k entries), and the step went from 0.113 to 0.117 ms (32-graph batch 0.177 -> 0.205, window 128 level).
 constexpr bool TILE_BF16_PIPE = false;
 constexpr int TILE_BF16_WPE = 6, TILE_BF16_WPE_DST = 5;     // wavefronts per SIMD the bfloat16 tile kernels are compiled for
 typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
