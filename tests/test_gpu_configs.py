@@ -3,9 +3,10 @@ float64 CPU oracle on the same seeded inputs (q, k, v, grad-out = N(0,1) / sqrt(
 2345, all nodes), with the stated tolerances applied as they stand: float32 outputs rtol 1e-5 / atol 1e-5, gradients
 rtol 1e-4 (atol 1e-5); bfloat16 rtol 2e-2 (atol 2e-2).
 
-  configuration 2: 32 causal graphs, lengths uniform in [64, 1024] (seed 2345), k = 4, merged block-diagonally
+  configuration 2: 32 causal graphs, lengths uniform in [64, 1024] (seed 2345), k = 4, merged block-diagonally (float32, bfloat16)
   configuration 3 in bfloat16: L = 8192, k = 4, causal (float32: tests/test_gpu_parity.py::test_headline_graph_full_parity)
-  configuration 4: L = 4096, causal, k in {1, 2, 4, 8, 16, 32}, and the window-128 graph (FullyConnected)
+  configuration 4: L = 4096, causal, k in {1, 2, 4, 8, 16, 32}, and the window-128 graph (FullyConnected); k = 32 and the
+                   window graph also in bfloat16
 """
 import numpy as np
 import pytest
@@ -63,6 +64,15 @@ def test_cfg2_batch_of_32_graphs_fp32():
     run_layer(src, dst, n, 8, 64, torch.float32)
 
 
+def test_cfg2_batch_of_32_graphs_bf16():
+    from bpt_amd import graphbuilder as gb
+    lengths = np.random.default_rng(2345).integers(64, 1025, 32)
+    cache = {}
+    graphs = [cache.setdefault(int(L), gb.BinaryPartition(int(L), True, 4, 10)) for L in lengths]
+    src, dst, _, _, n = gb.merge_graphs(graphs)
+    run_layer(src, dst, n, 8, 64, torch.bfloat16)
+
+
 def test_cfg3_bf16_full_size():
     from bpt_amd import graphbuilder as gb
     g = gb.BinaryPartition(8192, True, 4, 10)
@@ -86,3 +96,12 @@ def test_cfg4_window_128_fp32():
     src, dst, _ = g.get_edges()
     assert (g.number_of_nodes, len(src)) == (4097, 524224)
     run_layer(src, dst, g.number_of_nodes, 8, 64, torch.float32)
+
+
+@pytest.mark.parametrize("which", ["k32", "window128"])
+def test_cfg4_dense_graphs_bf16(which):
+    """The two densest graphs of configuration 4 in bfloat16 (tile kernels on the bfloat16 matrix instructions)."""
+    from bpt_amd import graphbuilder as gb
+    g = gb.BinaryPartition(4096, True, 32, 10) if which == "k32" else gb.FullyConnected(4096, True, 128)
+    src, dst, _ = g.get_edges()
+    run_layer(src, dst, g.number_of_nodes, 8, 64, torch.bfloat16)
