@@ -370,7 +370,7 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     if not _attention_groups(plan, dropout_p, bias, q, k, cfg):
         ref = plan.ref
     elif _tiles(q, h, d, plan, dropout_p, bias, cfg):
-        plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=_tile_seg_len(plan))
+        plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=_tile_seg_len(plan), prefer_device=True)
         ref = ctypes.byref(plan.ensure_groups(TILE_ROWS)["struct"])
     else:
         ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, cfg))["struct"])
@@ -416,8 +416,8 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     if _attention_groups(plan_in, dropout_p, bias, q, k, cfg) and plan_in.covers_all_edges and plan_out.covers_all_edges:
         if _tiles(q, h, d, plan_in, dropout_p, bias, cfg) and _tiles_backward(plan_in, q.dtype):
             seg = _tile_seg_len(plan_in)
-            plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg)
-            plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg)
+            plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg, prefer_device=True)
+            plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg, prefer_device=True)
             # the destination side writes (p, ds) in its own layout; the source side finds them through its pair mapping
             in_ref = ctypes.byref(plan_in.ensure_groups(TILE_ROWS)["struct"])
             out_ref = ctypes.byref(plan_out.linked_to(plan_in, TILE_ROWS, partner_order=None))

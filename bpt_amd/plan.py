@@ -478,14 +478,17 @@ class PlanCache:
                 total -= p.device_bytes()
 
     @staticmethod
-    def _key(tensors, n_rows, n_index, seg_len):
+    def _key(tensors, n_rows, n_index, seg_len, on_device):
         return tuple((t.data_ptr(), t.numel(), t._version, str(t.device)) if t is not None else None
-                     for t in tensors) + (n_rows, n_index, seg_len, DEVICE_BUILD)
+                     for t in tensors) + (n_rows, n_index, seg_len, on_device)
 
-    def get(self, row, indptr, eid, indices, n_rows=None, n_index_nodes=None, seg_len=DEFAULT_SEG_LEN):
-        """n_rows None: as many rows as `row` mentions (ops that only produce edge outputs)."""
+    def get(self, row, indptr, eid, indices, n_rows=None, n_index_nodes=None, seg_len=DEFAULT_SEG_LEN, prefer_device=False):
+        """n_rows None: as many rows as `row` mentions (ops that only produce edge outputs).  prefer_device: build on the GPU
+        whatever the graph's size, unless set_device_build() fixed the place (the tile kernels ask for this: the GPU
+        builder's groups of 16 run them as fast or faster on every graph measured)."""
         tensors = (row, indptr, eid, indices)
-        key = self._key(tensors, n_rows, n_index_nodes, seg_len)
+        on_device = _build_on_device(eid, n_rows) or bool(prefer_device and DEVICE_BUILD is None and eid.is_cuda and n_rows is not None)
+        key = self._key(tensors, n_rows, n_index_nodes, seg_len, on_device)
         with self._lock:
             hit = self._d.get(key)
             if hit is not None:
@@ -495,7 +498,7 @@ class PlanCache:
                     self._evict()                   # row groups and pair mappings are added to plans after insertion
                 return hit[0]
         self.misses += 1
-        if _build_on_device(eid, n_rows):
+        if on_device:
             nr = n_rows if n_rows is not None else (int(row[-1]) + 1 if row.numel() else 0)
             ni = n_index_nodes if n_index_nodes is not None else nr
             plan = DevicePlan(row, indptr, eid, indices, nr, ni, eid.device, seg_len)
