@@ -1,0 +1,50 @@
+"""The fused step under HIP graph capture: a caller that records forward + backward once and replays it (a training
+loop with a fixed graph) must get, on every replay, exactly what the eager launches give.  The graph is replayed
+several times with eager work of the same library and synchronisations in between, inputs are changed in place
+between replays, and every replay is compared bit for bit with an eager step on the same inputs.  float32 runs the
+tile forward with the row-group or tile backward, bfloat16 the tile kernels throughout; one case uses dropout (a
+function of seed, edge id and head: the same under replay)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("dtype,dropout", [(torch.float32, 0.0), (torch.bfloat16, 0.0), (torch.float32, 0.2)])
+@pytest.mark.parametrize("L", [1024, 8192])          # tile backward (fewer than 12288 rows) and, in float32, row-group backward
+def test_graph_replay_equals_eager(L, dtype, dropout):
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd import graphop
+    g = gb.BinaryPartition(L, True, 4, 10)
+    src, dst, _ = g.get_edges()
+    n = g.number_of_nodes
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, n)
+    args = tuple(x.to(DEV) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
+    gen = torch.Generator().manual_seed(77)
+    q, k, v, do = ((torch.randn(n, 8, 64, generator=gen) / 8).to(dtype).to(DEV) for _ in range(4))
+    seed = 1234
+
+    def step():
+        o, lse = graphop.attention_forward(*args[4:], q, k, v, dropout_p=dropout, seed=seed)
+        return (o, lse) + tuple(graphop.attention_backward(*args, q, k, v, o, lse, do, dropout_p=dropout, seed=seed))
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):                      # plans are built and cached before the capture
+        for _ in range(2):
+            step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gout = step()
+    for rep in range(4):
+        if rep:                                        # new inputs, written in place: the graph reads the same buffers
+            for t in (q, k, v, do):
+                t.mul_(-0.5).add_(0.01 * rep)
+        want = step()                                  # eager work of the same library between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b, name in zip(gout, want, ("o", "lse", "dq", "dk", "dv")):
+            assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager result"
