@@ -219,9 +219,14 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t) / steps
 
-    t_eager = timed(step, args.steps, args.warmup)
+    # The timed region is exactly --steps steps between two synchronisations.  It is run three times and the shortest
+    # run is reported (all three are in the JSON line): the host of a shared box stalls now and then for tens of
+    # milliseconds (measured: single calls of 40 ms inside loops whose other calls take 0.05 ms), which a loop of 40 ms
+    # cannot absorb.
+    runs_eager = [timed(step, args.steps, args.warmup if i == 0 else 2) for i in range(3)]
+    t_eager = min(runs_eager)
     t_step, mode = t_eager, "eager"
-    t_graph_replay = None
+    t_graph_replay, runs_graph = None, []
     if not args.no_graph:
         try:
             side = torch.cuda.Stream()
@@ -236,7 +241,8 @@ def main():
             g.replay(); torch.cuda.synchronize()
             same = all(torch.equal(a, b) for a, b in zip(gout, ref))
             if same:
-                t_graph_replay = timed(g.replay, args.steps, args.warmup)
+                runs_graph = [timed(g.replay, args.steps, args.warmup if i == 0 else 2) for i in range(3)]
+                t_graph_replay = min(runs_graph)
                 same = all(torch.equal(a, b) for a, b in zip(gout, ref))
             if same and t_graph_replay < t_step:
                 t_step, mode = t_graph_replay, "hipgraph-replay"
@@ -330,7 +336,7 @@ def main():
             x.backward(gh)
             return x
 
-        t_stack = timed(stack_step, 5, 2)
+        t_stack = min(timed(stack_step, 5, 2) for _ in range(3))
         block = {"layers": args.block_layers, "d_model": dm, "d_ff": 4 * dm, "ms_per_layer_fwd_bwd": round(t_stack / args.block_layers * 1e3, 4),
                  "attention_ms_per_layer": round(t_step * 1e3, 4), "attention_share": round(t_step * args.block_layers / t_stack, 3)}
         log(f"block stack: {block}")
@@ -357,6 +363,8 @@ def main():
                           "measured_copy_GBps": round(copy_gbs, 1), "frac_of_measured_copy": round(step_gbs / copy_gbs, 4)},
         "ms_per_step_eager": t_eager * 1e3,
         "ms_per_step_graph": None if t_graph_replay is None else t_graph_replay * 1e3,
+        "timed_runs_ms_per_step": {"eager": [round(t * 1e3, 5) for t in runs_eager], "graph": [round(t * 1e3, 5) for t in runs_graph],
+                                   "reported": "shortest of three runs of --steps steps each"},
         "kernel_ms": {k_: round(v_, 5) for k_, v_ in kernels.items()},
     }
     if plan_build is not None:

@@ -48,3 +48,39 @@ def test_graph_replay_equals_eager(L, dtype, dropout):
         torch.cuda.synchronize()
         for a, b, name in zip(gout, want, ("o", "lse", "dq", "dk", "dv")):
             assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager result"
+
+
+def test_kept_workspaces_give_the_same_results_and_can_be_released():
+    """Ops keep one workspace per device and stream and reuse it from call to call: results equal those with a fresh
+    allocation per call, two different ops in a row do not disturb each other, and release_workspaces() drops the buffers."""
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd import graphop
+    g = gb.BinaryPartition(2048, False, 4, 10)            # non-causal: rows of 2048 edges, split rows on both sides
+    src, dst, _ = g.get_edges()
+    n = g.number_of_nodes
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, n)
+    args = tuple(x.to(DEV) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
+    gen = torch.Generator().manual_seed(5)
+    q, k, v, do = ((torch.randn(n, 8, 64, generator=gen) / 8).to(DEV) for _ in range(4))
+    w = torch.randn(len(src), 8, generator=gen).to(DEV)
+
+    def run():
+        o, lse = graphop.attention_forward(*args[4:], q, k, v)
+        y = graphop.vector_spmm_forward(*args[4:], w, v)                       # another op between forward and backward
+        return (o, lse, y) + tuple(graphop.attention_backward(*args, q, k, v, o, lse, do))
+
+    graphop.release_workspaces()
+    assert not graphop._SCRATCH
+    kept = run()
+    assert len(graphop._SCRATCH) == 1
+    again = run()
+    old, graphop.KEEP_WORKSPACES = graphop.KEEP_WORKSPACES, False
+    try:
+        fresh = run()
+    finally:
+        graphop.KEEP_WORKSPACES = old
+    torch.cuda.synchronize()
+    for a, b, c in zip(kept, again, fresh):
+        assert torch.equal(a, b) and torch.equal(a, c)
+    graphop.release_workspaces()
+    assert not graphop._SCRATCH
