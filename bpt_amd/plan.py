@@ -225,7 +225,15 @@ class Plan:
         position entry' * R + member' of the same edge in the groups of `plan_src` (the plan of the other CSR side of the
         same graph, groups built with `partner_order`).  The row-group kernels link the destination side to the source
         side, the tile kernels the source side to the destination side."""
-        mine, theirs = self.ensure_groups(R, order), plan_src.ensure_groups(R, partner_order)
+        o_mine, o_theirs = (GROUP_ORDER if order is None else order), (GROUP_ORDER if partner_order is None else partner_order)
+        if (R, o_mine) not in self._groups and (R, o_theirs) not in plan_src._groups and plan_src is not self:
+            # both sides still to be grouped: the partner's groups are built on a second thread meanwhile (the builder
+            # is a plain C function, called with the interpreter lock released)
+            other = _group_pool().submit(plan_src.ensure_groups, R, partner_order)
+            mine = self.ensure_groups(R, order)
+            theirs = other.result()
+        else:
+            mine, theirs = self.ensure_groups(R, order), plan_src.ensure_groups(R, partner_order)
         key = (id(plan_src), R, order, partner_order)
         with self._lock:
             hit = self._links.get(key)
@@ -238,6 +246,17 @@ class Plan:
                 hit = (st, pairs, plan_src)          # keeps the mapping and the partner alive
                 self._links[key] = hit
         return hit[0]
+
+
+_GROUP_POOL = None
+
+
+def _group_pool():
+    global _GROUP_POOL
+    if _GROUP_POOL is None:
+        import concurrent.futures
+        _GROUP_POOL = concurrent.futures.ThreadPoolExecutor(max_workers=1, thread_name_prefix="bpt-groups")
+    return _GROUP_POOL
 
 
 def set_device_build(on):
