@@ -1638,16 +1638,19 @@ __device__ __forceinline__ bool tile_begin(const bpt_plan &P, TileCtx &t) {
 // The entry list of a group is staged, TILE_CHUNK entries at a time, in a wavefront-private piece of LDS as (neighbour,
 // mask) pairs: every lane needs five of them per block (its A-operand row and the four rows / masks of its lane
 // group), which would otherwise be five dependent global loads in front of every block's row loads.
-__device__ __forceinline__ void tile_stage_entries(const bpt_plan &P, int2 *lds, int p0, int cnt, int lane) {
+__device__ __forceinline__ void tile_stage_entries(const bpt_plan &P, int2 *lds, int p0, int cnt, int lane, int *first = nullptr) {
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
 #pragma unroll
     for (int u = 0; u < TILE_CHUNK / WAVE; ++u) {
         const int e = u * WAVE + lane;
         const int4 x = entries[p0 + min(e, cnt - 1)];           // past the end: the last entry with an empty mask
         lds[e] = make_int2(x.x, e < cnt ? x.y : 0);
+        if (first) first[e] = x.z;                              // number of the entry's first pair (members follow in ascending order)
     }
     wave_lds_fence();
 }
+// number of the pair (entry, member c) among the plan's pairs: the entry's first pair + the members before c in its mask
+__device__ __forceinline__ int tile_pair_number(int first, int mask, int c) { return first + __popc((uint32_t)mask & ((1u << c) - 1u)); }
 
 // this lane's 16 columns of a node row (bytes offa + 64 t), as the A or B operand of a product over columns
 __device__ __forceinline__ void tile_load16(const char *row, float (&out)[16]) {
@@ -1844,12 +1847,13 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 
 // Backward on tiles, destination side: per block the scores and dO . v of all 16 x 16 pairs (two products over the
 // columns), p = 2^(s - lse), ds = p (dO . v - delta) scale, dq += ds K (third product; K is read a second time in the
-// column layout, which the L1 serves).  (p, ds) of the pairs that exist go to a scratch in THIS side's layout,
-// pds[(u * H + head) * 16 + m] for entry u and member m: the 16 lanes of a lane group write 128 contiguous bytes.  The
-// source side looks its pairs up there through its pair mapping (grp_pairs).  Writing in the source side's layout instead
-// (scattered 8-byte stores here, contiguous reads there) cost this kernel a third of its time (126 against 85 us at
-// L = 4096, k = 32); letting the source side recompute p and ds (two more products there, delta (n, H) handed over)
-// measured slower than either on every graph tried.
+// column layout, which the L1 serves).  (p, ds) of the pairs that exist go to a scratch in THIS side's order, compact:
+// pds[head * n_edges + t] for the pair number t of (entry, member) = the entry's first pair + the rank of the member in
+// its mask, so the lanes of an entry write one contiguous run and the runs of consecutive entries follow each other.  The
+// source side looks its pairs up there through its pair mapping (grp_pairs = this side's pair numbers).  Writing in the
+// source side's layout instead (scattered 8-byte stores here, contiguous reads there) cost this kernel a third of its
+// time (126 against 85 us at L = 4096, k = 32); letting the source side recompute p and ds (two more products there,
+// delta (n, H) handed over) measured slower than either on every graph tried.
 template <typename T, int H, int D, int HW, bool PIPE, bool DROP, bool BIAS>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : 3))) void k_attn_bwd_dst_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
@@ -1860,10 +1864,13 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     TileCtx t;
     if (!tile_begin<T, H, D, HW>(P, t)) return;
     __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    __shared__ int fst_lds[HW][TILE_CHUNK];
     int2 *ent = ent_lds[t.wv];
+    int *fst = fst_lds[t.wv];
     const int c = t.c, g = t.g;
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
     const size_t mrow = (size_t)max(t.member.x, 0) * (C * sizeof(T)) + t.offa;
+    float2 *const pds_h = pds + (size_t)t.head * (size_t)P.n_edges;     // this head's part of the scratch
     float qb[16], dob[16], delta, lse_c;
     {
         float ob[16];
@@ -1889,22 +1896,23 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
-        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
             B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+            B.pos[0] = tile_pair_number(f4.x, B.mk[0], c); B.pos[1] = tile_pair_number(f4.y, B.mk[1], c);
+            B.pos[2] = tile_pair_number(f4.z, B.mk[2], c); B.pos[3] = tile_pair_number(f4.w, B.mk[3], c);
             const size_t arow = (size_t)((uint32_t)ea.x * (uint32_t)(C * sizeof(T))) + t.offa;
             tile_load16(kb + arow, B.kr);
             tile_load16(vb + arow, B.va);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
+            for (int r = 0; r < 4; ++r)
                 B.kc[r] = *reinterpret_cast<const float4 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
-                B.pos[r] = p0 + TILE_R * b + 4 * g + r;            // (past the group's end the masks are empty)
-            }
             if constexpr (BIAS) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
@@ -1923,7 +1931,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 ds[r] = pe * (dp[r] * mt - delta) * scale;
                 pe *= mt;                                         // what multiplies v (forward) and dO (dV)
                 if (has) {
-                    pds[((size_t)B.pos[r] * H + t.head) * TILE_R + c] = make_float2(pe, ds[r]);
+                    pds_h[B.pos[r]] = make_float2(pe, ds[r]);
                     if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
                 }
             }
@@ -1937,7 +1945,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 
 // Backward on tiles, source side (groups of the out-CSR plan: members = source rows, entries = destinations):
 // dk += ds^T q, dv += p^T dO with (p, ds) of every pair fetched from the scratch the destination side filled, at the
-// position u' * 16 + m' that this plan's grp_pairs gives for (entry, member).
+// destination side's pair number that this plan's grp_pairs gives for (entry, member).
 template <typename T, int H, int D, int HW, bool PIPE>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 3 : 4))) void k_attn_bwd_src_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ d_o, const float2 *__restrict__ pds, T *__restrict__ dk, T *__restrict__ dv,
@@ -1949,6 +1957,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     int2 *ent = ent_lds[t.wv];
     const int c = t.c, g = t.g;
     const char *qb = reinterpret_cast<const char *>(q), *db = reinterpret_cast<const char *>(d_o);
+    const float2 *const pds_h = pds + (size_t)t.head * (size_t)P.n_edges;
     floatx4v ak[4], av[4];
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) { ak[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; av[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; }
@@ -1972,7 +1981,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 B.dr[r] = *reinterpret_cast<const float4 *>(db + off);
                 // (positions past the group's end are read at its last entry: their masks are empty)
                 const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
-                B.w[r] = pds[((size_t)(pos >> 4) * H + t.head) * TILE_R + (pos & 15)];
+                B.w[r] = pds_h[pos];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -2000,7 +2009,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 //   stands for column 16 g + 8 t + j in both operands) and columns 4 c .. 4 c + 3 of the rows of entries 4 g + r (8 bytes;
 //   the B operand of output columns {4 c + nb} takes element nb of each of the four, packed by byte permutes).
 // Probabilities and ds are rounded to bfloat16 where they enter a product (the softmax denominator is summed unrounded);
-// the scratch between the two backward kernels holds (p, ds) as two bfloat16 in 4 bytes, in the destination side's layout.
+// the scratch between the two backward kernels holds (p, ds) as two bfloat16 in 4 bytes, by head and destination-side pair number.
 // The two-stage register pipeline of tile_walk does not pay here: at six wavefronts per SIMD it spills (2.4 x slower),
 // at four it measured 5 to 10 % slower on the sparse graphs and level on the window graph.  Tiles of 32 rows (two member
 // blocks per wavefront on the same loaded rows, three or four wavefronts per SIMD) did not pay either: the entry lists
@@ -2154,11 +2163,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     TileCtx t;
     if (!tile_begin<bf16_t, H, D, HW>(P, t)) return;
     __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    __shared__ int fst_lds[HW][TILE_CHUNK];
     int2 *ent = ent_lds[t.wv];
+    int *fst = fst_lds[t.wv];
     const int c = t.c, g = t.g;
     const uint32_t offr = (uint32_t)((t.head * D + 16 * g) * 2), offc = (uint32_t)((t.head * D + 4 * c) * 2);
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
     const size_t mrow = (size_t)max(t.member.x, 0) * RB + offr;
+    uint32_t *const pds_h = pds + (size_t)t.head * (size_t)P.n_edges;     // this head's part of the scratch
     Bf8 qb[2], dob[2];
     float delta, lse_c;
     {
@@ -2186,26 +2198,28 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     struct Blk {
         Bf8 kr[2], va[2];
         uint2 kc[4];
-        int mk[4], pos0;
+        int mk[4], pos[4];
         int xe[DROP || BIAS ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
-        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
             B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+            B.pos[0] = tile_pair_number(f4.x, B.mk[0], c); B.pos[1] = tile_pair_number(f4.y, B.mk[1], c);
+            B.pos[2] = tile_pair_number(f4.z, B.mk[2], c); B.pos[3] = tile_pair_number(f4.w, B.mk[3], c);
             const size_t arow = (size_t)((uint32_t)ea.x * (uint32_t)RB) + offr;
             tile_load_row_bf16(kb + arow, B.kr);
             tile_load_row_bf16(vb + arow, B.va);
 #pragma unroll
             for (int r = 0; r < 4; ++r) B.kc[r] = *reinterpret_cast<const uint2 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
-            B.pos0 = p0 + TILE_R * b + 4 * g;                     // (past the group's end the masks are empty)
             if constexpr (BIAS) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
@@ -2224,7 +2238,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
                 ds[r] = pe * (dp[r] * mt - delta) * scale;
                 pe *= mt;                                         // what multiplies v (forward) and dO (dV)
                 if (has) {
-                    pds[((size_t)(B.pos0 + r) * H + t.head) * TILE_R + c] = pack_bf16(pe, ds[r]);
+                    pds_h[B.pos[r]] = pack_bf16(pe, ds[r]);
                     if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
                 }
             }
@@ -2251,6 +2265,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
     const int c = t.c, g = t.g;
     const uint32_t offc = (uint32_t)((t.head * D + 4 * c) * 2);
     const char *qb = reinterpret_cast<const char *>(q), *db = reinterpret_cast<const char *>(d_o);
+    const uint32_t *const pds_h = pds + (size_t)t.head * (size_t)P.n_edges;
     floatx4v ak[4], av[4];
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) { ak[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; av[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; }
@@ -2274,7 +2289,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
                 B.dr[r] = *reinterpret_cast<const uint2 *>(db + off);
                 // (positions past the group's end are read at its last entry: their masks are empty)
                 const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
-                B.w[r] = pds[((size_t)(pos >> 4) * H + t.head) * TILE_R + (pos & 15)];
+                B.w[r] = pds_h[pos];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -3132,19 +3147,16 @@ inline bool grouped_backward(const bpt_plan *Pin, const bpt_plan *Pout, int h, i
     return has_groups(Pin, h, d, elem) && has_groups(Pout, h, d, elem) && Pin->grp_R == Pout->grp_R && Pin->grp_pairs;
 }
 
-// float2 (p, ds) scratch of the fused backward: one per (entry, member) of the source-side groups (plus the
-// look-ahead padding), or one per edge for the per-row kernels
+// the tile kernels run the backward when both sides carry tiles and the source side the destination side's pair numbers
 inline bool tiled_backward(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {
-    return has_tiles(Pin, h, d, elem) && has_tiles(Pout, h, d, elem) && Pout->grp_pairs &&
-           fits32((Pin->n_grp_entries + GRP_PAD_ENTRIES) * TILE_R, (int64_t)h * 8);
+    return has_tiles(Pin, h, d, elem) && has_tiles(Pout, h, d, elem) && Pout->grp_pairs;
 }
 
 // float2 (p, ds) scratch of the fused backward: one per (entry, member) of the source-side groups (plus the
-// look-ahead padding), or one per edge for the per-row kernels
+// look-ahead padding) for the row-group kernels, one per edge for the per-row and the tile kernels
 inline int64_t pds_bytes(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d, size_t elem) {
     int64_t n = Pin->n_edges;
     if (Pout && grouped_backward(Pin, Pout, h, d, elem)) n = std::max(n, (Pout->n_grp_entries + GRP_PAD_ENTRIES) * Pout->grp_R);
-    if (Pout && tiled_backward(Pin, Pout, h, d, elem)) n = std::max(n, (Pin->n_grp_entries + GRP_PAD_ENTRIES) * Pin->grp_R);
     return 2 * round16(n * h * 4);
 }
 

@@ -447,9 +447,9 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
             seg = _tile_seg_len(plan_in)
             plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg, prefer_device=True)
             plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg, prefer_device=True)
-            # the destination side writes (p, ds) in its own layout; the source side finds them through its pair mapping
+            # the destination side writes (p, ds) by its own pair numbers; the source side finds them through its pair mapping
             in_ref = ctypes.byref(plan_in.ensure_groups(TILE_ROWS)["struct"])
-            out_ref = ctypes.byref(plan_out.linked_to(plan_in, TILE_ROWS, partner_order=None))
+            out_ref = ctypes.byref(plan_out.linked_to(plan_in, TILE_ROWS, partner_order=None, pair_numbers=True))
         else:
             R = _group_rows(q, h, d, plan_in, cfg)
             in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))

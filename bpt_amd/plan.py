@@ -142,6 +142,21 @@ def link_groups_host(grp_dst, grp_src, n_edges):
     return out
 
 
+def pair_numbers_host(grp_mine, grp_theirs, n_edges):
+    """For every (entry, member) of `grp_mine` the number, among the pairs of `grp_theirs`, of the pair that is the same
+    edge (pairs are numbered entry by entry, members ascending: grp["pair_eid"][number] = edge id); 0 where the entry has
+    no such member and in the GROUP_PAD_ENTRIES * R elements of padding.  int32, length (n_entries + GROUP_PAD_ENTRIES) * R."""
+    pe = np.asarray(grp_theirs["pair_eid"], dtype=np.int64)
+    if len(pe) != n_edges or (n_edges and (np.bincount(pe, minlength=n_edges) != 1).any()):
+        raise ValueError("the partner's groups do not cover every edge exactly once")
+    number = np.zeros(n_edges + 1, dtype=np.int32)
+    number[pe] = np.arange(n_edges, dtype=np.int32)
+    se = np.asarray(grp_mine["slot_eid"], dtype=np.int64)
+    out = np.zeros((len(se) + GROUP_PAD_ENTRIES) * grp_mine["R"], dtype=np.int32)
+    out[:se.size] = np.where(se >= 0, number[np.maximum(se, 0)], 0).reshape(-1)
+    return out
+
+
 def _tensor_bytes(obj):
     """Bytes of the torch tensors reachable from a plan's containers (dicts, tuples, lists)."""
     if isinstance(obj, torch.Tensor):
@@ -220,13 +235,15 @@ class Plan:
                 self._groups[(R, order_mode)] = hit
         return hit
 
-    def linked_to(self, plan_src, R=GROUP_R, order=None, partner_order=GROUP_ORDER_SRC):
+    def linked_to(self, plan_src, R=GROUP_R, order=None, partner_order=GROUP_ORDER_SRC, pair_numbers=False):
         """`bpt_plan` of this plan whose grp_pairs maps each (entry, member) of its groups (built with `order`) to the
         position entry' * R + member' of the same edge in the groups of `plan_src` (the plan of the other CSR side of the
-        same graph, groups built with `partner_order`).  The row-group kernels link the destination side to the source
-        side, the tile kernels the source side to the destination side."""
+        same graph, groups built with `partner_order`) or, with pair_numbers, to the NUMBER of that pair there (the
+        entry's first pair + the rank of the member in its mask; 0 where the pair does not exist).  The row-group kernels
+        link the destination side to the source side by positions, the tile kernels the source side to the destination
+        side by pair numbers."""
         o_mine, o_theirs = (GROUP_ORDER if order is None else order), (GROUP_ORDER if partner_order is None else partner_order)
-        if (R, o_mine) not in self._groups and (R, o_theirs) not in plan_src._groups and plan_src is not self:
+        if isinstance(plan_src, Plan) and plan_src is not self and (R, o_mine) not in self._groups and (R, o_theirs) not in plan_src._groups:
             # both sides still to be grouped: the partner's groups are built on a second thread meanwhile (the builder
             # is a plain C function, called with the interpreter lock released)
             other = _group_pool().submit(plan_src.ensure_groups, R, partner_order)
@@ -234,13 +251,16 @@ class Plan:
             theirs = other.result()
         else:
             mine, theirs = self.ensure_groups(R, order), plan_src.ensure_groups(R, partner_order)
-        key = (id(plan_src), R, order, partner_order)
+        key = (id(plan_src), R, order, partner_order) + ((True,) if pair_numbers else ())
         with self._lock:
             hit = self._links.get(key)
             if hit is None:
                 if self.n_edges != plan_src.n_edges or not (self.covers_all_edges and plan_src.covers_all_edges):
                     raise ValueError("the two plans do not describe the same edge set")
-                pairs = torch.from_numpy(link_groups_host(mine["host"], theirs["host"], self.n_edges)).to(self.device)
+                if pair_numbers:
+                    pairs = torch.from_numpy(pair_numbers_host(mine["host"], theirs["host"], self.n_edges)).to(self.device)
+                else:
+                    pairs = torch.from_numpy(link_groups_host(mine["host"], theirs["host"], self.n_edges)).to(self.device)
                 st = PlanStruct.from_buffer_copy(mine["struct"])
                 st.grp_pairs = pairs.data_ptr()
                 hit = (st, pairs, plan_src)          # keeps the mapping and the partner alive
@@ -422,10 +442,11 @@ class DevicePlan:
                 self._groups[(R, by_mask)] = hit
         return hit
 
-    def linked_to(self, plan_src, R=GROUP_R, order=None, partner_order=GROUP_ORDER_SRC):
-        """As Plan.linked_to, with the pair mapping computed on the GPU (bpt_plan_link_device)."""
+    def linked_to(self, plan_src, R=GROUP_R, order=None, partner_order=GROUP_ORDER_SRC, pair_numbers=False):
+        """As Plan.linked_to, with the pair mapping computed on the GPU (bpt_plan_link_device; the pair numbers by an
+        inverse permutation and a gather)."""
         mine, theirs = self.ensure_groups(R, order), plan_src.ensure_groups(R, partner_order)
-        key = (id(plan_src), R, order, partner_order)
+        key = (id(plan_src), R, order, partner_order) + ((True,) if pair_numbers else ())
         with self._lock:
             hit = self._links.get(key)
             if hit is None:
@@ -435,7 +456,18 @@ class DevicePlan:
                 if not isinstance(plan_src, DevicePlan):
                     # the partner was planned on the host (the two sides of a bipartite graph can fall on either side
                     # of the size rule): map the pairs there, from the downloaded group arrays
-                    pairs = torch.from_numpy(link_groups_host(mine["host"], theirs["host"], E)).to(self.device)
+                    mapped = (pair_numbers_host if pair_numbers else link_groups_host)(mine["host"], theirs["host"], E)
+                    pairs = torch.from_numpy(mapped).to(self.device)
+                    st = PlanStruct.from_buffer_copy(mine["struct"])
+                    st.grp_pairs = pairs.data_ptr()
+                    hit = (st, pairs, plan_src)
+                    self._links[key] = hit
+                    return hit[0]
+                if pair_numbers:
+                    number = torch.zeros(E + 1, dtype=torch.int32, device=self.device)
+                    number[theirs["dev"]["pair_eid"][:E].long()] = torch.arange(E, dtype=torch.int32, device=self.device)
+                    pairs = number[mine["dev"]["eids"].long()]          # absent members carry the edge id E: number 0
+                    torch.cuda.current_stream(self.device).synchronize()
                     st = PlanStruct.from_buffer_copy(mine["struct"])
                     st.grp_pairs = pairs.data_ptr()
                     hit = (st, pairs, plan_src)

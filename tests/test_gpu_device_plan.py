@@ -123,6 +123,16 @@ def test_device_plan_equals_model_and_host(name, seg):
             want = model.link_groups(grps[1], grps[0], len(src), GROUP_PAD_ENTRIES)
             got = host(plans[1][0]._links[(id(plans[0][0]), R, None, None)][1])
             assert np.array_equal(got, want) and st.grp_pairs
+            # ... and by pair numbers (what the tile kernels' scratch is indexed by): the number of the same edge's pair
+            # on the destination side, from the model's own pair lists
+            from bpt_amd.plan import pair_numbers_host
+            st = plans[1][0].linked_to(plans[0][0], R, partner_order=None, pair_numbers=True)
+            got = host(plans[1][0]._links[(id(plans[0][0]), R, None, None, True)][1])
+            want = pair_numbers_host(grps[1], grps[0], len(src))
+            assert np.array_equal(got, want) and st.grp_pairs
+            number = {int(e): i for i, e in enumerate(grps[0]["pair_eid"])}
+            se = np.asarray(grps[1]["slot_eid"]).reshape(-1)
+            assert all(want[i] == number[int(e)] for i, e in enumerate(se) if e >= 0) and not want[len(se):].any()
 
 
 def test_device_plan_without_indices_and_with_uncovered_slots():

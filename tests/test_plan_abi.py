@@ -164,3 +164,32 @@ def test_noalloc_entry_refuses_a_plan_that_does_not_fit_its_scratch():
     big = _lib.PlanStruct(None, None, None, None, None, 0, 0, 0, 0, 10 ** 6)       # a million partial rows
     assert alib.bpt_attention_forward_noalloc(ctypes.byref(big), None, None, None, None, None, None, 0.125, 0.0, 0, 8, 64, 0, None) == -8
     assert b"scratch" in alib.bpt_strerror(-8)
+
+
+def test_pair_numbers_of_host_built_groups():
+    """plan.pair_numbers_host: every (entry, member) of the source-side groups gets the number of the same edge's pair in
+    the destination-side groups (pairs numbered entry by entry, members ascending), checked through the edge ids."""
+    import numpy as np
+    from bpt_amd import graphbuilder as gb, plan
+    g = gb.BinaryPartition(300, True, 2, 10)
+    src, dst, _ = g.get_edges()
+    n = g.number_of_nodes
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, n, as_torch=False)
+    a_in, _ = plan.build_plan_host(COL, IC, in_csr[2], in_csr[1], n, n, 64)
+    a_out, _ = plan.build_plan_host(ROW, IR, out_csr[2], out_csr[1], n, n, 64)
+    g_in = plan.build_groups_host(a_in, n, R=16, max_pairs=0)
+    g_out = plan.build_groups_host(a_out, n, R=16, max_pairs=0)
+    pairs = plan.pair_numbers_host(g_out, g_in, len(src))
+    se = np.asarray(g_out["slot_eid"]).reshape(-1)
+    assert len(pairs) == (len(g_out["slot_eid"]) + plan.GROUP_PAD_ENTRIES) * 16 and not pairs[len(se):].any()
+    assert np.array_equal(np.asarray(g_in["pair_eid"])[pairs[:len(se)][se >= 0]], se[se >= 0])      # same edge on both sides
+    assert not pairs[:len(se)][se < 0].any()
+    # the pair number of (entry, member) on the destination side = the entry's first pair + rank of the member in its mask
+    ent = np.asarray(g_in["entries"]).reshape(-1, 4)
+    sd = np.asarray(g_in["slot_eid"]).reshape(-1, 16)
+    for u in (0, len(ent) // 2, len(ent) - 1):
+        members = [m for m in range(16) if (ent[u, 1] >> m) & 1]
+        assert [int(g_in["pair_eid"][ent[u, 2] + i]) for i in range(len(members))] == [int(sd[u, m]) for m in members]
+    with pytest.raises(ValueError):
+        bad = dict(g_in, pair_eid=np.zeros_like(g_in["pair_eid"]))
+        plan.pair_numbers_host(g_out, bad, len(src))
