@@ -227,17 +227,54 @@ __global__ __launch_bounds__(BLOCK) void k_combine_sum(const int32_t *__restrict
     combine_sum_block<T>(heavy + 3 * blockIdx.x, ws + (size_t)blockIdx.z * ws_stride, blockIdx.z == 0 ? Y0 : Y1, C, accumulate != 0);
 }
 
-// The three sums of the fused backward in one launch: blocks x < n_a combine rows of list A into YA (z = 0 only),
-// the others rows of list B into YB0 (z = 0) and YB1 (z = 1).
+// The three sums of the fused backward in one launch, four columns per lane (C a multiple of 256, float partials): grid
+// (n_a + n_b, C / 256, 2); blocks x < n_a combine rows of list A into YA (z = 0 only), the others rows of list B into YB0
+// (z = 0) and YB1 (z = 1).  Every column is added in the order combine_sum_block uses (wave w takes slots w, w + 4, ...;
+// the four wave sums in wave order).
+template <typename T> __device__ __forceinline__ void store4(T *p, float4 v);
+template <> __device__ __forceinline__ void store4<float>(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t *p, float4 v) {
+    *reinterpret_cast<uint2 *>(p) = make_uint2((uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16),
+                                               (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16));
+}
+template <typename T>
+__device__ __forceinline__ void combine_sum_block4(const int32_t *__restrict__ hv, const float *__restrict__ ws, T *__restrict__ Y, int C) {
+    __shared__ float4 part[WAVES_PER_BLOCK][WAVE];
+    const int row = hv[0], s0 = hv[1], ns = hv[2];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int j = (blockIdx.y * WAVE + lane) * 4;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float *col = ws + (size_t)s0 * C + j;
+    int k = w;
+    for (; k + 7 * WAVES_PER_BLOCK < ns; k += 8 * WAVES_PER_BLOCK) {
+        float4 t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = *reinterpret_cast<const float4 *>(col + (size_t)(k + u * WAVES_PER_BLOCK) * C);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { s.x += t[u].x; s.y += t[u].y; s.z += t[u].z; s.w += t[u].w; }
+    }
+    for (; k < ns; k += WAVES_PER_BLOCK) {
+        const float4 t = *reinterpret_cast<const float4 *>(col + (size_t)k * C);
+        s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+    }
+    part[w][lane] = s;
+    __syncthreads();
+    if (w == 0) {
+        float4 r = part[0][lane];
+#pragma unroll
+        for (int i = 1; i < WAVES_PER_BLOCK; ++i) { r.x += part[i][lane].x; r.y += part[i][lane].y; r.z += part[i][lane].z; r.w += part[i][lane].w; }
+        store4<T>(Y + (size_t)row * C + j, r);
+    }
+}
 template <typename T>
 __global__ __launch_bounds__(BLOCK) void k_combine_sum3(const int32_t *__restrict__ heavy_a, int n_a, const float *__restrict__ ws_a,
-                                                        T *__restrict__ YA, const int32_t *__restrict__ heavy_b,
-                                                        const float *__restrict__ ws_b, T *__restrict__ YB0, T *__restrict__ YB1, int C,
-                                                        size_t ws_stride_b) {
+                                                           T *__restrict__ YA, const int32_t *__restrict__ heavy_b,
+                                                           const float *__restrict__ ws_b, T *__restrict__ YB0, T *__restrict__ YB1, int C,
+                                                           size_t ws_stride_b) {
     if ((int)blockIdx.x < n_a) {
-        if (blockIdx.z == 0) combine_sum_block<T>(heavy_a + 3 * blockIdx.x, ws_a, YA, C);
+        if (blockIdx.z == 0) combine_sum_block4<T>(heavy_a + 3 * blockIdx.x, ws_a, YA, C);
     } else {
-        combine_sum_block<T>(heavy_b + 3 * (blockIdx.x - n_a), ws_b + (size_t)blockIdx.z * ws_stride_b, blockIdx.z == 0 ? YB0 : YB1, C);
+        combine_sum_block4<T>(heavy_b + 3 * (blockIdx.x - n_a), ws_b + (size_t)blockIdx.z * ws_stride_b, blockIdx.z == 0 ? YB0 : YB1, C);
     }
 }
 
@@ -3285,7 +3322,7 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
             }
             st = launch_status();
             if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;
-            hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / WAVE, 2), dim3(BLOCK), 0, s, Pin->heavy,
+            hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / (4 * WAVE), 2), dim3(BLOCK), 0, s, Pin->heavy,
                                (int)Pin->n_heavy, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
                                (size_t)Pout->n_slots * H * D);
             return launch_status();
@@ -3319,7 +3356,7 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
             }
             st = launch_status();
             if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;
-            hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / WAVE, 2), dim3(BLOCK), 0, s, Pin->heavy,
+            hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / (4 * WAVE), 2), dim3(BLOCK), 0, s, Pin->heavy,
                                (int)Pin->n_heavy, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
                                (size_t)Pout->n_slots * H * D);
             return launch_status();
@@ -3378,7 +3415,7 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     st = launch_status();
     if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;
     // partial rows of dq (destination side) and of dk, dv (source side) in one launch
-    hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / WAVE, 2), dim3(BLOCK), 0, s, Pin->heavy,
+    hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / (4 * WAVE), 2), dim3(BLOCK), 0, s, Pin->heavy,
                        (int)Pin->n_heavy, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
                        (size_t)Pout->n_slots * H * D);
     return launch_status();
