@@ -237,8 +237,15 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t *p, float4 v) 
     *reinterpret_cast<uint2 *>(p) = make_uint2((uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16),
                                                (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16));
 }
+template <typename T> __device__ __forceinline__ float4 load4(const T *p);
+template <> __device__ __forceinline__ float4 load4<float>(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+template <> __device__ __forceinline__ float4 load4<bf16_t>(const bf16_t *p) {
+    const uint2 x = *reinterpret_cast<const uint2 *>(p);
+    return make_float4(__uint_as_float(x.x << 16), __uint_as_float(x.x & 0xffff0000u), __uint_as_float(x.y << 16), __uint_as_float(x.y & 0xffff0000u));
+}
 template <typename T>
-__device__ __forceinline__ void combine_sum_block4(const int32_t *__restrict__ hv, const float *__restrict__ ws, T *__restrict__ Y, int C) {
+__device__ __forceinline__ void combine_sum_block4(const int32_t *__restrict__ hv, const float *__restrict__ ws, T *__restrict__ Y, int C,
+                                                   bool accumulate = false) {
     __shared__ float4 part[WAVES_PER_BLOCK][WAVE];
     const int row = hv[0], s0 = hv[1], ns = hv[2];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -263,6 +270,10 @@ __device__ __forceinline__ void combine_sum_block4(const int32_t *__restrict__ h
         float4 r = part[0][lane];
 #pragma unroll
         for (int i = 1; i < WAVES_PER_BLOCK; ++i) { r.x += part[i][lane].x; r.y += part[i][lane].y; r.z += part[i][lane].z; r.w += part[i][lane].w; }
+        if (accumulate) {
+            const float4 y = load4<T>(Y + (size_t)row * C + j);
+            r.x += y.x; r.y += y.y; r.z += y.z; r.w += y.w;
+        }
         store4<T>(Y + (size_t)row * C + j, r);
     }
 }
@@ -276,6 +287,13 @@ __global__ __launch_bounds__(BLOCK) void k_combine_sum3(const int32_t *__restric
     } else {
         combine_sum_block4<T>(heavy_b + 3 * (blockIdx.x - n_a), ws_b + (size_t)blockIdx.z * ws_stride_b, blockIdx.z == 0 ? YB0 : YB1, C);
     }
+}
+
+// k_combine_sum for the specialised shapes (float partials, C a multiple of 256): grid (n_heavy, C / 256, n_out)
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_combine_sum_v4(const int32_t *__restrict__ heavy, const float *__restrict__ ws, T *__restrict__ Y0,
+                                                          T *__restrict__ Y1, int C, size_t ws_stride, int accumulate = 0) {
+    combine_sum_block4<T>(heavy + 3 * blockIdx.x, ws + (size_t)blockIdx.z * ws_stride, blockIdx.z == 0 ? Y0 : Y1, C, accumulate != 0);
 }
 
 // dB[eid[p], d] = sum_h dy[eid[p], h] * A[row, h, d]      (graphop_kernel.cu:79-94)
@@ -2966,7 +2984,7 @@ int run_spmm_fast(const bpt_plan *P, const void *W0, const void *X0, void *Y0, c
     }
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
-    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy, H * D / WAVE, NOUT), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
+    hipLaunchKernelGGL((k_combine_sum_v4<T>), dim3((int)P->n_heavy, H * D / (4 * WAVE), NOUT), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
                        (T *)Y0, (T *)Y1, H * D, (size_t)P->n_slots * H * D);
     return launch_status();
 }
@@ -3010,7 +3028,7 @@ int run_nme_bwd_fast(const bpt_plan *P, const void *A, const void *B, const void
     int st = launch_status();
     if (st != BPT_OK) return st;
     if (P->n_heavy > 0) {
-        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
+        hipLaunchKernelGGL((k_combine_sum_v4<T>), dim3((int)P->n_heavy, H * D / (4 * WAVE), 1), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
                            (T *)dA, (T *)nullptr, H * D, (size_t)0);
         st = launch_status();
         if (st != BPT_OK) return st;
@@ -3151,7 +3169,7 @@ int run_spmm_grp(const bpt_plan *P, const void *W, const void *X, void *Y, float
 #undef LAUNCH_SPMM
     int st = launch_status();
     if (st != BPT_OK || P->n_heavy == 0) return st;
-    hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)P->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
+    hipLaunchKernelGGL((k_combine_sum_v4<T>), dim3((int)P->n_heavy, H * D / (4 * WAVE), 1), dim3(BLOCK), 0, s, P->heavy, (const float *)ws,
                        (T *)Y, (T *)nullptr, H * D, (size_t)0, accumulate);
     return launch_status();
 }
@@ -3391,7 +3409,7 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     int st = launch_status();
     if (st != BPT_OK) return st;
     if (Pin->n_heavy > 0 && !grouped) {
-        hipLaunchKernelGGL((k_combine_sum<T>), dim3((int)Pin->n_heavy, H * D / WAVE, 1), dim3(BLOCK), 0, s, Pin->heavy,
+        hipLaunchKernelGGL((k_combine_sum_v4<T>), dim3((int)Pin->n_heavy, H * D / (4 * WAVE), 1), dim3(BLOCK), 0, s, Pin->heavy,
                            (const float *)ws_rows, (T *)dq, (T *)nullptr, H * D, (size_t)0);
         st = launch_status();
         if (st != BPT_OK) return st;
