@@ -45,7 +45,9 @@ typedef enum {
 
 /* Device-resident plan of one CSR side (see bptg_plan_fill / bptg_group_plan for the array contents).
  * The grp_* fields are optional (n_groups == 0: none); the fused attention entries use them to let one
- * wavefront own up to grp_R rows that share neighbours, loading each neighbour row once for all, and so do the
+ * wavefront own up to grp_R rows that share neighbours, loading each neighbour row once for all (grp_R = 4 or 8:
+ * row-group kernels; grp_R = 16 with d = 64, f32 or bf16: the kernels that multiply 16 x 16 blocks of
+ * (row, neighbour) pairs on the matrix cores, one wavefront per group and head), and so do the
  * SDDMM / SpMM-shaped ops (maskedmm_csr, vector_spmm, rel_bias) when the plan also carries grp_eids and the shape
  * has specialised kernels; without groups every row (segment) has a wavefront of its own. */
 typedef struct {
@@ -58,12 +60,18 @@ typedef struct {
     const int32_t *grp_members;  /* n_groups * grp_R * 2 : (row, slot), row = -1 unused */
     const int32_t *grp_ptr;      /* n_groups + 1 : entry range of each group */
     const int32_t *grp_entries;  /* n_grp_entries * 4 : neighbour id, member mask, first pair, 0 */
-    const int32_t *grp_pairs;    /* (n_grp_entries + 8) * grp_R or NULL.  On the destination-side plan of the
-                                    fused backward: for (entry u, member m) of this plan, at [u * grp_R + m], the
-                                    position u' * grp_R + m' of the same edge in the source-side plan (the
-                                    per-pair scratch is laid out in that order); where the entry's mask has
-                                    no bit m, and in the 8 entries of padding, the spare position
-                                    (n_grp_entries of the source side + 8) * grp_R - 1 */
+    const int32_t *grp_pairs;    /* (n_grp_entries + 8) * grp_R or NULL.  Links the two sides' plans for the
+                                    fused backward, whose per-pair scratch one side writes and the other reads.
+                                    grp_R = 4 or 8 (row groups): on the DESTINATION-side plan, for (entry u,
+                                    member m) of this plan, at [u * grp_R + m], the position u' * grp_R + m' of
+                                    the same edge in the source-side plan (the scratch is laid out in that
+                                    order); where the entry's mask has no bit m, and in the 8 entries of
+                                    padding, the spare position (n_grp_entries of the source side + 8) * grp_R - 1.
+                                    grp_R = 16 (tiles): on the SOURCE-side plan, at [u * 16 + m], the pair number
+                                    of the same edge in the destination-side plan, i.e. that side's
+                                    grp_entries[u'].first_pair + (number of mask bits below m'), in 0 .. n_edges-1
+                                    (the scratch is compact, one record per edge and head); 0 where the mask has
+                                    no bit m and in the padding (never dereferenced) */
     const int32_t *grp_chunks;   /* 9 : groups grp_chunks[x] .. grp_chunks[x+1]-1 are walked by XCD x */
     int64_t n_groups, grp_R;
     int64_t grp_max_chunk;       /* largest chunk length; the row-group kernels launch 8 * grp_max_chunk workgroups */
