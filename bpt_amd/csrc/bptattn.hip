@@ -2803,6 +2803,305 @@ __global__ __launch_bounds__(WAVE) void k_sddmm_grp(bpt_plan P, const T *__restr
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// rel_pos score term (modules/attention.py:69-71) over the plan of the destinations with the edge types as indices: the
+// table's rows are shared by all heads and few (at most 1000, 64 columns), so the products go to the matrix cores.
+// ------------------------------------------------------------------------------------------
+// 16 consecutive elements as floats
+template <typename T> __device__ __forceinline__ void rel_load16(const T *p, float (&out)[16]);
+template <> __device__ __forceinline__ void rel_load16<float>(const float *p, float (&out)[16]) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const float4 x = *reinterpret_cast<const float4 *>(p + 4 * t);
+        out[4 * t] = x.x; out[4 * t + 1] = x.y; out[4 * t + 2] = x.z; out[4 * t + 3] = x.w;
+    }
+}
+template <> __device__ __forceinline__ void rel_load16<bf16_t>(const bf16_t *p, float (&out)[16]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const uint4 x = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(p) + 16 * t);
+        const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            out[8 * t + 2 * i] = __uint_as_float(w[i] << 16);
+            out[8 * t + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+}
+
+// A work item (a row or a segment of a long row) and the types and edge ids of its first 64 slots (lane l: slot b + l).
+struct RelHead {
+    int row, b, e, out_slot;
+    int type, edge;
+};
+__device__ __forceinline__ void rel_head_load(const bpt_plan &P, const int4 item, int lane, RelHead &r) {
+    // the item is the same for all lanes of the wavefront: keep it in scalar registers
+    r.row = __builtin_amdgcn_readfirstlane(item.x); r.b = __builtin_amdgcn_readfirstlane(item.y);
+    r.e = __builtin_amdgcn_readfirstlane(item.z); r.out_slot = __builtin_amdgcn_readfirstlane(item.w);
+    const int slot = r.b + min(lane, max(min(WAVE, r.e - r.b), 1) - 1);        // lanes past the end repeat the last slot
+    r.type = r.b < r.e ? P.idx[slot] : 0;
+    r.edge = r.b < r.e ? P.eid[slot] : 0;
+}
+
+// bias[eid[p], head] = q[row(p), head, :] . table[idx[p], :] for every slot p of the plan (idx = edge type).  The heads
+// of an item's row are rows of the A operand of v_mfma_f32_16x16x4f32 (row number c of A = head c % H), 16 consecutive
+// slots of the item the 16 columns of B; lane (g, c) holds columns 16 g .. 16 g + 15 of q for head c % H and of the table
+// row of slot c, and receives the results of heads 4 g .. 4 g + 3 for slot c, which it stores as one vector where
+// 4 g < H.  Each wavefront takes the items gw, gw + GW, ... and keeps their loads ahead of their use in three steps
+// (descriptor; types and edge ids of the first 64 slots; the q row and the table rows of the first 16 slots), each one
+// item further ahead than the one that needs its result; within an item the table rows of the next 16 slots are in
+// flight during the products.
+template <typename T, int H>
+__global__ __launch_bounds__(BLOCK) void k_rel_bias_rows(bpt_plan P, const T *__restrict__ q, const T *__restrict__ table, float *__restrict__ bias) {
+    constexpr int D = 64;
+    static_assert(H == 4 || H == 8 || H == 16, "four consecutive heads per lane");
+    const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+    const int GW = (int)gridDim.x * WAVES_PER_BLOCK, i_begin = (int)blockIdx.x * WAVES_PER_BLOCK + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int i_end = (int)P.n_items;
+    const int4 *items = reinterpret_cast<const int4 *>(P.items);
+    const int4 none = make_int4(0, 0, 0, -1);
+    struct Body { float aq[16], bt[16]; };
+    auto body_load = [&](const RelHead &r, Body &y) {
+        rel_load16<T>(q + ((size_t)r.row * H + (c % H)) * D + 16 * g, y.aq);
+        rel_load16<T>(table + (size_t)lane_bcast(r.type, c) * D + 16 * g, y.bt);
+    };
+    RelHead hd, hd_next;
+    Body bd, bd_next;
+    rel_head_load(P, i_begin < i_end ? items[i_begin] : none, lane, hd_next);
+    body_load(hd_next, bd_next);
+    hd = hd_next;
+    rel_head_load(P, i_begin + GW < i_end ? items[i_begin + GW] : none, lane, hd_next);
+    int4 desc = i_begin + 2 * GW < i_end ? items[i_begin + 2 * GW] : none;
+    for (int i = i_begin; i < i_end; i += GW) {
+        bd = bd_next;
+        body_load(hd_next, bd_next);                     // the item after this one
+        const RelHead cur = hd;
+        hd = hd_next;
+        rel_head_load(P, desc, lane, hd_next);           // the second after
+        desc = i + 3 * GW < i_end ? items[i + 3 * GW] : none;
+        for (int p0 = cur.b; p0 < cur.e; p0 += WAVE) {
+            const int cnt = min(WAVE, cur.e - p0);
+            int type = cur.type, edge = cur.edge;
+            float bt[2][16];
+            if (p0 == cur.b) {
+#pragma unroll
+                for (int t = 0; t < 16; ++t) bt[0][t] = bd.bt[t];
+            } else {                                     // (items longer than 64 slots: the rest, fetched on the spot)
+                const int slot = p0 + min(lane, cnt - 1);
+                type = P.idx[slot]; edge = P.eid[slot];
+                rel_load16<T>(table + (size_t)lane_bcast(type, c) * D + 16 * g, bt[0]);
+            }
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk) {
+                if (16 * blk < cnt) {
+                    if (16 * (blk + 1) < cnt) rel_load16<T>(table + (size_t)lane_bcast(type, 16 * (blk + 1) + c) * D + 16 * g, bt[(blk + 1) & 1]);
+                    const floatx4v acc = tile_dot(bd.aq, bt[blk & 1]);
+                    const int e = lane_bcast(edge, 16 * blk + c);
+                    if (16 * blk + c < cnt && 4 * g < H)
+                        *reinterpret_cast<float4 *>(bias + (size_t)e * H + 4 * g) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+                }
+            }
+        }
+    }
+}
+
+// Gradients of that term from ds[e, head] = dL/d(score of edge e before scaling): dq[row] += sum over the row's slots of
+// ds[eid] * table[type] (all heads), and the table's gradient dtable[t] = sum over the slots of type t and the heads of
+// ds[eid, head] * q[row, head].  Lane l owns column l.  Each wavefront walks every GW-th of the plan's work items (rows
+// and segments of long rows; a segment's part of dq goes to the workspace slot of the item, which k_combine_sum_v4
+// adds to dq) and keeps its own sums per edge type in LDS (used[type] = the type's number among the n_used types
+// that occur); the wavefronts of a workgroup add theirs in a fixed order and the workgroup writes one partial table,
+// part[(u * gridDim.x + block) * 64 + column], which k_rel_table_sum adds up.  Every sum has one owner and a fixed order.
+// The loads of an item run ahead of its use in three steps (descriptor; types and edge ids of its first 64 slots; their ds
+// values and numbers and the item's q and dq rows), each one item further ahead than the one that needs its result.
+template <int H>
+struct RelBody {             // what the walk of those slots needs: per lane the type's number and the ds values of its slot;
+    int u;                   // the item's q row and, for a whole row, the dq row it adds to (lane l: column l)
+    float dsv[H];
+    float qh[H], old[H];
+};
+template <typename T, int H>
+__device__ __forceinline__ void rel_body_load(const RelHead &r, const float *__restrict__ ds, const T *__restrict__ q, const T *__restrict__ dq,
+                                              const int32_t *__restrict__ used, int lane, RelBody<H> &y) {
+    constexpr int D = 64;
+    y.u = used[r.type];
+#pragma unroll
+    for (int h = 0; h < H; h += 4) {
+        const float4 x = *reinterpret_cast<const float4 *>(ds + (size_t)r.edge * H + h);
+        y.dsv[h] = x.x; y.dsv[h + 1] = x.y; y.dsv[h + 2] = x.z; y.dsv[h + 3] = x.w;
+    }
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+        y.qh[h] = Elem<T>::ld(q + ((size_t)r.row * H + h) * D + lane);
+        y.old[h] = r.out_slot < 0 ? Elem<T>::ld(dq + ((size_t)r.row * H + h) * D + lane) : 0.f;
+    }
+}
+template <typename T, int H, int NW>
+__global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const float *__restrict__ ds, const T *__restrict__ q,
+                                                            const T *__restrict__ table, const int32_t *__restrict__ used, int n_used,
+                                                            T *__restrict__ dq, float *__restrict__ ws_dq, float *__restrict__ part) {
+    constexpr int D = 64, C = H * D, AHEAD = H >= 16 ? 4 : 8;
+    extern __shared__ float rel_lds[];                    // NW tables of n_used x 64 sums, then NW x 64 x H staged ds values
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    float *acc = rel_lds + (size_t)w * n_used * D;
+    float *stage = rel_lds + (size_t)NW * n_used * D + (size_t)w * WAVE * H;
+    for (int u = 0; u < n_used; ++u) acc[u * D + lane] = 0.f;
+    // wavefront gw of GW takes the items gw, gw + GW, ...: the segments of a long row, which are neighbours, go to different wavefronts
+    const int GW = (int)gridDim.x * NW, i_begin = (int)blockIdx.x * NW + w, i_end = (int)P.n_items;
+    const int4 *items = reinterpret_cast<const int4 *>(P.items);
+    const int4 none = make_int4(0, 0, 0, -1);             // (an empty row: nothing to read, nothing to write)
+    RelHead hd, hd_next;
+    RelBody<H> bd, bd_next;
+    rel_head_load(P, i_begin < i_end ? items[i_begin] : none, lane, hd_next);
+    rel_body_load<T, H>(hd_next, ds, q, dq, used, lane, bd_next);
+    hd = hd_next;
+    rel_head_load(P, i_begin + GW < i_end ? items[i_begin + GW] : none, lane, hd_next);
+    int4 desc = i_begin + 2 * GW < i_end ? items[i_begin + 2 * GW] : none;
+    // one chunk of at most 64 slots whose ds values are staged: lane j of (type, u) belongs to slot j of the chunk
+    auto walk = [&](int cnt, int type, int u, const float (&qh)[H], float (&dqa)[H]) {
+        wave_lds_fence();
+        float tv[2][AHEAD];                               // this lane's column of the table rows of AHEAD slots, fetched together
+        auto fetch = [&](int j0, float (&t)[AHEAD]) {
+#pragma unroll
+            for (int x = 0; x < AHEAD; ++x) t[x] = Elem<T>::ld(table + (size_t)__builtin_amdgcn_readlane(type, min(j0 + x, cnt - 1)) * D + lane);
+        };
+        auto use = [&](int j0, const float (&t)[AHEAD]) {
+            // the ds values of the AHEAD slots first (zeros are staged for the slots past the chunk's end, which so add nothing),
+            // then four slots at a time: the sums so far, the products, the new sums.  The reads of the sums
+            // come before the products so that their latency is covered; where slots of a four have the same type, the
+            // later one's sum takes the earlier ones' terms in slot order, as if the four were added one after the other.
+            float4 dv[AHEAD][H / 4];
+#pragma unroll
+            for (int x = 0; x < AHEAD; ++x)
+#pragma unroll
+                for (int h = 0; h < H; h += 4) dv[x][h / 4] = *reinterpret_cast<const float4 *>(stage + min(j0 + x, WAVE - 1) * H + h);
+#pragma unroll
+            for (int x0 = 0; x0 < AHEAD; x0 += 4) {
+                if (j0 + x0 < cnt) {
+                    int un[4];
+                    float *sum[4];
+                    float before[4], gsum[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        un[x] = __builtin_amdgcn_readlane(u, min(j0 + x0 + x, cnt - 1));
+                        sum[x] = acc + un[x] * D + lane;
+                        before[x] = *sum[x];
+                    }
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const float tx = t[x0 + x];
+                        gsum[x] = 0.f;
+#pragma unroll
+                        for (int h = 0; h < H; h += 4) {
+                            const float4 d4 = dv[x0 + x][h / 4];
+                            gsum[x] = fmaf(d4.x, qh[h], gsum[x]); gsum[x] = fmaf(d4.y, qh[h + 1], gsum[x]);
+                            gsum[x] = fmaf(d4.z, qh[h + 2], gsum[x]); gsum[x] = fmaf(d4.w, qh[h + 3], gsum[x]);
+                            dqa[h] = fmaf(d4.x, tx, dqa[h]); dqa[h + 1] = fmaf(d4.y, tx, dqa[h + 1]);
+                            dqa[h + 2] = fmaf(d4.z, tx, dqa[h + 2]); dqa[h + 3] = fmaf(d4.w, tx, dqa[h + 3]);
+                        }
+                    }
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        float v = before[x];
+#pragma unroll
+                        for (int y = 0; y < x; ++y) v += un[y] == un[x] ? gsum[y] : 0.f;
+                        *sum[x] = v + gsum[x];
+                    }
+                }
+            }
+        };
+        fetch(0, tv[0]);
+        for (int j0 = 0; j0 < cnt; j0 += 2 * AHEAD) {
+            fetch(j0 + AHEAD, tv[1]);
+            use(j0, tv[0]);
+            fetch(j0 + 2 * AHEAD, tv[0]);
+            use(j0 + AHEAD, tv[1]);
+        }
+        wave_lds_fence();
+    };
+    for (int i = i_begin; i < i_end; i += GW) {
+        bd = bd_next;
+        rel_body_load<T, H>(hd_next, ds, q, dq, used, lane, bd_next);          // the item after this one
+        const RelHead cur = hd;
+        hd = hd_next;
+        rel_head_load(P, desc, lane, hd_next);                                   // the second after
+        desc = i + 3 * GW < i_end ? items[i + 3 * GW] : none;
+        float dqa[H];
+#pragma unroll
+        for (int h = 0; h < H; ++h) dqa[h] = 0.f;
+        if (cur.b < cur.e) {
+#pragma unroll
+            for (int h = 0; h < H; h += 4)
+                *reinterpret_cast<float4 *>(stage + lane * H + h) =
+                    lane < cur.e - cur.b ? make_float4(bd.dsv[h], bd.dsv[h + 1], bd.dsv[h + 2], bd.dsv[h + 3]) : make_float4(0.f, 0.f, 0.f, 0.f);
+            walk(min(WAVE, cur.e - cur.b), cur.type, bd.u, bd.qh, dqa);
+        }
+        for (int p0 = cur.b + WAVE; p0 < cur.e; p0 += WAVE) {                  // (items longer than 64 slots: the rest, fetched on the spot)
+            const int cnt = min(WAVE, cur.e - p0);
+            const int slot = p0 + min(lane, cnt - 1);
+            const int type = P.idx[slot], edge = P.eid[slot];
+#pragma unroll
+            for (int h = 0; h < H; h += 4)
+                *reinterpret_cast<float4 *>(stage + lane * H + h) =
+                    lane < cnt ? *reinterpret_cast<const float4 *>(ds + (size_t)edge * H + h) : make_float4(0.f, 0.f, 0.f, 0.f);
+            walk(cnt, type, used[type], bd.qh, dqa);
+        }
+        if (cur.out_slot < 0) {
+            if (cur.b < cur.e) {
+#pragma unroll
+                for (int h = 0; h < H; ++h) Elem<T>::st(dq + ((size_t)cur.row * H + h) * D + lane, bd.old[h] + dqa[h]);
+            }
+        } else {
+#pragma unroll
+            for (int h = 0; h < H; ++h) ws_dq[(size_t)cur.out_slot * C + h * D + lane] = dqa[h];
+        }
+    }
+    __syncthreads();
+    for (int u = w; u < n_used; u += NW) {
+        float sum = rel_lds[(size_t)u * D + lane];
+#pragma unroll
+        for (int x = 1; x < NW; ++x) sum += rel_lds[((size_t)x * n_used + u) * D + lane];
+        part[((size_t)u * gridDim.x + blockIdx.x) * D + lane] = sum;
+    }
+}
+
+// dtable[type] = the sum of the n_parts partial rows of the type's number u = used[type] (zero for a type that does
+// not occur).  One workgroup per type; 16 lanes cover a row (four columns each), so a wavefront reads four partial rows
+// per load: lane group s of wave w adds the rows 4 w + s, 4 w + s + 16, ...; the 16 sums are then added in a fixed order.
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_rel_table_sum(const float *__restrict__ part, const int32_t *__restrict__ used, int n_parts,
+                                                         T *__restrict__ dtable) {
+    constexpr int D = 64, GROUPS = BLOCK / 16;
+    __shared__ float4 sums[GROUPS][16];
+    const int type = blockIdx.x, u = used[type], grp = threadIdx.x >> 4, c4 = (threadIdx.x & 15) * 4;
+    if (u < 0) {
+        if (threadIdx.x < 16) store4<T>(dtable + (size_t)type * D + c4, make_float4(0.f, 0.f, 0.f, 0.f));
+        return;
+    }
+    const float *p = part + (size_t)u * n_parts * D + c4;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    int x = grp;
+    for (; x + 7 * GROUPS < n_parts; x += 8 * GROUPS) {
+        float4 t[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) t[k] = *reinterpret_cast<const float4 *>(p + (size_t)(x + k * GROUPS) * D);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { s.x += t[k].x; s.y += t[k].y; s.z += t[k].z; s.w += t[k].w; }
+    }
+    for (; x < n_parts; x += GROUPS) {
+        const float4 t = *reinterpret_cast<const float4 *>(p + (size_t)x * D);
+        s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+    }
+    sums[grp][threadIdx.x & 15] = s;
+    __syncthreads();
+    if (threadIdx.x < 16) {
+        float4 tot = sums[0][threadIdx.x];
+#pragma unroll
+        for (int k = 1; k < GROUPS; ++k) { const float4 t = sums[k][threadIdx.x]; tot.x += t.x; tot.y += t.y; tot.z += t.z; tot.w += t.w; }
+        store4<T>(dtable + (size_t)type * D + c4, tot);
+    }
+}
+
 // Measurement aid: what the memory system delivers to row gathers.  Every wavefront reads `iters` batches of
 // IN_FLIGHT pseudo-random 1 KB rows (16 bytes per lane, the access pattern of the attention kernels' neighbour rows)
 // of a region and keeps a checksum, so that nothing but the loads is timed.
@@ -2994,9 +3293,58 @@ bool spmm_grp_ok(const bpt_plan *P, int h, int d, int dtype);
 template <typename T, int H, int D> constexpr int head_slices();
 inline int group_grid(const bpt_plan *P);
 
+// shapes of the matrix-core kernel of the rel_pos term and of its gradient kernel
+inline bool rel_rows_shape(int h, int d, int dtype) {
+    return !g_force_generic.load(std::memory_order_relaxed) && d == 64 && (h == 4 || h == 8 || h == 16) && (dtype == BPT_F32 || dtype == BPT_BF16);
+}
+
+constexpr int REL_FWD_MAX_BLOCKS = 256 * 5;   // workgroups of four wavefronts: five wavefronts per SIMD of 256 compute units
+constexpr int REL_MAX_PARTS = 512;        // partial tables of the gradient kernel: two workgroups per compute unit
+
+// wavefronts per workgroup of k_rel_bias_bwd for n_used types (0: too many for the 64 KB of LDS a workgroup may take)
+inline int rel_bwd_waves(int64_t n_used, int h) {
+    for (int nw = 4; nw >= 1; nw >>= 1)
+        if ((int64_t)nw * (n_used * 64 + WAVE * h) * 4 <= 65536) return nw;
+    return 0;
+}
+
+template <typename T, int H>
+int run_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const void *table, const int32_t *used, int64_t n_types, int64_t n_used,
+                     void *dq, void *dtable, float *ws, hipStream_t s) {
+    const int nw = rel_bwd_waves(n_used, H);
+    const int n_parts = (int)std::min<int64_t>(REL_MAX_PARTS, std::max<int64_t>(1, (P->n_edges + nw * 128 - 1) / (nw * 128)));
+    const size_t lds = (size_t)nw * ((size_t)n_used * 64 + WAVE * H) * 4;
+    float *ws_dq = ws, *part = ws + (size_t)P->n_slots * H * 64;       // partial rows of dq of the split rows, then the partial tables
+#define L(NW) hipLaunchKernelGGL((k_rel_bias_bwd<T, H, NW>), dim3(n_parts), dim3(NW * WAVE), lds, s, *P, ds, (const T *)q, (const T *)table, used, \
+                                 (int)n_used, (T *)dq, ws_dq, part)
+    if (P->n_edges > 0) {
+        if (nw == 4) L(4); else if (nw == 2) L(2); else L(1);
+        int st = launch_status();
+        if (st != BPT_OK) return st;
+        if (P->n_heavy > 0) {
+            hipLaunchKernelGGL((k_combine_sum_v4<T>), dim3((unsigned)P->n_heavy, H * 64 / 256, 1), dim3(BLOCK), 0, s, P->heavy, ws_dq, (T *)dq,
+                               (T *)nullptr, H * 64, (size_t)0, 1);
+            st = launch_status();
+            if (st != BPT_OK) return st;
+        }
+    }
+#undef L
+    // (without edges there are no partial tables: every row of dtable becomes zero)
+    hipLaunchKernelGGL((k_rel_table_sum<T>), dim3((unsigned)n_types), dim3(BLOCK), 0, s, part, used, P->n_edges > 0 ? n_parts : 0, (T *)dtable);
+    return launch_status();
+}
+
 template <typename T, int H, int D>
 int run_rel_bias(const bpt_plan *P, const void *A, const void *table, float *bias, hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
+    if constexpr (D == 64 && (H == 4 || H == 8 || H == 16)) {
+        if (!g_force_generic.load(std::memory_order_relaxed) && aligned16(bias)) {      // rows on the matrix cores
+            // a wavefront per work item up to the number the GPU holds at once (five per SIMD), several items per wavefront beyond
+            const int blocks = (int)std::min<int64_t>(grid_for(P), REL_FWD_MAX_BLOCKS);
+            hipLaunchKernelGGL((k_rel_bias_rows<T, H>), dim3(blocks), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)table, bias);
+            return launch_status();
+        }
+    }
     if (spmm_grp_ok(P, H, D, sizeof(T) == 2 ? BPT_BF16 : BPT_F32)) {      // row groups: one load of a table row per group entry
         constexpr int HS = head_slices<T, H, D>();
         if (P->grp_R == 8)
@@ -3570,6 +3918,30 @@ int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table,
 #define X(HH, DD) if (h == HH && d == DD) return run_rel_bias<T, HH, DD>(plan, q, table, bias, s);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
+int64_t bpt_rel_bias_backward_workspace_bytes(const bpt_plan *plan, int64_t n_used, int h) {
+    if (!plan || n_used < 0 || h < 1) return 0;
+    return (plan->n_slots * h * 64 + n_used * REL_MAX_PARTS * 64) * 4;
+}
+
+int bpt_rel_bias_backward(const bpt_plan *plan, const float *ds, const void *q, const void *table, const int32_t *used, int64_t n_types,
+                          int64_t n_used, void *dq, void *dtable, void *workspace, int64_t workspace_bytes, int h, int d, int dtype,
+                          void *stream) {
+    CHECK(check_plan(plan, true));
+    CHECK(check_shape(h, d, dtype));
+    if (n_types < 0 || n_used < 0 || n_used > n_types) return BPT_ERR_SIZE;
+    if (!rel_rows_shape(h, d, dtype) || rel_bwd_waves(n_used, h) == 0) return BPT_ERR_UNSUPPORTED;
+    if (n_types == 0) return BPT_OK;
+    if (!used || !dtable || (plan->n_edges > 0 && (!ds || !q || !table || !dq))) return BPT_ERR_NULL;
+    if (!aligned16(ds)) return BPT_ERR_UNSUPPORTED;
+    if (!workspace || workspace_bytes < bpt_rel_bias_backward_workspace_bytes(plan, n_used, h) || !aligned16(workspace)) return BPT_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+#define X(HH) if (h == HH) return run_rel_bias_bwd<T, HH>(plan, ds, q, table, used, n_types, n_used, dq, dtable, (float *)workspace, s);
+    if (dtype == BPT_F32) { using T = float; X(4) X(8) X(16) }
+    if (dtype == BPT_BF16) { using T = bf16_t; X(4) X(8) X(16) }
 #undef X
     return BPT_ERR_UNSUPPORTED;
 }

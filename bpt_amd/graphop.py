@@ -367,9 +367,47 @@ def rel_bias_forward(col, indptr_c, eid_c, etype_slot, q, table):
     bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
     bias[E].zero_()
     with torch.cuda.device_of(q):
-        check_attn(_LIB.bpt_rel_bias_forward(_spmm_ref(plan, q, h, d, cfg), _ptr(q), _ptr(table), _ptr(bias), h, d, _dtype(q), _stream()),
-                   "rel_bias_forward")
+        ref = plan.ref if rel_rows_supported(q) else _spmm_ref(plan, q, h, d, cfg)      # the row kernel walks the plain CSR
+        check_attn(_LIB.bpt_rel_bias_forward(ref, _ptr(q), _ptr(table), _ptr(bias), h, d, _dtype(q), _stream()), "rel_bias_forward")
     return bias
+
+
+REL_MAX_USED_TYPES = 240      # edge types that may occur in one graph for rel_bias_backward (the kernel's on-chip sums)
+
+
+def rel_rows_supported(q):
+    """True if the rel_pos term of q's (h, d, dtype) has the kernels that walk the plain CSR of the destinations."""
+    h, d = _hd(q)
+    return q.dim() == 3 and d == 64 and h in (4, 8, 16) and q.dtype in (torch.float32, torch.bfloat16)
+
+
+def rel_bias_backward(col, indptr_c, eid_c, etype_slot, used, n_used, ds, q, table, dq):
+    """Gradients of the rel_pos score term (modules/attention.py:55-56,69-71: autograd of nn.Embedding and of
+    node_mul_edge) from ds (E or more rows, h) float32 = dL/d(score before scaling) per edge and head:
+    dq[row] += sum_p ds[eid_c[p]] * table[etype_slot[p]] in place, and returns dtable (n_types, d) with
+    dtable[t] = sum over the slots of type t and the heads of ds * q[row].  used (n_types,) int32: the number of every
+    type that occurs among the n_used of them, -1 for the others.  Raises if rel_rows_supported(q) is False or
+    n_used > REL_MAX_USED_TYPES."""
+    _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, etype_slot=etype_slot, used=used, ds=ds, q=q, table=table, dq=dq)
+    _same_dtype(q, table, dq)
+    h, d = _hd(q)
+    if table.dim() != 2 or table.size(1) != d:
+        raise ValueError(f"table must be (n_types, {d})")
+    if used.dtype != torch.int32 or used.numel() != table.size(0):
+        raise ValueError("used must be int32 with one element per table row")
+    if ds.dtype != torch.float32 or ds.dim() != 2 or ds.size(1) != h or ds.size(0) < eid_c.size(0):
+        raise ValueError(f"ds must be float32 (>= {eid_c.size(0)}, {h})")
+    if dq.shape != q.shape:
+        raise ValueError("dq must have the shape of q")
+    _expect_index(eid_c, etype_slot)
+    plan = plan_cache.get(col, indptr_c, eid_c, etype_slot, q.size(0), table.size(0))
+    dtable = torch.empty_like(table)
+    with torch.cuda.device_of(q):
+        nws = int(_LIB.bpt_rel_bias_backward_workspace_bytes(plan.ref, int(n_used), h))
+        ws = _scratch(max(nws, 16), q.device)
+        check_attn(_LIB.bpt_rel_bias_backward(plan.ref, _ptr(ds), _ptr(q), _ptr(table), _ptr(used), table.size(0), int(n_used), _ptr(dq),
+                                              _ptr(dtable), _ptr(ws), nws, h, d, _dtype(q), _stream()), "rel_bias_backward")
+    return dtable
 
 
 def _check_bias(bias, n_edges, h, device, cfg):
@@ -596,4 +634,14 @@ def set_grouped_ops(on):
 
 def set_force_generic(on):
     """Testing hook (process-wide, an atomic flag inside the library): route every op through the shape-generic kernels."""
+    global _FORCE_GENERIC
+    _FORCE_GENERIC = bool(on)
     return bool(_LIB.bpt_set_force_generic(1 if on else 0))
+
+
+_FORCE_GENERIC = False
+
+
+def force_generic_enabled():
+    """What set_force_generic last set."""
+    return _FORCE_GENERIC

@@ -97,33 +97,38 @@ class BPTRelAttention(Function):
     """BPTAttention with the rel_pos score term of modules/attention.py:69-71, s = (q.k + q.table[etype]) * scale,
     without the (E, d) rows of the embedding lookup: a small kernel writes the (E, h) term q[dst].table[etype], the
     fused kernels add it to the scores, and the backward kernel returns ds = dL/d(q.k + term) per edge and head,
-    from which two SpMMs form the term's gradients: dq += sum_e ds[e] table[etype[e]] over the in-CSR with the edge
-    types as column indices, and dtable[t] = sum_h sum_{e of type t} ds[e, h] q[dst(e), h] over a CSR whose rows
-    are the edge types.  All sums are row-owned (no atomics)."""
+    from which the term's gradients follow: dq += sum_e ds[e] table[etype[e]] over the in-CSR and
+    dtable[t] = sum_h sum_{e of type t} ds[e, h] q[dst(e), h].  One kernel forms both where the shape has it
+    (graphop.rel_bias_backward); otherwise two SpMMs do, the first over the in-CSR with the edge types as column indices,
+    the second over a CSR whose rows are the edge types.  All sums are row-owned (no atomics)."""
 
     @staticmethod
     def forward(ctx, row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed,
                 table, etype):
         aux = _rel_aux(etype, col, indptr_c, eid_c, table.size(0))
         table = table.contiguous()
-        bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux[0], q, table)
+        bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["etype_slot"], q, table)
         o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed, bias=bias)
         ctx.save_for_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, bias, table)
-        ctx.scale, ctx.dropout_p, ctx.seed, ctx.aux = scale, dropout_p, seed, aux
+        ctx.scale, ctx.dropout_p, ctx.seed, ctx.aux, ctx.etype = scale, dropout_p, seed, aux, etype
         return o
 
     @staticmethod
     def backward(ctx, do):
         row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, bias, table = ctx.saved_tensors
-        etype_slot, t_row, t_indptr, t_order, t_dst = ctx.aux
+        aux = ctx.aux
         dq, dk, dv, ds = _g.attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c,
                                                q, k, v, o, lse, do, ctx.scale, ctx.dropout_p, ctx.seed, bias=bias)
-        h = q.size(1)
-        ds = ds.to(q.dtype)
-        table_h = table.unsqueeze(1).expand(-1, h, -1).contiguous()
-        dq = vector_spmm_forward(col, indptr_c, eid_c, etype_slot, ds, table_h, n_rows=q.size(0), out=dq)
-        dtable = vector_spmm_forward(t_row, t_indptr, t_order, t_dst, ds, q, n_rows=table.size(0))
-        dtable = dtable.float().sum(1).to(table.dtype)
+        if _g.rel_rows_supported(q) and aux["n_used"] <= _g.REL_MAX_USED_TYPES and not _g.force_generic_enabled():
+            dtable = _g.rel_bias_backward(col, indptr_c, eid_c, aux["etype_slot"], aux["used"], aux["n_used"], ds, q, table, dq)
+        else:
+            t_row, t_indptr, t_order, t_dst = _rel_type_rows(aux, ctx.etype, col, indptr_c, eid_c, table.size(0))
+            h = q.size(1)
+            ds = ds.to(q.dtype)
+            table_h = table.unsqueeze(1).expand(-1, h, -1).contiguous()
+            dq = vector_spmm_forward(col, indptr_c, eid_c, aux["etype_slot"], ds, table_h, n_rows=q.size(0), out=dq)
+            dtable = vector_spmm_forward(t_row, t_indptr, t_order, t_dst, ds, q, n_rows=table.size(0))
+            dtable = dtable.float().sum(1).to(table.dtype)
         return None, None, None, None, None, None, None, None, dq, dk, dv, None, None, None, dtable, None
 
 
@@ -131,21 +136,38 @@ _rel_aux_cache = {}
 
 
 def _rel_aux(etype, col, indptr_c, eid_c, n_types):
-    """Index tensors of the rel_pos term, cached per (etype, in-CSR): the edge type of every in-CSR slot, and the
-    CSR whose row t lists the edges of type t (_type_csr) together with the destination node of each of its slots."""
+    """Index tensors of the rel_pos term, cached per (etype, in-CSR): etype_slot, the edge type of every in-CSR slot;
+    used (n_types,) int32, the number of every type that occurs in a slot among the n_used of them (-1 for the others).
+    Built where etype lives; two scalars are read back (the range check and n_used)."""
     key = tuple((t.data_ptr(), t.numel(), t._version) for t in (etype, col, indptr_c, eid_c)) + (str(etype.device), n_types)
     hit = _rel_aux_cache.get(key)
     if hit is None:
+        et = etype.detach()
+        if et.dim() != 1 or et.dtype != torch.int64:
+            raise ValueError("etype must be a 1-D int64 tensor")
+        if et.numel() and (int(et.min()) < 0 or int(et.max()) >= n_types):
+            raise ValueError("edge type out of range")
+        etype_slot = et.index_select(0, eid_c).contiguous()
+        present = torch.zeros(n_types, dtype=torch.bool, device=et.device).index_fill_(0, etype_slot, True)
+        number = torch.cumsum(present, 0, dtype=torch.int32) - 1
+        used = torch.where(present, number, torch.full_like(number, -1)).contiguous()
+        hit = {"etype_slot": etype_slot, "used": used, "n_used": int(present.sum()), "keep": (etype, col, indptr_c, eid_c)}
+        if len(_rel_aux_cache) > 16:
+            _rel_aux_cache.clear()
+        _rel_aux_cache[key] = hit           # "keep" holds the tensors so that their data_ptrs are not reused while cached
+    return hit
+
+
+def _rel_type_rows(aux, etype, col, indptr_c, eid_c, n_types):
+    """For the SpMM form of the table's gradient: the CSR whose row t lists the edges of type t (_type_csr) and the
+    destination node of each of its slots; kept with the other index tensors of the graph."""
+    if "type_rows" not in aux:
         t_row, t_indptr, t_order = _type_csr(etype, n_types)
-        etype_slot = etype.index_select(0, eid_c).contiguous()
         slot_dst = torch.repeat_interleave(col, indptr_c[1:] - indptr_c[:-1], output_size=eid_c.numel())   # destination of every in-CSR slot
         dst_of_eid = torch.empty_like(slot_dst)
         dst_of_eid[eid_c] = slot_dst
-        hit = (etype_slot, t_row, t_indptr, t_order, dst_of_eid.index_select(0, t_order).contiguous(), (etype, col, indptr_c, eid_c))
-        if len(_rel_aux_cache) > 16:
-            _rel_aux_cache.clear()
-        _rel_aux_cache[key] = hit           # holds the tensors so that their data_ptrs are not reused while cached
-    return hit[:5]
+        aux["type_rows"] = (t_row, t_indptr, t_order, dst_of_eid.index_select(0, t_order).contiguous())
+    return aux["type_rows"]
 
 
 def sparse_softmax(row, indptr, eid, x):

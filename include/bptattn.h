@@ -167,6 +167,22 @@ int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const
 int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, float *bias,
                          int h, int d, int dtype, void *stream);
 
+/* Gradients of that score term, the backward of embed_ak + node_mul_edge in modules/attention.py:55-56,69-71 (autograd of
+ * nn.Embedding and graphop.py's NodeMulEdgeFunction.backward), from ds (n_edges or more rows, h) float32 =
+ * dL/d(score of the edge before scaling), which bpt_attention_backward returns in ds_out:
+ *   dq[row, head, :] += sum over the slots p of the row of ds[eid[p], head] * table[idx[p], :]      (added to dq)
+ *   dtable[t, :]      = sum over the slots p with idx[p] == t and the heads of ds[eid[p], head] * q[row(p), head, :]
+ * without the (n_edges, d) gradient rows of the embedding lookup.  `plan` as for bpt_rel_bias_forward.
+ * used (n_types) int32: for every edge type that occurs in plan->idx its number among those types, 0 .. n_used - 1
+ * (any order), and -1 for the others, whose rows of dtable become zero.  dq and dtable have the dtype of q and table.
+ * workspace: bpt_rel_bias_backward_workspace_bytes(plan, n_used, h) bytes, 16-byte aligned.  Row-owned sums in a fixed order, no atomics.
+ * h in {4, 8, 16}, d = 64, f32 or bf16, and as many used types as fit the kernel's on-chip sums (240 at least);
+ * BPT_ERR_UNSUPPORTED otherwise (compose bpt_vector_spmm_forward calls instead). */
+int64_t bpt_rel_bias_backward_workspace_bytes(const bpt_plan *plan, int64_t n_used, int h);
+int bpt_rel_bias_backward(const bpt_plan *plan, const float *ds, const void *q, const void *table, const int32_t *used,
+                          int64_t n_types, int64_t n_used, void *dq, void *dtable, void *workspace, int64_t workspace_bytes,
+                          int h, int d, int dtype, void *stream);
+
 /* Fused attention layer core = modules/attention.py:66-77:
  *   o[dst] = sum_{e: src->dst} drop( softmax_dst( (q[dst].k[src] + bias[e]) * scale ) )[e] * v[src]
  * plan_in: rows = destinations (the reference's COL/INDPTR_C/in_csr), plan_out: rows = sources.

@@ -1,0 +1,133 @@
+"""GPU parity of the rel_pos score term's own kernels (modules/attention.py:55-56,69-71: embed_ak looked up per edge, then
+node_mul_edge, and their autograd) against the CPU oracle's node_mul_edge on the looked-up rows.
+
+Tolerances as everywhere: fp32 outputs rtol 1e-5 / atol 1e-5, fp32 gradients rtol 1e-4, bf16 2e-2.  The oracle runs in
+float64 on the same float32 / bf16 input values.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from test_gpu_parity import DEV, GTOL, TOL, case, close, f64, rand
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from bpt_amd import graphop, op
+    return graphop, op
+
+
+def edge_types(E, n_types, n_used, seed):
+    """E edge types out of n_types of which exactly min(n_used, E) occur, scattered over the range."""
+    rng = np.random.default_rng(seed)
+    pool = np.sort(rng.choice(n_types, size=min(n_used, n_types), replace=False))
+    et = pool[rng.integers(0, len(pool), E)]
+    m = min(len(pool), E)
+    et[rng.permutation(E)[:m]] = pool[:m]                # every type of the pool occurs
+    return et.astype(np.int64)
+
+
+def used_map(etype_slot, n_types):
+    present = np.zeros(n_types, dtype=bool)
+    present[etype_slot] = True
+    used = np.where(present, np.cumsum(present) - 1, -1).astype(np.int32)
+    return used, int(present.sum())
+
+
+SHAPES = [(torch.float32, 8), (torch.float32, 4), (torch.float32, 16), (torch.bfloat16, 8), (torch.bfloat16, 16)]
+GRAPH_NAMES = ["bpt512_k4", "bpt300_causal_k2", "multigraph", "fc_w100", "blocks8x30"]
+
+
+@pytest.mark.parametrize("dtype,h", SHAPES)
+@pytest.mark.parametrize("gname", GRAPH_NAMES)
+def test_score_term_matches_node_mul_edge_of_the_looked_up_rows(ops, gname, dtype, h):
+    graphop, _ = ops
+    d, n_types = 64, 1000
+    c = case(gname)
+    q = rand((c.n, h, d), dtype, 11, 0.5).to(DEV)
+    table = rand((n_types, d), dtype, 12, 0.5).to(DEV)
+    et = edge_types(c.E, n_types, 55, 13)
+    etype_slot = torch.from_numpy(et[c.np_in[2]]).to(DEV)
+    bias = graphop.rel_bias_forward(*c.inn[:3], etype_slot, q, table)
+    assert bias.shape == (c.E + 1, h) and bias.dtype == torch.float32
+    want = oracle.node_mul_edge_forward(*c.np_in[:3], f64(q), f64(table)[et])
+    close(bias[:c.E], want, TOL[torch.float32] if dtype == torch.float32 else TOL[dtype], "score term")
+    assert float(bias[c.E].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("n_types,n_used", [(1000, 55), (37, 37), (1000, 100), (400, 230), (5, 1)])
+@pytest.mark.parametrize("dtype,h", SHAPES)
+@pytest.mark.parametrize("gname", GRAPH_NAMES)
+def test_score_term_gradients_match_node_mul_edge_backward(ops, gname, dtype, h, n_types, n_used):
+    """dq gains node_mul_edge's dA, dtable is its dB summed per edge type (the embedding's gradient); the counts of used
+    types cover one, two and four wavefronts per workgroup of the kernel."""
+    graphop, _ = ops
+    if (n_types, n_used) in ((1000, 100), (400, 230), (5, 1)) and gname not in ("bpt512_k4", "multigraph"):
+        pytest.skip("the type counts are varied on two graphs")
+    d = 64
+    c = case(gname)
+    q = rand((c.n, h, d), dtype, 21, 0.5).to(DEV)
+    table = rand((n_types, d), dtype, 22, 0.5).to(DEV)
+    ds = torch.cat([rand((c.E, h), torch.float32, 23, 0.1), torch.zeros(1, h)]).to(DEV)     # (E + 1, h) as the fused backward returns it
+    dq0 = rand((c.n, h, d), dtype, 24, 0.5).to(DEV)
+    et = edge_types(c.E, n_types, n_used, 25)
+    etype_slot_np = et[c.np_in[2]]
+    used, nu = used_map(etype_slot_np, n_types)
+    assert nu == min(n_used, c.E)
+    dq = dq0.clone()
+    dtable = graphop.rel_bias_backward(*c.inn[:3], torch.from_numpy(etype_slot_np).to(DEV), torch.from_numpy(used).to(DEV), nu, ds, q, table, dq)
+    dA, dB = oracle.node_mul_edge_backward(*c.np_in[:3], f64(q), f64(table)[et], f64(ds[:c.E]))
+    want_table = np.zeros((n_types, d))
+    np.add.at(want_table, et, dB)
+    # both are raw sums of unnormalised N(0, 0.1) x N(0, 0.5) products: max_deg terms for a row of dq (on top of dq0), h * E / n_used
+    # for a row of the table (terms)
+    close(dq, f64(dq0) + dA, GTOL[dtype], "dq", c.max_deg)
+    close(dtable, want_table, GTOL[dtype], "dtable", h * c.E / max(nu, 1))
+    again = graphop.rel_bias_backward(*c.inn[:3], torch.from_numpy(etype_slot_np).to(DEV), torch.from_numpy(used).to(DEV), nu, ds, q, table,
+                                      dq0.clone())
+    assert torch.equal(again, dtable), "the sums have a fixed order: the same bits every run"
+
+
+def test_too_many_used_types_is_refused_and_the_layer_takes_the_spmm_form(ops):
+    graphop, op = ops
+    h, d, n_types = 8, 64, 1000
+    c = case("bpt512_k4")
+    q, k, v, do = (rand((c.n, h, d), torch.float32, s, 1.0 / 8).to(DEV) for s in (31, 32, 33, 34))
+    table = rand((n_types, d), torch.float32, 35, 1.0 / 8).to(DEV)
+    et = edge_types(c.E, n_types, 300, 36)
+    etype_slot_np = et[c.np_in[2]]
+    used, nu = used_map(etype_slot_np, n_types)
+    assert nu == 300 > graphop.REL_MAX_USED_TYPES
+    ds = torch.zeros(c.E + 1, h, device=DEV)
+    with pytest.raises(RuntimeError, match="status -7"):
+        graphop.rel_bias_backward(*c.inn[:3], torch.from_numpy(etype_slot_np).to(DEV), torch.from_numpy(used).to(DEV), nu, ds, q, table,
+                                  torch.zeros_like(q))
+    from oracle import torch_ops
+    etype = torch.from_numpy(et).to(DEV)
+    for t in (q, k, v, table):
+        t.requires_grad_(True)
+    o = op.bpt_attention(*c.out, *c.inn, q, k, v, rel_table=table, etype=etype)
+    o.backward(do)
+    t64 = lambda x: x.detach().cpu().double()
+    ro, rdq, rdk, rdv, rdak = torch_ops.attention_fwd_bwd(torch.from_numpy(c.src), torch.from_numpy(c.dst), t64(q), t64(k), t64(v), t64(do),
+                                                          ak=t64(table)[etype.cpu()])
+    rdt = torch.zeros(n_types, d, dtype=torch.float64).index_add_(0, etype.cpu(), rdak)
+    close(o, ro.numpy(), TOL[torch.float32], "o")
+    close(q.grad, rdq.numpy(), GTOL[torch.float32], "dq")
+    close(table.grad, rdt.numpy(), GTOL[torch.float32], "dtable", h * c.E / nu)
+
+
+def test_graph_without_edges_gives_a_zero_table_gradient(ops):
+    graphop, _ = ops
+    h, d, n_types = 8, 64, 12
+    i64 = lambda *a: torch.tensor(a, dtype=torch.int64, device=DEV)
+    col, indptr, eid, et = i64(), i64(0), i64(), i64()
+    q = rand((5, h, d), torch.float32, 41).to(DEV)
+    table = rand((n_types, d), torch.float32, 42).to(DEV)
+    dq = torch.ones_like(q)
+    used = torch.full((n_types,), -1, dtype=torch.int32, device=DEV)
+    dtable = graphop.rel_bias_backward(col, indptr, eid, et, used, 0, torch.zeros(1, h, device=DEV), q, table, dq)
+    assert float(dtable.abs().max()) == 0.0 and torch.equal(dq, torch.ones_like(q))
