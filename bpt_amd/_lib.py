@@ -59,9 +59,9 @@ ATTN_API = {
     "bpt_vector_spmm_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_vector_spmm_accumulate": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_vector_spmm_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
-    "bpt_rel_bias_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp] + _tail),
+    "bpt_rel_bias_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_i64, c_vp] + _tail),
     "bpt_rel_bias_backward_workspace_bytes": (c_i64, [_PP, c_i64, ctypes.c_int]),
-    "bpt_rel_bias_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_i64] + _tail),
+    "bpt_rel_bias_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float, ctypes.c_float,
                                             ctypes.c_uint64] + _tail),
     "bpt_attention_forward_noalloc": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, ctypes.c_float, ctypes.c_float,

@@ -2843,59 +2843,75 @@ __device__ __forceinline__ void rel_head_load(const bpt_plan &P, const int4 item
     r.edge = r.b < r.e ? P.eid[slot] : 0;
 }
 
-// bias[eid[p], head] = q[row(p), head, :] . table[idx[p], :] for every slot p of the plan (idx = edge type).  The heads
-// of an item's row are rows of the A operand of v_mfma_f32_16x16x4f32 (row number c of A = head c % H), 16 consecutive
-// slots of the item the 16 columns of B; lane (g, c) holds columns 16 g .. 16 g + 15 of q for head c % H and of the table
-// row of slot c, and receives the results of heads 4 g .. 4 g + 3 for slot c, which it stores as one vector where
-// 4 g < H.  Each wavefront takes the items gw, gw + GW, ... and keeps their loads ahead of their use in three steps
-// (descriptor; types and edge ids of the first 64 slots; the q row and the table rows of the first 16 slots), each one
-// item further ahead than the one that needs its result; within an item the table rows of the next 16 slots are in
-// flight during the products.
+// The rows of the table that a graph uses, as floats in LDS: row u (`pitch` floats apart) = table[used_types[u]].  All
+// threads of the workgroup.
+template <typename T>
+__device__ __forceinline__ void rel_table_to_lds(const T *__restrict__ table, const int32_t *__restrict__ used_types, int n_used, float *lds,
+                                                 int pitch) {
+    for (int x = threadIdx.x; x < n_used * 16; x += blockDim.x) {
+        const int u = x >> 4, c4 = (x & 15) * 4;
+        *reinterpret_cast<float4 *>(lds + u * pitch + c4) = load4<T>(table + (size_t)used_types[u] * 64 + c4);
+    }
+}
+
+// bias[eid[p], head] = q[row(p), head, :] . table[used_types[idx[p]], :] for every slot p of the plan (idx = the number of
+// the edge's type among the n_used types that occur).  The heads of an item's row are rows of the A operand of
+// v_mfma_f32_16x16x4f32 (row number c of A = head c % H), 16 consecutive slots of the item the 16 columns of B; lane
+// (g, c) holds columns 16 g .. 16 g + 15 of q for head c % H and of the table row of slot c, and receives the results of
+// heads 4 g .. 4 g + 3 for slot c, which it stores as one vector where 4 g < H.  The table rows come from a copy in LDS
+// (rows REL_LDS_PITCH floats apart, so that the 16 rows of an operand fall into different banks): fetched from memory
+// block by block they would cost one round trip each, far longer than a block's products.  A wavefront takes
+// REL_FWD_ITEMS work items and fetches for all of them at once first the items, then their q rows and the type numbers
+// and edge ids of their first 64 slots.
+constexpr int REL_FWD_ITEMS = 4, REL_LDS_PITCH = 68;
 template <typename T, int H>
-__global__ __launch_bounds__(BLOCK) void k_rel_bias_rows(bpt_plan P, const T *__restrict__ q, const T *__restrict__ table, float *__restrict__ bias) {
-    constexpr int D = 64;
+__global__ __launch_bounds__(BLOCK) void k_rel_bias_rows(bpt_plan P, const T *__restrict__ q, const T *__restrict__ table,
+                                                         const int32_t *__restrict__ used_types, int n_used, float *__restrict__ bias) {
+    constexpr int D = 64, K = REL_FWD_ITEMS;
     static_assert(H == 4 || H == 8 || H == 16, "four consecutive heads per lane");
+    extern __shared__ float rel_lds[];
     const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
-    const int GW = (int)gridDim.x * WAVES_PER_BLOCK, i_begin = (int)blockIdx.x * WAVES_PER_BLOCK + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int i_end = (int)P.n_items;
+    // wavefront gw of GW takes the items gw, gw + GW, ...: the segments of a long row, which are neighbours and all full, go to
+    // different wavefronts
+    const int GW = (int)gridDim.x * WAVES_PER_BLOCK, i0 = (int)blockIdx.x * WAVES_PER_BLOCK + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int n_items = (int)P.n_items;
     const int4 *items = reinterpret_cast<const int4 *>(P.items);
-    const int4 none = make_int4(0, 0, 0, -1);
-    struct Body { float aq[16], bt[16]; };
-    auto body_load = [&](const RelHead &r, Body &y) {
-        rel_load16<T>(q + ((size_t)r.row * H + (c % H)) * D + 16 * g, y.aq);
-        rel_load16<T>(table + (size_t)lane_bcast(r.type, c) * D + 16 * g, y.bt);
-    };
-    RelHead hd, hd_next;
-    Body bd, bd_next;
-    rel_head_load(P, i_begin < i_end ? items[i_begin] : none, lane, hd_next);
-    body_load(hd_next, bd_next);
-    hd = hd_next;
-    rel_head_load(P, i_begin + GW < i_end ? items[i_begin + GW] : none, lane, hd_next);
-    int4 desc = i_begin + 2 * GW < i_end ? items[i_begin + 2 * GW] : none;
-    for (int i = i_begin; i < i_end; i += GW) {
-        bd = bd_next;
-        body_load(hd_next, bd_next);                     // the item after this one
-        const RelHead cur = hd;
-        hd = hd_next;
-        rel_head_load(P, desc, lane, hd_next);           // the second after
-        desc = i + 3 * GW < i_end ? items[i + 3 * GW] : none;
-        for (int p0 = cur.b; p0 < cur.e; p0 += WAVE) {
-            const int cnt = min(WAVE, cur.e - p0);
-            int type = cur.type, edge = cur.edge;
-            float bt[2][16];
-            if (p0 == cur.b) {
+    int4 desc[K];
 #pragma unroll
-                for (int t = 0; t < 16; ++t) bt[0][t] = bd.bt[t];
-            } else {                                     // (items longer than 64 slots: the rest, fetched on the spot)
+    for (int k = 0; k < K; ++k) desc[k] = items[min(i0 + k * GW, n_items - 1)];
+    rel_table_to_lds<T>(table, used_types, n_used, rel_lds, REL_LDS_PITCH);
+    RelHead hd[K];
+    float aq[K][16];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        if (i0 + k * GW >= n_items) desc[k].z = desc[k].y;  // (past the last item: nothing to do)
+        rel_head_load(P, desc[k], lane, hd[k]);
+        rel_load16<T>(q + ((size_t)hd[k].row * H + (c % H)) * D + 16 * g, aq[k]);
+    }
+    __syncthreads();
+    auto table_rows = [&](int type, int first, float (&bt)[16]) {          // of the 16 slots from `first` of a chunk (lane l: slot l)
+        const float *row = rel_lds + lane_bcast(type, first + c) * REL_LDS_PITCH + 16 * g;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float4 x = *reinterpret_cast<const float4 *>(row + 4 * t);
+            bt[4 * t] = x.x; bt[4 * t + 1] = x.y; bt[4 * t + 2] = x.z; bt[4 * t + 3] = x.w;
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        for (int p0 = hd[k].b; p0 < hd[k].e; p0 += WAVE) {
+            const int cnt = min(WAVE, hd[k].e - p0);
+            int type = hd[k].type, edge = hd[k].edge;
+            if (p0 != hd[k].b) {                             // (items longer than 64 slots: the rest, fetched on the spot)
                 const int slot = p0 + min(lane, cnt - 1);
                 type = P.idx[slot]; edge = P.eid[slot];
-                rel_load16<T>(table + (size_t)lane_bcast(type, c) * D + 16 * g, bt[0]);
             }
 #pragma unroll
             for (int blk = 0; blk < 4; ++blk) {
                 if (16 * blk < cnt) {
-                    if (16 * (blk + 1) < cnt) rel_load16<T>(table + (size_t)lane_bcast(type, 16 * (blk + 1) + c) * D + 16 * g, bt[(blk + 1) & 1]);
-                    const floatx4v acc = tile_dot(bd.aq, bt[blk & 1]);
+                    float bt[16];
+                    table_rows(type, 16 * blk, bt);
+                    const floatx4v acc = tile_dot(aq[k], bt);
                     const int e = lane_bcast(edge, 16 * blk + c);
                     if (16 * blk + c < cnt && 4 * g < H)
                         *reinterpret_cast<float4 *>(bias + (size_t)e * H + 4 * g) = make_float4(acc[0], acc[1], acc[2], acc[3]);
@@ -2906,25 +2922,23 @@ __global__ __launch_bounds__(BLOCK) void k_rel_bias_rows(bpt_plan P, const T *__
 }
 
 // Gradients of that term from ds[e, head] = dL/d(score of edge e before scaling): dq[row] += sum over the row's slots of
-// ds[eid] * table[type] (all heads), and the table's gradient dtable[t] = sum over the slots of type t and the heads of
-// ds[eid, head] * q[row, head].  Lane l owns column l.  Each wavefront walks every GW-th of the plan's work items (rows
-// and segments of long rows; a segment's part of dq goes to the workspace slot of the item, which k_combine_sum_v4
-// adds to dq) and keeps its own sums per edge type in LDS (used[type] = the type's number among the n_used types
-// that occur); the wavefronts of a workgroup add theirs in a fixed order and the workgroup writes one partial table,
-// part[(u * gridDim.x + block) * 64 + column], which k_rel_table_sum adds up.  Every sum has one owner and a fixed order.
-// The loads of an item run ahead of its use in three steps (descriptor; types and edge ids of its first 64 slots; their ds
-// values and numbers and the item's q and dq rows), each one item further ahead than the one that needs its result.
+// ds[eid] * table row of the slot's type (all heads), and the table's gradient, for type number u, the sum over the slots
+// with idx = u and the heads of ds[eid, head] * q[row, head].  Lane l owns column l.  Each wavefront walks every GW-th of
+// the plan's work items (rows and segments of long rows; a segment's part of dq goes to the workspace slot of the item,
+// which k_combine_sum_v4 adds to dq) and keeps its own sums per type number in LDS, beside the workgroup's copy of the
+// table rows in use; the wavefronts of a workgroup add theirs in a fixed order and the workgroup writes one partial
+// table, part[(u * gridDim.x + block) * 64 + column], which k_rel_table_sum adds up.  Every sum has one owner and a fixed
+// order.  The loads of an item run ahead of its use in three steps (descriptor; type numbers and edge ids of its first 64
+// slots; their ds values and the item's q and dq rows), each one item further ahead than the one that needs its result.
 template <int H>
-struct RelBody {             // what the walk of those slots needs: per lane the type's number and the ds values of its slot;
-    int u;                   // the item's q row and, for a whole row, the dq row it adds to (lane l: column l)
-    float dsv[H];
+struct RelBody {             // what the walk of those slots needs: per lane the ds values of its slot; the item's q row
+    float dsv[H];            // and, for a whole row, the dq row it adds to (lane l: column l)
     float qh[H], old[H];
 };
 template <typename T, int H>
 __device__ __forceinline__ void rel_body_load(const RelHead &r, const float *__restrict__ ds, const T *__restrict__ q, const T *__restrict__ dq,
-                                              const int32_t *__restrict__ used, int lane, RelBody<H> &y) {
+                                              int lane, RelBody<H> &y) {
     constexpr int D = 64;
-    y.u = used[r.type];
 #pragma unroll
     for (int h = 0; h < H; h += 4) {
         const float4 x = *reinterpret_cast<const float4 *>(ds + (size_t)r.edge * H + h);
@@ -2938,14 +2952,16 @@ __device__ __forceinline__ void rel_body_load(const RelHead &r, const float *__r
 }
 template <typename T, int H, int NW>
 __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const float *__restrict__ ds, const T *__restrict__ q,
-                                                            const T *__restrict__ table, const int32_t *__restrict__ used, int n_used,
+                                                            const T *__restrict__ table, const int32_t *__restrict__ used_types, int n_used,
                                                             T *__restrict__ dq, float *__restrict__ ws_dq, float *__restrict__ part) {
     constexpr int D = 64, C = H * D, AHEAD = H >= 16 ? 4 : 8;
-    extern __shared__ float rel_lds[];                    // NW tables of n_used x 64 sums, then NW x 64 x H staged ds values
+    extern __shared__ float rel_lds[];                    // NW tables of n_used x 64 sums, the table rows in use, NW x 64 x H staged ds values
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     float *acc = rel_lds + (size_t)w * n_used * D;
-    float *stage = rel_lds + (size_t)NW * n_used * D + (size_t)w * WAVE * H;
+    const float *rows = rel_lds + (size_t)NW * n_used * D;
+    float *stage = rel_lds + (size_t)(NW + 1) * n_used * D + (size_t)w * WAVE * H;
     for (int u = 0; u < n_used; ++u) acc[u * D + lane] = 0.f;
+    rel_table_to_lds<T>(table, used_types, n_used, rel_lds + (size_t)NW * n_used * D, D);
     // wavefront gw of GW takes the items gw, gw + GW, ...: the segments of a long row, which are neighbours, go to different wavefronts
     const int GW = (int)gridDim.x * NW, i_begin = (int)blockIdx.x * NW + w, i_end = (int)P.n_items;
     const int4 *items = reinterpret_cast<const int4 *>(P.items);
@@ -2953,23 +2969,20 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
     RelHead hd, hd_next;
     RelBody<H> bd, bd_next;
     rel_head_load(P, i_begin < i_end ? items[i_begin] : none, lane, hd_next);
-    rel_body_load<T, H>(hd_next, ds, q, dq, used, lane, bd_next);
+    rel_body_load<T, H>(hd_next, ds, q, dq, lane, bd_next);
     hd = hd_next;
     rel_head_load(P, i_begin + GW < i_end ? items[i_begin + GW] : none, lane, hd_next);
     int4 desc = i_begin + 2 * GW < i_end ? items[i_begin + 2 * GW] : none;
-    // one chunk of at most 64 slots whose ds values are staged: lane j of (type, u) belongs to slot j of the chunk
-    auto walk = [&](int cnt, int type, int u, const float (&qh)[H], float (&dqa)[H]) {
+    __syncthreads();
+    // one chunk of at most 64 slots whose ds values are staged: lane j of u (type numbers) belongs to slot j of the chunk
+    auto walk = [&](int cnt, int u, const float (&qh)[H], float (&dqa)[H]) {
         wave_lds_fence();
-        float tv[2][AHEAD];                               // this lane's column of the table rows of AHEAD slots, fetched together
-        auto fetch = [&](int j0, float (&t)[AHEAD]) {
-#pragma unroll
-            for (int x = 0; x < AHEAD; ++x) t[x] = Elem<T>::ld(table + (size_t)__builtin_amdgcn_readlane(type, min(j0 + x, cnt - 1)) * D + lane);
-        };
-        auto use = [&](int j0, const float (&t)[AHEAD]) {
-            // the ds values of the AHEAD slots first (zeros are staged for the slots past the chunk's end, which so add nothing),
-            // then four slots at a time: the sums so far, the products, the new sums.  The reads of the sums
-            // come before the products so that their latency is covered; where slots of a four have the same type, the
-            // later one's sum takes the earlier ones' terms in slot order, as if the four were added one after the other.
+        for (int j0 = 0; j0 < cnt; j0 += AHEAD) {
+            // the ds values of AHEAD slots first (zeros are staged for the slots past the chunk's end, which so add nothing),
+            // then four slots at a time: the sums so far and the table rows, the products, the new sums.  The reads of
+            // the sums come before the products so that their latency is covered; where slots of a four have the same
+            // type, the later one's sum takes the earlier ones' terms in slot order, as if the four were added one
+            // after the other.
             float4 dv[AHEAD][H / 4];
 #pragma unroll
             for (int x = 0; x < AHEAD; ++x)
@@ -2979,25 +2992,23 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
             for (int x0 = 0; x0 < AHEAD; x0 += 4) {
                 if (j0 + x0 < cnt) {
                     int un[4];
-                    float *sum[4];
-                    float before[4], gsum[4];
+                    float before[4], gsum[4], tv[4];
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
                         un[x] = __builtin_amdgcn_readlane(u, min(j0 + x0 + x, cnt - 1));
-                        sum[x] = acc + un[x] * D + lane;
-                        before[x] = *sum[x];
+                        before[x] = acc[un[x] * D + lane];
+                        tv[x] = rows[un[x] * D + lane];
                     }
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        const float tx = t[x0 + x];
                         gsum[x] = 0.f;
 #pragma unroll
                         for (int h = 0; h < H; h += 4) {
                             const float4 d4 = dv[x0 + x][h / 4];
                             gsum[x] = fmaf(d4.x, qh[h], gsum[x]); gsum[x] = fmaf(d4.y, qh[h + 1], gsum[x]);
                             gsum[x] = fmaf(d4.z, qh[h + 2], gsum[x]); gsum[x] = fmaf(d4.w, qh[h + 3], gsum[x]);
-                            dqa[h] = fmaf(d4.x, tx, dqa[h]); dqa[h + 1] = fmaf(d4.y, tx, dqa[h + 1]);
-                            dqa[h + 2] = fmaf(d4.z, tx, dqa[h + 2]); dqa[h + 3] = fmaf(d4.w, tx, dqa[h + 3]);
+                            dqa[h] = fmaf(d4.x, tv[x], dqa[h]); dqa[h + 1] = fmaf(d4.y, tv[x], dqa[h + 1]);
+                            dqa[h + 2] = fmaf(d4.z, tv[x], dqa[h + 2]); dqa[h + 3] = fmaf(d4.w, tv[x], dqa[h + 3]);
                         }
                     }
 #pragma unroll
@@ -3005,23 +3016,16 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
                         float v = before[x];
 #pragma unroll
                         for (int y = 0; y < x; ++y) v += un[y] == un[x] ? gsum[y] : 0.f;
-                        *sum[x] = v + gsum[x];
+                        acc[un[x] * D + lane] = v + gsum[x];
                     }
                 }
             }
-        };
-        fetch(0, tv[0]);
-        for (int j0 = 0; j0 < cnt; j0 += 2 * AHEAD) {
-            fetch(j0 + AHEAD, tv[1]);
-            use(j0, tv[0]);
-            fetch(j0 + 2 * AHEAD, tv[0]);
-            use(j0 + AHEAD, tv[1]);
         }
         wave_lds_fence();
     };
     for (int i = i_begin; i < i_end; i += GW) {
         bd = bd_next;
-        rel_body_load<T, H>(hd_next, ds, q, dq, used, lane, bd_next);          // the item after this one
+        rel_body_load<T, H>(hd_next, ds, q, dq, lane, bd_next);                // the item after this one
         const RelHead cur = hd;
         hd = hd_next;
         rel_head_load(P, desc, lane, hd_next);                                   // the second after
@@ -3034,17 +3038,17 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
             for (int h = 0; h < H; h += 4)
                 *reinterpret_cast<float4 *>(stage + lane * H + h) =
                     lane < cur.e - cur.b ? make_float4(bd.dsv[h], bd.dsv[h + 1], bd.dsv[h + 2], bd.dsv[h + 3]) : make_float4(0.f, 0.f, 0.f, 0.f);
-            walk(min(WAVE, cur.e - cur.b), cur.type, bd.u, bd.qh, dqa);
+            walk(min(WAVE, cur.e - cur.b), cur.type, bd.qh, dqa);
         }
         for (int p0 = cur.b + WAVE; p0 < cur.e; p0 += WAVE) {                  // (items longer than 64 slots: the rest, fetched on the spot)
             const int cnt = min(WAVE, cur.e - p0);
             const int slot = p0 + min(lane, cnt - 1);
-            const int type = P.idx[slot], edge = P.eid[slot];
+            const int u = P.idx[slot], edge = P.eid[slot];
 #pragma unroll
             for (int h = 0; h < H; h += 4)
                 *reinterpret_cast<float4 *>(stage + lane * H + h) =
                     lane < cnt ? *reinterpret_cast<const float4 *>(ds + (size_t)edge * H + h) : make_float4(0.f, 0.f, 0.f, 0.f);
-            walk(cnt, type, used[type], bd.qh, dqa);
+            walk(cnt, u, bd.qh, dqa);
         }
         if (cur.out_slot < 0) {
             if (cur.b < cur.e) {
@@ -3298,28 +3302,54 @@ inline bool rel_rows_shape(int h, int d, int dtype) {
     return !g_force_generic.load(std::memory_order_relaxed) && d == 64 && (h == 4 || h == 8 || h == 16) && (dtype == BPT_F32 || dtype == BPT_BF16);
 }
 
-constexpr int REL_FWD_MAX_BLOCKS = 256 * 5;   // workgroups of four wavefronts: five wavefronts per SIMD of 256 compute units
 constexpr int REL_MAX_PARTS = 512;        // partial tables of the gradient kernel: two workgroups per compute unit
+constexpr int REL_MAX_USED = 240;         // type numbers whose table rows fit the 64 KB of LDS of the score kernel
 
-// wavefronts per workgroup of k_rel_bias_bwd for n_used types (0: too many for the 64 KB of LDS a workgroup may take)
+// LDS of k_rel_bias_bwd with nw wavefronts: their sums, the table rows, their staged ds values
+inline size_t rel_bwd_lds(int nw, int64_t n_used, int h) { return ((size_t)(nw + 1) * n_used * 64 + (size_t)nw * WAVE * h) * 4; }
+// wavefronts per workgroup of k_rel_bias_bwd for n_used types: four or two while two workgroups fit a compute unit's
+// 160 KB of LDS, else one
 inline int rel_bwd_waves(int64_t n_used, int h) {
-    for (int nw = 4; nw >= 1; nw >>= 1)
-        if ((int64_t)nw * (n_used * 64 + WAVE * h) * 4 <= 65536) return nw;
-    return 0;
+    for (int nw = 4; nw >= 2; nw >>= 1)
+        if (rel_bwd_lds(nw, n_used, h) <= 80 * 1024) return nw;
+    return rel_bwd_lds(1, n_used, h) <= 128 * 1024 ? 1 : 0;
+}
+
+// a kernel may take more than 64 KB of dynamic LDS only after it has been told so (once per kernel and device)
+template <typename K>
+int allow_large_lds(K kernel, size_t bytes) {
+    static std::atomic<uint32_t> done{0};
+    if (bytes <= 64 * 1024) return BPT_OK;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32) return BPT_ERR_UNSUPPORTED;
+    if (done.load(std::memory_order_acquire) & (1u << dev)) return BPT_OK;
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return (int)e;
+    done.fetch_or(1u << dev, std::memory_order_release);
+    return BPT_OK;
+}
+
+template <typename T, int H, int NW>
+int launch_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const void *table, const int32_t *used_types, int64_t n_used,
+                        void *dq, float *ws_dq, float *part, int n_parts, hipStream_t s) {
+    const size_t lds = rel_bwd_lds(NW, n_used, H);
+    const int st = allow_large_lds(k_rel_bias_bwd<T, H, NW>, lds);
+    if (st != BPT_OK) return st;
+    hipLaunchKernelGGL((k_rel_bias_bwd<T, H, NW>), dim3(n_parts), dim3(NW * WAVE), lds, s, *P, ds, (const T *)q, (const T *)table, used_types,
+                       (int)n_used, (T *)dq, ws_dq, part);
+    return launch_status();
 }
 
 template <typename T, int H>
-int run_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const void *table, const int32_t *used, int64_t n_types, int64_t n_used,
-                     void *dq, void *dtable, float *ws, hipStream_t s) {
+int run_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const void *table, const int32_t *used, const int32_t *used_types,
+                     int64_t n_types, int64_t n_used, void *dq, void *dtable, float *ws, hipStream_t s) {
     const int nw = rel_bwd_waves(n_used, H);
     const int n_parts = (int)std::min<int64_t>(REL_MAX_PARTS, std::max<int64_t>(1, (P->n_edges + nw * 128 - 1) / (nw * 128)));
-    const size_t lds = (size_t)nw * ((size_t)n_used * 64 + WAVE * H) * 4;
     float *ws_dq = ws, *part = ws + (size_t)P->n_slots * H * 64;       // partial rows of dq of the split rows, then the partial tables
-#define L(NW) hipLaunchKernelGGL((k_rel_bias_bwd<T, H, NW>), dim3(n_parts), dim3(NW * WAVE), lds, s, *P, ds, (const T *)q, (const T *)table, used, \
-                                 (int)n_used, (T *)dq, ws_dq, part)
     if (P->n_edges > 0) {
-        if (nw == 4) L(4); else if (nw == 2) L(2); else L(1);
-        int st = launch_status();
+        int st = nw == 4   ? launch_rel_bias_bwd<T, H, 4>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s)
+                 : nw == 2 ? launch_rel_bias_bwd<T, H, 2>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s)
+                           : launch_rel_bias_bwd<T, H, 1>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s);
         if (st != BPT_OK) return st;
         if (P->n_heavy > 0) {
             hipLaunchKernelGGL((k_combine_sum_v4<T>), dim3((unsigned)P->n_heavy, H * 64 / 256, 1), dim3(BLOCK), 0, s, P->heavy, ws_dq, (T *)dq,
@@ -3328,23 +3358,24 @@ int run_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const vo
             if (st != BPT_OK) return st;
         }
     }
-#undef L
     // (without edges there are no partial tables: every row of dtable becomes zero)
     hipLaunchKernelGGL((k_rel_table_sum<T>), dim3((unsigned)n_types), dim3(BLOCK), 0, s, part, used, P->n_edges > 0 ? n_parts : 0, (T *)dtable);
+    return launch_status();
+}
+
+// the score term with the table rows in LDS: plan indices are type numbers
+template <typename T, int H>
+int run_rel_bias_rows(const bpt_plan *P, const void *q, const void *table, const int32_t *used_types, int64_t n_used, float *bias, hipStream_t s) {
+    if (P->n_items == 0) return BPT_OK;
+    const int64_t waves = (P->n_items + REL_FWD_ITEMS - 1) / REL_FWD_ITEMS;
+    hipLaunchKernelGGL((k_rel_bias_rows<T, H>), dim3((unsigned)((waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK)), dim3(BLOCK),
+                       (size_t)n_used * REL_LDS_PITCH * 4, s, *P, (const T *)q, (const T *)table, used_types, (int)n_used, bias);
     return launch_status();
 }
 
 template <typename T, int H, int D>
 int run_rel_bias(const bpt_plan *P, const void *A, const void *table, float *bias, hipStream_t s) {
     if (P->n_items == 0) return BPT_OK;
-    if constexpr (D == 64 && (H == 4 || H == 8 || H == 16)) {
-        if (!g_force_generic.load(std::memory_order_relaxed) && aligned16(bias)) {      // rows on the matrix cores
-            // a wavefront per work item up to the number the GPU holds at once (five per SIMD), several items per wavefront beyond
-            const int blocks = (int)std::min<int64_t>(grid_for(P), REL_FWD_MAX_BLOCKS);
-            hipLaunchKernelGGL((k_rel_bias_rows<T, H>), dim3(blocks), dim3(BLOCK), 0, s, *P, (const T *)A, (const T *)table, bias);
-            return launch_status();
-        }
-    }
     if (spmm_grp_ok(P, H, D, sizeof(T) == 2 ? BPT_BF16 : BPT_F32)) {      // row groups: one load of a table row per group entry
         constexpr int HS = head_slices<T, H, D>();
         if (P->grp_R == 8)
@@ -3909,12 +3940,22 @@ int bpt_maskedmm_csr_backward(const bpt_plan *plan_r, const bpt_plan *plan_c, co
     return spmm(plan_c, dy, A, dB, workspace, h, d, dtype, (hipStream_t)stream);
 }
 
-int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, float *bias, int h, int d, int dtype, void *stream) {
+int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, const int32_t *used_types, int64_t n_used, float *bias, int h,
+                         int d, int dtype, void *stream) {
     CHECK(check_plan(plan, true));
     CHECK(check_shape(h, d, dtype));
     if (plan->n_edges > 0 && (!q || !table || !bias)) return BPT_ERR_NULL;
-    if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(table)) return BPT_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
+    if (used_types) {                       // plan indices are type numbers: the kernel with the table rows in LDS
+        if (n_used < 0) return BPT_ERR_SIZE;
+        if (!rel_rows_shape(h, d, dtype) || n_used > REL_MAX_USED || !aligned16(q) || !aligned16(table) || !aligned16(bias)) return BPT_ERR_UNSUPPORTED;
+#define X(HH) if (h == HH) return run_rel_bias_rows<T, HH>(plan, q, table, used_types, n_used, bias, s);
+        if (dtype == BPT_F32) { using T = float; X(4) X(8) X(16) }
+        if (dtype == BPT_BF16) { using T = bf16_t; X(4) X(8) X(16) }
+#undef X
+        return BPT_ERR_UNSUPPORTED;
+    }
+    if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(table)) return BPT_ERR_UNSUPPORTED;
 #define X(HH, DD) if (h == HH && d == DD) return run_rel_bias<T, HH, DD>(plan, q, table, bias, s);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
@@ -3927,19 +3968,19 @@ int64_t bpt_rel_bias_backward_workspace_bytes(const bpt_plan *plan, int64_t n_us
     return (plan->n_slots * h * 64 + n_used * REL_MAX_PARTS * 64) * 4;
 }
 
-int bpt_rel_bias_backward(const bpt_plan *plan, const float *ds, const void *q, const void *table, const int32_t *used, int64_t n_types,
-                          int64_t n_used, void *dq, void *dtable, void *workspace, int64_t workspace_bytes, int h, int d, int dtype,
-                          void *stream) {
+int bpt_rel_bias_backward(const bpt_plan *plan, const float *ds, const void *q, const void *table, const int32_t *used,
+                          const int32_t *used_types, int64_t n_types, int64_t n_used, void *dq, void *dtable, void *workspace,
+                          int64_t workspace_bytes, int h, int d, int dtype, void *stream) {
     CHECK(check_plan(plan, true));
     CHECK(check_shape(h, d, dtype));
     if (n_types < 0 || n_used < 0 || n_used > n_types) return BPT_ERR_SIZE;
-    if (!rel_rows_shape(h, d, dtype) || rel_bwd_waves(n_used, h) == 0) return BPT_ERR_UNSUPPORTED;
+    if (!rel_rows_shape(h, d, dtype) || n_used > REL_MAX_USED || rel_bwd_waves(n_used, h) == 0) return BPT_ERR_UNSUPPORTED;
     if (n_types == 0) return BPT_OK;
-    if (!used || !dtable || (plan->n_edges > 0 && (!ds || !q || !table || !dq))) return BPT_ERR_NULL;
-    if (!aligned16(ds)) return BPT_ERR_UNSUPPORTED;
+    if (!used || !dtable || (n_used > 0 && !used_types) || (plan->n_edges > 0 && (!ds || !q || !table || !dq))) return BPT_ERR_NULL;
+    if (!aligned16(ds) || !aligned16(table)) return BPT_ERR_UNSUPPORTED;
     if (!workspace || workspace_bytes < bpt_rel_bias_backward_workspace_bytes(plan, n_used, h) || !aligned16(workspace)) return BPT_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
-#define X(HH) if (h == HH) return run_rel_bias_bwd<T, HH>(plan, ds, q, table, used, n_types, n_used, dq, dtable, (float *)workspace, s);
+#define X(HH) if (h == HH) return run_rel_bias_bwd<T, HH>(plan, ds, q, table, used, used_types, n_types, n_used, dq, dtable, (float *)workspace, s);
     if (dtype == BPT_F32) { using T = float; X(4) X(8) X(16) }
     if (dtype == BPT_BF16) { using T = bf16_t; X(4) X(8) X(16) }
 #undef X

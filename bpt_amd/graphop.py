@@ -350,63 +350,76 @@ def attention_supported(q):
     return q.dim() == 3 and (h, d) in fast.get(q.dtype, ())
 
 
-def rel_bias_forward(col, indptr_c, eid_c, etype_slot, q, table):
+def rel_bias_forward(col, indptr_c, eid_c, type_slot, q, table, used_types=None):
     """The rel_pos score term of modules/attention.py:69-71 without the (E, d) embedding rows:
-    bias[eid_c[p], head] = q[row(p), head, :] . table[etype_slot[p], :], where etype_slot[p] is the type of the edge
-    in slot p of the in-CSR (etype[eid_c]).  Returns float32 (E + 1, h); the last row is a zero spare row that the
-    fused kernels read for absent pairs."""
+    bias[eid_c[p], head] = q[row(p), head, :] . table[type(p), :] for every slot p of the in-CSR.  Returns float32
+    (E + 1, h); the last row is a zero spare row that the fused kernels read for absent pairs.
+    used_types None: type_slot[p] is the type of the edge in slot p (etype[eid_c]).
+    used_types (n_used,) int32, the types that occur: type_slot[p] is the NUMBER of the slot's type in that list; takes the
+    kernel that keeps those table rows on chip (needs rel_rows_supported(q) and n_used <= REL_MAX_USED_TYPES)."""
     cfg = _SETTINGS
-    _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, etype_slot=etype_slot, q=q, table=table)
+    _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, type_slot=type_slot, q=q, table=table)
     _same_dtype(q, table)
     h, d = _hd(q)
     if table.dim() != 2 or table.size(1) != d:
         raise ValueError(f"table must be (n_types, {d})")
-    _expect_index(eid_c, etype_slot)
-    plan = plan_cache.get(col, indptr_c, eid_c, etype_slot, q.size(0), table.size(0))
+    _expect_index(eid_c, type_slot)
     E = eid_c.size(0)
+    if used_types is not None:
+        _check_input(used_types, "used_types")
+        if used_types.dtype != torch.int32 or used_types.dim() != 1 or used_types.numel() > table.size(0):
+            raise ValueError("used_types must be a 1-D int32 tensor of at most table.size(0) elements")
+        plan = plan_cache.get(col, indptr_c, eid_c, type_slot, q.size(0), max(used_types.numel(), 1))
+        ref, n_used = plan.ref, used_types.numel()
+    else:
+        plan = plan_cache.get(col, indptr_c, eid_c, type_slot, q.size(0), table.size(0))
+        ref, n_used = _spmm_ref(plan, q, h, d, cfg), 0
     bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
     bias[E].zero_()
     with torch.cuda.device_of(q):
-        ref = plan.ref if rel_rows_supported(q) else _spmm_ref(plan, q, h, d, cfg)      # the row kernel walks the plain CSR
-        check_attn(_LIB.bpt_rel_bias_forward(ref, _ptr(q), _ptr(table), _ptr(bias), h, d, _dtype(q), _stream()), "rel_bias_forward")
+        check_attn(_LIB.bpt_rel_bias_forward(ref, _ptr(q), _ptr(table), _ptr(used_types) if used_types is not None else None, n_used,
+                                             _ptr(bias), h, d, _dtype(q), _stream()), "rel_bias_forward")
     return bias
 
 
-REL_MAX_USED_TYPES = 240      # edge types that may occur in one graph for rel_bias_backward (the kernel's on-chip sums)
+REL_MAX_USED_TYPES = 240      # edge types that may occur in one graph for the kernels that keep their table rows on chip
 
 
 def rel_rows_supported(q):
-    """True if the rel_pos term of q's (h, d, dtype) has the kernels that walk the plain CSR of the destinations."""
+    """True if the rel_pos term of q's (h, d, dtype) has the kernels that keep the table rows in use on chip."""
     h, d = _hd(q)
     return q.dim() == 3 and d == 64 and h in (4, 8, 16) and q.dtype in (torch.float32, torch.bfloat16)
 
 
-def rel_bias_backward(col, indptr_c, eid_c, etype_slot, used, n_used, ds, q, table, dq):
+def rel_bias_backward(col, indptr_c, eid_c, number_slot, used, used_types, ds, q, table, dq):
     """Gradients of the rel_pos score term (modules/attention.py:55-56,69-71: autograd of nn.Embedding and of
     node_mul_edge) from ds (E or more rows, h) float32 = dL/d(score before scaling) per edge and head:
-    dq[row] += sum_p ds[eid_c[p]] * table[etype_slot[p]] in place, and returns dtable (n_types, d) with
-    dtable[t] = sum over the slots of type t and the heads of ds * q[row].  used (n_types,) int32: the number of every
-    type that occurs among the n_used of them, -1 for the others.  Raises if rel_rows_supported(q) is False or
-    n_used > REL_MAX_USED_TYPES."""
-    _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, etype_slot=etype_slot, used=used, ds=ds, q=q, table=table, dq=dq)
+    dq[row] += sum_p ds[eid_c[p]] * table[type(p)] in place, and returns dtable (n_types, d) with
+    dtable[t] = sum over the slots of type t and the heads of ds * q[row].  used_types (n_used,) int32: the types that
+    occur; number_slot[p]: the number of slot p's type in that list; used (n_types,) int32: the number of every type
+    in the list, -1 for the others.  Raises if rel_rows_supported(q) is False or n_used > REL_MAX_USED_TYPES."""
+    _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, number_slot=number_slot, used=used, used_types=used_types, ds=ds, q=q, table=table, dq=dq)
     _same_dtype(q, table, dq)
     h, d = _hd(q)
     if table.dim() != 2 or table.size(1) != d:
         raise ValueError(f"table must be (n_types, {d})")
     if used.dtype != torch.int32 or used.numel() != table.size(0):
         raise ValueError("used must be int32 with one element per table row")
+    if used_types.dtype != torch.int32 or used_types.dim() != 1 or used_types.numel() > table.size(0):
+        raise ValueError("used_types must be a 1-D int32 tensor of at most table.size(0) elements")
     if ds.dtype != torch.float32 or ds.dim() != 2 or ds.size(1) != h or ds.size(0) < eid_c.size(0):
         raise ValueError(f"ds must be float32 (>= {eid_c.size(0)}, {h})")
     if dq.shape != q.shape:
         raise ValueError("dq must have the shape of q")
-    _expect_index(eid_c, etype_slot)
-    plan = plan_cache.get(col, indptr_c, eid_c, etype_slot, q.size(0), table.size(0))
+    _expect_index(eid_c, number_slot)
+    n_used = used_types.numel()
+    plan = plan_cache.get(col, indptr_c, eid_c, number_slot, q.size(0), max(n_used, 1))
     dtable = torch.empty_like(table)
     with torch.cuda.device_of(q):
-        nws = int(_LIB.bpt_rel_bias_backward_workspace_bytes(plan.ref, int(n_used), h))
+        nws = int(_LIB.bpt_rel_bias_backward_workspace_bytes(plan.ref, n_used, h))
         ws = _scratch(max(nws, 16), q.device)
-        check_attn(_LIB.bpt_rel_bias_backward(plan.ref, _ptr(ds), _ptr(q), _ptr(table), _ptr(used), table.size(0), int(n_used), _ptr(dq),
-                                              _ptr(dtable), _ptr(ws), nws, h, d, _dtype(q), _stream()), "rel_bias_backward")
+        check_attn(_LIB.bpt_rel_bias_backward(plan.ref, _ptr(ds), _ptr(q), _ptr(table), _ptr(used), _ptr(used_types), table.size(0), n_used,
+                                              _ptr(dq), _ptr(dtable), _ptr(ws), nws, h, d, _dtype(q), _stream()), "rel_bias_backward")
     return dtable
 
 

@@ -107,7 +107,11 @@ class BPTRelAttention(Function):
                 table, etype):
         aux = _rel_aux(etype, col, indptr_c, eid_c, table.size(0))
         table = table.contiguous()
-        bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["etype_slot"], q, table)
+        ctx.on_chip = _g.rel_rows_supported(q) and aux["n_used"] <= _g.REL_MAX_USED_TYPES and not _g.force_generic_enabled()
+        if ctx.on_chip:
+            bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["number_slot"], q, table, used_types=aux["used_types"])
+        else:
+            bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["etype_slot"], q, table)
         o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed, bias=bias)
         ctx.save_for_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, bias, table)
         ctx.scale, ctx.dropout_p, ctx.seed, ctx.aux, ctx.etype = scale, dropout_p, seed, aux, etype
@@ -119,8 +123,8 @@ class BPTRelAttention(Function):
         aux = ctx.aux
         dq, dk, dv, ds = _g.attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c,
                                                q, k, v, o, lse, do, ctx.scale, ctx.dropout_p, ctx.seed, bias=bias)
-        if _g.rel_rows_supported(q) and aux["n_used"] <= _g.REL_MAX_USED_TYPES and not _g.force_generic_enabled():
-            dtable = _g.rel_bias_backward(col, indptr_c, eid_c, aux["etype_slot"], aux["used"], aux["n_used"], ds, q, table, dq)
+        if ctx.on_chip:
+            dtable = _g.rel_bias_backward(col, indptr_c, eid_c, aux["number_slot"], aux["used"], aux["used_types"], ds, q, table, dq)
         else:
             t_row, t_indptr, t_order, t_dst = _rel_type_rows(aux, ctx.etype, col, indptr_c, eid_c, table.size(0))
             h = q.size(1)
@@ -137,8 +141,9 @@ _rel_aux_cache = {}
 
 def _rel_aux(etype, col, indptr_c, eid_c, n_types):
     """Index tensors of the rel_pos term, cached per (etype, in-CSR): etype_slot, the edge type of every in-CSR slot;
-    used (n_types,) int32, the number of every type that occurs in a slot among the n_used of them (-1 for the others).
-    Built where etype lives; two scalars are read back (the range check and n_used)."""
+    used_types (n_used,) int32, the types that occur in a slot, ascending; used (n_types,) int32, the number of every
+    type in that list (-1 for the others); number_slot, the number of every slot's type.  Built where etype lives;
+    two scalars are read back (the range check and n_used)."""
     key = tuple((t.data_ptr(), t.numel(), t._version) for t in (etype, col, indptr_c, eid_c)) + (str(etype.device), n_types)
     hit = _rel_aux_cache.get(key)
     if hit is None:
@@ -151,7 +156,9 @@ def _rel_aux(etype, col, indptr_c, eid_c, n_types):
         present = torch.zeros(n_types, dtype=torch.bool, device=et.device).index_fill_(0, etype_slot, True)
         number = torch.cumsum(present, 0, dtype=torch.int32) - 1
         used = torch.where(present, number, torch.full_like(number, -1)).contiguous()
-        hit = {"etype_slot": etype_slot, "used": used, "n_used": int(present.sum()), "keep": (etype, col, indptr_c, eid_c)}
+        used_types = torch.nonzero(present).flatten().to(torch.int32)           # (the read-back of n_used)
+        hit = {"etype_slot": etype_slot, "used": used, "used_types": used_types, "n_used": used_types.numel(),
+               "number_slot": used.index_select(0, etype_slot).to(torch.int64), "keep": (etype, col, indptr_c, eid_c)}
         if len(_rel_aux_cache) > 16:
             _rel_aux_cache.clear()
         _rel_aux_cache[key] = hit           # "keep" holds the tensors so that their data_ptrs are not reused while cached

@@ -160,28 +160,32 @@ int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const
                              int h, int d, int dtype, void *stream);
 
 /* Score term of the relative positions, modules/attention.py:69-71 (embed_ak looked up per edge, then
- * node_mul_edge): bias[eid[p], head] = sum_d q[row, head, d] * table[idx[p], d] over `plan`, whose rows are the
- * destinations and whose idx[p] is the edge TYPE of the edge in slot p (a plan built with the edge types as
- * `indices`, n_index_nodes = rows of table).  bias is float32 (n_edges, h) or larger; the (n_edges, d) rows of the
- * reference's nn.Embedding lookup are never materialised.  Compile-time shapes only (BPT_ERR_UNSUPPORTED else). */
-int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, float *bias,
-                         int h, int d, int dtype, void *stream);
+ * node_mul_edge): bias[eid[p], head] = sum_d q[row, head, d] * table[type(p), d] over `plan`, whose rows are the
+ * destinations (a plan built with the types as `indices`).  bias is float32 (n_edges, h) or larger; the (n_edges, d)
+ * rows of the reference's nn.Embedding lookup are never materialised.
+ * used_types == NULL: idx[p] is the edge TYPE of the edge in slot p (n_index_nodes = rows of table); compile-time
+ * shapes only (BPT_ERR_UNSUPPORTED else).
+ * used_types (n_used) int32: the edge types that occur, in any order without repeats, and idx[p] is the NUMBER of the
+ * slot's type in that list (n_index_nodes = n_used).  The kernel keeps those rows of the table on chip and multiplies
+ * on the matrix cores; h in {4, 8, 16}, d = 64, f32 or bf16, n_used <= 240 (BPT_ERR_UNSUPPORTED else). */
+int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, const int32_t *used_types, int64_t n_used,
+                         float *bias, int h, int d, int dtype, void *stream);
 
 /* Gradients of that score term, the backward of embed_ak + node_mul_edge in modules/attention.py:55-56,69-71 (autograd of
  * nn.Embedding and graphop.py's NodeMulEdgeFunction.backward), from ds (n_edges or more rows, h) float32 =
  * dL/d(score of the edge before scaling), which bpt_attention_backward returns in ds_out:
- *   dq[row, head, :] += sum over the slots p of the row of ds[eid[p], head] * table[idx[p], :]      (added to dq)
- *   dtable[t, :]      = sum over the slots p with idx[p] == t and the heads of ds[eid[p], head] * q[row(p), head, :]
- * without the (n_edges, d) gradient rows of the embedding lookup.  `plan` as for bpt_rel_bias_forward.
- * used (n_types) int32: for every edge type that occurs in plan->idx its number among those types, 0 .. n_used - 1
- * (any order), and -1 for the others, whose rows of dtable become zero.  dq and dtable have the dtype of q and table.
- * workspace: bpt_rel_bias_backward_workspace_bytes(plan, n_used, h) bytes, 16-byte aligned.  Row-owned sums in a fixed order, no atomics.
- * h in {4, 8, 16}, d = 64, f32 or bf16, and as many used types as fit the kernel's on-chip sums (240 at least);
+ *   dq[row, head, :] += sum over the slots p of the row of ds[eid[p], head] * table[type(p), :]      (added to dq)
+ *   dtable[t, :]      = sum over the slots p of type t and the heads of ds[eid[p], head] * q[row(p), head, :]
+ * without the (n_edges, d) gradient rows of the embedding lookup.  `plan` and used_types (n_used) as for
+ * bpt_rel_bias_forward with used_types: idx[p] is the number of the slot's type.  used (n_types) int32 is the inverse:
+ * for every type in used_types its number, -1 for the others, whose rows of dtable become zero.  dq and dtable have the
+ * dtype of q and table.  workspace: bpt_rel_bias_backward_workspace_bytes(plan, n_used, h) bytes, 16-byte aligned.
+ * Row-owned sums in a fixed order, no atomics.  h in {4, 8, 16}, d = 64, f32 or bf16, n_used <= 240;
  * BPT_ERR_UNSUPPORTED otherwise (compose bpt_vector_spmm_forward calls instead). */
 int64_t bpt_rel_bias_backward_workspace_bytes(const bpt_plan *plan, int64_t n_used, int h);
 int bpt_rel_bias_backward(const bpt_plan *plan, const float *ds, const void *q, const void *table, const int32_t *used,
-                          int64_t n_types, int64_t n_used, void *dq, void *dtable, void *workspace, int64_t workspace_bytes,
-                          int h, int d, int dtype, void *stream);
+                          const int32_t *used_types, int64_t n_types, int64_t n_used, void *dq, void *dtable, void *workspace,
+                          int64_t workspace_bytes, int h, int d, int dtype, void *stream);
 
 /* Fused attention layer core = modules/attention.py:66-77:
  *   o[dst] = sum_{e: src->dst} drop( softmax_dst( (q[dst].k[src] + bias[e]) * scale ) )[e] * v[src]

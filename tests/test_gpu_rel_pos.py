@@ -30,31 +30,48 @@ def edge_types(E, n_types, n_used, seed):
     return et.astype(np.int64)
 
 
-def used_map(etype_slot, n_types):
-    present = np.zeros(n_types, dtype=bool)
-    present[etype_slot] = True
-    used = np.where(present, np.cumsum(present) - 1, -1).astype(np.int32)
-    return used, int(present.sum())
+def used_map(etype_slot, n_types, seed=None):
+    """(used, used_types, number_slot): the types that occur (ascending, or shuffled with `seed`: any order is allowed),
+    the number of every type in that list (-1: does not occur) and the number of every slot's type."""
+    used_types = np.unique(etype_slot).astype(np.int32)
+    if seed is not None:
+        used_types = np.random.default_rng(seed).permutation(used_types)
+    used = np.full(n_types, -1, dtype=np.int32)
+    used[used_types] = np.arange(len(used_types), dtype=np.int32)
+    return used, used_types, used[etype_slot].astype(np.int64)
+
+
+def dev(a):
+    return torch.from_numpy(a).to(DEV)
 
 
 SHAPES = [(torch.float32, 8), (torch.float32, 4), (torch.float32, 16), (torch.bfloat16, 8), (torch.bfloat16, 16)]
 GRAPH_NAMES = ["bpt512_k4", "bpt300_causal_k2", "multigraph", "fc_w100", "blocks8x30"]
 
 
+@pytest.mark.parametrize("on_chip", [True, False])
 @pytest.mark.parametrize("dtype,h", SHAPES)
 @pytest.mark.parametrize("gname", GRAPH_NAMES)
-def test_score_term_matches_node_mul_edge_of_the_looked_up_rows(ops, gname, dtype, h):
+def test_score_term_matches_node_mul_edge_of_the_looked_up_rows(ops, gname, dtype, h, on_chip):
+    """on_chip: the kernel that keeps the table rows in use in LDS (plan indices = type numbers); otherwise the one that
+    gathers table rows by type."""
     graphop, _ = ops
+    if not on_chip and (dtype, h) == (torch.float32, 4) and gname != "bpt512_k4":
+        pytest.skip("one graph is enough for the gathering kernel of this shape")
     d, n_types = 64, 1000
     c = case(gname)
     q = rand((c.n, h, d), dtype, 11, 0.5).to(DEV)
     table = rand((n_types, d), dtype, 12, 0.5).to(DEV)
     et = edge_types(c.E, n_types, 55, 13)
-    etype_slot = torch.from_numpy(et[c.np_in[2]]).to(DEV)
-    bias = graphop.rel_bias_forward(*c.inn[:3], etype_slot, q, table)
+    etype_slot = et[c.np_in[2]]
+    if on_chip:
+        used, used_types, number_slot = used_map(etype_slot, n_types, seed=14)
+        bias = graphop.rel_bias_forward(*c.inn[:3], dev(number_slot), q, table, used_types=dev(used_types))
+    else:
+        bias = graphop.rel_bias_forward(*c.inn[:3], dev(etype_slot), q, table)
     assert bias.shape == (c.E + 1, h) and bias.dtype == torch.float32
     want = oracle.node_mul_edge_forward(*c.np_in[:3], f64(q), f64(table)[et])
-    close(bias[:c.E], want, TOL[torch.float32] if dtype == torch.float32 else TOL[dtype], "score term")
+    close(bias[:c.E], want, TOL[dtype], "score term")
     assert float(bias[c.E].abs().max()) == 0.0
 
 
@@ -74,20 +91,19 @@ def test_score_term_gradients_match_node_mul_edge_backward(ops, gname, dtype, h,
     ds = torch.cat([rand((c.E, h), torch.float32, 23, 0.1), torch.zeros(1, h)]).to(DEV)     # (E + 1, h) as the fused backward returns it
     dq0 = rand((c.n, h, d), dtype, 24, 0.5).to(DEV)
     et = edge_types(c.E, n_types, n_used, 25)
-    etype_slot_np = et[c.np_in[2]]
-    used, nu = used_map(etype_slot_np, n_types)
-    assert nu == min(n_used, c.E)
+    used, used_types, number_slot = used_map(et[c.np_in[2]], n_types, seed=26 if n_used == 55 else None)
+    assert len(used_types) == min(n_used, c.E)
+    args = (*c.inn[:3], dev(number_slot), dev(used), dev(used_types), ds, q, table)
     dq = dq0.clone()
-    dtable = graphop.rel_bias_backward(*c.inn[:3], torch.from_numpy(etype_slot_np).to(DEV), torch.from_numpy(used).to(DEV), nu, ds, q, table, dq)
+    dtable = graphop.rel_bias_backward(*args, dq)
     dA, dB = oracle.node_mul_edge_backward(*c.np_in[:3], f64(q), f64(table)[et], f64(ds[:c.E]))
     want_table = np.zeros((n_types, d))
     np.add.at(want_table, et, dB)
     # both are raw sums of unnormalised N(0, 0.1) x N(0, 0.5) products: max_deg terms for a row of dq (on top of dq0), h * E / n_used
     # for a row of the table (terms)
     close(dq, f64(dq0) + dA, GTOL[dtype], "dq", c.max_deg)
-    close(dtable, want_table, GTOL[dtype], "dtable", h * c.E / max(nu, 1))
-    again = graphop.rel_bias_backward(*c.inn[:3], torch.from_numpy(etype_slot_np).to(DEV), torch.from_numpy(used).to(DEV), nu, ds, q, table,
-                                      dq0.clone())
+    close(dtable, want_table, GTOL[dtype], "dtable", h * c.E / max(len(used_types), 1))
+    again = graphop.rel_bias_backward(*args, dq0.clone())
     assert torch.equal(again, dtable), "the sums have a fixed order: the same bits every run"
 
 
@@ -98,13 +114,13 @@ def test_too_many_used_types_is_refused_and_the_layer_takes_the_spmm_form(ops):
     q, k, v, do = (rand((c.n, h, d), torch.float32, s, 1.0 / 8).to(DEV) for s in (31, 32, 33, 34))
     table = rand((n_types, d), torch.float32, 35, 1.0 / 8).to(DEV)
     et = edge_types(c.E, n_types, 300, 36)
-    etype_slot_np = et[c.np_in[2]]
-    used, nu = used_map(etype_slot_np, n_types)
-    assert nu == 300 > graphop.REL_MAX_USED_TYPES
+    used, used_types, number_slot = used_map(et[c.np_in[2]], n_types)
+    assert len(used_types) == 300 > graphop.REL_MAX_USED_TYPES
     ds = torch.zeros(c.E + 1, h, device=DEV)
     with pytest.raises(RuntimeError, match="status -7"):
-        graphop.rel_bias_backward(*c.inn[:3], torch.from_numpy(etype_slot_np).to(DEV), torch.from_numpy(used).to(DEV), nu, ds, q, table,
-                                  torch.zeros_like(q))
+        graphop.rel_bias_forward(*c.inn[:3], dev(number_slot), q, table, used_types=dev(used_types))
+    with pytest.raises(RuntimeError, match="status -7"):
+        graphop.rel_bias_backward(*c.inn[:3], dev(number_slot), dev(used), dev(used_types), ds, q, table, torch.zeros_like(q))
     from oracle import torch_ops
     etype = torch.from_numpy(et).to(DEV)
     for t in (q, k, v, table):
@@ -117,7 +133,7 @@ def test_too_many_used_types_is_refused_and_the_layer_takes_the_spmm_form(ops):
     rdt = torch.zeros(n_types, d, dtype=torch.float64).index_add_(0, etype.cpu(), rdak)
     close(o, ro.numpy(), TOL[torch.float32], "o")
     close(q.grad, rdq.numpy(), GTOL[torch.float32], "dq")
-    close(table.grad, rdt.numpy(), GTOL[torch.float32], "dtable", h * c.E / nu)
+    close(table.grad, rdt.numpy(), GTOL[torch.float32], "dtable", h * c.E / 300)
 
 
 def test_graph_without_edges_gives_a_zero_table_gradient(ops):
@@ -129,5 +145,6 @@ def test_graph_without_edges_gives_a_zero_table_gradient(ops):
     table = rand((n_types, d), torch.float32, 42).to(DEV)
     dq = torch.ones_like(q)
     used = torch.full((n_types,), -1, dtype=torch.int32, device=DEV)
-    dtable = graphop.rel_bias_backward(col, indptr, eid, et, used, 0, torch.zeros(1, h, device=DEV), q, table, dq)
+    used_types = torch.zeros(0, dtype=torch.int32, device=DEV)
+    dtable = graphop.rel_bias_backward(col, indptr, eid, et, used, used_types, torch.zeros(1, h, device=DEV), q, table, dq)
     assert float(dtable.abs().max()) == 0.0 and torch.equal(dq, torch.ones_like(q))
