@@ -245,11 +245,11 @@ template <> __device__ __forceinline__ float4 load4<bf16_t>(const bf16_t *p) {
 }
 template <typename T>
 __device__ __forceinline__ void combine_sum_block4(const int32_t *__restrict__ hv, const float *__restrict__ ws, T *__restrict__ Y, int C,
-                                                   bool accumulate = false) {
+                                                   bool accumulate = false, int strip = -1) {
     __shared__ float4 part[WAVES_PER_BLOCK][WAVE];
     const int row = hv[0], s0 = hv[1], ns = hv[2];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int j = (blockIdx.y * WAVE + lane) * 4;
+    const int j = ((strip < 0 ? (int)blockIdx.y : strip) * WAVE + lane) * 4;     // strip of 256 columns: the grid's y unless given
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     const float *col = ws + (size_t)s0 * C + j;
     int k = w;
@@ -2880,6 +2880,7 @@ __global__ __launch_bounds__(BLOCK) void k_rel_bias_rows(bpt_plan P, const T *__
 #pragma unroll
     for (int k = 0; k < K; ++k) desc[k] = items[min(i0 + k * GW, n_items - 1)];
     rel_table_to_lds<T>(table, used_types, n_used, rel_lds, REL_LDS_PITCH);
+    if (blockIdx.x == 0 && threadIdx.x < H) bias[(size_t)P.n_edges * H + threadIdx.x] = 0.f;     // the spare row the fused kernels read for absent pairs
     RelHead hd[K];
     float aq[K][16];
 #pragma unroll
@@ -3073,11 +3074,11 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
 // not occur).  One workgroup per type; 16 lanes cover a row (four columns each), so a wavefront reads four partial rows
 // per load: lane group s of wave w adds the rows 4 w + s, 4 w + s + 16, ...; the 16 sums are then added in a fixed order.
 template <typename T>
-__global__ __launch_bounds__(BLOCK) void k_rel_table_sum(const float *__restrict__ part, const int32_t *__restrict__ used, int n_parts,
-                                                         T *__restrict__ dtable) {
+__device__ __forceinline__ void rel_table_sum_block(int type, const float *__restrict__ part, const int32_t *__restrict__ used, int n_parts,
+                                                    T *__restrict__ dtable) {
     constexpr int D = 64, GROUPS = BLOCK / 16;
     __shared__ float4 sums[GROUPS][16];
-    const int type = blockIdx.x, u = used[type], grp = threadIdx.x >> 4, c4 = (threadIdx.x & 15) * 4;
+    const int u = used[type], grp = threadIdx.x >> 4, c4 = (threadIdx.x & 15) * 4;
     if (u < 0) {
         if (threadIdx.x < 16) store4<T>(dtable + (size_t)type * D + c4, make_float4(0.f, 0.f, 0.f, 0.f));
         return;
@@ -3103,6 +3104,22 @@ __global__ __launch_bounds__(BLOCK) void k_rel_table_sum(const float *__restrict
 #pragma unroll
         for (int k = 1; k < GROUPS; ++k) { const float4 t = sums[k][threadIdx.x]; tot.x += t.x; tot.y += t.y; tot.z += t.z; tot.w += t.w; }
         store4<T>(dtable + (size_t)type * D + c4, tot);
+    }
+}
+
+// What is left after k_rel_bias_bwd, in one launch of n_types + n_heavy * C / 256 workgroups: the first n_types sum
+// the partial tables (above), the others add the partial dq rows of the split rows to dq (one workgroup per split row
+// and strip of 256 columns, in the order combine_sum_block uses).
+template <typename T>
+__global__ __launch_bounds__(BLOCK) void k_rel_finish(const float *__restrict__ part, const int32_t *__restrict__ used, int n_parts, int n_types,
+                                                      T *__restrict__ dtable, const int32_t *__restrict__ heavy, const float *__restrict__ ws_dq,
+                                                      T *__restrict__ dq, int C) {
+    const int b = blockIdx.x;
+    if (b < n_types) {
+        rel_table_sum_block<T>(b, part, used, n_parts, dtable);
+    } else {
+        const int strips = C / 256, x = b - n_types;
+        combine_sum_block4<T>(heavy + 3 * (x / strips), ws_dq, dq, C, true, x % strips);
     }
 }
 
@@ -3351,15 +3368,12 @@ int run_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const vo
                  : nw == 2 ? launch_rel_bias_bwd<T, H, 2>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s)
                            : launch_rel_bias_bwd<T, H, 1>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s);
         if (st != BPT_OK) return st;
-        if (P->n_heavy > 0) {
-            hipLaunchKernelGGL((k_combine_sum_v4<T>), dim3((unsigned)P->n_heavy, H * 64 / 256, 1), dim3(BLOCK), 0, s, P->heavy, ws_dq, (T *)dq,
-                               (T *)nullptr, H * 64, (size_t)0, 1);
-            st = launch_status();
-            if (st != BPT_OK) return st;
-        }
     }
-    // (without edges there are no partial tables: every row of dtable becomes zero)
-    hipLaunchKernelGGL((k_rel_table_sum<T>), dim3((unsigned)n_types), dim3(BLOCK), 0, s, part, used, P->n_edges > 0 ? n_parts : 0, (T *)dtable);
+    // (without edges there are no partial tables and no partial rows: every row of dtable becomes zero)
+    const bool edges = P->n_edges > 0;
+    const int n_split = edges ? (int)P->n_heavy : 0;
+    hipLaunchKernelGGL((k_rel_finish<T>), dim3((unsigned)(n_types + (int64_t)n_split * (H * 64 / 256))), dim3(BLOCK), 0, s, part, used,
+                       edges ? n_parts : 0, (int)n_types, (T *)dtable, P->heavy, ws_dq, (T *)dq, H * 64);
     return launch_status();
 }
 

@@ -375,7 +375,8 @@ def rel_bias_forward(col, indptr_c, eid_c, type_slot, q, table, used_types=None)
         plan = plan_cache.get(col, indptr_c, eid_c, type_slot, q.size(0), table.size(0))
         ref, n_used = _spmm_ref(plan, q, h, d, cfg), 0
     bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
-    bias[E].zero_()
+    if used_types is None or not plan.n_items:
+        bias[E].zero_()                     # (the kernel of the other form clears the spare row itself)
     with torch.cuda.device_of(q):
         check_attn(_LIB.bpt_rel_bias_forward(ref, _ptr(q), _ptr(table), _ptr(used_types) if used_types is not None else None, n_used,
                                              _ptr(bias), h, d, _dtype(q), _stream()), "rel_bias_forward")

@@ -167,7 +167,8 @@ int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const
  * shapes only (BPT_ERR_UNSUPPORTED else).
  * used_types (n_used) int32: the edge types that occur, in any order without repeats, and idx[p] is the NUMBER of the
  * slot's type in that list (n_index_nodes = n_used).  The kernel keeps those rows of the table on chip and multiplies
- * on the matrix cores; h in {4, 8, 16}, d = 64, f32 or bf16, n_used <= 240 (BPT_ERR_UNSUPPORTED else). */
+ * on the matrix cores; h in {4, 8, 16}, d = 64, f32 or bf16, n_used <= 240 (BPT_ERR_UNSUPPORTED else).  In this form
+ * bias must have n_edges + 1 rows: the kernel also clears row n_edges, the spare row of bpt_attention_forward. */
 int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, const int32_t *used_types, int64_t n_used,
                          float *bias, int h, int d, int dtype, void *stream);
 

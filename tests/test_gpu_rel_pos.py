@@ -49,15 +49,17 @@ SHAPES = [(torch.float32, 8), (torch.float32, 4), (torch.float32, 16), (torch.bf
 GRAPH_NAMES = ["bpt512_k4", "bpt300_causal_k2", "multigraph", "fc_w100", "blocks8x30"]
 
 
-@pytest.mark.parametrize("on_chip", [True, False])
-@pytest.mark.parametrize("dtype,h", SHAPES)
-@pytest.mark.parametrize("gname", GRAPH_NAMES)
+def _score_cases():
+    """Every graph and shape with the table rows on chip; the kernel that gathers them by type on two graphs."""
+    return [(g, dt, h, True) for g in GRAPH_NAMES for dt, h in SHAPES] + \
+           [(g, dt, h, False) for g in ("bpt512_k4", "multigraph") for dt, h in SHAPES]
+
+
+@pytest.mark.parametrize("gname,dtype,h,on_chip", _score_cases())
 def test_score_term_matches_node_mul_edge_of_the_looked_up_rows(ops, gname, dtype, h, on_chip):
     """on_chip: the kernel that keeps the table rows in use in LDS (plan indices = type numbers); otherwise the one that
     gathers table rows by type."""
     graphop, _ = ops
-    if not on_chip and (dtype, h) == (torch.float32, 4) and gname != "bpt512_k4":
-        pytest.skip("one graph is enough for the gathering kernel of this shape")
     d, n_types = 64, 1000
     c = case(gname)
     q = rand((c.n, h, d), dtype, 11, 0.5).to(DEV)
@@ -75,15 +77,17 @@ def test_score_term_matches_node_mul_edge_of_the_looked_up_rows(ops, gname, dtyp
     assert float(bias[c.E].abs().max()) == 0.0
 
 
-@pytest.mark.parametrize("n_types,n_used", [(1000, 55), (37, 37), (1000, 100), (400, 230), (5, 1)])
-@pytest.mark.parametrize("dtype,h", SHAPES)
-@pytest.mark.parametrize("gname", GRAPH_NAMES)
+def _gradient_cases():
+    """55 of 1000 and 37 of 37 types on every graph; 100 and 230 used types (two and one wavefronts per workgroup of the
+    kernel instead of four) and a single type on two graphs."""
+    return [(g, dt, h, nt, nu) for g in GRAPH_NAMES for dt, h in SHAPES for nt, nu in ((1000, 55), (37, 37))] + \
+           [(g, dt, h, nt, nu) for g in ("bpt512_k4", "multigraph") for dt, h in SHAPES for nt, nu in ((1000, 100), (400, 230), (5, 1))]
+
+
+@pytest.mark.parametrize("gname,dtype,h,n_types,n_used", _gradient_cases())
 def test_score_term_gradients_match_node_mul_edge_backward(ops, gname, dtype, h, n_types, n_used):
-    """dq gains node_mul_edge's dA, dtable is its dB summed per edge type (the embedding's gradient); the counts of used
-    types cover one, two and four wavefronts per workgroup of the kernel."""
+    """dq gains node_mul_edge's dA, dtable is its dB summed per edge type (the embedding's gradient)."""
     graphop, _ = ops
-    if (n_types, n_used) in ((1000, 100), (400, 230), (5, 1)) and gname not in ("bpt512_k4", "multigraph"):
-        pytest.skip("the type counts are varied on two graphs")
     d = 64
     c = case(gname)
     q = rand((c.n, h, d), dtype, 21, 0.5).to(DEV)
