@@ -11,6 +11,7 @@ SDDMM -> edge-softmax -> SpMM pass, and vector_spmm_backward returns the complet
 reference's launch drops trailing units of the transposed side, graphop_kernel.cu:566,588).
 """
 import collections
+import contextlib
 import ctypes
 import math
 import threading
@@ -111,8 +112,34 @@ def _expect_index(eid, indices):
         raise ValueError("eid and indices must be 1-D tensors of the same length")
 
 
+# The per-call host work counts on small graphs, where a step's kernels take tens of microseconds: the current stream and
+# device come from torch's raw accessors (a fraction of a microsecond; torch.cuda.current_stream() builds a Stream object,
+# about 10 us a call), and the device guard is entered only when the tensors live on another device than the current one.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
+def _current_device():
+    return _raw_device() if _raw_device is not None else torch.cuda.current_device()
+
+
+def _stream_handle(index=None):
+    """The current stream of the device (default: the current device) as an integer handle."""
+    if _raw_stream is not None:
+        return _raw_stream(_current_device() if index is None else index)
+    return torch.cuda.current_stream(index).cuda_stream
+
+
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return ctypes.c_void_p(_stream_handle())
+
+
+_NO_GUARD = contextlib.nullcontext()
+
+
+def _on_device_of(t):
+    """Context in which t's device is the current one (what the kernels launch on and the raw stream accessor reads)."""
+    return _NO_GUARD if t.device.index == _current_device() else torch.cuda.device_of(t)
 
 
 def _ptr(t):
@@ -142,7 +169,8 @@ KEEP_WORKSPACES = True
 def _scratch(n, device):
     if not KEEP_WORKSPACES or torch.cuda.is_current_stream_capturing():
         return torch.empty(n, dtype=torch.uint8, device=device)
-    key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
+    index = device.index if device.index is not None else _current_device()
+    key = (index, _stream_handle(index))
     with _SCRATCH_LOCK:
         buf = _SCRATCH.get(key)
         if buf is None or buf.numel() < n:
@@ -184,7 +212,7 @@ def maskedmm_csr_forward(row, indptr, eid, indices, A, B):
     plan = plan_cache.get(row, indptr, eid, indices, A.size(0), B.size(0))
     e = eid.size(0)
     y = _edge_out(plan, (e,) if A.dim() == 2 else (e, h), A)
-    with torch.cuda.device_of(A):
+    with _on_device_of(A):
         check_attn(_LIB.bpt_maskedmm_csr_forward(_spmm_ref(plan, A, h, d, cfg), _ptr(A), _ptr(B), _ptr(y), h, d, _dtype(A), _stream()),
                    "maskedmm_csr_forward")
     return y
@@ -208,7 +236,7 @@ def maskedmm_csr_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c,
     dA, dB = torch.empty_like(A), torch.empty_like(B)
     dt = _dtype(A)
     ws, nws = _workspace(OP_MASKEDMM_BWD, plan_r, plan_c, h, d, dt, A.device)
-    with torch.cuda.device_of(A):
+    with _on_device_of(A):
         check_attn(_LIB.bpt_maskedmm_csr_backward(_spmm_ref(plan_r, A, h, d, cfg), _spmm_ref(plan_c, A, h, d, cfg), _ptr(A), _ptr(B), _ptr(dy), _ptr(dA), _ptr(dB),
                                                   _ptr(ws), nws, h, d, dt, _stream()), "maskedmm_csr_backward")
     return [dA, dB]
@@ -224,7 +252,7 @@ def node_mul_edge_forward(row, indptr, eid, A, B):
     plan = plan_cache.get(row, indptr, eid, None, A.size(0), None)
     e = eid.size(0)
     y = _edge_out(plan, (e,) if A.dim() == 2 else (e, h), A)
-    with torch.cuda.device_of(A):
+    with _on_device_of(A):
         check_attn(_LIB.bpt_node_mul_edge_forward(plan.ref, _ptr(A), _ptr(B), _ptr(y), h, d, _dtype(A), _stream()),
                    "node_mul_edge_forward")
     return y
@@ -244,7 +272,7 @@ def node_mul_edge_backward(row, indptr, eid, A, B, dy):
     dB = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(B)
     dt = _dtype(A)
     ws, nws = _workspace(OP_NME_BWD, plan, None, h, d, dt, A.device)
-    with torch.cuda.device_of(A):
+    with _on_device_of(A):
         check_attn(_LIB.bpt_node_mul_edge_backward(plan.ref, _ptr(A), _ptr(B), _ptr(dy), _ptr(dA), _ptr(dB),
                                                    _ptr(ws), nws, h, d, dt, _stream()), "node_mul_edge_backward")
     return [dA, dB]
@@ -259,7 +287,7 @@ def sparse_softmax_forward(row, indptr, eid, x):
     plan = plan_cache.get(row, indptr, eid, None, None, None)
     y = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(x)
     ws, nws = _workspace(OP_SOFTMAX_FWD, plan, None, _edge_h(x), 1, _dtype(x), x.device)
-    with torch.cuda.device_of(x):
+    with _on_device_of(x):
         check_attn(_LIB.bpt_sparse_softmax_forward(plan.ref, _ptr(x), _ptr(y), _ptr(ws), nws, _edge_h(x), _dtype(x), _stream()),
                    "sparse_softmax_forward")
     return y
@@ -276,7 +304,7 @@ def sparse_softmax_backward(row, indptr, eid, y, dy):
     plan = plan_cache.get(row, indptr, eid, None, None, None)
     dx = (torch.empty_like if plan.covers_all_edges else torch.zeros_like)(dy)
     ws, nws = _workspace(OP_SOFTMAX_BWD, plan, None, _edge_h(dy), 1, _dtype(y), y.device)
-    with torch.cuda.device_of(y):
+    with _on_device_of(y):
         check_attn(_LIB.bpt_sparse_softmax_backward(plan.ref, _ptr(y), _ptr(dy), _ptr(dx), _ptr(ws), nws, _edge_h(dy), _dtype(y),
                                                     _stream()),
                    "sparse_softmax_backward")
@@ -303,7 +331,7 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None, out
     ws, nws = _workspace(OP_SPMM_FWD, plan, None, h, d, dt, x.device)
     if out is not None and (out.shape != y.shape or out.dtype != y.dtype or out.device != y.device or not out.is_contiguous()):
         raise ValueError("out must be a contiguous tensor of the result's shape, dtype and device")
-    with torch.cuda.device_of(x):
+    with _on_device_of(x):
         ref = _spmm_ref(plan, x, h, d, cfg)
         if out is not None:
             st = _LIB.bpt_vector_spmm_accumulate(ref, _ptr(edata), _ptr(x), _ptr(out), _ptr(ws), nws, h, d, dt, _stream())
@@ -336,7 +364,7 @@ def vector_spmm_backward(row, indptr, eid, indices, col, indptr_t, eid_t, indice
     dx = torch.empty_like(x)
     dt = _dtype(x)
     ws, nws = _workspace(OP_SPMM_BWD, plan, plan_t, h, d, dt, x.device)
-    with torch.cuda.device_of(x):
+    with _on_device_of(x):
         check_attn(_LIB.bpt_vector_spmm_backward(_spmm_ref(plan, x, h, d, cfg), _spmm_ref(plan_t, x, h, d, cfg), _ptr(edata), _ptr(dy), _ptr(x), _ptr(dedata), _ptr(dx),
                                                  _ptr(ws), nws, h, d, dt, _stream()), "vector_spmm_backward")
     return [dedata, dx]
@@ -377,7 +405,7 @@ def rel_bias_forward(col, indptr_c, eid_c, type_slot, q, table, used_types=None)
     bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
     if used_types is None or not plan.n_items:
         bias[E].zero_()                     # (the kernel of the other form clears the spare row itself)
-    with torch.cuda.device_of(q):
+    with _on_device_of(q):
         check_attn(_LIB.bpt_rel_bias_forward(ref, _ptr(q), _ptr(table), _ptr(used_types) if used_types is not None else None, n_used,
                                              _ptr(bias), h, d, _dtype(q), _stream()), "rel_bias_forward")
     return bias
@@ -416,7 +444,7 @@ def rel_bias_backward(col, indptr_c, eid_c, number_slot, used, used_types, ds, q
     n_used = used_types.numel()
     plan = plan_cache.get(col, indptr_c, eid_c, number_slot, q.size(0), max(n_used, 1))
     dtable = torch.empty_like(table)
-    with torch.cuda.device_of(q):
+    with _on_device_of(q):
         nws = int(_LIB.bpt_rel_bias_backward_workspace_bytes(plan.ref, n_used, h))
         ws = _scratch(max(nws, 16), q.device)
         check_attn(_LIB.bpt_rel_bias_backward(plan.ref, _ptr(ds), _ptr(q), _ptr(table), _ptr(used), _ptr(used_types), table.size(0), n_used,
@@ -459,7 +487,7 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
     ws, nws = _workspace(OP_ATTN_FWD, plan, None, h, d, dt, q.device)
-    with torch.cuda.device_of(q):
+    with _on_device_of(q):
         check_attn(_LIB.bpt_attention_forward(ref, _ptr(q), _ptr(k), _ptr(v), _ptr(bias), _ptr(o), _ptr(lse), _ptr(ws), nws,
                                               scale, float(dropout_p), int(seed) & (2 ** 64 - 1), h, d, dt, _stream()),
                    "attention_forward")
@@ -507,7 +535,7 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
             in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
             out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
-    with torch.cuda.device_of(q):
+    with _on_device_of(q):
         check_attn(_LIB.bpt_attention_backward(in_ref, out_ref, _ptr(q), _ptr(k), _ptr(v), _ptr(bias), _ptr(o), _ptr(do),
                                                _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ds), _ptr(ws), nws,
                                                scale, float(dropout_p), int(seed) & (2 ** 64 - 1), h, d, dt, _stream()),

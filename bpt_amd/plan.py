@@ -530,7 +530,7 @@ class PlanCache:
 
     @staticmethod
     def _key(tensors, n_rows, n_index, seg_len, on_device):
-        return tuple((t.data_ptr(), t.numel(), t._version, str(t.device)) if t is not None else None
+        return tuple((t.data_ptr(), t.numel(), t._version, t.device) if t is not None else None
                      for t in tensors) + (n_rows, n_index, seg_len, on_device)
 
     def get(self, row, indptr, eid, indices, n_rows=None, n_index_nodes=None, seg_len=DEFAULT_SEG_LEN, prefer_device=False):
