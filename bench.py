@@ -341,6 +341,31 @@ def main():
                  "attention_ms_per_layer": round(t_step * 1e3, 4), "attention_share": round(t_step * args.block_layers / t_stack, 3)}
         log(f"block stack: {block}")
 
+    variants = None
+    if args.block_layers > 0 and not args.unfused and not args.rel_pos and args.dropout == 0:
+        # the same step with the layer's two optional terms inside the fused kernels (modules/attention.py:69-73), eager,
+        # shortest of three short runs each: the rel_pos score term (table (1000, d_head), the graph's own edge types) and
+        # attention dropout 0.1
+        from bpt_amd import op as op_mod
+        table = (torch.randn(1000, D, generator=torch.Generator().manual_seed(3)) / 8).to(tdtype).to(dev)
+        et = torch.from_numpy(np.asarray(etype, dtype=np.int64)).to(dev)
+
+        def variant_step(**kw):
+            def f():
+                qq, kk, vv, tt = (x.detach().requires_grad_(True) for x in (q, k, v, table))
+                if "rel" in kw:
+                    kw2 = dict(rel_table=tt, etype=et)
+                else:
+                    kw2 = {}
+                o = op_mod.bpt_attention(*gargs, qq, kk, vv, dropout_p=kw.get("p", 0.0), seed=2345, **kw2)
+                o.backward(do)
+            return f
+
+        variants = {name: round(min(timed(variant_step(**kw), 200, 20) for _ in range(3)) * 1e3, 4)
+                    for name, kw in (("rel_pos_ms_per_step", dict(rel=True)), ("dropout_0.1_ms_per_step", dict(p=0.1)),
+                                     ("rel_pos_dropout_0.1_ms_per_step", dict(rel=True, p=0.1)))}
+        log(f"variants: {variants}")
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(src, dst, N, H, D, 2345)
@@ -372,6 +397,8 @@ def main():
         out["plan_build"] = plan_build
     if block is not None:
         out["block_stack"] = block
+    if variants is not None:
+        out["variants"] = variants
     log(json.dumps(out, indent=1))
     print(json.dumps(out), flush=True)
 
