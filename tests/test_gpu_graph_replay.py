@@ -50,6 +50,52 @@ def test_graph_replay_equals_eager(L, dtype, dropout):
             assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager result"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_graph_replay_of_the_step_with_the_rel_pos_term_equals_eager(dtype):
+    """The same with the rel_pos score term: its score kernel, the fused kernels that add it, and the kernels that form
+    the gradients of q and of the table from the per-edge ds (more than 64 KB of LDS per workgroup, partial tables in
+    the kept workspace), the table changed in place between replays like the other inputs."""
+    import numpy as np
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd import graphop, op
+    g = gb.BinaryPartition(8192, True, 4, 10)
+    src, dst, etype = g.get_edges()
+    n = g.number_of_nodes
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, n)
+    args = tuple(x.to(DEV) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
+    gen = torch.Generator().manual_seed(78)
+    q, k, v, do = ((torch.randn(n, 8, 64, generator=gen) / 8).to(dtype).to(DEV) for _ in range(4))
+    table = (torch.randn(1000, 64, generator=gen) / 8).to(dtype).to(DEV)
+    aux = op._rel_aux(torch.from_numpy(np.asarray(etype, dtype=np.int64)).to(DEV), *args[4:7], 1000)
+    assert 1 < aux["n_used"] <= graphop.REL_MAX_USED_TYPES
+
+    def step():
+        bias = graphop.rel_bias_forward(*args[4:7], aux["number_slot"], q, table, used_types=aux["used_types"])
+        o, lse = graphop.attention_forward(*args[4:], q, k, v, bias=bias)
+        dq, dk, dv, ds = graphop.attention_backward(*args, q, k, v, o, lse, do, bias=bias)
+        dtable = graphop.rel_bias_backward(*args[4:7], aux["number_slot"], aux["used"], aux["used_types"], ds, q, table, dq)
+        return o, lse, dq, dk, dv, dtable
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):                      # plans are built and cached before the capture
+        for _ in range(2):
+            step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gout = step()
+    for rep in range(4):
+        if rep:
+            for t in (q, k, v, do, table):
+                t.mul_(-0.5).add_(0.01 * rep)
+        want = step()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b, name in zip(gout, want, ("o", "lse", "dq", "dk", "dv", "dtable")):
+            assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager result"
+
+
 def test_kept_workspaces_give_the_same_results_and_can_be_released():
     """Ops keep one workspace per device and stream and reuse it from call to call: results equal those with a fresh
     allocation per call, two different ops in a row do not disturb each other, and release_workspaces() drops the buffers."""
