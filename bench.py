@@ -111,6 +111,8 @@ def main():
     ap.add_argument("--plan", default="auto", choices=["auto", "host", "device"],
                     help="where launch plans and row groups are built: on the host (libbptgraph), on the GPU (libbptplan), "
                          "or by graph size and density (the library's default)")
+    ap.add_argument("--tile-backward", default="auto", choices=["auto", "on", "off"],
+                    help="fused backward on the dense tiles of 16 rows (on), on the row groups (off), or the library's choice by dtype and graph")
     ap.add_argument("--block-layers", type=int, default=None,
                     help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the "
                          "workload's graph, a few steps, reported as block_stack; default: 12 for the headline workload, else 0")
@@ -129,6 +131,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
     graphop.set_row_groups(not args.rows)
+    graphop.TILE_BACKWARD = {"auto": None, "on": True, "off": False}[args.tile_backward]
     graphop.set_group_rows(args.group_rows)
     from bpt_amd import plan as plan_mod
     plan_mod.set_device_build({"auto": None, "host": False, "device": True}[args.plan])

@@ -523,7 +523,7 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref
     if _attention_groups(plan_in, dropout_p, bias, q, k, cfg) and plan_in.covers_all_edges and plan_out.covers_all_edges:
-        if _tiles(q, h, d, plan_in, dropout_p, bias, cfg) and _tiles_backward(plan_in, q.dtype):
+        if _tiles(q, h, d, plan_in, dropout_p, bias, cfg) and _tiles_backward(plan_in, q.dtype, bias):
             seg = _tile_seg_len(plan_in)
             plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg, prefer_device=True)
             plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg, prefer_device=True)
@@ -623,16 +623,19 @@ def _tiles(q, h, d, plan, dropout_p, bias, cfg):
             and d == 64 and h <= 16)
 
 
-def _tiles_backward(plan, dtype):
-    """The backward runs on tiles where that measured faster than the row-group kernels (float32, 8 x 64): on small graphs,
-    which the row groups of 8 cannot spread over the GPU (L = 4096: k = 1 ... 4 run level to 3 % faster), and on graphs of
-    mean degree 32 and more (L = 4096, k = 8 ... 32: 15 to 27 %; window 128: 1.9 x; L = 32768, k = 8, 16 heads: 3 %); at
-    L = 8192, k = 4 and on the 32-graph batch the row-group kernels win (0.203 against 0.213 ms, 0.323 against 0.329).
-    bfloat16 rows: always (a block costs six matrix instructions instead of 32 to 48; every graph measured runs faster,
-    L = 8192, k = 4: 0.112 against 0.135 ms; L = 32768, k = 8, 16 heads: 1.20 against 1.49; window 128: 0.081 against 0.188)."""
+def _tiles_backward(plan, dtype, bias=None):
+    """The backward runs on tiles wherever the forward does, except in float32 with the score term on large sparse graphs.
+    float32 (8 x 64), step time on tiles against row groups: L = 8192, k = 4 0.175 against 0.187 ms, with attention
+    dropout 0.178 against 0.203; the 32-graph batch 0.298 against 0.307; L = 32768, k = 4 0.807 against 0.841; L = 4096,
+    k = 1 ... 32 level to 27 % faster, window 128 1.9 x.  With the score term the tile kernels fetch it per pair and head
+    (a wavefront owns one head) where the row-group kernel fetches all heads of a pair at once, and lose their lead on
+    graphs of 12288 rows and more with mean degree under 32 (L = 8192, k = 4: 0.285 against 0.284 ms; the 32-graph batch
+    0.461 against 0.449): those stay on the row groups.  bfloat16 rows: always tiles (a block costs six matrix instructions
+    instead of 32 to 48; every graph measured runs faster, L = 8192, k = 4: 0.112 against 0.135 ms; L = 32768, k = 8, 16
+    heads: 1.20 against 1.49; window 128: 0.081 against 0.188)."""
     if TILE_BACKWARD is not None:
         return TILE_BACKWARD
-    if dtype == torch.bfloat16:
+    if dtype == torch.bfloat16 or bias is None:
         return True
     return plan.n_rows < 12288 or plan.n_edges >= 32 * max(plan.n_rows, 1)
 

@@ -1,9 +1,9 @@
 """The fused step under HIP graph capture: a caller that records forward + backward once and replays it (a training
 loop with a fixed graph) must get, on every replay, exactly what the eager launches give.  The graph is replayed
 several times with eager work of the same library and synchronisations in between, inputs are changed in place
-between replays, and every replay is compared bit for bit with an eager step on the same inputs.  float32 runs the
-tile forward with the row-group or tile backward, bfloat16 the tile kernels throughout; one case uses dropout (a
-function of seed, edge id and head: the same under replay)."""
+between replays, and every replay is compared bit for bit with an eager step on the same inputs.  The tile kernels
+forward and backward in float32 and bfloat16, and in float32 also the tile forward with the row-group backward; with and
+without dropout (a function of seed, edge id and head: the same under replay)."""
 import pytest
 import torch
 
@@ -12,11 +12,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("dtype,dropout", [(torch.float32, 0.0), (torch.bfloat16, 0.0), (torch.float32, 0.2)])
-@pytest.mark.parametrize("L", [1024, 8192])          # tile backward (fewer than 12288 rows) and, in float32, row-group backward
-def test_graph_replay_equals_eager(L, dtype, dropout):
+@pytest.mark.parametrize("dtype,dropout,tile_backward", [(torch.float32, 0.0, None), (torch.bfloat16, 0.0, None), (torch.float32, 0.2, None),
+                                                         (torch.float32, 0.0, False), (torch.float32, 0.2, False)])
+@pytest.mark.parametrize("L", [1024, 8192])
+def test_graph_replay_equals_eager(L, dtype, dropout, tile_backward, monkeypatch):
+    """tile_backward None: the library's choice (tiles); False: the backward on the row groups."""
     from bpt_amd import graphbuilder as gb
     from bpt_amd import graphop
+    monkeypatch.setattr(graphop, "TILE_BACKWARD", tile_backward)
     g = gb.BinaryPartition(L, True, 4, 10)
     src, dst, _ = g.get_edges()
     n = g.number_of_nodes
