@@ -1910,7 +1910,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 // time (126 against 85 us at L = 4096, k = 32); letting the source side recompute p and ds (two more products there,
 // delta (n, H) handed over) measured slower than either on every graph tried.
 template <typename T, int H, int D, int HW, bool PIPE, bool DROP, bool BIAS>
-__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : 3))) void k_attn_bwd_dst_tile(
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : DROP || BIAS ? 3 : 4))) void k_attn_bwd_dst_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
     const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds, float *__restrict__ ws_dq,
     float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv, const float *__restrict__ bias,
@@ -1926,9 +1926,12 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
     const size_t mrow = (size_t)max(t.member.x, 0) * (C * sizeof(T)) + t.offa;
     float2 *const pds_h = pds + (size_t)t.head * (size_t)P.n_edges;     // this head's part of the scratch
-    float qb[16], dob[16], delta, lse_c;
+    // the member's dO columns live in LDS (lane-major, read back before every product with them): with them in registers
+    // the kernel needs 144 and a SIMD holds three wavefronts, without them 128 and four
+    __shared__ float4 dob_lds[HW][4][WAVE];
+    float qb[16], delta, lse_c;
     {
-        float ob[16];
+        float ob[16], dob[16];
         tile_load16(reinterpret_cast<const char *>(q) + mrow, qb);
         tile_load16(reinterpret_cast<const char *>(d_o) + mrow, dob);
         tile_load16(reinterpret_cast<const char *>(o) + mrow, ob);
@@ -1938,6 +1941,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         part += __shfl_xor(part, 16);
         delta = part + __shfl_xor(part, 32);                      // dO . O of member c, this head
         lse_c = lse[(size_t)max(t.member.x, 0) * H + t.head];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dob_lds[t.wv][i][t.lane] = make_float4(dob[4 * i], dob[4 * i + 1], dob[4 * i + 2], dob[4 * i + 3]);
     }
     floatx4v acc[4];
 #pragma unroll
@@ -1974,7 +1979,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             }
         };
         auto compute = [&](const Blk &B) {
-            const floatx4v st = tile_dot(B.kr, qb), dp = tile_dot(B.va, dob);
+            const floatx4v st = tile_dot(B.kr, qb);
+            float dob[16];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float4 x = dob_lds[t.wv][i][t.lane];
+                dob[4 * i] = x.x; dob[4 * i + 1] = x.y; dob[4 * i + 2] = x.z; dob[4 * i + 3] = x.w;
+            }
+            const floatx4v dp = tile_dot(B.va, dob);
             float ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
