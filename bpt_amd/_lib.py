@@ -18,7 +18,7 @@ class PlanStruct(ctypes.Structure):
                 ("n_rows", c_i64), ("n_edges", c_i64), ("n_items", c_i64), ("n_heavy", c_i64), ("n_slots", c_i64),
                 ("grp_members", c_vp), ("grp_ptr", c_vp), ("grp_entries", c_vp), ("grp_pairs", c_vp),
                 ("grp_chunks", c_vp), ("n_groups", c_i64), ("grp_R", c_i64), ("grp_max_chunk", c_i64),
-                ("n_grp_entries", c_i64), ("grp_eids", c_vp)]
+                ("n_grp_entries", c_i64), ("grp_eids", c_vp), ("grp_bias_idx", c_vp)]
 
 
 class PlanInfo(ctypes.Structure):

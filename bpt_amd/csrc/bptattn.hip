@@ -1773,6 +1773,17 @@ __device__ __forceinline__ void tile_pair_eids(const bpt_plan &P, int first_entr
 #pragma unroll
     for (int r = 0; r < 4; ++r) xe[r] = P.grp_eids[(size_t)min(first_entry + r, p_end - 1) * TILE_R + c];
 }
+// the rows of the score term (and of its gradient) of the same pairs: the plan's own numbering where it gives one
+// (grp_bias_idx), else the edge ids
+__device__ __forceinline__ void tile_pair_bias_rows(const bpt_plan &P, int first_entry, int p_end, int c, const int (&xe)[4], int (&bi)[4]) {
+    if (P.grp_bias_idx) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) bi[r] = P.grp_bias_idx[(size_t)min(first_entry + r, p_end - 1) * TILE_R + c];
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) bi[r] = xe[r];
+    }
+}
 
 // PIPE: the rows of the next block are loaded while one is used (two-stage register pipeline).  Pays on graphs with few,
 // tall tiles (a dense window graph: 9 blocks per tile, two wavefronts per SIMD in all), costs a wavefront per SIMD:
@@ -1832,13 +1843,18 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         float4 vr[4];
         int mk[4];
         int xe[DROP || BIAS ? 4 : 1];
+        int bi[BIAS ? 4 : 1];                                     // rows of the score term of the block's pairs
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            if constexpr (DROP) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            else if constexpr (BIAS) {
+                if (!P.grp_bias_idx) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            }
+            if constexpr (BIAS) tile_pair_bias_rows(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe, B.bi);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -1850,7 +1866,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 B.vr[r] = *reinterpret_cast<const float4 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
             if constexpr (BIAS) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.bi[r] * (uint32_t)H) + t.head];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -1952,13 +1968,18 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         float4 kc[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 g + r
         int pos[4], mk[4];
         int xe[DROP || BIAS ? 4 : 1];
+        int bi[BIAS ? 4 : 1];                                     // rows of the score term of the block's pairs
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            if constexpr (DROP) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            else if constexpr (BIAS) {
+                if (!P.grp_bias_idx) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            }
+            if constexpr (BIAS) tile_pair_bias_rows(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe, B.bi);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -1975,7 +1996,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 B.kc[r] = *reinterpret_cast<const float4 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
             if constexpr (BIAS) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.bi[r] * (uint32_t)H) + t.head];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -1999,7 +2020,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 pe *= mt;                                         // what multiplies v (forward) and dO (dV)
                 if (has) {
                     pds_h[B.pos[r]] = make_float2(pe, ds[r]);
-                    if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
+                    if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.bi[BIAS ? r : 0] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
                 }
             }
             tile_axpy(ds, B.kc, acc);
@@ -2151,13 +2172,18 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
         uint2 vr[4];
         int mk[4];
         int xe[DROP || BIAS ? 4 : 1];
+        int bi[BIAS ? 4 : 1];                                     // rows of the score term of the block's pairs
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            if constexpr (DROP) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            else if constexpr (BIAS) {
+                if (!P.grp_bias_idx) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            }
+            if constexpr (BIAS) tile_pair_bias_rows(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe, B.bi);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -2168,7 +2194,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             for (int r = 0; r < 4; ++r) B.vr[r] = *reinterpret_cast<const uint2 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
             if constexpr (BIAS) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.bi[r] * (uint32_t)H) + t.head];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -2267,13 +2293,18 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
         uint2 kc[4];
         int mk[4], pos[4];
         int xe[DROP || BIAS ? 4 : 1];
+        int bi[BIAS ? 4 : 1];                                     // rows of the score term of the block's pairs
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP || BIAS) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            if constexpr (DROP) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            else if constexpr (BIAS) {
+                if (!P.grp_bias_idx) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
+            }
+            if constexpr (BIAS) tile_pair_bias_rows(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe, B.bi);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -2289,7 +2320,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             for (int r = 0; r < 4; ++r) B.kc[r] = *reinterpret_cast<const uint2 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
             if constexpr (BIAS) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.bi[r] * (uint32_t)H) + t.head];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -2306,7 +2337,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
                 pe *= mt;                                         // what multiplies v (forward) and dO (dV)
                 if (has) {
                     pds_h[B.pos[r]] = pack_bf16(pe, ds[r]);
-                    if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.xe[r] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
+                    if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.bi[BIAS ? r : 0] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
                 }
             }
             Bf4 da;
@@ -4103,6 +4134,8 @@ int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k,
     if ((drop.thr != 0 || bias) && !has_groups(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4) && !has_tiles(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4))
         return BPT_ERR_UNSUPPORTED;
     if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
+    // only the tile kernels look the rows of the score term up in a numbering of the plan's own
+    if (bias && plan_in->grp_bias_idx && !has_tiles(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_PLAN;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(workspace))
         return BPT_ERR_UNSUPPORTED;
     const int64_t need = bpt_workspace_bytes(BPT_OP_ATTN_FWD, plan_in, nullptr, h, d, dtype);
@@ -4143,6 +4176,7 @@ int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, co
         return BPT_ERR_UNSUPPORTED;
     if ((bias != nullptr) != (ds_out != nullptr)) return BPT_ERR_NULL;       // the score term and its gradient go together
     if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
+    if (bias && plan_in->grp_bias_idx && !tiled_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_PLAN;
     // (the two sides may have different row counts: attention to a memory of another length, attention.py:144-168)
     if (plan_in->n_edges != plan_out->n_edges) return BPT_ERR_PLAN;
     if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return BPT_ERR_NULL;

@@ -461,11 +461,12 @@ def _check_bias(bias, n_edges, h, device, cfg):
         raise RuntimeError("the per-edge score term needs the row-group kernels")
 
 
-def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, dropout_p=0.0, seed=0, bias=None):
+def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, dropout_p=0.0, seed=0, bias=None, bias_by_pair=False):
     """o[dst] = sum over in-edges drop(softmax((q[dst].k[src] + bias[e])*scale)) v[src]; returns (o, lse) with lse
     (n, h) float32 in base-2 units.  Arithmetic of modules/attention.py:66-77 in one pass.  dropout_p > 0
     drops attention probabilities as attention.py:73 does; the mask is a function of (seed, graph), see
-    attention_dropout_mask.  bias: None or the float32 (E + 1, h) score term of rel_bias_forward."""
+    attention_dropout_mask.  bias: None or the float32 (E + 1, h) score term of rel_bias_forward, its rows by edge id or,
+    with bias_by_pair, by the numbers attention_pair_rows() gives the edges (tile kernels only)."""
     cfg = _SETTINGS
     _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v)
     _check_bias(bias, eid_c.size(0), _hd(q)[0], q.device, cfg)
@@ -476,13 +477,17 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     _expect_shape(v, k.shape, "v")
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
+    tiles = False
     if not _attention_groups(plan, dropout_p, bias, q, k, cfg):
         ref = plan.ref
     elif _tiles(q, h, d, plan, dropout_p, bias, cfg):
         plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=_tile_seg_len(plan), prefer_device=True)
-        ref = ctypes.byref(plan.ensure_groups(TILE_ROWS)["struct"])
+        ref = ctypes.byref(plan.bias_rows(TILE_ROWS)["struct"] if bias_by_pair else plan.ensure_groups(TILE_ROWS)["struct"])
+        tiles = True
     else:
         ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, cfg))["struct"])
+    if bias_by_pair and not (tiles and bias is not None):
+        raise RuntimeError("bias_by_pair: this call does not run on the tile kernels (ask attention_pair_rows() first)")
     o = torch.empty_like(q)
     lse = torch.empty((q.size(0), h), dtype=torch.float32, device=q.device)
     dt = _dtype(q)
@@ -495,9 +500,10 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
 
 
 def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, do, scale=None,
-                       dropout_p=0.0, seed=0, bias=None):
-    """(dq, dk, dv) of attention_forward (same dropout_p, seed and bias).  With bias a fourth result: ds, float32
-    (E, h), the gradient with respect to q.k + bias of every edge and head (= the gradient of bias)."""
+                       dropout_p=0.0, seed=0, bias=None, bias_by_pair=False):
+    """(dq, dk, dv) of attention_forward (same dropout_p, seed, bias and bias_by_pair).  With bias a fourth result: ds,
+    float32 (E, h), the gradient with respect to q.k + bias of every edge and head (= the gradient of bias), its rows in the
+    order of bias's."""
     cfg = _SETTINGS
     _check_all(row=row, indptr_r=indptr_r, eid_r=eid_r, indices_r=indices_r, col=col, indptr_c=indptr_c,
                eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v, o=o, lse=lse)
@@ -522,18 +528,22 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     ds = torch.empty((eid_c.size(0) + 1, h), dtype=torch.float32, device=q.device) if bias is not None else None
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref
+    tiles = False
     if _attention_groups(plan_in, dropout_p, bias, q, k, cfg) and plan_in.covers_all_edges and plan_out.covers_all_edges:
         if _tiles(q, h, d, plan_in, dropout_p, bias, cfg) and _tiles_backward(plan_in, q.dtype, bias):
             seg = _tile_seg_len(plan_in)
             plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg, prefer_device=True)
             plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg, prefer_device=True)
             # the destination side writes (p, ds) by its own pair numbers; the source side finds them through its pair mapping
-            in_ref = ctypes.byref(plan_in.ensure_groups(TILE_ROWS)["struct"])
+            in_ref = ctypes.byref(plan_in.bias_rows(TILE_ROWS)["struct"] if bias_by_pair else plan_in.ensure_groups(TILE_ROWS)["struct"])
             out_ref = ctypes.byref(plan_out.linked_to(plan_in, TILE_ROWS, partner_order=None, pair_numbers=True))
+            tiles = True
         else:
             R = _group_rows(q, h, d, plan_in, cfg)
             in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
             out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
+    if bias_by_pair and not (tiles and bias is not None):
+        raise RuntimeError("bias_by_pair: this call does not run on the tile kernels (ask attention_pair_rows() first)")
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
     with _on_device_of(q):
         check_attn(_LIB.bpt_attention_backward(in_ref, out_ref, _ptr(q), _ptr(k), _ptr(v), _ptr(bias), _ptr(o), _ptr(do),
@@ -543,6 +553,27 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     if bias is not None:
         return dq, dk, dv, ds[:-1]
     return dq, dk, dv
+
+
+def attention_pair_rows(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p=0.0):
+    """For a step with a per-edge score term: None, or, where attention_forward and attention_backward will both run on
+    the tile kernels for these arguments, the (E,) int64 tensor that numbers the edges the way the tiles meet them (the pair
+    numbers of the in-CSR's tile plan).  A score term stored in that order (row number[e] for edge e) and passed with
+    bias_by_pair=True is read, and its gradient written, in neighbouring rows per tile instead of rows scattered by edge
+    id."""
+    cfg = _SETTINGS
+    if q.dim() != 3 or not q.is_cuda:
+        return None
+    h, d = _hd(q)
+    plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0))
+    plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0))
+    marker = q                                             # (stands for "a score term is given" in the choices below)
+    if not (attention_supported(q) and _attention_groups(plan_in, dropout_p, marker, q, k, cfg) and plan_in.covers_all_edges
+            and plan_out.covers_all_edges and _tiles(q, h, d, plan_in, dropout_p, marker, cfg)
+            and _tiles_backward(plan_in, q.dtype, marker)):
+        return None
+    plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=_tile_seg_len(plan_in), prefer_device=True)
+    return plan_in.bias_rows(TILE_ROWS)["pair_of_eid"]
 
 
 def attention_dropout_mask(col, indptr_c, eid_c, indices_c, q, k, dropout_p, seed):
@@ -624,20 +655,16 @@ def _tiles(q, h, d, plan, dropout_p, bias, cfg):
 
 
 def _tiles_backward(plan, dtype, bias=None):
-    """The backward runs on tiles wherever the forward does, except in float32 with the score term on large sparse graphs.
-    float32 (8 x 64), step time on tiles against row groups: L = 8192, k = 4 0.175 against 0.187 ms, with attention
-    dropout 0.178 against 0.203; the 32-graph batch 0.298 against 0.307; L = 32768, k = 4 0.807 against 0.841; L = 4096,
-    k = 1 ... 32 level to 27 % faster, window 128 1.9 x.  With the score term the tile kernels fetch it per pair and head
-    (a wavefront owns one head) where the row-group kernel fetches all heads of a pair at once, and lose their lead on
-    graphs of 12288 rows and more with mean degree under 32 (L = 8192, k = 4: 0.285 against 0.284 ms; the 32-graph batch
-    0.461 against 0.449): those stay on the row groups.  bfloat16 rows: always tiles (a block costs six matrix instructions
-    instead of 32 to 48; every graph measured runs faster, L = 8192, k = 4: 0.112 against 0.135 ms; L = 32768, k = 8, 16
-    heads: 1.20 against 1.49; window 128: 0.081 against 0.188)."""
+    """The backward runs on tiles wherever the forward does.  float32 (8 x 64), step time on tiles against row groups:
+    L = 8192, k = 4 0.175 against 0.187 ms, with attention dropout 0.178 against 0.203; the 32-graph batch 0.298 against
+    0.307; L = 32768, k = 4 0.807 against 0.841; L = 4096, k = 1 ... 32 level to 27 % faster, window 128 1.9 x.  With the
+    score term: L = 8192, k = 4 0.281 against 0.288 ms and the 32-graph batch 0.445 against 0.449 when the term is stored
+    in the tiles' own order (attention_pair_rows), level with it stored by edge id.  bfloat16: a block costs six matrix
+    instructions instead of 32 to 48 and every graph measured runs faster (L = 8192, k = 4: 0.112 against 0.135 ms;
+    L = 32768, k = 8, 16 heads: 1.20 against 1.49; window 128: 0.081 against 0.188)."""
     if TILE_BACKWARD is not None:
         return TILE_BACKWARD
-    if dtype == torch.bfloat16 or bias is None:
-        return True
-    return plan.n_rows < 12288 or plan.n_edges >= 32 * max(plan.n_rows, 1)
+    return True
 
 
 def _tile_seg_len(plan):

@@ -108,11 +108,22 @@ class BPTRelAttention(Function):
         aux = _rel_aux(etype, col, indptr_c, eid_c, table.size(0))
         table = table.contiguous()
         ctx.on_chip = _g.rel_rows_supported(q) and aux["n_used"] <= _g.REL_MAX_USED_TYPES and not _g.force_generic_enabled()
+        # where forward and backward both run on the tile kernels, the term and its gradient are stored in the order in
+        # which the tiles meet the edges (rows_slot: the row of every in-CSR slot) instead of by edge id
+        pair = _g.attention_pair_rows(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p) if ctx.on_chip else None
+        ctx.rows_slot = None
+        if pair is not None:
+            held = aux.get("rows_slot")
+            if held is None or held[0] is not pair:
+                held = aux["rows_slot"] = (pair, pair.index_select(0, eid_c).contiguous())
+            ctx.rows_slot = held[1]
         if ctx.on_chip:
-            bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["number_slot"], q, table, used_types=aux["used_types"])
+            bias = _g.rel_bias_forward(col, indptr_c, eid_c if ctx.rows_slot is None else ctx.rows_slot, aux["number_slot"], q, table,
+                                       used_types=aux["used_types"])
         else:
             bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["etype_slot"], q, table)
-        o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed, bias=bias)
+        o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed, bias=bias,
+                                      bias_by_pair=ctx.rows_slot is not None)
         ctx.save_for_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, bias, table)
         ctx.scale, ctx.dropout_p, ctx.seed, ctx.aux, ctx.etype = scale, dropout_p, seed, aux, etype
         return o
@@ -122,9 +133,11 @@ class BPTRelAttention(Function):
         row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, bias, table = ctx.saved_tensors
         aux = ctx.aux
         dq, dk, dv, ds = _g.attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c,
-                                               q, k, v, o, lse, do, ctx.scale, ctx.dropout_p, ctx.seed, bias=bias)
+                                               q, k, v, o, lse, do, ctx.scale, ctx.dropout_p, ctx.seed, bias=bias,
+                                               bias_by_pair=ctx.rows_slot is not None)
         if ctx.on_chip:
-            dtable = _g.rel_bias_backward(col, indptr_c, eid_c, aux["number_slot"], aux["used"], aux["used_types"], ds, q, table, dq)
+            dtable = _g.rel_bias_backward(col, indptr_c, eid_c if ctx.rows_slot is None else ctx.rows_slot, aux["number_slot"], aux["used"],
+                                          aux["used_types"], ds, q, table, dq)
         else:
             t_row, t_indptr, t_order, t_dst = _rel_type_rows(aux, ctx.etype, col, indptr_c, eid_c, table.size(0))
             h = q.size(1)

@@ -142,6 +142,19 @@ def link_groups_host(grp_dst, grp_src, n_edges):
     return out
 
 
+def _bias_rows_of(groups_struct, pair_eid, eids, n_edges):
+    """For a plan's tile groups: the struct with grp_bias_idx = the pair number of every (entry, member) (n_edges where
+    there is no such pair), laid out like grp_eids, and the pair number of every edge id."""
+    device = eids.device
+    pair_of_eid = torch.empty(n_edges + 1, dtype=torch.int64, device=device)
+    pair_of_eid[pair_eid.to(torch.int64)] = torch.arange(n_edges, dtype=torch.int64, device=device)
+    pair_of_eid[n_edges] = n_edges
+    bias_idx = pair_of_eid.index_select(0, eids.reshape(-1).to(torch.int64)).to(torch.int32).contiguous()
+    st = PlanStruct.from_buffer_copy(groups_struct)
+    st.grp_bias_idx = bias_idx.data_ptr()
+    return {"struct": st, "bias_idx": bias_idx, "pair_of_eid": pair_of_eid[:n_edges].contiguous()}
+
+
 def pair_numbers_host(grp_mine, grp_theirs, n_edges):
     """For every (entry, member) of `grp_mine` the number, among the pairs of `grp_theirs`, of the pair that is the same
     edge (pairs are numbered entry by entry, members ascending: grp["pair_eid"][number] = edge id); 0 where the entry has
@@ -173,7 +186,8 @@ class Plan:
 
     def device_bytes(self):
         """Device memory held by this plan, its row groups and pair mappings."""
-        return _tensor_bytes(self._dev) + _tensor_bytes(list(self._groups.values())) + _tensor_bytes(list(self._links.values()))
+        return (_tensor_bytes(self._dev) + _tensor_bytes(list(self._groups.values())) + _tensor_bytes(list(self._links.values()))
+                + _tensor_bytes(list(self._bias_rows.values())))
 
     def __init__(self, row, indptr, eid, indices, n_rows, n_index_nodes, device, seg_len=DEFAULT_SEG_LEN):
         arrays, info = build_plan_host(row, indptr, eid, indices, n_rows, n_index_nodes, seg_len)
@@ -187,6 +201,7 @@ class Plan:
         self._host = arrays                  # kept for the (lazy) row-group construction
         self._groups = {}
         self._links = {}
+        self._bias_rows = {}
         self._lock = threading.Lock()
         # one allocation, 256-byte aligned sections (the items array is read as 16-byte vectors)
         self.seg_len = arrays["seg_len"]
@@ -233,6 +248,20 @@ class Plan:
                 st.grp_eids = dev["eids"].data_ptr()
                 hit = {"host": grp, "dev": dev, "struct": st}
                 self._groups[(R, order_mode)] = hit
+        return hit
+
+    def bias_rows(self, R=TILE_GROUP_R):
+        """The tile groups with the rows of the per-edge score term numbered by the plan's own pairs (grp_bias_idx): dict
+        with "struct" (the `bpt_plan`) and "pair_of_eid" (the pair number of every edge id).  Needs a plan that covers
+        every edge."""
+        with self._lock:
+            hit = self._bias_rows.get(R)
+        if hit is None:
+            g = self.ensure_groups(R)
+            pair_eid = torch.from_numpy(np.ascontiguousarray(g["host"]["pair_eid"])).to(self.device)
+            hit = _bias_rows_of(g["struct"], pair_eid, g["dev"]["eids"], self.n_edges)
+            with self._lock:
+                self._bias_rows[R] = hit
         return hit
 
     def linked_to(self, plan_src, R=GROUP_R, order=None, partner_order=GROUP_ORDER_SRC, pair_numbers=False):
@@ -342,7 +371,7 @@ class DevicePlan:
         if seg_len is None:
             seg_len = FORCE_SEG_LEN if FORCE_SEG_LEN is not None else self._auto_seg_len(row, indptr)
         self.seg_len = int(seg_len)
-        self._groups, self._links, self._lock = {}, {}, threading.Lock()
+        self._groups, self._links, self._bias_rows, self._lock = {}, {}, {}, threading.Lock()
         lib = plan_lib()
         U, E = int(row.numel()), self.n_edges
         b = (ctypes.c_int64 * 4)()
@@ -440,6 +469,18 @@ class DevicePlan:
                 hit = _Groups(dev=dev, struct=st, R=R, n_edges=E)
                 torch.cuda.current_stream(self.device).synchronize()      # the clones above ran on the building stream
                 self._groups[(R, by_mask)] = hit
+        return hit
+
+    def bias_rows(self, R=TILE_GROUP_R):
+        """As Plan.bias_rows, from the groups built on the GPU."""
+        with self._lock:
+            hit = self._bias_rows.get(R)
+        if hit is None:
+            g = self.ensure_groups(R)
+            hit = _bias_rows_of(g["struct"], g["dev"]["pair_eid"], g["dev"]["eids"], self.n_edges)
+            torch.cuda.current_stream(self.device).synchronize()      # complete before another stream may read it
+            with self._lock:
+                self._bias_rows[R] = hit
         return hit
 
     def linked_to(self, plan_src, R=GROUP_R, order=None, partner_order=GROUP_ORDER_SRC, pair_numbers=False):

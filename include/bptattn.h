@@ -80,6 +80,12 @@ typedef struct {
                                     [u * grp_R + m]; n_edges where the entry's mask has no bit m and in the 8
                                     entries of padding.  Needed by the attention calls that take a per-edge score
                                     term or dropout and by the row-group kernels of the SDDMM / SpMM-shaped ops */
+    const int32_t *grp_bias_idx; /* NULL, or laid out like grp_eids (grp_R = 16 only): the row of `bias` and of `ds_out`
+                                    that belongs to (entry u, member m), n_edges where there is no such pair.  NULL: the
+                                    edge id (grp_eids).  With the plan's own pair numbers here (the entry's first pair +
+                                    the member's rank in the mask) a tile's rows of the score term are neighbours in
+                                    memory instead of scattered by edge id; forward and backward must then be given the
+                                    same numbering, and whoever produces `bias` / consumes `ds_out` uses it too */
 } bpt_plan;
 
 const char *bpt_strerror(int status);

@@ -152,3 +152,46 @@ def test_graph_without_edges_gives_a_zero_table_gradient(ops):
     used_types = torch.zeros(0, dtype=torch.int32, device=DEV)
     dtable = graphop.rel_bias_backward(col, indptr, eid, et, used, used_types, torch.zeros(1, h, device=DEV), q, table, dq)
     assert float(dtable.abs().max()) == 0.0 and torch.equal(dq, torch.ones_like(q))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("gname", ["bpt512_k4", "multigraph", "fc_w100"])
+@pytest.mark.parametrize("p", [0.0, 0.25])
+def test_score_term_in_the_order_of_the_tiles_gives_the_same_step(ops, gname, dtype, p):
+    """A score term stored by the tile plan's pair numbers (attention_pair_rows, bias_by_pair) instead of by edge id:
+    the same o, lse, dq, dk, dv bit for bit, and ds the same values in the other order."""
+    graphop, _ = ops
+    h, d = 8, 64
+    c = case(gname)
+    q, k, v, do = (rand((c.n, h, d), dtype, s, 1.0 / 8).to(DEV) for s in (51, 52, 53, 54))
+    term = rand((c.E, h), torch.float32, 55, 0.5).to(DEV)
+    pair = graphop.attention_pair_rows(*c.out, *c.inn, q, k, p)
+    assert pair is not None and pair.shape == (c.E,) and torch.equal(torch.sort(pair).values, torch.arange(c.E, device=DEV))
+    zero = torch.zeros(1, h, device=DEV)
+    by_eid = torch.cat([term, zero])
+    by_pair = torch.cat([torch.empty_like(term).index_copy_(0, pair, term), zero])
+    got = {}
+    for name, bias, flag in (("eid", by_eid, False), ("pair", by_pair, True)):
+        o, lse = graphop.attention_forward(*c.inn, q, k, v, dropout_p=p, seed=77, bias=bias, bias_by_pair=flag)
+        got[name] = (o, lse) + tuple(graphop.attention_backward(*c.out, *c.inn, q, k, v, o, lse, do, dropout_p=p, seed=77, bias=bias,
+                                                               bias_by_pair=flag))
+    for a, b, what in zip(got["eid"][:5], got["pair"][:5], ("o", "lse", "dq", "dk", "dv")):
+        assert torch.equal(a, b), what
+    assert torch.equal(got["eid"][5], got["pair"][5].index_select(0, pair)), "ds"
+
+
+def test_the_order_of_the_tiles_is_offered_only_where_both_passes_run_on_tiles(ops):
+    graphop, _ = ops
+    c = case("bpt512_k4")
+    q, k, v = (rand((c.n, 8, 64), torch.float32, s, 1.0 / 8).to(DEV) for s in (61, 62, 63))
+    assert graphop.attention_pair_rows(*c.out, *c.inn, q, k) is not None
+    old = graphop.set_group_rows(4)                       # row groups of 4: no tiles
+    try:
+        assert graphop.attention_pair_rows(*c.out, *c.inn, q, k) is None
+        bias = torch.zeros(c.E + 1, 8, device=DEV)
+        with pytest.raises(RuntimeError, match="bias_by_pair"):
+            graphop.attention_forward(*c.inn, q, k, v, bias=bias, bias_by_pair=True)
+    finally:
+        graphop.set_group_rows(old)
+    q32 = rand((c.n, 8, 32), torch.float32, 64, 1.0 / 8).to(DEV)          # 32 columns per head: no tile kernels
+    assert graphop.attention_pair_rows(*c.out, *c.inn, q32, q32) is None

@@ -37,12 +37,8 @@ def test_backward_rule():
     f32, bf16 = torch.float32, torch.bfloat16
     term = torch.empty(1)                                                  # (any tensor: a score term is given)
     for plan in (fake_plan(8191, 98305), fake_plan(65535, 3293955), fake_plan(16383, 430237), fake_plan(33598, 573520)):
-        assert graphop._tiles_backward(plan, f32)                          # float32 without the score term: always
-        assert graphop._tiles_backward(plan, bf16) and graphop._tiles_backward(plan, bf16, term)     # bfloat16: always
-    assert graphop._tiles_backward(fake_plan(8191, 98305), f32, term)            # with the term: small graph
-    assert graphop._tiles_backward(fake_plan(65535, 3293955), f32, term)         # mean degree 50
-    assert not graphop._tiles_backward(fake_plan(16383, 430237), f32, term)      # L = 8192, k = 4: row groups
-    assert not graphop._tiles_backward(fake_plan(33598, 573520), f32, term)      # the 32-graph batch
+        for dtype in (f32, bf16):                                          # wherever the forward runs on tiles
+            assert graphop._tiles_backward(plan, dtype) and graphop._tiles_backward(plan, dtype, term)
     old = graphop.TILE_BACKWARD
     try:
         graphop.TILE_BACKWARD = False
