@@ -105,6 +105,38 @@ def test_attention_checks(g):
         g.rel_bias_forward(*INN[:3], INN[3][:-1], node(), torch.zeros(1000, D))                    # a type per slot
 
 
+def test_rel_bias_checks(g):
+    """The score term's own ops: every tensor against the graph and the table before a plan is asked for."""
+    i32 = lambda n, v=0: torch.full((n,), v, dtype=torch.int32)
+    table, used, used_types, ds = torch.zeros(1000, D), i32(1000, -1), i32(3), torch.zeros(E + 1, H)
+    ok = (*INN[:3], INN[3], used, used_types, ds, node(), table, node())
+    def bad(**kw):
+        names = ("col", "indptr_c", "eid_c", "number_slot", "used", "used_types", "ds", "q", "table", "dq")
+        args = [kw.get(n, a) for n, a in zip(names, ok)]
+        with pytest.raises(ValueError):
+            g.rel_bias_backward(*args)
+    bad(table=torch.zeros(1000, D // 2))                 # other head size
+    bad(used=i32(999, -1))                               # one entry per table row
+    bad(used=torch.full((1000,), -1, dtype=torch.int64))
+    bad(used_types=torch.zeros(3, dtype=torch.int64))
+    bad(used_types=i32(1001))                            # more used types than types
+    bad(ds=torch.zeros(E - 1, H))                        # a row per edge
+    bad(ds=torch.zeros(E + 1, H - 1))
+    bad(ds=torch.zeros(E + 1, H, dtype=torch.float64))
+    bad(dq=node(n=N - 1))
+    bad(number_slot=INN[3][:-1])                         # a type number per slot
+    with pytest.raises(AssertionError):
+        g.rel_bias_backward(*ok)                         # (well formed: reaches the plan cache)
+    with pytest.raises(ValueError):
+        g.rel_bias_forward(*INN[:3], INN[3], node(), table, used_types=torch.zeros(3, dtype=torch.int64))
+    with pytest.raises(ValueError):
+        g.rel_bias_forward(*INN[:3], INN[3], node(), table, used_types=i32(1001))
+    with pytest.raises(ValueError):
+        g.rel_bias_forward(*INN[:3], INN[3], node(), torch.zeros(1000, D + 1), used_types=i32(3))
+    with pytest.raises(AssertionError):
+        g.rel_bias_forward(*INN[:3], INN[3], node(), table, used_types=i32(3))
+
+
 def test_well_formed_calls_get_past_the_checks(g):
     # the same calls with fitting tensors reach the plan cache (which this fixture turns into an AssertionError)
     with pytest.raises(AssertionError):
