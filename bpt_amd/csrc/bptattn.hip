@@ -3368,11 +3368,11 @@ constexpr int REL_MAX_USED = 240;         // type numbers whose table rows fit t
 // LDS of k_rel_bias_bwd with nw wavefronts: their sums, the table rows, their staged ds values
 inline size_t rel_bwd_lds(int nw, int64_t n_used, int h) { return ((size_t)(nw + 1) * n_used * 64 + (size_t)nw * WAVE * h) * 4; }
 // wavefronts per workgroup of k_rel_bias_bwd for n_used types: four or two while two workgroups fit a compute unit's
-// 160 KB of LDS, else one
-inline int rel_bwd_waves(int64_t n_used, int h) {
+// 160 KB of LDS, else one (large_lds false: while one workgroup stays inside the 64 KB every kernel may take)
+inline int rel_bwd_waves(int64_t n_used, int h, bool large_lds = true) {
     for (int nw = 4; nw >= 2; nw >>= 1)
-        if (rel_bwd_lds(nw, n_used, h) <= 80 * 1024) return nw;
-    return rel_bwd_lds(1, n_used, h) <= 128 * 1024 ? 1 : 0;
+        if (rel_bwd_lds(nw, n_used, h) <= (large_lds ? 80 : 64) * 1024) return nw;
+    return rel_bwd_lds(1, n_used, h) <= (large_lds ? 128 : 64) * 1024 ? 1 : 0;
 }
 
 // a kernel may take more than 64 KB of dynamic LDS only after it has been told so (once per kernel and device)
@@ -3384,7 +3384,10 @@ int allow_large_lds(K kernel, size_t bytes) {
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32) return BPT_ERR_UNSUPPORTED;
     if (done.load(std::memory_order_acquire) & (1u << dev)) return BPT_OK;
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return (int)e;
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return BPT_ERR_UNSUPPORTED;          // (the caller then takes a configuration inside 64 KB)
+    }
     done.fetch_or(1u << dev, std::memory_order_release);
     return BPT_OK;
 }
@@ -3403,13 +3406,22 @@ int launch_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const
 template <typename T, int H>
 int run_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const void *table, const int32_t *used, const int32_t *used_types,
                      int64_t n_types, int64_t n_used, void *dq, void *dtable, float *ws, hipStream_t s) {
-    const int nw = rel_bwd_waves(n_used, H);
-    const int n_parts = (int)std::min<int64_t>(REL_MAX_PARTS, std::max<int64_t>(1, (P->n_edges + nw * 128 - 1) / (nw * 128)));
     float *ws_dq = ws, *part = ws + (size_t)P->n_slots * H * 64;       // partial rows of dq of the split rows, then the partial tables
+    int n_parts = 0;
+    auto launch = [&](int nw) {
+        n_parts = (int)std::min<int64_t>(REL_MAX_PARTS, std::max<int64_t>(1, (P->n_edges + nw * 128 - 1) / (nw * 128)));
+        return nw == 4   ? launch_rel_bias_bwd<T, H, 4>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s)
+               : nw == 2 ? launch_rel_bias_bwd<T, H, 2>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s)
+                         : launch_rel_bias_bwd<T, H, 1>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s);
+    };
     if (P->n_edges > 0) {
-        int st = nw == 4   ? launch_rel_bias_bwd<T, H, 4>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s)
-                 : nw == 2 ? launch_rel_bias_bwd<T, H, 2>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s)
-                           : launch_rel_bias_bwd<T, H, 1>(P, ds, q, table, used_types, n_used, dq, ws_dq, part, n_parts, s);
+        const int nw = rel_bwd_waves(n_used, H);
+        int st = launch(nw);
+        if (st == BPT_ERR_UNSUPPORTED && rel_bwd_lds(nw, n_used, H) > 64 * 1024) {      // more than 64 KB of LDS refused by the runtime
+            const int small = rel_bwd_waves(n_used, H, false);
+            if (small == 0) return BPT_ERR_UNSUPPORTED;
+            st = launch(small);
+        }
         if (st != BPT_OK) return st;
     }
     // (without edges there are no partial tables and no partial rows: every row of dtable becomes zero)
