@@ -3367,12 +3367,19 @@ constexpr int REL_MAX_USED = 240;         // type numbers whose table rows fit t
 
 // LDS of k_rel_bias_bwd with nw wavefronts: their sums, the table rows, their staged ds values
 inline size_t rel_bwd_lds(int nw, int64_t n_used, int h) { return ((size_t)(nw + 1) * n_used * 64 + (size_t)nw * WAVE * h) * 4; }
-// wavefronts per workgroup of k_rel_bias_bwd for n_used types: four or two while two workgroups fit a compute unit's
-// 160 KB of LDS, else one (large_lds false: while one workgroup stays inside the 64 KB every kernel may take)
+// wavefronts per workgroup of k_rel_bias_bwd for n_used types: the 4, 2 or 1 that put most wavefronts on a compute unit
+// (workgroups that fit its 160 KB of LDS x wavefronts each; more per workgroup on a tie: fewer partial tables), a
+// workgroup taking at most 144 KB (large_lds false: at most the 64 KB every kernel may take).  0: no configuration fits.
 inline int rel_bwd_waves(int64_t n_used, int h, bool large_lds = true) {
-    for (int nw = 4; nw >= 2; nw >>= 1)
-        if (rel_bwd_lds(nw, n_used, h) <= (large_lds ? 80 : 64) * 1024) return nw;
-    return rel_bwd_lds(1, n_used, h) <= (large_lds ? 128 : 64) * 1024 ? 1 : 0;
+    const size_t cap = (large_lds ? 144 : 64) * 1024;
+    int best = 0, best_waves = 0;
+    for (int nw = 4; nw >= 1; nw >>= 1) {
+        const size_t lds = rel_bwd_lds(nw, n_used, h);
+        if (lds > cap) continue;
+        const int waves = nw * (int)((160 * 1024) / lds);
+        if (waves > best_waves) { best = nw; best_waves = waves; }
+    }
+    return best;
 }
 
 // a kernel may take more than 64 KB of dynamic LDS only after it has been told so (once per kernel and device)
