@@ -18,7 +18,7 @@ class PlanStruct(ctypes.Structure):
                 ("n_rows", c_i64), ("n_edges", c_i64), ("n_items", c_i64), ("n_heavy", c_i64), ("n_slots", c_i64),
                 ("grp_members", c_vp), ("grp_ptr", c_vp), ("grp_entries", c_vp), ("grp_pairs", c_vp),
                 ("grp_chunks", c_vp), ("n_groups", c_i64), ("grp_R", c_i64), ("grp_max_chunk", c_i64),
-                ("n_grp_entries", c_i64), ("grp_eids", c_vp), ("grp_bias_idx", c_vp)]
+                ("n_grp_entries", c_i64), ("grp_eids", c_vp), ("bias_by_pair", c_i64)]
 
 
 class PlanInfo(ctypes.Structure):
@@ -60,6 +60,7 @@ ATTN_API = {
     "bpt_vector_spmm_accumulate": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_vector_spmm_backward": (ctypes.c_int, [_PP, _PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_rel_bias_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_i64, c_vp] + _tail),
+    "bpt_rel_bias_forward_tiles": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp] + _tail),
     "bpt_rel_bias_backward_workspace_bytes": (c_i64, [_PP, c_i64, ctypes.c_int]),
     "bpt_rel_bias_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float, ctypes.c_float,

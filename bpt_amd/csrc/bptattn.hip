@@ -21,6 +21,8 @@
 #include <cmath>
 #include <cstdint>
 #include <mutex>
+#include <utility>
+#include <vector>
 
 #include "../../include/bptattn.h"
 
@@ -1773,16 +1775,14 @@ __device__ __forceinline__ void tile_pair_eids(const bpt_plan &P, int first_entr
 #pragma unroll
     for (int r = 0; r < 4; ++r) xe[r] = P.grp_eids[(size_t)min(first_entry + r, p_end - 1) * TILE_R + c];
 }
-// the rows of the score term (and of its gradient) of the same pairs: the plan's own numbering where it gives one
-// (grp_bias_idx), else the edge ids
-__device__ __forceinline__ void tile_pair_bias_rows(const bpt_plan &P, int first_entry, int p_end, int c, const int (&xe)[4], int (&bi)[4]) {
-    if (P.grp_bias_idx) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) bi[r] = P.grp_bias_idx[(size_t)min(first_entry + r, p_end - 1) * TILE_R + c];
-    } else {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) bi[r] = xe[r];
-    }
+// Where the score term of the pair (entry, member c) sits and its gradient goes.  BIAS == 1, stored by edge id: row eid
+// of (n_edges + 1, H), the spare last row for a pair that does not exist.  BIAS == 2, stored in the plan's own order:
+// head-major at the pair's number, x[head * n_edges + number]: the lanes of an entry touch one run of memory and no
+// index is read on the way; a pair that does not exist gets a neighbour's place, which is read and not used.
+template <int H, int BIAS>
+__device__ __forceinline__ uint32_t tile_bias_at(const bpt_plan &P, int head, int eid, int number) {
+    if constexpr (BIAS == 2) return (uint32_t)head * (uint32_t)P.n_edges + (uint32_t)min(number, (int)P.n_edges - 1);
+    else return (uint32_t)eid * (uint32_t)H + (uint32_t)head;
 }
 
 // PIPE: the rows of the next block are loaded while one is used (two-stage register pipeline).  Pays on graphs with few,
@@ -1818,7 +1818,7 @@ __device__ __forceinline__ void tile_walk(int nblk, Issue &&issue, Compute &&com
     }
 }
 
-template <typename T, int H, int D, int HW, bool PIPE, bool DROP, bool BIAS>
+template <typename T, int H, int D, int HW, bool PIPE, bool DROP, int BIAS>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 3 : 4))) void k_attn_fwd_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o, float *__restrict__ lse,
     float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv,
@@ -1827,7 +1827,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     TileCtx t;
     if (!tile_begin<T, H, D, HW>(P, t)) return;
     __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    __shared__ int fst_lds[HW][BIAS == 2 ? TILE_CHUNK : 1];      // the entries' first pair numbers: where a term in pair order sits
     int2 *ent = ent_lds[t.wv];
+    int *fst = BIAS == 2 ? fst_lds[t.wv] : nullptr;
     const int c = t.c, g = t.g;
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
     float qb[16];
@@ -1842,19 +1844,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         float kr[16];
         float4 vr[4];
         int mk[4];
-        int xe[DROP || BIAS ? 4 : 1];
-        int bi[BIAS ? 4 : 1];                                     // rows of the score term of the block's pairs
+        int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
-        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            else if constexpr (BIAS) {
-                if (!P.grp_bias_idx) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            }
-            if constexpr (BIAS) tile_pair_bias_rows(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe, B.bi);
+            if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -1864,9 +1861,15 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 B.vr[r] = *reinterpret_cast<const float4 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
-            if constexpr (BIAS) {
+            if constexpr (BIAS == 1) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.bi[r] * (uint32_t)H) + t.head];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 1>(P, t.head, B.xe[BIAS == 1 ? r : 0], 0)];
+            }
+            if constexpr (BIAS == 2) {
+                const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
+                const int fv[4] = {f4.x, f4.y, f4.z, f4.w};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 2>(P, t.head, 0, tile_pair_number(fv[r], B.mk[r], c))];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -1925,8 +1928,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 // source side's layout instead (scattered 8-byte stores here, contiguous reads there) cost this kernel a third of its
 // time (126 against 85 us at L = 4096, k = 32); letting the source side recompute p and ds (two more products there,
 // delta (n, H) handed over) measured slower than either on every graph tried.
-template <typename T, int H, int D, int HW, bool PIPE, bool DROP, bool BIAS>
-__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : DROP || BIAS ? 3 : 4))) void k_attn_bwd_dst_tile(
+template <typename T, int H, int D, int HW, bool PIPE, bool DROP, int BIAS>
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : DROP || BIAS == 1 ? 3 : 4))) void k_attn_bwd_dst_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
     const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds, float *__restrict__ ws_dq,
     float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv, const float *__restrict__ bias,
@@ -1967,19 +1970,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         float kr[16], va[16];
         float4 kc[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 g + r
         int pos[4], mk[4];
-        int xe[DROP || BIAS ? 4 : 1];
-        int bi[BIAS ? 4 : 1];                                     // rows of the score term of the block's pairs
+        int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            else if constexpr (BIAS) {
-                if (!P.grp_bias_idx) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            }
-            if constexpr (BIAS) tile_pair_bias_rows(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe, B.bi);
+            if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -1996,7 +1994,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 B.kc[r] = *reinterpret_cast<const float4 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
             if constexpr (BIAS) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.bi[r] * (uint32_t)H) + t.head];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -2020,7 +2018,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 pe *= mt;                                         // what multiplies v (forward) and dO (dV)
                 if (has) {
                     pds_h[B.pos[r]] = make_float2(pe, ds[r]);
-                    if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.bi[BIAS ? r : 0] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
+                    if constexpr (BIAS) ds_out[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])] = ds[r];   // dL/d(score before scaling)
                 }
             }
             tile_axpy(ds, B.kc, acc);
@@ -2148,7 +2146,7 @@ __device__ __forceinline__ void tile_load_row_bf16(const char *p, Bf8 (&out)[2])
     out[1].q = *reinterpret_cast<const uint4 *>(p + 16);
 }
 
-template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, bool BIAS>
+template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, int BIAS>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP || BIAS ? WPE - 1 : WPE))) void k_attn_fwd_tile_bf16(
     bpt_plan P, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v, bf16_t *__restrict__ o,
     float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr,
@@ -2157,7 +2155,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     TileCtx t;
     if (!tile_begin<bf16_t, H, D, HW>(P, t)) return;
     __shared__ int2 ent_lds[HW][TILE_CHUNK];
+    __shared__ int fst_lds[HW][BIAS == 2 ? TILE_CHUNK : 1];      // the entries' first pair numbers: where a term in pair order sits
     int2 *ent = ent_lds[t.wv];
+    int *fst = BIAS == 2 ? fst_lds[t.wv] : nullptr;
     const int c = t.c, g = t.g;
     const uint32_t offr = (uint32_t)((t.head * D + 16 * g) * 2), offc = (uint32_t)((t.head * D + 4 * c) * 2);
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
@@ -2171,19 +2171,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
         Bf8 kr[2];
         uint2 vr[4];
         int mk[4];
-        int xe[DROP || BIAS ? 4 : 1];
-        int bi[BIAS ? 4 : 1];                                     // rows of the score term of the block's pairs
+        int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
-        tile_stage_entries(P, ent, p0, cnt, t.lane);
+        tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            else if constexpr (BIAS) {
-                if (!P.grp_bias_idx) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            }
-            if constexpr (BIAS) tile_pair_bias_rows(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe, B.bi);
+            if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -2192,9 +2187,15 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             tile_load_row_bf16(kb + (size_t)((uint32_t)ea.x * (uint32_t)RB) + offr, B.kr);
 #pragma unroll
             for (int r = 0; r < 4; ++r) B.vr[r] = *reinterpret_cast<const uint2 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
-            if constexpr (BIAS) {
+            if constexpr (BIAS == 1) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.bi[r] * (uint32_t)H) + t.head];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 1>(P, t.head, B.xe[BIAS == 1 ? r : 0], 0)];
+            }
+            if constexpr (BIAS == 2) {
+                const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
+                const int fv[4] = {f4.x, f4.y, f4.z, f4.w};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 2>(P, t.head, 0, tile_pair_number(fv[r], B.mk[r], c))];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -2246,7 +2247,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     }
 }
 
-template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, bool BIAS>
+template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, int BIAS>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP || BIAS ? WPE - 1 : WPE))) void k_attn_bwd_dst_tile_bf16(
     bpt_plan P, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v, const bf16_t *__restrict__ o,
     const bf16_t *__restrict__ d_o, const float *__restrict__ lse, bf16_t *__restrict__ dq, uint32_t *__restrict__ pds,
@@ -2292,19 +2293,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
         Bf8 kr[2], va[2];
         uint2 kc[4];
         int mk[4], pos[4];
-        int xe[DROP || BIAS ? 4 : 1];
-        int bi[BIAS ? 4 : 1];                                     // rows of the score term of the block's pairs
+        int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            else if constexpr (BIAS) {
-                if (!P.grp_bias_idx) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            }
-            if constexpr (BIAS) tile_pair_bias_rows(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe, B.bi);
+            if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
@@ -2320,7 +2316,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             for (int r = 0; r < 4; ++r) B.kc[r] = *reinterpret_cast<const uint2 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
             if constexpr (BIAS) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[(size_t)((uint32_t)B.bi[r] * (uint32_t)H) + t.head];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -2337,7 +2333,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
                 pe *= mt;                                         // what multiplies v (forward) and dO (dV)
                 if (has) {
                     pds_h[B.pos[r]] = pack_bf16(pe, ds[r]);
-                    if constexpr (BIAS) ds_out[(size_t)((uint32_t)B.bi[BIAS ? r : 0] * (uint32_t)H) + t.head] = ds[r];   // dL/d(score before scaling)
+                    if constexpr (BIAS) ds_out[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])] = ds[r];   // dL/d(score before scaling)
                 }
             }
             Bf4 da;
@@ -2923,7 +2919,8 @@ __global__ __launch_bounds__(BLOCK) void k_rel_bias_rows(bpt_plan P, const T *__
 #pragma unroll
     for (int k = 0; k < K; ++k) desc[k] = items[min(i0 + k * GW, n_items - 1)];
     rel_table_to_lds<T>(table, used_types, n_used, rel_lds, REL_LDS_PITCH);
-    if (blockIdx.x == 0 && threadIdx.x < H) bias[(size_t)P.n_edges * H + threadIdx.x] = 0.f;     // the spare row the fused kernels read for absent pairs
+    const bool head_major = P.bias_by_pair != 0;                // results at bias[head * n_edges + eid] instead of bias[eid * H + head]
+    if (blockIdx.x == 0 && threadIdx.x < H && !head_major) bias[(size_t)P.n_edges * H + threadIdx.x] = 0.f;     // the spare row the fused kernels read for absent pairs
     RelHead hd[K];
     float aq[K][16];
 #pragma unroll
@@ -2957,10 +2954,83 @@ __global__ __launch_bounds__(BLOCK) void k_rel_bias_rows(bpt_plan P, const T *__
                     table_rows(type, 16 * blk, bt);
                     const floatx4v acc = tile_dot(aq[k], bt);
                     const int e = lane_bcast(edge, 16 * blk + c);
-                    if (16 * blk + c < cnt && 4 * g < H)
-                        *reinterpret_cast<float4 *>(bias + (size_t)e * H + 4 * g) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+                    if (16 * blk + c < cnt && 4 * g < H) {
+                        if (head_major) {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) bias[(size_t)(4 * g + r) * (size_t)P.n_edges + e] = acc[r];
+                        } else {
+                            *reinterpret_cast<float4 *>(bias + (size_t)e * H + 4 * g) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+                        }
+                    }
                 }
             }
+        }
+    }
+}
+
+// The same term over the TILE plan of the attention kernels, for a term kept in that plan's pair order (bias_by_pair:
+// one value per pair and head at bias[head * n_edges + pair number]).  One wavefront per (tile, head), as in the attention
+// kernels.  First the products of the tile's 16 member rows with every table row in use, QT[type number][member] (16
+// type numbers per step: A = table rows, B = the members' q), which go to a wavefront-private piece of LDS; then the
+// lanes walk the tile's pairs, which are consecutive numbers, and every pair picks its value by what pair_tm[number] =
+// type number | member << 8 says.  The per-pair arrays are read and written in runs; the table rows in use are staged in
+// LDS once per workgroup (fetched from memory step by step, each step waits for two dependent loads: 32 us against
+// the products' 7).
+template <typename T>
+__device__ __forceinline__ void rel_cols16(const T *row, int g, float (&out)[16]) {     // columns 16 t + 4 g + e of a 64-column row
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const float4 x = load4<T>(row + 16 * t + 4 * g);
+        out[4 * t] = x.x; out[4 * t + 1] = x.y; out[4 * t + 2] = x.z; out[4 * t + 3] = x.w;
+    }
+}
+template <typename T, int H, int HW>
+__global__ __launch_bounds__(HW * WAVE) void k_rel_bias_tiles(bpt_plan P, const T *__restrict__ q, const T *__restrict__ table,
+                                                              const int32_t *__restrict__ used_types, int n_used,
+                                                              const int32_t *__restrict__ pair_tm, float *__restrict__ bias) {
+    constexpr int D = 64, C = H * D;
+    extern __shared__ float rel_lds[];                        // the table rows in use, then QT of every wavefront
+    const int n16 = (n_used + 15) & ~15;
+    rel_table_to_lds<T>(table, used_types, n_used, rel_lds, REL_LDS_PITCH);
+    TileCtx t;
+    const bool mine = tile_begin<T, H, D, HW>(P, t) && t.p_begin < t.p_end;
+    __syncthreads();
+    if (!mine) return;
+    float *qt = rel_lds + (size_t)n_used * REL_LDS_PITCH + (size_t)t.wv * n16 * TILE_R;
+    auto table_rows = [&](int tb, float (&out)[16]) {           // of type numbers tb + c: this lane's columns
+        const float *row = rel_lds + min(tb + t.c, n_used - 1) * REL_LDS_PITCH + 4 * t.g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 x = *reinterpret_cast<const float4 *>(row + 16 * i);
+            out[4 * i] = x.x; out[4 * i + 1] = x.y; out[4 * i + 2] = x.z; out[4 * i + 3] = x.w;
+        }
+    };
+    const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+    const int4 last = entries[t.p_end - 1];
+    const int first = __builtin_amdgcn_readfirstlane(entries[t.p_begin].z), end = __builtin_amdgcn_readfirstlane(last.z + __popc((uint32_t)last.y));
+    constexpr int AHEAD = 4;                                    // pairs per lane whose loads are in flight together
+    int tm[AHEAD];
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) tm[k] = pair_tm[min(first + t.lane + k * WAVE, end - 1)];
+    float qb[16];
+    rel_cols16<T>(q + (size_t)max(t.member.x, 0) * C + t.head * D, t.g, qb);
+    for (int tb = 0; tb < n16; tb += TILE_R) {
+        float kr[16];
+        table_rows(tb, kr);
+        const floatx4v st = tile_dot(kr, qb);                   // register r: (type number tb + 4 g + r, member c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) qt[(tb + 4 * t.g + r) * TILE_R + t.c] = st[r];
+    }
+    wave_lds_fence();
+    float *out = bias + (size_t)t.head * (size_t)P.n_edges;
+    for (int x = first + t.lane; x < end; x += AHEAD * WAVE) {
+        int nt[AHEAD];
+#pragma unroll
+        for (int k = 0; k < AHEAD; ++k) nt[k] = pair_tm[min(x + (AHEAD + k) * WAVE, end - 1)];
+#pragma unroll
+        for (int k = 0; k < AHEAD; ++k) {
+            if (x + k * WAVE < end) out[x + k * WAVE] = qt[(tm[k] & 0xff) * TILE_R + (tm[k] >> 8)];
+            tm[k] = nt[k];
         }
     }
 }
@@ -2979,15 +3049,25 @@ struct RelBody {             // what the walk of those slots needs: per lane the
     float dsv[H];            // and, for a whole row, the dq row it adds to (lane l: column l)
     float qh[H], old[H];
 };
-template <typename T, int H>
-__device__ __forceinline__ void rel_body_load(const RelHead &r, const float *__restrict__ ds, const T *__restrict__ q, const T *__restrict__ dq,
-                                              int lane, RelBody<H> &y) {
-    constexpr int D = 64;
+// the H values of ds that belong to `edge`: a row of (n_edges, H), or with head_major one of each head's n_edges values
+template <int H>
+__device__ __forceinline__ void rel_ds_load(const float *__restrict__ ds, int edge, bool head_major, size_t n_edges, float (&out)[H]) {
+    if (head_major) {
 #pragma unroll
-    for (int h = 0; h < H; h += 4) {
-        const float4 x = *reinterpret_cast<const float4 *>(ds + (size_t)r.edge * H + h);
-        y.dsv[h] = x.x; y.dsv[h + 1] = x.y; y.dsv[h + 2] = x.z; y.dsv[h + 3] = x.w;
+        for (int h = 0; h < H; ++h) out[h] = ds[(size_t)h * n_edges + edge];
+    } else {
+#pragma unroll
+        for (int h = 0; h < H; h += 4) {
+            const float4 x = *reinterpret_cast<const float4 *>(ds + (size_t)edge * H + h);
+            out[h] = x.x; out[h + 1] = x.y; out[h + 2] = x.z; out[h + 3] = x.w;
+        }
     }
+}
+template <typename T, int H>
+__device__ __forceinline__ void rel_body_load(const RelHead &r, const float *__restrict__ ds, bool head_major, size_t n_edges, const T *__restrict__ q,
+                                              const T *__restrict__ dq, int lane, RelBody<H> &y) {
+    constexpr int D = 64;
+    rel_ds_load<H>(ds, r.edge, head_major, n_edges, y.dsv);
 #pragma unroll
     for (int h = 0; h < H; ++h) {
         y.qh[h] = Elem<T>::ld(q + ((size_t)r.row * H + h) * D + lane);
@@ -3001,6 +3081,7 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
     constexpr int D = 64, C = H * D, AHEAD = H >= 16 ? 4 : 8;
     extern __shared__ float rel_lds[];                    // NW tables of n_used x 64 sums, the table rows in use, NW x 64 x H staged ds values
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const bool head_major = P.bias_by_pair != 0;                // ds[head * n_edges + eid] instead of ds[eid * H + head]
     float *acc = rel_lds + (size_t)w * n_used * D;
     const float *rows = rel_lds + (size_t)NW * n_used * D;
     float *stage = rel_lds + (size_t)(NW + 1) * n_used * D + (size_t)w * WAVE * H;
@@ -3013,7 +3094,7 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
     RelHead hd, hd_next;
     RelBody<H> bd, bd_next;
     rel_head_load(P, i_begin < i_end ? items[i_begin] : none, lane, hd_next);
-    rel_body_load<T, H>(hd_next, ds, q, dq, lane, bd_next);
+    rel_body_load<T, H>(hd_next, ds, head_major, (size_t)P.n_edges, q, dq, lane, bd_next);
     hd = hd_next;
     rel_head_load(P, i_begin + GW < i_end ? items[i_begin + GW] : none, lane, hd_next);
     int4 desc = i_begin + 2 * GW < i_end ? items[i_begin + 2 * GW] : none;
@@ -3069,7 +3150,7 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
     };
     for (int i = i_begin; i < i_end; i += GW) {
         bd = bd_next;
-        rel_body_load<T, H>(hd_next, ds, q, dq, lane, bd_next);                // the item after this one
+        rel_body_load<T, H>(hd_next, ds, head_major, (size_t)P.n_edges, q, dq, lane, bd_next);                // the item after this one
         const RelHead cur = hd;
         hd = hd_next;
         rel_head_load(P, desc, lane, hd_next);                                   // the second after
@@ -3088,10 +3169,12 @@ __global__ __launch_bounds__(NW * WAVE) void k_rel_bias_bwd(bpt_plan P, const fl
             const int cnt = min(WAVE, cur.e - p0);
             const int slot = p0 + min(lane, cnt - 1);
             const int u = P.idx[slot], edge = P.eid[slot];
+            float rest[H];
+            rel_ds_load<H>(ds, edge, head_major, (size_t)P.n_edges, rest);
 #pragma unroll
             for (int h = 0; h < H; h += 4)
                 *reinterpret_cast<float4 *>(stage + lane * H + h) =
-                    lane < cnt ? *reinterpret_cast<const float4 *>(ds + (size_t)edge * H + h) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    lane < cnt ? make_float4(rest[h], rest[h + 1], rest[h + 2], rest[h + 3]) : make_float4(0.f, 0.f, 0.f, 0.f);
             walk(cnt, u, bd.qh, dqa);
         }
         if (cur.out_slot < 0) {
@@ -3382,22 +3465,27 @@ inline int rel_bwd_waves(int64_t n_used, int h, bool large_lds = true) {
     return best;
 }
 
-// a kernel may take more than 64 KB of dynamic LDS only after it has been told so (once per kernel and device)
-template <typename K>
-int allow_large_lds(K kernel, size_t bytes) {
-    static std::atomic<uint32_t> done{0};
+// a kernel may take more than 64 KB of dynamic LDS only after it has been told so (once per kernel and device; kernels of
+// one signature are different kernels, so what has been done is kept by kernel address)
+inline int allow_large_lds_at(const void *kernel, size_t bytes) {
+    static std::mutex lock;
+    static std::vector<std::pair<const void *, int>> done;
     if (bytes <= 64 * 1024) return BPT_OK;
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32) return BPT_ERR_UNSUPPORTED;
-    if (done.load(std::memory_order_acquire) & (1u << dev)) return BPT_OK;
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (hipGetDevice(&dev) != hipSuccess) return BPT_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> hold(lock);
+    for (const auto &x : done)
+        if (x.first == kernel && x.second == dev) return BPT_OK;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) {
         (void)hipGetLastError();
         return BPT_ERR_UNSUPPORTED;          // (the caller then takes a configuration inside 64 KB)
     }
-    done.fetch_or(1u << dev, std::memory_order_release);
+    done.emplace_back(kernel, dev);
     return BPT_OK;
 }
+template <typename K>
+int allow_large_lds(K kernel, size_t bytes) { return allow_large_lds_at(reinterpret_cast<const void *>(kernel), bytes); }
 
 template <typename T, int H, int NW>
 int launch_rel_bias_bwd(const bpt_plan *P, const float *ds, const void *q, const void *table, const int32_t *used_types, int64_t n_used,
@@ -3447,6 +3535,27 @@ int run_rel_bias_rows(const bpt_plan *P, const void *q, const void *table, const
     hipLaunchKernelGGL((k_rel_bias_rows<T, H>), dim3((unsigned)((waves + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK)), dim3(BLOCK),
                        (size_t)n_used * REL_LDS_PITCH * 4, s, *P, (const T *)q, (const T *)table, used_types, (int)n_used, bias);
     return launch_status();
+}
+
+// the score term over the attention kernels' tile plan, in that plan's pair order
+template <typename T, int H, int HW>
+int launch_rel_bias_tiles(const bpt_plan *P, const void *q, const void *table, const int32_t *used_types, int64_t n_used, const int32_t *pair_tm,
+                          float *bias, size_t lds, hipStream_t s) {
+    const int st = allow_large_lds(k_rel_bias_tiles<T, H, HW>, lds);
+    if (st != BPT_OK) return st;
+    hipLaunchKernelGGL((k_rel_bias_tiles<T, H, HW>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), lds, s, *P, (const T *)q, (const T *)table,
+                       used_types, (int)n_used, pair_tm, bias);
+    return launch_status();
+}
+template <typename T, int H>
+int run_rel_bias_tiles(const bpt_plan *P, const void *q, const void *table, const int32_t *used_types, int64_t n_used, const int32_t *pair_tm,
+                       float *bias, hipStream_t s) {
+    // the table rows once per workgroup, QT once per wavefront (= head); eight heads share the rows where that fits 64 KB
+    auto lds = [&](int hw) { return ((size_t)n_used * REL_LDS_PITCH + (size_t)hw * (size_t)((n_used + 15) & ~(int64_t)15) * TILE_R) * 4; };
+    if constexpr (H >= 8) {
+        if (lds(8) <= 64 * 1024) return launch_rel_bias_tiles<T, H, 8>(P, q, table, used_types, n_used, pair_tm, bias, lds(8), s);
+    }
+    return launch_rel_bias_tiles<T, H, 4>(P, q, table, used_types, n_used, pair_tm, bias, lds(4), s);
 }
 
 template <typename T, int H, int D>
@@ -3670,6 +3779,9 @@ inline int64_t pds_bytes(const bpt_plan *Pin, const bpt_plan *Pout, int h, int d
     return 2 * round16(n * h * 4);
 }
 
+// how the tile kernels find the score term: 0 none, 1 by edge id, 2 in the plan's own pair order, head-major
+inline int tile_bias_mode(const bpt_plan *P, const float *bias) { return !bias ? 0 : P->bias_by_pair ? 2 : 1; }
+
 template <typename T, int H, int D>
 int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v, void *o, float *lse, void *ws, float scale, Dropout drop,
                  const float *bias, hipStream_t s) {
@@ -3684,11 +3796,13 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
 #define LAUNCH_FWD_TILE(PI, DR, BI)                                                                                                  \
     hipLaunchKernelGGL((k_attn_fwd_tile<T, H, D, HW, PI, DR, BI>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), 0, s, *P, (const T *)q, \
                        (const T *)k, (const T *)v, (T *)o, lse, ws_acc, ws_ml, scale * LOG2E, drop.thr, drop.seed, drop.inv, bias)
-                switch ((drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0)) {
-                case 0: if (tall_tiles(P, H)) LAUNCH_FWD_TILE(true, false, false); else LAUNCH_FWD_TILE(false, false, false); break;
-                case 1: LAUNCH_FWD_TILE(false, true, false); break;
-                case 2: LAUNCH_FWD_TILE(false, false, true); break;
-                default: LAUNCH_FWD_TILE(false, true, true); break;
+                switch ((drop.thr != 0 ? 1 : 0) + 2 * tile_bias_mode(P, bias)) {
+                case 0: if (tall_tiles(P, H)) LAUNCH_FWD_TILE(true, false, 0); else LAUNCH_FWD_TILE(false, false, 0); break;
+                case 1: LAUNCH_FWD_TILE(false, true, 0); break;
+                case 2: LAUNCH_FWD_TILE(false, false, 1); break;
+                case 3: LAUNCH_FWD_TILE(false, true, 1); break;
+                case 4: LAUNCH_FWD_TILE(false, false, 2); break;
+                default: LAUNCH_FWD_TILE(false, true, 2); break;
                 }
 #undef LAUNCH_FWD_TILE
                 goto launched;
@@ -3701,11 +3815,13 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     hipLaunchKernelGGL((k_attn_fwd_tile_bf16<H, D, HW, TILE_BF16_WPE, TILE_BF16_PIPE, DR, BI>), dim3(group_grid(P) * (H / HW)), dim3(HW * WAVE), \
                        0, s, *P, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (bf16_t *)o, lse, ws_acc, ws_ml, scale * LOG2E,   \
                        drop.thr, drop.seed, drop.inv, bias)
-                switch ((drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0)) {
-                case 0: LAUNCH_FWD_TILE(false, false); break;
-                case 1: LAUNCH_FWD_TILE(true, false); break;
-                case 2: LAUNCH_FWD_TILE(false, true); break;
-                default: LAUNCH_FWD_TILE(true, true); break;
+                switch ((drop.thr != 0 ? 1 : 0) + 2 * tile_bias_mode(P, bias)) {
+                case 0: LAUNCH_FWD_TILE(false, 0); break;
+                case 1: LAUNCH_FWD_TILE(true, 0); break;
+                case 2: LAUNCH_FWD_TILE(false, 1); break;
+                case 3: LAUNCH_FWD_TILE(true, 1); break;
+                case 4: LAUNCH_FWD_TILE(false, 2); break;
+                default: LAUNCH_FWD_TILE(true, 2); break;
                 }
 #undef LAUNCH_FWD_TILE
                 goto launched;
@@ -3774,11 +3890,13 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
     hipLaunchKernelGGL((k_attn_bwd_dst_tile<T, H, D, HW, PI, DR, BI>), dim3(group_grid(Pin) * (H / HW)), dim3(HW * WAVE), 0, s, *Pin,     \
                        (const T *)q, (const T *)k, (const T *)v, (const T *)o, (const T *)d_o, lse, (T *)dq, pds, ws_rows, scale,         \
                        scale * LOG2E, drop.thr, drop.seed, drop.inv, bias, ds_out)
-                switch ((drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0)) {
-                case 0: if (tall_tiles(Pin, H)) LAUNCH_DST_TILE(true, false, false); else LAUNCH_DST_TILE(false, false, false); break;
-                case 1: LAUNCH_DST_TILE(false, true, false); break;
-                case 2: LAUNCH_DST_TILE(false, false, true); break;
-                default: LAUNCH_DST_TILE(false, true, true); break;
+                switch ((drop.thr != 0 ? 1 : 0) + 2 * tile_bias_mode(Pin, bias)) {
+                case 0: if (tall_tiles(Pin, H)) LAUNCH_DST_TILE(true, false, 0); else LAUNCH_DST_TILE(false, false, 0); break;
+                case 1: LAUNCH_DST_TILE(false, true, 0); break;
+                case 2: LAUNCH_DST_TILE(false, false, 1); break;
+                case 3: LAUNCH_DST_TILE(false, true, 1); break;
+                case 4: LAUNCH_DST_TILE(false, false, 2); break;
+                default: LAUNCH_DST_TILE(false, true, 2); break;
                 }
 #undef LAUNCH_DST_TILE
             }
@@ -3812,11 +3930,13 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
                        dim3(HW * WAVE), 0, s, *Pin, (const bf16_t *)q, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)o,             \
                        (const bf16_t *)d_o, lse, (bf16_t *)dq, (uint32_t *)ws, ws_rows, scale, scale * LOG2E, drop.thr, drop.seed,          \
                        drop.inv, bias, ds_out)
-                switch ((drop.thr != 0 ? 1 : 0) + (bias ? 2 : 0)) {
-                case 0: LAUNCH_DST_TILE(false, false); break;
-                case 1: LAUNCH_DST_TILE(true, false); break;
-                case 2: LAUNCH_DST_TILE(false, true); break;
-                default: LAUNCH_DST_TILE(true, true); break;
+                switch ((drop.thr != 0 ? 1 : 0) + 2 * tile_bias_mode(Pin, bias)) {
+                case 0: LAUNCH_DST_TILE(false, 0); break;
+                case 1: LAUNCH_DST_TILE(true, 0); break;
+                case 2: LAUNCH_DST_TILE(false, 1); break;
+                case 3: LAUNCH_DST_TILE(true, 1); break;
+                case 4: LAUNCH_DST_TILE(false, 2); break;
+                default: LAUNCH_DST_TILE(true, 2); break;
                 }
 #undef LAUNCH_DST_TILE
             }
@@ -4021,6 +4141,7 @@ int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table,
     CHECK(check_plan(plan, true));
     CHECK(check_shape(h, d, dtype));
     if (plan->n_edges > 0 && (!q || !table || !bias)) return BPT_ERR_NULL;
+    if (plan->bias_by_pair && !used_types) return BPT_ERR_UNSUPPORTED;      // only the kernel below writes the head-major form
     hipStream_t s = (hipStream_t)stream;
     if (used_types) {                       // plan indices are type numbers: the kernel with the table rows in LDS
         if (n_used < 0) return BPT_ERR_SIZE;
@@ -4035,6 +4156,24 @@ int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table,
 #define X(HH, DD) if (h == HH && d == DD) return run_rel_bias<T, HH, DD>(plan, q, table, bias, s);
     if (dtype == BPT_F32) { using T = float; BPT_FAST_SHAPES_F32(X) }
     if (dtype == BPT_BF16) { using T = bf16_t; BPT_FAST_SHAPES_BF16(X) }
+#undef X
+    return BPT_ERR_UNSUPPORTED;
+}
+
+int bpt_rel_bias_forward_tiles(const bpt_plan *plan, const void *q, const void *table, const int32_t *used_types, int64_t n_used,
+                               const int32_t *pair_types, float *bias, int h, int d, int dtype, void *stream) {
+    CHECK(check_plan(plan, true));
+    CHECK(check_shape(h, d, dtype));
+    if (n_used < 0) return BPT_ERR_SIZE;
+    if (!rel_rows_shape(h, d, dtype) || n_used > REL_MAX_USED || !has_tiles(plan, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_UNSUPPORTED;
+    if (plan->n_edges == 0) return BPT_OK;
+    if (!q || !table || !used_types || !pair_types || !bias) return BPT_ERR_NULL;
+    if (n_used == 0) return BPT_ERR_SIZE;                        // (edges without a type in use)
+    if (!aligned16(q) || !aligned16(table)) return BPT_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+#define X(HH) if (h == HH) return run_rel_bias_tiles<T, HH>(plan, q, table, used_types, n_used, pair_types, bias, s);
+    if (dtype == BPT_F32) { using T = float; X(4) X(8) X(16) }
+    if (dtype == BPT_BF16) { using T = bf16_t; X(4) X(8) X(16) }
 #undef X
     return BPT_ERR_UNSUPPORTED;
 }
@@ -4154,7 +4293,7 @@ int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k,
         return BPT_ERR_UNSUPPORTED;
     if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
     // only the tile kernels look the rows of the score term up in a numbering of the plan's own
-    if (bias && plan_in->grp_bias_idx && !has_tiles(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_PLAN;
+    if (bias && plan_in->bias_by_pair && !has_tiles(plan_in, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_PLAN;
     if (!fast_shape(h, d, dtype) || !aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(workspace))
         return BPT_ERR_UNSUPPORTED;
     const int64_t need = bpt_workspace_bytes(BPT_OP_ATTN_FWD, plan_in, nullptr, h, d, dtype);
@@ -4195,7 +4334,7 @@ int bpt_attention_backward(const bpt_plan *plan_in, const bpt_plan *plan_out, co
         return BPT_ERR_UNSUPPORTED;
     if ((bias != nullptr) != (ds_out != nullptr)) return BPT_ERR_NULL;       // the score term and its gradient go together
     if ((bias || drop.thr != 0) && !plan_in->grp_eids) return BPT_ERR_PLAN;
-    if (bias && plan_in->grp_bias_idx && !tiled_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_PLAN;
+    if (bias && plan_in->bias_by_pair && !tiled_backward(plan_in, plan_out, h, d, dtype == BPT_BF16 ? 2 : 4)) return BPT_ERR_PLAN;
     // (the two sides may have different row counts: attention to a memory of another length, attention.py:144-168)
     if (plan_in->n_edges != plan_out->n_edges) return BPT_ERR_PLAN;
     if (!q || !k || !v || !o || !d_o || !lse || !dq || !dk || !dv) return BPT_ERR_NULL;

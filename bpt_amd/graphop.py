@@ -18,7 +18,7 @@ import threading
 
 import torch
 
-from ._lib import attn_lib, check_attn
+from ._lib import PlanStruct, attn_lib, check_attn
 from .plan import GROUP_ORDER_SRC, TILE_GROUP_R, plan_cache
 
 __all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forward", "node_mul_edge_backward",
@@ -378,13 +378,22 @@ def attention_supported(q):
     return q.dim() == 3 and (h, d) in fast.get(q.dtype, ())
 
 
-def rel_bias_forward(col, indptr_c, eid_c, type_slot, q, table, used_types=None):
+def _by_pair(plan_struct):
+    """A copy of a `bpt_plan` with bias_by_pair set: the per-edge term it reads or writes is (h, E), head-major."""
+    st = PlanStruct.from_buffer_copy(plan_struct)
+    st.bias_by_pair = 1
+    return st
+
+
+def rel_bias_forward(col, indptr_c, eid_c, type_slot, q, table, used_types=None, by_pair=False):
     """The rel_pos score term of modules/attention.py:69-71 without the (E, d) embedding rows:
     bias[eid_c[p], head] = q[row(p), head, :] . table[type(p), :] for every slot p of the in-CSR.  Returns float32
     (E + 1, h); the last row is a zero spare row that the fused kernels read for absent pairs.
     used_types None: type_slot[p] is the type of the edge in slot p (etype[eid_c]).
     used_types (n_used,) int32, the types that occur: type_slot[p] is the NUMBER of the slot's type in that list; takes the
-    kernel that keeps those table rows on chip (needs rel_rows_supported(q) and n_used <= REL_MAX_USED_TYPES)."""
+    kernel that keeps those table rows on chip (needs rel_rows_supported(q) and n_used <= REL_MAX_USED_TYPES).
+    by_pair (with used_types only): returns float32 (h, E) instead, bias[head, eid_c[p]], the form attention_forward takes
+    with bias_by_pair=True when eid_c[p] is the number attention_pair_rows() gives the slot's edge."""
     cfg = _SETTINGS
     _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, type_slot=type_slot, q=q, table=table)
     _same_dtype(q, table)
@@ -398,12 +407,14 @@ def rel_bias_forward(col, indptr_c, eid_c, type_slot, q, table, used_types=None)
         if used_types.dtype != torch.int32 or used_types.dim() != 1 or used_types.numel() > table.size(0):
             raise ValueError("used_types must be a 1-D int32 tensor of at most table.size(0) elements")
         plan = plan_cache.get(col, indptr_c, eid_c, type_slot, q.size(0), max(used_types.numel(), 1))
-        ref, n_used = plan.ref, used_types.numel()
+        ref, n_used = (ctypes.byref(_by_pair(plan.struct)) if by_pair else plan.ref), used_types.numel()
     else:
+        if by_pair:
+            raise ValueError("by_pair needs used_types")
         plan = plan_cache.get(col, indptr_c, eid_c, type_slot, q.size(0), table.size(0))
         ref, n_used = _spmm_ref(plan, q, h, d, cfg), 0
-    bias = (torch.empty if plan.covers_all_edges else torch.zeros)((E + 1, h), dtype=torch.float32, device=q.device)
-    if used_types is None or not plan.n_items:
+    bias = (torch.empty if plan.covers_all_edges else torch.zeros)((h, E) if by_pair else (E + 1, h), dtype=torch.float32, device=q.device)
+    if not by_pair and (used_types is None or not plan.n_items):
         bias[E].zero_()                     # (the kernel of the other form clears the spare row itself)
     with _on_device_of(q):
         check_attn(_LIB.bpt_rel_bias_forward(ref, _ptr(q), _ptr(table), _ptr(used_types) if used_types is not None else None, n_used,
@@ -420,13 +431,14 @@ def rel_rows_supported(q):
     return q.dim() == 3 and d == 64 and h in (4, 8, 16) and q.dtype in (torch.float32, torch.bfloat16)
 
 
-def rel_bias_backward(col, indptr_c, eid_c, number_slot, used, used_types, ds, q, table, dq):
+def rel_bias_backward(col, indptr_c, eid_c, number_slot, used, used_types, ds, q, table, dq, by_pair=False):
     """Gradients of the rel_pos score term (modules/attention.py:55-56,69-71: autograd of nn.Embedding and of
     node_mul_edge) from ds (E or more rows, h) float32 = dL/d(score before scaling) per edge and head:
     dq[row] += sum_p ds[eid_c[p]] * table[type(p)] in place, and returns dtable (n_types, d) with
     dtable[t] = sum over the slots of type t and the heads of ds * q[row].  used_types (n_used,) int32: the types that
     occur; number_slot[p]: the number of slot p's type in that list; used (n_types,) int32: the number of every type
-    in the list, -1 for the others.  Raises if rel_rows_supported(q) is False or n_used > REL_MAX_USED_TYPES."""
+    in the list, -1 for the others.  by_pair: ds is (h, E), ds[head, eid_c[p]], as attention_backward returns it with
+    bias_by_pair=True.  Raises if rel_rows_supported(q) is False or n_used > REL_MAX_USED_TYPES."""
     _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, number_slot=number_slot, used=used, used_types=used_types, ds=ds, q=q, table=table, dq=dq)
     _same_dtype(q, table, dq)
     h, d = _hd(q)
@@ -436,7 +448,10 @@ def rel_bias_backward(col, indptr_c, eid_c, number_slot, used, used_types, ds, q
         raise ValueError("used must be int32 with one element per table row")
     if used_types.dtype != torch.int32 or used_types.dim() != 1 or used_types.numel() > table.size(0):
         raise ValueError("used_types must be a 1-D int32 tensor of at most table.size(0) elements")
-    if ds.dtype != torch.float32 or ds.dim() != 2 or ds.size(1) != h or ds.size(0) < eid_c.size(0):
+    if by_pair:
+        if ds.dtype != torch.float32 or tuple(ds.shape) != (h, eid_c.size(0)):
+            raise ValueError(f"ds must be float32 ({h}, {eid_c.size(0)})")
+    elif ds.dtype != torch.float32 or ds.dim() != 2 or ds.size(1) != h or ds.size(0) < eid_c.size(0):
         raise ValueError(f"ds must be float32 (>= {eid_c.size(0)}, {h})")
     if dq.shape != q.shape:
         raise ValueError("dq must have the shape of q")
@@ -444,19 +459,21 @@ def rel_bias_backward(col, indptr_c, eid_c, number_slot, used, used_types, ds, q
     n_used = used_types.numel()
     plan = plan_cache.get(col, indptr_c, eid_c, number_slot, q.size(0), max(n_used, 1))
     dtable = torch.empty_like(table)
+    ref = ctypes.byref(_by_pair(plan.struct)) if by_pair else plan.ref
     with _on_device_of(q):
-        nws = int(_LIB.bpt_rel_bias_backward_workspace_bytes(plan.ref, n_used, h))
+        nws = int(_LIB.bpt_rel_bias_backward_workspace_bytes(ref, n_used, h))
         ws = _scratch(max(nws, 16), q.device)
-        check_attn(_LIB.bpt_rel_bias_backward(plan.ref, _ptr(ds), _ptr(q), _ptr(table), _ptr(used), _ptr(used_types), table.size(0), n_used,
+        check_attn(_LIB.bpt_rel_bias_backward(ref, _ptr(ds), _ptr(q), _ptr(table), _ptr(used), _ptr(used_types), table.size(0), n_used,
                                               _ptr(dq), _ptr(dtable), _ptr(ws), nws, h, d, _dtype(q), _stream()), "rel_bias_backward")
     return dtable
 
 
-def _check_bias(bias, n_edges, h, device, cfg):
+def _check_bias(bias, n_edges, h, device, cfg, by_pair=False):
     if bias is None:
         return
-    if bias.dtype != torch.float32 or tuple(bias.shape) != (n_edges + 1, h) or not bias.is_contiguous() or bias.device != device:
-        raise ValueError(f"bias must be a contiguous float32 ({n_edges + 1}, {h}) tensor on {device}")
+    shape = (h, n_edges) if by_pair else (n_edges + 1, h)
+    if bias.dtype != torch.float32 or tuple(bias.shape) != shape or not bias.is_contiguous() or bias.device != device:
+        raise ValueError(f"bias must be a contiguous float32 {shape} tensor on {device}")
     if not cfg.use_groups:
         raise RuntimeError("the per-edge score term needs the row-group kernels")
 
@@ -465,11 +482,12 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     """o[dst] = sum over in-edges drop(softmax((q[dst].k[src] + bias[e])*scale)) v[src]; returns (o, lse) with lse
     (n, h) float32 in base-2 units.  Arithmetic of modules/attention.py:66-77 in one pass.  dropout_p > 0
     drops attention probabilities as attention.py:73 does; the mask is a function of (seed, graph), see
-    attention_dropout_mask.  bias: None or the float32 (E + 1, h) score term of rel_bias_forward, its rows by edge id or,
-    with bias_by_pair, by the numbers attention_pair_rows() gives the edges (tile kernels only)."""
+    attention_dropout_mask.  bias: None or the float32 score term of rel_bias_forward: (E + 1, h) with its rows by edge
+    id, or with bias_by_pair (h, E) with the edges in the order of the numbers attention_pair_rows() gives them (tile
+    kernels only)."""
     cfg = _SETTINGS
     _check_all(col=col, indptr_c=indptr_c, eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v)
-    _check_bias(bias, eid_c.size(0), _hd(q)[0], q.device, cfg)
+    _check_bias(bias, eid_c.size(0), _hd(q)[0], q.device, cfg, bias_by_pair)
     _same_dtype(q, k, v)
     h, d = _hd(q)
     _expect_index(eid_c, indices_c)
@@ -504,8 +522,8 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
 def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, v, o, lse, do, scale=None,
                        dropout_p=0.0, seed=0, bias=None, bias_by_pair=False):
     """(dq, dk, dv) of attention_forward (same dropout_p, seed, bias and bias_by_pair).  With bias a fourth result: ds,
-    float32 (E, h), the gradient with respect to q.k + bias of every edge and head (= the gradient of bias), its rows in the
-    order of bias's."""
+    float32 (E, h), or (h, E) with bias_by_pair, the gradient with respect to q.k + bias of every edge and head (= the
+    gradient of bias), laid out like bias."""
     cfg = _SETTINGS
     _check_all(row=row, indptr_r=indptr_r, eid_r=eid_r, indices_r=indices_r, col=col, indptr_c=indptr_c,
                eid_c=eid_c, indices_c=indices_c, q=q, k=k, v=v, o=o, lse=lse)
@@ -527,8 +545,8 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), prefer_device=on_gpu)
     plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), prefer_device=on_gpu)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    _check_bias(bias, eid_c.size(0), h, q.device, cfg)
-    ds = torch.empty((eid_c.size(0) + 1, h), dtype=torch.float32, device=q.device) if bias is not None else None
+    _check_bias(bias, eid_c.size(0), h, q.device, cfg, bias_by_pair)
+    ds = torch.empty((h, eid_c.size(0)) if bias_by_pair else (eid_c.size(0) + 1, h), dtype=torch.float32, device=q.device) if bias is not None else None
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref
     tiles = False
@@ -554,16 +572,13 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
                                                scale, float(dropout_p), int(seed) & (2 ** 64 - 1), h, d, dt, _stream()),
                    "attention_backward")
     if bias is not None:
-        return dq, dk, dv, ds[:-1]
+        return dq, dk, dv, ds if bias_by_pair else ds[:-1]
     return dq, dk, dv
 
 
-def attention_pair_rows(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p=0.0):
-    """For a step with a per-edge score term: None, or, where attention_forward and attention_backward will both run on
-    the tile kernels for these arguments, the (E,) int64 tensor that numbers the edges the way the tiles meet them (the pair
-    numbers of the in-CSR's tile plan).  A score term stored in that order (row number[e] for edge e) and passed with
-    bias_by_pair=True is read, and its gradient written, in neighbouring rows per tile instead of rows scattered by edge
-    id."""
+def _pair_order(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p):
+    """The in-CSR's tile plan and its pair-order tables (DevicePlan.bias_rows) where attention_forward and
+    attention_backward will both run on the tile kernels with a per-edge score term for these arguments, else None."""
     cfg = _SETTINGS
     if q.dim() != 3 or not q.is_cuda:
         return None
@@ -577,7 +592,51 @@ def attention_pair_rows(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, i
             and _tiles_backward(plan_in, q.dtype, marker)):
         return None
     plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=_tile_seg_len(plan_in), prefer_device=True)
-    return plan_in.bias_rows(TILE_ROWS)["pair_of_eid"]
+    return plan_in, plan_in.bias_rows(TILE_ROWS)
+
+
+def attention_pair_rows(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p=0.0):
+    """For a step with a per-edge score term: None, or, where attention_forward and attention_backward will both run on
+    the tile kernels for these arguments, the (E,) int64 tensor that numbers the edges the way the tiles meet them (the pair
+    numbers of the in-CSR's tile plan).  A score term stored in that order, head-major ((h, E): the value of edge e and a
+    head at [head, number[e]]), and passed with bias_by_pair=True is read, and its gradient written, in runs of
+    neighbouring values per tile, with no index read on the way, instead of rows scattered by edge id."""
+    hit = _pair_order(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p)
+    return None if hit is None else hit[1]["pair_of_eid"]
+
+
+def attention_pair_members(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p=0.0):
+    """Where attention_pair_rows gives numbers: the (E,) int32 tensor with, for every pair number, which of its tile's
+    16 rows the pair's destination is (what rel_bias_forward_tiles needs beside the pair's edge type); else None."""
+    hit = _pair_order(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p)
+    return None if hit is None else hit[1]["member_of_pair"]
+
+
+def rel_bias_forward_tiles(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, table, used_types, pair_types,
+                           dropout_p=0.0):
+    """The rel_pos score term of modules/attention.py:69-71 in the pair order of the tile kernels: float32 (h, E) with
+    [head, t] = q[dst of pair t, head, :] . table[used_types[pair_types[t] & 255], :], the form attention_forward takes with
+    bias_by_pair=True.  pair_types (E,) int32: per pair number (attention_pair_rows) the number of its edge's type in
+    used_types, plus its attention_pair_members() value << 8.  Needs rel_rows_supported(q), at most
+    REL_MAX_USED_TYPES types in use and arguments for which attention_pair_rows() gives numbers (RuntimeError else)."""
+    _check_all(q=q, table=table, used_types=used_types, pair_types=pair_types)
+    _same_dtype(q, table)
+    h, d = _hd(q)
+    if table.dim() != 2 or table.size(1) != d:
+        raise ValueError(f"table must be (n_types, {d})")
+    E = eid_c.size(0)
+    if used_types.dtype != torch.int32 or used_types.dim() != 1 or used_types.numel() > table.size(0):
+        raise ValueError("used_types must be a 1-D int32 tensor of at most table.size(0) elements")
+    if pair_types.dtype != torch.int32 or tuple(pair_types.shape) != (E,):
+        raise ValueError(f"pair_types must be int32 ({E},)")
+    hit = _pair_order(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p)
+    if hit is None:
+        raise RuntimeError("rel_bias_forward_tiles: these arguments do not run on the tile kernels (ask attention_pair_rows() first)")
+    bias = torch.empty((h, E), dtype=torch.float32, device=q.device)
+    with _on_device_of(q):
+        check_attn(_LIB.bpt_rel_bias_forward_tiles(ctypes.byref(hit[1]["struct"]), _ptr(q), _ptr(table), _ptr(used_types), used_types.numel(),
+                                                   _ptr(pair_types), _ptr(bias), h, d, _dtype(q), _stream()), "rel_bias_forward_tiles")
+    return bias
 
 
 def attention_dropout_mask(col, indptr_c, eid_c, indices_c, q, k, dropout_p, seed):

@@ -108,18 +108,22 @@ class BPTRelAttention(Function):
         aux = _rel_aux(etype, col, indptr_c, eid_c, table.size(0))
         table = table.contiguous()
         ctx.on_chip = _g.rel_rows_supported(q) and aux["n_used"] <= _g.REL_MAX_USED_TYPES and not _g.force_generic_enabled()
-        # where forward and backward both run on the tile kernels, the term and its gradient are stored in the order in
-        # which the tiles meet the edges (rows_slot: the row of every in-CSR slot) instead of by edge id
-        pair = _g.attention_pair_rows(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k, dropout_p) if ctx.on_chip else None
+        # where forward and backward both run on the tile kernels, the term and its gradient are stored head-major in the
+        # order in which the tiles meet the edges (rows_slot: the place of every in-CSR slot) instead of by edge id
+        graph = (row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k)
+        pair = _g.attention_pair_rows(*graph, dropout_p) if ctx.on_chip else None
         ctx.rows_slot = None
         if pair is not None:
             held = aux.get("rows_slot")
             if held is None or held[0] is not pair:
-                held = aux["rows_slot"] = (pair, pair.index_select(0, eid_c).contiguous())
+                rows_slot = pair.index_select(0, eid_c).contiguous()
+                # per pair number: the number of its edge's type and which row of its tile its destination is
+                types = torch.empty_like(aux["number_slot"]).index_copy_(0, rows_slot, aux["number_slot"]).to(torch.int32)
+                held = aux["rows_slot"] = (pair, rows_slot, (types | (_g.attention_pair_members(*graph, dropout_p) << 8)).contiguous())
             ctx.rows_slot = held[1]
-        if ctx.on_chip:
-            bias = _g.rel_bias_forward(col, indptr_c, eid_c if ctx.rows_slot is None else ctx.rows_slot, aux["number_slot"], q, table,
-                                       used_types=aux["used_types"])
+            bias = _g.rel_bias_forward_tiles(*graph, table, aux["used_types"], held[2], dropout_p)
+        elif ctx.on_chip:
+            bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["number_slot"], q, table, used_types=aux["used_types"])
         else:
             bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["etype_slot"], q, table)
         o, lse = _g.attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale, dropout_p, seed, bias=bias,
@@ -137,7 +141,7 @@ class BPTRelAttention(Function):
                                                bias_by_pair=ctx.rows_slot is not None)
         if ctx.on_chip:
             dtable = _g.rel_bias_backward(col, indptr_c, eid_c if ctx.rows_slot is None else ctx.rows_slot, aux["number_slot"], aux["used"],
-                                          aux["used_types"], ds, q, table, dq)
+                                          aux["used_types"], ds, q, table, dq, by_pair=ctx.rows_slot is not None)
         else:
             t_row, t_indptr, t_order, t_dst = _rel_type_rows(aux, ctx.etype, col, indptr_c, eid_c, table.size(0))
             h = q.size(1)

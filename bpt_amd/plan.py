@@ -143,16 +143,17 @@ def link_groups_host(grp_dst, grp_src, n_edges):
 
 
 def _bias_rows_of(groups_struct, pair_eid, eids, n_edges):
-    """For a plan's tile groups: the struct with grp_bias_idx = the pair number of every (entry, member) (n_edges where
-    there is no such pair), laid out like grp_eids, and the pair number of every edge id."""
-    device = eids.device
-    pair_of_eid = torch.empty(n_edges + 1, dtype=torch.int64, device=device)
-    pair_of_eid[pair_eid.to(torch.int64)] = torch.arange(n_edges, dtype=torch.int64, device=device)
-    pair_of_eid[n_edges] = n_edges
-    bias_idx = pair_of_eid.index_select(0, eids.reshape(-1).to(torch.int64)).to(torch.int32).contiguous()
+    """For a plan's tile groups: the struct with bias_by_pair set (the per-edge score term is read, and its gradient
+    written, head-major at the plan's own pair numbers), the pair number of every edge id, and for every pair number its
+    member index in its tile (the position of its bit in its entry's mask), int32."""
+    pair_of_eid = torch.empty(n_edges, dtype=torch.int64, device=pair_eid.device)
+    pair_of_eid[pair_eid[:n_edges].to(torch.int64)] = torch.arange(n_edges, dtype=torch.int64, device=pair_eid.device)
+    # eids is (entries, R) with n_edges where an entry has no such member: the pairs in their own order are its other elements
+    R = int(groups_struct.grp_R)
+    member = (torch.nonzero(eids.reshape(-1) < n_edges).flatten() % R).to(torch.int32)
     st = PlanStruct.from_buffer_copy(groups_struct)
-    st.grp_bias_idx = bias_idx.data_ptr()
-    return {"struct": st, "bias_idx": bias_idx, "pair_of_eid": pair_of_eid[:n_edges].contiguous()}
+    st.bias_by_pair = 1
+    return {"struct": st, "pair_of_eid": pair_of_eid, "member_of_pair": member}
 
 
 def pair_numbers_host(grp_mine, grp_theirs, n_edges):
@@ -251,9 +252,9 @@ class Plan:
         return hit
 
     def bias_rows(self, R=TILE_GROUP_R):
-        """The tile groups with the rows of the per-edge score term numbered by the plan's own pairs (grp_bias_idx): dict
-        with "struct" (the `bpt_plan`) and "pair_of_eid" (the pair number of every edge id).  Needs a plan that covers
-        every edge."""
+        """The tile groups for a per-edge score term stored in the order of the plan's own pairs (bias_by_pair): dict
+        with "struct" (the `bpt_plan`), "pair_of_eid" (the pair number of every edge id) and "member_of_pair" (the member
+        index of every pair in its tile).  Needs a plan that covers every edge."""
         with self._lock:
             hit = self._bias_rows.get(R)
         if hit is None:

@@ -80,12 +80,15 @@ typedef struct {
                                     [u * grp_R + m]; n_edges where the entry's mask has no bit m and in the 8
                                     entries of padding.  Needed by the attention calls that take a per-edge score
                                     term or dropout and by the row-group kernels of the SDDMM / SpMM-shaped ops */
-    const int32_t *grp_bias_idx; /* NULL, or laid out like grp_eids (grp_R = 16 only): the row of `bias` and of `ds_out`
-                                    that belongs to (entry u, member m), n_edges where there is no such pair.  NULL: the
-                                    edge id (grp_eids).  With the plan's own pair numbers here (the entry's first pair +
-                                    the member's rank in the mask) a tile's rows of the score term are neighbours in
-                                    memory instead of scattered by edge id; forward and backward must then be given the
-                                    same numbering, and whoever produces `bias` / consumes `ds_out` uses it too */
+    int64_t bias_by_pair;        /* 0: the per-edge score term `bias` and its gradient `ds_out` are (n_edges + 1, h)
+                                    arrays with one row per edge id.  Non-zero (grp_R = 16 only): they are (h, n_edges)
+                                    arrays, head-major, and the value of (entry u, member m) sits at
+                                    [head * n_edges + grp_entries[u].first_pair + (number of mask bits below m)], the
+                                    plan's own pair number: a tile's values are neighbours in memory and no index is
+                                    read on the way.  Forward and backward must be given the same setting, and whoever
+                                    produces `bias` / consumes `ds_out` uses the same places: bpt_rel_bias_forward /
+                                    _backward do when THEIR plan has the flag set and carries, as eid, the pair number
+                                    of every slot's edge */
 } bpt_plan;
 
 const char *bpt_strerror(int status);
@@ -174,9 +177,23 @@ int bpt_vector_spmm_backward(const bpt_plan *plan, const bpt_plan *plan_t, const
  * used_types (n_used) int32: the edge types that occur, in any order without repeats, and idx[p] is the NUMBER of the
  * slot's type in that list (n_index_nodes = n_used).  The kernel keeps those rows of the table on chip and multiplies
  * on the matrix cores; h in {4, 8, 16}, d = 64, f32 or bf16, n_used <= 240 (BPT_ERR_UNSUPPORTED else).  In this form
- * bias must have n_edges + 1 rows: the kernel also clears row n_edges, the spare row of bpt_attention_forward. */
+ * bias must have n_edges + 1 rows: the kernel also clears row n_edges, the spare row of bpt_attention_forward.
+ * With plan->bias_by_pair set (this form only) the result goes to bias[head * n_edges + eid[p]] instead, (h, n_edges)
+ * floats, the layout bpt_attention_forward reads when its plan has the flag; eid[p] then has to be the attention
+ * plan's pair number of the slot's edge. */
 int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table, const int32_t *used_types, int64_t n_used,
                          float *bias, int h, int d, int dtype, void *stream);
+
+/* The same score term (modules/attention.py:69-71) for a term kept in the pair order of the attention kernels' tile plan:
+ * `plan` is that plan (the destination side's, grp_R = 16), and the value of pair number t and a head goes to
+ * bias[head * n_edges + t], (h, n_edges) floats, the layout bpt_attention_forward reads with plan->bias_by_pair.
+ * pair_types (n_edges) int32: for pair number t, (number of its edge's type in used_types) | (its member index in the tile,
+ * i.e. the position of its mask bit) << 8.  used_types (n_used) as for bpt_rel_bias_forward.  One wavefront per tile and
+ * head multiplies the tile's 16 rows of q with all n_used table rows on the matrix cores, and every pair picks its value;
+ * all per-pair reads and writes are contiguous.  h in {4, 8, 16}, d = 64, f32 or bf16, n_used <= 240, a plan with tiles
+ * (BPT_ERR_UNSUPPORTED else). */
+int bpt_rel_bias_forward_tiles(const bpt_plan *plan, const void *q, const void *table, const int32_t *used_types, int64_t n_used,
+                               const int32_t *pair_types, float *bias, int h, int d, int dtype, void *stream);
 
 /* Gradients of that score term, the backward of embed_ak + node_mul_edge in modules/attention.py:55-56,69-71 (autograd of
  * nn.Embedding and graphop.py's NodeMulEdgeFunction.backward), from ds (n_edges or more rows, h) float32 =
@@ -187,6 +204,8 @@ int bpt_rel_bias_forward(const bpt_plan *plan, const void *q, const void *table,
  * bpt_rel_bias_forward with used_types: idx[p] is the number of the slot's type.  used (n_types) int32 is the inverse:
  * for every type in used_types its number, -1 for the others, whose rows of dtable become zero.  dq and dtable have the
  * dtype of q and table.  workspace: bpt_rel_bias_backward_workspace_bytes(plan, n_used, h) bytes, 16-byte aligned.
+ * With plan->bias_by_pair set, ds is read as (h, n_edges), ds[head * n_edges + eid[p]], the layout
+ * bpt_attention_backward writes when its plan has the flag.
  * Row-owned sums in a fixed order, no atomics.  h in {4, 8, 16}, d = 64, f32 or bf16, n_used <= 240;
  * BPT_ERR_UNSUPPORTED otherwise (compose bpt_vector_spmm_forward calls instead). */
 int64_t bpt_rel_bias_backward_workspace_bytes(const bpt_plan *plan, int64_t n_used, int h);
@@ -200,8 +219,10 @@ int bpt_rel_bias_backward(const bpt_plan *plan, const float *ds, const void *q, 
  * lse (n, h) float32 receives the base-2 log-sum-exp of the scaled scores, needed by backward.
  * f32 and bf16 only (accumulation in f32).
  * bias: NULL, or float32 (n_edges + 1, h): per edge and head, added to q.k before scaling (the rel_pos term,
- * bpt_rel_bias_forward); row n_edges is a spare row that is read for absent pairs and never used.  Needs the row
- * groups with grp_eids (BPT_ERR_UNSUPPORTED / BPT_ERR_PLAN without them).
+ * bpt_rel_bias_forward); row n_edges is a spare row that is read for absent pairs and never used.  With
+ * plan_in->bias_by_pair set: float32 (h, n_edges) in the plan's pair order (see bpt_plan; tile kernels only,
+ * BPT_ERR_PLAN where they do not run).  Needs the row groups with grp_eids (BPT_ERR_UNSUPPORTED / BPT_ERR_PLAN
+ * without them).
  * dropout_p in [0, 1): dropout on the attention probabilities (attention.py:73); 0 = none.  Each (edge, head) is
  * kept with probability 1 - p and scaled by 1 / (1 - p); the decision is a hash of (dropout_seed, edge id, head),
  * so it does not depend on the plan and backward only needs the same p and seed.  Needs the row groups with
@@ -210,7 +231,8 @@ int bpt_attention_forward(const bpt_plan *plan_in, const void *q, const void *k,
                           void *o, float *lse, void *workspace, int64_t workspace_bytes,
                           float scale, float dropout_p, uint64_t dropout_seed, int h, int d, int dtype, void *stream);
 
-/* Backward of bpt_attention_forward.  With bias, ds_out (float32 (n_edges + 1, h), row n_edges spare) receives
+/* Backward of bpt_attention_forward.  With bias, ds_out (float32 (n_edges + 1, h), row n_edges spare; with
+ * plan_in->bias_by_pair (h, n_edges), laid out like bias) receives
  * dL/d(q.k + bias) of every edge and head, from which the caller forms the gradients of what produced the bias
  * (for rel_pos: dq += sum_e ds[e] * table[type(e)], dtable[t] = sum_{e of type t} sum_h ds[e, h] * q[dst(e), h]);
  * bias and ds_out are both given or both NULL. */

@@ -111,6 +111,59 @@ def test_score_term_gradients_match_node_mul_edge_backward(ops, gname, dtype, h,
     assert torch.equal(again, dtable), "the sums have a fixed order: the same bits every run"
 
 
+@pytest.mark.parametrize("dtype,h", SHAPES)
+@pytest.mark.parametrize("gname", ["bpt512_k4", "multigraph", "fc_w100"])
+def test_head_major_form_of_the_score_term_kernels(ops, gname, dtype, h):
+    """by_pair: the term goes to, and its gradient comes from, (h, E) arrays at the places the plan's eid array names (any
+    permutation of the edges will do here): the same bits as the (E, h) form, moved."""
+    graphop, _ = ops
+    d, n_types = 64, 1000
+    c = case(gname)
+    q = rand((c.n, h, d), dtype, 71, 0.5).to(DEV)
+    table = rand((n_types, d), dtype, 72, 0.5).to(DEV)
+    et = edge_types(c.E, n_types, 55, 73)
+    used, used_types, number_slot = used_map(et[c.np_in[2]], n_types)
+    place = torch.from_numpy(np.random.default_rng(74).permutation(c.E)).to(DEV)           # place of edge e
+    place_slot = place.index_select(0, c.inn[2]).contiguous()
+    tail = (dev(number_slot), q, table)
+    by_eid = graphop.rel_bias_forward(*c.inn[:3], *tail, used_types=dev(used_types))
+    moved = graphop.rel_bias_forward(*c.inn[:2], place_slot, *tail, used_types=dev(used_types), by_pair=True)
+    assert moved.shape == (h, c.E)
+    assert torch.equal(moved.t().index_select(0, place), by_eid[:c.E])
+    ds = rand((c.E, h), torch.float32, 75, 0.1).to(DEV)
+    ds_moved = torch.empty_like(ds).index_copy_(0, place, ds).t().contiguous()
+    dq0 = rand((c.n, h, d), dtype, 76, 0.5).to(DEV)
+    maps = (dev(number_slot), dev(used), dev(used_types))
+    dq_a, dq_b = dq0.clone(), dq0.clone()
+    dt_a = graphop.rel_bias_backward(*c.inn[:3], *maps, torch.cat([ds, torch.zeros(1, h, device=DEV)]), q, table, dq_a)
+    dt_b = graphop.rel_bias_backward(*c.inn[:2], place_slot, *maps, ds_moved, q, table, dq_b, by_pair=True)
+    assert torch.equal(dt_a, dt_b) and torch.equal(dq_a, dq_b)
+    with pytest.raises(ValueError, match="used_types"):
+        graphop.rel_bias_forward(*c.inn[:2], place_slot, dev(et[c.np_in[2]]), q, table, by_pair=True)
+
+
+@pytest.mark.parametrize("dtype,h", SHAPES)
+@pytest.mark.parametrize("gname,n_types,n_used", [("bpt512_k4", 1000, 55), ("bpt300_causal_k2", 37, 37), ("multigraph", 400, 230),
+                                                  ("fc_w100", 1000, 100), ("blocks8x30", 5, 1)])
+def test_score_term_over_the_tile_plan(ops, gname, dtype, h, n_types, n_used):
+    """rel_bias_forward_tiles: the term in the tiles' pair order, head-major, against node_mul_edge of the looked-up rows."""
+    graphop, _ = ops
+    d = 64
+    c = case(gname)
+    q = rand((c.n, h, d), dtype, 81, 0.5).to(DEV)
+    table = rand((n_types, d), dtype, 82, 0.5).to(DEV)
+    et = edge_types(c.E, n_types, n_used, 83)
+    used, used_types, _ = used_map(et, n_types, seed=84)
+    pair = graphop.attention_pair_rows(*c.out, *c.inn, q, q)
+    member = graphop.attention_pair_members(*c.out, *c.inn, q, q)
+    assert pair is not None and member.shape == (c.E,) and member.dtype == torch.int32 and 0 <= int(member.min()) and int(member.max()) < 16
+    number_pair = torch.empty(c.E, dtype=torch.int32, device=DEV).index_copy_(0, pair, dev(used[et]))
+    bias = graphop.rel_bias_forward_tiles(*c.out, *c.inn, q, q, table, dev(used_types), (number_pair | (member << 8)).contiguous())
+    assert bias.shape == (h, c.E) and bias.dtype == torch.float32
+    want = oracle.node_mul_edge_forward(*c.np_in[:3], f64(q), f64(table)[et])
+    close(bias.t().index_select(0, pair), want, TOL[dtype], "score term")
+
+
 def test_too_many_used_types_is_refused_and_the_layer_takes_the_spmm_form(ops):
     graphop, op = ops
     h, d, n_types = 8, 64, 1000
@@ -158,8 +211,8 @@ def test_graph_without_edges_gives_a_zero_table_gradient(ops):
 @pytest.mark.parametrize("gname", ["bpt512_k4", "multigraph", "fc_w100"])
 @pytest.mark.parametrize("p", [0.0, 0.25])
 def test_score_term_in_the_order_of_the_tiles_gives_the_same_step(ops, gname, dtype, p):
-    """A score term stored by the tile plan's pair numbers (attention_pair_rows, bias_by_pair) instead of by edge id:
-    the same o, lse, dq, dk, dv bit for bit, and ds the same values in the other order."""
+    """A score term stored head-major at the tile plan's pair numbers (attention_pair_rows, bias_by_pair) instead of by
+    edge id: the same o, lse, dq, dk, dv bit for bit, and ds the same values in the other layout."""
     graphop, _ = ops
     h, d = 8, 64
     c = case(gname)
@@ -169,7 +222,7 @@ def test_score_term_in_the_order_of_the_tiles_gives_the_same_step(ops, gname, dt
     assert pair is not None and pair.shape == (c.E,) and torch.equal(torch.sort(pair).values, torch.arange(c.E, device=DEV))
     zero = torch.zeros(1, h, device=DEV)
     by_eid = torch.cat([term, zero])
-    by_pair = torch.cat([torch.empty_like(term).index_copy_(0, pair, term), zero])
+    by_pair = torch.empty_like(term).index_copy_(0, pair, term).t().contiguous()          # (h, E)
     got = {}
     for name, bias, flag in (("eid", by_eid, False), ("pair", by_pair, True)):
         o, lse = graphop.attention_forward(*c.inn, q, k, v, dropout_p=p, seed=77, bias=bias, bias_by_pair=flag)
@@ -177,7 +230,8 @@ def test_score_term_in_the_order_of_the_tiles_gives_the_same_step(ops, gname, dt
                                                                bias_by_pair=flag))
     for a, b, what in zip(got["eid"][:5], got["pair"][:5], ("o", "lse", "dq", "dk", "dv")):
         assert torch.equal(a, b), what
-    assert torch.equal(got["eid"][5], got["pair"][5].index_select(0, pair)), "ds"
+    assert got["pair"][5].shape == (h, c.E)
+    assert torch.equal(got["eid"][5], got["pair"][5].t().index_select(0, pair)), "ds"
 
 
 def test_the_order_of_the_tiles_is_offered_only_where_both_passes_run_on_tiles(ops):
@@ -188,7 +242,7 @@ def test_the_order_of_the_tiles_is_offered_only_where_both_passes_run_on_tiles(o
     old = graphop.set_group_rows(4)                       # row groups of 4: no tiles
     try:
         assert graphop.attention_pair_rows(*c.out, *c.inn, q, k) is None
-        bias = torch.zeros(c.E + 1, 8, device=DEV)
+        bias = torch.zeros(8, c.E, device=DEV)
         with pytest.raises(RuntimeError, match="bias_by_pair"):
             graphop.attention_forward(*c.inn, q, k, v, bias=bias, bias_by_pair=True)
     finally:
