@@ -7,6 +7,8 @@ rtol 1e-4 (atol 1e-5); bfloat16 rtol 2e-2 (atol 2e-2).
   configuration 3 in bfloat16: L = 8192, k = 4, causal (float32: tests/test_gpu_parity.py::test_headline_graph_full_parity)
   configuration 4: L = 4096, causal, k in {1, 2, 4, 8, 16, 32}, and the window-128 graph (FullyConnected); k = 32 and the
                    window graph also in bfloat16
+  configuration 3 with the rel_pos score term (modules/attention.py:69-71; table (1000, 64), the graph's own edge types),
+                   float32 and bfloat16, and the same on L = 4096, k = 8 with 16 heads
 """
 import numpy as np
 import pytest
@@ -105,3 +107,47 @@ def test_cfg4_dense_graphs_bf16(which):
     g = gb.BinaryPartition(4096, True, 32, 10) if which == "k32" else gb.FullyConnected(4096, True, 128)
     src, dst, _ = g.get_edges()
     run_layer(src, dst, g.number_of_nodes, 8, 64, torch.bfloat16)
+
+
+def run_layer_with_rel_pos(g, h, d, dtype, n_types=1000):
+    """The fused layer with the score term q[dst] . table[etype] against the oracle's op sequence on the looked-up rows; the
+    table's gradient is the oracle's per-edge dak summed per edge type."""
+    from bpt_amd import graphbuilder as gb
+    from bpt_amd import op
+    src, dst, etype = g.get_edges()[:3]
+    n = g.number_of_nodes
+    etype = np.asarray(etype, dtype=np.int64)
+    assert 0 <= etype.min() and etype.max() < n_types
+    csr = gb.get_csrs(src, dst, n, as_torch=False)
+    out_csr, in_csr, ROW, IR, COL, IC = csr
+    t = lambda a: torch.from_numpy(a).to(DEV)
+    args = (t(ROW), t(IR), t(out_csr[2]), t(out_csr[1]), t(COL), t(IC), t(in_csr[2]), t(in_csr[1]))
+    gen = torch.Generator().manual_seed(2345)
+    q, k, v, do = ((torch.randn(n, h, d, generator=gen) / 8).to(dtype) for _ in range(4))
+    table = (torch.randn(n_types, d, generator=gen) / 8).to(dtype)
+    qd, kd, vd, td = (x.to(DEV).requires_grad_(True) for x in (q, k, v, table))
+    o = op.bpt_attention(*args, qd, kd, vd, rel_table=td, etype=t(etype))
+    o.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    ak = f64(table)[etype]
+    ro, ra = oracle.attention_forward(csr, f64(q), f64(k), f64(v), ak=ak)
+    rdq, rdk, rdv, rdak = oracle.attention_backward(csr, f64(q), f64(k), f64(v), ra, f64(do), ak=ak)
+    rdt = np.zeros((n_types, d))
+    np.add.at(rdt, etype, rdak)
+    check(o, ro, TOL[dtype], "o")
+    for got, want, nm in ((qd.grad, rdq, "dq"), (kd.grad, rdk, "dk"), (vd.grad, rdv, "dv")):
+        check(got, want, GTOL[dtype], nm)
+    check(td.grad, rdt, GTOL[dtype], "dtable")
+    return len(np.unique(etype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cfg3_with_rel_pos_full_size(dtype):
+    from bpt_amd import graphbuilder as gb
+    g = gb.BinaryPartition(8192, True, 4, 10)
+    assert run_layer_with_rel_pos(g, 8, 64, dtype) == 55
+
+
+def test_16_heads_with_rel_pos_l4096_k8():
+    from bpt_amd import graphbuilder as gb
+    run_layer_with_rel_pos(gb.BinaryPartition(4096, True, 8, 10), 16, 64, torch.float32)
