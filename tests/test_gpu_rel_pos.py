@@ -164,6 +164,34 @@ def test_score_term_over_the_tile_plan(ops, gname, dtype, h, n_types, n_used):
     close(bias.t().index_select(0, pair), want, TOL[dtype], "score term")
 
 
+@pytest.mark.parametrize("gname", ["bpt512_k4", "multigraph"])
+def test_layer_with_the_term_is_the_same_on_host_built_and_gpu_built_plans(ops, gname):
+    """The pair order and the member index of every pair come from either builder's tile groups (which need not be the same
+    groups): the same step within the stated tolerances."""
+    from bpt_amd import plan
+    _, op = ops
+    h, d, n_types = 8, 64, 40
+    c = case(gname)
+    etype = torch.from_numpy(np.random.default_rng(91).integers(0, n_types, c.E)).to(DEV)
+    got = []
+    for on_gpu in (False, True):
+        plan.plan_cache.clear()
+        old = plan.set_device_build(on_gpu)
+        try:
+            q, k, v, do = (rand((c.n, h, d), torch.float32, s, 1.0 / 8).to(DEV) for s in (92, 93, 94, 95))
+            table = rand((n_types, d), torch.float32, 96, 1.0 / 8).to(DEV)
+            for t in (q, k, v, table):
+                t.requires_grad_(True)
+            o = op.bpt_attention(*c.out, *c.inn, q, k, v, rel_table=table, etype=etype)
+            o.backward(do)
+            got.append((o.detach(), q.grad, k.grad, v.grad, table.grad))
+        finally:
+            plan.set_device_build(old)
+            plan.plan_cache.clear()
+    for a, b, what in zip(*got, ("o", "dq", "dk", "dv", "dtable")):
+        close(a, f64(b), TOL[torch.float32] if what == "o" else GTOL[torch.float32], what)
+
+
 def test_too_many_used_types_is_refused_and_the_layer_takes_the_spmm_form(ops):
     graphop, op = ops
     h, d, n_types = 8, 64, 1000
