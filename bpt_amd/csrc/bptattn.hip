@@ -3008,6 +3008,7 @@ __global__ __launch_bounds__(HW * WAVE) void k_rel_bias_tiles(bpt_plan P, const 
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
     const int4 last = entries[t.p_end - 1];
     const int first = __builtin_amdgcn_readfirstlane(entries[t.p_begin].z), end = __builtin_amdgcn_readfirstlane(last.z + __popc((uint32_t)last.y));
+    if (end <= first) return;
     constexpr int AHEAD = 4;                                    // pairs per lane whose loads are in flight together
     int tm[AHEAD];
 #pragma unroll
