@@ -540,12 +540,12 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     if lse.dtype != torch.float32 or lse.device != q.device:
         raise ValueError("lse must be the float32 tensor that attention_forward returned")
     _expect_shape(lse, (q.size(0), h), "lse")
+    _check_bias(bias, eid_c.size(0), h, q.device, cfg, bias_by_pair)
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     on_gpu = _tiles(q, h, d, None, dropout_p, bias, cfg)        # (as in attention_forward)
     plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), prefer_device=on_gpu)
     plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), prefer_device=on_gpu)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    _check_bias(bias, eid_c.size(0), h, q.device, cfg, bias_by_pair)
     ds = torch.empty((h, eid_c.size(0)) if bias_by_pair else (eid_c.size(0) + 1, h), dtype=torch.float32, device=q.device) if bias is not None else None
     dt = _dtype(q)
     in_ref, out_ref = plan_in.ref, plan_out.ref

@@ -137,6 +137,33 @@ def test_rel_bias_checks(g):
         g.rel_bias_forward(*INN[:3], INN[3], node(), table, used_types=i32(3))
 
 
+def test_score_term_in_pair_order_checks(g):
+    """The (h, E) forms: the term over the tile plan, ds of the gradient op, bias of the fused calls."""
+    i32 = lambda n, v=0: torch.full((n,), v, dtype=torch.int32)
+    table, used_types = torch.zeros(1000, D), i32(3)
+    def tiles(**kw):
+        args = dict(q=node(), k=node(), table=table, used_types=used_types, pair_types=i32(E))
+        args.update(kw)
+        return g.rel_bias_forward_tiles(*OUT, *INN, args["q"], args["k"], args["table"], args["used_types"], args["pair_types"])
+    for kw in (dict(pair_types=i32(E - 1)), dict(pair_types=torch.zeros(E, dtype=torch.int64)), dict(table=torch.zeros(1000, D // 2)),
+               dict(used_types=torch.zeros(3, dtype=torch.int64)), dict(used_types=i32(1001))):
+        with pytest.raises(ValueError):
+            tiles(**kw)
+    with pytest.raises(RuntimeError, match="tile kernels"):
+        tiles()                                          # (well formed, but no tile kernels run on host tensors)
+    used = i32(1000, -1)
+    for ds in (torch.zeros(E + 1, H), torch.zeros(H, E + 1), torch.zeros(H, E, dtype=torch.float64)):
+        with pytest.raises(ValueError):
+            g.rel_bias_backward(*INN[:3], INN[3], used, used_types, ds, node(), table, node(), by_pair=True)
+    with pytest.raises(ValueError, match="used_types"):
+        g.rel_bias_forward(*INN[:3], INN[3], node(), table, by_pair=True)
+    for bias in (torch.zeros(E + 1, H), torch.zeros(H, E + 1)):
+        with pytest.raises(ValueError):
+            g.attention_forward(*INN, node(), node(), node(), bias=bias, bias_by_pair=True)
+        with pytest.raises(ValueError):
+            g.attention_backward(*OUT, *INN, node(), node(), node(), node(), torch.zeros(N, H), node(), bias=bias, bias_by_pair=True)
+
+
 def test_well_formed_calls_get_past_the_checks(g):
     # the same calls with fitting tensors reach the plan cache (which this fixture turns into an AssertionError)
     with pytest.raises(AssertionError):
