@@ -7,6 +7,7 @@ rtol 1e-4 (atol 1e-5); bfloat16 rtol 2e-2 (atol 2e-2).
   configuration 3 in bfloat16: L = 8192, k = 4, causal (float32: tests/test_gpu_parity.py::test_headline_graph_full_parity)
   configuration 4: L = 4096, causal, k in {1, 2, 4, 8, 16, 32}, and the window-128 graph (FullyConnected); k = 32 and the
                    window graph also in bfloat16
+  configuration 5: L = 32768, k = 8, causal, 16 heads, bfloat16 and float32 (half a minute of oracle time each)
   configuration 3 with the rel_pos score term (modules/attention.py:69-71; table (1000, 64), the graph's own edge types),
                    float32 and bfloat16, and the same on L = 4096, k = 8 with 16 heads
 """
@@ -107,6 +108,15 @@ def test_cfg4_dense_graphs_bf16(which):
     g = gb.BinaryPartition(4096, True, 32, 10) if which == "k32" else gb.FullyConnected(4096, True, 128)
     src, dst, _ = g.get_edges()
     run_layer(src, dst, g.number_of_nodes, 8, 64, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_cfg5_full_size(dtype):
+    from bpt_amd import graphbuilder as gb
+    g = gb.BinaryPartition(32768, True, 8, 10)
+    src, dst, _ = g.get_edges()
+    assert (g.number_of_nodes, len(src)) == (65535, 3293955)
+    run_layer(src, dst, g.number_of_nodes, 16, 64, dtype)
 
 
 def run_layer_with_rel_pos(g, h, d, dtype, n_types=1000):
