@@ -121,7 +121,15 @@ class BPTRelAttention(Function):
                 types = torch.empty_like(aux["number_slot"]).index_copy_(0, rows_slot, aux["number_slot"]).to(torch.int32)
                 held = aux["rows_slot"] = (pair, rows_slot, (types | (_g.attention_pair_members(*graph, dropout_p) << 8)).contiguous())
             ctx.rows_slot = held[1]
-            bias = _g.rel_bias_forward_tiles(*graph, table, aux["used_types"], held[2], dropout_p)
+            try:
+                bias = _g.rel_bias_forward_tiles(*graph, table, aux["used_types"], held[2], dropout_p)
+            except RuntimeError as err:
+                # (many types in use need more than 64 KB of LDS there, which a runtime may refuse: the kernel over the
+                # in-CSR writes the same layout from within 64 KB)
+                if "(status -7)" not in str(err):
+                    raise
+                bias = _g.rel_bias_forward(col, indptr_c, ctx.rows_slot, aux["number_slot"], q, table, used_types=aux["used_types"],
+                                           by_pair=True)
         elif ctx.on_chip:
             bias = _g.rel_bias_forward(col, indptr_c, eid_c, aux["number_slot"], q, table, used_types=aux["used_types"])
         else:

@@ -192,6 +192,33 @@ def test_layer_with_the_term_is_the_same_on_host_built_and_gpu_built_plans(ops, 
         close(a, f64(b), TOL[torch.float32] if what == "o" else GTOL[torch.float32], what)
 
 
+def test_layer_falls_back_to_the_in_csr_kernel_where_the_tile_form_is_refused(ops, monkeypatch):
+    """BPTRelAttention where rel_bias_forward_tiles reports an unsupported configuration (forced here): the term comes from
+    the kernel over the in-CSR, in the same layout, and the step is the same within the stated tolerances."""
+    graphop, op = ops
+    h, d, n_types = 8, 64, 60
+    c = case("bpt512_k4")
+    etype = torch.from_numpy(np.random.default_rng(111).integers(0, n_types, c.E)).to(DEV)
+    def step():
+        q, k, v, do = (rand((c.n, h, d), torch.float32, s, 1.0 / 8).to(DEV) for s in (112, 113, 114, 115))
+        table = rand((n_types, d), torch.float32, 116, 1.0 / 8).to(DEV)
+        for t in (q, k, v, table):
+            t.requires_grad_(True)
+        o = op.bpt_attention(*c.out, *c.inn, q, k, v, rel_table=table, etype=etype)
+        o.backward(do)
+        return o.detach(), q.grad, k.grad, v.grad, table.grad
+    want = step()
+    calls = []
+    def refused(*a, **kw):
+        calls.append(1)
+        raise RuntimeError("rel_bias_forward_tiles: unsupported (status -7)")
+    monkeypatch.setattr(graphop, "rel_bias_forward_tiles", refused)
+    got = step()
+    assert calls, "the tile form was not asked for: the test does not reach the fallback"
+    for a, b, what in zip(got, want, ("o", "dq", "dk", "dv", "dtable")):
+        close(a, f64(b), TOL[torch.float32] if what == "o" else GTOL[torch.float32], what)
+
+
 def test_too_many_used_types_is_refused_and_the_layer_takes_the_spmm_form(ops):
     graphop, op = ops
     h, d, n_types = 8, 64, 1000
