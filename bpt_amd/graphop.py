@@ -494,16 +494,19 @@ def attention_forward(col, indptr_c, eid_c, indices_c, q, k, v, scale=None, drop
     _expect_shape(k, (k.size(0),) + tuple(q.shape[1:]), "k")
     _expect_shape(v, k.shape, "v")
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
-    # (where the tile kernels may run, the plan that the choices below look at comes from the GPU builder too: 0.2 ms
-    # instead of 1.5 ms for a new graph of 16 K rows)
-    plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), prefer_device=_tiles(q, h, d, None, dropout_p, bias, cfg))
-    tiles = False
-    if not _attention_groups(plan, dropout_p, bias, q, k, cfg):
-        ref = plan.ref
-    elif _tiles(q, h, d, plan, dropout_p, bias, cfg):
-        plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=_tile_seg_len(plan), prefer_device=True)
+    seg = _tile_seg_without_plan(col, eid_c.size(0), q, k, h, d, dropout_p, bias, cfg)
+    if seg is None:
+        # the choices look at a plan of the graph (where the tile kernels may run it comes from the GPU builder too:
+        # 0.2 ms instead of 1.5 ms for a new graph of 16 K rows)
+        plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), prefer_device=_tiles(q, h, d, None, dropout_p, bias, cfg))
+        if _attention_groups(plan, dropout_p, bias, q, k, cfg) and _tiles(q, h, d, plan, dropout_p, bias, cfg):
+            seg = _tile_seg_len(plan)
+    tiles = seg is not None
+    if tiles:
+        plan = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg, prefer_device=True)
         ref = ctypes.byref(plan.bias_rows(TILE_ROWS)["struct"] if bias_by_pair else plan.ensure_groups(TILE_ROWS)["struct"])
-        tiles = True
+    elif not _attention_groups(plan, dropout_p, bias, q, k, cfg):
+        ref = plan.ref
     else:
         ref = ctypes.byref(plan.ensure_groups(_forward_rows(q, h, d, plan, cfg))["struct"])
     if bias_by_pair and not (tiles and bias is not None):
@@ -543,26 +546,36 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
     _check_bias(bias, eid_c.size(0), h, q.device, cfg, bias_by_pair)
     scale = 1.0 / math.sqrt(d) if scale is None else float(scale)
     on_gpu = _tiles(q, h, d, None, dropout_p, bias, cfg)        # (as in attention_forward)
-    plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), prefer_device=on_gpu)
-    plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), prefer_device=on_gpu)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     ds = torch.empty((h, eid_c.size(0)) if bias_by_pair else (eid_c.size(0) + 1, h), dtype=torch.float32, device=q.device) if bias is not None else None
     dt = _dtype(q)
-    in_ref, out_ref = plan_in.ref, plan_out.ref
-    tiles = False
-    if _attention_groups(plan_in, dropout_p, bias, q, k, cfg) and plan_in.covers_all_edges and plan_out.covers_all_edges:
-        if _tiles(q, h, d, plan_in, dropout_p, bias, cfg) and _tiles_backward(plan_in, q.dtype, bias):
-            seg = _tile_seg_len(plan_in)
-            plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg, prefer_device=True)
-            plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg, prefer_device=True)
-            # the destination side writes (p, ds) by its own pair numbers; the source side finds them through its pair mapping
-            in_ref = ctypes.byref(plan_in.bias_rows(TILE_ROWS)["struct"] if bias_by_pair else plan_in.ensure_groups(TILE_ROWS)["struct"])
-            out_ref = ctypes.byref(plan_out.linked_to(plan_in, TILE_ROWS, partner_order=None, pair_numbers=True))
-            tiles = True
-        else:
-            R = _group_rows(q, h, d, plan_in, cfg)
-            in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
-            out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
+    def tile_plans(seg):
+        """The two tile plans and the structs the kernels take, or None where a side does not cover every edge."""
+        pi = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg, prefer_device=True)
+        po = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg, prefer_device=True)
+        if not (pi.covers_all_edges and po.covers_all_edges):
+            return None
+        # the destination side writes (p, ds) by its own pair numbers; the source side finds them through its pair mapping
+        return (pi, po, ctypes.byref(pi.bias_rows(TILE_ROWS)["struct"] if bias_by_pair else pi.ensure_groups(TILE_ROWS)["struct"]),
+                ctypes.byref(po.linked_to(pi, TILE_ROWS, partner_order=None, pair_numbers=True)))
+
+    # as in attention_forward: the tile plans straight away where the tile kernels are certain
+    seg = _tile_seg_without_plan(col, eid_c.size(0), q, k, h, d, dropout_p, bias, cfg) if _tiles_backward(None, q.dtype, bias) else None
+    chosen = tile_plans(seg) if seg is not None else None
+    if chosen is None:
+        plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), prefer_device=on_gpu)
+        plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), prefer_device=on_gpu)
+        in_ref, out_ref = plan_in.ref, plan_out.ref
+        if _attention_groups(plan_in, dropout_p, bias, q, k, cfg) and plan_in.covers_all_edges and plan_out.covers_all_edges:
+            if _tiles(q, h, d, plan_in, dropout_p, bias, cfg) and _tiles_backward(plan_in, q.dtype, bias):
+                chosen = tile_plans(_tile_seg_len(plan_in))
+            else:
+                R = _group_rows(q, h, d, plan_in, cfg)
+                in_ref = ctypes.byref(plan_in.linked_to(plan_out, R))
+                out_ref = ctypes.byref(plan_out.ensure_groups(R, GROUP_ORDER_SRC)["struct"])
+    tiles = chosen is not None
+    if tiles:
+        plan_in, plan_out, in_ref, out_ref = chosen
     if bias_by_pair and not (tiles and bias is not None):
         raise RuntimeError("bias_by_pair: this call does not run on the tile kernels (ask attention_pair_rows() first)")
     ws, nws = _workspace(OP_ATTN_BWD, plan_in, plan_out, h, d, dt, q.device, plan_ref=in_ref, plan_t_ref=out_ref)
@@ -583,10 +596,17 @@ def _pair_order(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c
     if q.dim() != 3 or not q.is_cuda:
         return None
     h, d = _hd(q)
+    marker = q                                             # (stands for "a score term is given" in the choices below)
+    seg = _tile_seg_without_plan(col, eid_c.size(0), q, k, h, d, dropout_p, marker, cfg) if attention_supported(q) and \
+        _tiles_backward(None, q.dtype, marker) else None
+    if seg is not None:
+        plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), seg_len=seg, prefer_device=True)
+        plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), seg_len=seg, prefer_device=True)
+        if plan_in.covers_all_edges and plan_out.covers_all_edges:
+            return plan_in, plan_in.bias_rows(TILE_ROWS)
     on_gpu = _tiles(q, h, d, None, dropout_p, q, cfg)
     plan_in = plan_cache.get(col, indptr_c, eid_c, indices_c, q.size(0), k.size(0), prefer_device=on_gpu)
     plan_out = plan_cache.get(row, indptr_r, eid_r, indices_r, k.size(0), q.size(0), prefer_device=on_gpu)
-    marker = q                                             # (stands for "a score term is given" in the choices below)
     if not (attention_supported(q) and _attention_groups(plan_in, dropout_p, marker, q, k, cfg) and plan_in.covers_all_edges
             and plan_out.covers_all_edges and _tiles(q, h, d, plan_in, dropout_p, marker, cfg)
             and _tiles_backward(plan_in, q.dtype, marker)):
@@ -728,6 +748,23 @@ def _tiles_backward(plan, dtype, bias=None):
     if TILE_BACKWARD is not None:
         return TILE_BACKWARD
     return True
+
+
+def _tile_seg_without_plan(units, n_edges, q, k, h, d, dropout_p, bias, cfg):
+    """The work-item length of the tile plans where the tile kernels are certain for this call without a plan of the
+    graph to look at, else None (the choices then look at one).  Certain: the shape has tile kernels, the node tensors
+    fit 32-bit offsets, and the graph has at least _MIN_GROUP_ITEMS rows with edges (`units` lists them; a plan has at
+    least one work item per such row) or the call carries dropout or a score term.  The length is _tile_seg_len's."""
+    if not (cfg.use_groups and _tiles(q, h, d, None, dropout_p, bias, cfg)):
+        return None
+    if max(q.size(0), k.size(0)) * h * d * q.element_size() >= 2 ** 32:
+        return None
+    if not (units.numel() >= _MIN_GROUP_ITEMS or dropout_p > 0.0 or bias is not None):
+        return None
+    if TILE_SEG_LEN is not None:
+        return TILE_SEG_LEN
+    deg = n_edges / max(q.size(0), 1)
+    return 64 if deg < 32 else (128 if deg < 80 else 256)
 
 
 def _tile_seg_len(plan):
