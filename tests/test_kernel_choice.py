@@ -1,5 +1,5 @@
 """Which kernel family a call takes is decided on the host from the plan's sizes and the dtype (graphop._tiles,
-_tiles_backward, _tile_seg_len) and where a plan is built from its size and the caller's preference
+_tiles_backward, _tile_seg_len, and _tile_seg_without_plan where no plan is needed to decide) and where a plan is built from its size and the caller's preference
 (plan._build_on_device, PlanCache.get(prefer_device=...)).  CPU only: the rules are plain functions of sizes."""
 from types import SimpleNamespace
 
@@ -51,6 +51,37 @@ def test_segment_length_of_the_tile_plans_follows_the_mean_degree():
     assert graphop._tile_seg_len(fake_plan(16383, 430237)) == 64           # 26 edges per row
     assert graphop._tile_seg_len(fake_plan(65535, 3293955)) == 128         # 50
     assert graphop._tile_seg_len(fake_plan(4097, 524224)) == 256           # 128
+
+
+def test_choice_of_the_tile_kernels_without_a_plan_to_look_at():
+    """_tile_seg_without_plan: the same answers as the rules that look at a plan wherever it gives one, None elsewhere."""
+    cfg = graphop._SETTINGS
+    q = torch.empty(16383, 8, 64)
+    units = lambda n: torch.empty(n, dtype=torch.int64)
+    seg = lambda un, E, qq=q, p=0.0, bias=None, c=None: graphop._tile_seg_without_plan(units(un), E, qq, qq, qq.size(1), qq.size(2), p, bias,
+                                                                                        cfg if c is None else c)
+    assert seg(16383, 430237) == graphop._tile_seg_len(fake_plan(16383, 430237)) == 64
+    assert seg(65535, 3293955, torch.empty(65535, 16, 64, dtype=torch.bfloat16)) == 128
+    assert seg(4097, 524224, torch.empty(4097, 8, 64)) == 256
+    assert seg(1535, 28378, torch.empty(1535, 8, 64)) is None              # few rows with edges: the plan's work items decide
+    assert seg(1536, 28378, torch.empty(1536, 8, 64)) == 64
+    assert seg(100, 1000, torch.empty(100, 8, 64), p=0.1) == 64            # dropout and the score term take groups anyway
+    assert seg(100, 1000, torch.empty(100, 8, 64), bias=object()) == 64
+    assert seg(16383, 430237, torch.empty(16383, 8, 32)) is None           # no tile kernels for 32 columns per head
+    assert seg(16383, 430237, torch.empty(16383, 8, 64, dtype=torch.float64)) is None
+    big = SimpleNamespace(size=lambda i: (1 << 22, 16, 64)[i], element_size=lambda: 4, dtype=torch.float32)
+    assert graphop._tile_seg_without_plan(units(1 << 22), 1 << 24, big, big, 16, 64, 0.0, None, cfg) is None     # 16 GiB of rows: no 32-bit offsets
+    old = graphop.set_group_rows(8)
+    try:
+        assert seg(16383, 430237, c=graphop._SETTINGS) is None             # a caller fixing the rows per group: no tiles
+    finally:
+        graphop.set_group_rows(old)
+    old = graphop.TILE_SEG_LEN
+    try:
+        graphop.TILE_SEG_LEN = 96
+        assert seg(16383, 430237) == 96
+    finally:
+        graphop.TILE_SEG_LEN = old
 
 
 def test_where_a_plan_is_built():
