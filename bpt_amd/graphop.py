@@ -406,7 +406,8 @@ def rel_bias_forward(col, indptr_c, eid_c, type_slot, q, table, used_types=None,
         _check_input(used_types, "used_types")
         if used_types.dtype != torch.int32 or used_types.dim() != 1 or used_types.numel() > table.size(0):
             raise ValueError("used_types must be a 1-D int32 tensor of at most table.size(0) elements")
-        plan = plan_cache.get(col, indptr_c, eid_c, type_slot, q.size(0), max(used_types.numel(), 1))
+        # (only work items are walked, no row groups: the GPU builder's plan, 0.2 ms instead of 2 ms for a new graph of 16 K rows)
+        plan = plan_cache.get(col, indptr_c, eid_c, type_slot, q.size(0), max(used_types.numel(), 1), prefer_device=True)
         ref, n_used = (ctypes.byref(_by_pair(plan.struct)) if by_pair else plan.ref), used_types.numel()
     else:
         if by_pair:
@@ -457,7 +458,7 @@ def rel_bias_backward(col, indptr_c, eid_c, number_slot, used, used_types, ds, q
         raise ValueError("dq must have the shape of q")
     _expect_index(eid_c, number_slot)
     n_used = used_types.numel()
-    plan = plan_cache.get(col, indptr_c, eid_c, number_slot, q.size(0), max(n_used, 1))
+    plan = plan_cache.get(col, indptr_c, eid_c, number_slot, q.size(0), max(n_used, 1), prefer_device=True)       # (as in rel_bias_forward)
     dtable = torch.empty_like(table)
     ref = ctypes.byref(_by_pair(plan.struct)) if by_pair else plan.ref
     with _on_device_of(q):
