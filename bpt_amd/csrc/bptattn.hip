@@ -1929,7 +1929,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 // time (126 against 85 us at L = 4096, k = 32); letting the source side recompute p and ds (two more products there,
 // delta (n, H) handed over) measured slower than either on every graph tried.
 template <typename T, int H, int D, int HW, bool PIPE, bool DROP, int BIAS>
-__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : DROP || BIAS == 1 ? 3 : 4))) void k_attn_bwd_dst_tile(
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : DROP && BIAS ? 3 : 4))) void k_attn_bwd_dst_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
     const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds, float *__restrict__ ws_dq,
     float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv, const float *__restrict__ bias,
@@ -1969,7 +1969,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     struct Blk {
         float kr[16], va[16];
         float4 kc[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 g + r
-        int pos[4], mk[4];
+        int pos[4], has;                                           // bit r of has: the pair (entry 4 g + r, member c) exists
         int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
@@ -1983,15 +1983,15 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
-            B.pos[0] = tile_pair_number(f4.x, B.mk[0], c); B.pos[1] = tile_pair_number(f4.y, B.mk[1], c);
-            B.pos[2] = tile_pair_number(f4.z, B.mk[2], c); B.pos[3] = tile_pair_number(f4.w, B.mk[3], c);
-            const size_t arow = (size_t)((uint32_t)ea.x * (uint32_t)(C * sizeof(T))) + t.offa;
+            B.has = ((e01.y >> c) & 1) | (((e01.w >> c) & 1) << 1) | (((e23.y >> c) & 1) << 2) | (((e23.w >> c) & 1) << 3);
+            B.pos[0] = tile_pair_number(f4.x, e01.y, c); B.pos[1] = tile_pair_number(f4.y, e01.w, c);
+            B.pos[2] = tile_pair_number(f4.z, e23.y, c); B.pos[3] = tile_pair_number(f4.w, e23.w, c);
+            const uint32_t arow = (uint32_t)ea.x * (uint32_t)(C * sizeof(T)) + t.offa;
             tile_load16(kb + arow, B.kr);
             tile_load16(vb + arow, B.va);
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                B.kc[r] = *reinterpret_cast<const float4 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
+                B.kc[r] = *reinterpret_cast<const float4 *>(kb + ((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T)) + t.offv));
             if constexpr (BIAS) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])];
@@ -2009,7 +2009,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             float ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const bool has = (B.mk[r] >> c) & 1;
+                const bool has = (B.has >> r) & 1;
                 float pe = has ? __builtin_amdgcn_exp2f((BIAS ? fmaf(B.bz[BIAS ? r : 0], scale_log2e, st[r]) : st[r]) - lse_c) : 0.f;
                 float mt = 1.f;                                   // dropout multiplier of this pair (as in the forward)
                 if constexpr (DROP)
