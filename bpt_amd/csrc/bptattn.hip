@@ -1843,7 +1843,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     struct Blk {
         float kr[16];
         float4 vr[4];
-        int mk[4];
+        int has;                                                  // bit r: the pair (entry 4 g + r, member c) exists
         int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
@@ -1856,11 +1856,12 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
-            tile_load16(kb + (size_t)((uint32_t)ea.x * (uint32_t)(C * sizeof(T))) + t.offa, B.kr);
+            const int mk[4] = {e01.y, e01.w, e23.y, e23.w};
+            B.has = ((mk[0] >> c) & 1) | (((mk[1] >> c) & 1) << 1) | (((mk[2] >> c) & 1) << 2) | (((mk[3] >> c) & 1) << 3);
+            tile_load16(kb + ((uint32_t)ea.x * (uint32_t)(C * sizeof(T)) + t.offa), B.kr);
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                B.vr[r] = *reinterpret_cast<const float4 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv);
+                B.vr[r] = *reinterpret_cast<const float4 *>(vb + ((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T)) + t.offv));
             if constexpr (BIAS == 1) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 1>(P, t.head, B.xe[BIAS == 1 ? r : 0], 0)];
@@ -1869,14 +1870,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
                 const int fv[4] = {f4.x, f4.y, f4.z, f4.w};
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 2>(P, t.head, 0, tile_pair_number(fv[r], B.mk[r], c))];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 2>(P, t.head, 0, tile_pair_number(fv[r], mk[r], c))];
             }
         };
         auto compute = [&](const Blk &B) {
             const floatx4v st = tile_dot(B.kr, qb);
             float sc[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sc[r] = ((B.mk[r] >> c) & 1) ? (BIAS ? fmaf(B.bz[BIAS ? r : 0], scale_log2e, st[r]) : st[r]) : -INFINITY;
+            for (int r = 0; r < 4; ++r) sc[r] = ((B.has >> r) & 1) ? (BIAS ? fmaf(B.bz[BIAS ? r : 0], scale_log2e, st[r]) : st[r]) : -INFINITY;
             const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
             if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
                 float gm = fmaxf(mb, __shfl_xor(mb, 16));
@@ -2050,7 +2051,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     struct Blk {
         float4 qr[4], dr[4];
         float2 w[4];
-        int mk[4];
+        int has;                                                  // bit r: the pair (entry 4 g + r, member c) exists
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
@@ -2059,10 +2060,10 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+            B.has = ((e01.y >> c) & 1) | (((e01.w >> c) & 1) << 1) | (((e23.y >> c) & 1) << 2) | (((e23.w >> c) & 1) << 3);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const size_t off = (size_t)((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T))) + t.offv;
+                const uint32_t off = (uint32_t)idxv[r] * (uint32_t)(C * sizeof(T)) + t.offv;
                 B.qr[r] = *reinterpret_cast<const float4 *>(qb + off);
                 B.dr[r] = *reinterpret_cast<const float4 *>(db + off);
                 // (positions past the group's end are read at its last entry: their masks are empty)
@@ -2074,7 +2075,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             float pe[4], ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const bool has = (B.mk[r] >> c) & 1;              // the scratch of pairs that do not exist is not initialised
+                const bool has = (B.has >> r) & 1;              // the scratch of pairs that do not exist is not initialised
                 pe[r] = has ? B.w[r].x : 0.f;
                 ds[r] = has ? B.w[r].y : 0.f;
             }
