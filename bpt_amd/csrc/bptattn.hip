@@ -2171,7 +2171,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     struct Blk {
         Bf8 kr[2];
         uint2 vr[4];
-        int mk[4];
+        int has;                                                  // bit r: the pair (entry 4 g + r, member c) exists
         int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
@@ -2184,10 +2184,11 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
-            tile_load_row_bf16(kb + (size_t)((uint32_t)ea.x * (uint32_t)RB) + offr, B.kr);
+            const int mk[4] = {e01.y, e01.w, e23.y, e23.w};
+            B.has = ((mk[0] >> c) & 1) | (((mk[1] >> c) & 1) << 1) | (((mk[2] >> c) & 1) << 2) | (((mk[3] >> c) & 1) << 3);
+            tile_load_row_bf16(kb + ((uint32_t)ea.x * (uint32_t)RB + offr), B.kr);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) B.vr[r] = *reinterpret_cast<const uint2 *>(vb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
+            for (int r = 0; r < 4; ++r) B.vr[r] = *reinterpret_cast<const uint2 *>(vb + ((uint32_t)idxv[r] * (uint32_t)RB + offc));
             if constexpr (BIAS == 1) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 1>(P, t.head, B.xe[BIAS == 1 ? r : 0], 0)];
@@ -2196,14 +2197,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
                 const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
                 const int fv[4] = {f4.x, f4.y, f4.z, f4.w};
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 2>(P, t.head, 0, tile_pair_number(fv[r], B.mk[r], c))];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 2>(P, t.head, 0, tile_pair_number(fv[r], mk[r], c))];
             }
         };
         auto compute = [&](const Blk &B) {
             const floatx4v st = tile_dot_bf16(B.kr, qb);
             float sc[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sc[r] = ((B.mk[r] >> c) & 1) ? (BIAS ? st[r] + B.bz[BIAS ? r : 0] : st[r]) * scale_log2e : -INFINITY;
+            for (int r = 0; r < 4; ++r) sc[r] = ((B.has >> r) & 1) ? (BIAS ? st[r] + B.bz[BIAS ? r : 0] : st[r]) * scale_log2e : -INFINITY;
             const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
             if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
                 float gm = fmaxf(mb, __shfl_xor(mb, 16));
@@ -2293,7 +2294,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     struct Blk {
         Bf8 kr[2], va[2];
         uint2 kc[4];
-        int mk[4], pos[4];
+        int has, pos[4];                                           // bit r of has: the pair (entry 4 g + r, member c) exists
         int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
@@ -2307,14 +2308,14 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
-            B.pos[0] = tile_pair_number(f4.x, B.mk[0], c); B.pos[1] = tile_pair_number(f4.y, B.mk[1], c);
-            B.pos[2] = tile_pair_number(f4.z, B.mk[2], c); B.pos[3] = tile_pair_number(f4.w, B.mk[3], c);
-            const size_t arow = (size_t)((uint32_t)ea.x * (uint32_t)RB) + offr;
+            B.has = ((e01.y >> c) & 1) | (((e01.w >> c) & 1) << 1) | (((e23.y >> c) & 1) << 2) | (((e23.w >> c) & 1) << 3);
+            B.pos[0] = tile_pair_number(f4.x, e01.y, c); B.pos[1] = tile_pair_number(f4.y, e01.w, c);
+            B.pos[2] = tile_pair_number(f4.z, e23.y, c); B.pos[3] = tile_pair_number(f4.w, e23.w, c);
+            const uint32_t arow = (uint32_t)ea.x * (uint32_t)RB + offr;
             tile_load_row_bf16(kb + arow, B.kr);
             tile_load_row_bf16(vb + arow, B.va);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) B.kc[r] = *reinterpret_cast<const uint2 *>(kb + (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc);
+            for (int r = 0; r < 4; ++r) B.kc[r] = *reinterpret_cast<const uint2 *>(kb + ((uint32_t)idxv[r] * (uint32_t)RB + offc));
             if constexpr (BIAS) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])];
@@ -2325,7 +2326,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             float ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const bool has = (B.mk[r] >> c) & 1;
+                const bool has = (B.has >> r) & 1;
                 float pe = has ? __builtin_amdgcn_exp2f((BIAS ? st[r] + B.bz[BIAS ? r : 0] : st[r]) * scale_log2e - lse_c) : 0.f;
                 float mt = 1.f;                                   // dropout multiplier of this pair (as in the forward)
                 if constexpr (DROP)
@@ -2367,7 +2368,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
     struct Blk {
         uint2 qr[4], dr[4];
         uint32_t w[4];
-        int mk[4];
+        int has;                                                  // bit r: the pair (entry 4 g + r, member c) exists
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
@@ -2376,10 +2377,10 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            B.mk[0] = e01.y; B.mk[1] = e01.w; B.mk[2] = e23.y; B.mk[3] = e23.w;
+            B.has = ((e01.y >> c) & 1) | (((e01.w >> c) & 1) << 1) | (((e23.y >> c) & 1) << 2) | (((e23.w >> c) & 1) << 3);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const size_t off = (size_t)((uint32_t)idxv[r] * (uint32_t)RB) + offc;
+                const uint32_t off = (uint32_t)idxv[r] * (uint32_t)RB + offc;
                 B.qr[r] = *reinterpret_cast<const uint2 *>(qb + off);
                 B.dr[r] = *reinterpret_cast<const uint2 *>(db + off);
                 // (positions past the group's end are read at its last entry: their masks are empty)
@@ -2390,7 +2391,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
         auto compute = [&](const Blk &B) {
             uint32_t w[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) w[r] = ((B.mk[r] >> c) & 1) ? B.w[r] : 0u;     // the scratch of pairs that do not exist is not initialised
+            for (int r = 0; r < 4; ++r) w[r] = ((B.has >> r) & 1) ? B.w[r] : 0u;     // the scratch of pairs that do not exist is not initialised
             Bf4 pa, da;
             pa.u[0] = pack_lo16(w[0], w[1]); pa.u[1] = pack_lo16(w[2], w[3]);
             da.u[0] = pack_hi16(w[0], w[1]); da.u[1] = pack_hi16(w[2], w[3]);
