@@ -90,6 +90,105 @@ def cpu_baseline(src, dst, N, H, D, seed, budget_s=25.0):
             "sample": f"{len(times)} timed fwd+bwd passes of the full workload after 1 warm-up (median {med * 1e3:.1f} ms), fp32"}
 
 
+def timed(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t) / steps
+
+
+def median(xs):
+    return sorted(xs)[len(xs) // 2]
+
+
+def graph_replay_runs(step, ref, steps, warmup, runs=3):
+    """Three timed runs of the replay of a HIP graph of `step`, or [] where capture fails or a replay does not
+    reproduce the eager results `ref` bit for bit."""
+    import torch
+    try:
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            gout = step()
+        g.replay(); torch.cuda.synchronize()
+        g.replay(); torch.cuda.synchronize()
+        if ref is not None and not all(torch.equal(a, b) for a, b in zip(gout, ref)):
+            log("HIP graph replay did not reproduce the eager result; using eager timing")
+            return []
+        out = [timed(g.replay, steps, warmup if i == 0 else 2) for i in range(runs)]
+        if ref is not None and not all(torch.equal(a, b) for a, b in zip(gout, ref)):
+            log("HIP graph replay did not reproduce the eager result; using eager timing")
+            return []
+        return out
+    except Exception as exc:          # graph capture is an optimisation of the launch path only
+        log("HIP graph capture unavailable:", exc)
+        return []
+
+
+def device_inputs(workload, dtype_name, dev, seed=2345):
+    """Graph arguments and node tensors of a workload on the device: (desc, N, E, H, D, gargs, (q, k, v, do), host parts)."""
+    import torch
+    from bpt_amd import graphbuilder as gb
+    desc, graphs, H, D, default_dtype = make_workload(workload)
+    dtype_name = dtype_name or default_dtype
+    tdtype = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
+    t0 = time.perf_counter()
+    src, dst, etype, _, N = gb.merge_graphs(graphs)
+    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, N)
+    t_graph = time.perf_counter() - t0
+    gargs = tuple(x.to(dev) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
+    gen = torch.Generator().manual_seed(seed)
+    qkvd = tuple((torch.randn(N, H, D, generator=gen) / 8).to(tdtype).to(dev) for _ in range(4))
+    host = dict(src=src, dst=dst, etype=etype, out_csr=out_csr, in_csr=in_csr, ROW=ROW, IR=IR, COL=COL, IC=IC, t_graph=t_graph, gen=gen)
+    return desc, dtype_name, N, len(src), H, D, gargs, qkvd, host
+
+
+def measure_side_workload(name, dtype_name, dev, steps, no_graph, label=None):
+    """ms per fused fwd+bwd step of another BASELINE configuration (median and shortest of three runs of `steps` steps,
+    eager launches or HIP-graph replay, whichever median is lower), with its edges/s and share of the HBM roofline."""
+    import torch
+    from bpt_amd import graphop
+    from bpt_amd import plan as plan_mod
+    desc, dtype_name, N, E, H, D, gargs, (q, k, v, do), host = device_inputs(name, dtype_name, dev)
+    scale = None
+
+    def step():
+        o, lse = graphop.attention_forward(*gargs[4:], q, k, v)
+        dq, dk, dv = graphop.attention_backward(*gargs, q, k, v, o, lse, do)
+        return o, dq, dk, dv
+
+    ref = step()
+    torch.cuda.synchronize()
+    runs = [timed(step, steps, 10 if i == 0 else 2) for i in range(3)]
+    t, tmin, mode = median(runs), min(runs), "eager"
+    if not no_graph:
+        gr = graph_replay_runs(step, ref, steps, 10)
+        if gr and median(gr) < t:
+            t, tmin, mode = median(gr), min(gr), "hipgraph-replay"
+    esize = {"f32": 4, "bf16": 2}[dtype_name]
+    alg = algorithmic_bytes(N, E, H, D, esize)["total"]
+    flops = 2.0 * 12 * E * H * D                     # 12 E C multiply-adds per step
+    res = {"workload": desc, "dtype": dtype_name, "n_nodes": N, "n_edges": E, "ms_per_step": round(t * 1e3, 5), "ms_per_step_min": round(tmin * 1e3, 5),
+           "launch": mode, "edges_per_s": round(E / t, 1), "algorithmic_bytes": alg,
+           "step_frac_of_hbm_peak": round(alg / t / 1e9 / HBM_PEAK_GBS, 4),
+           "useful_tflops": round(flops / t / 1e12, 2), "matrix_peak_tflops": {"f32": 157.3, "bf16": 2500.0}[dtype_name]}
+    del q, k, v, do, gargs, ref
+    plan_mod.plan_cache.clear()
+    graphop.release_workspaces()
+    torch.cuda.empty_cache()
+    log(f"workload {label or name}: {res}")
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -113,6 +212,9 @@ def main():
                          "or by graph size and density (the library's default)")
     ap.add_argument("--tile-backward", default="auto", choices=["auto", "on", "off"],
                     help="fused backward on the dense tiles of 16 rows (on), on the row groups (off), or the library's choice by dtype and graph")
+    ap.add_argument("--side-workloads", default="auto", choices=["auto", "all", "none"],
+                    help="also time the other BASELINE configurations (cfg1, cfg2, cfg3 bf16, cfg4 k=1 / k=32 / window 128, cfg5 bf16), "
+                         "50 steps x 3 runs each, reported as `workloads`; auto: with the default headline line only")
     ap.add_argument("--block-layers", type=int, default=None,
                     help="also time fwd+bwd of a stack of this many transformer blocks (d_model = heads*d_head, d_ff = 4x) on the "
                          "workload's graph, a few steps, reported as block_stack; default: 12 for the headline workload, else 0")
@@ -135,20 +237,12 @@ def main():
     graphop.set_group_rows(args.group_rows)
     from bpt_amd import plan as plan_mod
     plan_mod.set_device_build({"auto": None, "host": False, "device": True}[args.plan])
-    desc, graphs, H, D, default_dtype = make_workload(args.workload)
-    dtype_name = args.dtype or default_dtype
+    desc, dtype_name, N, E, H, D, gargs, (q, k, v, do), host = device_inputs(args.workload, args.dtype, dev)
     tdtype = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
     esize = {"f32": 4, "bf16": 2}[dtype_name]
-
-    t0 = time.perf_counter()
-    src, dst, etype, _, N = gb.merge_graphs(graphs)
-    E = len(src)
-    out_csr, in_csr, ROW, IR, COL, IC = gb.get_csrs(src, dst, N)
-    t_graph = time.perf_counter() - t0
-    gargs = tuple(x.to(dev) for x in (ROW, IR, out_csr[2], out_csr[1], COL, IC, in_csr[2], in_csr[1]))
-    gen = torch.Generator().manual_seed(2345)
-    q, k, v, do = ((torch.randn(N, H, D, generator=gen) / 8).to(tdtype).to(dev) for _ in range(4))
-    log(f"{desc}: N={N} E={E} dtype={dtype_name}; host graph+CSR build {t_graph * 1e3:.1f} ms")
+    src, dst, etype, out_csr, in_csr, gen = host["src"], host["dst"], host["etype"], host["out_csr"], host["in_csr"], host["gen"]
+    ROW, IR, COL, IC = host["ROW"], host["IR"], host["COL"], host["IC"]
+    log(f"{desc}: N={N} E={E} dtype={dtype_name}; host graph+CSR build {host['t_graph'] * 1e3:.1f} ms")
 
     if args.rel_pos and not args.unfused:
         # rel_pos inside the fused kernels: per-edge score term from the (1000, d) table, table gradient by SpMMs
@@ -212,47 +306,19 @@ def main():
         ref = step()
         torch.cuda.synchronize()
 
-    def timed(fn, steps, warmup):
-        for _ in range(warmup):
-            fn()
-        torch.cuda.synchronize()
-        t = time.perf_counter()
-        for _ in range(steps):
-            fn()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t) / steps
-
-    # The timed region is exactly --steps steps between two synchronisations.  It is run three times and the shortest
-    # run is reported (all three are in the JSON line): the host of a shared box stalls now and then for tens of
-    # milliseconds (measured: single calls of 40 ms inside loops whose other calls take 0.05 ms), which a loop of 40 ms
-    # cannot absorb.
+    # The timed region is exactly --steps steps between two synchronisations.  It is run three times; the MEDIAN run is
+    # the reported ms_per_step and the shortest one is kept beside it (all three are in the JSON line): the host of a
+    # shared box stalls now and then for tens of milliseconds, which shows as one slow run of the three.
     runs_eager = [timed(step, args.steps, args.warmup if i == 0 else 2) for i in range(3)]
-    t_eager = min(runs_eager)
-    t_step, mode = t_eager, "eager"
+    t_eager, t_eager_min = median(runs_eager), min(runs_eager)
+    t_step, t_step_min, mode = t_eager, t_eager_min, "eager"
     t_graph_replay, runs_graph = None, []
     if not args.no_graph:
-        try:
-            side = torch.cuda.Stream()
-            with torch.cuda.stream(side):
-                for _ in range(3):
-                    step()
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                gout = step()
-            g.replay(); torch.cuda.synchronize()
-            g.replay(); torch.cuda.synchronize()
-            same = all(torch.equal(a, b) for a, b in zip(gout, ref))
-            if same:
-                runs_graph = [timed(g.replay, args.steps, args.warmup if i == 0 else 2) for i in range(3)]
-                t_graph_replay = min(runs_graph)
-                same = all(torch.equal(a, b) for a, b in zip(gout, ref))
-            if same and t_graph_replay < t_step:
-                t_step, mode = t_graph_replay, "hipgraph-replay"
-            elif not same:
-                log("HIP graph replay did not reproduce the eager result; using eager timing")
-        except Exception as exc:          # graph capture is an optimisation of the launch path only
-            log("HIP graph capture unavailable:", exc)
+        runs_graph = graph_replay_runs(step, ref, args.steps, args.warmup)
+        if runs_graph:
+            t_graph_replay = median(runs_graph)
+            if t_graph_replay < t_step:
+                t_step, t_step_min, mode = t_graph_replay, min(runs_graph), "hipgraph-replay"
 
     # ---- per-kernel durations, HIP events recorded by the library around the kernel on its launch stream
     lib = attn_lib()
@@ -281,6 +347,8 @@ def main():
             traffic = json.load(open(tpath)).get(f"{args.workload}-{dtype_name}", {}).get(dom)
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                    "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, scaled by the "
+                                      "256 MiB copies of the same run (profiles/attn_fused_cfg3_f32_hbm_traffic.txt); not measured in this run",
                     "algorithmic_bytes": alg[dom], "avg_launch_ms": round(kernels[dom], 5)}
 
     # what this GPU's memory system delivers to a plain streaming kernel: device-to-device copies of 256 MiB (read +
@@ -339,7 +407,7 @@ def main():
             x.backward(gh)
             return x
 
-        t_stack = min(timed(stack_step, 5, 2) for _ in range(3))
+        t_stack = median([timed(stack_step, 5, 2) for _ in range(3)])
         block = {"layers": args.block_layers, "d_model": dm, "d_ff": 4 * dm, "ms_per_layer_fwd_bwd": round(t_stack / args.block_layers * 1e3, 4),
                  "attention_ms_per_layer": round(t_step * 1e3, 4), "attention_share": round(t_step * args.block_layers / t_stack, 3)}
         log(f"block stack: {block}")
@@ -366,21 +434,12 @@ def main():
 
         def best_of_eager_and_replay(fn):
             # as for the headline step: eager launches (through autograd here, about 0.2 ms of host work per step) or the
-            # replay of a HIP graph of the same step, whichever is faster
-            t = min(timed(fn, 200, 20) for _ in range(3))
+            # replay of a HIP graph of the same step, whichever median of three runs is lower
+            t = median([timed(fn, 100, 10) for _ in range(3)])
             if not args.no_graph:
-                try:
-                    side = torch.cuda.Stream()
-                    with torch.cuda.stream(side):
-                        for _ in range(3):
-                            fn()
-                    torch.cuda.synchronize()
-                    gv = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(gv):
-                        fn()
-                    t = min([t] + [timed(gv.replay, 200, 20) for _ in range(3)])
-                except Exception as exc:
-                    log("HIP graph capture unavailable for a variant:", exc)
+                gr = graph_replay_runs(fn, None, 100, 10)
+                if gr:
+                    t = min(t, median(gr))
             return t
 
         variants = {name: round(best_of_eager_and_replay(variant_step(**kw)) * 1e3, 4)
@@ -392,11 +451,24 @@ def main():
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(src, dst, N, H, D, 2345)
 
+    # the other BASELINE configurations, a short run each (the default line only: --side-workloads none switches them off)
+    side = None
+    if args.side_workloads == "all" or (args.side_workloads == "auto" and args.block_layers > 0 and args.workload == "cfg3"
+                                        and dtype_name == "f32" and not args.unfused and not args.rel_pos and args.dropout == 0):
+        del q, k, v, do
+        plan_mod.plan_cache.clear()
+        graphop.release_workspaces()
+        torch.cuda.empty_cache()
+        side = {}
+        for label, wl, dt in (("cfg1", "cfg1", "f32"), ("cfg2", "cfg2", "f32"), ("cfg3-bf16", "cfg3", "bf16"), ("cfg4-k1", "cfg4-k1", "f32"),
+                              ("cfg4-k32", "cfg4-k32", "f32"), ("cfg4-w128", "cfg4-w128", "f32"), ("cfg5-bf16", "cfg5", "bf16")):
+            side[label] = measure_side_workload(wl, dt, dev, 50, args.no_graph, label)
+
     step_gbs = alg["total"] / t_step / 1e9
     out = {
         "metric": "attention edges/s fwd+bwd at n=8192 k=4 8h\u00d764; % of HBM roofline",
         "value": E / t_step, "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": t_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": t_step * 1e3, "ms_per_step_min": t_step_min * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype_name, "data": "synthetic",
         "config": {"workload": desc + (" (op chain with rel_pos)" if args.rel_pos and args.unfused else " (fused fwd+bwd with rel_pos)" if args.rel_pos else " (unfused op chain)" if args.unfused else
                                        f" (fused fwd+bwd, attention dropout {args.dropout})" if args.dropout > 0 else " (fused fwd+bwd)"), "n_nodes": N,
@@ -411,7 +483,7 @@ def main():
         "ms_per_step_eager": t_eager * 1e3,
         "ms_per_step_graph": None if t_graph_replay is None else t_graph_replay * 1e3,
         "timed_runs_ms_per_step": {"eager": [round(t * 1e3, 5) for t in runs_eager], "graph": [round(t * 1e3, 5) for t in runs_graph],
-                                   "reported": "shortest of three runs of --steps steps each"},
+                                   "reported": "ms_per_step = median of three runs of --steps steps each (of the faster launch mode); ms_per_step_min = the shortest"},
         "kernel_ms": {k_: round(v_, 5) for k_, v_ in kernels.items()},
     }
     if plan_build is not None:
@@ -421,6 +493,8 @@ def main():
         out["block_stack"] = block
     if variants is not None:
         out["variants"] = variants
+    if side is not None:
+        out["workloads"] = side
     log(json.dumps(out, indent=1))
     print(json.dumps(out), flush=True)
 

@@ -18,7 +18,8 @@ class PlanStruct(ctypes.Structure):
                 ("n_rows", c_i64), ("n_edges", c_i64), ("n_items", c_i64), ("n_heavy", c_i64), ("n_slots", c_i64),
                 ("grp_members", c_vp), ("grp_ptr", c_vp), ("grp_entries", c_vp), ("grp_pairs", c_vp),
                 ("grp_chunks", c_vp), ("n_groups", c_i64), ("grp_R", c_i64), ("grp_max_chunk", c_i64),
-                ("n_grp_entries", c_i64), ("grp_eids", c_vp), ("bias_by_pair", c_i64)]
+                ("n_grp_entries", c_i64), ("grp_eids", c_vp), ("bias_by_pair", c_i64),
+                ("n_index_nodes", c_i64), ("grp_slot_heavy", c_vp), ("grp_arrive", c_vp)]
 
 
 class PlanInfo(ctypes.Structure):
@@ -46,6 +47,7 @@ _PP = ctypes.POINTER(PlanStruct)
 _tail = [ctypes.c_int, ctypes.c_int, ctypes.c_int, c_vp]          # h, d, dtype, stream
 ATTN_API = {
     "bpt_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "bpt_plan_struct_bytes": (c_i64, []),
     "bpt_set_force_generic": (ctypes.c_int, [ctypes.c_int]),
     "bpt_profile_kernel": (ctypes.c_int, [ctypes.c_int, c_vp, c_vp]),
     "bpt_gather_probe": (ctypes.c_int, [c_vp, c_i64, ctypes.c_int, ctypes.c_int, ctypes.c_int, c_vp, c_vp]),
@@ -62,6 +64,7 @@ ATTN_API = {
     "bpt_rel_bias_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_i64, c_vp] + _tail),
     "bpt_rel_bias_forward_tiles": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp] + _tail),
     "bpt_rel_bias_backward_workspace_bytes": (c_i64, [_PP, c_i64, ctypes.c_int]),
+    "bpt_rel_bias_backward_supported": (ctypes.c_int, [c_i64, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "bpt_rel_bias_backward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_vp, c_vp, c_vp, c_i64] + _tail),
     "bpt_attention_forward": (ctypes.c_int, [_PP, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, ctypes.c_float, ctypes.c_float,
                                             ctypes.c_uint64] + _tail),
@@ -112,7 +115,11 @@ def graph_lib():
 def attn_lib():
     global _attn
     if _attn is None:
-        _attn = _load(ATTN_SO, ATTN_API, "libbptattn (HIP kernels)")
+        lib = _load(ATTN_SO, ATTN_API, "libbptattn (HIP kernels)")
+        if lib.bpt_plan_struct_bytes() != ctypes.sizeof(PlanStruct):
+            raise ImportError(f"libbptattn was built for a bpt_plan of {lib.bpt_plan_struct_bytes()} bytes, this binding passes "
+                              f"{ctypes.sizeof(PlanStruct)}: rebuild with `python -m bpt_amd._build`")
+        _attn = lib
     return _attn
 
 
@@ -128,6 +135,17 @@ def check_graph(status):
         raise ValueError("bptgraph: " + graph_lib().bptg_strerror(status).decode())
 
 
+class BptStatusError(RuntimeError):
+    """A non-zero status of a libbptattn call; `.status` is the code (negative: bpt_status, positive: hipError_t)."""
+
+    def __init__(self, status, what):
+        super().__init__(f"{what}: " + attn_lib().bpt_strerror(status).decode() + f" (status {status})")
+        self.status = int(status)
+
+
+BPT_ERR_UNSUPPORTED = -7
+
+
 def check_attn(status, what):
     if status != 0:
-        raise RuntimeError(f"{what}: " + attn_lib().bpt_strerror(status).decode() + f" (status {status})")
+        raise BptStatusError(status, what)

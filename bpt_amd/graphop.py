@@ -18,7 +18,7 @@ import threading
 
 import torch
 
-from ._lib import PlanStruct, attn_lib, check_attn
+from ._lib import BPT_ERR_UNSUPPORTED, BptStatusError, PlanStruct, attn_lib, check_attn
 from .plan import GROUP_ORDER_SRC, TILE_GROUP_R, plan_cache
 
 __all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forward", "node_mul_edge_backward",
@@ -337,7 +337,7 @@ def vector_spmm_forward(row, indptr, eid, indices, edata, x, *, n_rows=None, out
             st = _LIB.bpt_vector_spmm_accumulate(ref, _ptr(edata), _ptr(x), _ptr(out), _ptr(ws), nws, h, d, dt, _stream())
             if st == 0:
                 return out
-            if st != -7:                      # BPT_ERR_UNSUPPORTED: no row-group kernel for this call
+            if st != BPT_ERR_UNSUPPORTED:     # no row-group kernel for this call
                 check_attn(st, "vector_spmm_accumulate")
         check_attn(_LIB.bpt_vector_spmm_forward(ref, _ptr(edata), _ptr(x), _ptr(y), _ptr(ws), nws, h, d, dt, _stream()),
                    "vector_spmm_forward")
@@ -430,6 +430,16 @@ def rel_rows_supported(q):
     """True if the rel_pos term of q's (h, d, dtype) has the kernels that keep the table rows in use on chip."""
     h, d = _hd(q)
     return q.dim() == 3 and d == 64 and h in (4, 8, 16) and q.dtype in (torch.float32, torch.bfloat16)
+
+
+def rel_bias_backward_supported(q, n_used):
+    """True if rel_bias_backward has a kernel configuration for n_used types in use on q's device (asked before the forward,
+    so that a step never finds out in its backward that the gradient kernel does not fit)."""
+    if not (rel_rows_supported(q) and n_used <= REL_MAX_USED_TYPES):
+        return False
+    h, d = _hd(q)
+    with _on_device_of(q):
+        return _LIB.bpt_rel_bias_backward_supported(int(n_used), h, d, _dtype(q)) == 0
 
 
 def rel_bias_backward(col, indptr_c, eid_c, number_slot, used, used_types, ds, q, table, dq, by_pair=False):

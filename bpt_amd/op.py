@@ -107,7 +107,9 @@ class BPTRelAttention(Function):
                 table, etype):
         aux = _rel_aux(etype, col, indptr_c, eid_c, table.size(0))
         table = table.contiguous()
-        ctx.on_chip = _g.rel_rows_supported(q) and aux["n_used"] <= _g.REL_MAX_USED_TYPES and not _g.force_generic_enabled()
+        # (the gradient kernel's configuration is asked for here: the SpMM form is then chosen for both passes up front)
+        ctx.on_chip = (_g.rel_rows_supported(q) and aux["n_used"] <= _g.REL_MAX_USED_TYPES and not _g.force_generic_enabled()
+                       and _g.rel_bias_backward_supported(q, aux["n_used"]))
         # where forward and backward both run on the tile kernels, the term and its gradient are stored head-major in the
         # order in which the tiles meet the edges (rows_slot: the place of every in-CSR slot) instead of by edge id
         graph = (row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, q, k)
@@ -123,10 +125,10 @@ class BPTRelAttention(Function):
             ctx.rows_slot = held[1]
             try:
                 bias = _g.rel_bias_forward_tiles(*graph, table, aux["used_types"], held[2], dropout_p)
-            except RuntimeError as err:
+            except _g.BptStatusError as err:
                 # (many types in use need more than 64 KB of LDS there, which a runtime may refuse: the kernel over the
                 # in-CSR writes the same layout from within 64 KB)
-                if "(status -7)" not in str(err):
+                if err.status != _g.BPT_ERR_UNSUPPORTED:
                     raise
                 bias = _g.rel_bias_forward(col, indptr_c, ctx.rows_slot, aux["number_slot"], q, table, used_types=aux["used_types"],
                                            by_pair=True)

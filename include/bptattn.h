@@ -89,26 +89,30 @@ typedef struct {
                                     produces `bias` / consumes `ds_out` uses the same places: bpt_rel_bias_forward /
                                     _backward do when THEIR plan has the flag set and carries, as eid, the pair number
                                     of every slot's edge */
+    int64_t n_index_nodes;       /* rows of the node tensor that idx points into (the other side's node count: attention to a
+                                    memory of another length, modules/attention.py:144-168); 0 = the same as n_rows.  The
+                                    row-group and tile kernels address rows of BOTH node tensors with 32-bit byte offsets and
+                                    are taken only when max(n_rows, n_index_nodes) * h * d * sizeof(element) < 4 GiB; a
+                                    caller whose neighbour tensor has more rows than n_rows must say so here */
+    const int32_t *grp_slot_heavy; /* n_slots or NULL: for every partial-row slot the index into `heavy` of the row it belongs to */
+    int32_t *grp_arrive;         /* 2 * 16 * n_heavy int32, ALL ZERO when the plan is handed over, or NULL.  With it (and
+                                    grp_slot_heavy) the tile kernels of bpt_attention_forward / _backward merge the partial
+                                    results of a split row themselves: every wavefront that has stored a segment's partial
+                                    row bumps the row's counter (one per row and head; the first 16 * n_heavy for the
+                                    forward, the rest for the backward), and the one that arrives last adds the segments in
+                                    slot order and sets the counter back to zero, so the separate combine launches go away
+                                    and the buffer is zero again when the call has run.  The sums stay a fixed function of
+                                    the plan (no floating-point atomics).  The counters belong to the plan: two calls that
+                                    use the same plan must not overlap on the GPU (calls on one stream never do); a call
+                                    that fails half way leaves them undefined.  NULL: partial rows are merged by a
+                                    separate launch, as for all other kernels */
 } bpt_plan;
 
+/* sizeof(bpt_plan) as this library was compiled: a binding checks its own mirror of the struct against it before the first call
+ * (a shorter struct would make the library read past the caller's memory). */
+int64_t bpt_plan_struct_bytes(void);
+
 const char *bpt_strerror(int status);
-
-/* 1: force the shape-generic kernels even where a specialised one exists (testing). Returns the old value. */
-int bpt_set_force_generic(int on);
-
-/* Measurement aid (no counterpart in the reference): while `which` is one of BPT_KERNEL_*, every launch
- * of that main kernel of the fused path is bracketed by hipEventRecord(start_event) / (stop_event) on
- * the launch stream, so a benchmark can time one kernel with HIP events; 0 switches it off. */
-enum { BPT_KERNEL_NONE = 0, BPT_KERNEL_ATTN_FWD = 1, BPT_KERNEL_ATTN_BWD_DST = 2, BPT_KERNEL_ATTN_BWD_SRC = 3 };
-int bpt_profile_kernel(int which, void *start_event, void *stop_event);
-
-/* Measurement aid (no counterpart in the reference): launches a kernel in which waves_per_cu wavefronts per compute unit
- * (a multiple of 4, at most 64) each read `iters` batches of in_flight (2, 4 or 8) pseudo-random 1 KB rows of `region`
- * (region_bytes of device memory, 16-byte aligned), the access pattern of the attention kernels' neighbour-row gathers.
- * Timed with events by the caller, 256 * waves_per_cu * iters * in_flight KB / duration is the rate at which this GPU's
- * memory system feeds such gathers: the practical ceiling of these kernels (lower than the streaming bandwidth).
- * sink: one float of device memory (never written in practice). */
-int bpt_gather_probe(const void *region, int64_t region_bytes, int waves_per_cu, int in_flight, int iters, float *sink, void *stream);
 
 /* Bytes of workspace the call needs (0 possible).  op: one of the BPT_OP_* below. */
 enum {
@@ -209,6 +213,11 @@ int bpt_rel_bias_forward_tiles(const bpt_plan *plan, const void *q, const void *
  * Row-owned sums in a fixed order, no atomics.  h in {4, 8, 16}, d = 64, f32 or bf16, n_used <= 240;
  * BPT_ERR_UNSUPPORTED otherwise (compose bpt_vector_spmm_forward calls instead). */
 int64_t bpt_rel_bias_backward_workspace_bytes(const bpt_plan *plan, int64_t n_used, int h);
+/* BPT_OK if bpt_rel_bias_backward has a kernel configuration for n_used types in use that the current device accepts (its
+ * per-type sums live in LDS; many types with many heads need more than the 64 KB a runtime grants without asking), else
+ * BPT_ERR_UNSUPPORTED.  Nothing is launched.  A caller asks BEFORE the forward, so that it can form the term's gradients with
+ * bpt_vector_spmm_forward calls from the start instead of finding out in the backward. */
+int bpt_rel_bias_backward_supported(int64_t n_used, int h, int d, int dtype);
 int bpt_rel_bias_backward(const bpt_plan *plan, const float *ds, const void *q, const void *table, const int32_t *used,
                           const int32_t *used_types, int64_t n_types, int64_t n_used, void *dq, void *dtable, void *workspace,
                           int64_t workspace_bytes, int h, int d, int dtype, void *stream);

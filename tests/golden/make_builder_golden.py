@@ -33,16 +33,28 @@ OUT_DIR = os.path.join(ROOT, "oracle", "_ref")
 
 
 def build_reference_builder():
+    """Compile the reference's builder.pyx into oracle/_ref/ (the built module only).  The generated C++
+    is reference source in another form: it is written to a temporary directory and removed after the
+    compile, so that it neither stays in the tree nor travels anywhere with it."""
+    import shutil
+    import tempfile
     os.makedirs(OUT_DIR, exist_ok=True)
-    cpp = os.path.join(OUT_DIR, "ref_builder.cpp")
+    stale = os.path.join(OUT_DIR, "ref_builder.cpp")
+    if os.path.exists(stale):
+        os.remove(stale)
     # cython names the module after the .pyx file: PyInit_builder
     so = os.path.join(OUT_DIR, "builder" + sysconfig.get_config_var("EXT_SUFFIX"))
-    subprocess.check_call([sys.executable, "-m", "cython", "--cplus", "-2", REF_PYX, "-o", cpp])
-    subprocess.check_call([
-        "g++", "-O2", "-shared", "-fPIC", "-w",
-        "-DNPY_NO_DEPRECATED_API=NPY_1_7_API_VERSION",
-        "-I", sysconfig.get_paths()["include"], "-I", np.get_include(),
-        cpp, "-o", so])
+    tmp = tempfile.mkdtemp(prefix="bpt_ref_builder_")
+    try:
+        cpp = os.path.join(tmp, "ref_builder.cpp")
+        subprocess.check_call([sys.executable, "-m", "cython", "--cplus", "-2", REF_PYX, "-o", cpp])
+        subprocess.check_call([
+            "g++", "-O2", "-shared", "-fPIC", "-w",
+            "-DNPY_NO_DEPRECATED_API=NPY_1_7_API_VERSION",
+            "-I", sysconfig.get_paths()["include"], "-I", np.get_include(),
+            cpp, "-o", so])
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
     spec = importlib.util.spec_from_file_location("builder", so)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)

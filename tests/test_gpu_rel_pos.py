@@ -211,7 +211,7 @@ def test_layer_falls_back_to_the_in_csr_kernel_where_the_tile_form_is_refused(op
     calls = []
     def refused(*a, **kw):
         calls.append(1)
-        raise RuntimeError("rel_bias_forward_tiles: unsupported (status -7)")
+        raise graphop.BptStatusError(graphop.BPT_ERR_UNSUPPORTED, "rel_bias_forward_tiles")
     monkeypatch.setattr(graphop, "rel_bias_forward_tiles", refused)
     got = step()
     assert calls, "the tile form was not asked for: the test does not reach the fallback"

@@ -23,8 +23,10 @@ def _declared(header, prefix):
 
 def test_libraries_export_every_declared_symbol():
     g = _declared("bptgraph.h", "bptg_")
-    a = _declared("bptattn.h", "bpt_")
+    a = sorted(_declared("bptattn.h", "bpt_") + _declared("bptattn_measure.h", "bpt_"))
     assert len(g) >= 8 and len(a) >= 13
+    # the drop-in header carries no process-global hooks: those live in the measurement header
+    assert not {"bpt_profile_kernel", "bpt_gather_probe", "bpt_set_force_generic"} & set(_declared("bptattn.h", "bpt_"))
     glib, alib = _lib.graph_lib(), _lib.attn_lib()
     for name in g:
         assert hasattr(glib, name), name
@@ -37,6 +39,42 @@ def test_libraries_export_every_declared_symbol():
         assert hasattr(plib, name), name
     # the Python bindings cover exactly the declared API
     assert sorted(_lib.GRAPH_API) == g and sorted(_lib.ATTN_API) == a and sorted(_lib.PLAN_API) == p
+
+
+def _header_plan_fields():
+    """(name, is_pointer) of every member of `bpt_plan` as include/bptattn.h declares it, in order."""
+    text = open(os.path.join(ROOT, "include", "bptattn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    body = re.search(r"typedef struct \{(.*?)\} bpt_plan;", text, flags=re.S).group(1)
+    fields = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        m = re.match(r"(const\s+)?(int32_t|int64_t)\s+(.*)", decl, flags=re.S)
+        assert m, decl
+        for name in m.group(3).split(","):
+            name = name.strip()
+            fields.append((name.lstrip("* "), name.startswith("*")))
+    return fields
+
+
+def test_binding_mirrors_the_plan_struct_of_the_header():
+    """The ctypes mirror has the header's members in the header's order, and its size is the library's sizeof(bpt_plan):
+    a binding that is one member short would make the library read past the caller's struct."""
+    fields = _header_plan_fields()
+    mirror = [(n, t is ctypes.c_void_p) for n, t in _lib.PlanStruct._fields_]
+    assert mirror == fields
+    assert all(t in (ctypes.c_void_p, ctypes.c_int64) for _, t in _lib.PlanStruct._fields_)
+    assert _lib.attn_lib().bpt_plan_struct_bytes() == ctypes.sizeof(_lib.PlanStruct) == 8 * len(fields)
+
+
+def test_integration_document_shows_the_whole_plan_struct():
+    """The ctypes stub printed for integrators names every member of bpt_plan."""
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    for name, _ in _header_plan_fields():
+        assert '"' + name + '"' in doc, name
+    assert "bpt_plan_struct_bytes" in doc
 
 
 def test_error_strings_and_argument_errors_without_gpu():
