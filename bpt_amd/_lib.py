@@ -19,7 +19,7 @@ class PlanStruct(ctypes.Structure):
                 ("grp_members", c_vp), ("grp_ptr", c_vp), ("grp_entries", c_vp), ("grp_pairs", c_vp),
                 ("grp_chunks", c_vp), ("n_groups", c_i64), ("grp_R", c_i64), ("grp_max_chunk", c_i64),
                 ("n_grp_entries", c_i64), ("grp_eids", c_vp), ("bias_by_pair", c_i64),
-                ("n_index_nodes", c_i64), ("grp_slot_heavy", c_vp), ("grp_arrive", c_vp)]
+                ("n_index_nodes", c_i64)]
 
 
 class PlanInfo(ctypes.Structure):

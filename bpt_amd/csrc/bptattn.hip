@@ -1770,143 +1770,6 @@ __device__ __forceinline__ void tile_store_rows(const TileCtx &t, const floatx4v
     }
 }
 
-// ---- Split rows merged by the kernel that produced their segments (plans with grp_arrive / grp_slot_heavy).
-// A wavefront that has stored the partial result of a segment (a member with slot >= 0) makes its stores visible to the
-// device, then adds one to the counter of (split row, head).  Whoever brings a counter to the row's number of segments
-// was the last to arrive: every segment of that row and head is in the workspace, and this wavefront merges them in slot
-// order (lane group sg = lane / 16 folds slots sg, sg + 4, ..., four columns per lane; the four lane groups are added in
-// order 0 .. 3), writes the finished row and sets the counter back to zero for the next launch.  The counter is the only
-// atomic: the floating-point sums are a fixed function of the plan.  REGION 0: forward, 1: backward (a plan's forward
-// and backward may then overlap on two streams).
-constexpr int ARRIVE_HEADS = 16;                   // counters per split row (the tile kernels take h <= 16)
-
-template <int REGION>
-__device__ __forceinline__ uint64_t tile_arrive(const bpt_plan &P, const TileCtx &t, int &hi) {
-    const bool split = t.g == 0 && t.member.x >= 0 && t.member.y >= 0;
-    hi = 0;
-    if (__builtin_amdgcn_ballot_w64(split) == 0) return 0;
-    __threadfence();                                              // release: the partial rows before the arrival
-    bool last = false;
-    if (split) {
-        hi = P.grp_slot_heavy[t.member.y];
-        int32_t *ctr = P.grp_arrive + ((size_t)REGION * (size_t)P.n_heavy + (size_t)hi) * ARRIVE_HEADS + t.head;
-        last = atomicAdd(ctr, 1) == P.heavy[3 * hi + 2] - 1;
-        if (last) atomicExch(ctr, 0);                             // nobody else touches it before the next launch
-    }
-    const uint64_t todo = __builtin_amdgcn_ballot_w64(last);
-    if (todo != 0) __threadfence();                               // acquire: the other wavefronts' partial rows
-    return todo;
-}
-
-// o and lse of one split row and head from the (m, l, acc) partials of its segments
-template <typename T, int H, int D>
-__device__ __forceinline__ void tile_finish_softmax(int row, int s0, int ns, int head, int lane, const float *ws_acc, const float *ws_ml,
-                                                    T *__restrict__ o, float *__restrict__ lse) {
-    constexpr int C = H * D;
-    static_assert(D == 64, "sixteen lanes of four columns");
-    const int sg = lane >> 4, cq = lane & 15;
-    const float *ml = ws_ml + ((size_t)s0 * H + head) * 2;       // slot stride 2 * H
-    const float *col = ws_acc + (size_t)s0 * C + head * D + 4 * cq;   // slot stride C
-    float M = M_INIT_LOG2, L = 0.f;
-    float4 A = make_float4(0.f, 0.f, 0.f, 0.f);
-    int kk = sg;
-    for (; kk + 12 < ns; kk += 16) {
-        float tm[4], tl[4];
-        float4 ta[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const size_t sl = (size_t)(kk + 4 * u);
-            tm[u] = ml[sl * 2 * H];
-            tl[u] = ml[sl * 2 * H + 1];
-            ta[u] = *reinterpret_cast<const float4 *>(col + sl * C);
-        }
-        const float mx = fmaxf(fmaxf(M, tm[0]), fmaxf(fmaxf(tm[1], tm[2]), tm[3]));
-        const float resc = __builtin_amdgcn_exp2f(M - mx);
-        L *= resc; A.x *= resc; A.y *= resc; A.z *= resc; A.w *= resc;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const float wgt = __builtin_amdgcn_exp2f(tm[u] - mx);
-            L = fmaf(tl[u], wgt, L);
-            A.x = fmaf(ta[u].x, wgt, A.x); A.y = fmaf(ta[u].y, wgt, A.y); A.z = fmaf(ta[u].z, wgt, A.z); A.w = fmaf(ta[u].w, wgt, A.w);
-        }
-        M = mx;
-    }
-    for (; kk < ns; kk += 4) {
-        const float tm = ml[(size_t)kk * 2 * H], tl = ml[(size_t)kk * 2 * H + 1];
-        const float4 ta = *reinterpret_cast<const float4 *>(col + (size_t)kk * C);
-        const float mx = fmaxf(M, tm), resc = __builtin_amdgcn_exp2f(M - mx), wgt = __builtin_amdgcn_exp2f(tm - mx);
-        L = fmaf(tl, wgt, L * resc);
-        A.x = fmaf(ta.x, wgt, A.x * resc); A.y = fmaf(ta.y, wgt, A.y * resc); A.z = fmaf(ta.z, wgt, A.z * resc); A.w = fmaf(ta.w, wgt, A.w * resc);
-        M = mx;
-    }
-    float Mx = fmaxf(M, __shfl_xor(M, 16));
-    Mx = fmaxf(Mx, __shfl_xor(Mx, 32));
-    const float wl = __builtin_amdgcn_exp2f(M - Mx);
-    L *= wl; A.x *= wl; A.y *= wl; A.z *= wl; A.w *= wl;
-    float Ls = 0.f;
-    float4 As = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {                                 // the four lane groups in order
-        Ls += __shfl(L, cq + 16 * i);
-        As.x += __shfl(A.x, cq + 16 * i); As.y += __shfl(A.y, cq + 16 * i); As.z += __shfl(A.z, cq + 16 * i); As.w += __shfl(A.w, cq + 16 * i);
-    }
-    if (sg == 0) {
-        const float inv = Ls > 0.f ? 1.f / Ls : 0.f;
-        store4<T>(o + (size_t)row * C + head * D + 4 * cq, make_float4(As.x * inv, As.y * inv, As.z * inv, As.w * inv));
-    }
-    if (lane == 0) lse[(size_t)row * H + head] = Ls > 0.f ? Mx + log2f(Ls) : 0.f;
-}
-
-// one output row and head = the sum of its segments' partial rows
-template <typename T, int H, int D>
-__device__ __forceinline__ void tile_finish_sum(int row, int s0, int ns, int head, int lane, const float *ws, T *__restrict__ out) {
-    constexpr int C = H * D;
-    static_assert(D == 64, "sixteen lanes of four columns");
-    const int sg = lane >> 4, cq = lane & 15;
-    const float *col = ws + (size_t)s0 * C + head * D + 4 * cq;
-    float4 S = make_float4(0.f, 0.f, 0.f, 0.f);
-    int kk = sg;
-    for (; kk + 28 < ns; kk += 32) {
-        float4 ta[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) ta[u] = *reinterpret_cast<const float4 *>(col + (size_t)(kk + 4 * u) * C);
-#pragma unroll
-        for (int u = 0; u < 8; ++u) { S.x += ta[u].x; S.y += ta[u].y; S.z += ta[u].z; S.w += ta[u].w; }
-    }
-    for (; kk < ns; kk += 4) {
-        const float4 ta = *reinterpret_cast<const float4 *>(col + (size_t)kk * C);
-        S.x += ta.x; S.y += ta.y; S.z += ta.z; S.w += ta.w;
-    }
-    float4 R = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        R.x += __shfl(S.x, cq + 16 * i); R.y += __shfl(S.y, cq + 16 * i); R.z += __shfl(S.z, cq + 16 * i); R.w += __shfl(S.w, cq + 16 * i);
-    }
-    if (sg == 0) store4<T>(out + (size_t)row * C + head * D + 4 * cq, R);
-}
-
-// What a tile kernel does after storing its members' rows.  KIND 0: forward (ws_a = accumulators, ws_b = (m, l) pairs, out_a = o,
-// lse); KIND 1: one sum (ws_a -> out_a); KIND 2: two sums (ws_a -> out_a, ws_b -> out_b).
-template <typename T, int H, int D, int KIND>
-__device__ __forceinline__ void tile_finish_split(const bpt_plan &P, const TileCtx &t, const float *ws_a, const float *ws_b, T *__restrict__ out_a,
-                                                  T *__restrict__ out_b, float *__restrict__ lse) {
-    if (!P.grp_arrive || !P.grp_slot_heavy) return;               // (the host then launches the combine kernels)
-    int hi;
-    uint64_t todo = tile_arrive<KIND == 0 ? 0 : 1>(P, t, hi);
-    while (todo != 0) {
-        const int m = __builtin_ctzll(todo);
-        todo &= todo - 1;
-        const int row = lane_bcast(t.member.x, m), h3 = 3 * lane_bcast(hi, m);
-        const int s0 = P.heavy[h3 + 1], ns = P.heavy[h3 + 2];
-        if constexpr (KIND == 0) {
-            tile_finish_softmax<T, H, D>(row, s0, ns, t.head, t.lane, ws_a, ws_b, out_a, lse);
-        } else {
-            tile_finish_sum<T, H, D>(row, s0, ns, t.head, t.lane, ws_a, out_a);
-            if constexpr (KIND == 2) tile_finish_sum<T, H, D>(row, s0, ns, t.head, t.lane, ws_b, out_b);
-        }
-    }
-}
-
 // Edge ids of this lane's four pairs of a block, (entry 4 g + r, member c): what the dropout hash and the score term are
 // indexed by (n_edges, the spare row, where the pair does not exist; past the group's end the last entry is read again).
 __device__ __forceinline__ void tile_pair_eids(const bpt_plan &P, int first_entry, int p_end, int c, int (&xe)[4]) {
@@ -2056,7 +1919,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             ws_ml[((size_t)t.member.y * H + t.head) * 2 + 1] = lt;
         }
     }
-    tile_finish_split<T, H, D, 0>(P, t, ws_acc, ws_ml, o, (T *)nullptr, lse);
 }
 
 // Backward on tiles, destination side: per block the scores and dO . v of all 16 x 16 pairs (two products over the
@@ -2167,7 +2029,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         wave_lds_fence();
     }
     tile_store_rows<H, D, false>(t, acc, 1.f, dq, ws_dq);
-    tile_finish_split<T, H, D, 1>(P, t, ws_dq, nullptr, dq, (T *)nullptr, nullptr);
 }
 
 // Backward on tiles, source side (groups of the out-CSR plan: members = source rows, entries = destinations):
@@ -2227,7 +2088,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     }
     tile_store_rows<H, D, false>(t, ak, 1.f, dk, ws_dk);
     tile_store_rows<H, D, false>(t, av, 1.f, dv, ws_dv);
-    tile_finish_split<T, H, D, 2>(P, t, ws_dk, ws_dv, dk, dv, nullptr);
 }
 
 // ---- Dense tiles for bfloat16 rows.  Same walk and the same lane roles as the float32 tile kernels above, on
@@ -2388,7 +2248,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             ws_ml[((size_t)t.member.y * H + t.head) * 2 + 1] = lt;
         }
     }
-    tile_finish_split<bf16_t, H, D, 0>(P, t, ws_acc, ws_ml, o, (bf16_t *)nullptr, lse);
 }
 
 template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, int BIAS>
@@ -2489,7 +2348,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
         wave_lds_fence();
     }
     tile_store_rows<H, D, false>(t, acc, 1.f, dq, ws_dq);
-    tile_finish_split<bf16_t, H, D, 1>(P, t, ws_dq, nullptr, dq, (bf16_t *)nullptr, nullptr);
 }
 
 template <int H, int D, int HW, int WPE, bool PIPE>
@@ -2546,7 +2404,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
     }
     tile_store_rows<H, D, false>(t, ak, 1.f, dk, ws_dk);
     tile_store_rows<H, D, false>(t, av, 1.f, dv, ws_dv);
-    tile_finish_split<bf16_t, H, D, 2>(P, t, ws_dk, ws_dv, dk, dv, nullptr);
 }
 
 // Backward, destination side.  Writes (p, ds) of every pair to pds[(t * H + head)], t = the pair's
@@ -3873,9 +3730,6 @@ inline bool has_tiles(const bpt_plan *P, int h, int d, size_t elem) {
            fits32(std::max(P->n_rows, P->n_index_nodes), (int64_t)h * d * (int64_t)elem);
 }
 
-// the tile kernels merge the partial rows of split nodes themselves when the plan brings the arrival counters
-inline bool merges_split_rows(const bpt_plan *P) { return P->n_heavy == 0 || (P->grp_arrive && P->grp_slot_heavy); }
-
 // Few and tall tiles (fewer wavefronts than three per SIMD, six or more blocks each on average): the kernels then read one
 // block ahead in registers instead of counting on other wavefronts to cover the loads.
 inline bool tall_tiles(const bpt_plan *P, int h) {
@@ -3952,7 +3806,6 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     if (P->n_items == 0) return BPT_OK;
     float *ws_acc = (float *)ws;
     float *ws_ml = ws_acc ? ws_acc + (size_t)P->n_slots * H * D : nullptr;
-    bool merged = false;                                         // split rows merged by the kernel itself (tile kernels, plans with counters)
     {
         ProfScope prof(BPT_KERNEL_ATTN_FWD, s);
         if constexpr (D == 64 && sizeof(T) == 4) {
@@ -3970,7 +3823,6 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
                 default: LAUNCH_FWD_TILE(false, true, 2); break;
                 }
 #undef LAUNCH_FWD_TILE
-                merged = merges_split_rows(P);
                 goto launched;
             }
         }
@@ -3990,7 +3842,6 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
                 default: LAUNCH_FWD_TILE(true, 2); break;
                 }
 #undef LAUNCH_FWD_TILE
-                merged = merges_split_rows(P);
                 goto launched;
             }
         }
@@ -4030,7 +3881,7 @@ int run_attn_fwd(const bpt_plan *P, const void *q, const void *k, const void *v,
     launched:;
     }
     int st = launch_status();
-    if (st != BPT_OK || P->n_heavy == 0 || merged) return st;
+    if (st != BPT_OK || P->n_heavy == 0) return st;
     hipLaunchKernelGGL((k_attn_fwd_combine<T, H, D>), dim3((int)P->n_heavy, H * D / WAVE), dim3(BLOCK), 0, s, P->heavy,
                        (const float *)ws_acc, (const float *)ws_ml, (T *)o, lse);
     return launch_status();
@@ -4079,11 +3930,9 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
                                        (const T *)q, (const T *)d_o, (const float2 *)pds, (T *)dk, (T *)dv, ws_dk, ws_dv);
             }
             st = launch_status();
-            // what is left to merge: the partial rows of the sides whose plan has no arrival counters
-            const int n_a = merges_split_rows(Pin) ? 0 : (int)Pin->n_heavy, n_b = merges_split_rows(Pout) ? 0 : (int)Pout->n_heavy;
-            if (st != BPT_OK || n_a + n_b == 0) return st;
-            hipLaunchKernelGGL((k_combine_sum3<T>), dim3(n_a + n_b, H * D / (4 * WAVE), 2), dim3(BLOCK), 0, s, Pin->heavy,
-                               n_a, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
+            if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;
+            hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / (4 * WAVE), 2), dim3(BLOCK), 0, s, Pin->heavy,
+                               (int)Pin->n_heavy, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
                                (size_t)Pout->n_slots * H * D);
             return launch_status();
         }
@@ -4117,11 +3966,9 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
                                    *Pout, (const bf16_t *)q, (const bf16_t *)d_o, (const uint32_t *)ws, (bf16_t *)dk, (bf16_t *)dv, ws_dk, ws_dv);
             }
             st = launch_status();
-            // what is left to merge: the partial rows of the sides whose plan has no arrival counters
-            const int n_a = merges_split_rows(Pin) ? 0 : (int)Pin->n_heavy, n_b = merges_split_rows(Pout) ? 0 : (int)Pout->n_heavy;
-            if (st != BPT_OK || n_a + n_b == 0) return st;
-            hipLaunchKernelGGL((k_combine_sum3<T>), dim3(n_a + n_b, H * D / (4 * WAVE), 2), dim3(BLOCK), 0, s, Pin->heavy,
-                               n_a, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
+            if (st != BPT_OK || Pin->n_heavy + Pout->n_heavy == 0) return st;
+            hipLaunchKernelGGL((k_combine_sum3<T>), dim3((int)(Pin->n_heavy + Pout->n_heavy), H * D / (4 * WAVE), 2), dim3(BLOCK), 0, s, Pin->heavy,
+                               (int)Pin->n_heavy, (const float *)ws_rows, (T *)dq, Pout->heavy, (const float *)ws_dk, (T *)dk, (T *)dv, H * D,
                                (size_t)Pout->n_slots * H * D);
             return launch_status();
         }

@@ -171,25 +171,6 @@ def pair_numbers_host(grp_mine, grp_theirs, n_edges):
     return out
 
 
-MERGE_IN_KERNEL = True   # plans carry the arrival counters with which the tile kernels merge split rows themselves
-
-
-def _split_row_sync(heavy, n_heavy, n_slots, device):
-    """(slot_heavy, arrive) for a plan whose `heavy` (n_heavy, 3) int32 device tensor lists (row, first slot, slots) of
-    its split rows: for every partial-row slot the index of its row in that list, and the zeroed arrival counters
-    (2 regions x 16 heads per split row) with which the tile kernels find the last wavefront to finish a row."""
-    if not (MERGE_IN_KERNEL and n_heavy > 0 and n_slots > 0):
-        return None, None
-    hv = heavy[:n_heavy].long()
-    counts = hv[:, 2]
-    owner = torch.repeat_interleave(torch.arange(n_heavy, device=device), counts)
-    starts = torch.cumsum(counts, 0) - counts
-    pos = torch.repeat_interleave(hv[:, 1] - starts, counts) + torch.arange(owner.numel(), device=device)
-    slot_heavy = torch.zeros(n_slots, dtype=torch.int32, device=device)
-    slot_heavy[pos] = owner.int()
-    return slot_heavy, torch.zeros(2 * 16 * n_heavy, dtype=torch.int32, device=device)
-
-
 def _tensor_bytes(obj):
     """Bytes of the torch tensors reachable from a plan's containers (dicts, tuples, lists)."""
     if isinstance(obj, torch.Tensor):
@@ -233,12 +214,6 @@ class Plan:
             d["heavy"].data_ptr() if self.n_heavy else None,
             self.n_rows, self.n_edges, self.n_items, self.n_heavy, self.n_slots)
         self.struct.n_index_nodes = self.n_index_nodes
-        if self.device.type == "cuda":
-            slot_heavy, arrive = _split_row_sync(d["heavy"].view(-1, 3), self.n_heavy, self.n_slots, self.device)
-            if arrive is not None:
-                d["slot_heavy"], d["arrive"] = slot_heavy, arrive
-                self.struct.grp_slot_heavy, self.struct.grp_arrive = slot_heavy.data_ptr(), arrive.data_ptr()
-                torch.cuda.current_stream(self.device).synchronize()      # zeroed before any stream can use the plan
 
     @property
     def ref(self):
@@ -429,16 +404,12 @@ class DevicePlan:
         self._max_items = max(self.n_items, 1)
         self._dev = {"rowptr": rowptr, "idx": idx, "eid": eid32, "items": items, "heavy": heavy}
         d = self._dev
-        slot_heavy, arrive = _split_row_sync(heavy.view(-1, 3), self.n_heavy, self.n_slots, self.device)
         torch.cuda.current_stream(self.device).synchronize()      # the plan is complete before any stream can use it
         self.struct = PlanStruct(
             d["rowptr"].data_ptr(), d["idx"].data_ptr() if E else None, d["eid"].data_ptr() if E else None,
             d["items"].data_ptr() if self.n_items else None, d["heavy"].data_ptr() if self.n_heavy else None,
             self.n_rows, E, self.n_items, self.n_heavy, self.n_slots)
         self.struct.n_index_nodes = self.n_index_nodes
-        if arrive is not None:
-            d["slot_heavy"], d["arrive"] = slot_heavy, arrive
-            self.struct.grp_slot_heavy, self.struct.grp_arrive = slot_heavy.data_ptr(), arrive.data_ptr()
 
     def _auto_seg_len(self, row, indptr):
         """auto_seg_len on the device: the 90 % quantile of the non-empty rows' degrees."""

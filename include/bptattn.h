@@ -94,18 +94,6 @@ typedef struct {
                                     row-group and tile kernels address rows of BOTH node tensors with 32-bit byte offsets and
                                     are taken only when max(n_rows, n_index_nodes) * h * d * sizeof(element) < 4 GiB; a
                                     caller whose neighbour tensor has more rows than n_rows must say so here */
-    const int32_t *grp_slot_heavy; /* n_slots or NULL: for every partial-row slot the index into `heavy` of the row it belongs to */
-    int32_t *grp_arrive;         /* 2 * 16 * n_heavy int32, ALL ZERO when the plan is handed over, or NULL.  With it (and
-                                    grp_slot_heavy) the tile kernels of bpt_attention_forward / _backward merge the partial
-                                    results of a split row themselves: every wavefront that has stored a segment's partial
-                                    row bumps the row's counter (one per row and head; the first 16 * n_heavy for the
-                                    forward, the rest for the backward), and the one that arrives last adds the segments in
-                                    slot order and sets the counter back to zero, so the separate combine launches go away
-                                    and the buffer is zero again when the call has run.  The sums stay a fixed function of
-                                    the plan (no floating-point atomics).  The counters belong to the plan: two calls that
-                                    use the same plan must not overlap on the GPU (calls on one stream never do); a call
-                                    that fails half way leaves them undefined.  NULL: partial rows are merged by a
-                                    separate launch, as for all other kernels */
 } bpt_plan;
 
 /* sizeof(bpt_plan) as this library was compiled: a binding checks its own mirror of the struct against it before the first call
