@@ -189,6 +189,46 @@ def measure_side_workload(name, dtype_name, dev, steps, no_graph, label=None):
     return res
 
 
+def measure_narrow_heads(dev, steps, no_graph, h=6, d=50):
+    """The reference's other head shape (6 heads x 50, configs/imdb-4.yml:10-12) on cfg2's batch of 32 graphs, float32, through
+    `op.bpt_attention` and autograd: the fused kernels on zero-padded heads against the unfused op chain on the shape-generic
+    kernels (median of three runs each, eager launches or HIP-graph replay, whichever median is lower)."""
+    import torch
+    from bpt_amd import graphop, op
+    from bpt_amd import plan as plan_mod
+    desc, _, N, E, _, _, gargs, _, host = device_inputs("cfg2", "f32", dev)
+    gen = torch.Generator().manual_seed(2345)
+    q, k, v, do = ((torch.randn(N, h, d, generator=gen) / math.sqrt(d)).to(dev) for _ in range(4))
+
+    def make(fused):
+        def step():
+            qq, kk, vv = (x.detach().requires_grad_(True) for x in (q, k, v))
+            o = op.bpt_attention(*gargs, qq, kk, vv, fused=fused)
+            o.backward(do)
+            return o, qq.grad, kk.grad, vv.grad
+        return step
+
+    res = {"workload": desc.replace("8x64", f"{h}x{d}") + " (op.bpt_attention fwd+bwd through autograd)", "dtype": "f32", "n_nodes": N, "n_edges": E}
+    for name, fused in (("fused_padded", None), ("op_chain", False)):
+        step = make(fused)
+        ref = step()
+        torch.cuda.synchronize()
+        t = median([timed(step, steps, 5 if i == 0 else 2) for i in range(3)])
+        if not no_graph:
+            gr = graph_replay_runs(step, None, steps, 5)
+            if gr:
+                t = min(t, median(gr))
+        res[name + "_ms_per_step"] = round(t * 1e3, 5)
+    res["edges_per_s"] = round(E / (res["fused_padded_ms_per_step"] * 1e-3), 1)
+    res["fused_over_chain"] = round(res["op_chain_ms_per_step"] / res["fused_padded_ms_per_step"], 2)
+    del q, k, v, do, gargs
+    plan_mod.plan_cache.clear()
+    graphop.release_workspaces()
+    torch.cuda.empty_cache()
+    log(f"workload tc32-{h}x{d}: {res}")
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -463,6 +503,7 @@ def main():
         for label, wl, dt in (("cfg1", "cfg1", "f32"), ("cfg2", "cfg2", "f32"), ("cfg3-bf16", "cfg3", "bf16"), ("cfg4-k1", "cfg4-k1", "f32"),
                               ("cfg4-k32", "cfg4-k32", "f32"), ("cfg4-w128", "cfg4-w128", "f32"), ("cfg5-bf16", "cfg5", "bf16")):
             side[label] = measure_side_workload(wl, dt, dev, 50, args.no_graph, label)
+        side["tc32-6x50"] = measure_narrow_heads(dev, 30, args.no_graph)
 
     step_gbs = alg["total"] / t_step / 1e9
     out = {

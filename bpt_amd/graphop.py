@@ -378,6 +378,19 @@ def attention_supported(q):
     return q.dim() == 3 and (h, d) in fast.get(q.dtype, ())
 
 
+def attention_padded_shape(q):
+    """(h', 64) if the fused kernels can run q's (h, d, dtype) after zero-padding every head to 64 columns and the heads to the next
+    compiled count (the reference's kernels take any d, graphop_kernel.cu:269-304; its configs use 6 x 50 and 8 x 40 beside 8 x 64),
+    else None.  Zero columns add nothing to q.k, and a zero head (q = k = v = 0) gives a zero output row and zero gradients."""
+    if q.dim() != 3 or q.dtype not in (torch.float32, torch.bfloat16) or attention_supported(q):
+        return None
+    h, d = _hd(q)
+    if d > 64:
+        return None
+    heads = sorted(hh for hh, dd in {torch.float32: {(4, 64), (8, 64), (16, 64)}, torch.bfloat16: {(8, 64), (16, 64)}}[q.dtype] if hh >= h)
+    return (heads[0], 64) if heads else None
+
+
 def _by_pair(plan_struct):
     """A copy of a `bpt_plan` with bias_by_pair set: the per-edge term it reads or writes is (h, E), head-major."""
     st = PlanStruct.from_buffer_copy(plan_struct)

@@ -298,10 +298,26 @@ def bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices
     scale = 1.0 / math.sqrt(q.size(-1)) if scale is None else float(scale)
     if (rel_table is None) != (etype is None):
         raise ValueError("rel_table and etype go together")
+    padded = None
     if fused is None:
         fused = _g.attention_supported(q)
+        if not fused and not _g.force_generic_enabled():
+            padded = _g.attention_padded_shape(q)
+            fused = padded is not None
         if (dropout_p > 0 or rel_table is not None) and not _g.row_groups_enabled():
             fused = False                       # only the row-group kernels implement dropout and the rel_pos term
+    elif fused and not _g.attention_supported(q):
+        padded = _g.attention_padded_shape(q)
+    if fused and padded is not None:
+        # heads of fewer than 64 columns (6 x 50, 8 x 40 in the reference's configs): the fused kernels run on zero-padded copies
+        # (h', 64) with the scale of the real d; the pads and the slices are ordinary differentiable torch ops
+        h, d = q.size(1), q.size(2)
+        hp, dp = padded
+        grow = lambda x: torch.nn.functional.pad(x, (0, dp - d, 0, hp - h))
+        o = bpt_attention(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, indices_c, grow(q), grow(k), grow(v), scale=scale,
+                          fused=True, dropout_p=dropout_p, seed=seed,
+                          rel_table=None if rel_table is None else torch.nn.functional.pad(rel_table, (0, dp - d)), etype=etype)
+        return o[:, :h, :d].contiguous()
     if fused:
         if dropout_p > 0 and seed is None:
             seed = int(torch.randint(0, 2 ** 62, (1,)).item())

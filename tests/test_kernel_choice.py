@@ -100,3 +100,21 @@ def test_where_a_plan_is_built():
         assert not plan._build_on_device(fake, 1 << 20)
     finally:
         plan.set_device_build(old)
+
+
+def test_padded_shape_of_narrow_heads():
+    """Heads of fewer than 64 columns run the fused kernels zero-padded to (h', 64): 6 x 50 and 8 x 40 are the reference's
+    other head shapes (configs/imdb-4.yml:10-12, configs/ptb-6.yml:12-14); shapes with kernels of their own are not padded."""
+    import torch
+    from bpt_amd import graphop
+    t = lambda h, d, dt=torch.float32: torch.zeros(3, h, d, dtype=dt)
+    assert graphop.attention_padded_shape(t(6, 50)) == (8, 64)
+    assert graphop.attention_padded_shape(t(8, 40)) == (8, 64)
+    assert graphop.attention_padded_shape(t(8, 40, torch.bfloat16)) == (8, 64)
+    assert graphop.attention_padded_shape(t(2, 16, torch.bfloat16)) == (8, 64)      # bfloat16 has no 4-head kernels
+    assert graphop.attention_padded_shape(t(3, 24)) == (4, 64)
+    assert graphop.attention_padded_shape(t(12, 64)) == (16, 64)
+    assert graphop.attention_padded_shape(t(8, 64)) is None and graphop.attention_padded_shape(t(8, 32)) is None      # own kernels
+    assert graphop.attention_padded_shape(t(8, 80)) is None and graphop.attention_padded_shape(t(20, 50)) is None   # too wide / too many heads
+    assert graphop.attention_padded_shape(t(6, 50, torch.float64)) is None
+    assert graphop.attention_padded_shape(torch.zeros(3, 50)) is None              # 2-D (single head) calls take the op chain
