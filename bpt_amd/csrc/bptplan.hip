@@ -360,7 +360,7 @@ __global__ void k_chunks(const int32_t *work, const int32_t *prefix, const int32
 }
 
 __global__ void k_group_keys(const int32_t *work, const int32_t *chunks, const int32_t *pinfo, int64_t max_groups, int32_t R,
-                             uint32_t *key) {
+                             int by_work, uint32_t *key) {
     const int64_t g = (int64_t)blockIdx.x * TPB + threadIdx.x;
     if (g >= max_groups) return;
     if (g >= n_groups_of(pinfo, R)) {
@@ -369,7 +369,7 @@ __global__ void k_group_keys(const int32_t *work, const int32_t *chunks, const i
     }
     uint32_t c = 0;
     for (int x = 1; x <= 7; ++x) c += (chunks[x] <= g) ? 1u : 0u;
-    key[g] = (c << 16) | (0xFFFFu - (uint32_t)work[g]);
+    key[g] = (c << 16) | (by_work ? 0xFFFFu - (uint32_t)work[g] : 0u);      // (the sort is stable: locality order otherwise)
 }
 
 __global__ void k_invert(const int32_t *order, const int32_t *count, int idx_of_count, int64_t max_n, int32_t *inv) {
@@ -915,7 +915,9 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
     if (max_items < 0 || n_edges < 0 || n_index_nodes < 0 || max_items >= INT32_MAX || n_edges >= INT32_MAX ||
         n_index_nodes >= INT32_MAX)
         return BPT_ERR_SIZE;
-    if (R < 1 || R > 16 || seg_len < 1 || by_mask < 0 || by_mask > 2) return BPT_ERR_SHAPE;
+    if (R < 1 || R > 16 || seg_len < 1 || by_mask < 0 || (by_mask & 3) > 2 || by_mask > 6) return BPT_ERR_SHAPE;
+    const int by_work = (by_mask & 4) ? 0 : 1;                   // + 4: the groups of a range keep their locality order
+    by_mask &= 3;
     if ((int64_t)R * seg_len + FIXED_WORK > 0xFFFF) return BPT_ERR_UNSUPPORTED;       // the work of a group is a 16-bit sort key
     if ((n_edges + 8) * R >= INT32_MAX) return BPT_ERR_SIZE;
     if (!plan_info || !grp_ptr || !entries || !grp_eids || !chunks || !group_info || !workspace) return BPT_ERR_NULL;
@@ -956,7 +958,7 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
     hipLaunchKernelGGL(k_chunks, dim3(1), dim3(64), 0, s, w.work, w.prefix, plan_info, R, chunks, group_info);
     HIP_TRY(hipGetLastError());
     if (max_groups > 0) {
-        LAUNCH(k_group_keys, max_groups, w.work, chunks, plan_info, max_groups, R, w.key_s);
+        LAUNCH(k_group_keys, max_groups, w.work, chunks, plan_info, max_groups, R, by_work, w.key_s);
         tb = tmp;
         HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key_s, w.key, w.iota, w.gorder, max_groups, 32, s));
         LAUNCH(k_invert, max_groups, w.gorder, group_info, (int)BPT_GI_N_GROUPS, max_groups, w.inv);

@@ -19,6 +19,7 @@ import threading
 import torch
 
 from ._lib import BPT_ERR_UNSUPPORTED, BptStatusError, PlanStruct, attn_lib, check_attn
+from . import plan as _plan
 from .plan import GROUP_ORDER_SRC, TILE_GROUP_R, plan_cache
 
 __all__ = ["maskedmm_csr_forward", "maskedmm_csr_backward", "node_mul_edge_forward", "node_mul_edge_backward",
@@ -581,7 +582,7 @@ def attention_backward(row, indptr_r, eid_r, indices_r, col, indptr_c, eid_c, in
             return None
         # the destination side writes (p, ds) by its own pair numbers; the source side finds them through its pair mapping
         return (pi, po, ctypes.byref(pi.bias_rows(TILE_ROWS)["struct"] if bias_by_pair else pi.ensure_groups(TILE_ROWS)["struct"]),
-                ctypes.byref(po.linked_to(pi, TILE_ROWS, partner_order=None, pair_numbers=True)))
+                ctypes.byref(po.linked_to(pi, TILE_ROWS, order=_plan.tile_order_src(po.n_rows, po.n_edges), partner_order=None, pair_numbers=True)))
 
     # as in attention_forward: the tile plans straight away where the tile kernels are certain
     seg = _tile_seg_without_plan(col, eid_c.size(0), q, k, h, d, dropout_p, bias, cfg) if _tiles_backward(None, q.dtype, bias) else None

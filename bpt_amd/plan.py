@@ -25,6 +25,18 @@ GROUP_ORDER_SRC = 2 + 8  # source-side groups of the fused backward: aligned ent
 GROUP_MAX_PAIRS = None  # cap on the edges of one group: None = 48 per member row, 0 = no cap
 GROUP_PAD_ENTRIES = 8  # the kernels' software pipeline reads per-entry arrays this far past the end
 TILE_GROUP_R = 16      # rows per group of the dense-tile kernels
+TILE_ORDER_SRC = None   # order of the SOURCE-side tile groups of the fused backward: None = tile_order_src()'s choice
+
+
+def tile_order_src(n_rows, n_edges):
+    """Order of the source-side tile groups.  On large sparse graphs the groups of an XCD's range keep their locality order
+    (0: groups that run at the same time read the same q / dO rows; measured at L = 8192, k = 4: that kernel's HBM reads
+    245 -> 115 MB and 55 -> 51 us; L = 32768, k = 8 in bfloat16: 455 -> 418 us; the 32-graph batch 95 -> 91 us); on small or
+    dense graphs the order by decreasing work (2 + 4) wins, whose last groups are the lightest (L = 4096, k = 32: 57 against
+    70 us in locality order)."""
+    if TILE_ORDER_SRC is not None:
+        return TILE_ORDER_SRC
+    return 0 if (n_rows >= 12288 and n_edges <= 64 * n_rows) else 2 + 4
 TILE_MAX_PAIRS = 0     # cap on the edges of such a group (0 = none, None = as the other groups)
 _CACHE_SIZE = 64                 # plans kept by the cache (PlanCache.set_limits)
 _CACHE_BYTES = 2 << 30           # and the device memory they may hold together: least recently used plans go first
@@ -433,7 +445,7 @@ class DevicePlan:
         by member mask (+4), or for the aligned order of the host builder (+8), which is sequential by construction, its
         parallel stand-in (entries by neighbour id mod 16, then id); else ascending neighbour."""
         order_mode = GROUP_ORDER if order_mode is None else order_mode
-        by_mask = 2 if order_mode & 8 else (1 if order_mode & 4 else 0)
+        by_mask = (2 if order_mode & 8 else (1 if order_mode & 4 else 0)) + (0 if order_mode & 2 else 4)
         with self._lock:
             hit = self._groups.get((R, by_mask))
             if hit is None:

@@ -77,7 +77,9 @@ int bpt_plan_build_device(const int64_t *row, const int64_t *indptr_units, int64
  * into 8 ranges of equal work (one per XCD) and ordered by decreasing work inside a range; the entries of a group
  * (its distinct neighbours) are in ascending neighbour order (by_mask = 0), sorted by member mask, larger first
  * (by_mask = 1), or by (neighbour mod 16, neighbour) (by_mask = 2: every group walks the id range in the same
- * interleaved way, so groups that run side by side ask for a shared row at about the same step).
+ * interleaved way, so groups that run side by side ask for a shared row at about the same step).  by_mask + 4: the
+ * groups of a range keep their locality order instead of the order by decreasing work (fewer bytes from HBM: the groups
+ * that run at the same time read the same rows; longer tail: the last groups of a range are not the lightest).
  * plan_info is the info block bpt_plan_build_device wrote (device memory; groups are only built when its flags
  * say that the plan covers every edge, else n_groups = 0).  max_items = bounds[0].
  *   members   (bounds[2], R, 2)    grp_ptr (bounds[2] + 1)      entries (n_edges + 1, 4)

@@ -62,7 +62,10 @@ def item_keys(items, idx32, n_index, red):
 def group_plan(arrays, n_index, R, by_mask):
     """Row groups: the items in the order of their largest neighbour, R consecutive ones per group; the groups
     numbered by locality (smallest neighbour), cut into 8 ranges of equal work, by decreasing work inside a range.
-    by_mask: entry order inside a group: 0 / False ascending neighbour, 1 / True by member mask, 2 interleaved."""
+    by_mask: entry order inside a group: 0 / False ascending neighbour, 1 / True by member mask, 2 interleaved; + 4: the groups
+    of a range keep their locality order instead of the order by decreasing work."""
+    by_work = not (int(by_mask) & 4)
+    by_mask = int(by_mask) & 3
     items, idx32, eid32 = arrays["items"], arrays["idx"], arrays["eid"]
     n_items, E = len(items), len(eid32)
     kmax = item_keys(items, idx32, n_index, np.max)
@@ -86,7 +89,7 @@ def group_plan(arrays, n_index, R, by_mask):
         chunks[x] = int(np.count_nonzero(prefix + w // 2 < total * x // 8))
     chunks[8] = ng
     chunk_of = np.searchsorted(chunks[1:8], np.arange(ng), side="right")
-    gorder = np.argsort((chunk_of << 16) | (0xFFFF - w), kind="stable")
+    gorder = np.argsort((chunk_of << 16) | ((0xFFFF - w) if by_work else 0), kind="stable")
     inv = np.empty(ng, dtype=np.int64)
     inv[gorder] = np.arange(ng)
     members = np.full((ng, R, 2), -1, dtype=np.int32)

@@ -106,8 +106,8 @@ def test_device_plan_equals_model_and_host(name, seg):
         plans.append((dp, arrays))
     for R in (4, 8, 16):
         grps = []
-        for (dp, arrays), by_mask in zip(plans, (1, 2) if R != 16 else (0, 0)):
-            hit = dp.ensure_groups(R, {0: 2, 1: 6, 2: 10}[by_mask])
+        for (dp, arrays), by_mask in zip(plans, (1, 2) if R != 16 else (0, 5)):       # (5: entries by mask, groups in locality order)
+            hit = dp.ensure_groups(R, {0: 2, 1: 6, 2: 10, 5: 4}[by_mask])
             grp = model.group_plan(arrays, n, R, by_mask)
             check_groups(hit, grp, len(src))
             grps.append(grp)

@@ -118,3 +118,20 @@ def test_padded_shape_of_narrow_heads():
     assert graphop.attention_padded_shape(t(8, 80)) is None and graphop.attention_padded_shape(t(20, 50)) is None   # too wide / too many heads
     assert graphop.attention_padded_shape(t(6, 50, torch.float64)) is None
     assert graphop.attention_padded_shape(torch.zeros(3, 50)) is None              # 2-D (single head) calls take the op chain
+
+
+def test_order_of_the_source_side_tile_groups():
+    """Large sparse graphs keep the locality order of the groups inside an XCD's range on the source side of the backward,
+    small or dense ones the order by decreasing work; plan.TILE_ORDER_SRC overrides."""
+    from bpt_amd import plan
+    assert plan.tile_order_src(16383, 430237) == 0            # L = 8192, k = 4
+    assert plan.tile_order_src(65535, 3293955) == 0           # L = 32768, k = 8
+    assert plan.tile_order_src(33598, 573520) == 0            # the batch of 32 graphs
+    assert plan.tile_order_src(8191, 784687) == 6             # L = 4096, k = 32: dense
+    assert plan.tile_order_src(8191, 98305) == 6              # L = 4096, k = 1: small
+    assert plan.tile_order_src(1023, 28378) == 6
+    old, plan.TILE_ORDER_SRC = plan.TILE_ORDER_SRC, 10
+    try:
+        assert plan.tile_order_src(16383, 430237) == 10
+    finally:
+        plan.TILE_ORDER_SRC = old
