@@ -378,7 +378,8 @@ __global__ void k_invert(const int32_t *order, const int32_t *count, int idx_of_
     inv[order[i]] = (int32_t)i;
 }
 
-// members of the groups in their final order, and one sort record per edge slot
+// members of the groups in their final order (members given), and one sort record per edge slot (ekey given).  inv == nullptr:
+// the records carry the locality number of their group (the tile plans number their groups only once the entries are known).
 __global__ void k_members_and_records(const int32_t *items, const int32_t *idx32, const int32_t *jorder, const int32_t *lpos,
                                       const int32_t *inv, const int32_t *pinfo, int64_t max_groups, int64_t n_edges, int32_t R,
                                       int32_t *members, uint64_t *ekey, int32_t *eval) {
@@ -388,21 +389,55 @@ __global__ void k_members_and_records(const int32_t *items, const int32_t *idx32
     const int64_t g0 = j / R;
     const int32_t m = (int32_t)(j % R);
     if (g0 >= ng) return;
-    const int32_t gi = inv[lpos[g0]];
-    int32_t *mem = members + ((int64_t)gi * R + m) * 2;
+    const int32_t gi = inv ? inv[lpos[g0]] : lpos[g0];
     if (j >= n_items) {
-        mem[0] = -1;
-        mem[1] = -1;
+        if (members) {
+            members[((int64_t)gi * R + m) * 2] = -1;
+            members[((int64_t)gi * R + m) * 2 + 1] = -1;
+        }
         return;
     }
     const int4 it = reinterpret_cast<const int4 *>(items)[jorder[j]];
-    mem[0] = it.x;
-    mem[1] = it.w;
+    if (members) {
+        members[((int64_t)gi * R + m) * 2] = it.x;
+        members[((int64_t)gi * R + m) * 2 + 1] = it.w;
+    }
+    if (!ekey) return;
     const int32_t p_end = it.z < n_edges ? it.z : (int32_t)n_edges;
     for (int32_t p = it.y > 0 ? it.y : 0; p < p_end; ++p) {
         ekey[p] = ((uint64_t)(uint32_t)gi << 35) | ((uint64_t)(uint32_t)idx32[p] << 4) | (uint64_t)m;
         eval[p] = p;
     }
+}
+
+// Tile plans: what a group costs the matrix kernels is its number of blocks of R entries (a block costs the same whether a
+// third or all of its pairs exist), known once the entries are: work[l] = 4 * (blocks + 1) for the group with locality
+// number l, from the entries' group numbers (ascending, ent_g[u] = l).
+__global__ void k_block_work(const int32_t *ent_g, const int32_t *ginfo, int64_t max_groups, int32_t R, int32_t *work) {
+    const int64_t l = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (l > max_groups) return;
+    const int32_t ng = ginfo[BPT_GI_N_GROUPS], ne = ginfo[BPT_GI_N_ENTRIES];
+    if (l >= ng) {
+        work[l] = 0;
+        return;
+    }
+    int32_t bound[2];
+    for (int t = 0; t < 2; ++t) {                         // first entry whose group is >= l + t
+        int32_t lo = 0, hi = ne;
+        while (lo < hi) {
+            const int32_t mid = (lo + hi) >> 1;
+            if (ent_g[mid] < (int32_t)l + t) lo = mid + 1; else hi = mid;
+        }
+        bound[t] = lo;
+    }
+    work[l] = 4 * ((bound[1] - bound[0] + R - 1) / R + 1);
+}
+
+// the entries' groups from locality numbers to final numbers
+__global__ void k_renumber(int32_t *ent_g, const int32_t *inv, int64_t n_edges, const int32_t *ginfo) {
+    const int64_t u = (int64_t)blockIdx.x * TPB + threadIdx.x;
+    if (u >= n_edges || u >= ginfo[BPT_GI_N_ENTRIES]) return;
+    ent_g[u] = inv[ent_g[u]];
 }
 
 __global__ void k_pad_records(uint64_t *ekey, int32_t *eval, int64_t n_edges, const int32_t *pinfo) {
@@ -464,7 +499,7 @@ __global__ void k_entry_keys(const int32_t *ent_g, const int32_t *ent_mask, cons
     uint64_t k = PAD64;
     if (u < ginfo[BPT_GI_N_ENTRIES]) {
         const uint64_t g = (uint64_t)(uint32_t)ent_g[u], x = (uint64_t)(uint32_t)ent_idx[u];
-        k = (mode == 1) ? ((g << 16) | (uint64_t)(0xFFFF ^ ent_mask[u])) : ((g << 35) | ((x & 15) << 31) | x);
+        k = (mode == 1) ? ((g << 16) | (uint64_t)(0xFFFF ^ ent_mask[u])) : (mode == 2) ? ((g << 35) | ((x & 15) << 31) | x) : ((g << 31) | x);
     }
     ekey[u] = k;
 }
@@ -952,19 +987,31 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
         HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key_s, w.key, w.iota, w.lorder, max_groups, 32, s));
         LAUNCH(k_invert, max_groups, w.lorder, group_info, (int)BPT_GI_N_GROUPS, max_groups, w.lpos);
     }
-    LAUNCH(k_gather_work, max_groups + 1, w.work0, w.lorder, group_info, max_groups, w.work);
-    tb = tmp;
-    HIP_TRY(scan_i32(w.tmp, tb, w.work, w.prefix, max_groups + 1, s));
-    hipLaunchKernelGGL(k_chunks, dim3(1), dim3(64), 0, s, w.work, w.prefix, plan_info, R, chunks, group_info);
-    HIP_TRY(hipGetLastError());
-    if (max_groups > 0) {
-        LAUNCH(k_group_keys, max_groups, w.work, chunks, plan_info, max_groups, R, by_work, w.key_s);
-        tb = tmp;
-        HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb, w.key_s, w.key, w.iota, w.gorder, max_groups, 32, s));
-        LAUNCH(k_invert, max_groups, w.gorder, group_info, (int)BPT_GI_N_GROUPS, max_groups, w.inv);
-        LAUNCH(k_members_and_records, max_groups * R, items, idx32, w.jorder, w.lpos, w.inv, plan_info, max_groups, n_edges, R, members,
-               w.ekey, w.eval);
+    // Tiles (R = 16) are cut into ranges and ordered by their blocks of entries, which are known only after the record sort
+    // below: their records carry the locality numbers first.  The other groups are balanced by their pairs, as formed.
+    const bool by_blocks = (R == 16);
+    auto number_groups = [&]() -> int {                   // w.work (locality numbering) -> chunks, w.gorder, w.inv
+        size_t tb2 = tmp;
+        HIP_TRY(scan_i32(w.tmp, tb2, w.work, w.prefix, max_groups + 1, s));
+        hipLaunchKernelGGL(k_chunks, dim3(1), dim3(64), 0, s, w.work, w.prefix, plan_info, R, chunks, group_info);
+        HIP_TRY(hipGetLastError());
+        if (max_groups > 0) {
+            LAUNCH(k_group_keys, max_groups, w.work, chunks, plan_info, max_groups, R, by_work, w.key_s);
+            LAUNCH(k_iota_i32, max_groups, w.iota, max_groups);
+            tb2 = tmp;
+            HIP_TRY(sort_pairs<uint32_t>(w.tmp, tb2, w.key_s, w.key, w.iota, w.gorder, max_groups, 32, s));
+            LAUNCH(k_invert, max_groups, w.gorder, group_info, (int)BPT_GI_N_GROUPS, max_groups, w.inv);
+        }
+        return BPT_OK;
+    };
+    if (!by_blocks) {
+        LAUNCH(k_gather_work, max_groups + 1, w.work0, w.lorder, group_info, max_groups, w.work);
+        const int st = number_groups();
+        if (st != BPT_OK) return st;
     }
+    if (max_groups > 0)
+        LAUNCH(k_members_and_records, max_groups * R, items, idx32, w.jorder, w.lpos, by_blocks ? (const int32_t *)nullptr : w.inv, plan_info,
+               max_groups, n_edges, R, by_blocks ? (int32_t *)nullptr : members, w.ekey, w.eval);
     // entries: distinct (group, neighbour, multiplicity) of the records sorted by (group, neighbour, member)
     LAUNCH(k_fill_i32, (n_edges + 8) * R, grp_eids, (n_edges + 8) * R, (int32_t)n_edges);
     if (n_edges > 0) {
@@ -982,14 +1029,25 @@ int bpt_plan_group_device(const int32_t *items, const int32_t *idx32, const int3
     HIP_TRY(scan_i32(w.tmp, tb, w.mult, w.ebase, n_edges + 1, s));
     LAUNCH(k_entry_fill, n_edges, w.ekey_s, w.rank, w.run, w.ebase, n_edges, plan_info, w.ent_of, w.ent_idx, w.ent_g,
            w.ent_mask, group_info);
-    // entry order inside a group: neighbour order, or by member mask (larger first, neighbour order inside a mask)
+    if (by_blocks) {
+        // the tiles' cost is known now: their ranges, their final numbers, their members; the entries take the final numbers
+        LAUNCH(k_block_work, max_groups + 1, w.ent_g, group_info, max_groups, R, w.work);
+        const int st = number_groups();
+        if (st != BPT_OK) return st;
+        if (max_groups > 0)
+            LAUNCH(k_members_and_records, max_groups * R, items, idx32, w.jorder, w.lpos, w.inv, plan_info, max_groups, n_edges, R, members,
+                   (uint64_t *)nullptr, (int32_t *)nullptr);
+        if (n_edges > 0) LAUNCH(k_renumber, n_edges, w.ent_g, w.inv, n_edges, group_info);
+    }
+    // entry order inside a group: neighbour order, or by member mask (larger first, neighbour order inside a mask); the
+    // entries of renumbered groups are sorted in every case
     int32_t *perm = w.iota;                               // new position -> entry as numbered above
     LAUNCH(k_iota_i32, n_edges, w.iota, n_edges);
-    if (by_mask != 0 && n_edges > 0) {
+    if ((by_mask != 0 || by_blocks) && n_edges > 0) {
         LAUNCH(k_entry_keys, n_edges, w.ent_g, w.ent_mask, w.ent_idx, n_edges, group_info, (int)by_mask, w.ekey);
         tb = tmp;
         HIP_TRY(sort_pairs<uint64_t>(w.tmp, tb, w.ekey, w.mkey_s, w.iota, w.eval, n_edges,
-                                     (by_mask == 1 ? 16 : 35) + bits_for((uint64_t)max_groups), s));
+                                     (by_mask == 1 ? 16 : by_mask == 2 ? 35 : 31) + bits_for((uint64_t)max_groups), s));
         perm = w.eval;
     }
     LAUNCH(k_invert, n_edges, perm, group_info, (int)BPT_GI_N_ENTRIES, n_edges, w.newpos);

@@ -74,7 +74,9 @@ int bpt_plan_build_device(const int64_t *row, const int64_t *indptr_units, int64
 /* Row groups of R rows over a base plan (the arrays bpt_plan's grp_* fields point at).  The items are taken in
  * the order of their largest neighbour id, R consecutive ones form a group; the groups are numbered by the smallest
  * neighbour id any member reads (groups that read the same rows end up on the same XCD at about the same time), cut
- * into 8 ranges of equal work (one per XCD) and ordered by decreasing work inside a range; the entries of a group
+ * into 8 ranges of equal work (one per XCD) and ordered by decreasing work inside a range (work: the group's pairs plus a
+ * fixed cost; for R = 16, the tile kernels' plans, its number of blocks of 16 entries plus one, which is what a tile costs the
+ * matrix kernels whether a third or all of a block's pairs exist); the entries of a group
  * (its distinct neighbours) are in ascending neighbour order (by_mask = 0), sorted by member mask, larger first
  * (by_mask = 1), or by (neighbour mod 16, neighbour) (by_mask = 2: every group walks the id range in the same
  * interleaved way, so groups that run side by side ask for a shared row at about the same step).  by_mask + 4: the

@@ -59,44 +59,10 @@ def item_keys(items, idx32, n_index, red):
     return out
 
 
-def group_plan(arrays, n_index, R, by_mask):
-    """Row groups: the items in the order of their largest neighbour, R consecutive ones per group; the groups
-    numbered by locality (smallest neighbour), cut into 8 ranges of equal work, by decreasing work inside a range.
-    by_mask: entry order inside a group: 0 / False ascending neighbour, 1 / True by member mask, 2 interleaved; + 4: the groups
-    of a range keep their locality order instead of the order by decreasing work."""
-    by_work = not (int(by_mask) & 4)
-    by_mask = int(by_mask) & 3
-    items, idx32, eid32 = arrays["items"], arrays["idx"], arrays["eid"]
-    n_items, E = len(items), len(eid32)
-    kmax = item_keys(items, idx32, n_index, np.max)
-    jorder = np.argsort(kmax, kind="stable")
-    ng = -(-n_items // R)
-    lens = (items[:, 2] - items[:, 1]).astype(np.int64)
-    w0 = np.zeros(ng, dtype=np.int64)
-    np.add.at(w0, np.arange(n_items) // R, lens[jorder])
-    w0 += FIXED_WORK
-    # locality numbering of the groups: by the smallest neighbour id any member reads
-    kmin = item_keys(items, idx32, n_index, np.min)
-    gk = np.full(ng, np.iinfo(np.int64).max, dtype=np.int64)
-    np.minimum.at(gk, np.arange(n_items) // R, kmin[jorder])
-    lorder = np.argsort(gk, kind="stable")
-    lpos = np.empty(ng, dtype=np.int64)
-    lpos[lorder] = np.arange(ng)
-    w = w0[lorder]
-    prefix, total = _excl(w)[:-1], int(w.sum())
-    chunks = np.zeros(9, dtype=np.int32)
-    for x in range(1, 8):
-        chunks[x] = int(np.count_nonzero(prefix + w // 2 < total * x // 8))
-    chunks[8] = ng
-    chunk_of = np.searchsorted(chunks[1:8], np.arange(ng), side="right")
-    gorder = np.argsort((chunk_of << 16) | ((0xFFFF - w) if by_work else 0), kind="stable")
-    inv = np.empty(ng, dtype=np.int64)
-    inv[gorder] = np.arange(ng)
-    members = np.full((ng, R, 2), -1, dtype=np.int32)
-    g_of_item, m_of_item = inv[lpos[np.arange(n_items) // R]], np.arange(n_items) % R
-    members[g_of_item, m_of_item, 0] = items[jorder, 0]
-    members[g_of_item, m_of_item, 1] = items[jorder, 3]
-    # one record per edge slot, sorted by (group, neighbour, member); equal records keep the slot order
+def _entries_of(items, idx32, eid32, jorder, g_of_item, m_of_item, R):
+    """One record per edge slot sorted by (group, neighbour, member), equal records in slot order; an entry per (group,
+    neighbour) and per repeat of an edge in one member.  Returns ent_idx, ent_g, mask, slot_eid in that order."""
+    E = len(eid32)
     key = np.zeros(E, dtype=np.int64)
     for j, it in enumerate(jorder.tolist()):
         b, e = items[it, 1], items[it, 2]
@@ -123,6 +89,54 @@ def group_plan(arrays, n_index, R, by_mask):
     ent_g[u] = skey >> 35
     np.bitwise_or.at(mask, u, 1 << mem)
     slot_eid[u, mem] = eid32[order]
+    return ent_idx, ent_g, mask, slot_eid
+
+
+def group_plan(arrays, n_index, R, by_mask):
+    """Row groups: the items in the order of their largest neighbour, R consecutive ones per group; the groups
+    numbered by locality (smallest neighbour), cut into 8 ranges of equal work, by decreasing work inside a range.
+    Work: the group's pairs plus a fixed cost; for the tile plans (R = 16) its blocks of R entries, 4 * (blocks + 1) (what
+    the matrix kernels pay for), known only once the entries of the locality-numbered groups are.
+    by_mask: entry order inside a group: 0 / False ascending neighbour, 1 / True by member mask, 2 interleaved; + 4: the groups
+    of a range keep their locality order instead of the order by decreasing work."""
+    by_work = not (int(by_mask) & 4)
+    by_mask = int(by_mask) & 3
+    items, idx32, eid32 = arrays["items"], arrays["idx"], arrays["eid"]
+    n_items, E = len(items), len(eid32)
+    kmax = item_keys(items, idx32, n_index, np.max)
+    jorder = np.argsort(kmax, kind="stable")
+    ng = -(-n_items // R)
+    lens = (items[:, 2] - items[:, 1]).astype(np.int64)
+    w0 = np.zeros(ng, dtype=np.int64)
+    np.add.at(w0, np.arange(n_items) // R, lens[jorder])
+    w0 += FIXED_WORK
+    # locality numbering of the groups: by the smallest neighbour id any member reads
+    kmin = item_keys(items, idx32, n_index, np.min)
+    gk = np.full(ng, np.iinfo(np.int64).max, dtype=np.int64)
+    np.minimum.at(gk, np.arange(n_items) // R, kmin[jorder])
+    lorder = np.argsort(gk, kind="stable")
+    lpos = np.empty(ng, dtype=np.int64)
+    lpos[lorder] = np.arange(ng)
+    m_of_item = np.arange(n_items) % R
+    if R == 16:
+        _, prov_g, _, _ = _entries_of(items, idx32, eid32, jorder, lpos[np.arange(n_items) // R], m_of_item, R)
+        w = 4 * (-(-np.bincount(prov_g, minlength=ng)[:ng] // R) + 1)
+    else:
+        w = w0[lorder]
+    prefix, total = _excl(w)[:-1], int(w.sum())
+    chunks = np.zeros(9, dtype=np.int32)
+    for x in range(1, 8):
+        chunks[x] = int(np.count_nonzero(prefix + w // 2 < total * x // 8))
+    chunks[8] = ng
+    chunk_of = np.searchsorted(chunks[1:8], np.arange(ng), side="right")
+    gorder = np.argsort((chunk_of << 16) | ((0xFFFF - w) if by_work else 0), kind="stable")
+    inv = np.empty(ng, dtype=np.int64)
+    inv[gorder] = np.arange(ng)
+    members = np.full((ng, R, 2), -1, dtype=np.int32)
+    g_of_item = inv[lpos[np.arange(n_items) // R]]
+    members[g_of_item, m_of_item, 0] = items[jorder, 0]
+    members[g_of_item, m_of_item, 1] = items[jorder, 3]
+    ent_idx, ent_g, mask, slot_eid = _entries_of(items, idx32, eid32, jorder, g_of_item, m_of_item, R)
     if int(by_mask) == 1:        # by member mask, larger first
         perm = np.argsort((ent_g << 16) | (0xFFFF ^ mask), kind="stable")
         ent_idx, ent_g, mask, slot_eid = ent_idx[perm], ent_g[perm], mask[perm], slot_eid[perm]
