@@ -91,15 +91,27 @@ def cpu_baseline(src, dst, N, H, D, seed, budget_s=25.0):
 
 
 def timed(fn, steps, warmup):
+    """Seconds per call of fn over `steps` calls between two synchronisations.  Python's cyclic garbage collector is off
+    inside the timed region, as in timeit: a full collection of this process's heap takes 25-45 ms, which a region of
+    30 ms cannot absorb (it showed as one run in three at twice the time of the others)."""
+    import gc
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    t = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t) / steps
+    gc_was_on = gc.isenabled()
+    gc.collect()
+    gc.disable()
+    try:
+        t = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+    finally:
+        if gc_was_on:
+            gc.enable()
+    return dt / steps
 
 
 def median(xs):
