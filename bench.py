@@ -91,27 +91,32 @@ def cpu_baseline(src, dst, N, H, D, seed, budget_s=25.0):
 
 
 def timed(fn, steps, warmup):
-    """Seconds per call of fn over `steps` calls between two synchronisations.  Python's cyclic garbage collector is off
-    inside the timed region, as in timeit: a full collection of this process's heap takes 25-45 ms, which a region of
-    30 ms cannot absorb (it showed as one run in three at twice the time of the others)."""
-    import gc
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t) / steps
+
+
+def timed_runs(fn, steps, warmups):
+    """Seconds per call of fn, one figure per entry of `warmups` (that many untimed calls, then `steps` timed ones between
+    two synchronisations).  Python's cyclic garbage collector is off from before the first warm-up to after the last run,
+    as in timeit: a full collection of this process's heap takes 25-45 ms, which a timed region of 30 ms cannot absorb (it
+    showed as one run in three at twice the time of the others), and a collection between the runs would leave the GPU
+    idle right before a timed region."""
+    import gc
     gc_was_on = gc.isenabled()
     gc.collect()
     gc.disable()
     try:
-        t = time.perf_counter()
-        for _ in range(steps):
-            fn()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t
+        return [timed(fn, steps, w) for w in warmups]
     finally:
         if gc_was_on:
             gc.enable()
-    return dt / steps
 
 
 def median(xs):
@@ -136,7 +141,7 @@ def graph_replay_runs(step, ref, steps, warmup, runs=3):
         if ref is not None and not all(torch.equal(a, b) for a, b in zip(gout, ref)):
             log("HIP graph replay did not reproduce the eager result; using eager timing")
             return []
-        out = [timed(g.replay, steps, warmup if i == 0 else 2) for i in range(runs)]
+        out = timed_runs(g.replay, steps, [warmup if i == 0 else 2 for i in range(runs)])
         if ref is not None and not all(torch.equal(a, b) for a, b in zip(gout, ref)):
             log("HIP graph replay did not reproduce the eager result; using eager timing")
             return []
@@ -180,7 +185,7 @@ def measure_side_workload(name, dtype_name, dev, steps, no_graph, label=None):
 
     ref = step()
     torch.cuda.synchronize()
-    runs = [timed(step, steps, 10 if i == 0 else 2) for i in range(3)]
+    runs = timed_runs(step, steps, [10, 2, 2])
     t, tmin, mode = median(runs), min(runs), "eager"
     if not no_graph:
         gr = graph_replay_runs(step, ref, steps, 10)
@@ -225,7 +230,7 @@ def measure_narrow_heads(dev, steps, no_graph, h=6, d=50):
         step = make(fused)
         ref = step()
         torch.cuda.synchronize()
-        t = median([timed(step, steps, 5 if i == 0 else 2) for i in range(3)])
+        t = median(timed_runs(step, steps, [5, 2, 2]))
         if not no_graph:
             gr = graph_replay_runs(step, None, steps, 5)
             if gr:
@@ -361,7 +366,7 @@ def main():
     # The timed region is exactly --steps steps between two synchronisations.  It is run three times; the MEDIAN run is
     # the reported ms_per_step and the shortest one is kept beside it (all three are in the JSON line): the host of a
     # shared box stalls now and then for tens of milliseconds, which shows as one slow run of the three.
-    runs_eager = [timed(step, args.steps, args.warmup if i == 0 else 2) for i in range(3)]
+    runs_eager = timed_runs(step, args.steps, [args.warmup, 2, 2])
     t_eager, t_eager_min = median(runs_eager), min(runs_eager)
     t_step, t_step_min, mode = t_eager, t_eager_min, "eager"
     t_graph_replay, runs_graph = None, []
@@ -459,7 +464,7 @@ def main():
             x.backward(gh)
             return x
 
-        t_stack = median([timed(stack_step, 5, 2) for _ in range(3)])
+        t_stack = median(timed_runs(stack_step, 5, [2, 2, 2]))
         block = {"layers": args.block_layers, "d_model": dm, "d_ff": 4 * dm, "ms_per_layer_fwd_bwd": round(t_stack / args.block_layers * 1e3, 4),
                  "attention_ms_per_layer": round(t_step * 1e3, 4), "attention_share": round(t_step * args.block_layers / t_stack, 3)}
         log(f"block stack: {block}")
@@ -487,7 +492,7 @@ def main():
         def best_of_eager_and_replay(fn):
             # as for the headline step: eager launches (through autograd here, about 0.2 ms of host work per step) or the
             # replay of a HIP graph of the same step, whichever median of three runs is lower
-            t = median([timed(fn, 100, 10) for _ in range(3)])
+            t = median(timed_runs(fn, 100, [10, 10, 10]))
             if not args.no_graph:
                 gr = graph_replay_runs(fn, None, 100, 10)
                 if gr:
