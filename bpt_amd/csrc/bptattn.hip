@@ -1646,12 +1646,15 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
 // v_mfma_f32_16x16x4f32: D[i][n] += sum_k A[i][k] B[k][n], lane (c = lane % 16, g = lane / 16) supplies A[c][g] and
 // B[g][c] and holds D[4 g + r][c] in register r.  Which column of a row a (step, g) pair stands for is free as long as
 // A and B agree, so operands are loaded as 16-byte vectors:
-//   scores S^T = K Q^T : A = K[entry c][16 t + 4 g + e], B = q[member c][16 t + 4 g + e] (steps t, e = 0..3);
-//                        register r of lane (c, g) = score of (entry 4 g + r, member c);
+//   scores S^T = K Q^T : A = K[entry e(c)][16 t + 4 g + e], B = q[member c][16 t + 4 g + e] (steps t, e = 0..3), where
+//                        row c of the product is entry e(c) = 4 (c % 4) + c / 4 of the block, so that
+//                        register r of lane (c, g) = score of (entry 4 r + g, member c);
 //   output O += P V    : A = register r of the probabilities as they stand (row = member c, k = g stands for entry
-//                        4 g + r), B = V[entry 4 g + r][4 c + nb]; register r' of accumulator nb of lane (c, g) =
+//                        4 r + g), B = V[entry 4 r + g][4 c + nb]; register r' of accumulator nb of lane (c, g) =
 //                        O[member 4 g + r'][4 c + nb]: four consecutive columns per lane, 256 contiguous bytes per
-//                        member and 16 lanes.
+//                        member and 16 lanes.  Step r of such a product covers the neighbouring entries 4 r .. 4 r + 3:
+//                        past the end of a group's entry list (half of its last block on average) steps are left out.
+//   (The bfloat16 kernels below keep entry 4 g + r in register r: their products over the entries are one instruction.)
 // Softmax state is per lane for member c (the four lanes of a member hold partial denominators that are added at the
 // end); the exponent reference is raised lazily as in the matrix-core forward above.
 constexpr int TILE_R = 16;
@@ -1719,7 +1722,7 @@ __device__ __forceinline__ void tile_load16(const char *row, float (&out)[16]) {
     }
 }
 
-// register r of the result of lane (c, g) = sum over the 64 columns of a[entry c] * b[member c] for (entry 4 g + r, member c)
+// register r of the result of lane (c, g) = sum over the 64 columns of a[row 4 g + r] * b[member c], a[row c] = what lane c passes
 __device__ __forceinline__ floatx4v tile_dot(const float (&a)[16], const float (&b)[16]) {
     floatx4v s0 = floatx4v{0.f, 0.f, 0.f, 0.f}, s1 = s0;
 #pragma unroll
@@ -1731,14 +1734,18 @@ __device__ __forceinline__ floatx4v tile_dot(const float (&a)[16], const float (
 }
 
 // acc[nb][r'] (member 4 g + r', column 4 c + nb) += sum over the block's entries of w[member][entry] * row[entry][column]:
-// w = this lane's four weights (member c with entries 4 g + r), rows = columns 4 c .. 4 c + 3 of the rows of entries 4 g + r
-__device__ __forceinline__ void tile_axpy(const float (&w)[4], const float4 (&rows)[4], floatx4v (&acc)[4]) {
+// w = this lane's four weights (member c with entries 4 r + g), rows = columns 4 c .. 4 c + 3 of the rows of entries 4 r + g.
+// Step r of the product stands for the four NEIGHBOURING entries 4 r .. 4 r + 3 (one per lane group), so a step whose
+// entries lie past the end of the group's list (nv = the block's entries that exist) is left out.
+__device__ __forceinline__ void tile_axpy_upto(const float (&w)[4], const float4 (&rows)[4], floatx4v (&acc)[4], int nv) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].x, acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].y, acc[1], 0, 0, 0);
-        acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].z, acc[2], 0, 0, 0);
-        acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].w, acc[3], 0, 0, 0);
+        if (4 * r < nv) {
+            acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].x, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].y, acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].z, acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].w, acc[3], 0, 0, 0);
+        }
     }
 }
 
@@ -1770,12 +1777,16 @@ __device__ __forceinline__ void tile_store_rows(const TileCtx &t, const floatx4v
     }
 }
 
-// Edge ids of this lane's four pairs of a block, (entry 4 g + r, member c): what the dropout hash and the score term are
+// Edge ids of this lane's four pairs of a block, (entry first_entry + step * r, member c): what the dropout hash and the score term are
 // indexed by (n_edges, the spare row, where the pair does not exist; past the group's end the last entry is read again).
-__device__ __forceinline__ void tile_pair_eids(const bpt_plan &P, int first_entry, int p_end, int c, int (&xe)[4]) {
+__device__ __forceinline__ void tile_pair_eids(const bpt_plan &P, int first_entry, int p_end, int c, int (&xe)[4], int step = 1) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) xe[r] = P.grp_eids[(size_t)min(first_entry + r, p_end - 1) * TILE_R + c];
+    for (int r = 0; r < 4; ++r) xe[r] = P.grp_eids[(size_t)min(first_entry + step * r, p_end - 1) * TILE_R + c];
 }
+// Which entry of a block lane c loads as row c of the products over the columns, in the float32 tile kernels: the
+// scores of entries 4 r + g have to come out in register r of lane group g (row 4 g + r of the product), so that step r
+// of the products over the entries stands for four NEIGHBOURING entries and can be left out past the end of the list.
+__device__ __forceinline__ int tile_entry_of_row(int c) { return 4 * (c & 3) + (c >> 2); }
 // Where the score term of the pair (entry, member c) sits and its gradient goes.  BIAS == 1, stored by edge id: row eid
 // of (n_edges + 1, H), the spare last row for a pair that does not exist.  BIAS == 2, stored in the plan's own order:
 // head-major at the pair's number, x[head * n_edges + number]: the lanes of an entry touch one run of memory and no
@@ -1844,7 +1855,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     struct Blk {
         float kr[16];
         float4 vr[4];
-        int has;                                                  // bit r: the pair (entry 4 g + r, member c) exists
+        int has, nv;                                              // bit r of has: the pair (entry 4 r + g, member c) exists; nv: entries of the block that exist
         int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
@@ -1852,12 +1863,15 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            const int2 ea = ent[TILE_R * b + c];
-            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
-            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
-            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            const int mk[4] = {e01.y, e01.w, e23.y, e23.w};
+            if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + g, t.p_end, c, B.xe, 4);
+            B.nv = min(TILE_R, cnt - TILE_R * b);
+            const int2 ea = ent[TILE_R * b + tile_entry_of_row(c)];
+            int idxv[4], mk[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int2 en = ent[TILE_R * b + 4 * r + g];
+                idxv[r] = en.x; mk[r] = en.y;
+            }
             B.has = ((mk[0] >> c) & 1) | (((mk[1] >> c) & 1) << 1) | (((mk[2] >> c) & 1) << 2) | (((mk[3] >> c) & 1) << 3);
             tile_load16(kb + ((uint32_t)ea.x * (uint32_t)(C * sizeof(T)) + t.offa), B.kr);
 #pragma unroll
@@ -1868,10 +1882,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 1>(P, t.head, B.xe[BIAS == 1 ? r : 0], 0)];
             }
             if constexpr (BIAS == 2) {
-                const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
-                const int fv[4] = {f4.x, f4.y, f4.z, f4.w};
 #pragma unroll
-                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 2>(P, t.head, 0, tile_pair_number(fv[r], mk[r], c))];
+                for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, 2>(P, t.head, 0, tile_pair_number(fst[TILE_R * b + 4 * r + g], mk[r], c))];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -1903,7 +1915,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 if constexpr (DROP)
                     pr[r] *= dropout_keep((uint32_t)B.xe[DROP ? r : 0] * (uint32_t)H + (uint32_t)t.head, drop_seed, drop_thr, drop_inv);
             }
-            tile_axpy(pr, B.vr, acc);
+            tile_axpy_upto(pr, B.vr, acc, B.nv);
         };
         tile_walk<PIPE, Blk>(nblk, issue, compute);
         wave_lds_fence();                                         // the piece is read to the end before the next one is staged
@@ -1970,8 +1982,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
     struct Blk {
         float kr[16], va[16];
-        float4 kc[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 g + r
-        int pos[4], has;                                           // bit r of has: the pair (entry 4 g + r, member c) exists
+        float4 kc[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 r + g
+        int pos[4], has, nv;                                       // bit r of has: the pair (entry 4 r + g, member c) exists; nv: entries of the block that exist
         int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
     };
@@ -1979,15 +1991,18 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
-            if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            const int2 ea = ent[TILE_R * b + c];
-            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
-            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
-            const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
-            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            B.has = ((e01.y >> c) & 1) | (((e01.w >> c) & 1) << 1) | (((e23.y >> c) & 1) << 2) | (((e23.w >> c) & 1) << 3);
-            B.pos[0] = tile_pair_number(f4.x, e01.y, c); B.pos[1] = tile_pair_number(f4.y, e01.w, c);
-            B.pos[2] = tile_pair_number(f4.z, e23.y, c); B.pos[3] = tile_pair_number(f4.w, e23.w, c);
+            if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + g, t.p_end, c, B.xe, 4);
+            B.nv = min(TILE_R, cnt - TILE_R * b);
+            const int2 ea = ent[TILE_R * b + tile_entry_of_row(c)];
+            int idxv[4];
+            B.has = 0;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int2 en = ent[TILE_R * b + 4 * r + g];
+                idxv[r] = en.x;
+                B.has |= ((en.y >> c) & 1) << r;
+                B.pos[r] = tile_pair_number(fst[TILE_R * b + 4 * r + g], en.y, c);
+            }
             const uint32_t arow = (uint32_t)ea.x * (uint32_t)(C * sizeof(T)) + t.offa;
             tile_load16(kb + arow, B.kr);
             tile_load16(vb + arow, B.va);
@@ -2023,7 +2038,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                     if constexpr (BIAS) ds_out[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])] = ds[r];   // dL/d(score before scaling)
                 }
             }
-            tile_axpy(ds, B.kc, acc);
+            tile_axpy_upto(ds, B.kc, acc, B.nv);
         };
         tile_walk<PIPE, Blk>(nblk, issue, compute);
         wave_lds_fence();
@@ -2049,26 +2064,28 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     floatx4v ak[4], av[4];
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) { ak[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; av[nb] = floatx4v{0.f, 0.f, 0.f, 0.f}; }
+    // Both products contract over the block's entries, four per step; lane group g takes entries 4 r + g in step r, so that
+    // the steps past the end of the group's list (half of a group's last block on average) can be left out.
     struct Blk {
         float4 qr[4], dr[4];
         float2 w[4];
-        int has;                                                  // bit r: the pair (entry 4 g + r, member c) exists
+        int has, nv;                                              // bit r of has: the pair (entry 4 r + g, member c) exists; nv: entries of the block that exist
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
         auto issue = [&](Blk &B, int b) {
-            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
-            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
-            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
-            B.has = ((e01.y >> c) & 1) | (((e01.w >> c) & 1) << 1) | (((e23.y >> c) & 1) << 2) | (((e23.w >> c) & 1) << 3);
+            B.nv = min(TILE_R, cnt - TILE_R * b);
+            B.has = 0;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const uint32_t off = (uint32_t)idxv[r] * (uint32_t)(C * sizeof(T)) + t.offv;
+                const int2 en = ent[TILE_R * b + 4 * r + g];
+                B.has |= ((en.y >> c) & 1) << r;
+                const uint32_t off = (uint32_t)en.x * (uint32_t)(C * sizeof(T)) + t.offv;
                 B.qr[r] = *reinterpret_cast<const float4 *>(qb + off);
                 B.dr[r] = *reinterpret_cast<const float4 *>(db + off);
                 // (positions past the group's end are read at its last entry: their masks are empty)
-                const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
+                const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * r + g, t.p_end - 1) * TILE_R + c];
                 B.w[r] = pds_h[pos];
             }
         };
@@ -2080,8 +2097,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 pe[r] = has ? B.w[r].x : 0.f;
                 ds[r] = has ? B.w[r].y : 0.f;
             }
-            tile_axpy(ds, B.qr, ak);
-            tile_axpy(pe, B.dr, av);
+            tile_axpy_upto(ds, B.qr, ak, B.nv);
+            tile_axpy_upto(pe, B.dr, av, B.nv);
         };
         tile_walk<PIPE, Blk>(nblk, issue, compute);
         wave_lds_fence();
