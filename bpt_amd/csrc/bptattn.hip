@@ -1745,6 +1745,10 @@ __device__ __forceinline__ void tile_axpy_upto(const float (&w)[4], const float4
             acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].y, acc[1], 0, 0, 0);
             acc[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].z, acc[2], 0, 0, 0);
             acc[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[r], rows[r].w, acc[3], 0, 0, 0);
+        } else {
+            // (the step's rows are marked as read: left in flight, they would make the next block's loads wait for
+            // everything that is outstanding, this block's stores included)
+            asm volatile("" ::"v"(rows[r].x), "v"(rows[r].y), "v"(rows[r].z), "v"(rows[r].w));
         }
     }
 }
