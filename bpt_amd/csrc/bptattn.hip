@@ -2027,6 +2027,10 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 dob[4 * i] = x.x; dob[4 * i + 1] = x.y; dob[4 * i + 2] = x.z; dob[4 * i + 3] = x.w;
             }
             const floatx4v dp = tile_dot(B.va, dob);
+            // The rows of the third product are waited for here, while loads are all that is in flight: behind the stores
+            // below, a wait for them would be a wait for the stores' completion as well.
+            // (Not in the variants with dropout or the score term: they have no register to spare for rows that arrive early.)
+            if constexpr (!DROP && BIAS == 0) asm volatile("" ::"v"(B.kc[0].w), "v"(B.kc[1].w), "v"(B.kc[2].w), "v"(B.kc[3].w));
             float ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
