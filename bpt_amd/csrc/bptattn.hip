@@ -2349,6 +2349,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
         };
         auto compute = [&](const Blk &B) {
             const floatx4v st = tile_dot_bf16(B.kr, qb), dp = tile_dot_bf16(B.va, dob);
+            // (as in the float32 kernel: the rows of the third product are waited for before the stores, not behind them)
+            if constexpr (!DROP && BIAS == 0) asm volatile("" ::"v"(B.kc[0].y), "v"(B.kc[1].y), "v"(B.kc[2].y), "v"(B.kc[3].y));
             float ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
