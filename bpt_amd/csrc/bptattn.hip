@@ -3058,9 +3058,15 @@ __global__ __launch_bounds__(HW * WAVE) void k_rel_bias_tiles(bpt_plan P, const 
         int nt[AHEAD];
 #pragma unroll
         for (int k = 0; k < AHEAD; ++k) nt[k] = pair_tm[min(x + (AHEAD + k) * WAVE, end - 1)];
+        float val[AHEAD];
+#pragma unroll
+        for (int k = 0; k < AHEAD; ++k) val[k] = qt[(tm[k] & 0xff) * TILE_R + (tm[k] >> 8)];
+        // (the next round's loads are waited for before this round's stores: behind them the wait would include the stores)
+#pragma unroll
+        for (int k = 0; k < AHEAD; ++k) asm volatile("" ::"v"(nt[k]));
 #pragma unroll
         for (int k = 0; k < AHEAD; ++k) {
-            if (x + k * WAVE < end) out[x + k * WAVE] = qt[(tm[k] & 0xff) * TILE_R + (tm[k] >> 8)];
+            if (x + k * WAVE < end) out[x + k * WAVE] = val[k];
             tm[k] = nt[k];
         }
     }
