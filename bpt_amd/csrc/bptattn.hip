@@ -2082,9 +2082,30 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
+        // Where this lane's four pairs of block b sit in the scratch (positions past the group's end are read at its last
+        // entry: their masks are empty).  They are fetched one block ahead, so that the (p, ds) loads of a block leave
+        // together with its row loads instead of one round trip later.
+        auto positions = [&](int b, int (&pos)[4]) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) pos[r] = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * r + g, t.p_end - 1) * TILE_R + c];
+        };
+        int pos_ahead[4], ahead_of = -1;                          // the positions of block ahead_of
         auto issue = [&](Blk &B, int b) {
             B.nv = min(TILE_R, cnt - TILE_R * b);
             B.has = 0;
+            int pos[4];
+            if constexpr (PIPE) {                                 // (rows are read a block ahead there, and registers are short)
+                positions(b, pos);
+            } else {
+                if (b == ahead_of) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) pos[r] = pos_ahead[r];
+                } else {
+                    positions(b, pos);
+                }
+                if (b + 1 < nblk) positions(b + 1, pos_ahead);
+                ahead_of = b + 1;
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int2 en = ent[TILE_R * b + 4 * r + g];
@@ -2092,9 +2113,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 const uint32_t off = (uint32_t)en.x * (uint32_t)(C * sizeof(T)) + t.offv;
                 B.qr[r] = *reinterpret_cast<const float4 *>(qb + off);
                 B.dr[r] = *reinterpret_cast<const float4 *>(db + off);
-                // (positions past the group's end are read at its last entry: their masks are empty)
-                const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * r + g, t.p_end - 1) * TILE_R + c];
-                B.w[r] = pds_h[pos];
+                B.w[r] = pds_h[pos[r]];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -2411,7 +2430,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
                 const uint32_t off = (uint32_t)idxv[r] * (uint32_t)RB + offc;
                 B.qr[r] = *reinterpret_cast<const uint2 *>(qb + off);
                 B.dr[r] = *reinterpret_cast<const uint2 *>(db + off);
-                // (positions past the group's end are read at its last entry: their masks are empty)
+                // (positions past the group's end are read at its last entry: their masks are empty.  Fetching them a block
+                // ahead, as the float32 kernel does, costs this kernel registers it does not have: 31.8 -> 32.9 us)
                 const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
                 B.w[r] = pds_h[pos];
             }
