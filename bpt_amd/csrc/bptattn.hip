@@ -2148,7 +2148,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 // shrink by a third on the destination side but only by an eighth on the source side (L = 8192, k = 4: 67 k -> 46 k and
 // 71 k -> 62 k entries), and the step went from 0.113 to 0.117 ms (32-graph batch 0.177 -> 0.205, window 128 level).
 constexpr bool TILE_BF16_PIPE = false;
-constexpr int TILE_BF16_WPE = 6, TILE_BF16_WPE_DST = 5;     // wavefronts per SIMD the bfloat16 tile kernels are compiled for
+constexpr int TILE_BF16_WPE = 6, TILE_BF16_WPE_DST = 5, TILE_BF16_WPE_SRC = 5;     // wavefronts per SIMD the bfloat16 tile kernels are compiled for
 typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
 typedef float floatx2v __attribute__((ext_vector_type(2)));
@@ -2420,20 +2420,35 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         tile_stage_entries(P, ent, p0, cnt, t.lane);
+        // (the positions of a block's pairs in the scratch are fetched one block ahead, as in the float32 kernel, so that the
+        // (p, ds) loads leave with the row loads; positions past the group's end are read at its last entry: their masks are
+        // empty.  The four registers this takes are why the kernel is compiled for five wavefronts per SIMD, not six: with
+        // six it spills and loses what the prefetch gains)
+        auto positions = [&](int b, int (&pos)[4]) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) pos[r] = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
+        };
+        int pos_ahead[4], ahead_of = -1;
         auto issue = [&](Blk &B, int b) {
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
             B.has = ((e01.y >> c) & 1) | (((e01.w >> c) & 1) << 1) | (((e23.y >> c) & 1) << 2) | (((e23.w >> c) & 1) << 3);
+            int pos[4];
+            if (b == ahead_of) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) pos[r] = pos_ahead[r];
+            } else {
+                positions(b, pos);
+            }
+            if (b + 1 < nblk) positions(b + 1, pos_ahead);
+            ahead_of = b + 1;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const uint32_t off = (uint32_t)idxv[r] * (uint32_t)RB + offc;
                 B.qr[r] = *reinterpret_cast<const uint2 *>(qb + off);
                 B.dr[r] = *reinterpret_cast<const uint2 *>(db + off);
-                // (positions past the group's end are read at its last entry: their masks are empty.  Fetching them a block
-                // ahead, as the float32 kernel does, costs this kernel registers it does not have: 31.8 -> 32.9 us)
-                const int pos = P.grp_pairs[(size_t)min(p0 + TILE_R * b + 4 * g + r, t.p_end - 1) * TILE_R + c];
-                B.w[r] = pds_h[pos];
+                B.w[r] = pds_h[pos[r]];
             }
         };
         auto compute = [&](const Blk &B) {
@@ -4015,7 +4030,7 @@ int run_attn_bwd(const bpt_plan *Pin, const bpt_plan *Pout, const void *q, const
             if (st != BPT_OK) return st;
             {
                 ProfScope prof(BPT_KERNEL_ATTN_BWD_SRC, s);
-                hipLaunchKernelGGL((k_attn_bwd_src_tile_bf16<H, D, HW, TILE_BF16_WPE, TILE_BF16_PIPE>), dim3(group_grid(Pout) * (H / HW)), dim3(HW * WAVE), 0, s,
+                hipLaunchKernelGGL((k_attn_bwd_src_tile_bf16<H, D, HW, TILE_BF16_WPE_SRC, TILE_BF16_PIPE>), dim3(group_grid(Pout) * (H / HW)), dim3(HW * WAVE), 0, s,
                                    *Pout, (const bf16_t *)q, (const bf16_t *)d_o, (const uint32_t *)ws, (bf16_t *)dk, (bf16_t *)dv, ws_dk, ws_dv);
             }
             st = launch_status();
