@@ -1699,16 +1699,32 @@ __device__ __forceinline__ bool tile_begin(const bpt_plan &P, TileCtx &t) {
 // The entry list of a group is staged, TILE_CHUNK entries at a time, in a wavefront-private piece of LDS as (neighbour,
 // mask) pairs: every lane needs five of them per block (its A-operand row and the four rows / masks of its lane
 // group), which would otherwise be five dependent global loads in front of every block's row loads.
-__device__ __forceinline__ void tile_stage_entries(const bpt_plan &P, int2 *lds, int p0, int cnt, int lane, int *first = nullptr) {
+struct TileEntryRegs {
+    int4 x[TILE_CHUNK / WAVE];
+};
+// first half: the loads.  A kernel asks for its first piece before it reads its members' rows, so that the two round trips
+// run side by side; in source order the compiler puts the members' arithmetic (and its wait) in front of these loads.
+__device__ __forceinline__ void tile_ask_entries(const bpt_plan &P, int p0, int cnt, int lane, TileEntryRegs &r) {
     const int4 *entries = reinterpret_cast<const int4 *>(P.grp_entries);
+#pragma unroll
+    for (int u = 0; u < TILE_CHUNK / WAVE; ++u) r.x[u] = entries[p0 + min(u * WAVE + lane, cnt - 1)];   // past the end: the last entry again
+}
+// second half: into the wavefront's piece of LDS
+__device__ __forceinline__ void tile_put_entries(const TileEntryRegs &r, int2 *lds, int cnt, int lane, int *first = nullptr) {
 #pragma unroll
     for (int u = 0; u < TILE_CHUNK / WAVE; ++u) {
         const int e = u * WAVE + lane;
-        const int4 x = entries[p0 + min(e, cnt - 1)];           // past the end: the last entry with an empty mask
-        lds[e] = make_int2(x.x, e < cnt ? x.y : 0);
-        if (first) first[e] = x.z;                              // number of the entry's first pair (members follow in ascending order)
+        int nbr = r.x[u].x, mask = r.x[u].y;
+        asm volatile("" : "+v"(nbr), "+v"(mask));                 // (the values are used from here on: nothing of this half moves up to the loads)
+        lds[e] = make_int2(nbr, e < cnt ? mask : 0);              // past the end: an empty mask
+        if (first) first[e] = r.x[u].z;                          // number of the entry's first pair (members follow in ascending order)
     }
     wave_lds_fence();
+}
+__device__ __forceinline__ void tile_stage_entries(const bpt_plan &P, int2 *lds, int p0, int cnt, int lane, int *first = nullptr) {
+    TileEntryRegs r;
+    tile_ask_entries(P, p0, cnt, lane, r);
+    tile_put_entries(r, lds, cnt, lane, first);
 }
 // number of the pair (entry, member c) among the plan's pairs: the entry's first pair + the members before c in its mask
 __device__ __forceinline__ int tile_pair_number(int first, int mask, int c) { return first + __popc((uint32_t)mask & ((1u << c) - 1u)); }
@@ -1834,6 +1850,44 @@ __device__ __forceinline__ void tile_walk(int nblk, Issue &&issue, Compute &&com
     }
 }
 
+// The rows a block needs FIRST (the K rows of its scores) are asked for one block ahead, the others (V) when the block
+// begins: sixteen more registers instead of the thirty-two of the two-stage pipeline, so four wavefronts per SIMD stay.
+// once_loads_left(): called once the first loads have left, for work that waits for loads asked for before them.
+template <typename Blk, typename IssueFirst, typename IssueRest, typename Compute, typename Hook>
+__device__ __forceinline__ void tile_walk_first_ahead(int nblk, IssueFirst &&first, IssueRest &&rest, Compute &&compute, Hook &&once_loads_left) {
+    Blk A, B;
+    first(A, 0);
+    issue_loads_first();
+    once_loads_left();
+    int b = 0;
+    for (; b + 2 < nblk; b += 2) {
+        rest(A, b);
+        first(B, b + 1);
+        issue_loads_first();
+        compute(A);
+        issue_loads_first();
+        rest(B, b + 1);
+        first(A, b + 2);
+        issue_loads_first();
+        compute(B);
+        issue_loads_first();
+    }
+    rest(A, b);
+    if (b + 1 < nblk) {
+        first(B, b + 1);
+        issue_loads_first();
+        compute(A);
+        issue_loads_first();
+        rest(B, b + 1);
+        issue_loads_first();
+        compute(B);
+    } else {
+        issue_loads_first();
+        compute(A);
+    }
+    issue_loads_first();
+}
+
 template <typename T, int H, int D, int HW, bool PIPE, bool DROP, int BIAS>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 3 : 4))) void k_attn_fwd_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, T *__restrict__ o, float *__restrict__ lse,
@@ -1846,12 +1900,18 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     __shared__ int fst_lds[HW][BIAS == 2 ? TILE_CHUNK : 1];      // the entries' first pair numbers: where a term in pair order sits
     int2 *ent = ent_lds[t.wv];
     int *fst = BIAS == 2 ? fst_lds[t.wv] : nullptr;
+    TileEntryRegs er;
+    if (t.p_end > t.p_begin) tile_ask_entries(P, t.p_begin, min(TILE_CHUNK, t.p_end - t.p_begin), t.lane, er);
+    issue_loads_first();
     const int c = t.c, g = t.g;
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
     float qb[16];
-    tile_load16(reinterpret_cast<const char *>(q) + (size_t)max(t.member.x, 0) * (C * sizeof(T)) + t.offa, qb);
-#pragma unroll
-    for (int i = 0; i < 16; ++i) qb[i] *= scale_log2e;
+    // The members' q rows are asked for behind the first block's K rows: asked for here, ahead of the loop, they are waited
+    // for before the entry list is (one more round trip in front of the K rows).  They stay as they are and the scores are
+    // scaled instead, so nothing has to happen to them between their arrival and the first product.
+    const char *const qrow = reinterpret_cast<const char *>(q) + (size_t)max(t.member.x, 0) * (C * sizeof(T)) + t.offa;
+    constexpr bool AHEAD = !PIPE && !DROP;                        // (with dropout the sixteen registers are not there)
+    if constexpr (!AHEAD) tile_load16(qrow, qb);
     floatx4v acc[4];
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
@@ -1865,11 +1925,15 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
-        tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
-        auto issue = [&](Blk &B, int b) {
+        if (p0 != t.p_begin) tile_ask_entries(P, p0, cnt, t.lane, er);
+        tile_put_entries(er, ent, cnt, t.lane, fst);
+        auto issue_k = [&](Blk &B, int b) {
+            const int2 ea = ent[TILE_R * b + tile_entry_of_row(c)];
+            tile_load16(kb + ((uint32_t)ea.x * (uint32_t)(C * sizeof(T)) + t.offa), B.kr);
+        };
+        auto issue_rest = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + g, t.p_end, c, B.xe, 4);
             B.nv = min(TILE_R, cnt - TILE_R * b);
-            const int2 ea = ent[TILE_R * b + tile_entry_of_row(c)];
             int idxv[4], mk[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -1877,7 +1941,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 idxv[r] = en.x; mk[r] = en.y;
             }
             B.has = ((mk[0] >> c) & 1) | (((mk[1] >> c) & 1) << 1) | (((mk[2] >> c) & 1) << 2) | (((mk[3] >> c) & 1) << 3);
-            tile_load16(kb + ((uint32_t)ea.x * (uint32_t)(C * sizeof(T)) + t.offa), B.kr);
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 B.vr[r] = *reinterpret_cast<const float4 *>(vb + ((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T)) + t.offv));
@@ -1894,7 +1957,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             const floatx4v st = tile_dot(B.kr, qb);
             float sc[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sc[r] = ((B.has >> r) & 1) ? (BIAS ? fmaf(B.bz[BIAS ? r : 0], scale_log2e, st[r]) : st[r]) : -INFINITY;
+            for (int r = 0; r < 4; ++r)
+                sc[r] = ((B.has >> r) & 1) ? (BIAS ? fmaf(st[r], scale_log2e, B.bz[BIAS ? r : 0] * scale_log2e) : st[r] * scale_log2e) : -INFINITY;
             const float mb = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
             if (__builtin_amdgcn_ballot_w64(mb > mref + MFMA_TAU) != 0) {
                 float gm = fmaxf(mb, __shfl_xor(mb, 16));
@@ -1921,7 +1985,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             }
             tile_axpy_upto(pr, B.vr, acc, B.nv);
         };
-        tile_walk<PIPE, Blk>(nblk, issue, compute);
+        auto issue = [&](Blk &B, int b) { issue_k(B, b); issue_rest(B, b); };
+        if constexpr (!AHEAD) tile_walk<PIPE, Blk>(nblk, issue, compute);
+        else tile_walk_first_ahead<Blk>(nblk, issue_k, issue_rest, compute, [&]() { if (p0 == t.p_begin) tile_load16(qrow, qb); });
         wave_lds_fence();                                         // the piece is read to the end before the next one is staged
     }
     float lt = lrun + __shfl_xor(lrun, 16);
@@ -1959,6 +2025,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     __shared__ int fst_lds[HW][TILE_CHUNK];
     int2 *ent = ent_lds[t.wv];
     int *fst = fst_lds[t.wv];
+    TileEntryRegs er;
+    if (t.p_end > t.p_begin) tile_ask_entries(P, t.p_begin, min(TILE_CHUNK, t.p_end - t.p_begin), t.lane, er);
+    issue_loads_first();
     const int c = t.c, g = t.g;
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
     const size_t mrow = (size_t)max(t.member.x, 0) * (C * sizeof(T)) + t.offa;
@@ -1966,6 +2035,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     // the member's dO columns live in LDS (lane-major, read back before every product with them): with them in registers
     // the kernel needs 144 and a SIMD holds three wavefronts, without them 128 and four
     __shared__ float4 dob_lds[HW][4][WAVE];
+    // (q stays as it is and the scores are scaled, as in the forward: the same roundings in both)
     float qb[16], delta, lse_c;
     {
         float ob[16], dob[16];
@@ -1974,7 +2044,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         tile_load16(reinterpret_cast<const char *>(o) + mrow, ob);
         float part = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { part = fmaf(dob[i], ob[i], part); qb[i] *= scale_log2e; }
+        for (int i = 0; i < 16; ++i) part = fmaf(dob[i], ob[i], part);
         part += __shfl_xor(part, 16);
         delta = part + __shfl_xor(part, 32);                      // dO . O of member c, this head
         lse_c = lse[(size_t)max(t.member.x, 0) * H + t.head];
@@ -1993,7 +2063,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
-        tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
+        if (p0 != t.p_begin) tile_ask_entries(P, p0, cnt, t.lane, er);
+        tile_put_entries(er, ent, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + g, t.p_end, c, B.xe, 4);
             B.nv = min(TILE_R, cnt - TILE_R * b);
@@ -2035,7 +2106,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const bool has = (B.has >> r) & 1;
-                float pe = has ? __builtin_amdgcn_exp2f((BIAS ? fmaf(B.bz[BIAS ? r : 0], scale_log2e, st[r]) : st[r]) - lse_c) : 0.f;
+                float pe = has ? __builtin_amdgcn_exp2f((BIAS ? fmaf(st[r], scale_log2e, B.bz[BIAS ? r : 0] * scale_log2e) : st[r] * scale_log2e) - lse_c) : 0.f;
                 float mt = 1.f;                                   // dropout multiplier of this pair (as in the forward)
                 if constexpr (DROP)
                     mt = dropout_keep((uint32_t)B.xe[DROP ? r : 0] * (uint32_t)H + (uint32_t)t.head, drop_seed, drop_thr, drop_inv);
@@ -2148,7 +2219,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 // shrink by a third on the destination side but only by an eighth on the source side (L = 8192, k = 4: 67 k -> 46 k and
 // 71 k -> 62 k entries), and the step went from 0.113 to 0.117 ms (32-graph batch 0.177 -> 0.205, window 128 level).
 constexpr bool TILE_BF16_PIPE = false;
-constexpr int TILE_BF16_WPE = 6, TILE_BF16_WPE_DST = 5, TILE_BF16_WPE_SRC = 5;     // wavefronts per SIMD the bfloat16 tile kernels are compiled for
+constexpr int TILE_BF16_WPE = 5, TILE_BF16_WPE_DST = 5, TILE_BF16_WPE_SRC = 5;     // wavefronts per SIMD the bfloat16 tile kernels are compiled for
 typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
 typedef float floatx2v __attribute__((ext_vector_type(2)));
@@ -2193,7 +2264,7 @@ __device__ __forceinline__ void tile_load_row_bf16(const char *p, Bf8 (&out)[2])
 }
 
 template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, int BIAS>
-__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP || BIAS ? WPE - 1 : WPE))) void k_attn_fwd_tile_bf16(
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_fwd_tile_bf16(
     bpt_plan P, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v, bf16_t *__restrict__ o,
     float *__restrict__ lse, float *__restrict__ ws_acc, float *__restrict__ ws_ml, float scale_log2e, uint32_t drop_thr,
     uint32_t drop_seed, float drop_inv, const float *__restrict__ bias) {
@@ -2204,6 +2275,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     __shared__ int fst_lds[HW][BIAS == 2 ? TILE_CHUNK : 1];      // the entries' first pair numbers: where a term in pair order sits
     int2 *ent = ent_lds[t.wv];
     int *fst = BIAS == 2 ? fst_lds[t.wv] : nullptr;
+    TileEntryRegs er;
+    if (t.p_end > t.p_begin) tile_ask_entries(P, t.p_begin, min(TILE_CHUNK, t.p_end - t.p_begin), t.lane, er);
+    issue_loads_first();
     const int c = t.c, g = t.g;
     const uint32_t offr = (uint32_t)((t.head * D + 16 * g) * 2), offc = (uint32_t)((t.head * D + 4 * c) * 2);
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
@@ -2222,16 +2296,16 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
-        tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
-        auto issue = [&](Blk &B, int b) {
+        if (p0 != t.p_begin) tile_ask_entries(P, p0, cnt, t.lane, er);
+        tile_put_entries(er, ent, cnt, t.lane, fst);
+        auto issue_k = [&](Blk &B, int b) { tile_load_row_bf16(kb + ((uint32_t)ent[TILE_R * b + c].x * (uint32_t)RB + offr), B.kr); };
+        auto issue_rest = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
             const int mk[4] = {e01.y, e01.w, e23.y, e23.w};
             B.has = ((mk[0] >> c) & 1) | (((mk[1] >> c) & 1) << 1) | (((mk[2] >> c) & 1) << 2) | (((mk[3] >> c) & 1) << 3);
-            tile_load_row_bf16(kb + ((uint32_t)ea.x * (uint32_t)RB + offr), B.kr);
 #pragma unroll
             for (int r = 0; r < 4; ++r) B.vr[r] = *reinterpret_cast<const uint2 *>(vb + ((uint32_t)idxv[r] * (uint32_t)RB + offc));
             if constexpr (BIAS == 1) {
@@ -2278,7 +2352,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             pa.u[1] = pack_bf16(pr[2], pr[3]);
             tile_axpy_bf16(pa, B.vr, acc);
         };
-        tile_walk<PIPE, Blk>(nblk, issue, compute);
+        auto issue = [&](Blk &B, int b) { issue_k(B, b); issue_rest(B, b); };
+        if constexpr (PIPE || DROP || BIAS != 0) tile_walk<PIPE, Blk>(nblk, issue, compute);      // (the K rows ahead: eight registers more)
+        else tile_walk_first_ahead<Blk>(nblk, issue_k, issue_rest, compute, []() {});
         wave_lds_fence();
     }
     float lt = lrun + __shfl_xor(lrun, 16);
@@ -2307,6 +2383,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     __shared__ int fst_lds[HW][TILE_CHUNK];
     int2 *ent = ent_lds[t.wv];
     int *fst = fst_lds[t.wv];
+    TileEntryRegs er;
+    if (t.p_end > t.p_begin) tile_ask_entries(P, t.p_begin, min(TILE_CHUNK, t.p_end - t.p_begin), t.lane, er);
+    issue_loads_first();
     const int c = t.c, g = t.g;
     const uint32_t offr = (uint32_t)((t.head * D + 16 * g) * 2), offc = (uint32_t)((t.head * D + 4 * c) * 2);
     const char *kb = reinterpret_cast<const char *>(k), *vb = reinterpret_cast<const char *>(v);
@@ -2345,7 +2424,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     };
     for (int p0 = t.p_begin; p0 < t.p_end; p0 += TILE_CHUNK) {
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
-        tile_stage_entries(P, ent, p0, cnt, t.lane, fst);
+        if (p0 != t.p_begin) tile_ask_entries(P, p0, cnt, t.lane, er);
+        tile_put_entries(er, ent, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int2 ea = ent[TILE_R * b + c];
