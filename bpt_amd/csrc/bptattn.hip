@@ -1817,6 +1817,27 @@ __device__ __forceinline__ uint32_t tile_bias_at(const bpt_plan &P, int head, in
     else return (uint32_t)eid * (uint32_t)H + (uint32_t)head;
 }
 
+// The rows of a block's entries come from memory in the layout of the products over the entries (lane (c, g): columns
+// 4 c .. 4 c + 3 of the rows of entries 4 r + g: the sixteen lanes of a lane group read one row's 256 contiguous bytes).
+// The products over the COLUMNS want lane c to hold sixteen columns of ONE row (entry tile_entry_of_row(c)); loaded that
+// way, neighbouring lanes read different rows and the texture addresser spends four cycles on every group of four lanes
+// instead of one.  So the rows are loaded once, in the first layout, and turned in a wavefront-private piece of LDS:
+// rows of TILE_KT_STRIDE floats (64 + 4: the sixteen rows of a read fall on different banks).
+constexpr int TILE_KT_STRIDE = 68;
+__device__ __forceinline__ void tile_rows_to_operand(float *kt, const float4 (&rows)[4], int c, int g, float (&out)[16]) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+        *reinterpret_cast<floatx4v *>(kt + (4 * r + g) * TILE_KT_STRIDE + 4 * c) = floatx4v{rows[r].x, rows[r].y, rows[r].z, rows[r].w};
+    wave_lds_fence();
+    const float *src = kt + tile_entry_of_row(c) * TILE_KT_STRIDE + 4 * g;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const floatx4v x = *reinterpret_cast<const floatx4v *>(src + 16 * t);
+        out[4 * t] = x[0]; out[4 * t + 1] = x[1]; out[4 * t + 2] = x[2]; out[4 * t + 3] = x[3];
+    }
+    wave_lds_fence();                                             // (read before the next block's rows are written)
+}
+
 // PIPE: the rows of the next block are loaded while one is used (two-stage register pipeline).  Pays on graphs with few,
 // tall tiles (a dense window graph: 9 blocks per tile, two wavefronts per SIMD in all), costs a wavefront per SIMD:
 // at L = 8192, k = 4 (1217 tiles of 4 blocks) the forward takes 47 us with it and 44 without.
@@ -1900,6 +1921,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     __shared__ int fst_lds[HW][BIAS == 2 ? TILE_CHUNK : 1];      // the entries' first pair numbers: where a term in pair order sits
     int2 *ent = ent_lds[t.wv];
     int *fst = BIAS == 2 ? fst_lds[t.wv] : nullptr;
+    __shared__ float kt_lds[HW][TILE_R * TILE_KT_STRIDE];
+    float *kt = kt_lds[t.wv];
     TileEntryRegs er;
     if (t.p_end > t.p_begin) tile_ask_entries(P, t.p_begin, min(TILE_CHUNK, t.p_end - t.p_begin), t.lane, er);
     issue_loads_first();
@@ -1917,7 +1940,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
     float mref = M_INIT_LOG2, lrun = 0.f;
     struct Blk {
-        float kr[16];
+        float4 kq[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 r + g
         float4 vr[4];
         int has, nv;                                              // bit r of has: the pair (entry 4 r + g, member c) exists; nv: entries of the block that exist
         int xe[DROP || BIAS == 1 ? 4 : 1];
@@ -1928,8 +1951,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         if (p0 != t.p_begin) tile_ask_entries(P, p0, cnt, t.lane, er);
         tile_put_entries(er, ent, cnt, t.lane, fst);
         auto issue_k = [&](Blk &B, int b) {
-            const int2 ea = ent[TILE_R * b + tile_entry_of_row(c)];
-            tile_load16(kb + ((uint32_t)ea.x * (uint32_t)(C * sizeof(T)) + t.offa), B.kr);
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                B.kq[r] = *reinterpret_cast<const float4 *>(kb + ((uint32_t)ent[TILE_R * b + 4 * r + g].x * (uint32_t)(C * sizeof(T)) + t.offv));
         };
         auto issue_rest = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + g, t.p_end, c, B.xe, 4);
@@ -1954,7 +1978,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
             }
         };
         auto compute = [&](const Blk &B) {
-            const floatx4v st = tile_dot(B.kr, qb);
+            float kr[16];
+            tile_rows_to_operand(kt, B.kq, c, g, kr);
+            const floatx4v st = tile_dot(kr, qb);
             float sc[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -2025,6 +2051,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     __shared__ int fst_lds[HW][TILE_CHUNK];
     int2 *ent = ent_lds[t.wv];
     int *fst = fst_lds[t.wv];
+    __shared__ float kt_lds[HW][TILE_R * TILE_KT_STRIDE];
+    float *kt = kt_lds[t.wv];
     TileEntryRegs er;
     if (t.p_end > t.p_begin) tile_ask_entries(P, t.p_begin, min(TILE_CHUNK, t.p_end - t.p_begin), t.lane, er);
     issue_loads_first();
@@ -2055,8 +2083,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
     struct Blk {
-        float kr[16], va[16];
-        float4 kc[4];                                             // columns 4 c .. 4 c + 3 of the K rows of entries 4 r + g
+        float4 kc[4], vc[4];                                      // columns 4 c .. 4 c + 3 of the K / V rows of entries 4 r + g
         int pos[4], has, nv;                                       // bit r of has: the pair (entry 4 r + g, member c) exists; nv: entries of the block that exist
         int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
@@ -2068,7 +2095,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
         auto issue = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + g, t.p_end, c, B.xe, 4);
             B.nv = min(TILE_R, cnt - TILE_R * b);
-            const int2 ea = ent[TILE_R * b + tile_entry_of_row(c)];
             int idxv[4];
             B.has = 0;
 #pragma unroll
@@ -2078,30 +2104,33 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
                 B.has |= ((en.y >> c) & 1) << r;
                 B.pos[r] = tile_pair_number(fst[TILE_R * b + 4 * r + g], en.y, c);
             }
-            const uint32_t arow = (uint32_t)ea.x * (uint32_t)(C * sizeof(T)) + t.offa;
-            tile_load16(kb + arow, B.kr);
-            tile_load16(vb + arow, B.va);
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 B.kc[r] = *reinterpret_cast<const float4 *>(kb + ((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T)) + t.offv));
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                B.vc[r] = *reinterpret_cast<const float4 *>(vb + ((uint32_t)idxv[r] * (uint32_t)(C * sizeof(T)) + t.offv));
             if constexpr (BIAS) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])];
             }
         };
         auto compute = [&](const Blk &B) {
-            const floatx4v st = tile_dot(B.kr, qb);
+            floatx4v st;
+            {
+                float kr[16];
+                tile_rows_to_operand(kt, B.kc, c, g, kr);
+                st = tile_dot(kr, qb);
+            }
+            float va[16];
+            tile_rows_to_operand(kt, B.vc, c, g, va);
             float dob[16];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float4 x = dob_lds[t.wv][i][t.lane];
                 dob[4 * i] = x.x; dob[4 * i + 1] = x.y; dob[4 * i + 2] = x.z; dob[4 * i + 3] = x.w;
             }
-            const floatx4v dp = tile_dot(B.va, dob);
-            // The rows of the third product are waited for here, while loads are all that is in flight: behind the stores
-            // below, a wait for them would be a wait for the stores' completion as well.
-            // (Not in the variants with dropout or the score term: they have no register to spare for rows that arrive early.)
-            if constexpr (!DROP && BIAS == 0) asm volatile("" ::"v"(B.kc[0].w), "v"(B.kc[1].w), "v"(B.kc[2].w), "v"(B.kc[3].w));
+            const floatx4v dp = tile_dot(va, dob);
             float ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
