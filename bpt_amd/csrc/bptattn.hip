@@ -2291,6 +2291,25 @@ __device__ __forceinline__ void tile_load_row_bf16(const char *p, Bf8 (&out)[2])
     out[0].q = *reinterpret_cast<const uint4 *>(p);
     out[1].q = *reinterpret_cast<const uint4 *>(p + 16);
 }
+// As tile_rows_to_operand: the rows of a block's entries, loaded as columns 4 c .. 4 c + 3 of the rows of entries 4 g + r
+// (the sixteen lanes of a lane group read one row's 128 contiguous bytes), turned in a wavefront-private piece of LDS
+// into the operand of the products over the columns (lane (c, g): columns 16 g .. 16 g + 15 of the row of entry c).
+// Rows of TILE_KT_BYTES_BF16 = 128 + 16 bytes: the sixteen rows of a read fall on different banks.
+constexpr int TILE_KT_BYTES_BF16 = 144;
+typedef uint32_t uintx2v __attribute__((ext_vector_type(2)));
+typedef uint32_t uintx4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void tile_rows_to_operand_bf16(char *kt, const uint2 (&rows)[4], int c, int g, Bf8 (&out)[2]) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) *reinterpret_cast<uintx2v *>(kt + (4 * g + r) * TILE_KT_BYTES_BF16 + 8 * c) = uintx2v{rows[r].x, rows[r].y};
+    wave_lds_fence();
+    const char *src = kt + c * TILE_KT_BYTES_BF16 + 32 * g;
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+        const uintx4v x = *reinterpret_cast<const uintx4v *>(src + 16 * h2);
+        out[h2].q = make_uint4(x[0], x[1], x[2], x[3]);
+    }
+    wave_lds_fence();                                             // (read before the next block's rows are written)
+}
 
 template <int H, int D, int HW, int WPE, bool PIPE, bool DROP, int BIAS>
 __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))) void k_attn_fwd_tile_bf16(
@@ -2304,6 +2323,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
     __shared__ int fst_lds[HW][BIAS == 2 ? TILE_CHUNK : 1];      // the entries' first pair numbers: where a term in pair order sits
     int2 *ent = ent_lds[t.wv];
     int *fst = BIAS == 2 ? fst_lds[t.wv] : nullptr;
+    __shared__ __attribute__((aligned(16))) char kt_lds[HW][TILE_R * TILE_KT_BYTES_BF16];
+    char *kt = kt_lds[t.wv];
     TileEntryRegs er;
     if (t.p_end > t.p_begin) tile_ask_entries(P, t.p_begin, min(TILE_CHUNK, t.p_end - t.p_begin), t.lane, er);
     issue_loads_first();
@@ -2317,7 +2338,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
     for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
     float mref = M_INIT_LOG2, lrun = 0.f;
     struct Blk {
-        Bf8 kr[2];
+        uint2 kq[4];                                              // columns 4 c .. 4 c + 3 of the K rows of entries 4 g + r
         uint2 vr[4];
         int has;                                                  // bit r: the pair (entry 4 g + r, member c) exists
         int xe[DROP || BIAS == 1 ? 4 : 1];
@@ -2327,7 +2348,13 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
         const int cnt = min(TILE_CHUNK, t.p_end - p0), nblk = (cnt + TILE_R - 1) / TILE_R;
         if (p0 != t.p_begin) tile_ask_entries(P, p0, cnt, t.lane, er);
         tile_put_entries(er, ent, cnt, t.lane, fst);
-        auto issue_k = [&](Blk &B, int b) { tile_load_row_bf16(kb + ((uint32_t)ent[TILE_R * b + c].x * (uint32_t)RB + offr), B.kr); };
+        auto issue_k = [&](Blk &B, int b) {
+            const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
+            const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
+            const int idxv[4] = {e01.x, e01.z, e23.x, e23.z};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) B.kq[r] = *reinterpret_cast<const uint2 *>(kb + ((uint32_t)idxv[r] * (uint32_t)RB + offc));
+        };
         auto issue_rest = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
@@ -2349,7 +2376,9 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(WPE))
             }
         };
         auto compute = [&](const Blk &B) {
-            const floatx4v st = tile_dot_bf16(B.kr, qb);
+            Bf8 kr[2];
+            tile_rows_to_operand_bf16(kt, B.kq, c, g, kr);
+            const floatx4v st = tile_dot_bf16(kr, qb);
             float sc[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) sc[r] = ((B.has >> r) & 1) ? (BIAS ? st[r] + B.bz[BIAS ? r : 0] : st[r]) * scale_log2e : -INFINITY;
@@ -2412,6 +2441,8 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
     __shared__ int fst_lds[HW][TILE_CHUNK];
     int2 *ent = ent_lds[t.wv];
     int *fst = fst_lds[t.wv];
+    __shared__ __attribute__((aligned(16))) char kt_lds[HW][TILE_R * TILE_KT_BYTES_BF16];
+    char *kt = kt_lds[t.wv];
     TileEntryRegs er;
     if (t.p_end > t.p_begin) tile_ask_entries(P, t.p_begin, min(TILE_CHUNK, t.p_end - t.p_begin), t.lane, er);
     issue_loads_first();
@@ -2445,8 +2476,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) acc[nb] = floatx4v{0.f, 0.f, 0.f, 0.f};
     struct Blk {
-        Bf8 kr[2], va[2];
-        uint2 kc[4];
+        uint2 kc[4], vc[4];                                       // columns 4 c .. 4 c + 3 of the K / V rows of entries 4 g + r
         int has, pos[4];                                           // bit r of has: the pair (entry 4 g + r, member c) exists
         int xe[DROP || BIAS == 1 ? 4 : 1];
         float bz[BIAS ? 4 : 1];
@@ -2457,7 +2487,6 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
         tile_put_entries(er, ent, cnt, t.lane, fst);
         auto issue = [&](Blk &B, int b) {
             if constexpr (DROP || BIAS == 1) tile_pair_eids(P, p0 + TILE_R * b + 4 * g, t.p_end, c, B.xe);
-            const int2 ea = ent[TILE_R * b + c];
             const int4 e01 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g]);
             const int4 e23 = *reinterpret_cast<const int4 *>(&ent[TILE_R * b + 4 * g + 2]);
             const int4 f4 = *reinterpret_cast<const int4 *>(&fst[TILE_R * b + 4 * g]);
@@ -2465,20 +2494,21 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(DROP 
             B.has = ((e01.y >> c) & 1) | (((e01.w >> c) & 1) << 1) | (((e23.y >> c) & 1) << 2) | (((e23.w >> c) & 1) << 3);
             B.pos[0] = tile_pair_number(f4.x, e01.y, c); B.pos[1] = tile_pair_number(f4.y, e01.w, c);
             B.pos[2] = tile_pair_number(f4.z, e23.y, c); B.pos[3] = tile_pair_number(f4.w, e23.w, c);
-            const uint32_t arow = (uint32_t)ea.x * (uint32_t)RB + offr;
-            tile_load_row_bf16(kb + arow, B.kr);
-            tile_load_row_bf16(vb + arow, B.va);
 #pragma unroll
             for (int r = 0; r < 4; ++r) B.kc[r] = *reinterpret_cast<const uint2 *>(kb + ((uint32_t)idxv[r] * (uint32_t)RB + offc));
+#pragma unroll
+            for (int r = 0; r < 4; ++r) B.vc[r] = *reinterpret_cast<const uint2 *>(vb + ((uint32_t)idxv[r] * (uint32_t)RB + offc));
             if constexpr (BIAS) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) B.bz[r] = bias[tile_bias_at<H, BIAS>(P, t.head, B.xe[BIAS == 1 ? r : 0], B.pos[r])];
             }
         };
         auto compute = [&](const Blk &B) {
-            const floatx4v st = tile_dot_bf16(B.kr, qb), dp = tile_dot_bf16(B.va, dob);
-            // (as in the float32 kernel: the rows of the third product are waited for before the stores, not behind them)
-            if constexpr (!DROP && BIAS == 0) asm volatile("" ::"v"(B.kc[0].y), "v"(B.kc[1].y), "v"(B.kc[2].y), "v"(B.kc[3].y));
+            Bf8 kr[2];
+            tile_rows_to_operand_bf16(kt, B.kc, c, g, kr);
+            const floatx4v st = tile_dot_bf16(kr, qb);
+            tile_rows_to_operand_bf16(kt, B.vc, c, g, kr);
+            const floatx4v dp = tile_dot_bf16(kr, dob);
             float ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
