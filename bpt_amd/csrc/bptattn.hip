@@ -1933,7 +1933,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
     // for before the entry list is (one more round trip in front of the K rows).  They stay as they are and the scores are
     // scaled instead, so nothing has to happen to them between their arrival and the first product.
     const char *const qrow = reinterpret_cast<const char *>(q) + (size_t)max(t.member.x, 0) * (C * sizeof(T)) + t.offa;
-    constexpr bool AHEAD = !PIPE && !DROP;                        // (with dropout the sixteen registers are not there)
+    constexpr bool AHEAD = !PIPE && !DROP && BIAS == 0;         // (with dropout or the score term the sixteen registers are not there)
     if constexpr (!AHEAD) tile_load16(qrow, qb);
     floatx4v acc[4];
 #pragma unroll
@@ -2030,8 +2030,11 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 }
 
 // Backward on tiles, destination side: per block the scores and dO . v of all 16 x 16 pairs (two products over the
-// columns), p = 2^(s - lse), ds = p (dO . v - delta) scale, dq += ds K (third product; K is read a second time in the
-// column layout, which the L1 serves).  (p, ds) of the pairs that exist go to a scratch in THIS side's order, compact:
+// columns, the K and V rows turned in LDS from the layout they are loaded in), p = 2^(s - lse),
+// ds = p (dO . v - delta) scale, dq += ds K (third product, on the K rows as loaded).  With dropout or a score term the
+// kernel is compiled for three wavefronts per SIMD: at four it keeps the members' q rows in scratch memory and reads
+// them back for every block (83 against 58 us with dropout at L = 8192, k = 4).
+// (p, ds) of the pairs that exist go to a scratch in THIS side's order, compact:
 // pds[head * n_edges + t] for the pair number t of (entry, member) = the entry's first pair + the rank of the member in
 // its mask, so the lanes of an entry write one contiguous run and the runs of consecutive entries follow each other.  The
 // source side looks its pairs up there through its pair mapping (grp_pairs = this side's pair numbers).  Writing in the
@@ -2039,7 +2042,7 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 // time (126 against 85 us at L = 4096, k = 32); letting the source side recompute p and ds (two more products there,
 // delta (n, H) handed over) measured slower than either on every graph tried.
 template <typename T, int H, int D, int HW, bool PIPE, bool DROP, int BIAS>
-__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : DROP && BIAS ? 3 : 4))) void k_attn_bwd_dst_tile(
+__global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE ? 2 : DROP || BIAS ? 3 : 4))) void k_attn_bwd_dst_tile(
     bpt_plan P, const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, const T *__restrict__ o,
     const T *__restrict__ d_o, const float *__restrict__ lse, T *__restrict__ dq, float2 *__restrict__ pds, float *__restrict__ ws_dq,
     float scale, float scale_log2e, uint32_t drop_thr, uint32_t drop_seed, float drop_inv, const float *__restrict__ bias,
