@@ -1645,7 +1645,8 @@ __global__ __launch_bounds__(2 * WAVE) __attribute__((amdgpu_waves_per_eu(sizeof
 //
 // v_mfma_f32_16x16x4f32: D[i][n] += sum_k A[i][k] B[k][n], lane (c = lane % 16, g = lane / 16) supplies A[c][g] and
 // B[g][c] and holds D[4 g + r][c] in register r.  Which column of a row a (step, g) pair stands for is free as long as
-// A and B agree, so operands are loaded as 16-byte vectors:
+// A and B agree, so operands are held as 16-byte vectors (the members' rows are loaded that way; the entries' rows
+// reach the first layout below through LDS, see tile_rows_to_operand):
 //   scores S^T = K Q^T : A = K[entry e(c)][16 t + 4 g + e], B = q[member c][16 t + 4 g + e] (steps t, e = 0..3), where
 //                        row c of the product is entry e(c) = 4 (c % 4) + c / 4 of the block, so that
 //                        register r of lane (c, g) = score of (entry 4 r + g, member c);
@@ -2239,10 +2240,11 @@ __global__ __launch_bounds__(HW * WAVE) __attribute__((amdgpu_waves_per_eu(PIPE 
 
 // ---- Dense tiles for bfloat16 rows.  Same walk and the same lane roles as the float32 tile kernels above, on
 // v_mfma_f32_16x16x32_bf16 (products over the 64 columns: two instructions) and v_mfma_f32_16x16x16_bf16 (products over
-// the 16 entries of a block: one instruction per four output columns), operands as loaded, float32 accumulation:
-//   lane (c, g) loads columns 16 g .. 16 g + 15 of the row of entry c (32 contiguous bytes; slot j of step t of the product
-//   stands for column 16 g + 8 t + j in both operands) and columns 4 c .. 4 c + 3 of the rows of entries 4 g + r (8 bytes;
-//   the B operand of output columns {4 c + nb} takes element nb of each of the four, packed by byte permutes).
+// the 16 entries of a block: one instruction per four output columns), float32 accumulation:
+//   lane (c, g) holds columns 16 g .. 16 g + 15 of the row of entry c (32 contiguous bytes; slot j of step t of the product
+//   stands for column 16 g + 8 t + j in both operands; the members' rows are loaded that way, the entries' rows turned in
+//   LDS, see tile_rows_to_operand_bf16) and loads columns 4 c .. 4 c + 3 of the rows of entries 4 g + r (8 bytes; the B
+//   operand of output columns {4 c + nb} takes element nb of each of the four, packed by byte permutes).
 // Probabilities and ds are rounded to bfloat16 where they enter a product (the softmax denominator is summed unrounded);
 // the scratch between the two backward kernels holds (p, ds) as two bfloat16 in 4 bytes, by head and destination-side pair number.
 // The two-stage register pipeline of tile_walk does not pay here: at six wavefronts per SIMD it spills (2.4 x slower),
