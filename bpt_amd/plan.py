@@ -37,6 +37,20 @@ def tile_order_src(n_rows, n_edges):
     if TILE_ORDER_SRC is not None:
         return TILE_ORDER_SRC
     return 0 if (n_rows >= 12288 and n_edges <= 64 * n_rows) else 2 + 4
+TILE_ORDER_DST = None   # order of the DESTINATION-side tile groups (the forward's and the fused backward's): None = tile_order_dst()'s choice
+
+
+def tile_order_dst(n_index_nodes):
+    """Order of the destination-side tile groups (what ensure_groups takes for groups of TILE_GROUP_R rows when no order is
+    named).  By decreasing work inside an XCD's range (2 + 4: the last groups are the lightest) tiles that read the same
+    K / V rows do not run at the same time and the rows are fetched about twice; that costs nothing while K and V fit the
+    memory-side cache, and locality order (4) is slower there (L = 8192, k = 4: 0.142 against 0.144 ms; the 32-graph
+    batch 0.264 against 0.267; 32 767 nodes level).  Beyond it the second fetch is HBM traffic and locality order wins:
+    65 535 nodes, 8 heads float32 0.669 -> 0.641 ms (bfloat16 level), 131 071 nodes 1.425 -> 1.268 (bfloat16
+    0.813 -> 0.786), L = 32768, k = 8 with 16 heads float32 1.547 -> 1.447, bfloat16 0.912 -> 0.895."""
+    if TILE_ORDER_DST is not None:
+        return TILE_ORDER_DST
+    return 4 if n_index_nodes >= 49152 else 2 + 4
 TILE_MAX_PAIRS = 0     # cap on the edges of such a group (0 = none, None = as the other groups)
 _CACHE_SIZE = 64                 # plans kept by the cache (PlanCache.set_limits)
 _CACHE_BYTES = 2 << 30           # and the device memory they may hold together: least recently used plans go first
@@ -232,11 +246,15 @@ class Plan:
         return ctypes.byref(self.struct)
 
     # ---- row groups for the fused attention kernels ----
+    def default_order(self, R):
+        """The group order where a caller names none: tile groups by tile_order_dst, the others GROUP_ORDER."""
+        return tile_order_dst(self.n_index_nodes) if R == TILE_GROUP_R else GROUP_ORDER
+
     def ensure_groups(self, R=GROUP_R, order_mode=None):
         """Builds the row-group arrays for groups of R rows once (host) and uploads them.  Returns a dict with
         the host arrays ("host") and the `bpt_plan` carrying them ("struct").  Groups of TILE_GROUP_R rows (the dense-tile
         kernels) have no cap on their edges: a tile costs the same whether its pairs exist or not."""
-        order_mode = GROUP_ORDER if order_mode is None else order_mode
+        order_mode = self.default_order(R) if order_mode is None else order_mode
         with self._lock:
             hit = self._groups.get((R, order_mode))
             if hit is None:
@@ -287,7 +305,7 @@ class Plan:
         entry's first pair + the rank of the member in its mask; 0 where the pair does not exist).  The row-group kernels
         link the destination side to the source side by positions, the tile kernels the source side to the destination
         side by pair numbers."""
-        o_mine, o_theirs = (GROUP_ORDER if order is None else order), (GROUP_ORDER if partner_order is None else partner_order)
+        o_mine, o_theirs = (self.default_order(R) if order is None else order), (plan_src.default_order(R) if partner_order is None else partner_order)
         if isinstance(plan_src, Plan) and plan_src is not self and (R, o_mine) not in self._groups and (R, o_theirs) not in plan_src._groups:
             # both sides still to be grouped: the partner's groups are built on a second thread meanwhile (the builder
             # is a plain C function, called with the interpreter lock released)
@@ -440,11 +458,15 @@ class DevicePlan:
     def ref(self):
         return ctypes.byref(self.struct)
 
+    def default_order(self, R):
+        """The group order where a caller names none: tile groups by tile_order_dst, the others GROUP_ORDER."""
+        return tile_order_dst(self.n_index_nodes) if R == TILE_GROUP_R else GROUP_ORDER
+
     def ensure_groups(self, R=GROUP_R, order_mode=None):
         """Row groups of R rows built on the GPU (bpt_plan_group_device).  Of order_mode only the entry order counts:
         by member mask (+4), or for the aligned order of the host builder (+8), which is sequential by construction, its
         parallel stand-in (entries by neighbour id mod 16, then id); else ascending neighbour."""
-        order_mode = GROUP_ORDER if order_mode is None else order_mode
+        order_mode = self.default_order(R) if order_mode is None else order_mode
         by_mask = (2 if order_mode & 8 else (1 if order_mode & 4 else 0)) + (0 if order_mode & 2 else 4)
         with self._lock:
             hit = self._groups.get((R, by_mask))
