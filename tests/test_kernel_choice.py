@@ -135,3 +135,32 @@ def test_order_of_the_source_side_tile_groups():
         assert plan.tile_order_src(16383, 430237) == 10
     finally:
         plan.TILE_ORDER_SRC = old
+
+
+def test_order_of_the_destination_side_tile_groups():
+    """Destination-side tile groups run by decreasing work inside an XCD's range while K and V fit the memory-side cache
+    and keep their locality order from 49 152 nodes on; plan.TILE_ORDER_DST overrides; groups of other sizes keep
+    GROUP_ORDER; a plan's default is what ensure_groups and linked_to use when no order is named."""
+    import numpy as np
+    from bpt_amd import graphbuilder as gb, plan
+    assert plan.tile_order_dst(16383) == 6                    # L = 8192, k = 4
+    assert plan.tile_order_dst(33598) == 6                    # the batch of 32 graphs
+    assert plan.tile_order_dst(65535) == 4                    # L = 32768
+    assert plan.tile_order_dst(49152) == 4 and plan.tile_order_dst(49151) == 6
+    g = gb.BinaryPartition(64, True, 2, 10)
+    src, dst, _ = g.get_edges()
+    n = g.number_of_nodes
+    _, in_csr, _, _, COL, INDPTR_C = gb.get_csrs(src, dst, n)
+    p = plan.Plan(COL, INDPTR_C, in_csr[2], in_csr[1], n, n, torch.device("cpu"))
+    assert p.default_order(plan.TILE_GROUP_R) == 6 and p.default_order(plan.GROUP_R) == plan.GROUP_ORDER
+    old, plan.TILE_ORDER_DST = plan.TILE_ORDER_DST, 4
+    try:
+        assert plan.tile_order_dst(16383) == 4 and p.default_order(plan.TILE_GROUP_R) == 4
+        a = p.ensure_groups(plan.TILE_GROUP_R)                # built in locality order now ...
+        assert a is p.ensure_groups(plan.TILE_GROUP_R, 4)     # ... the same groups as when the order is named
+    finally:
+        plan.TILE_ORDER_DST = old
+    assert p.ensure_groups(plan.TILE_GROUP_R) is p.ensure_groups(plan.TILE_GROUP_R, 6)
+    assert p.ensure_groups(plan.TILE_GROUP_R) is not a
+    chunks = np.asarray(a["host"]["chunks"])
+    assert chunks[0] == 0 and chunks[-1] == len(a["host"]["grp_ptr"]) - 1
