@@ -185,7 +185,7 @@ def measure_side_workload(name, dtype_name, dev, steps, no_graph, label=None):
 
     ref = step()
     torch.cuda.synchronize()
-    runs = timed_runs(step, steps, [10, 2, 2])
+    runs = timed_runs(step, steps, [max(10, steps // 10), 2, 2])
     t, tmin, mode = median(runs), min(runs), "eager"
     if not no_graph:
         gr = graph_replay_runs(step, ref, steps, 10)
@@ -519,8 +519,8 @@ def main():
         side = {}
         for label, wl, dt in (("cfg1", "cfg1", "f32"), ("cfg2", "cfg2", "f32"), ("cfg3-bf16", "cfg3", "bf16"), ("cfg4-k1", "cfg4-k1", "f32"),
                               ("cfg4-k32", "cfg4-k32", "f32"), ("cfg4-w128", "cfg4-w128", "f32"), ("cfg5-bf16", "cfg5", "bf16")):
-            side[label] = measure_side_workload(wl, dt, dev, 50, args.no_graph, label)
-        side["tc32-6x50"] = measure_narrow_heads(dev, 30, args.no_graph)
+            side[label] = measure_side_workload(wl, dt, dev, args.steps, args.no_graph, label)      # (as many steps as the headline: 50 read 3-5 % long)
+        side["tc32-6x50"] = measure_narrow_heads(dev, max(30, args.steps // 4), args.no_graph)
 
     step_gbs = alg["total"] / t_step / 1e9
     out = {
